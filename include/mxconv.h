@@ -1,0 +1,292 @@
+/*
+ * mxconv - MI355X (gfx950) forward convolution behind a C ABI.
+ *
+ * This is the boundary a PopLibs maintainer binds instead of building a
+ * Poplar graph: every entry point takes plain pointers, sizes and a HIP
+ * stream, never a C++ or framework type, and reports failure through a status
+ * code plus a thread-local message (mxconv_last_error).  No exception crosses
+ * it.  Each declaration cites the reference interface it stands in for
+ * (paths relative to the PopLibs source tree).
+ *
+ * Device tensors:
+ *   activations / output  channels-last  [B][field...][G*C]
+ *   weights               packed by mxconv_pack_weights for the chosen plan
+ *   bias                  [G*Co] in the output element type
+ * The external layouts of the reference ([B][G*C][field...] activations,
+ * [G][Co][Ci][kernel...] weights; include/poplin/Convolution.hpp:323-328) are
+ * converted on the device by mxconv_acts_to_internal / mxconv_pack_weights /
+ * mxconv_acts_to_external, the counterpart of creating tensors with
+ * createInput / createWeights and letting convolution() rearrange others
+ * (lib/poplin/Convolution.cpp:2569-2628).
+ */
+#ifndef MXCONV_H
+#define MXCONV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MXCONV_MAX_FIELD_DIMS 4
+/* "No such element", as poplin::getInputIndex returns it
+ * (include/poplin/ConvUtil.hpp:22-26). */
+#define MXCONV_NO_INDEX 0xFFFFFFFFu
+
+typedef enum mxconv_status {
+  MXCONV_OK = 0,
+  /* poputil::poplibs_error (include/poputil/exceptions.hpp:17-21): bad shape,
+   * rank, type or parameter combination. */
+  MXCONV_INVALID_PARAMS = 1,
+  /* poplar::invalid_option: unknown option key or value
+   * (tests/poplin/ConvTest.cpp:684-698). */
+  MXCONV_INVALID_OPTION = 2,
+  /* A valid request this build has no kernel for. */
+  MXCONV_UNSUPPORTED = 3,
+  /* poplar::graph_memory_allocation_error; the harness maps it to exit code
+   * 77 (tools/single_conv_layer.cpp:1531-1537). */
+  MXCONV_OUT_OF_MEMORY = 4,
+  MXCONV_WORKSPACE_TOO_SMALL = 5,
+  MXCONV_BUFFER_TOO_SMALL = 6,
+  MXCONV_HIP_ERROR = 7,
+  MXCONV_NULL_ARGUMENT = 8
+} mxconv_status;
+
+/* poplar::QUARTER / HALF / FLOAT as used for ConvParams::inputType and
+ * outputType (include/poplin/ConvParams.hpp:96-97). */
+typedef enum mxconv_type {
+  MXCONV_QUARTER = 0, /* 8-bit float + metadata byte, see mxconv_fwd_quarter */
+  MXCONV_HALF = 1,    /* IEEE binary16 */
+  MXCONV_FLOAT = 2    /* IEEE binary32 */
+} mxconv_type;
+
+/* poplin::ConvParams::InputTransform (include/poplin/ConvParams.hpp:17-59). */
+typedef struct mxconv_input_transform {
+  uint32_t truncation_lower[MXCONV_MAX_FIELD_DIMS];
+  uint32_t truncation_upper[MXCONV_MAX_FIELD_DIMS];
+  uint32_t dilation[MXCONV_MAX_FIELD_DIMS];
+  uint32_t padding_lower[MXCONV_MAX_FIELD_DIMS];
+  uint32_t padding_upper[MXCONV_MAX_FIELD_DIMS];
+  uint8_t flip[MXCONV_MAX_FIELD_DIMS];
+} mxconv_input_transform;
+
+/* poplin::ConvParams::OutputTransform (include/poplin/ConvParams.hpp:61-94). */
+typedef struct mxconv_output_transform {
+  uint32_t truncation_lower[MXCONV_MAX_FIELD_DIMS];
+  uint32_t truncation_upper[MXCONV_MAX_FIELD_DIMS];
+  uint32_t stride[MXCONV_MAX_FIELD_DIMS];
+  uint32_t padding_lower[MXCONV_MAX_FIELD_DIMS];
+  uint32_t padding_upper[MXCONV_MAX_FIELD_DIMS];
+} mxconv_output_transform;
+
+/* poplin::ConvParams (include/poplin/ConvParams.hpp:16-224).  Only the first
+ * num_field_dims entries of each array are meaningful. */
+typedef struct mxconv_params {
+  int32_t input_type;  /* mxconv_type */
+  int32_t output_type; /* mxconv_type */
+  uint32_t num_field_dims;
+  uint32_t reserved;
+  uint64_t batch_size;
+  uint64_t input_field_shape[MXCONV_MAX_FIELD_DIMS];
+  uint64_t kernel_shape[MXCONV_MAX_FIELD_DIMS];
+  uint64_t input_channels_per_conv_group;
+  uint64_t output_channels_per_conv_group;
+  uint64_t num_conv_groups;
+  mxconv_input_transform input_transform;
+  mxconv_input_transform kernel_transform;
+  mxconv_output_transform output_transform;
+} mxconv_params;
+
+typedef struct mxconv_plan mxconv_plan;
+/* hipStream_t without pulling in the HIP headers. */
+typedef struct ihipStream_t *mxconv_stream;
+
+/* Message of the last failing call on this thread (empty string if none). */
+const char *mxconv_last_error(void);
+const char *mxconv_status_string(mxconv_status status);
+
+/* ---- descriptor algebra (host only, no GPU needed) ---------------------- */
+
+/* ConvParams(inputType, outputType, batchSize, inputFieldShape, kernelShape,
+ * inputChannels, outputChannels, numConvGroups) with identity transforms:
+ * dilation and stride 1, everything else 0 / false
+ * (lib/poplin/ConvParams.cpp:132-152, 268-290). */
+mxconv_status mxconv_params_init(mxconv_params *p, int32_t input_type,
+                                 int32_t output_type, uint64_t batch_size,
+                                 uint32_t num_field_dims,
+                                 const uint64_t *input_field_shape,
+                                 const uint64_t *kernel_shape,
+                                 uint64_t input_channels_per_conv_group,
+                                 uint64_t output_channels_per_conv_group,
+                                 uint64_t num_conv_groups);
+
+/* ConvParams::validate (lib/poplin/ConvParams.cpp:172-266). */
+mxconv_status mxconv_params_validate(const mxconv_params *p);
+
+/* ConvParams::canonicalize (lib/poplin/ConvParams.cpp:468-629), including the
+ * all-zero-output normal form of getZeroConv
+ * (lib/poplin/ConvUtilInternal.cpp:40-76). */
+mxconv_status mxconv_params_canonicalize(const mxconv_params *p,
+                                         mxconv_params *canonical);
+
+/* isZeroConvolution (lib/poplin/ConvUtilInternal.cpp:24-38); canonicalizes
+ * first, as CanonicalConvParams does. */
+mxconv_status mxconv_params_is_zero_convolution(const mxconv_params *p,
+                                                int *is_zero);
+
+/* Size queries of ConvParams (lib/poplin/ConvParams.cpp:631-698). */
+typedef enum mxconv_size_query {
+  MXCONV_TRUNCATED_INPUT_SIZE = 0,     /* getTruncatedInputSize */
+  MXCONV_TRUNCATED_KERNEL_SIZE = 1,    /* getTruncatedKernelSize */
+  MXCONV_TRANSFORMED_INPUT_SIZE = 2,   /* getTransformedInputSize */
+  MXCONV_TRANSFORMED_KERNEL_SIZE = 3,  /* getTransformedKernelSize */
+  MXCONV_UNTRANSFORMED_OUTPUT_SIZE = 4, /* getUntransformedOutputSize */
+  MXCONV_OUTPUT_SIZE = 5               /* getOutputSize */
+} mxconv_size_query;
+mxconv_status mxconv_params_size(const mxconv_params *p, int32_t query,
+                                 uint32_t dim, uint64_t *size);
+
+/* operator== and operator< of ConvParams (lib/poplin/ConvParams.cpp:103-119):
+ * *order is <0, 0 or >0. */
+mxconv_status mxconv_params_compare(const mxconv_params *a,
+                                    const mxconv_params *b, int *order);
+/* std::hash<poplin::ConvParams> (lib/poplin/ConvParams.cpp:734-751): equal
+ * parameters hash equally; the value itself is this build's. */
+mxconv_status mxconv_params_hash(const mxconv_params *p, uint64_t *hash);
+
+/* operator>>(std::istream&, ConvParams&) (lib/poplin/ConvParams.cpp:365-458):
+ * JSON with keys dataType | inputType, outputType, batchSize, numConvGroups,
+ * inputChannelsPerConvGroup, outputChannelsPerConvGroup, inputFieldShape,
+ * kernelShape, inputTransform, kernelTransform, outputTransform. */
+mxconv_status mxconv_params_from_json(const char *json, mxconv_params *p);
+/* operator<<(std::ostream&, const ConvParams&)
+ * (lib/poplin/ConvParams.cpp:292-363).  Writes at most `capacity` bytes
+ * including the terminator; *needed receives the full length + 1. */
+mxconv_status mxconv_params_to_string(const mxconv_params *p, char *buffer,
+                                      size_t capacity, size_t *needed);
+
+/* poplin::getInputIndex / getKernelIndex (lib/poplin/ConvUtil.cpp:234-309). */
+mxconv_status mxconv_get_input_index(const mxconv_params *p, uint32_t dim,
+                                     uint32_t output_index,
+                                     uint32_t kernel_index, uint32_t *index);
+mxconv_status mxconv_get_kernel_index(const mxconv_params *p, uint32_t dim,
+                                      uint32_t output_index,
+                                      uint32_t input_index, uint32_t *index);
+
+/* Range queries of include/poplin/ConvUtil.hpp:34-86; every range is
+ * half-open {begin, end} and {0, 0} when empty. */
+typedef enum mxconv_range_query {
+  /* getOutputRangeForKernelRange(dim, a, b): a = output bounds, b = kernels */
+  MXCONV_OUTPUT_RANGE_FOR_KERNEL_RANGE = 0,
+  /* getOutputRangeForInputRange(dim, a, b): a = output bounds, b = inputs */
+  MXCONV_OUTPUT_RANGE_FOR_INPUT_RANGE = 1,
+  /* getInputRange(dim, a, b): a = output range, b = kernel range */
+  MXCONV_INPUT_RANGE = 2,
+  /* getKernelRange(dim, a, b): a = output range, b = input range */
+  MXCONV_KERNEL_RANGE = 3
+} mxconv_range_query;
+mxconv_status mxconv_get_range(const mxconv_params *p, int32_t query,
+                               uint32_t dim, const uint32_t a[2],
+                               const uint32_t b[2], uint32_t result[2]);
+
+/* getNumberOfMACs (lib/poplin/PerformanceEstimation.hpp:1641-1666) and
+ * getFwdFlops = 2 * MACs (lib/poplin/Convolution.cpp:3217-3221).  MACs that
+ * fall on padding are not counted. */
+mxconv_status mxconv_get_number_of_macs(const mxconv_params *p, uint64_t *macs);
+mxconv_status mxconv_get_fwd_flops(const mxconv_params *p, uint64_t *flops);
+
+/* convolutionValidateOptions (include/poplin/Convolution.hpp:719): the
+ * key/value pairs of a poplar::OptionFlags.  Keys of
+ * lib/poplin/ConvOptions.cpp:105-152 are recognised; partialsType, pass and
+ * planConstraints influence the plan, the remaining (IPU-only) ones are
+ * checked for well-formed values and otherwise ignored. */
+mxconv_status mxconv_validate_options(const char *const *keys,
+                                      const char *const *values,
+                                      size_t num_options);
+
+/* ---- planning ----------------------------------------------------------- */
+
+/* getPlan (lib/poplin/ConvPlan.cpp:1877-1923): validates and canonicalizes
+ * the parameters, applies validateLayerParams
+ * (lib/poplin/ConvValidation.cpp:11-70) and chooses the gfx950 kernel and its
+ * tile shape.  Touches no GPU.  The plan is immutable and may be shared
+ * between threads and streams. */
+mxconv_status mxconv_plan_create(const mxconv_params *p,
+                                 const char *const *option_keys,
+                                 const char *const *option_values,
+                                 size_t num_options, mxconv_plan **plan);
+void mxconv_plan_destroy(mxconv_plan *plan);
+
+/* reportPlanInfo (include/poplin/Convolution.hpp:584-587). */
+mxconv_status mxconv_plan_describe(const mxconv_plan *plan, char *buffer,
+                                   size_t capacity, size_t *needed);
+
+/* Sizes, in bytes, of the device buffers mxconv_fwd works on; what
+ * createInput / createWeights / createConvOutput / createBiases allocate in
+ * the reference (lib/poplin/Convolution.cpp:1563-1577, 1713-1728, 1813-1825,
+ * include/poplin/Convolution.hpp:316-319). */
+typedef enum mxconv_buffer {
+  MXCONV_BUFFER_INPUT = 0,
+  MXCONV_BUFFER_WEIGHTS_PACKED = 1,
+  MXCONV_BUFFER_OUTPUT = 2,
+  MXCONV_BUFFER_BIAS = 3,
+  MXCONV_BUFFER_WORKSPACE = 4,
+  MXCONV_BUFFER_WEIGHTS_EXTERNAL = 5
+} mxconv_buffer;
+mxconv_status mxconv_plan_buffer_bytes(const mxconv_plan *plan, int32_t which,
+                                       size_t *bytes);
+
+/* ---- device work (all asynchronous on `stream`) ------------------------- */
+
+/* Weights [G][Co][Ci][kernel...] (input element type) -> the plan's packed
+ * layout.  Role of createWeights + the weight rearrangement of
+ * lib/poplin/Convolution.cpp:2569-2628. */
+mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
+                                  const void *weights_external,
+                                  void *weights_packed, mxconv_stream stream);
+
+/* Activations [B][G*Ci][field...] -> channels-last, and the output back from
+ * channels-last to [B][G*Co][field...] (actsToInternalShape /
+ * actsToExternalShape, lib/poplin/ConvUtilInternal.cpp:147-175). */
+mxconv_status mxconv_acts_to_internal(const mxconv_plan *plan,
+                                      const void *acts_external,
+                                      void *acts_internal,
+                                      mxconv_stream stream);
+mxconv_status mxconv_acts_to_external(const mxconv_plan *plan,
+                                      const void *out_internal,
+                                      void *out_external, mxconv_stream stream);
+
+/* poplin::convolutionWithOutput (include/poplin/Convolution.hpp:377-384) with
+ * the optional addBias (include/poplin/Convolution.hpp:570-572) fused:
+ *   out[b][o...][g*Co+oc] = cast_outputType( bias[g*Co+oc] +
+ *       sum_{ic,k...} in'[b][o*s + k'...][g*Ci+ic] * w[g][oc][ic][k...] )
+ * accumulated in fp32.  `bias` may be NULL.  For HALF and FLOAT inputs. */
+mxconv_status mxconv_fwd(const mxconv_plan *plan, const void *in,
+                         const void *weights_packed, const void *bias,
+                         void *out, void *workspace, size_t workspace_bytes,
+                         mxconv_stream stream);
+
+/* The same for QUARTER inputs.  Each metadata byte is
+ * (format << 7) | (scale & 0x3f): format 1 = E4M3 ("F143"), 0 = E5M2
+ * ("F152"); scale is a signed 6-bit power of two, value = fp8 * 2^scale (bit
+ * layout of lib/popops/Cast.cpp:168-209).  The product carries 2^(sIn + sW)
+ * (lib/poplin/codelets/inlineAssemblerConv.hpp:28-33).  The 8-bit encodings
+ * are OCP E4M3FN / E5M2, the ones gfx950's matrix cores consume. */
+mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
+                                 uint8_t in_metadata,
+                                 const void *weights_packed,
+                                 uint8_t weights_metadata, const void *bias,
+                                 void *out, void *workspace,
+                                 size_t workspace_bytes, mxconv_stream stream);
+
+/* poplin::addBias (lib/poplin/Convolution.cpp:3637-3648) on a channels-last
+ * tensor of `outer_elems` x `channels` elements of `type`. */
+mxconv_status mxconv_add_bias(int32_t type, void *acts_internal,
+                              const void *bias, uint64_t outer_elems,
+                              uint64_t channels, mxconv_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXCONV_H */

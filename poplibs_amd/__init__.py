@@ -1,0 +1,12 @@
+"""Python binding of the mxconv C ABI (include/mxconv.h).
+
+This package is the ctypes stub a Python caller binds; all logic lives in
+libmxconv.so (C++ host layer + HIP kernels for gfx950).  There is no CPU or
+PyTorch fallback: importing works without a GPU (descriptor algebra and
+planning are host code), any device call without the built library or without
+a GPU raises.
+"""
+from .capi import (  # noqa: F401
+    FLOAT, HALF, QUARTER, ConvParams, InputTransform, MxconvError,
+    OutputTransform, Plan, Status, add_bias, build_library, lib, library_path,
+    quarter_metadata, validate_options)

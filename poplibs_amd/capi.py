@@ -1,0 +1,540 @@
+"""ctypes declarations for include/mxconv.h and thin Python conveniences.
+
+`ConvParams`, `InputTransform` and `OutputTransform` carry the field names of
+poplin::ConvParams (include/poplin/ConvParams.hpp:16-224) so that tests read
+like the reference's; they only marshal into `mxconv_params` - validation,
+canonicalisation, size and range algebra all run in the C++ library.
+"""
+import ctypes
+import os
+import subprocess
+from ctypes import (POINTER, Structure, byref, c_char_p, c_int, c_int32,
+                    c_size_t, c_uint8, c_uint32, c_uint64, c_void_p)
+
+MAX_FIELD_DIMS = 4
+NO_INDEX = 0xFFFFFFFF
+QUARTER, HALF, FLOAT = 0, 1, 2
+TYPE_NAMES = {QUARTER: "quarter", HALF: "half", FLOAT: "float"}
+TYPE_BYTES = {QUARTER: 1, HALF: 2, FLOAT: 4}
+
+
+class Status:
+    OK = 0
+    INVALID_PARAMS = 1
+    INVALID_OPTION = 2
+    UNSUPPORTED = 3
+    OUT_OF_MEMORY = 4
+    WORKSPACE_TOO_SMALL = 5
+    BUFFER_TOO_SMALL = 6
+    HIP_ERROR = 7
+    NULL_ARGUMENT = 8
+
+
+class MxconvError(RuntimeError):
+    """A failing C ABI call; `.status` is the mxconv_status value.
+
+    INVALID_PARAMS corresponds to poputil::poplibs_error and INVALID_OPTION to
+    poplar::invalid_option in the reference.
+    """
+
+    def __init__(self, status, message):
+        super().__init__(f"mxconv status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+_U32x = c_uint32 * MAX_FIELD_DIMS
+_U64x = c_uint64 * MAX_FIELD_DIMS
+_U8x = c_uint8 * MAX_FIELD_DIMS
+
+
+class _CInputTransform(Structure):
+    _fields_ = [("truncation_lower", _U32x), ("truncation_upper", _U32x),
+                ("dilation", _U32x), ("padding_lower", _U32x),
+                ("padding_upper", _U32x), ("flip", _U8x)]
+
+
+class _COutputTransform(Structure):
+    _fields_ = [("truncation_lower", _U32x), ("truncation_upper", _U32x),
+                ("stride", _U32x), ("padding_lower", _U32x),
+                ("padding_upper", _U32x)]
+
+
+class CParams(Structure):
+    _fields_ = [("input_type", c_int32), ("output_type", c_int32),
+                ("num_field_dims", c_uint32), ("reserved", c_uint32),
+                ("batch_size", c_uint64), ("input_field_shape", _U64x),
+                ("kernel_shape", _U64x),
+                ("input_channels_per_conv_group", c_uint64),
+                ("output_channels_per_conv_group", c_uint64),
+                ("num_conv_groups", c_uint64),
+                ("input_transform", _CInputTransform),
+                ("kernel_transform", _CInputTransform),
+                ("output_transform", _COutputTransform)]
+
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmxconv.so")
+_lib = None
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def build_library(force=False):
+    """Compile libmxconv.so for gfx950 (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-C", _HERE, "-j8", "all"]
+    if force:
+        cmd.insert(1, "-B")
+    subprocess.check_call(cmd)
+
+
+def lib():
+    """The loaded C ABI library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError(
+            f"{_LIB_PATH} is missing: build it with "
+            "`python -c 'import __graft_entry__ as g; g.build()'` or "
+            "`make -C poplibs_amd`. There is no fallback implementation.")
+    L = ctypes.CDLL(_LIB_PATH)
+    P = POINTER(CParams)
+    sigs = {
+        "mxconv_last_error": (c_char_p, []),
+        "mxconv_status_string": (c_char_p, [c_int]),
+        "mxconv_params_init": (c_int, [P, c_int32, c_int32, c_uint64, c_uint32,
+                                       POINTER(c_uint64), POINTER(c_uint64),
+                                       c_uint64, c_uint64, c_uint64]),
+        "mxconv_params_validate": (c_int, [P]),
+        "mxconv_params_canonicalize": (c_int, [P, P]),
+        "mxconv_params_is_zero_convolution": (c_int, [P, POINTER(c_int)]),
+        "mxconv_params_size": (c_int, [P, c_int32, c_uint32,
+                                       POINTER(c_uint64)]),
+        "mxconv_params_compare": (c_int, [P, P, POINTER(c_int)]),
+        "mxconv_params_hash": (c_int, [P, POINTER(c_uint64)]),
+        "mxconv_params_from_json": (c_int, [c_char_p, P]),
+        "mxconv_params_to_string": (c_int, [P, c_char_p, c_size_t,
+                                            POINTER(c_size_t)]),
+        "mxconv_get_input_index": (c_int, [P, c_uint32, c_uint32, c_uint32,
+                                           POINTER(c_uint32)]),
+        "mxconv_get_kernel_index": (c_int, [P, c_uint32, c_uint32, c_uint32,
+                                            POINTER(c_uint32)]),
+        "mxconv_get_range": (c_int, [P, c_int32, c_uint32, POINTER(c_uint32),
+                                     POINTER(c_uint32), POINTER(c_uint32)]),
+        "mxconv_get_number_of_macs": (c_int, [P, POINTER(c_uint64)]),
+        "mxconv_get_fwd_flops": (c_int, [P, POINTER(c_uint64)]),
+        "mxconv_validate_options": (c_int, [POINTER(c_char_p),
+                                            POINTER(c_char_p), c_size_t]),
+        "mxconv_plan_create": (c_int, [P, POINTER(c_char_p), POINTER(c_char_p),
+                                       c_size_t, POINTER(c_void_p)]),
+        "mxconv_plan_destroy": (None, [c_void_p]),
+        "mxconv_plan_describe": (c_int, [c_void_p, c_char_p, c_size_t,
+                                         POINTER(c_size_t)]),
+        "mxconv_plan_buffer_bytes": (c_int, [c_void_p, c_int32,
+                                             POINTER(c_size_t)]),
+        "mxconv_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p,
+                                        c_void_p]),
+        "mxconv_acts_to_internal": (c_int, [c_void_p, c_void_p, c_void_p,
+                                            c_void_p]),
+        "mxconv_acts_to_external": (c_int, [c_void_p, c_void_p, c_void_p,
+                                            c_void_p]),
+        "mxconv_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_size_t, c_void_p]),
+        "mxconv_fwd_quarter": (c_int, [c_void_p, c_void_p, c_uint8, c_void_p,
+                                       c_uint8, c_void_p, c_void_p, c_void_p,
+                                       c_size_t, c_void_p]),
+        "mxconv_add_bias": (c_int, [c_int32, c_void_p, c_void_p, c_uint64,
+                                    c_uint64, c_void_p]),
+    }
+    for name, (restype, argtypes) in sigs.items():
+        fn = getattr(L, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    L._declared = sorted(sigs)
+    _lib = L
+    return L
+
+
+def _check(status):
+    if status != Status.OK:
+        raise MxconvError(status, lib().mxconv_last_error().decode())
+
+
+class InputTransform:
+    def __init__(self, n=0, truncationLower=None, truncationUpper=None,
+                 dilation=None, paddingLower=None, paddingUpper=None,
+                 flip=None):
+        self.truncationLower = list(truncationLower or [0] * n)
+        self.truncationUpper = list(truncationUpper or [0] * n)
+        self.dilation = list(dilation or [1] * n)
+        self.paddingLower = list(paddingLower or [0] * n)
+        self.paddingUpper = list(paddingUpper or [0] * n)
+        self.flip = list(flip or [False] * n)
+
+    def _fields(self):
+        return (self.truncationLower, self.truncationUpper, self.dilation,
+                self.paddingLower, self.paddingUpper, self.flip)
+
+    def __eq__(self, o):
+        return self._fields() == o._fields()
+
+    def __repr__(self):
+        return ("InputTransform(truncationLower=%r, truncationUpper=%r, "
+                "dilation=%r, paddingLower=%r, paddingUpper=%r, flip=%r)"
+                % self._fields())
+
+
+class OutputTransform:
+    def __init__(self, n=0, truncationLower=None, truncationUpper=None,
+                 stride=None, paddingLower=None, paddingUpper=None):
+        self.truncationLower = list(truncationLower or [0] * n)
+        self.truncationUpper = list(truncationUpper or [0] * n)
+        self.stride = list(stride or [1] * n)
+        self.paddingLower = list(paddingLower or [0] * n)
+        self.paddingUpper = list(paddingUpper or [0] * n)
+
+    def _fields(self):
+        return (self.truncationLower, self.truncationUpper, self.stride,
+                self.paddingLower, self.paddingUpper)
+
+    def __eq__(self, o):
+        return self._fields() == o._fields()
+
+    def __repr__(self):
+        return ("OutputTransform(truncationLower=%r, truncationUpper=%r, "
+                "stride=%r, paddingLower=%r, paddingUpper=%r)" % self._fields())
+
+
+class ConvParams:
+    """Mirror of poplin::ConvParams; see the module docstring."""
+
+    def __init__(self, inputType, outputType=None, batchSize=1,
+                 inputFieldShape=(), kernelShape=(),
+                 inputChannelsPerConvGroup=1, outputChannelsPerConvGroup=1,
+                 numConvGroups=1, inputTransform=None, kernelTransform=None,
+                 outputTransform=None):
+        n = len(inputFieldShape)
+        self.inputType = inputType
+        self.outputType = inputType if outputType is None else outputType
+        self.batchSize = batchSize
+        self.inputFieldShape = list(inputFieldShape)
+        self.kernelShape = list(kernelShape)
+        self.inputChannelsPerConvGroup = inputChannelsPerConvGroup
+        self.outputChannelsPerConvGroup = outputChannelsPerConvGroup
+        self.numConvGroups = numConvGroups
+        self.inputTransform = inputTransform or InputTransform(n)
+        self.kernelTransform = kernelTransform or InputTransform(n)
+        self.outputTransform = outputTransform or OutputTransform(n)
+
+    # -- marshalling ------------------------------------------------------
+    def to_c(self):
+        n = len(self.inputFieldShape)
+        if n > MAX_FIELD_DIMS:
+            raise MxconvError(Status.INVALID_PARAMS,
+                              "too many field dimensions")
+        c = CParams()
+        c.input_type, c.output_type = self.inputType, self.outputType
+        c.num_field_dims = n
+        c.batch_size = self.batchSize
+        c.input_channels_per_conv_group = self.inputChannelsPerConvGroup
+        c.output_channels_per_conv_group = self.outputChannelsPerConvGroup
+        c.num_conv_groups = self.numConvGroups
+        if len(self.kernelShape) != n:
+            raise MxconvError(
+                Status.INVALID_PARAMS,
+                "Number of kernel field dimensions does not match the number "
+                "of input field dimensions")
+        for d in range(n):
+            c.input_field_shape[d] = self.inputFieldShape[d]
+            c.kernel_shape[d] = self.kernelShape[d]
+
+        def put(dst, src, what):
+            if len(src) != n:
+                raise MxconvError(
+                    Status.INVALID_PARAMS,
+                    f"Number of {what} dimensions ({len(src)}) does not match "
+                    f"the number of field dimensions ({n})")
+            for d in range(n):
+                dst[d] = int(src[d])
+
+        for ct, t, name in ((c.input_transform, self.inputTransform, "input"),
+                            (c.kernel_transform, self.kernelTransform,
+                             "kernel")):
+            put(ct.truncation_lower, t.truncationLower, name + " truncation")
+            put(ct.truncation_upper, t.truncationUpper, name + " truncation")
+            put(ct.dilation, t.dilation, name + " dilation")
+            put(ct.padding_lower, t.paddingLower, name + " padding")
+            put(ct.padding_upper, t.paddingUpper, name + " padding")
+            put(ct.flip, t.flip, name + " flip")
+        ot, o = c.output_transform, self.outputTransform
+        put(ot.truncation_lower, o.truncationLower, "output truncation")
+        put(ot.truncation_upper, o.truncationUpper, "output truncation")
+        put(ot.stride, o.stride, "stride")
+        put(ot.padding_lower, o.paddingLower, "output padding")
+        put(ot.padding_upper, o.paddingUpper, "output padding")
+        return c
+
+    @staticmethod
+    def from_c(c):
+        n = c.num_field_dims
+
+        def it(t):
+            return InputTransform(
+                n, list(t.truncation_lower[:n]), list(t.truncation_upper[:n]),
+                list(t.dilation[:n]), list(t.padding_lower[:n]),
+                list(t.padding_upper[:n]), [bool(f) for f in t.flip[:n]])
+
+        o = c.output_transform
+        return ConvParams(
+            c.input_type, c.output_type, c.batch_size,
+            list(c.input_field_shape[:n]), list(c.kernel_shape[:n]),
+            c.input_channels_per_conv_group, c.output_channels_per_conv_group,
+            c.num_conv_groups, it(c.input_transform), it(c.kernel_transform),
+            OutputTransform(n, list(o.truncation_lower[:n]),
+                            list(o.truncation_upper[:n]), list(o.stride[:n]),
+                            list(o.padding_lower[:n]),
+                            list(o.padding_upper[:n])))
+
+    @staticmethod
+    def from_json(text):
+        c = CParams()
+        _check(lib().mxconv_params_from_json(text.encode(), byref(c)))
+        return ConvParams.from_c(c)
+
+    def _fields(self):
+        return (self.inputType, self.outputType, self.batchSize,
+                self.inputFieldShape, self.kernelShape,
+                self.inputChannelsPerConvGroup,
+                self.outputChannelsPerConvGroup, self.numConvGroups)
+
+    def __eq__(self, o):
+        return (self._fields() == o._fields()
+                and self.inputTransform == o.inputTransform
+                and self.kernelTransform == o.kernelTransform
+                and self.outputTransform == o.outputTransform)
+
+    def __repr__(self):
+        return ("ConvParams(%s->%s, batch=%d, field=%r, kernel=%r, Ci=%d, "
+                "Co=%d, G=%d, in=%r, k=%r, out=%r)" % (
+                    TYPE_NAMES[self.inputType], TYPE_NAMES[self.outputType],
+                    self.batchSize, self.inputFieldShape, self.kernelShape,
+                    self.inputChannelsPerConvGroup,
+                    self.outputChannelsPerConvGroup, self.numConvGroups,
+                    self.inputTransform, self.kernelTransform,
+                    self.outputTransform))
+
+    # -- the reference's member functions, answered by the C++ library ----
+    def validate(self):
+        _check(lib().mxconv_params_validate(byref(self.to_c())))
+
+    def canonicalize(self):
+        out = CParams()
+        _check(lib().mxconv_params_canonicalize(byref(self.to_c()),
+                                                byref(out)))
+        return ConvParams.from_c(out)
+
+    def _size(self, query, dim):
+        v = c_uint64()
+        _check(lib().mxconv_params_size(byref(self.to_c()), query, dim,
+                                        byref(v)))
+        return v.value
+
+    def getTruncatedInputSize(self, dim):
+        return self._size(0, dim)
+
+    def getTruncatedKernelSize(self, dim):
+        return self._size(1, dim)
+
+    def getTransformedInputSize(self, dim):
+        return self._size(2, dim)
+
+    def getTransformedKernelSize(self, dim):
+        return self._size(3, dim)
+
+    def getUntransformedOutputSize(self, dim):
+        return self._size(4, dim)
+
+    def getOutputSize(self, dim):
+        return self._size(5, dim)
+
+    def getOutputFieldShape(self):
+        return [self.getOutputSize(d)
+                for d in range(len(self.inputFieldShape))]
+
+    def getNumFieldDims(self):
+        return len(self.inputFieldShape)
+
+    def getNumInputChans(self):
+        return self.inputChannelsPerConvGroup * self.numConvGroups
+
+    def getNumOutputChans(self):
+        return self.outputChannelsPerConvGroup * self.numConvGroups
+
+    def isZeroConvolution(self):
+        v = c_int()
+        _check(lib().mxconv_params_is_zero_convolution(byref(self.to_c()),
+                                                       byref(v)))
+        return bool(v.value)
+
+    def compare(self, other):
+        v = c_int()
+        _check(lib().mxconv_params_compare(byref(self.to_c()),
+                                           byref(other.to_c()), byref(v)))
+        return v.value
+
+    def hash(self):
+        v = c_uint64()
+        _check(lib().mxconv_params_hash(byref(self.to_c()), byref(v)))
+        return v.value
+
+    def __str__(self):
+        need = c_size_t()
+        c = self.to_c()
+        _check(lib().mxconv_params_to_string(byref(c), None, 0, byref(need)))
+        buf = ctypes.create_string_buffer(need.value)
+        _check(lib().mxconv_params_to_string(byref(c), buf, need.value,
+                                             byref(need)))
+        return buf.value.decode()
+
+    # ConvUtil (include/poplin/ConvUtil.hpp)
+    def getInputIndex(self, dim, outputIndex, kernelIndex):
+        v = c_uint32()
+        _check(lib().mxconv_get_input_index(byref(self.to_c()), dim,
+                                            outputIndex, kernelIndex,
+                                            byref(v)))
+        return v.value
+
+    def getKernelIndex(self, dim, outputIndex, inputIndex):
+        v = c_uint32()
+        _check(lib().mxconv_get_kernel_index(byref(self.to_c()), dim,
+                                             outputIndex, inputIndex,
+                                             byref(v)))
+        return v.value
+
+    def _range(self, query, dim, a, b):
+        A = (c_uint32 * 2)(*a)
+        B = (c_uint32 * 2)(*b)
+        R = (c_uint32 * 2)()
+        _check(lib().mxconv_get_range(byref(self.to_c()), query, dim, A, B, R))
+        return (R[0], R[1])
+
+    def getOutputRangeForKernelRange(self, dim, outputRange, kernelRange):
+        return self._range(0, dim, outputRange, kernelRange)
+
+    def getOutputRangeForKernelIndex(self, dim, outputRange, kernelIndex):
+        return self._range(0, dim, outputRange, (kernelIndex, kernelIndex + 1))
+
+    def getOutputRangeForInputRange(self, dim, outputRange, inputRange):
+        return self._range(1, dim, outputRange, inputRange)
+
+    def getOutputRangeForInputIndex(self, dim, outputRange, inputIndex):
+        return self._range(1, dim, outputRange, (inputIndex, inputIndex + 1))
+
+    def getInputRange(self, dim, outputRange, kernel):
+        if isinstance(kernel, int):
+            kernel = (kernel, kernel + 1)
+        return self._range(2, dim, outputRange, kernel)
+
+    def getKernelRange(self, dim, outputRange, inp):
+        if isinstance(inp, int):
+            inp = (inp, inp + 1)
+        return self._range(3, dim, outputRange, inp)
+
+    def getNumberOfMACs(self):
+        v = c_uint64()
+        _check(lib().mxconv_get_number_of_macs(byref(self.to_c()), byref(v)))
+        return v.value
+
+    def getFwdFlops(self):
+        v = c_uint64()
+        _check(lib().mxconv_get_fwd_flops(byref(self.to_c()), byref(v)))
+        return v.value
+
+
+def _option_arrays(options):
+    options = options or {}
+    keys = (c_char_p * max(len(options), 1))()
+    values = (c_char_p * max(len(options), 1))()
+    for i, (k, v) in enumerate(options.items()):
+        keys[i] = str(k).encode()
+        values[i] = str(v).encode()
+    return keys, values, len(options)
+
+
+def validate_options(options):
+    """convolutionValidateOptions (include/poplin/Convolution.hpp:719)."""
+    keys, values, n = _option_arrays(options)
+    _check(lib().mxconv_validate_options(keys, values, n))
+
+
+def quarter_metadata(fmt, scale):
+    """Metadata byte of a quarter tensor: format 1 = E4M3, 0 = E5M2."""
+    return ((fmt & 1) << 7) | (scale & 0x3f)
+
+
+BUF_INPUT, BUF_WEIGHTS_PACKED, BUF_OUTPUT, BUF_BIAS, BUF_WORKSPACE, \
+    BUF_WEIGHTS_EXTERNAL = range(6)
+
+
+class Plan:
+    """Owns an mxconv_plan.  Device pointers are plain integers (for torch
+    tensors: `t.data_ptr()`); `stream` is a hipStream_t value or 0."""
+
+    def __init__(self, params, options=None):
+        self.params = params
+        keys, values, n = _option_arrays(options)
+        self._h = c_void_p()
+        _check(lib().mxconv_plan_create(byref(params.to_c()), keys, values, n,
+                                        byref(self._h)))
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h and _lib is not None:
+            _lib.mxconv_plan_destroy(h)
+            self._h = None
+
+    def describe(self):
+        need = c_size_t()
+        _check(lib().mxconv_plan_describe(self._h, None, 0, byref(need)))
+        buf = ctypes.create_string_buffer(need.value)
+        _check(lib().mxconv_plan_describe(self._h, buf, need.value,
+                                          byref(need)))
+        return buf.value.decode()
+
+    def buffer_bytes(self, which):
+        v = c_size_t()
+        _check(lib().mxconv_plan_buffer_bytes(self._h, which, byref(v)))
+        return v.value
+
+    def pack_weights(self, weights_external, weights_packed, stream=0):
+        _check(lib().mxconv_pack_weights(self._h, weights_external,
+                                         weights_packed, stream))
+
+    def acts_to_internal(self, external, internal, stream=0):
+        _check(lib().mxconv_acts_to_internal(self._h, external, internal,
+                                             stream))
+
+    def acts_to_external(self, internal, external, stream=0):
+        _check(lib().mxconv_acts_to_external(self._h, internal, external,
+                                             stream))
+
+    def fwd(self, inp, weights_packed, out, bias=None, workspace=None,
+            workspace_bytes=0, stream=0):
+        _check(lib().mxconv_fwd(self._h, inp, weights_packed, bias, out,
+                                workspace, workspace_bytes, stream))
+
+    def fwd_quarter(self, inp, in_metadata, weights_packed, weights_metadata,
+                    out, bias=None, workspace=None, workspace_bytes=0,
+                    stream=0):
+        _check(lib().mxconv_fwd_quarter(self._h, inp, in_metadata,
+                                        weights_packed, weights_metadata, bias,
+                                        out, workspace, workspace_bytes,
+                                        stream))
+
+
+def add_bias(type_id, acts, bias, outer_elems, channels, stream=0):
+    _check(lib().mxconv_add_bias(type_id, acts, bias, outer_elems, channels,
+                                 stream))

@@ -1,0 +1,63 @@
+// Device-side element conversions shared by the kernels.
+#ifndef poplibs_amd_device_types_hpp
+#define poplibs_amd_device_types_hpp
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mxk {
+
+/// OCP 8-bit float -> fp32 in software.  E4M3FN: bias 7, S.1111.111 is NaN, no
+/// infinities.  E5M2: bias 15, IEEE-like infinities / NaNs.  Every finite code
+/// is exactly representable in fp32 (and in fp16).
+__device__ __forceinline__ float decodeFp8(uint32_t code, int format) {
+  const uint32_t sign = (code & 0x80u) << 24;
+  uint32_t bits;
+  if (format == 1) { // E4M3FN
+    const uint32_t e = (code >> 3) & 0xfu, m = code & 7u;
+    if (e == 0xfu && m == 7u)
+      bits = 0x7fc00000u;
+    else if (e == 0u)
+      return __uint_as_float(sign | __float_as_uint(float(m) * 0x1p-9f));
+    else
+      bits = ((e + 120u) << 23) | (m << 20); // 127 - 7 = 120
+  } else { // E5M2
+    const uint32_t e = (code >> 2) & 0x1fu, m = code & 3u;
+    if (e == 0x1fu)
+      bits = m ? 0x7fc00000u : 0x7f800000u;
+    else if (e == 0u)
+      return __uint_as_float(sign | __float_as_uint(float(m) * 0x1p-16f));
+    else
+      bits = ((e + 112u) << 23) | (m << 21); // 127 - 15 = 112
+  }
+  return __uint_as_float(sign | bits);
+}
+
+template <class T> struct Load;
+template <> struct Load<float> {
+  static __device__ __forceinline__ float at(const float *p, size_t i, int) {
+    return p[i];
+  }
+};
+template <> struct Load<__half> {
+  static __device__ __forceinline__ float at(const __half *p, size_t i, int) {
+    return __half2float(p[i]);
+  }
+};
+template <> struct Load<uint8_t> {
+  static __device__ __forceinline__ float at(const uint8_t *p, size_t i,
+                                             int format) {
+    return decodeFp8(p[i], format);
+  }
+};
+
+/// fp32 -> output element, round to nearest even.
+__device__ __forceinline__ void storeOut(float *p, size_t i, float v) {
+  p[i] = v;
+}
+__device__ __forceinline__ void storeOut(__half *p, size_t i, float v) {
+  p[i] = __float2half_rn(v);
+}
+
+} // namespace mxk
+#endif

@@ -1,0 +1,100 @@
+// Host-callable launchers of the gfx950 kernels and the plain-data
+// descriptors they take.  Everything here is independent of the ConvParams
+// C++ class so that the kernels see only what they need.
+#ifndef poplibs_amd_kernels_hpp
+#define poplibs_amd_kernels_hpp
+#include <cstddef>
+#include <cstdint>
+#include <hip/hip_runtime_api.h>
+
+namespace mxk {
+
+constexpr int kMaxDims = 4;
+
+// Element type ids shared with the C ABI (mxconv_type).
+enum : int { kQuarter = 0, kHalf = 1, kFloat = 2 };
+// FP8 encodings (bit 7 of a quarter metadata byte).
+enum : int { kE5M2 = 0, kE4M3 = 1 };
+
+/// One spatial dimension of an input or kernel transform.
+struct DimTransform {
+  uint32_t size, truncLo, truncHi, dilation, padLo, padHi, flip;
+  uint32_t transformedSize; // padLo + dilated(size - truncLo - truncHi) + padHi
+};
+
+/// Everything the any-parameter direct kernel needs.
+struct GenericDesc {
+  uint32_t numDims;
+  uint32_t batch, groups, inChansPerGroup, outChansPerGroup;
+  DimTransform in[kMaxDims];
+  DimTransform kernel[kMaxDims];
+  uint32_t outSize[kMaxDims];
+  uint32_t outTruncLo[kMaxDims], outStride[kMaxDims];
+  uint32_t outPadLo[kMaxDims], outPadHi[kMaxDims];
+  uint32_t kernelElems; // product of kernel sizes
+  uint64_t outElems;    // batch * prod(outSize) * groups * outChansPerGroup
+};
+
+/// Quarter (FP8) operands: encodings and the combined power-of-two scale.
+struct QuarterInfo {
+  int inFormat = kE4M3, weightFormat = kE4M3;
+  float scale = 1.0f; // 2^(scaleIn + scaleWeights)
+};
+
+/// Any ConvParams.  in: channels-last activations; weights: [G][K][Ci][Co];
+/// bias may be null; fp32 accumulation.
+hipError_t launchGeneric(const GenericDesc &d, int inType, int outType,
+                         const void *in, const void *weights, const void *bias,
+                         void *out, const QuarterInfo &q, hipStream_t stream);
+
+/// dst[i0][i1][i2][i3] = src[...] where dst dimension j walks source dimension
+/// perm[j]; srcDims are the source extents; elemBytes 1, 2 or 4.
+hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
+                          const int perm[4], int elemBytes, hipStream_t stream);
+
+/// Weights [G][Co][Ci][taps] -> [G][coPadded][kPadded] with k = tap * Ci + ci,
+/// zero-filled beyond Co and beyond taps * Ci: the B operand of the
+/// matrix-core kernel, K contiguous.
+hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
+                                  uint32_t co, uint32_t ci, uint32_t taps,
+                                  uint32_t coPadded, uint32_t kPadded,
+                                  int elemBytes, hipStream_t stream);
+
+/// acts[outer][c] += bias[c] for `type` elements (kHalf or kFloat).
+hipError_t launchAddBias(int type, void *acts, const void *bias,
+                         uint64_t outerElems, uint64_t channels,
+                         hipStream_t stream);
+
+/// Implicit-GEMM forward convolution on the matrix cores (2-D field, stride,
+/// zero padding and kernel dilation only).
+struct IgemmDesc {
+  uint32_t batch, groups, inChansPerGroup, outChansPerGroup;
+  uint32_t inH, inW, outH, outW, kH, kW;
+  // input row = outRow * strideH + kRow * dilH - padH, read when it lies in
+  // [loH, hiH) and taken as zero otherwise; the same along W.
+  int32_t padH, padW;
+  uint32_t strideH, strideW, dilH, dilW;
+  uint32_t loH, hiH, loW, hiW;
+  // Tile shape chosen by the planner.
+  uint32_t blockM, blockN, blockK;
+};
+hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
+                       const void *in, const void *weightsPacked,
+                       const void *bias, void *out, const QuarterInfo &q,
+                       hipStream_t stream);
+
+/// Depthwise (one input and one output channel per group) direct convolution,
+/// 2-D field, stride, zero padding, kernel dilation.
+struct DepthwiseDesc {
+  uint32_t batch, channels;
+  uint32_t inH, inW, outH, outW, kH, kW;
+  int32_t padH, padW; // as in IgemmDesc
+  uint32_t strideH, strideW, dilH, dilW;
+  uint32_t loH, hiH, loW, hiW;
+};
+hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
+                           const void *in, const void *weightsPacked,
+                           const void *bias, void *out, hipStream_t stream);
+
+} // namespace mxk
+#endif

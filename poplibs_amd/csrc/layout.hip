@@ -1,0 +1,155 @@
+// Layout conversions between the external tensor layouts of the convolution
+// API ([B][G*C][field...] activations, [G][Co][Ci][kernel...] weights) and the
+// device layouts the kernels use, plus the stand-alone bias add.  None of
+// these sit on the timed path: tensors live in the device layout.
+#include "device_types.hpp"
+#include "kernels.hpp"
+
+namespace mxk {
+namespace {
+
+struct PermuteArgs {
+  uint64_t dstDims[4];
+  uint64_t srcStride[4]; // stride in the source of each destination dimension
+  uint64_t total;
+};
+
+template <class T>
+__global__ __launch_bounds__(256) void permuteKernel(PermuteArgs a,
+                                                     const T *__restrict__ src,
+                                                     T *__restrict__ dst) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= a.total)
+    return;
+  uint64_t rest = tid, srcIndex = 0;
+  for (int j = 3; j >= 0; --j) {
+    srcIndex += (rest % a.dstDims[j]) * a.srcStride[j];
+    rest /= a.dstDims[j];
+  }
+  dst[tid] = src[srcIndex];
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void packIgemmWeightsKernel(
+    const T *__restrict__ src, T *__restrict__ dst, uint32_t co, uint32_t ci,
+    uint32_t taps, uint32_t coPadded, uint32_t kPadded, uint64_t total) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= total)
+    return;
+  const uint32_t k = uint32_t(tid % kPadded);
+  const uint32_t n = uint32_t((tid / kPadded) % coPadded);
+  const uint64_t g = tid / (uint64_t(kPadded) * coPadded);
+  T v = T(0);
+  if (n < co && k < taps * ci) {
+    const uint32_t tap = k / ci, c = k % ci;
+    v = src[((g * co + n) * ci + c) * taps + tap];
+  }
+  dst[tid] = v;
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void addBiasKernel(T *acts,
+                                                     const T *__restrict__ bias,
+                                                     uint64_t total,
+                                                     uint64_t channels) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= total)
+    return;
+  const float v = Load<T>::at(acts, tid, 0) + Load<T>::at(bias, tid % channels, 0);
+  storeOut(acts, tid, v);
+}
+
+} // namespace
+
+hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
+                          const int perm[4], int elemBytes,
+                          hipStream_t stream) {
+  uint64_t srcStrides[4];
+  srcStrides[3] = 1;
+  for (int i = 2; i >= 0; --i)
+    srcStrides[i] = srcStrides[i + 1] * srcDims[i + 1];
+  PermuteArgs a;
+  a.total = 1;
+  for (int j = 0; j != 4; ++j) {
+    a.dstDims[j] = srcDims[perm[j]];
+    a.srcStride[j] = srcStrides[perm[j]];
+    a.total *= a.dstDims[j];
+  }
+  if (a.total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (a.total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  switch (elemBytes) {
+  case 1:
+    hipLaunchKernelGGL(permuteKernel<uint8_t>, grid, block, 0, stream, a,
+                       static_cast<const uint8_t *>(src),
+                       static_cast<uint8_t *>(dst));
+    break;
+  case 2:
+    hipLaunchKernelGGL(permuteKernel<uint16_t>, grid, block, 0, stream, a,
+                       static_cast<const uint16_t *>(src),
+                       static_cast<uint16_t *>(dst));
+    break;
+  case 4:
+    hipLaunchKernelGGL(permuteKernel<uint32_t>, grid, block, 0, stream, a,
+                       static_cast<const uint32_t *>(src),
+                       static_cast<uint32_t *>(dst));
+    break;
+  default:
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
+                                  uint32_t co, uint32_t ci, uint32_t taps,
+                                  uint32_t coPadded, uint32_t kPadded,
+                                  int elemBytes, hipStream_t stream) {
+  const uint64_t total = uint64_t(groups) * coPadded * kPadded;
+  if (total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  if (elemBytes == 1)
+    hipLaunchKernelGGL(packIgemmWeightsKernel<uint8_t>, grid, block, 0, stream,
+                       static_cast<const uint8_t *>(src),
+                       static_cast<uint8_t *>(dst), co, ci, taps, coPadded,
+                       kPadded, total);
+  else if (elemBytes == 2)
+    hipLaunchKernelGGL(packIgemmWeightsKernel<uint16_t>, grid, block, 0, stream,
+                       static_cast<const uint16_t *>(src),
+                       static_cast<uint16_t *>(dst), co, ci, taps, coPadded,
+                       kPadded, total);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launchAddBias(int type, void *acts, const void *bias,
+                         uint64_t outerElems, uint64_t channels,
+                         hipStream_t stream) {
+  const uint64_t total = outerElems * channels;
+  if (total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  if (type == kFloat)
+    hipLaunchKernelGGL(addBiasKernel<float>, grid, block, 0, stream,
+                       static_cast<float *>(acts),
+                       static_cast<const float *>(bias), total, channels);
+  else if (type == kHalf)
+    hipLaunchKernelGGL(addBiasKernel<__half>, grid, block, 0, stream,
+                       static_cast<__half *>(acts),
+                       static_cast<const __half *>(bias), total, channels);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+} // namespace mxk

@@ -1,0 +1,608 @@
+// The C ABI declared in mxconv.h: argument checking, translation of C++
+// exceptions into status codes, and dispatch to the kernel launchers.
+#include "mxconv.h"
+
+#include "../src/ConvOptions.hpp"
+#include "../src/Plan.hpp"
+#include "kernels.hpp"
+#include "poplar/exceptions.hpp"
+#include "poplin/ConvParams.hpp"
+#include "poplin/ConvUtil.hpp"
+#include "poputil/exceptions.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <sstream>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string lastError;
+
+mxconv_status fail(mxconv_status s, const std::string &message) {
+  lastError = message;
+  return s;
+}
+
+/// Runs `body`, mapping the exceptions of the C++ layer to status codes.
+template <class F> mxconv_status guarded(F &&body) {
+  try {
+    lastError.clear();
+    return body();
+  } catch (const poplar::invalid_option &e) {
+    return fail(MXCONV_INVALID_OPTION, e.what());
+  } catch (const poplar::graph_memory_allocation_error &e) {
+    return fail(MXCONV_OUT_OF_MEMORY, e.what());
+  } catch (const poputil::poplibs_error &e) {
+    return fail(MXCONV_INVALID_PARAMS, e.what());
+  } catch (const std::bad_alloc &) {
+    return fail(MXCONV_OUT_OF_MEMORY, "host allocation failed");
+  } catch (const std::exception &e) {
+    return fail(MXCONV_INVALID_PARAMS, e.what());
+  }
+}
+
+#define REQUIRE_ARG(p)                                                         \
+  if (!(p))                                                                    \
+  return fail(MXCONV_NULL_ARGUMENT, "null argument: " #p)
+
+mxconv_status copyOut(const std::string &text, char *buffer, size_t capacity,
+                      size_t *needed) {
+  if (needed)
+    *needed = text.size() + 1;
+  if (buffer && capacity) {
+    const size_t n = std::min(capacity - 1, text.size());
+    std::memcpy(buffer, text.data(), n);
+    buffer[n] = '\0';
+  }
+  if (buffer && capacity < text.size() + 1)
+    return fail(MXCONV_BUFFER_TOO_SMALL, "text truncated");
+  return MXCONV_OK;
+}
+
+std::vector<std::pair<std::string, std::string>>
+collectOptions(const char *const *keys, const char *const *values, size_t n) {
+  std::vector<std::pair<std::string, std::string>> flags;
+  for (size_t i = 0; i != n; ++i) {
+    if (!keys || !values || !keys[i] || !values[i])
+      throw poplar::invalid_option("null option key or value");
+    flags.emplace_back(keys[i], values[i]);
+  }
+  return flags;
+}
+
+mxconv_status hipStatus(hipError_t e, const char *what) {
+  if (e == hipSuccess)
+    return MXCONV_OK;
+  std::string message = std::string(what) + ": " + hipGetErrorString(e);
+  return fail(e == hipErrorOutOfMemory ? MXCONV_OUT_OF_MEMORY
+                                       : MXCONV_HIP_ERROR,
+              message);
+}
+
+void checkDim(const poplin::ConvParams &p, uint32_t dim) {
+  if (dim >= p.getNumFieldDims())
+    throw poputil::poplibs_error("dimension " + std::to_string(dim) +
+                                 " out of range");
+}
+
+mxk::QuarterInfo quarterInfo(uint8_t inMeta, uint8_t wMeta) {
+  auto scaleOf = [](uint8_t m) {
+    int s = m & 0x3f;
+    return (s & 0x20) ? s - 64 : s;
+  };
+  mxk::QuarterInfo q;
+  q.inFormat = (inMeta >> 7) & 1;
+  q.weightFormat = (wMeta >> 7) & 1;
+  q.scale = std::ldexp(1.0f, scaleOf(inMeta) + scaleOf(wMeta));
+  return q;
+}
+
+mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
+                      const void *bias, void *out, void *workspace,
+                      size_t workspaceBytes, const mxk::QuarterInfo &q,
+                      mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  if (plan->outputElems == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(out);
+  if (plan->inputElems != 0)
+    REQUIRE_ARG(in);
+  if (plan->weightElems != 0)
+    REQUIRE_ARG(w);
+  if (workspaceBytes < plan->workspaceBytes ||
+      (plan->workspaceBytes && !workspace))
+    return fail(MXCONV_WORKSPACE_TOO_SMALL,
+                "workspace of " + std::to_string(plan->workspaceBytes) +
+                    " bytes required");
+  const int inType = plan->params.inputType.id();
+  const int outType = plan->params.outputType.id();
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  switch (plan->kernel) {
+  case mxconv_plan::Kernel::IGEMM:
+    return hipStatus(mxk::launchIgemm(plan->igemm, inType, outType, in, w,
+                                      bias, out, q, s),
+                     "implicit-GEMM convolution launch");
+  case mxconv_plan::Kernel::DEPTHWISE:
+    return hipStatus(mxk::launchDepthwise(plan->depthwise, inType, outType, in,
+                                          w, bias, out, s),
+                     "depthwise convolution launch");
+  case mxconv_plan::Kernel::GENERIC:
+    break;
+  }
+  return hipStatus(mxk::launchGeneric(plan->generic, inType, outType, in, w,
+                                      bias, out, q, s),
+                   "generic convolution launch");
+}
+
+} // namespace
+
+extern "C" {
+
+const char *mxconv_last_error(void) { return lastError.c_str(); }
+
+const char *mxconv_status_string(mxconv_status status) {
+  switch (status) {
+  case MXCONV_OK:
+    return "ok";
+  case MXCONV_INVALID_PARAMS:
+    return "invalid parameters";
+  case MXCONV_INVALID_OPTION:
+    return "invalid option";
+  case MXCONV_UNSUPPORTED:
+    return "unsupported";
+  case MXCONV_OUT_OF_MEMORY:
+    return "out of memory";
+  case MXCONV_WORKSPACE_TOO_SMALL:
+    return "workspace too small";
+  case MXCONV_BUFFER_TOO_SMALL:
+    return "buffer too small";
+  case MXCONV_HIP_ERROR:
+    return "HIP error";
+  case MXCONV_NULL_ARGUMENT:
+    return "null argument";
+  }
+  return "unknown status";
+}
+
+mxconv_status mxconv_params_init(mxconv_params *p, int32_t input_type,
+                                 int32_t output_type, uint64_t batch_size,
+                                 uint32_t num_field_dims,
+                                 const uint64_t *input_field_shape,
+                                 const uint64_t *kernel_shape,
+                                 uint64_t input_channels_per_conv_group,
+                                 uint64_t output_channels_per_conv_group,
+                                 uint64_t num_conv_groups) {
+  REQUIRE_ARG(p);
+  return guarded([&] {
+    if (num_field_dims > MXCONV_MAX_FIELD_DIMS)
+      throw poputil::poplibs_error("too many field dimensions");
+    if (num_field_dims && (!input_field_shape || !kernel_shape))
+      throw poputil::poplibs_error("null shape");
+    if (input_type < 0 || input_type > 2 || output_type < 0 || output_type > 2)
+      throw poputil::poplibs_error("unknown element type id");
+    poplin::ConvParams cp(
+        poplar::Type(input_type), poplar::Type(output_type), batch_size,
+        std::vector<std::size_t>(input_field_shape,
+                                 input_field_shape + num_field_dims),
+        std::vector<std::size_t>(kernel_shape, kernel_shape + num_field_dims),
+        input_channels_per_conv_group, output_channels_per_conv_group,
+        num_conv_groups);
+    cp.toC(*p);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_validate(const mxconv_params *p) {
+  REQUIRE_ARG(p);
+  return guarded([&] {
+    poplin::ConvParams::fromC(*p).validate();
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_canonicalize(const mxconv_params *p,
+                                         mxconv_params *canonical) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(canonical);
+  return guarded([&] {
+    poplin::ConvParams::fromC(*p).canonicalize().toC(*canonical);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_is_zero_convolution(const mxconv_params *p,
+                                                int *is_zero) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(is_zero);
+  return guarded([&] {
+    *is_zero =
+        poplin::isZeroConvolution(poplin::ConvParams::fromC(*p).canonicalize());
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_size(const mxconv_params *p, int32_t query,
+                                 uint32_t dim, uint64_t *size) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(size);
+  return guarded([&] {
+    const auto cp = poplin::ConvParams::fromC(*p);
+    cp.validate();
+    checkDim(cp, dim);
+    switch (query) {
+    case MXCONV_TRUNCATED_INPUT_SIZE:
+      *size = cp.getTruncatedInputSize(dim);
+      break;
+    case MXCONV_TRUNCATED_KERNEL_SIZE:
+      *size = cp.getTruncatedKernelSize(dim);
+      break;
+    case MXCONV_TRANSFORMED_INPUT_SIZE:
+      *size = cp.getTransformedInputSize(dim);
+      break;
+    case MXCONV_TRANSFORMED_KERNEL_SIZE:
+      *size = cp.getTransformedKernelSize(dim);
+      break;
+    case MXCONV_UNTRANSFORMED_OUTPUT_SIZE:
+      *size = cp.getUntransformedOutputSize(dim);
+      break;
+    case MXCONV_OUTPUT_SIZE:
+      *size = cp.getOutputSize(dim);
+      break;
+    default:
+      throw poputil::poplibs_error("unknown size query");
+    }
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_compare(const mxconv_params *a,
+                                    const mxconv_params *b, int *order) {
+  REQUIRE_ARG(a);
+  REQUIRE_ARG(b);
+  REQUIRE_ARG(order);
+  return guarded([&] {
+    const auto pa = poplin::ConvParams::fromC(*a);
+    const auto pb = poplin::ConvParams::fromC(*b);
+    *order = pa < pb ? -1 : (pa == pb ? 0 : 1);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_hash(const mxconv_params *p, uint64_t *hash) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(hash);
+  return guarded([&] {
+    *hash = std::hash<poplin::ConvParams>()(poplin::ConvParams::fromC(*p));
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_from_json(const char *json, mxconv_params *p) {
+  REQUIRE_ARG(json);
+  REQUIRE_ARG(p);
+  return guarded([&] {
+    std::istringstream is(json);
+    poplin::ConvParams cp;
+    is >> cp;
+    cp.toC(*p);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_params_to_string(const mxconv_params *p, char *buffer,
+                                      size_t capacity, size_t *needed) {
+  REQUIRE_ARG(p);
+  return guarded([&] {
+    const auto cp = poplin::ConvParams::fromC(*p);
+    cp.validate();
+    std::ostringstream os;
+    os << cp;
+    return copyOut(os.str(), buffer, capacity, needed);
+  });
+}
+
+mxconv_status mxconv_get_input_index(const mxconv_params *p, uint32_t dim,
+                                     uint32_t output_index,
+                                     uint32_t kernel_index, uint32_t *index) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(index);
+  return guarded([&] {
+    const auto cp = poplin::ConvParams::fromC(*p);
+    cp.validate();
+    checkDim(cp, dim);
+    if (output_index >= cp.getOutputSize(dim) ||
+        kernel_index >= cp.kernelShape[dim])
+      throw poputil::poplibs_error("index out of range");
+    *index = poplin::getInputIndex(dim, output_index, kernel_index, cp);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_get_kernel_index(const mxconv_params *p, uint32_t dim,
+                                      uint32_t output_index,
+                                      uint32_t input_index, uint32_t *index) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(index);
+  return guarded([&] {
+    const auto cp = poplin::ConvParams::fromC(*p);
+    cp.validate();
+    checkDim(cp, dim);
+    if (output_index >= cp.getOutputSize(dim) ||
+        input_index >= cp.inputFieldShape[dim])
+      throw poputil::poplibs_error("index out of range");
+    *index = poplin::getKernelIndex(dim, output_index, input_index, cp);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_get_range(const mxconv_params *p, int32_t query,
+                               uint32_t dim, const uint32_t a[2],
+                               const uint32_t b[2], uint32_t result[2]) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(a);
+  REQUIRE_ARG(b);
+  REQUIRE_ARG(result);
+  return guarded([&] {
+    const auto cp = poplin::ConvParams::fromC(*p);
+    cp.validate();
+    checkDim(cp, dim);
+    const unsigned outSize = unsigned(cp.getOutputSize(dim));
+    const unsigned inSize = unsigned(cp.inputFieldShape[dim]);
+    const unsigned kSize = unsigned(cp.kernelShape[dim]);
+    auto check = [](const uint32_t r[2], unsigned limit, const char *what) {
+      if (r[0] > r[1] || r[1] > limit)
+        throw poputil::poplibs_error(std::string(what) + " range out of bounds");
+    };
+    check(a, outSize, "output");
+    poplin::Range r;
+    switch (query) {
+    case MXCONV_OUTPUT_RANGE_FOR_KERNEL_RANGE:
+      check(b, kSize, "kernel");
+      r = poplin::getOutputRangeForKernelRange(dim, {a[0], a[1]}, {b[0], b[1]},
+                                               cp);
+      break;
+    case MXCONV_OUTPUT_RANGE_FOR_INPUT_RANGE:
+      check(b, inSize, "input");
+      r = poplin::getOutputRangeForInputRange(dim, {a[0], a[1]}, {b[0], b[1]},
+                                              cp);
+      break;
+    case MXCONV_INPUT_RANGE:
+      check(b, kSize, "kernel");
+      r = poplin::getInputRange(dim, poplin::Range{a[0], a[1]},
+                                poplin::Range{b[0], b[1]}, cp);
+      break;
+    case MXCONV_KERNEL_RANGE:
+      check(b, inSize, "input");
+      r = poplin::getKernelRange(dim, poplin::Range{a[0], a[1]},
+                                 poplin::Range{b[0], b[1]}, cp);
+      break;
+    default:
+      throw poputil::poplibs_error("unknown range query");
+    }
+    result[0] = r.first;
+    result[1] = r.second;
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_get_number_of_macs(const mxconv_params *p,
+                                        uint64_t *macs) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(macs);
+  return guarded([&] {
+    const auto cp = poplin::ConvParams::fromC(*p);
+    cp.validate();
+    *macs = poplin::getNumberOfMACs(cp);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_get_fwd_flops(const mxconv_params *p, uint64_t *flops) {
+  REQUIRE_ARG(flops);
+  uint64_t macs = 0;
+  const mxconv_status s = mxconv_get_number_of_macs(p, &macs);
+  if (s == MXCONV_OK)
+    *flops = 2 * macs;
+  return s;
+}
+
+mxconv_status mxconv_validate_options(const char *const *keys,
+                                      const char *const *values,
+                                      size_t num_options) {
+  return guarded([&] {
+    poplin::ConvOptions options(collectOptions(keys, values, num_options));
+    (void)options;
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_plan_create(const mxconv_params *p,
+                                 const char *const *option_keys,
+                                 const char *const *option_values,
+                                 size_t num_options, mxconv_plan **plan) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(plan);
+  *plan = nullptr;
+  return guarded([&] {
+    poplin::ConvOptions options(
+        collectOptions(option_keys, option_values, num_options));
+    *plan = new mxconv_plan(
+        poplin::makePlan(poplin::ConvParams::fromC(*p), options));
+    return MXCONV_OK;
+  });
+}
+
+void mxconv_plan_destroy(mxconv_plan *plan) { delete plan; }
+
+mxconv_status mxconv_plan_describe(const mxconv_plan *plan, char *buffer,
+                                   size_t capacity, size_t *needed) {
+  REQUIRE_ARG(plan);
+  return guarded([&] {
+    std::ostringstream os;
+    os << plan->params << plan->describe();
+    return copyOut(os.str(), buffer, capacity, needed);
+  });
+}
+
+mxconv_status mxconv_plan_buffer_bytes(const mxconv_plan *plan, int32_t which,
+                                       size_t *bytes) {
+  REQUIRE_ARG(plan);
+  REQUIRE_ARG(bytes);
+  lastError.clear();
+  switch (which) {
+  case MXCONV_BUFFER_INPUT:
+    *bytes = plan->inputBytes();
+    return MXCONV_OK;
+  case MXCONV_BUFFER_WEIGHTS_PACKED:
+    *bytes = plan->weightPackedBytes();
+    return MXCONV_OK;
+  case MXCONV_BUFFER_OUTPUT:
+    *bytes = plan->outputBytes();
+    return MXCONV_OK;
+  case MXCONV_BUFFER_BIAS:
+    *bytes = plan->biasBytes();
+    return MXCONV_OK;
+  case MXCONV_BUFFER_WORKSPACE:
+    *bytes = plan->workspaceBytes;
+    return MXCONV_OK;
+  case MXCONV_BUFFER_WEIGHTS_EXTERNAL:
+    *bytes = plan->weightBytes();
+    return MXCONV_OK;
+  }
+  return fail(MXCONV_INVALID_PARAMS, "unknown buffer id");
+}
+
+mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
+                                  const void *weights_external,
+                                  void *weights_packed, mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  if (plan->weightPackedElems == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(weights_packed);
+  const auto &p = plan->params;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int elemBytes = int(p.inputType.size());
+  uint64_t taps = 1;
+  for (auto k : p.kernelShape)
+    taps *= k;
+  if (plan->kernel == mxconv_plan::Kernel::IGEMM) {
+    if (plan->weightElems != 0)
+      REQUIRE_ARG(weights_external);
+    return hipStatus(
+        mxk::launchPackIgemmWeights(
+            weights_external, weights_packed, uint32_t(p.numConvGroups),
+            uint32_t(p.outputChannelsPerConvGroup),
+            uint32_t(p.inputChannelsPerConvGroup), uint32_t(taps),
+            uint32_t(plan->coPadded), uint32_t(plan->kPadded), elemBytes, s),
+        "weight packing");
+  }
+  REQUIRE_ARG(weights_external);
+  // [G][Co][Ci][K] -> [G][K][Ci][Co]; with Co = Ci = 1 this is also the
+  // depthwise kernel's [K][C].
+  const uint64_t dims[4] = {p.numConvGroups, p.outputChannelsPerConvGroup,
+                            p.inputChannelsPerConvGroup, taps};
+  if (plan->kernel == mxconv_plan::Kernel::DEPTHWISE) {
+    const uint64_t dwDims[4] = {1, 1, p.numConvGroups, taps};
+    const int perm[4] = {0, 1, 3, 2};
+    return hipStatus(mxk::launchPermute4(weights_external, weights_packed,
+                                         dwDims, perm, elemBytes, s),
+                     "weight packing");
+  }
+  const int perm[4] = {0, 3, 2, 1};
+  return hipStatus(mxk::launchPermute4(weights_external, weights_packed, dims,
+                                       perm, elemBytes, s),
+                   "weight packing");
+}
+
+static mxconv_status transposeActs(const mxconv_plan *plan, const void *src,
+                                   void *dst, bool input, bool toInternal,
+                                   mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  const auto &p = plan->params;
+  uint64_t field = 1;
+  if (input)
+    for (auto s : p.inputFieldShape)
+      field *= s;
+  else
+    for (auto s : p.getOutputFieldShape())
+      field *= s;
+  const uint64_t chans = input ? p.getNumInputChans() : p.getNumOutputChans();
+  if (p.batchSize * field * chans == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(src);
+  REQUIRE_ARG(dst);
+  const int elemBytes = int((input ? p.inputType : p.outputType).size());
+  const int perm[4] = {0, 1, 3, 2};
+  uint64_t dims[4] = {1, p.batchSize, chans, field};
+  if (!toInternal)
+    std::swap(dims[2], dims[3]);
+  return hipStatus(mxk::launchPermute4(src, dst, dims, perm, elemBytes,
+                                       reinterpret_cast<hipStream_t>(stream)),
+                   "activation layout conversion");
+}
+
+mxconv_status mxconv_acts_to_internal(const mxconv_plan *plan,
+                                      const void *acts_external,
+                                      void *acts_internal,
+                                      mxconv_stream stream) {
+  return transposeActs(plan, acts_external, acts_internal, true, true, stream);
+}
+
+mxconv_status mxconv_acts_to_external(const mxconv_plan *plan,
+                                      const void *out_internal,
+                                      void *out_external,
+                                      mxconv_stream stream) {
+  return transposeActs(plan, out_internal, out_external, false, false, stream);
+}
+
+mxconv_status mxconv_fwd(const mxconv_plan *plan, const void *in,
+                         const void *weights_packed, const void *bias,
+                         void *out, void *workspace, size_t workspace_bytes,
+                         mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  if (plan->params.inputType == poplar::QUARTER)
+    return fail(MXCONV_INVALID_PARAMS,
+                "quarter inputs carry metadata: call mxconv_fwd_quarter");
+  return forward(plan, in, weights_packed, bias, out, workspace,
+                 workspace_bytes, mxk::QuarterInfo{}, stream);
+}
+
+mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
+                                 uint8_t in_metadata,
+                                 const void *weights_packed,
+                                 uint8_t weights_metadata, const void *bias,
+                                 void *out, void *workspace,
+                                 size_t workspace_bytes, mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  if (plan->params.inputType != poplar::QUARTER)
+    return fail(MXCONV_INVALID_PARAMS,
+                "mxconv_fwd_quarter needs a plan with quarter inputs");
+  return forward(plan, in, weights_packed, bias, out, workspace,
+                 workspace_bytes, quarterInfo(in_metadata, weights_metadata),
+                 stream);
+}
+
+mxconv_status mxconv_add_bias(int32_t type, void *acts_internal,
+                              const void *bias, uint64_t outer_elems,
+                              uint64_t channels, mxconv_stream stream) {
+  lastError.clear();
+  if (outer_elems * channels == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(acts_internal);
+  REQUIRE_ARG(bias);
+  if (type != MXCONV_HALF && type != MXCONV_FLOAT)
+    return fail(MXCONV_INVALID_PARAMS, "bias add takes half or float tensors");
+  return hipStatus(mxk::launchAddBias(type, acts_internal, bias, outer_elems,
+                                      channels,
+                                      reinterpret_cast<hipStream_t>(stream)),
+                   "bias add");
+}
+
+} // extern "C"

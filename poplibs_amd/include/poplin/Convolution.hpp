@@ -1,0 +1,154 @@
+// poplin's forward-convolution entry points for the MI355X build.
+//
+// The functions keep the names, argument order and error behaviour of
+// PopLibs' include/poplin/Convolution.hpp; what changes is what they act on.
+// PopLibs appends vertices to a poplar::Graph and a program::Sequence that an
+// Engine runs later; here a tensor is a device buffer (DeviceTensor), a
+// "program" is a HIP stream (Stream) on which the work is enqueued at once,
+// and the graph / debug-context arguments are gone.  All GPU work goes through
+// the C ABI of mxconv.h.
+#ifndef poplibs_amd_poplin_Convolution_hpp
+#define poplibs_amd_poplin_Convolution_hpp
+#include "poplar/OptionFlags.hpp"
+#include "poplar/Type.hpp"
+#include "poplin/ConvParams.hpp"
+
+#include <cstddef>
+#include <cstdint>
+#include <iosfwd>
+#include <memory>
+#include <vector>
+
+struct mxconv_plan;
+
+namespace poplin {
+
+/// Stands in for poplar::program::Sequence: work is enqueued on this stream
+/// in call order.  Owns the stream unless constructed from an existing one.
+class Stream {
+  struct Impl;
+  std::shared_ptr<Impl> impl_;
+
+public:
+  Stream();                        ///< creates a new stream
+  explicit Stream(void *hipStream); ///< wraps an existing hipStream_t
+  void *handle() const;
+  void synchronize() const; ///< blocks until everything enqueued has run
+};
+
+/// FP8 tensors carry a format and a power-of-two scale
+/// (poplar::QuarterMetadata in the Poplar SDK).
+struct QuarterMetadata {
+  enum class Format { F152 = 0, F143 = 1 };
+  Format format = Format::F143;
+  int scale = 0; ///< value = fp8 * 2^scale, -32..31
+  std::uint8_t byte() const {
+    return std::uint8_t((unsigned(format) << 7) | (unsigned(scale) & 0x3f));
+  }
+};
+
+/// Stands in for poplar::Tensor: a reference-counted device buffer with the
+/// logical (external) shape of the reference API and a tag for the physical
+/// layout it is held in.
+class DeviceTensor {
+public:
+  enum class Layout {
+    External,      ///< row-major in the logical shape
+    ChannelsLast,  ///< activations [B][field...][C]
+    PackedWeights  ///< weights as packed for one plan
+  };
+  DeviceTensor() = default;
+  /// Allocates `bytes` of device memory; throws
+  /// poplar::graph_memory_allocation_error when the device is out of memory.
+  DeviceTensor(poplar::Type type, std::vector<std::size_t> shape,
+               Layout layout, std::size_t bytes);
+
+  bool valid() const { return bool(buffer_); }
+  poplar::Type elementType() const { return type_; }
+  const std::vector<std::size_t> &shape() const { return shape_; }
+  std::size_t numElements() const;
+  std::size_t bytes() const { return bytes_; }
+  Layout layout() const { return layout_; }
+  void *data() const { return buffer_.get(); }
+  QuarterMetadata metadata; ///< meaningful for QUARTER tensors only
+
+private:
+  poplar::Type type_;
+  std::vector<std::size_t> shape_;
+  Layout layout_ = Layout::External;
+  std::size_t bytes_ = 0;
+  std::shared_ptr<void> buffer_;
+};
+
+/// Memo of plans keyed by (parameters, options); safe to share between
+/// threads (include/poplin/Convolution.hpp:724-733).
+class PlanningCache {
+public:
+  PlanningCache();
+  ~PlanningCache();
+  std::size_t size() const;
+  struct Impl;
+  std::unique_ptr<Impl> impl;
+};
+
+std::uint64_t getFwdFlops(const ConvParams &params);
+
+/// Weights [convGroups][outChansPerGroup][inChansPerGroup][kernel...], held
+/// packed for the plan of (params, options).
+DeviceTensor createWeights(const ConvParams &params,
+                           const poplar::OptionFlags &options = {},
+                           PlanningCache *cache = nullptr);
+/// Biases [outChans] in the activations' element type.
+DeviceTensor createBiases(const DeviceTensor &activations);
+DeviceTensor createBiases(const ConvParams &params,
+                          const poplar::OptionFlags &options = {},
+                          PlanningCache *cache = nullptr);
+/// Input [B][inChans][field...], held channels-last.
+DeviceTensor createInput(const ConvParams &params,
+                         const poplar::OptionFlags &options = {},
+                         PlanningCache *cache = nullptr);
+/// Output [B][outChans][outField...], held channels-last.
+DeviceTensor createConvOutput(const ConvParams &params,
+                              const poplar::OptionFlags &options = {},
+                              PlanningCache *cache = nullptr);
+
+/// Convolve `in` with `weights`; returns the output tensor.  Tensors in
+/// External layout are converted on the device first.
+/// transposeAndFlipWeights (the backward-pass weight view) is not part of the
+/// forward path and raises poputil::poplibs_error when true.
+DeviceTensor convolution(const DeviceTensor &in, const DeviceTensor &weights,
+                         const ConvParams &params,
+                         bool transposeAndFlipWeights, Stream &prog,
+                         const poplar::OptionFlags &options = {},
+                         PlanningCache *cache = nullptr);
+
+void convolutionWithOutput(const DeviceTensor &in, const DeviceTensor &weights,
+                           const DeviceTensor &out, const ConvParams &params,
+                           bool transposeAndFlipWeights, Stream &prog,
+                           const poplar::OptionFlags &options = {},
+                           PlanningCache *cache = nullptr);
+
+/// acts[b][c][...] += biases[c].
+void addBias(const DeviceTensor &in, const DeviceTensor &biases, Stream &prog);
+
+void reportPlanInfo(std::ostream &out, const ConvParams &params,
+                    const poplar::OptionFlags &options = {},
+                    PlanningCache *cache = nullptr);
+
+/// Throws poplar::invalid_option for an unknown key or value.
+void convolutionValidateOptions(const poplar::OptionFlags &options);
+
+/// Host <-> device transfer in the tensor's logical (external) layout and
+/// element type: the role of Engine::writeTensor / readTensor.  `params` and
+/// `options` select the plan whose packing a PackedWeights tensor uses.
+void writeTensor(const DeviceTensor &t, const void *host, Stream &prog,
+                 const ConvParams &params,
+                 const poplar::OptionFlags &options = {},
+                 PlanningCache *cache = nullptr);
+void readTensor(const DeviceTensor &t, void *host, Stream &prog,
+                const ConvParams &params,
+                const poplar::OptionFlags &options = {},
+                PlanningCache *cache = nullptr);
+
+} // namespace poplin
+#endif

@@ -1,0 +1,61 @@
+// Options of a convolution: the string key/value pairs of a
+// poplar::OptionFlags, checked as PopLibs checks them
+// (lib/poplin/ConvOptions.cpp:105-152, 193-329) and reduced to what the gfx950
+// planner uses.
+#ifndef poplibs_amd_ConvOptions_hpp
+#define poplibs_amd_ConvOptions_hpp
+#include "Json.hpp"
+#include "poplar/Type.hpp"
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace poplin {
+
+enum class Pass {
+  NONE,
+  NONE_MATMUL,
+  INFERENCE_FWD,
+  TRAINING_FWD,
+  TRAINING_BWD,
+  TRAINING_WU,
+  FC_INFERENCE_FWD,
+  FC_TRAINING_FWD,
+  FC_TRAINING_BWD,
+  FC_TRAINING_WU
+};
+const char *toString(Pass p);
+
+/// What planConstraints may pin for this build.  The PopLibs method names are
+/// mapped onto the gfx950 kernels that take over their role.
+struct PlanConstraints {
+  enum class Method { ANY, AMP, SLIC, HMAC, VMAC, OUTER_PRODUCT };
+  Method method = Method::ANY;
+  /// "gfx950" section: force a kernel ("generic", "igemm", "depthwise") and
+  /// tile extents; 0 / empty = planner's choice.
+  std::string kernel;
+  unsigned blockM = 0, blockN = 0, blockK = 0;
+  std::string text; // the JSON as given, kept for reporting and cache keys
+};
+
+class ConvOptions {
+public:
+  double availableMemoryProportion = .6;
+  Pass pass = Pass::NONE;
+  poplar::Type partialsType = poplar::FLOAT;
+  poplar::Type interTilePartialsType = poplar::FLOAT;
+  poplar::Type interIpuPartialsType = poplar::FLOAT;
+  PlanConstraints planConstraints;
+  std::string planConstraintsOutputFilename;
+
+  ConvOptions() = default;
+  /// Throws poplar::invalid_option on an unknown key or a malformed value.
+  explicit ConvOptions(
+      const std::vector<std::pair<std::string, std::string>> &flags);
+
+  /// Stable text form, used in plan-cache keys.
+  std::string key() const;
+};
+
+} // namespace poplin
+#endif

@@ -1,0 +1,437 @@
+// The C++ poplin entry points, written over the C ABI of mxconv.h.  Device
+// memory and host transfers use the HIP runtime directly; every kernel launch
+// goes through an mxconv_* call.
+#include "poplin/Convolution.hpp"
+#include "mxconv.h"
+#include "poplar/exceptions.hpp"
+#include "poputil/exceptions.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <map>
+#include <mutex>
+#include <ostream>
+#include <string>
+#include <tuple>
+
+namespace poplin {
+
+namespace {
+
+[[noreturn]] void raise(mxconv_status s) {
+  const std::string message = mxconv_last_error();
+  switch (s) {
+  case MXCONV_INVALID_OPTION:
+    throw poplar::invalid_option(message);
+  case MXCONV_OUT_OF_MEMORY:
+    throw poplar::graph_memory_allocation_error(message);
+  default:
+    throw poputil::poplibs_error(message.empty() ? mxconv_status_string(s)
+                                                 : message);
+  }
+}
+void check(mxconv_status s) {
+  if (s != MXCONV_OK)
+    raise(s);
+}
+void checkHip(hipError_t e, const char *what) {
+  if (e == hipSuccess)
+    return;
+  const std::string message = std::string(what) + ": " + hipGetErrorString(e);
+  if (e == hipErrorOutOfMemory)
+    throw poplar::graph_memory_allocation_error(message);
+  throw poputil::poplibs_error(message);
+}
+
+struct PlanHandle {
+  mxconv_plan *plan = nullptr;
+  explicit PlanHandle(mxconv_plan *p) : plan(p) {}
+  ~PlanHandle() { mxconv_plan_destroy(plan); }
+  PlanHandle(const PlanHandle &) = delete;
+  PlanHandle &operator=(const PlanHandle &) = delete;
+};
+
+std::shared_ptr<PlanHandle> createPlan(const ConvParams &params,
+                                       const poplar::OptionFlags &options) {
+  mxconv_params c;
+  params.toC(c);
+  std::vector<const char *> keys, values;
+  for (const auto &kv : options) {
+    keys.push_back(kv.first.c_str());
+    values.push_back(kv.second.c_str());
+  }
+  mxconv_plan *plan = nullptr;
+  check(mxconv_plan_create(&c, keys.data(), values.data(), keys.size(), &plan));
+  return std::make_shared<PlanHandle>(plan);
+}
+
+std::size_t bufferBytes(const mxconv_plan *plan, mxconv_buffer which) {
+  std::size_t bytes = 0;
+  check(mxconv_plan_buffer_bytes(plan, which, &bytes));
+  return bytes;
+}
+
+std::vector<std::size_t> actsShape(std::size_t batch, std::size_t chans,
+                                   const std::vector<std::size_t> &field) {
+  std::vector<std::size_t> shape{batch, chans};
+  shape.insert(shape.end(), field.begin(), field.end());
+  return shape;
+}
+
+mxconv_stream streamOf(const Stream &s) {
+  return static_cast<mxconv_stream>(s.handle());
+}
+
+} // namespace
+
+// ---- Stream ---------------------------------------------------------------
+
+struct Stream::Impl {
+  hipStream_t stream = nullptr;
+  bool owned = false;
+  ~Impl() {
+    if (owned && stream)
+      (void)hipStreamDestroy(stream);
+  }
+};
+
+Stream::Stream() : impl_(std::make_shared<Impl>()) {
+  checkHip(hipStreamCreate(&impl_->stream), "hipStreamCreate");
+  impl_->owned = true;
+}
+Stream::Stream(void *hipStream) : impl_(std::make_shared<Impl>()) {
+  impl_->stream = static_cast<hipStream_t>(hipStream);
+}
+void *Stream::handle() const { return impl_->stream; }
+void Stream::synchronize() const {
+  checkHip(hipStreamSynchronize(impl_->stream), "hipStreamSynchronize");
+}
+
+// ---- DeviceTensor ---------------------------------------------------------
+
+DeviceTensor::DeviceTensor(poplar::Type type, std::vector<std::size_t> shape,
+                           Layout layout, std::size_t bytes)
+    : type_(type), shape_(std::move(shape)), layout_(layout), bytes_(bytes) {
+  void *p = nullptr;
+  // A zero-sized tensor still gets a distinct, valid allocation.
+  checkHip(hipMalloc(&p, bytes ? bytes : 1), "hipMalloc");
+  buffer_ = std::shared_ptr<void>(p, [](void *q) { (void)hipFree(q); });
+}
+
+std::size_t DeviceTensor::numElements() const {
+  std::size_t n = 1;
+  for (auto s : shape_)
+    n *= s;
+  return n;
+}
+
+// ---- PlanningCache --------------------------------------------------------
+
+struct PlanningCache::Impl {
+  using Key = std::pair<ConvParams, poplar::OptionFlags>;
+  std::mutex mutex;
+  std::map<Key, std::shared_ptr<PlanHandle>> plans;
+};
+PlanningCache::PlanningCache() : impl(new Impl) {}
+PlanningCache::~PlanningCache() = default;
+std::size_t PlanningCache::size() const {
+  std::lock_guard<std::mutex> lock(impl->mutex);
+  return impl->plans.size();
+}
+
+namespace {
+std::shared_ptr<PlanHandle> getPlan(const ConvParams &params,
+                                    const poplar::OptionFlags &options,
+                                    PlanningCache *cache) {
+  if (!cache)
+    return createPlan(params, options);
+  // Plans are keyed by the canonical parameters, as in PopLibs, so that
+  // descriptors which differ only in unused padding share a plan.  The
+  // caller-visible tensor shapes are identical for both.
+  const PlanningCache::Impl::Key key{params.canonicalize(), options};
+  std::lock_guard<std::mutex> lock(cache->impl->mutex);
+  auto it = cache->impl->plans.find(key);
+  if (it != cache->impl->plans.end())
+    return it->second;
+  auto plan = createPlan(params, options);
+  cache->impl->plans.emplace(key, plan);
+  return plan;
+}
+} // namespace
+
+// ---- entry points ---------------------------------------------------------
+
+std::uint64_t getFwdFlops(const ConvParams &params) {
+  mxconv_params c;
+  params.toC(c);
+  std::uint64_t flops = 0;
+  check(mxconv_get_fwd_flops(&c, &flops));
+  return flops;
+}
+
+DeviceTensor createWeights(const ConvParams &params,
+                           const poplar::OptionFlags &options,
+                           PlanningCache *cache) {
+  auto plan = getPlan(params, options, cache);
+  std::vector<std::size_t> shape{params.numConvGroups,
+                                 params.outputChannelsPerConvGroup,
+                                 params.inputChannelsPerConvGroup};
+  shape.insert(shape.end(), params.kernelShape.begin(),
+               params.kernelShape.end());
+  return DeviceTensor(params.inputType, shape,
+                      DeviceTensor::Layout::PackedWeights,
+                      bufferBytes(plan->plan, MXCONV_BUFFER_WEIGHTS_PACKED));
+}
+
+DeviceTensor createBiases(const DeviceTensor &acts) {
+  if (acts.shape().size() < 2)
+    throw poputil::poplibs_error("createBiases: activations need at least "
+                                 "batch and channel dimensions");
+  const std::size_t chans = acts.shape()[1];
+  return DeviceTensor(acts.elementType(), {chans},
+                      DeviceTensor::Layout::External,
+                      chans * acts.elementType().size());
+}
+
+DeviceTensor createBiases(const ConvParams &params,
+                          const poplar::OptionFlags &options,
+                          PlanningCache *cache) {
+  auto plan = getPlan(params, options, cache);
+  return DeviceTensor(params.outputType, {params.getNumOutputChans()},
+                      DeviceTensor::Layout::External,
+                      bufferBytes(plan->plan, MXCONV_BUFFER_BIAS));
+}
+
+DeviceTensor createInput(const ConvParams &params,
+                         const poplar::OptionFlags &options,
+                         PlanningCache *cache) {
+  auto plan = getPlan(params, options, cache);
+  return DeviceTensor(params.inputType,
+                      actsShape(params.batchSize, params.getNumInputChans(),
+                                params.inputFieldShape),
+                      DeviceTensor::Layout::ChannelsLast,
+                      bufferBytes(plan->plan, MXCONV_BUFFER_INPUT));
+}
+
+DeviceTensor createConvOutput(const ConvParams &params,
+                              const poplar::OptionFlags &options,
+                              PlanningCache *cache) {
+  auto plan = getPlan(params, options, cache);
+  return DeviceTensor(params.outputType,
+                      actsShape(params.batchSize, params.getNumOutputChans(),
+                                params.getOutputFieldShape()),
+                      DeviceTensor::Layout::ChannelsLast,
+                      bufferBytes(plan->plan, MXCONV_BUFFER_OUTPUT));
+}
+
+namespace {
+
+/// verifyInputShapesAndTypes (lib/poplin/Convolution.cpp:105-162).
+void verify(const ConvParams &params, const DeviceTensor &in,
+            const DeviceTensor &weights, const DeviceTensor *out) {
+  const auto expectIn = actsShape(params.batchSize, params.getNumInputChans(),
+                                  params.inputFieldShape);
+  if (in.shape() != expectIn)
+    throw poputil::poplibs_error(
+        "Input tensor shape does not match the convolution parameters");
+  std::vector<std::size_t> expectW{params.numConvGroups,
+                                   params.outputChannelsPerConvGroup,
+                                   params.inputChannelsPerConvGroup};
+  expectW.insert(expectW.end(), params.kernelShape.begin(),
+                 params.kernelShape.end());
+  if (weights.shape() != expectW)
+    throw poputil::poplibs_error(
+        "Weights tensor shape does not match the convolution parameters");
+  if (in.elementType() != params.inputType ||
+      weights.elementType() != params.inputType)
+    throw poputil::poplibs_error("Input and weights element types must equal "
+                                 "the parameters' input type");
+  if (out) {
+    if (out->shape() != actsShape(params.batchSize, params.getNumOutputChans(),
+                                  params.getOutputFieldShape()))
+      throw poputil::poplibs_error(
+          "Output tensor shape does not match the convolution parameters");
+    if (out->elementType() != params.outputType)
+      throw poputil::poplibs_error(
+          "Output element type must equal the parameters' output type");
+  }
+}
+
+void run(const PlanHandle &plan, const ConvParams &params,
+         const DeviceTensor &in, const DeviceTensor &weights,
+         const DeviceTensor &out, Stream &prog) {
+  // Bring operands into the device layouts if the caller holds them in the
+  // external ones (PopLibs rearranges unsuitably laid-out operands the same
+  // way, lib/poplin/Convolution.cpp:2569-2628).
+  DeviceTensor inCl = in, wPacked = weights, outCl = out;
+  if (in.layout() == DeviceTensor::Layout::External) {
+    inCl = DeviceTensor(in.elementType(), in.shape(),
+                        DeviceTensor::Layout::ChannelsLast, in.bytes());
+    check(mxconv_acts_to_internal(plan.plan, in.data(), inCl.data(),
+                                  streamOf(prog)));
+  }
+  if (weights.layout() == DeviceTensor::Layout::External) {
+    wPacked = DeviceTensor(weights.elementType(), weights.shape(),
+                           DeviceTensor::Layout::PackedWeights,
+                           bufferBytes(plan.plan, MXCONV_BUFFER_WEIGHTS_PACKED));
+    check(mxconv_pack_weights(plan.plan, weights.data(), wPacked.data(),
+                              streamOf(prog)));
+  }
+  if (out.layout() == DeviceTensor::Layout::External)
+    outCl = DeviceTensor(out.elementType(), out.shape(),
+                         DeviceTensor::Layout::ChannelsLast, out.bytes());
+  const std::size_t wsBytes = bufferBytes(plan.plan, MXCONV_BUFFER_WORKSPACE);
+  DeviceTensor workspace;
+  if (wsBytes)
+    workspace = DeviceTensor(poplar::FLOAT, {wsBytes / 4},
+                             DeviceTensor::Layout::External, wsBytes);
+  if (params.inputType == poplar::QUARTER)
+    check(mxconv_fwd_quarter(plan.plan, inCl.data(), in.metadata.byte(),
+                             wPacked.data(), weights.metadata.byte(), nullptr,
+                             outCl.data(), workspace.data(), wsBytes,
+                             streamOf(prog)));
+  else
+    check(mxconv_fwd(plan.plan, inCl.data(), wPacked.data(), nullptr,
+                     outCl.data(), workspace.data(), wsBytes, streamOf(prog)));
+  if (out.layout() == DeviceTensor::Layout::External)
+    check(mxconv_acts_to_external(plan.plan, outCl.data(), out.data(),
+                                  streamOf(prog)));
+  // Temporaries are released when this function returns; work already
+  // enqueued on the stream must have finished with them by then.
+  if (inCl.data() != in.data() || wPacked.data() != weights.data() ||
+      outCl.data() != out.data() || wsBytes)
+    prog.synchronize();
+}
+
+} // namespace
+
+void convolutionWithOutput(const DeviceTensor &in, const DeviceTensor &weights,
+                           const DeviceTensor &out, const ConvParams &params,
+                           bool transposeAndFlipWeights, Stream &prog,
+                           const poplar::OptionFlags &options,
+                           PlanningCache *cache) {
+  if (transposeAndFlipWeights)
+    throw poputil::poplibs_error(
+        "transposeAndFlipWeights belongs to the backward pass, which this "
+        "build does not provide");
+  auto plan = getPlan(params, options, cache);
+  verify(params, in, weights, &out);
+  run(*plan, params, in, weights, out, prog);
+}
+
+DeviceTensor convolution(const DeviceTensor &in, const DeviceTensor &weights,
+                         const ConvParams &params,
+                         bool transposeAndFlipWeights, Stream &prog,
+                         const poplar::OptionFlags &options,
+                         PlanningCache *cache) {
+  DeviceTensor out = createConvOutput(params, options, cache);
+  convolutionWithOutput(in, weights, out, params, transposeAndFlipWeights, prog,
+                        options, cache);
+  return out;
+}
+
+void addBias(const DeviceTensor &in, const DeviceTensor &biases, Stream &prog) {
+  if (in.shape().size() < 2 || biases.shape().size() != 1 ||
+      biases.shape()[0] != in.shape()[1])
+    throw poputil::poplibs_error(
+        "addBias: bias must have one element per activation channel");
+  if (in.elementType() != biases.elementType())
+    throw poputil::poplibs_error(
+        "addBias: bias and activations must share an element type");
+  if (in.layout() != DeviceTensor::Layout::ChannelsLast)
+    throw poputil::poplibs_error(
+        "addBias: activations must be held channels-last (createInput / "
+        "createConvOutput / convolution results are)");
+  const std::size_t chans = in.shape()[1];
+  const std::size_t outer = chans ? in.numElements() / chans : 0;
+  check(mxconv_add_bias(in.elementType().id(), in.data(), biases.data(), outer,
+                        chans, streamOf(prog)));
+}
+
+void reportPlanInfo(std::ostream &out, const ConvParams &params,
+                    const poplar::OptionFlags &options, PlanningCache *cache) {
+  auto plan = getPlan(params, options, cache);
+  std::size_t needed = 0;
+  check(mxconv_plan_describe(plan->plan, nullptr, 0, &needed));
+  std::string text(needed, '\0');
+  check(mxconv_plan_describe(plan->plan, &text[0], text.size(), &needed));
+  text.resize(needed - 1);
+  out << text;
+}
+
+void convolutionValidateOptions(const poplar::OptionFlags &options) {
+  std::vector<const char *> keys, values;
+  for (const auto &kv : options) {
+    keys.push_back(kv.first.c_str());
+    values.push_back(kv.second.c_str());
+  }
+  check(mxconv_validate_options(keys.data(), values.data(), keys.size()));
+}
+
+void writeTensor(const DeviceTensor &t, const void *host, Stream &prog,
+                 const ConvParams &params, const poplar::OptionFlags &options,
+                 PlanningCache *cache) {
+  hipStream_t s = static_cast<hipStream_t>(prog.handle());
+  const std::size_t logicalBytes = t.numElements() * t.elementType().size();
+  if (t.layout() == DeviceTensor::Layout::External) {
+    if (logicalBytes)
+      checkHip(hipMemcpyAsync(t.data(), host, logicalBytes,
+                              hipMemcpyHostToDevice, s),
+               "hipMemcpyAsync");
+    prog.synchronize();
+    return;
+  }
+  auto plan = getPlan(params, options, cache);
+  DeviceTensor staging(t.elementType(), t.shape(),
+                       DeviceTensor::Layout::External, logicalBytes);
+  if (logicalBytes)
+    checkHip(hipMemcpyAsync(staging.data(), host, logicalBytes,
+                            hipMemcpyHostToDevice, s),
+             "hipMemcpyAsync");
+  if (t.layout() == DeviceTensor::Layout::PackedWeights) {
+    check(mxconv_pack_weights(plan->plan, staging.data(), t.data(),
+                              streamOf(prog)));
+  } else {
+    if (t.shape() != actsShape(params.batchSize, params.getNumInputChans(),
+                               params.inputFieldShape))
+      throw poputil::poplibs_error(
+          "writeTensor: only the convolution's input can be written in "
+          "channels-last layout");
+    check(mxconv_acts_to_internal(plan->plan, staging.data(), t.data(),
+                                  streamOf(prog)));
+  }
+  prog.synchronize(); // staging is released on return
+}
+
+void readTensor(const DeviceTensor &t, void *host, Stream &prog,
+                const ConvParams &params, const poplar::OptionFlags &options,
+                PlanningCache *cache) {
+  hipStream_t s = static_cast<hipStream_t>(prog.handle());
+  const std::size_t logicalBytes = t.numElements() * t.elementType().size();
+  if (t.layout() == DeviceTensor::Layout::External) {
+    if (logicalBytes)
+      checkHip(hipMemcpyAsync(host, t.data(), logicalBytes,
+                              hipMemcpyDeviceToHost, s),
+               "hipMemcpyAsync");
+    prog.synchronize();
+    return;
+  }
+  if (t.layout() != DeviceTensor::Layout::ChannelsLast ||
+      t.shape() != actsShape(params.batchSize, params.getNumOutputChans(),
+                             params.getOutputFieldShape()))
+    throw poputil::poplibs_error(
+        "readTensor: only the convolution's output can be read back from a "
+        "device layout");
+  auto plan = getPlan(params, options, cache);
+  DeviceTensor staging(t.elementType(), t.shape(),
+                       DeviceTensor::Layout::External, logicalBytes);
+  check(mxconv_acts_to_external(plan->plan, t.data(), staging.data(),
+                                streamOf(prog)));
+  if (logicalBytes)
+    checkHip(hipMemcpyAsync(host, staging.data(), logicalBytes,
+                            hipMemcpyDeviceToHost, s),
+             "hipMemcpyAsync");
+  prog.synchronize();
+}
+
+} // namespace poplin

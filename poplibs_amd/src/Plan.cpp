@@ -1,0 +1,318 @@
+#include "Plan.hpp"
+#include "poplar/exceptions.hpp"
+#include "poplin/ConvUtil.hpp"
+#include "poputil/exceptions.hpp"
+
+#include <algorithm>
+#include <sstream>
+
+namespace poplin {
+
+namespace {
+
+std::size_t product(const std::vector<std::size_t> &v) {
+  std::size_t p = 1;
+  for (auto x : v)
+    p *= x;
+  return p;
+}
+
+mxk::DimTransform toDim(const std::vector<std::size_t> &shape,
+                        const ConvParams::InputTransform &t, unsigned d,
+                        unsigned transformedSize) {
+  return {uint32_t(shape[d]), t.truncationLower[d], t.truncationUpper[d],
+          t.dilation[d],      t.paddingLower[d],    t.paddingUpper[d],
+          uint32_t(t.flip[d] ? 1 : 0), transformedSize};
+}
+
+mxk::GenericDesc makeGenericDesc(const ConvParams &p) {
+  mxk::GenericDesc g{};
+  g.numDims = uint32_t(p.getNumFieldDims());
+  g.batch = uint32_t(p.batchSize);
+  g.groups = uint32_t(p.numConvGroups);
+  g.inChansPerGroup = uint32_t(p.inputChannelsPerConvGroup);
+  g.outChansPerGroup = uint32_t(p.outputChannelsPerConvGroup);
+  g.kernelElems = 1;
+  g.outElems = uint64_t(p.batchSize) * p.getNumOutputChans();
+  for (unsigned d = 0; d != g.numDims; ++d) {
+    g.in[d] = toDim(p.inputFieldShape, p.inputTransform, d,
+                    p.getTransformedInputSize(d));
+    g.kernel[d] = toDim(p.kernelShape, p.kernelTransform, d,
+                        p.getTransformedKernelSize(d));
+    g.outSize[d] = uint32_t(p.getOutputSize(d));
+    g.outTruncLo[d] = p.outputTransform.truncationLower[d];
+    g.outStride[d] = p.outputTransform.stride[d];
+    g.outPadLo[d] = p.outputTransform.paddingLower[d];
+    g.outPadHi[d] = p.outputTransform.paddingUpper[d];
+    g.kernelElems *= uint32_t(p.kernelShape[d]);
+    g.outElems *= g.outSize[d];
+  }
+  return g;
+}
+
+/// The subset the fast kernels take: up to two field dimensions; input with
+/// truncation and zero padding only; kernel with dilation only; output with
+/// truncation and stride only.  Written as "input row = out*stride +
+/// k*dilation - pad, valid inside [lo, hi)".
+struct Simple2D {
+  bool ok = false;
+  std::string why;
+  uint32_t inH = 1, inW = 1, outH = 1, outW = 1, kH = 1, kW = 1;
+  int32_t padH = 0, padW = 0;
+  uint32_t strideH = 1, strideW = 1, dilH = 1, dilW = 1;
+  uint32_t loH = 0, hiH = 1, loW = 0, hiW = 1;
+};
+
+Simple2D asSimple2D(const ConvParams &p) {
+  Simple2D s;
+  const unsigned n = unsigned(p.getNumFieldDims());
+  if (n > 2) {
+    s.why = "more than two field dimensions";
+    return s;
+  }
+  for (unsigned d = 0; d != n; ++d) {
+    const auto &it = p.inputTransform, &kt = p.kernelTransform;
+    const auto &ot = p.outputTransform;
+    if (it.dilation[d] != 1 || it.flip[d]) {
+      s.why = "input dilation or flip";
+      return s;
+    }
+    if (kt.truncationLower[d] || kt.truncationUpper[d] || kt.paddingLower[d] ||
+        kt.paddingUpper[d] || kt.flip[d]) {
+      s.why = "kernel truncation, padding or flip";
+      return s;
+    }
+    if (ot.paddingLower[d] || ot.paddingUpper[d]) {
+      s.why = "output padding";
+      return s;
+    }
+    // conv index = o*stride + outTruncLo; padded input = conv + k*dil;
+    // input = padded - padLo + truncLo.
+    const int32_t pad = int32_t(it.paddingLower[d]) -
+                        int32_t(it.truncationLower[d]) -
+                        int32_t(ot.truncationLower[d]);
+    const uint32_t lo = it.truncationLower[d];
+    const uint32_t hi = uint32_t(p.inputFieldShape[d]) - it.truncationUpper[d];
+    const bool isW = (d + 1 == n);
+    (isW ? s.inW : s.inH) = uint32_t(p.inputFieldShape[d]);
+    (isW ? s.outW : s.outH) = uint32_t(p.getOutputSize(d));
+    (isW ? s.kW : s.kH) = uint32_t(p.kernelShape[d]);
+    (isW ? s.padW : s.padH) = pad;
+    (isW ? s.strideW : s.strideH) = ot.stride[d];
+    (isW ? s.dilW : s.dilH) = kt.dilation[d];
+    (isW ? s.loW : s.loH) = lo;
+    (isW ? s.hiW : s.hiH) = hi;
+  }
+  s.ok = true;
+  return s;
+}
+
+} // namespace
+
+mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
+  mxconv_plan plan;
+  plan.params = params;
+  plan.canonical = params.canonicalize(); // validates
+  plan.options = optionsIn;
+  ConvOptions &options = plan.options;
+  const ConvParams &p = plan.canonical;
+
+  if (p.getNumFieldDims() > mxk::kMaxDims)
+    throw poputil::poplibs_error("At most " + std::to_string(mxk::kMaxDims) +
+                                 " field dimensions are supported");
+
+  // validateLayerParams: partials at least as wide as the output; quarter
+  // inputs produce half outputs.  This build always accumulates in fp32, which
+  // satisfies every partials type the reference would settle on.
+  for (poplar::Type *t : {&options.partialsType, &options.interTilePartialsType,
+                          &options.interIpuPartialsType})
+    if (t->size() < params.outputType.size())
+      *t = params.outputType;
+  if (params.inputType == poplar::QUARTER && params.outputType != poplar::HALF)
+    throw poputil::poplibs_error(
+        "When the input type for a convolution is quarter, the output type "
+        "must be half, not " +
+        params.outputType.toString());
+  if (params.outputType == poplar::QUARTER)
+    throw poputil::poplibs_error("Unsupported convolution output element type "
+                                 "(must be float or half)");
+
+  plan.inputElems = params.batchSize * params.getNumInputChans() *
+                    product(params.inputFieldShape);
+  plan.outputElems = params.batchSize * params.getNumOutputChans() *
+                     product(params.getOutputFieldShape());
+  plan.weightElems = params.numConvGroups * params.outputChannelsPerConvGroup *
+                     params.inputChannelsPerConvGroup *
+                     product(params.kernelShape);
+  plan.biasElems = params.getNumOutputChans();
+  plan.generic = makeGenericDesc(p);
+  plan.zeroConv = isZeroConvolution(p);
+
+  using Kernel = mxconv_plan::Kernel;
+  using Method = PlanConstraints::Method;
+  const auto &pc = options.planConstraints;
+  const Simple2D s = asSimple2D(p);
+  const bool halfIn = params.inputType == poplar::HALF;
+  const bool quarterIn = params.inputType == poplar::QUARTER;
+  const std::size_t ci = p.inputChannelsPerConvGroup;
+  const std::size_t co = p.outputChannelsPerConvGroup;
+
+  // Which kernels can take this convolution at all?
+  std::string igemmWhyNot, dwWhyNot;
+  if (plan.zeroConv)
+    igemmWhyNot = dwWhyNot = "all outputs are zero";
+  else if (!s.ok)
+    igemmWhyNot = dwWhyNot = s.why;
+  else {
+    if (!(halfIn || quarterIn))
+      igemmWhyNot = "matrix-core kernel takes half or quarter inputs";
+    else if (ci % (halfIn ? 8 : 16) != 0)
+      igemmWhyNot = "input channels per group not a multiple of a 16-byte "
+                    "vector";
+    if (!halfIn)
+      dwWhyNot = "depthwise kernel takes half inputs";
+    else if (ci != 1 || co != 1)
+      dwWhyNot = "not one channel per group";
+    else if (p.numConvGroups % 8 != 0)
+      dwWhyNot = "channel count not a multiple of 8";
+  }
+
+  // Choose.  PopLibs method names map onto the kernels that take their role:
+  // AMP -> matrix cores; HMAC / VMAC / SLIC -> vector-ALU direct kernel.
+  Kernel chosen = Kernel::GENERIC;
+  std::string reason;
+  auto require = [&](const std::string &whyNot, const char *what) {
+    if (!whyNot.empty())
+      throw poplar::invalid_option(
+          std::string("planConstraints ask for the ") + what +
+          " kernel, which cannot take this convolution: " + whyNot);
+  };
+  if (pc.kernel == "generic") {
+    reason = "forced by planConstraints";
+  } else if (pc.kernel == "igemm") {
+    require(igemmWhyNot, "igemm");
+    chosen = Kernel::IGEMM;
+    reason = "forced by planConstraints";
+  } else if (pc.kernel == "depthwise") {
+    require(dwWhyNot, "depthwise");
+    chosen = Kernel::DEPTHWISE;
+    reason = "forced by planConstraints";
+  } else if (pc.method == Method::AMP && igemmWhyNot.empty()) {
+    chosen = Kernel::IGEMM;
+    reason = "method AMP -> matrix cores";
+  } else if ((pc.method == Method::HMAC || pc.method == Method::VMAC ||
+              pc.method == Method::SLIC) &&
+             dwWhyNot.empty()) {
+    chosen = Kernel::DEPTHWISE;
+    reason = "method " + std::string(pc.method == Method::HMAC   ? "HMAC"
+                                     : pc.method == Method::VMAC ? "VMAC"
+                                                                 : "SLIC") +
+             " -> vector-ALU direct kernel";
+  } else if (pc.method == Method::HMAC || pc.method == Method::VMAC ||
+             pc.method == Method::SLIC || pc.method == Method::OUTER_PRODUCT) {
+    reason = "vector-ALU method requested; generic direct kernel";
+  } else if (dwWhyNot.empty()) {
+    chosen = Kernel::DEPTHWISE;
+    reason = "one channel per group: memory-bound, vector-ALU direct kernel";
+  } else if (igemmWhyNot.empty()) {
+    chosen = Kernel::IGEMM;
+    reason = "dense channels: implicit GEMM on the matrix cores";
+  } else {
+    reason = "generic direct kernel (" + igemmWhyNot + ")";
+  }
+  plan.kernel = chosen;
+  plan.reason = reason;
+
+  if (chosen == Kernel::IGEMM) {
+    mxk::IgemmDesc &g = plan.igemm;
+    g.batch = uint32_t(p.batchSize);
+    g.groups = uint32_t(p.numConvGroups);
+    g.inChansPerGroup = uint32_t(ci);
+    g.outChansPerGroup = uint32_t(co);
+    g.inH = s.inH, g.inW = s.inW, g.outH = s.outH, g.outW = s.outW;
+    g.kH = s.kH, g.kW = s.kW, g.padH = s.padH, g.padW = s.padW;
+    g.strideH = s.strideH, g.strideW = s.strideW;
+    g.dilH = s.dilH, g.dilW = s.dilW;
+    g.loH = s.loH, g.hiH = s.hiH, g.loW = s.loW, g.hiW = s.hiW;
+    // Tile shape.  M = batch * outH * outW pixels, N = out channels of one
+    // group, K = kH * kW * in channels.  A 128-pixel tile keeps the A
+    // fragment reuse high; N is 128 unless the group has at most 64 output
+    // channels, when a narrower tile avoids computing padding.
+    g.blockM = pc.blockM ? pc.blockM : 128;
+    g.blockN = pc.blockN ? pc.blockN : (co <= 64 ? 64 : 128);
+    g.blockK = pc.blockK ? pc.blockK : (halfIn ? 32 : 64);
+    if (g.blockM != 128 || (g.blockN != 64 && g.blockN != 128) ||
+        g.blockK != (halfIn ? 32u : 64u))
+      throw poplar::invalid_option(
+          "planConstraints gfx950 tile not available: blockM must be 128, "
+          "blockN 64 or 128, blockK 32 (half) or 64 (quarter)");
+    const std::size_t k = std::size_t(s.kH) * s.kW * ci;
+    plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
+    plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;
+    plan.weightPackedElems = p.numConvGroups * plan.coPadded * plan.kPadded;
+  } else if (chosen == Kernel::DEPTHWISE) {
+    mxk::DepthwiseDesc &d = plan.depthwise;
+    d.batch = uint32_t(p.batchSize);
+    d.channels = uint32_t(p.numConvGroups);
+    d.inH = s.inH, d.inW = s.inW, d.outH = s.outH, d.outW = s.outW;
+    d.kH = s.kH, d.kW = s.kW, d.padH = s.padH, d.padW = s.padW;
+    d.strideH = s.strideH, d.strideW = s.strideW;
+    d.dilH = s.dilH, d.dilW = s.dilW;
+    d.loH = s.loH, d.hiH = s.hiH, d.loW = s.loW, d.hiW = s.hiW;
+    plan.weightPackedElems = plan.weightElems; // [kH*kW][C]
+  } else {
+    plan.weightPackedElems = plan.weightElems; // [G][K][Ci][Co]
+  }
+  return plan;
+}
+
+} // namespace poplin
+
+std::string mxconv_plan::describe() const {
+  std::ostringstream os;
+  os << "  Plan (gfx950: " << gfx950::numCUs << " CUs, "
+     << gfx950::ldsBytesPerCU / 1024 << " KB LDS/CU, wave"
+     << gfx950::wavefrontSize << "):\n";
+  os << "        kernel                     ";
+  switch (kernel) {
+  case Kernel::GENERIC:
+    os << "generic direct (vector ALU, any parameters)";
+    break;
+  case Kernel::IGEMM:
+    os << "implicit GEMM (MFMA, "
+       << (params.inputType == poplar::QUARTER ? "fp8" : "fp16")
+       << " operands, fp32 accumulate)";
+    break;
+  case Kernel::DEPTHWISE:
+    os << "depthwise direct (vector ALU, LDS halo tiles)";
+    break;
+  }
+  os << "\n        reason                     " << reason << "\n";
+  os << "        zeroConv                   " << (zeroConv ? "true" : "false")
+     << "\n";
+  os << "        partialsType               float\n";
+  if (kernel == Kernel::IGEMM) {
+    const auto &g = igemm;
+    const std::size_t m = std::size_t(g.batch) * g.outH * g.outW;
+    const std::size_t k = std::size_t(g.kH) * g.kW * g.inChansPerGroup;
+    const std::size_t tiles = (m + g.blockM - 1) / g.blockM *
+                              (coPadded / g.blockN) * g.groups;
+    os << "        gemm M x N x K             " << m << " x "
+       << g.outChansPerGroup << " x " << k << " (x " << g.groups
+       << " groups)\n";
+    os << "        block M x N x K            " << g.blockM << " x " << g.blockN
+       << " x " << g.blockK << "\n";
+    os << "        workgroups                 " << tiles << "\n";
+    os << "        packed weights             [G=" << g.groups << "]["
+       << coPadded << "][" << kPadded << "]\n";
+  } else if (kernel == Kernel::DEPTHWISE) {
+    const auto &d = depthwise;
+    os << "        channels                   " << d.channels << "\n";
+    os << "        packed weights             [" << d.kH * d.kW << "]["
+       << d.channels << "]\n";
+  } else {
+    os << "        packed weights             [G][K][Ci][Co]\n";
+  }
+  os << "        workspaceBytes             " << workspaceBytes << "\n";
+  return os.str();
+}

@@ -1,0 +1,66 @@
+// The gfx950 tile planner: what replaces PopLibs' IPU convolution planner
+// (getPlan, lib/poplin/ConvPlan.cpp:1877-1923) in this build.  A plan fixes
+// the kernel, its tile shape and the packed weight layout for one
+// (ConvParams, ConvOptions) pair; it is plain host data and creating it
+// touches no GPU.
+#ifndef poplibs_amd_Plan_hpp
+#define poplibs_amd_Plan_hpp
+#include "ConvOptions.hpp"
+#include "kernels.hpp"
+#include "poplin/ConvParams.hpp"
+#include <cstddef>
+#include <string>
+
+/// Fixed properties of the one target this library is written for.
+namespace gfx950 {
+constexpr unsigned numCUs = 256;
+constexpr unsigned numXCDs = 8;
+constexpr unsigned ldsBytesPerCU = 160 * 1024;
+constexpr unsigned wavefrontSize = 64;
+} // namespace gfx950
+
+struct mxconv_plan {
+  enum class Kernel { GENERIC, IGEMM, DEPTHWISE };
+
+  poplin::ConvParams params;    // as given by the caller
+  poplin::ConvParams canonical; // ConvParams::canonicalize() of it
+  poplin::ConvOptions options;
+  bool zeroConv = false;
+  Kernel kernel = Kernel::GENERIC;
+  std::string reason; // why this kernel was chosen
+
+  mxk::GenericDesc generic{};     // always valid: describes `canonical`
+  mxk::IgemmDesc igemm{};         // valid when kernel == IGEMM
+  mxk::DepthwiseDesc depthwise{}; // valid when kernel == DEPTHWISE
+
+  // Packed weights of the matrix-core kernel: [G][coPadded][kPadded].
+  std::size_t coPadded = 0, kPadded = 0;
+
+  std::size_t inputElems = 0, outputElems = 0, weightElems = 0,
+              weightPackedElems = 0, biasElems = 0;
+  std::size_t workspaceBytes = 0;
+
+  std::size_t inputBytes() const { return inputElems * params.inputType.size(); }
+  std::size_t outputBytes() const {
+    return outputElems * params.outputType.size();
+  }
+  std::size_t weightBytes() const {
+    return weightElems * params.inputType.size();
+  }
+  std::size_t weightPackedBytes() const {
+    return weightPackedElems * params.inputType.size();
+  }
+  std::size_t biasBytes() const { return biasElems * params.outputType.size(); }
+
+  std::string describe() const;
+};
+
+namespace poplin {
+
+/// validateLayerParams (lib/poplin/ConvValidation.cpp:11-70) followed by the
+/// kernel and tile choice.  Throws poputil::poplibs_error /
+/// poplar::invalid_option.
+mxconv_plan makePlan(const ConvParams &params, const ConvOptions &options);
+
+} // namespace poplin
+#endif
