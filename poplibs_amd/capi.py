@@ -95,6 +95,12 @@ def lib():
     global _lib
     if _lib is not None:
         return _lib
+    # A process must hold ONE HIP runtime.  PyTorch ships its own copy of
+    # libamdhip64 (same soname as the system one); callers here use torch
+    # tensors as device memory, so torch has to load first - the dynamic
+    # loader then binds libmxconv.so's libamdhip64.so.7 to that copy instead of
+    # mapping a second runtime that cannot see the first one's allocations.
+    import torch  # noqa: F401
     if not os.path.exists(_LIB_PATH):
         raise RuntimeError(
             f"{_LIB_PATH} is missing: build it with "
