@@ -1,0 +1,279 @@
+"""GPU parity of the matrix-core (implicit GEMM) and depthwise kernels against
+the CPU oracle, through the C ABI.
+
+Tolerances (relative L2 error against the double-precision oracle fed the same
+rounded inputs): fp16 in / fp32 accumulate <= 1e-3; fp8 in / fp32 accumulate
+<= 3e-2; +-1 data with fp32 output: exact.  The BASELINE configurations are
+run at full size and checked on a subset of batch images (the convolution is
+independent per image) plus size-independent properties."""
+import numpy as np
+import pytest
+
+import poplibs_amd as pa
+from helpers import make_params, random_data, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _plan_kernel(plan):
+    text = plan.describe()
+    for name in ("implicit GEMM", "depthwise direct", "generic direct"):
+        if name in text:
+            return name
+    raise AssertionError(text)
+
+
+def _run(oracle, p, seed, tol, expect_kernel, dist="normal", bias=True,
+         wscale=None, options=None):
+    from gpu_helpers import quantize, run_conv
+    acts, weights, biases = random_data(p, seed, dist)
+    if wscale is not None:
+        weights = weights * wscale
+    aq, ad = quantize(acts, p.inputType)
+    wq, wd = quantize(weights, p.inputType)
+    bq, bd = quantize(biases, p.outputType)
+    got, plan = run_conv(p, aq, wq, bq if bias else None, options,
+                         return_plan=True)
+    assert _plan_kernel(plan) == expect_kernel, plan.describe()
+    want = oracle.convolution(p, ad, wd, bd if bias else None, threads=8)
+    assert got.shape == want.shape
+    if tol == 0:
+        np.testing.assert_array_equal(got, want)
+    else:
+        err = rel_l2(got, want)
+        assert err <= tol, (err, p)
+    return got
+
+
+IGEMM_CASES = [
+    # BASELINE config 2 shape (3x3 s1 p1, 128->128, 28x28), reduced batch
+    dict(batch=2, field=(28, 28), kernel=(3, 3), ci=128, co=128, pad=1),
+    # BASELINE config 3 shape (1x1, 256->64, 56x56), reduced batch
+    dict(batch=1, field=(56, 56), kernel=(1, 1), ci=256, co=64),
+    # M, N, K all ragged against the 128 x {64,128} x 32 tile
+    dict(batch=3, field=(9, 7), kernel=(3, 3), ci=8, co=40, pad=1),
+    dict(batch=1, field=(5, 5), kernel=(2, 3), ci=24, co=130,
+         padLower=(1, 0), padUpper=(0, 2)),
+    # stride, kernel dilation, groups
+    dict(batch=2, field=(17, 15), kernel=(3, 3), ci=16, co=24, groups=3,
+         stride=(2, 1), kdil=(1, 2), pad=2),
+    # 1-D field and a tall kernel
+    dict(batch=2, field=(50,), kernel=(7,), ci=32, co=16, stride=3, pad=3),
+    # truncation folded into the window: input and output truncation
+    dict(batch=1, field=(12, 12), kernel=(3, 3), ci=8, co=8, itl=(1, 0),
+         itu=(0, 2), otl=(1, 1), otu=(0, 1), pad=1),
+    # 0-D field = plain matrix product
+    dict(batch=70, field=(), kernel=(), ci=64, co=96),
+]
+
+
+@pytest.mark.parametrize("kw", IGEMM_CASES)
+def test_igemm_fp16_matches_oracle(oracle, kw):
+    p = make_params(pa.HALF, **kw)
+    print("case", p, flush=True)
+    _run(oracle, p, 1, 1e-3, "implicit GEMM", wscale=0.1)
+
+
+@pytest.mark.parametrize("kw", IGEMM_CASES[2:6])
+def test_igemm_fp16_in_fp32_out_pm1_exact(oracle, kw):
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    print("case", p, flush=True)
+    _run(oracle, p, 2, 0, "implicit GEMM", dist="pm1")
+
+
+def test_igemm_blockN_override_and_amp_method(oracle):
+    p = make_params(pa.HALF, batch=1, field=(10, 10), kernel=(3, 3), ci=16,
+                    co=32, pad=1)
+    opts = {"planConstraints":
+            '{"method": {"type": "AMP"}, "gfx950": {"blockN": 128}}'}
+    _run(oracle, p, 3, 1e-3, "implicit GEMM", options=opts, wscale=0.1)
+
+
+DW_CASES = [
+    # BASELINE config 4 shape (3x3 s2 p1, C=96, 112x112), reduced batch
+    dict(batch=2, field=(112, 112), kernel=(3, 3), groups=96, stride=2, pad=1),
+    dict(batch=3, field=(9, 11), kernel=(3, 3), groups=8, pad=1),
+    dict(batch=1, field=(13, 7), kernel=(5, 2), groups=24, stride=(1, 2),
+         kdil=(2, 1), padLower=(3, 0), padUpper=(1, 1)),
+    dict(batch=2, field=(31,), kernel=(4,), groups=16, stride=2, pad=2),
+]
+
+
+@pytest.mark.parametrize("kw", DW_CASES)
+def test_depthwise_fp16_matches_oracle(oracle, kw):
+    p = make_params(pa.HALF, **kw)
+    print("case", p, flush=True)
+    _run(oracle, p, 4, 1e-3, "depthwise direct")
+
+
+def test_depthwise_fp32_out_pm1_exact(oracle):
+    p = make_params(pa.HALF, pa.FLOAT, **DW_CASES[1])
+    _run(oracle, p, 5, 0, "depthwise direct", dist="pm1")
+
+
+def _fp8_case(oracle, p, seed, fmt_a, fmt_w):
+    """values ~N(0,1) (weights scaled), per-tensor power-of-two scale chosen
+    so the largest magnitude lands below the format's maximum."""
+    from gpu_helpers import quantize, run_conv
+    acts, weights, _ = random_data(p, seed, "normal")
+    fan_in = p.inputChannelsPerConvGroup * int(np.prod(p.kernelShape))
+    weights = weights * np.sqrt(2.0 / max(fan_in, 1))
+
+    def scale_for(x, fmt):
+        maxv = 448.0 if fmt == oracle.E4M3 else 57344.0
+        m = np.abs(x).max()
+        return int(np.ceil(np.log2(m / maxv))) if m > 0 else 0
+
+    sa, sw = scale_for(acts, fmt_a), scale_for(weights, fmt_w)
+    aq, ad = quantize(acts, pa.QUARTER, oracle, fmt_a, sa)
+    wq, wd = quantize(weights, pa.QUARTER, oracle, fmt_w, sw)
+    got, plan = run_conv(p, aq, wq, None, None,
+                         in_meta=pa.quarter_metadata(fmt_a, sa),
+                         w_meta=pa.quarter_metadata(fmt_w, sw),
+                         return_plan=True)
+    want = oracle.convolution(p, ad, wd, threads=8)
+    return got, want, plan
+
+
+@pytest.mark.parametrize("fmt_a,fmt_w", [(1, 1), (1, 0), (0, 1), (0, 0)])
+def test_igemm_fp8_matches_oracle(oracle, fmt_a, fmt_w):
+    # BASELINE config 5 shape (3x3 s1 p1, 256->256, 14x14), reduced batch
+    p = make_params(pa.QUARTER, pa.HALF, batch=2, field=(14, 14),
+                    kernel=(3, 3), ci=256, co=256, pad=1)
+    got, want, plan = _fp8_case(oracle, p, 6, fmt_a, fmt_w)
+    assert _plan_kernel(plan) == "implicit GEMM"
+    err = rel_l2(got, want)
+    assert err <= 3e-2, err
+    # the inputs are exact in fp8, so the only error is fp32 accumulation and
+    # the fp16 output rounding: far below the fp8 budget
+    assert err <= 1e-3, err
+
+
+def test_igemm_fp8_ragged_shapes(oracle):
+    p = make_params(pa.QUARTER, pa.HALF, batch=3, field=(7, 9), kernel=(3, 2),
+                    ci=16, co=40, groups=2, stride=(1, 2), pad=1)
+    got, want, plan = _fp8_case(oracle, p, 7, 1, 1)
+    assert _plan_kernel(plan) == "implicit GEMM"
+    assert rel_l2(got, want) <= 1e-3
+
+
+def test_generic_fp8_matches_oracle(oracle):
+    # Ci = 4 is not a whole 16-byte vector: falls back to the generic kernel
+    p = make_params(pa.QUARTER, pa.HALF, batch=2, field=(6, 6), kernel=(3, 3),
+                    ci=4, co=5, pad=1)
+    got, want, plan = _fp8_case(oracle, p, 8, 1, 0)
+    assert _plan_kernel(plan) == "generic direct"
+    assert rel_l2(got, want) <= 1e-3
+
+
+def test_quarter_small_integer_data_is_exact(oracle):
+    """The reference draws quarter test data as small integers so that they
+    are exactly representable (lib/poplibs_test/Util.cpp:140-142); with a
+    fp32 accumulate the result is then exact up to the fp16 output."""
+    from gpu_helpers import quantize, run_conv
+    p = make_params(pa.QUARTER, pa.HALF, batch=1, field=(8, 8), kernel=(3, 3),
+                    ci=16, co=16, pad=1)
+    g = np.random.default_rng(9)
+    acts = g.integers(-3, 4, (1, 16, 8, 8)).astype(np.float64)
+    weights = g.integers(-1, 2, (1, 16, 16, 3, 3)).astype(np.float64)
+    aq, ad = quantize(acts, pa.QUARTER, oracle, 1, 0)
+    wq, wd = quantize(weights, pa.QUARTER, oracle, 1, 0)
+    np.testing.assert_array_equal(ad, acts)
+    got = run_conv(p, aq, wq, None, None, in_meta=0x80, w_meta=0x80)
+    want = oracle.convolution(p, ad, wd)
+    assert np.abs(want).max() < 2048  # exactly representable in fp16
+    np.testing.assert_array_equal(got, want)
+    # metadata scales multiply the result by 2^(sIn + sW)
+    got2 = run_conv(p, aq, wq, None, None,
+                    in_meta=pa.quarter_metadata(1, 1),
+                    w_meta=pa.quarter_metadata(1, 2))
+    np.testing.assert_array_equal(got2, want * 8.0)
+    got3 = run_conv(p, aq, wq, None, None,
+                    in_meta=pa.quarter_metadata(1, -2),
+                    w_meta=pa.quarter_metadata(1, -1))
+    np.testing.assert_array_equal(got3, want / 8.0)
+
+
+# ---- BASELINE configurations at full size ---------------------------------
+
+def _full_size(oracle, p, seed, tol, kernel, act_fn=None, w_std=1.0,
+               images=(0, -1)):
+    from gpu_helpers import quantize, run_conv
+    g = np.random.default_rng(seed)
+    acts = g.standard_normal((p.batchSize, p.getNumInputChans(),
+                              *p.inputFieldShape))
+    if act_fn:
+        acts = act_fn(acts)
+    weights = g.standard_normal(
+        (p.numConvGroups, p.outputChannelsPerConvGroup,
+         p.inputChannelsPerConvGroup, *p.kernelShape)) * w_std
+    aq, ad = quantize(acts, p.inputType)
+    wq, wd = quantize(weights, p.inputType)
+    got, plan = run_conv(p, aq, wq, None, None, return_plan=True)
+    assert _plan_kernel(plan) == kernel
+    one = pa.ConvParams.from_c(p.to_c())
+    one.batchSize = 1
+    for b in images:
+        want = oracle.convolution(one, ad[b:b + 1] if b >= 0 else ad[b:],
+                                  wd, threads=8)
+        err = rel_l2(got[b], want[0])
+        assert err <= tol, (b, err)
+    # size-independent property: images are independent, so reversing the
+    # batch reverses the output, bit for bit
+    got_rev = run_conv(p, aq[::-1].copy(), wq, None, None, plan=plan)
+    assert np.array_equal(got_rev, got[::-1])
+    return got
+
+
+def test_baseline_config2_full(oracle):
+    p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                    co=128, pad=1)
+    assert p.getFwdFlops() == 7050625024
+    _full_size(oracle, p, 0, 1e-3, "implicit GEMM",
+               w_std=np.sqrt(2.0 / (9 * 128)))
+
+
+def test_baseline_config3_full(oracle):
+    p = make_params(pa.HALF, batch=32, field=(56, 56), kernel=(1, 1), ci=256,
+                    co=64)
+    assert p.getFwdFlops() == 3288334336
+    _full_size(oracle, p, 0, 1e-3, "implicit GEMM",
+               act_fn=lambda x: np.maximum(x, 0), w_std=np.sqrt(2.0 / 256))
+
+
+def test_baseline_config4_full(oracle):
+    p = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                    groups=96, stride=2, pad=1)
+    assert p.getFwdFlops() == 171350016
+    assert p.getOutputFieldShape() == [56, 56]
+    _full_size(oracle, p, 0, 1e-3, "depthwise direct", w_std=np.sqrt(2.0 / 9))
+
+
+def test_baseline_config5_full(oracle):
+    from gpu_helpers import run_conv
+    p = make_params(pa.QUARTER, pa.HALF, batch=64, field=(14, 14),
+                    kernel=(3, 3), ci=256, co=256, pad=1)
+    assert p.getFwdFlops() == 13421772800
+    # quantise exactly as the configuration states, check three images; the
+    # oracle receives the dequantised values, so the error measured is that of
+    # the accumulation and the fp16 output rounding
+    from gpu_helpers import quantize
+    g = np.random.default_rng(0)
+    acts = g.standard_normal((64, 256, 14, 14))
+    weights = g.standard_normal((1, 256, 256, 3, 3)) * np.sqrt(2 / (9 * 256))
+    sa = int(np.ceil(np.log2(np.abs(acts).max() / 448.0)))
+    sw = int(np.ceil(np.log2(np.abs(weights).max() / 448.0)))
+    aq, ad = quantize(acts, pa.QUARTER, oracle, 1, sa)
+    wq, wd = quantize(weights, pa.QUARTER, oracle, 1, sw)
+    got, plan = run_conv(p, aq, wq, None, None,
+                         in_meta=pa.quarter_metadata(1, sa),
+                         w_meta=pa.quarter_metadata(1, sw), return_plan=True)
+    assert _plan_kernel(plan) == "implicit GEMM"
+    one = pa.ConvParams.from_c(p.to_c())
+    one.batchSize = 1
+    for b in (0, 31, 63):
+        want = oracle.convolution(one, ad[b:b + 1], wd, threads=8)
+        # against the dequantised inputs only accumulation and the fp16
+        # output round: well inside the 3e-2 fp8 budget
+        err = rel_l2(got[b], want[0])
+        assert err <= 3e-2 and err <= 1e-3, err
