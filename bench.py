@@ -1,0 +1,337 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X forward convolution behind the C ABI.
+
+A "step" is one forward convolution (one `mxconv_fwd` call) over one batch of
+synthetic, seeded input that is already resident in HBM in the device layout
+(channels-last activations, packed weights).  The headline workload is the
+ResNet-style 3x3 layer the metric is quoted on; the other configurations
+(1x1, depthwise, fp8) are measured the same way and reported inside the same
+JSON line under "other_workloads".
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+prints ONE JSON line.  Only one GPU is used; --gpus above 1 is refused.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"fp16": 2500.0, "fp8": 5000.0}   # MI355X dense MFMA
+PEAK_HBM_GBS = 8000.0                            # MI355X HBM3E
+
+
+def _workloads(pa):
+    """The BASELINE configurations 2-5 as ConvParams + data recipe."""
+    def params(t_in, t_out, batch, field, kernel, ci, co, groups, stride, pad):
+        p = pa.ConvParams(t_in, t_out, batch, list(field), list(kernel), ci,
+                          co, groups)
+        p.inputTransform.paddingLower = [pad] * len(field)
+        p.inputTransform.paddingUpper = [pad] * len(field)
+        p.outputTransform.stride = [stride] * len(field)
+        return p
+    return {
+        "c2": dict(
+            name="configs[1]: ResNet-style 3x3 conv N=32 28x28 Cin=Cout=128 "
+                 "stride 1 pad 1, fp16 in/weights, fp32 partials, fp16 out",
+            params=params(pa.HALF, pa.HALF, 32, (28, 28), (3, 3), 128, 128, 1,
+                          1, 1),
+            dtype="fp16", bound="mfma", relu=False, w_std=(2 / (9 * 128)) ** .5),
+        "c3": dict(
+            name="configs[2]: 1x1 conv N=32 56x56 Cin=256 Cout=64, fp16",
+            params=params(pa.HALF, pa.HALF, 32, (56, 56), (1, 1), 256, 64, 1,
+                          1, 0),
+            dtype="fp16", bound="hbm", relu=True, w_std=(2 / 256) ** .5),
+        "c4": dict(
+            name="configs[3]: depthwise 3x3 stride 2 pad 1 N=32 112x112 C=96, "
+                 "fp16 in, fp32 partials, fp16 out",
+            params=params(pa.HALF, pa.HALF, 32, (112, 112), (3, 3), 1, 1, 96,
+                          2, 1),
+            dtype="fp16", bound="hbm", relu=False, w_std=(2 / 9) ** .5),
+        "c5": dict(
+            name="configs[4]: fp8 E4M3 3x3 conv N=64 14x14 Cin=Cout=256 "
+                 "stride 1 pad 1, per-tensor 2^k scales, fp32 acc, fp16 out",
+            params=params(pa.QUARTER, pa.HALF, 64, (14, 14), (3, 3), 256, 256,
+                          1, 1, 1),
+            dtype="fp8", bound="mfma", relu=False,
+            w_std=(2 / (9 * 256)) ** .5),
+    }
+
+
+class Runner:
+    """Device buffers + plan of one workload; `launch(i)` enqueues one
+    forward convolution on buffer set i."""
+
+    def __init__(self, pa, capi, torch, wl, seed=0, sets=1):
+        self.pa, self.torch, self.wl = pa, torch, wl
+        p = self.p = wl["params"]
+        self.plan = pa.Plan(p)
+        dev = torch.device("cuda:0")
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        ashape = (p.batchSize, p.getNumInputChans(), *p.inputFieldShape)
+        wshape = (p.numConvGroups, p.outputChannelsPerConvGroup,
+                  p.inputChannelsPerConvGroup, *p.kernelShape)
+        acts = torch.randn(ashape, generator=g, dtype=torch.float32)
+        if wl["relu"]:
+            acts = acts.clamp_min(0)
+        weights = torch.randn(wshape, generator=g,
+                              dtype=torch.float32) * wl["w_std"]
+        self.in_meta = self.w_meta = 0x80
+        if p.inputType == pa.QUARTER:
+            import math
+            sa = math.ceil(math.log2(acts.abs().max().item() / 448.0))
+            sw = math.ceil(math.log2(weights.abs().max().item() / 448.0))
+            self.in_meta = pa.quarter_metadata(1, sa)
+            self.w_meta = pa.quarter_metadata(1, sw)
+            a_ext = (acts / 2.0 ** sa).to(torch.float8_e4m3fn).view(torch.uint8)
+            w_ext = (weights / 2.0 ** sw).to(torch.float8_e4m3fn).view(
+                torch.uint8)
+        else:
+            a_ext, w_ext = acts.half(), weights.half()
+        self.a_ext_host, self.w_ext_host = a_ext, w_ext
+        a_ext, w_ext = a_ext.to(dev), w_ext.to(dev)
+
+        def buf(which):
+            return torch.empty(max(self.plan.buffer_bytes(which), 16),
+                               dtype=torch.uint8, device=dev)
+
+        self.w_pack = buf(capi.BUF_WEIGHTS_PACKED)
+        self.ws = buf(capi.BUF_WORKSPACE)
+        self.ws_bytes = self.plan.buffer_bytes(capi.BUF_WORKSPACE)
+        s = torch.cuda.current_stream().cuda_stream
+        self.plan.pack_weights(w_ext.data_ptr(), self.w_pack.data_ptr(), s)
+        self.inputs, self.outputs = [], []
+        for _ in range(sets):
+            a_int = buf(capi.BUF_INPUT)
+            self.plan.acts_to_internal(a_ext.data_ptr(), a_int.data_ptr(), s)
+            self.inputs.append(a_int)
+            self.outputs.append(buf(capi.BUF_OUTPUT))
+        torch.cuda.synchronize()
+        self.flops = p.getFwdFlops()
+        self.bytes = (self.plan.buffer_bytes(capi.BUF_INPUT)
+                      + self.plan.buffer_bytes(capi.BUF_WEIGHTS_EXTERNAL)
+                      + self.plan.buffer_bytes(capi.BUF_OUTPUT))
+
+    def launch(self, i=0):
+        s = self.torch.cuda.current_stream().cuda_stream
+        k = i % len(self.inputs)
+        if self.p.inputType == self.pa.QUARTER:
+            self.plan.fwd_quarter(self.inputs[k].data_ptr(), self.in_meta,
+                                  self.w_pack.data_ptr(), self.w_meta,
+                                  self.outputs[k].data_ptr(), None,
+                                  self.ws.data_ptr(), self.ws_bytes, s)
+        else:
+            self.plan.fwd(self.inputs[k].data_ptr(), self.w_pack.data_ptr(),
+                          self.outputs[k].data_ptr(), None, self.ws.data_ptr(),
+                          self.ws_bytes, s)
+
+    def output_external(self, k=0):
+        """Output of buffer set k in the external [B][C][H][W] layout."""
+        torch, p = self.torch, self.p
+        dt = torch.float16 if p.outputType == self.pa.HALF else torch.float32
+        o_ext = torch.empty((p.batchSize, p.getNumOutputChans(),
+                             *p.getOutputFieldShape()), dtype=dt,
+                            device="cuda:0")
+        self.plan.acts_to_external(self.outputs[k].data_ptr(),
+                                   o_ext.data_ptr(),
+                                   torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        return o_ext.cpu().numpy().astype(np.float64)
+
+    def oracle_inputs(self, images):
+        """The rounded inputs as float64, for the oracle."""
+        import oracle
+        a, w = self.a_ext_host[images], self.w_ext_host
+        if self.p.inputType == self.pa.QUARTER:
+            return (oracle.quarter_to_double(a.numpy(), self.in_meta),
+                    oracle.quarter_to_double(w.numpy(), self.w_meta))
+        return a.double().numpy(), w.double().numpy()
+
+
+def time_steps(torch, runner, steps, warmup):
+    """Returns (wall seconds for `steps` steps, mean kernel seconds per launch
+    from HIP events on the launch stream, how the steps were issued)."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            runner.launch(i)
+        stream.synchronize()
+        # The steps are recorded once into a HIP graph and replayed, so that
+        # what is timed is the GPU work and not the Python launch loop.
+        mode = "hipGraph replay of the recorded steps"
+        graph = torch.cuda.CUDAGraph()
+        try:
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(steps):
+                    runner.launch(warmup + i)
+            graph.replay()  # untimed: instantiation + first upload
+            stream.synchronize()
+        except Exception as e:  # capture unsupported: eager launches
+            graph = None
+            mode = f"eager launches (graph capture failed: {e})"
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record(stream)
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                runner.launch(warmup + i)
+        stop.record(stream)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        kernel = start.elapsed_time(stop) * 1e-3 / steps
+    return wall, kernel, mode
+
+
+def parity(runner, images, tol):
+    import oracle
+    runner.launch(0)
+    got = runner.output_external(0)
+    acts, weights = runner.oracle_inputs(images)
+    one = runner.pa.ConvParams.from_c(runner.p.to_c())
+    one.batchSize = len(images)
+    want = oracle.convolution(one, acts, weights, threads=os.cpu_count() or 1)
+    err = (np.linalg.norm((got[images] - want).ravel())
+           / np.linalg.norm(want.ravel()))
+    if not err <= tol:
+        raise SystemExit(f"parity check failed: rel-L2 {err} > {tol}")
+    return float(err)
+
+
+def cpu_baseline(runner, budget_s=12.0):
+    """Times the single-threaded CPU oracle (a port of the reference's
+    poplibs_test::conv::convolution) on a bounded sample of the same
+    workload: the first n images of the batch."""
+    import oracle
+    p = runner.p
+    one = runner.pa.ConvParams.from_c(p.to_c())
+    one.batchSize = 1
+    acts, weights = runner.oracle_inputs([0])
+    t0 = time.perf_counter()
+    oracle.convolution(one, acts, weights, threads=1)
+    t1 = time.perf_counter() - t0
+    n = int(max(1, min(p.batchSize, round(budget_s / max(t1, 1e-3)))))
+    sample = runner.pa.ConvParams.from_c(p.to_c())
+    sample.batchSize = n
+    acts, weights = runner.oracle_inputs(list(range(n)))
+    t0 = time.perf_counter()
+    oracle.convolution(sample, acts, weights, threads=1)
+    t = time.perf_counter() - t0
+    return {"value": round(sample.getFwdFlops() / t / 1e12, 6),
+            "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"first {n} of {p.batchSize} images of the same "
+                      f"workload, {t:.2f} s, double precision, 1 thread"}
+
+
+def measured_traffic(key):
+    """HBM bytes per launch from committed rocprofv3 counter runs, if any."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(key, {}).get("bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2",
+                    help="headline workload (c2, c3, c4, c5)")
+    ap.add_argument("--only", action="store_true",
+                    help="skip the other workloads and the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no "
+                         "multi-GPU path, run with --gpus 1")
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU; there is no CPU fallback")
+    import poplibs_amd as pa
+    from poplibs_amd import capi
+    pa.lib()
+    wls = _workloads(pa)
+
+    def measure(key, steps, warmup):
+        wl = wls[key]
+        # HBM-bound workloads rotate over enough buffer sets to exceed the
+        # 256 MB Infinity Cache, so that reads really come from HBM.
+        probe = Runner(pa, capi, torch, wl, sets=1)
+        sets = 1
+        if wl["bound"] == "hbm":
+            sets = max(1, -(-300 * 2 ** 20 // probe.bytes))
+        runner = probe if sets == 1 else Runner(pa, capi, torch, wl, sets=sets)
+        tol = 3e-2 if wl["dtype"] == "fp8" else 1e-3
+        err = parity(runner, [0, wl["params"].batchSize - 1], tol)
+        wall, kernel, mode = time_steps(torch, runner, steps, warmup)
+        if wl["bound"] == "mfma":
+            achieved = runner.flops / kernel / 1e12
+            peak, unit = PEAK_TFLOPS[wl["dtype"]], "TFLOP/s"
+        else:
+            achieved = runner.bytes / kernel / 1e9
+            peak, unit = PEAK_HBM_GBS, "GB/s"
+        return dict(
+            runner=runner, wall=wall, kernel=kernel, mode=mode, err=err,
+            sets=sets,
+            roofline={"bound": wl["bound"], "achieved": round(achieved, 3),
+                      "peak": peak, "unit": unit,
+                      "frac": round(achieved / peak, 4),
+                      "traffic": measured_traffic(key),
+                      "kernel_us": round(kernel * 1e6, 3),
+                      "algorithmic_per_launch":
+                          runner.flops if wl["bound"] == "mfma"
+                          else runner.bytes})
+
+    head = measure(args.workload, args.steps, args.warmup)
+    wl, runner = wls[args.workload], head["runner"]
+    tflops = runner.flops * args.steps / head["wall"] / 1e12
+    line = {
+        "metric": "conv fwd TFLOP/s + % MFMA peak (fp16 3x3 N=32 28x28 "
+                  "C=128); depthwise GB/s",
+        "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["wall"] * 1e3 / args.steps, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": wl["dtype"], "data": "synthetic",
+        "config": {"workload": wl["name"], "flops_per_step": runner.flops,
+                   "bytes_per_step": runner.bytes,
+                   "issue": head["mode"], "buffer_sets": head["sets"],
+                   "parity_rel_l2_vs_oracle": head["err"]},
+        "roofline": head["roofline"],
+    }
+    if not args.only:
+        others = {}
+        for key in wls:
+            if key == args.workload:
+                continue
+            m = measure(key, args.steps, args.warmup)
+            r = m["runner"]
+            others[key] = {
+                "workload": wls[key]["name"],
+                "ms_per_step": round(m["wall"] * 1e3 / args.steps, 6),
+                "tflops": round(r.flops * args.steps / m["wall"] / 1e12, 3),
+                "gbytes_per_s": round(r.bytes * args.steps / m["wall"] / 1e9,
+                                      1),
+                "buffer_sets": m["sets"],
+                "parity_rel_l2_vs_oracle": m["err"],
+                "roofline": m["roofline"]}
+            del m, r
+            torch.cuda.empty_cache()
+        line["other_workloads"] = others
+        line["cpu_baseline"] = cpu_baseline(runner)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
