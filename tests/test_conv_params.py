@@ -1,0 +1,438 @@
+"""Host-side descriptor algebra (ConvParams, ConvUtil, MAC counting, options,
+planner) exercised through the C ABI; no GPU needed.  Known answers come from
+the reference's own unit tests (cited), the rest is pinned by brute force
+against an independent Python statement of the index definition."""
+import os
+import random
+
+import numpy as np
+import pytest
+
+import poplibs_amd as pa
+from poplibs_amd import MxconvError, Status
+from helpers import (NONE, input_index_def, make_params, output_size_def,
+                     random_data, random_params)
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+# ---- known answers held by the reference's tests --------------------------
+
+def test_getInputRange_flip_acts_and_weights():
+    # tests/poplin/ConvUtilTest.cpp:14-32
+    p = pa.ConvParams(pa.FLOAT, None, 1, [3, 1], [5, 1], 1, 1, 1)
+    p.inputTransform.paddingLower = [2, 0]
+    p.inputTransform.paddingUpper = [2, 0]
+    p.inputTransform.flip = [True, False]
+    p.kernelTransform.flip = [True, False]
+    assert p.getInputRange(0, (0, 2), 1) == (0, 2)
+
+
+def test_getKernelRange_truncate_input():
+    # tests/poplin/ConvUtilTest.cpp:34-51
+    p = pa.ConvParams(pa.FLOAT, None, 1, [3], [4], 1, 1, 1)
+    p.inputTransform.truncationUpper = [1]
+    p.inputTransform.dilation = [2]
+    p.inputTransform.paddingLower = [1]
+    assert p.getKernelRange(0, (0, 1), (0, 3)) == (1, 4)
+
+
+def test_read_conv_params_from_json():
+    # tests/poplin/ConvTest.cpp:651-682
+    uut = pa.ConvParams.from_json("""
+    {
+      "dataType": "float",
+      "batchSize": 1,
+      "numConvGroups": 2,
+      "inputChannelsPerConvGroup": 3,
+      "outputChannelsPerConvGroup": 4,
+      "kernelShape": [50, 60],
+      "inputFieldShape": [70, 80],
+      "inputTransform": {
+        "truncationLower": [1, 2],
+        "paddingUpper": [3, 4],
+        "flip": [true, false]
+      },
+      "outputTransform": {
+        "stride": [5, 6]
+      }
+    }""")
+    expected = pa.ConvParams(pa.FLOAT, None, 1, [70, 80], [50, 60], 3, 4, 2)
+    expected.inputTransform.truncationLower = [1, 2]
+    expected.inputTransform.paddingUpper = [3, 4]
+    expected.inputTransform.flip = [True, False]
+    expected.outputTransform.stride = [5, 6]
+    assert uut == expected
+    assert uut.compare(expected) == 0 and uut.hash() == expected.hash()
+
+
+def test_json_fixtures_of_the_reference():
+    dw = pa.ConvParams.from_json(
+        open(os.path.join(GOLDEN, "depthwise_conv_half.json")).read())
+    assert dw == pa.ConvParams(pa.HALF, None, 1, [28, 28], [5, 5], 1, 1, 24)
+    pw = pa.ConvParams.from_json(
+        open(os.path.join(GOLDEN, "pointwise_conv_float.json")).read())
+    assert pw == pa.ConvParams(pa.FLOAT, None, 2, [17, 32], [1, 1], 16, 25, 1)
+    assert pw.getOutputFieldShape() == [17, 32]
+
+
+def test_json_input_output_types_and_errors():
+    p = pa.ConvParams.from_json(
+        '{"inputType": "quarter", "outputType": "half", "batchSize": 2,'
+        ' "numConvGroups": 1, "inputChannelsPerConvGroup": 16,'
+        ' "outputChannelsPerConvGroup": 8, "inputFieldShape": [4],'
+        ' "kernelShape": [1], "kernelTransform": {"dilation": [3]}}')
+    assert (p.inputType, p.outputType) == (pa.QUARTER, pa.HALF)
+    assert p.kernelTransform.dilation == [3]
+    with pytest.raises(MxconvError) as e:  # lib/poplin/ConvParams.cpp:417-420
+        pa.ConvParams.from_json('{"inputFieldShape": [4, 4], "kernelShape": [1]}')
+    assert e.value.status == Status.INVALID_PARAMS
+    with pytest.raises(MxconvError):
+        pa.ConvParams.from_json('{"dataType": "double"}')
+    with pytest.raises(MxconvError):
+        pa.ConvParams.from_json('{"batchSize": ')
+
+
+def test_validate_options():
+    # tests/poplin/ConvTest.cpp:684-698
+    pa.validate_options({"partialsType": "half"})
+    for bad in ({"partialsType": "invalid_value"}, {"invalid_key": "half"}):
+        with pytest.raises(MxconvError) as e:
+            pa.validate_options(bad)
+        assert e.value.status == Status.INVALID_OPTION
+    pa.validate_options({"pass": "TRAINING_FWD",
+                         "availableMemoryProportion": "0.4",
+                         "enableFastReduce": "true"})
+    for bad in ({"pass": "FWD"}, {"availableMemoryProportion": "-1"},
+                {"enableFastReduce": "maybe"}):
+        with pytest.raises(MxconvError):
+            pa.validate_options(bad)
+
+
+def _pc(text):
+    pa.validate_options({"planConstraints": text})
+
+
+def _pc_bad(text):
+    with pytest.raises(MxconvError) as e:
+        _pc(text)
+    assert e.value.status == Status.INVALID_OPTION
+
+
+def test_plan_constraints_structure():
+    # tests/poplin/ConvOptionsTest.cpp:12-107 restated on the JSON form
+    _pc('{}')
+    _pc('{"0": {}}')
+    _pc('{"0": {}, "2": {}, " 5": {}}')
+    _pc_bad('{"": {}}')
+    _pc_bad('{"-1": {}}')
+    _pc_bad('{"a watched pot never boils": {}}')
+    _pc_bad('0')
+    # partition variables per dimension
+    _pc('{"0": {"partition": {"fieldSplit": {"0": 4, "2": 5}}}}')
+    _pc_bad('{"0": {"partition": {"fieldSplit": '
+            '{"5": "a watched pot never boils"}}}}')
+    _pc_bad('{"0": {"partition": {"fieldSplit": 0}}}')
+    _pc_bad('{"0": {"partition": {"fieldSplit": {"hello": "world"}}}}')
+    # split variables
+    _pc('{"0": {"partition": {"inChanSplit": {"serial": 4, "parallel": 5}}}}')
+    _pc_bad('{"0": {"partition": {"inChanSplit": '
+            '{"serial": "a watched pot never boils"}}}}')
+    _pc_bad('{"0": {"partition": {"outChanSplit": {"hello": "world"}}}}')
+    # transform
+    _pc('{"0": {"transform": {"swapOperands": false}}}')
+    _pc_bad('{"0": {"transform": {"a watched pot never boils": {}}}}')
+    _pc_bad('{"0": {"transform": {"swapOperands": '
+            '"a watched pot never boils"}}}')
+    _pc_bad('{"0": {"transform": 0}}')
+    # partition scalars
+    _pc('{"0": {"partition": {"convGroupSplit": 4}}}')
+    _pc_bad('{"0": {"partition": {"a watched pot never boils": {}}}}')
+    _pc_bad('{"0": {"partition": {"convGroupSplit": '
+            '"a watched pot never boils"}}}')
+    _pc_bad('{"0": {"something": {}}}')
+    # method (lib/poplin/ConvOptions.cpp:275-299)
+    for m in ("AMP", "SLIC", "HMAC", "VMAC", "OUTER_PRODUCT"):
+        _pc('{"method": {"type": "%s"}}' % m)
+    _pc_bad('{"method": {"type": "WINOGRAD"}}')
+    # the complete constraint of tests/poplin/ConvPlanTest.cpp:155-175
+    _pc('''{"method": {"type": "HMAC"}, "inChansPerGroup": 1,
+            "partialChansPerGroup": 1,
+            "0": {"transform": {"swapOperands": false, "expandDims": [],
+                                "outChanFlattenDims": []},
+                  "partition": {"fieldSplit": {"0": 1, "1": 1},
+                                "batchSplit": 1,
+                                "outChanSplit": {"parallel": 1, "serial": 1},
+                                "kernelSplit": {"0": 1, "1": 1},
+                                "inChanSplit": {"parallel": 1, "serial": 1},
+                                "convGroupSplit": 1}}}''')
+
+
+# ---- validate (lib/poplin/ConvParams.cpp:172-266) -------------------------
+
+@pytest.mark.parametrize("mutate,fragment", [
+    (lambda p: p.kernelShape.append(1), "kernel field dimensions"),
+    (lambda p: p.outputTransform.stride.__setitem__(0, 0), "Stride"),
+    (lambda p: p.inputTransform.dilation.__setitem__(1, 0), "Input dilation"),
+    (lambda p: p.kernelTransform.dilation.__setitem__(0, 0),
+     "Kernel dilation"),
+    (lambda p: p.inputTransform.paddingLower.append(0), "dimensions"),
+    (lambda p: p.inputTransform.truncationLower.__setitem__(0, 9),
+     "more than the size of the field"),
+    (lambda p: p.kernelTransform.truncationUpper.__setitem__(1, 4),
+     "more than the size of the kernel"),
+    (lambda p: (p.kernelTransform.truncationLower.__setitem__(0, 3)),
+     "zero size"),
+    (lambda p: p.kernelTransform.dilation.__setitem__(0, 5),
+     "less than the transformed kernel"),
+    (lambda p: p.outputTransform.truncationLower.__setitem__(0, 7),
+     "Output truncation"),
+])
+def test_validate_rejects(mutate, fragment):
+    p = make_params(field=(8, 8), kernel=(3, 3))
+    p.validate()
+    mutate(p)
+    with pytest.raises(MxconvError) as e:
+        p.validate()
+    assert e.value.status == Status.INVALID_PARAMS
+    assert fragment in e.value.message, e.value.message
+
+
+# ---- sizes: closed forms (lib/poplin/ConvParams.cpp:631-698) --------------
+
+def test_baseline_config_sizes_and_flops():
+    c1 = make_params(pa.FLOAT, field=(32, 32), kernel=(3, 3), ci=16, co=16,
+                     pad=1)
+    c2 = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                     co=128, pad=1)
+    c3 = make_params(pa.HALF, batch=32, field=(56, 56), kernel=(1, 1), ci=256,
+                     co=64)
+    c4 = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                     groups=96, stride=2, pad=1)
+    c5 = make_params(pa.QUARTER, pa.HALF, batch=64, field=(14, 14),
+                     kernel=(3, 3), ci=256, co=256, pad=1)
+    assert [c.getOutputFieldShape() for c in (c1, c2, c3, c4, c5)] == [
+        [32, 32], [28, 28], [56, 56], [56, 56], [14, 14]]
+    assert [c.getFwdFlops() for c in (c1, c2, c3, c4, c5)] == [
+        4524032, 7050625024, 3288334336, 171350016, 13421772800]
+    # closed form for 3x3 pad 1 on HxW: sum over taps of valid outputs
+    assert c2.getNumberOfMACs() == 32 * 128 * 128 * (28 + 27 + 27) ** 2
+    # c4: stride 2 over 112 with pad 1: rows k=0 -> 55 outputs, k=1,2 -> 56
+    assert c4.getNumberOfMACs() == 32 * 96 * (55 + 56 + 56) ** 2
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_sizes_match_definition_fuzz(seed):
+    p = random_params(random.Random(seed), max_dims=4, max_field=9)
+    for d in range(p.getNumFieldDims()):
+        assert p.getOutputSize(d) == output_size_def(p, d)
+        it = p.inputTransform
+        trunc = p.inputFieldShape[d] - it.truncationLower[d] \
+            - it.truncationUpper[d]
+        assert p.getTruncatedInputSize(d) == trunc
+        dil = 0 if trunc == 0 else 1 + (trunc - 1) * it.dilation[d]
+        assert p.getTransformedInputSize(d) == \
+            it.paddingLower[d] + dil + it.paddingUpper[d]
+        assert p.getUntransformedOutputSize(d) == \
+            p.getTransformedInputSize(d) - p.getTransformedKernelSize(d) + 1
+
+
+# ---- index and range algebra against brute force --------------------------
+
+@pytest.mark.parametrize("seed", range(40))
+def test_index_and_ranges_match_brute_force(seed):
+    rng = random.Random(100 + seed)
+    p = random_params(rng, max_dims=2, max_field=8)
+    for d in range(p.getNumFieldDims()):
+        O, K, I = p.getOutputSize(d), p.kernelShape[d], p.inputFieldShape[d]
+        table = {}
+        for o in range(O):
+            for k in range(K):
+                want = input_index_def(p, d, o, k)
+                got = p.getInputIndex(d, o, k)
+                assert got == (NONE if want is None else want)
+                if want is not None:
+                    table[(o, k)] = want
+                    assert p.getKernelIndex(d, o, want) == k
+        for o in range(O):
+            for i in range(I):
+                ks = [k for k in range(K) if table.get((o, k)) == i]
+                got = p.getKernelIndex(d, o, i)
+                assert got == (ks[0] if ks else NONE)
+
+        def span(values):
+            values = list(values)
+            return (min(values), max(values) + 1) if values else (0, 0)
+
+        for _ in range(6):
+            o0 = rng.randint(0, O)
+            o1 = rng.randint(o0, O)
+            k0 = rng.randint(0, K)
+            k1 = rng.randint(k0, K)
+            i0 = rng.randint(0, I)
+            i1 = rng.randint(i0, I)
+            pairs = [(o, k, i) for (o, k), i in table.items()
+                     if o0 <= o < o1]
+            assert p.getOutputRangeForKernelRange(d, (o0, o1), (k0, k1)) == \
+                span(o for o, k, i in pairs if k0 <= k < k1)
+            assert p.getOutputRangeForInputRange(d, (o0, o1), (i0, i1)) == \
+                span(o for o, k, i in pairs if i0 <= i < i1)
+            assert p.getInputRange(d, (o0, o1), (k0, k1)) == \
+                span(i for o, k, i in pairs if k0 <= k < k1)
+            assert p.getKernelRange(d, (o0, o1), (i0, i1)) == \
+                span(k for o, k, i in pairs if i0 <= i < i1)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_number_of_macs_counts_index_pairs(seed):
+    """getNumberOfMACs == number of (o, k) pairs per dimension with an input
+    element, times channels (lib/poplin/PerformanceEstimation.hpp:1641-1666).
+    The reference's formula divides a range size by a stride, which equals the
+    pair count whenever the participating outputs of a kernel index are
+    evenly spaced - true for every parameter set."""
+    p = random_params(random.Random(200 + seed), max_dims=3, max_field=9)
+    want = (p.numConvGroups * p.batchSize * p.outputChannelsPerConvGroup
+            * p.inputChannelsPerConvGroup)
+    for d in range(p.getNumFieldDims()):
+        want *= sum(input_index_def(p, d, o, k) is not None
+                    for o in range(p.getOutputSize(d))
+                    for k in range(p.kernelShape[d]))
+    assert p.getNumberOfMACs() == want
+    assert p.getFwdFlops() == 2 * want
+
+
+# ---- canonicalize (lib/poplin/ConvParams.cpp:468-629) ---------------------
+
+@pytest.mark.parametrize("seed", range(50))
+def test_canonicalize_invariants(oracle, seed):
+    p = random_params(random.Random(300 + seed), max_dims=3, max_field=7)
+    c = p.canonicalize()
+    c.validate()
+    # shapes preserved (lib/poplin/ConvParams.cpp:626), idempotent
+    # (lib/poplin/CanonicalConvParams.hpp:15-19)
+    assert c.getOutputFieldShape() == p.getOutputFieldShape()
+    assert (c.inputFieldShape, c.kernelShape) == (p.inputFieldShape,
+                                                  p.kernelShape)
+    assert c.canonicalize() == c
+    # and it is the same function of the data
+    acts, weights, biases = random_data(p, seed)
+    np.testing.assert_array_equal(
+        oracle.convolution(c, acts, weights, biases),
+        oracle.convolution(p, acts, weights, biases))
+    assert c.getNumberOfMACs() == p.getNumberOfMACs()
+
+
+def test_canonicalize_known_forms():
+    # config 4: the upper padding row/column is never read
+    c4 = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                     groups=96, stride=2, pad=1).canonicalize()
+    assert c4.inputTransform.paddingLower == [1, 1]
+    assert c4.inputTransform.paddingUpper == [0, 0]
+    assert c4.outputTransform.stride == [2, 2]
+    # one output element: stride collapses to 1
+    p = make_params(field=(5,), kernel=(5,), stride=3).canonicalize()
+    assert p.outputTransform.stride == [1]
+    # flip of a single surviving element is dropped, paddings swap
+    p = make_params(field=(4,), kernel=(1,), itl=1, itu=2, flipIn=True,
+                    padLower=2, padUpper=0, idil=3).canonicalize()
+    assert p.inputTransform.flip == [False]
+    assert p.inputTransform.dilation == [1]
+    # all-zero output -> the zero convolution of getZeroConv
+    z = make_params(field=(2,), kernel=(1,), padLower=4, otu=4)
+    assert z.isZeroConvolution()
+    zc = z.canonicalize()
+    assert zc.inputTransform.truncationUpper == [2]
+    assert zc.kernelTransform.truncationUpper == [1]
+    assert zc.outputTransform.paddingUpper == zc.getOutputFieldShape()
+    assert not make_params(field=(4,), kernel=(2,)).isZeroConvolution()
+    assert make_params(field=(4,), kernel=(2,), ci=0).isZeroConvolution()
+
+
+# ---- ordering, hashing, printing ------------------------------------------
+
+def test_compare_hash_and_print():
+    a = make_params(field=(4, 4), kernel=(3, 3), pad=1)
+    b = make_params(field=(4, 4), kernel=(3, 3), pad=1)
+    c = make_params(field=(4, 4), kernel=(3, 3), pad=1, stride=2)
+    assert a.compare(b) == 0 and a.hash() == b.hash()
+    assert a.compare(c) != 0 and a.compare(c) == -c.compare(a)
+    assert a.hash() != c.hash()
+    text = str(c)
+    # fixed layout of lib/poplin/ConvParams.cpp:292-363
+    assert text.startswith("\n  Params:\n        inputType                  "
+                           "float\n")
+    assert "        stride                     {2,2}\n" in text
+    assert "        flipInput                  {0,0}\n" in text
+    assert text.endswith("        outputFieldShape           {2,2}\n")
+
+
+# ---- planner --------------------------------------------------------------
+
+def _kernel_of(p, options=None):
+    text = pa.Plan(p, options).describe()
+    for name in ("implicit GEMM", "depthwise direct", "generic direct"):
+        if name in text:
+            return name
+    raise AssertionError(text)
+
+
+def test_planner_choices():
+    c1 = make_params(pa.FLOAT, field=(32, 32), kernel=(3, 3), ci=16, co=16,
+                     pad=1)
+    c2 = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                     co=128, pad=1)
+    c4 = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                     groups=96, stride=2, pad=1)
+    c5 = make_params(pa.QUARTER, pa.HALF, batch=64, field=(14, 14),
+                     kernel=(3, 3), ci=256, co=256, pad=1)
+    assert _kernel_of(c1) == "generic direct"      # fp32 inputs
+    assert _kernel_of(c2) == "implicit GEMM"
+    assert _kernel_of(c4) == "depthwise direct"
+    assert _kernel_of(c5) == "implicit GEMM"
+    # transforms outside the fast subset fall back
+    assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
+                                  co=8, idil=2)) == "generic direct"
+    assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
+                                  co=8, flipK=True)) == "generic direct"
+    assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
+                                  ci=8, co=8)) == "generic direct"
+    assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=4,
+                                  co=8)) == "generic direct"
+    # method names of the reference steer the choice
+    hmac = {"planConstraints": '{"method": {"type": "HMAC"}}'}
+    assert _kernel_of(c2, hmac) == "generic direct"
+    assert _kernel_of(c4, {"planConstraints":
+                           '{"method": {"type": "AMP"}}'}) == "depthwise direct"
+    forced = {"planConstraints": '{"gfx950": {"kernel": "generic"}}'}
+    assert _kernel_of(c2, forced) == "generic direct"
+    with pytest.raises(MxconvError) as e:
+        pa.Plan(c1, {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'})
+    assert e.value.status == Status.INVALID_OPTION
+    with pytest.raises(MxconvError):
+        pa.Plan(c2, {"planConstraints": '{"gfx950": {"blockM": 96}}'})
+
+
+def test_plan_buffers_and_type_rules():
+    from poplibs_amd import capi
+    c2 = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                     co=128, pad=1)
+    plan = pa.Plan(c2)
+    assert plan.buffer_bytes(capi.BUF_INPUT) == 6422528
+    assert plan.buffer_bytes(capi.BUF_WEIGHTS_EXTERNAL) == 294912
+    assert plan.buffer_bytes(capi.BUF_OUTPUT) == 6422528
+    assert plan.buffer_bytes(capi.BUF_BIAS) == 256
+    # quarter input requires half output (lib/poplin/ConvValidation.cpp:55-61)
+    bad = make_params(pa.QUARTER, pa.FLOAT, field=(4, 4), kernel=(1, 1), ci=16,
+                      co=16)
+    with pytest.raises(MxconvError) as e:
+        pa.Plan(bad)
+    assert e.value.status == Status.INVALID_PARAMS
+    # invalid parameters are rejected at planning time
+    with pytest.raises(MxconvError):
+        pa.Plan(make_params(field=(2, 2), kernel=(3, 3)))
+    # fwd on a quarter plan needs the metadata entry point; no GPU touched
+    q = pa.Plan(make_params(pa.QUARTER, pa.HALF, field=(4, 4), kernel=(1, 1),
+                            ci=16, co=16))
+    with pytest.raises(MxconvError) as e:
+        q.fwd(1, 1, 1)
+    assert "mxconv_fwd_quarter" in e.value.message
