@@ -10,16 +10,41 @@
 // Both operands are therefore contiguous along K in memory, which is how an
 // MFMA lane wants them: 16 bytes = 8 halves (or 16 fp8) of consecutive k.
 //
-// Workgroup: 256 threads = 4 wave64, tile 128 (M) x BN (N), BN = 64 or 128,
-// K step of 64 bytes per row (32 halves / 64 fp8).  Each k-step the
-// workgroup gathers the im2col A tile and the B tile with 16-byte global
-// loads (coalesced along channels, NHWC), stages them in LDS (double
-// buffered, rows padded from 64 to 80 bytes so that the 16 lanes of one LDS
-// read phase hit 64 distinct banks), and each wave multiplies its 64 x BN/2
-// sub-tile with v_mfma_f32_32x32x16_f16 (fp16) or
-// v_mfma_f32_32x32x64_f8f6f4 (fp8), accumulating in fp32.  The next k-step's
-// global loads are issued before the current step's MFMAs so that HBM/L2
-// latency hides behind the matrix cores.
+// Workgroup: 512 threads = 8 wave64, tile 128 (M) x BN (N), BN = 64 or 128,
+// K step of 128 bytes per row (64 halves / 128 fp8).
+//
+// Producer / consumer waves.  Waves 4-7 only move data; waves 0-3 only feed
+// the matrix cores (and run the epilogue); each SIMD holds one of each kind,
+// so MFMAs and memory instructions overlap even when the problem offers no
+// more than one workgroup per CU.  The two kinds meet at one workgroup
+// barrier per k-step.
+//
+// Data path.  Every k-step the producers gather the im2col A tile and the B
+// tile with 16-byte buffer loads that write straight into LDS
+// (buffer_load_dwordx4 ... lds): no staging registers, so the depth of the
+// prefetch is set by LDS capacity - all stages but one are in flight while
+// one is being multiplied.  Such a load puts lane l's 16 bytes at LDS base +
+// 16 l, i.e. one instruction fills 8 consecutive 128-byte tile rows.  To keep
+// the consumers' MFMA-operand reads (32 rows, same k) free of bank conflicts
+// the 16-byte chunks of row r are stored at position (chunk ^ (r & 7)); the
+// permutation is applied on the global side, by choosing which chunk each
+// lane fetches, and undone in the LDS read address.
+// Each consumer wave multiplies its 64 x BN/2 sub-tile with
+// v_mfma_f32_32x32x16_f16 (fp16) or v_mfma_f32_32x32x64_f8f6f4 (fp8),
+// accumulating in fp32.
+//
+// Addressing.  Everything per-row is computed once, before the loop: a byte
+// offset and a bit mask "kernel tap t reads inside the input".  In the loop
+// the wave-uniform part of the address (kernel tap, channel block) travels in
+// the scalar offset of the buffer load, and a row whose tap falls on padding
+// gets an out-of-range vector offset, for which the buffer unit delivers
+// zeros - no branch and no select on data.  When a k-step spans several
+// kernel taps (fewer than 128 bytes of channels per tap) the tap is per-lane
+// and the offsets are formed in vector registers.
+//
+// Epilogue.  The accumulators are scaled, biased, converted and written to
+// LDS, then all 8 waves copy whole 16-byte vectors to the channels-last
+// output, so that every store instruction covers full rows of the tile.
 //
 // This takes the role of PopLibs' AMP vertices ConvPartial1x1Out /
 // ConvPartialnx1 (lib/poplin/codelets/ConvPartial1x1Out.cpp:49-173,
@@ -29,17 +54,33 @@
 #include "device_types.hpp"
 #include "kernels.hpp"
 
+#include <type_traits>
+
 namespace mxk {
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+/// Compile-time loop: body(std::integral_constant<int, I>) for I in [0, N).
+template <int I, int N, class F>
+__device__ __forceinline__ void staticFor(F &&body) {
+  if constexpr (I < N) {
+    body(std::integral_constant<int, I>{});
+    staticFor<I + 1, N>(body);
+  }
+}
 
 constexpr int kBlockM = 128;
-constexpr int kRowBytes = 64;  // bytes of K per tile row and k-step
-constexpr int kLdsRow = 80;    // padded LDS row pitch
-constexpr int kThreads = 256;
+constexpr int kRowBytes = 128; // bytes of K per tile row and k-step
+constexpr int kThreads = 512;  // 4 consumer + 4 producer waves
+constexpr int kProducers = 256; // threads that move data
+constexpr int kChunks = kRowBytes / 16; // 16-byte chunks per row
+constexpr int kRowsPerPass = kProducers / kChunks; // rows per producer pass
+constexpr int kLoadBytes = 64 * 16; // LDS bytes one wave-wide load fills
+constexpr uint32_t kOutOfRange = 0x80000000u; // beyond any buffer we accept
 
 struct IgemmArgs {
   IgemmDesc d;
@@ -48,6 +89,8 @@ struct IgemmArgs {
   uint32_t kSteps;   // kPadded / elements per k-step
   uint32_t kPadded;  // row length of the packed weights, in elements
   uint32_t coPadded; // rows per group of the packed weights
+  uint32_t inBytes;  // size of the input tensor
+  uint32_t wBytes;   // size of the packed weights
 };
 
 /// Workgroups are dealt round-robin over the 8 XCDs, each with its own L2.
@@ -59,25 +102,72 @@ __device__ __forceinline__ uint32_t xcdSwizzle(uint32_t bid, uint32_t total) {
   return xcd * q + (xcd < rem ? xcd : rem) + idx;
 }
 
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t bufferOf(const void *p,
+                                                           uint32_t bytes) {
+  // Raw (stride 0) buffer of `bytes` bytes; 32-bit data format.
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), short(0),
+                                           int(bytes), 0x00020000);
+}
+
+/// `wait until at most n vector-memory operations are outstanding`, leaving
+/// the other counters alone (gfx9 encoding of s_waitcnt).
+#define MXK_WAIT_VMCNT(n)                                                      \
+  __builtin_amdgcn_s_waitcnt(((n)&15) | (((n) >> 4) << 14) | (7 << 4) |       \
+                             (15 << 8))
+
+/// Wait for this wave's LDS reads (and scalar loads) only.
+#define MXK_WAIT_LGKMCNT0() __builtin_amdgcn_s_waitcnt(0xC07F)
+
+/// Workgroup barrier without the release / acquire fences of
+/// __syncthreads().  Those fences would drain every outstanding buffer load
+/// (a load that writes LDS counts as a pending LDS write) at each k-step and
+/// with it the whole prefetch queue.  The callers wait for exactly what the
+/// other side needs - producers: the oldest stage's loads; consumers: their
+/// own LDS reads - before arriving here.
+__device__ __forceinline__ void stepBarrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+using LdsPtr = __attribute__((address_space(3))) void *;
+
+/// 16 bytes per lane from a buffer straight into LDS: lane l's data lands at
+/// dst + 16 l (dst is wave-uniform).  Out-of-range offsets deliver zeros.
+/// The builtin exists for the GPU target only; the host compilation pass,
+/// which merely needs the kernels' launch stubs, sees an empty body.
+__device__ __forceinline__ void loadToLds(__amdgpu_buffer_rsrc_t buffer,
+                                          LdsPtr dst, uint32_t vectorOffset,
+                                          uint32_t scalarOffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, dst, 16, vectorOffset,
+                                           scalarOffset, 0, 0);
+#endif
+}
+
 template <int EB> struct Mma;
 
-/// fp16: two K=16 steps per 64-byte row.
+/// Tile rows in LDS are 128 bytes, chunk c of row r at chunk position
+/// c ^ (r & 7).  `row` = lane & 31 is the row inside a 32-row block (block
+/// bases are multiples of 8, so r & 7 == lane & 7).
+
+/// fp16: K=16 steps of 32 bytes (two chunks, one per half-wave) per row.
 template <> struct Mma<2> {
   template <int TN, int FA, int FB>
   static __device__ __forceinline__ void
   step(const char *ldsA, const char *ldsB, int lane, floatx16 (&acc)[2][TN]) {
-    const int row = lane & 31, kb = (lane >> 5) * 16;
+    const int row = lane & 31;
+    const int swz = lane & 7, half = lane >> 5;
 #pragma unroll
-    for (int s = 0; s != 2; ++s) {
+    for (int s = 0; s != kRowBytes / 32; ++s) {
+      const int off = row * kRowBytes + (((s * 2 + half) ^ swz) << 4);
       half8 a[2], b[TN];
 #pragma unroll
       for (int i = 0; i != 2; ++i)
-        a[i] = *reinterpret_cast<const half8 *>(ldsA + (i * 32 + row) * kLdsRow +
-                                                s * 32 + kb);
+        a[i] = *reinterpret_cast<const half8 *>(ldsA + i * 32 * kRowBytes + off);
 #pragma unroll
       for (int j = 0; j != TN; ++j)
-        b[j] = *reinterpret_cast<const half8 *>(ldsB + (j * 32 + row) * kLdsRow +
-                                                s * 32 + kb);
+        b[j] = *reinterpret_cast<const half8 *>(ldsB + j * 32 * kRowBytes + off);
 #pragma unroll
       for (int i = 0; i != 2; ++i)
 #pragma unroll
@@ -88,47 +178,54 @@ template <> struct Mma<2> {
   }
 };
 
-/// fp8: one K=64 step per 64-byte row.  FA / FB: 0 = E4M3, 1 = E5M2 (the
-/// cbsz / blgp operand-format fields of the instruction).
+/// fp8: K=64 steps of 64 bytes (four chunks, two per half-wave) per row.
+/// FA / FB: 0 = E4M3, 1 = E5M2 (the cbsz / blgp operand-format fields).
 template <> struct Mma<1> {
   template <int TN, int FA, int FB>
   static __device__ __forceinline__ void
   step(const char *ldsA, const char *ldsB, int lane, floatx16 (&acc)[2][TN]) {
-    const int row = lane & 31, kb = (lane >> 5) * 32;
-    // 32 bytes per lane, fetched as two 16-byte LDS reads (rows are only
-    // 16-byte aligned).
-    auto load32 = [](const char *p) {
-      const uint4 lo = *reinterpret_cast<const uint4 *>(p);
-      const uint4 hi = *reinterpret_cast<const uint4 *>(p + 16);
-      return intx8{int(lo.x), int(lo.y), int(lo.z), int(lo.w),
-                   int(hi.x), int(hi.y), int(hi.z), int(hi.w)};
-    };
-    intx8 a[2], b[TN];
+    const int row = lane & 31;
+    const int swz = lane & 7, half = lane >> 5;
 #pragma unroll
-    for (int i = 0; i != 2; ++i)
-      a[i] = load32(ldsA + (i * 32 + row) * kLdsRow + kb);
+    for (int s = 0; s != kRowBytes / 64; ++s) {
+      const int c0 = s * 4 + half * 2;
+      const int off0 = row * kRowBytes + ((c0 ^ swz) << 4);
+      const int off1 = row * kRowBytes + (((c0 + 1) ^ swz) << 4);
+      auto load32 = [&](const char *p) {
+        const uintx4 lo = *reinterpret_cast<const uintx4 *>(p + off0);
+        const uintx4 hi = *reinterpret_cast<const uintx4 *>(p + off1);
+        return intx8{int(lo.x), int(lo.y), int(lo.z), int(lo.w),
+                     int(hi.x), int(hi.y), int(hi.z), int(hi.w)};
+      };
+      intx8 a[2], b[TN];
 #pragma unroll
-    for (int j = 0; j != TN; ++j)
-      b[j] = load32(ldsB + (j * 32 + row) * kLdsRow + kb);
-#pragma unroll
-    for (int i = 0; i != 2; ++i)
+      for (int i = 0; i != 2; ++i)
+        a[i] = load32(ldsA + i * 32 * kRowBytes);
 #pragma unroll
       for (int j = 0; j != TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-            a[i], b[j], acc[i][j], FA, FB, 0, 0, 0, 0);
+        b[j] = load32(ldsB + j * 32 * kRowBytes);
+#pragma unroll
+      for (int i = 0; i != 2; ++i)
+#pragma unroll
+        for (int j = 0; j != TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+              a[i], b[j], acc[i][j], FA, FB, 0, 0, 0, 0);
+    }
   }
 };
 
-template <int BN, int EB, int FA, int FB, class OutT>
+/// UNI: every k-step lies inside one kernel tap (Ci * EB is a multiple of
+/// 128 bytes), so tap and channel block are wave-uniform.
+template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
 __global__ __launch_bounds__(kThreads) void igemmKernel(
     IgemmArgs a, const char *__restrict__ in, const char *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out, float scale) {
   constexpr int TN = BN / 64;              // 32-column MFMA tiles per wave
-  constexpr int CE = 16 / EB;              // elements per 16-byte chunk
-  constexpr int BKE = kRowBytes / EB;      // elements per k-step
-  constexpr int BROWS = BN / 64;           // B rows loaded per thread
-  constexpr int kTileBytes = (kBlockM + BN) * kLdsRow;
-  __shared__ __align__(16) char lds[2 * kTileBytes];
+  constexpr int AROWS = kBlockM / kRowsPerPass; // A rows loaded per thread
+  constexpr int BROWS = BN / kRowsPerPass;      // B rows loaded per thread
+  constexpr int kTileBytes = (kBlockM + BN) * kRowBytes; // one stage
+  constexpr int kLoads = AROWS + BROWS; // loads per producer thread and step
+  extern __shared__ __align__(16) char lds[]; // NS * kTileBytes
 
   const IgemmDesc &d = a.d;
   const uint32_t tile = xcdSwizzle(blockIdx.x, gridDim.x);
@@ -137,134 +234,216 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   const uint32_t g = tile / (a.nTiles * a.mTiles);
 
   const int t = threadIdx.x;
-  const int chunk = t & 3, rowBase = t >> 2;
+  const bool producer = t >= kThreads - kProducers; // waves 4-7
   const uint32_t inChans = d.groups * d.inChansPerGroup;
   const uint32_t outChans = d.groups * d.outChansPerGroup;
+  const uint32_t ciBytes = d.inChansPerGroup * EB; // bytes of K per tap
+  const uint32_t pixelBytes = inChans * EB;
+  const uint32_t taps = d.kH * d.kW;
 
-  // The two A rows (output pixels) this thread gathers.
-  const char *rowPtr[2];
-  int ihBase[2], iwBase[2];
-  bool rowValid[2];
-#pragma unroll
-  for (int r = 0; r != 2; ++r) {
-    const uint32_t m = mTile * kBlockM + rowBase + r * 64;
-    rowValid[r] = m < a.M;
-    const uint32_t mm = rowValid[r] ? m : 0;
-    const uint32_t ow = mm % d.outW;
-    const uint32_t oh = (mm / d.outW) % d.outH;
-    const uint32_t b = mm / (d.outW * d.outH);
-    ihBase[r] = int(oh * d.strideH) - d.padH;
-    iwBase[r] = int(ow * d.strideW) - d.padW;
-    rowPtr[r] = in + (size_t(b) * d.inH * d.inW * inChans +
-                      size_t(g) * d.inChansPerGroup) *
-                         EB;
-  }
-  // Position of this thread's chunk inside K, kept as (kh, kw, ci).
-  uint32_t ci = chunk * CE, kw = 0, kh = 0;
-  auto normalise = [&] {
-    while (ci >= d.inChansPerGroup) {
-      ci -= d.inChansPerGroup;
-      if (++kw == d.kW) {
-        kw = 0;
-        ++kh;
-      }
-    }
-  };
-  normalise();
-
-  const char *bPtr = w + ((size_t(g) * a.coPadded + nTile * BN + rowBase) *
-                              a.kPadded +
-                          chunk * CE) *
-                             EB;
-  const size_t bRowSkip = size_t(64) * a.kPadded * EB;
-
-  uint4 aReg[2], bReg[BROWS];
-  auto loadGlobal = [&] {
-    const int ih0 = int(kh * d.dilH), iw0 = int(kw * d.dilW);
-#pragma unroll
-    for (int r = 0; r != 2; ++r) {
-      const int ih = ihBase[r] + ih0, iw = iwBase[r] + iw0;
-      const bool ok = rowValid[r] && kh < d.kH && ih >= int(d.loH) &&
-                      ih < int(d.hiH) && iw >= int(d.loW) && iw < int(d.hiW);
-      aReg[r] = ok ? *reinterpret_cast<const uint4 *>(
-                         rowPtr[r] +
-                         (size_t(uint32_t(ih) * d.inW + uint32_t(iw)) * inChans +
-                          ci) *
-                             EB)
-                   : uint4{0, 0, 0, 0};
-    }
-#pragma unroll
-    for (int r = 0; r != BROWS; ++r)
-      bReg[r] = *reinterpret_cast<const uint4 *>(bPtr + r * bRowSkip);
-  };
-  auto storeLds = [&](int buf) {
-    char *base = lds + buf * kTileBytes + rowBase * kLdsRow + chunk * 16;
-#pragma unroll
-    for (int r = 0; r != 2; ++r)
-      *reinterpret_cast<uint4 *>(base + r * 64 * kLdsRow) = aReg[r];
-#pragma unroll
-    for (int r = 0; r != BROWS; ++r)
-      *reinterpret_cast<uint4 *>(base + (kBlockM + r * 64) * kLdsRow) = bReg[r];
-  };
-  auto advance = [&] {
-    ci += BKE;
-    normalise();
-    bPtr += kRowBytes;
-  };
-
-  const int wave = t >> 6, lane = t & 63;
+  const int wave = (t >> 6) & 3, lane = t & 63;
   const int wm = wave >> 1, wn = wave & 1;
   floatx16 acc[2][TN];
-#pragma unroll
-  for (int i = 0; i != 2; ++i)
-#pragma unroll
-    for (int j = 0; j != TN; ++j)
-#pragma unroll
-      for (int v = 0; v != 16; ++v)
-        acc[i][j][v] = 0.0f;
 
-  loadGlobal();
-  storeLds(0);
-  __syncthreads();
-  for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
-    const int buf = kt & 1;
-    const bool more = kt + 1 != a.kSteps;
-    if (more) {
-      advance();
-      loadGlobal();
+  if (producer) {
+    const int pt = t - (kThreads - kProducers);
+    const int pw = pt >> 6; // producer wave
+    // Lane l of a load fills LDS row (l >> 3) of an 8-row block at chunk
+    // position (l & 7); it therefore fetches chunk (l & 7) ^ (row & 7).
+    const int rowInBlock = lane >> 3;
+    const int chunk = (lane & 7) ^ rowInBlock;
+    // The buffer starts `shift` bytes before the tensor, as many as the
+    // largest amount a padded window reaches above / left of an image, so
+    // that the per-row offset below is never negative: the buffer unit adds
+    // the vector and scalar offsets without wrapping.  Nothing in front of
+    // the tensor is ever read (such taps are masked).
+    const uint32_t shift = (uint32_t(d.padH > 0 ? d.padH : 0) * d.inW +
+                            uint32_t(d.padW > 0 ? d.padW : 0)) *
+                           pixelBytes;
+    const __amdgpu_buffer_rsrc_t inBuf =
+        bufferOf(in - shift, a.inBytes + shift);
+    const __amdgpu_buffer_rsrc_t wBuf = bufferOf(w, a.wBytes);
+
+    // Load r of this wave fills the 8-row block (r * 4 + pw) of the A tile.
+    // Per A row (output pixel) of this thread: the byte offset (from the
+    // shifted buffer start) of the input element under kernel tap (0, 0),
+    // channel chunk `chunk`, and one bit per kernel tap telling whether that
+    // tap reads inside the input.
+    uint32_t rowOff[AROWS], tapMask[AROWS];
+#pragma unroll
+    for (int r = 0; r != AROWS; ++r) {
+      const uint32_t m = mTile * kBlockM + (r * 4 + pw) * 8 + rowInBlock;
+      const bool rowValid = m < a.M;
+      const uint32_t mm = rowValid ? m : 0;
+      const uint32_t ow = mm % d.outW;
+      const uint32_t oh = (mm / d.outW) % d.outH;
+      const uint32_t b = mm / (d.outW * d.outH);
+      const int ihBase = int(oh * d.strideH) - d.padH;
+      const int iwBase = int(ow * d.strideW) - d.padW;
+      rowOff[r] =
+          shift +
+          ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
+              pixelBytes +
+          g * ciBytes + chunk * 16;
+      uint32_t mask = 0;
+      if (rowValid)
+        for (uint32_t kh = 0, tap = 0; kh != d.kH; ++kh) {
+          const int ih = ihBase + int(kh * d.dilH);
+          const bool hOk = ih >= int(d.loH) && ih < int(d.hiH);
+          for (uint32_t kw = 0; kw != d.kW; ++kw, ++tap) {
+            const int iw = iwBase + int(kw * d.dilW);
+            if (hOk && iw >= int(d.loW) && iw < int(d.hiW))
+              mask |= 1u << tap;
+          }
+        }
+      tapMask[r] = mask;
     }
-    const char *ldsA = lds + buf * kTileBytes + wm * 64 * kLdsRow;
-    const char *ldsB =
-        lds + buf * kTileBytes + (kBlockM + wn * (BN / 2)) * kLdsRow;
-    Mma<EB>::template step<TN, FA, FB>(ldsA, ldsB, lane, acc);
-    if (more)
-      storeLds(buf ^ 1);
-    __syncthreads();
-  }
 
-  // Epilogue.  Lane l of a 32x32 accumulator holds column l % 32 and rows
-  // 8 * (v / 4) + 4 * (l / 32) + v % 4 for v = 0..15.
-  const uint32_t col = lane & 31, rowOff = (lane >> 5) * 4;
+    // Position inside K of the data loaded next.  UNI: (tap, byte offset of
+    // the channel block inside the tap) of the whole k-step, wave-uniform.
+    // Otherwise the same pair for this thread's own 16-byte chunk.
+    uint32_t tap = 0, kh = 0, kw = 0, ciOff = UNI ? 0 : chunk * 16;
+    auto normalise = [&] {
+      while (ciOff >= ciBytes) {
+        ciOff -= ciBytes;
+        ++tap;
+        if (++kw == d.kW) {
+          kw = 0;
+          ++kh;
+        }
+      }
+    };
+    normalise();
+
+    uint32_t bOff[BROWS];
 #pragma unroll
-  for (int j = 0; j != TN; ++j) {
-    const uint32_t n = nTile * BN + wn * (BN / 2) + j * 32 + col;
-    if (n >= d.outChansPerGroup)
-      continue;
-    const uint32_t c = g * d.outChansPerGroup + n;
-    const float bv = bias ? Load<OutT>::at(bias, c, 0) : 0.0f;
+    for (int r = 0; r != BROWS; ++r)
+      bOff[r] = ((g * a.coPadded + nTile * BN + (r * 4 + pw) * 8 + rowInBlock) *
+                     a.kPadded) *
+                    EB +
+                chunk * 16;
+    uint32_t kByte = 0; // byte offset of the next k-step along a B row
+
+    // Issues the loads of the next k-step into LDS stage `stage` and moves on
+    // along K.  Beyond the last k-step every offset is out of range: the
+    // stage is filled with zeros that are never multiplied.
+    auto loadStage = [&](uint32_t stage) {
+      char *base = lds + stage * kTileBytes + pw * kLoadBytes;
+      const uint32_t tapOff = (kh * d.dilH * d.inW + kw * d.dilW) * pixelBytes;
+      const uint32_t tapBit = tap < taps ? (1u << tap) : 0u;
+#pragma unroll
+      for (int r = 0; r != AROWS; ++r) {
+        const bool ok = (tapMask[r] & tapBit) != 0;
+        LdsPtr dst = (LdsPtr)(base + r * 4 * kLoadBytes);
+        if constexpr (UNI)
+          loadToLds(inBuf, dst, ok ? rowOff[r] : kOutOfRange, tapOff + ciOff);
+        else
+          loadToLds(inBuf, dst,
+                    ok ? rowOff[r] - chunk * 16 + tapOff + ciOff : kOutOfRange,
+                    0);
+      }
+      const uint32_t kOff = kByte < a.kPadded * EB ? kByte : kOutOfRange;
+#pragma unroll
+      for (int r = 0; r != BROWS; ++r)
+        loadToLds(wBuf,
+                  (LdsPtr)(base + kBlockM * kRowBytes + r * 4 * kLoadBytes),
+                  bOff[r] + kOff, 0);
+      ciOff += kRowBytes;
+      normalise();
+      kByte += kRowBytes;
+    };
+
+    // NS - 1 k-steps in flight; wait for the oldest before each barrier.
+#pragma unroll
+    for (int s = 0; s != NS - 1; ++s)
+      loadStage(s);
+    MXK_WAIT_VMCNT((NS - 2) * kLoads);
+    stepBarrier(); // barrier 0: step 0 is in LDS stage 0
+    for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
+      // Stage (kt - 1) % NS was multiplied before the last barrier: refill it
+      // with step kt + NS - 1, then make sure step kt + 1 has landed.
+      loadStage((kt + NS - 1) % NS);
+      MXK_WAIT_VMCNT((NS - 2) * kLoads);
+      stepBarrier(); // barrier kt + 1
+    }
+    MXK_WAIT_VMCNT(0); // the trailing zero loads, before LDS is reused
+  } else {
 #pragma unroll
     for (int i = 0; i != 2; ++i)
 #pragma unroll
-      for (int v = 0; v != 16; ++v) {
-        const uint32_t m = mTile * kBlockM + wm * 64 + i * 32 + 8 * (v / 4) +
-                           rowOff + (v % 4);
-        if (m < a.M)
-          storeOut(out, size_t(m) * outChans + c, acc[i][j][v] * scale + bv);
-      }
+      for (int j = 0; j != TN; ++j)
+#pragma unroll
+        for (int v = 0; v != 16; ++v)
+          acc[i][j][v] = 0.0f;
+    stepBarrier(); // barrier 0
+    for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
+      const char *stage = lds + (kt % NS) * kTileBytes;
+      const char *ldsA = stage + wm * 64 * kRowBytes;
+      const char *ldsB = stage + (kBlockM + wn * (BN / 2)) * kRowBytes;
+      Mma<EB>::template step<TN, FA, FB>(ldsA, ldsB, lane, acc);
+      // The stage may be overwritten after the barrier: its reads must have
+      // returned.
+      MXK_WAIT_LGKMCNT0();
+      stepBarrier(); // barrier kt + 1: step kt + 1 has landed
+    }
+  }
+  // One more meeting point: the producers' trailing loads have landed, so
+  // LDS can be reused for the output tile.
+  __syncthreads();
+
+  // Epilogue.  All k-steps are consumed and every wave is past the last
+  // barrier, so LDS is free: the consumers lay the finished tile out as
+  // [128 rows][BN outputs] (+ 16 bytes of padding per row), then everybody
+  // copies it out.  Lane l of a 32x32 accumulator holds column l % 32 and
+  // rows 8 * (v / 4) + 4 * (l / 32) + v % 4 for v = 0..15.
+  constexpr int kOutRow = BN * int(sizeof(OutT)) + 16;
+  static_assert(kBlockM * kOutRow <= NS * kTileBytes, "epilogue tile fits LDS");
+  if (!producer) {
+    const uint32_t col = lane & 31, rowOff4 = (lane >> 5) * 4;
+#pragma unroll
+    for (int j = 0; j != TN; ++j) {
+      const uint32_t nLocal = wn * (BN / 2) + j * 32 + col;
+      const uint32_t n = nTile * BN + nLocal;
+      const float bv = (bias && n < d.outChansPerGroup)
+                           ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
+                           : 0.0f;
+#pragma unroll
+      for (int i = 0; i != 2; ++i)
+#pragma unroll
+        for (int v = 0; v != 16; ++v) {
+          const uint32_t mLocal =
+              wm * 64 + i * 32 + 8 * (v / 4) + rowOff4 + (v % 4);
+          storeOut(reinterpret_cast<OutT *>(lds + mLocal * kOutRow), nLocal,
+                   acc[i][j][v] * scale + bv);
+        }
+    }
+  }
+  __syncthreads();
+  constexpr int kVecElems = 16 / int(sizeof(OutT));
+  constexpr int kVecsPerRow = BN / kVecElems;
+  // 16-byte stores need the channel count (hence every row start) to be a
+  // multiple of the vector; otherwise fall back to single elements.
+  const bool vectorOk = outChans % kVecElems == 0 &&
+                        d.outChansPerGroup % kVecElems == 0;
+  for (int idx = t; idx < kBlockM * kVecsPerRow; idx += kThreads) {
+    const uint32_t mLocal = idx / kVecsPerRow, vec = idx % kVecsPerRow;
+    const uint32_t m = mTile * kBlockM + mLocal;
+    const uint32_t n = nTile * BN + vec * kVecElems;
+    if (m >= a.M || n >= d.outChansPerGroup)
+      continue;
+    const char *src = lds + mLocal * kOutRow + vec * 16;
+    OutT *dst = out + size_t(m) * outChans + g * d.outChansPerGroup + n;
+    if (vectorOk) {
+      *reinterpret_cast<uintx4 *>(dst) = *reinterpret_cast<const uintx4 *>(src);
+    } else {
+      const OutT *e = reinterpret_cast<const OutT *>(src);
+      for (int k = 0; k != kVecElems && n + k < d.outChansPerGroup; ++k)
+        dst[k] = e[k];
+    }
   }
 }
 
-template <int BN, int EB, int FA, int FB, class OutT>
+template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
 hipError_t run(const IgemmArgs &a, const void *in, const void *w,
                const void *bias, void *out, float scale, hipStream_t stream) {
   const uint64_t blocks = uint64_t(a.mTiles) * a.nTiles * a.d.groups;
@@ -272,9 +451,17 @@ hipError_t run(const IgemmArgs &a, const void *in, const void *w,
     return hipSuccess;
   if (blocks > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((igemmKernel<BN, EB, FA, FB, OutT>), dim3(uint32_t(blocks)),
-                     dim3(kThreads), 0, stream, a,
-                     static_cast<const char *>(in), static_cast<const char *>(w),
+  constexpr int ldsBytes = NS * (kBlockM + BN) * kRowBytes;
+  // More than the 64 KB a kernel gets by default: raise the limit once.
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void *>(&igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+  if (attr != hipSuccess)
+    return attr;
+  hipLaunchKernelGGL((igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>),
+                     dim3(uint32_t(blocks)), dim3(kThreads), ldsBytes, stream,
+                     a, static_cast<const char *>(in),
+                     static_cast<const char *>(w),
                      static_cast<const OutT *>(bias), static_cast<OutT *>(out),
                      scale);
   return hipGetLastError();
@@ -284,10 +471,20 @@ template <int BN, int EB, int FA, int FB>
 hipError_t runOut(const IgemmArgs &a, int outType, const void *in,
                   const void *w, const void *bias, void *out, float scale,
                   hipStream_t stream) {
+  const bool uni = (a.d.inChansPerGroup * EB) % kRowBytes == 0;
+  // Stages of LDS: 4 x 32 KB for the 128-wide tile (one workgroup per CU);
+  // 3 x 24 KB for the 64-wide one, so that two workgroups share a CU.
+  constexpr int NS = BN == 128 ? 4 : 3;
   if (outType == kHalf)
-    return run<BN, EB, FA, FB, __half>(a, in, w, bias, out, scale, stream);
+    return uni ? run<BN, NS, EB, FA, FB, true, __half>(a, in, w, bias, out, scale,
+                                                   stream)
+               : run<BN, NS, EB, FA, FB, false, __half>(a, in, w, bias, out, scale,
+                                                    stream);
   if (outType == kFloat)
-    return run<BN, EB, FA, FB, float>(a, in, w, bias, out, scale, stream);
+    return uni ? run<BN, NS, EB, FA, FB, true, float>(a, in, w, bias, out, scale,
+                                                  stream)
+               : run<BN, NS, EB, FA, FB, false, float>(a, in, w, bias, out, scale,
+                                                   stream);
   return hipErrorInvalidValue;
 }
 
@@ -322,7 +519,7 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
   // The shapes the kernel is compiled for; the planner only produces these.
   if (d.blockM != kBlockM || (d.blockN != 64 && d.blockN != 128) ||
       d.blockK != bke || d.inChansPerGroup % (16 / eb) != 0 ||
-      (inType != kHalf && inType != kQuarter))
+      (inType != kHalf && inType != kQuarter) || d.kH * d.kW > 32)
     return hipErrorInvalidValue;
   IgemmArgs a;
   a.d = d;
@@ -336,6 +533,17 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
   const uint32_t k = d.kH * d.kW * d.inChansPerGroup;
   a.kPadded = (k + bke - 1) / bke * bke;
   a.kSteps = a.kPadded / bke;
+  // Buffer addressing is 32-bit; the planner keeps larger tensors away.
+  const uint64_t inBytes =
+      uint64_t(d.batch) * d.inH * d.inW * d.groups * d.inChansPerGroup * eb;
+  const uint64_t wBytes = uint64_t(d.groups) * a.coPadded * a.kPadded * eb;
+  const uint64_t shift = (uint64_t(d.padH > 0 ? d.padH : 0) * d.inW +
+                          uint64_t(d.padW > 0 ? d.padW : 0)) *
+                         d.groups * d.inChansPerGroup * eb;
+  if (inBytes + shift >= kOutOfRange || wBytes >= kOutOfRange)
+    return hipErrorInvalidConfiguration;
+  a.inBytes = uint32_t(inBytes);
+  a.wBytes = uint32_t(wBytes);
   if (d.blockN == 128)
     return runType<128>(a, inType, outType, in, weightsPacked, bias, out, q,
                         stream);

@@ -169,6 +169,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     else if (ci % (halfIn ? 8 : 16) != 0)
       igemmWhyNot = "input channels per group not a multiple of a 16-byte "
                     "vector";
+    else if (std::size_t(s.kH) * s.kW > 32)
+      igemmWhyNot = "more than 32 kernel taps";
+    else if (plan.inputElems * params.inputType.size() >= (1ull << 30) ||
+             plan.weightElems * params.inputType.size() >= (1ull << 30))
+      igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     if (!halfIn)
       dwWhyNot = "depthwise kernel takes half inputs";
     else if (ci != 1 || co != 1)
@@ -240,12 +245,12 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     // channels, when a narrower tile avoids computing padding.
     g.blockM = pc.blockM ? pc.blockM : 128;
     g.blockN = pc.blockN ? pc.blockN : (co <= 64 ? 64 : 128);
-    g.blockK = pc.blockK ? pc.blockK : (halfIn ? 32 : 64);
+    g.blockK = pc.blockK ? pc.blockK : (halfIn ? 64 : 128);
     if (g.blockM != 128 || (g.blockN != 64 && g.blockN != 128) ||
-        g.blockK != (halfIn ? 32u : 64u))
+        g.blockK != (halfIn ? 64u : 128u))
       throw poplar::invalid_option(
           "planConstraints gfx950 tile not available: blockM must be 128, "
-          "blockN 64 or 128, blockK 32 (half) or 64 (quarter)");
+          "blockN 64 or 128, blockK 64 (half) or 128 (quarter)");
     const std::size_t k = std::size_t(s.kH) * s.kW * ci;
     plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
     plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;

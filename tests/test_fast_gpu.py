@@ -50,7 +50,7 @@ IGEMM_CASES = [
     dict(batch=2, field=(28, 28), kernel=(3, 3), ci=128, co=128, pad=1),
     # BASELINE config 3 shape (1x1, 256->64, 56x56), reduced batch
     dict(batch=1, field=(56, 56), kernel=(1, 1), ci=256, co=64),
-    # M, N, K all ragged against the 128 x {64,128} x 32 tile
+    # M, N, K all ragged against the 128 x {64,128} x 64 tile
     dict(batch=3, field=(9, 7), kernel=(3, 3), ci=8, co=40, pad=1),
     dict(batch=1, field=(5, 5), kernel=(2, 3), ci=24, co=130,
          padLower=(1, 0), padUpper=(0, 2)),
