@@ -1,0 +1,128 @@
+"""The single_conv_layer harness: option handling without a GPU, and on the
+GPU the cases the reference drives through its own tool
+(tests/poplin/CMakeLists.txt:991-3500), each compared with the host model by
+the tool itself (exit code 0 = match)."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOOL = os.path.join(ROOT, "tests", "tools", "single_conv_layer")
+
+
+def run(*args, timeout=120):
+    if not os.path.exists(TOOL):
+        subprocess.check_call(["make", "-C", os.path.dirname(TOOL)],
+                              stdout=subprocess.DEVNULL)
+    return subprocess.run([TOOL, *args], capture_output=True, text=True,
+                          timeout=timeout)
+
+
+def test_plan_only_reports_flops_and_plan():
+    r = run("--input-channels", "128", "--output-channels", "128", "--field",
+            "{28,28}", "--kernel-size", "3", "--padding", "1", "--batch-size",
+            "32", "--data-type", "half", "--plan-only")
+    assert r.returncode == 0, r.stderr
+    assert "Forward FLOPs: 7050625024" in r.stdout
+    assert "implicit GEMM" in r.stdout
+    assert "inputPaddingLower          {1,1}" in r.stdout
+
+
+def test_plan_constraints_and_options_are_validated():
+    base = ["--input-channels", "16", "--output-channels", "16", "--field",
+            "{8,8}", "--kernel-size", "3", "--plan-only"]
+    r = run(*base, "--fwd-plan-constraints", '{"method": {"type": "HMAC"}}')
+    assert r.returncode == 0 and "generic direct" in r.stdout
+    r = run(*base, "--fwd-plan-constraints", '{"method": {"type": "NOPE"}}')
+    assert r.returncode == 1 and "Not a valid method type" in r.stderr
+    r = run(*base, "--convolution-options", '{"partialsType": "half"}')
+    assert r.returncode == 0
+    r = run(*base, "--convolution-options", '{"partialsType": "double"}')
+    assert r.returncode == 1
+
+
+def test_usage_errors_exit_1():
+    assert run("--input-channels", "1").returncode == 1
+    assert run("--input-channels", "1", "--output-channels", "1", "--field",
+               "{4}", "--kernel-size", "9", "--plan-only").returncode == 1
+    assert run("--bogus").returncode == 1
+    assert run("--input-channels", "1", "--output-channels", "1", "--field",
+               "{4}", "--kernel-size", "1", "--single-phase",
+               "bwd").returncode == 1
+
+
+# name, arguments: modelled on the reference's ctest entries
+GPU_CASES = [
+    ("conv3x3_stride_1_padding_1",
+     "--input-channels 16 --output-channels 16 --field {14,14} "
+     "--kernel-size 3 --padding 1 --data-type half"),
+    ("conv1x1_stride_1",
+     "--input-channels 32 --output-channels 16 --field {14,14} "
+     "--kernel-size 1 --data-type half --batch-size 2"),
+    ("conv_fp32_baseline_config1",
+     "--input-channels 16 --output-channels 16 --field {32,32} "
+     "--kernel-size 3 --padding 1 --data-type float --bias 0"),
+    ("conv3x3_stride_2_float",
+     "--input-channels 3 --output-channels 5 --field {9,11} --kernel-size 3 "
+     "--stride 2 --padding-lower 1 --padding-upper 0 --data-type float"),
+    ("depthwise_5x5",
+     "--input-channels 1 --output-channels 1 --conv-groups 24 "
+     "--field {28,28} --kernel-size 5 --data-type half"),
+    ("conv_zero_batch",
+     "--input-channels 4 --output-channels 4 --field {4,4} --kernel-size 3 "
+     "--batch-size 0 --data-type half"),
+    ("conv_zero_in_chans",
+     "--input-channels 0 --output-channels 4 --field {4,4} --kernel-size 3 "
+     "--data-type half"),
+    ("conv_zero_out_chans",
+     "--input-channels 4 --output-channels 0 --field {4,4} --kernel-size 3 "
+     "--data-type half"),
+    ("conv_negative_padding_via_truncation",
+     "--input-channels 8 --output-channels 8 --field {12,12} --kernel-size 3 "
+     "--truncation-lower {1,0} --truncation-upper {0,2} --data-type half"),
+    ("conv_flips_and_dilation",
+     "--input-channels 2 --output-channels 3 --field {7,6} --kernel-size {3,2} "
+     "--flip-input {1,0} --flip-kernel {0,1} --in-dilation {2,1} "
+     "--kernel-dilation {1,2} --stride {2,2} --data-type float"),
+    ("conv_output_padding",
+     "--input-channels 2 --output-channels 2 --field {5,5} --kernel-size 2 "
+     "--output-padding-lower {1,0} --output-padding-upper {0,2} "
+     "--output-truncation-lower {1,1} --data-type float"),
+    ("conv_1d_and_3d",
+     "--input-channels 8 --output-channels 8 --field {5,6,7} "
+     "--kernel-size {2,3,2} --padding {1,0,1} --data-type half"),
+    ("conv_quarter_arch_2_AMP",
+     "--input-channels 32 --output-channels 16 --field {8,8} --kernel-size 3 "
+     "--padding 1 --input-type quarter --output-type half"),
+    ("conv_quarter_formats",
+     "--input-channels 16 --output-channels 16 --field {6,6} --kernel-size 1 "
+     "--input-type quarter --output-type half --fp8-format-fwd quart152 "
+     "--fp8-scale-fwd -1 --fp8-scale-weights 3"),
+    ("conv_uniform_data_large_accumulation",
+     "--input-channels 1024 --output-channels 16 --field {6,6} "
+     "--kernel-size 5 --padding 2 --data-type half"),
+    ("conv_determinism",
+     "--input-channels 16 --output-channels 16 --field {14,14} "
+     "--kernel-size 3 --padding 1 --data-type half "
+     "--num-determinism-checks 3"),
+    ("conv_forced_generic",
+     "--input-channels 16 --output-channels 16 --field {14,14} "
+     "--kernel-size 3 --padding 1 --data-type half "
+     "--fwd-plan-constraints {\"gfx950\":{\"kernel\":\"generic\"}}"),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,args", GPU_CASES, ids=[c[0] for c in GPU_CASES])
+def test_reference_style_cases(name, args):
+    print("case", name, flush=True)
+    r = run(*args.split())
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-2000:])
+    assert "Validation passed" in r.stdout
+    if "large_accumulation" in name:
+        assert "Using uniform random data" in r.stdout
+    elif "determinism" not in name and "quarter" not in name:
+        # (quarter: only 16 contiguous integers, so the reference's rule picks
+        # the integer-valued "uniform" mode even for small convolutions)
+        assert "no error tolerance" in r.stdout
