@@ -100,7 +100,7 @@ GPU_CASES = [
      "--input-type quarter --output-type half --fp8-format-fwd quart152 "
      "--fp8-scale-fwd -1 --fp8-scale-weights 3"),
     ("conv_uniform_data_large_accumulation",
-     "--input-channels 1024 --output-channels 16 --field {6,6} "
+     "--input-channels 2048 --output-channels 16 --field {6,6} "
      "--kernel-size 5 --padding 2 --data-type half"),
     ("conv_determinism",
      "--input-channels 16 --output-channels 16 --field {14,14} "
