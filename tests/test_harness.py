@@ -126,3 +126,43 @@ def test_reference_style_cases(name, args):
         # (quarter: only 16 contiguous integers, so the reference's rule picks
         # the integer-valued "uniform" mode even for small convolutions)
         assert "no error tolerance" in r.stdout
+
+
+RANDOM = os.path.join(ROOT, "tests", "tools", "single_conv_layer_random.py")
+
+
+def test_random_driver_is_reproducible_and_valid():
+    """Every emitted parameter set passes ConvParams::validate (via
+    --plan-only) and the same seed gives the same command."""
+    import sys
+    for seed in range(1, 9):
+        a = subprocess.run([sys.executable, RANDOM, "--seed", str(seed),
+                            "--dry-run"], capture_output=True, text=True)
+        b = subprocess.run([sys.executable, RANDOM, "--seed", str(seed),
+                            "--dry-run"], capture_output=True, text=True)
+        assert a.returncode == 0 and a.stdout == b.stdout
+        args = a.stdout.split()[1:]
+        r = run(*args, "--plan-only")
+        assert r.returncode == 0, (a.stdout, r.stderr)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(1, 31))
+def test_conv_random(seed):
+    """conv_random_N of tests/poplin/CMakeLists.txt:1040-1065."""
+    import sys
+    print("conv_random seed", seed, flush=True)
+    r = subprocess.run([sys.executable, RANDOM, "--seed", str(seed)],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-3000:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(1, 16))
+def test_conv_random_quarter(seed):
+    import sys
+    print("conv_random_quarter seed", seed, flush=True)
+    r = subprocess.run([sys.executable, RANDOM, "--seed", str(seed),
+                        "--input-type", "quarter"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-3000:])
