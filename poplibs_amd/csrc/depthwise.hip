@@ -1,23 +1,54 @@
 // Depthwise forward convolution (one input and one output channel per group):
 // the memory-bound case PopLibs serves with its HorizontalMac vertices
 // (lib/poplin/codelets/ConvPartialHorizontalMac.cpp:34-133).  No matrix cores:
-// 1.8 flop per byte, so the only thing that matters is moving each input
-// element from HBM once and writing each output once.
+// at 1.8 flop per byte the only thing that matters is to move every input
+// element from HBM once, write every output once, and keep enough bytes in
+// flight to cover HBM latency.
 //
-// Channels-last layout: a thread owns 8 consecutive channels (one 16-byte
-// vector) of one output pixel, so a wavefront's loads and stores are runs of
-// whole 16-byte vectors along the channel axis.  Products are formed and
-// accumulated in fp32.
+// Channels-last layout; the unit of work is a 16-byte vector of 8 consecutive
+// fp16 channels.  A workgroup produces a tile of tileH x tileW output pixels
+// for a block of up to 16 channel vectors:
+//   1. all of the input patch the tile needs ((tileH-1)*strideH +
+//      (kH-1)*dilH + 1 rows, likewise columns) is requested at once with
+//      16-byte buffer loads that write straight into LDS - one burst per
+//      workgroup, the deepest memory-level parallelism the hardware offers,
+//      no staging registers.  Patch elements that fall on padding get an
+//      out-of-range offset, for which the buffer unit delivers zeros, so the
+//      compute loop has no bounds checks;
+//   2. after one barrier each thread forms its outputs from LDS:
+//      products and sums in fp32 (v_fma_mix_f32 on the packed halves);
+//   3. 16-byte (fp16 output) or 2 x 16-byte (fp32 output) coalesced stores.
+// Several workgroups share a CU (the patch is kept under 52 KB of the 160 KB
+// LDS), so one workgroup's loads overlap another's arithmetic and stores.
+// Neighbouring tiles overlap by the kernel halo; workgroups are numbered so
+// that each XCD walks a contiguous run of tiles and the halo re-reads hit its
+// own L2 instead of HBM.
 #include "device_types.hpp"
 #include "kernels.hpp"
 
 namespace mxk {
 namespace {
 
+constexpr int kThreads = 256;
+constexpr uint32_t kOutOfRange = 0x80000000u;
+
+using LdsPtr = __attribute__((address_space(3))) void *;
+
 __device__ __forceinline__ uint32_t xcdSwizzle(uint32_t bid, uint32_t total) {
   const uint32_t xcd = bid & 7u, idx = bid >> 3;
   const uint32_t q = total >> 3, rem = total & 7u;
   return xcd * q + (xcd < rem ? xcd : rem) + idx;
+}
+
+/// 16 bytes per lane from a buffer straight into LDS: lane l's data lands at
+/// dst + 16 l (dst is wave-uniform); out-of-range offsets deliver zeros.  The
+/// builtin exists for the GPU target only; the host pass sees an empty body.
+__device__ __forceinline__ void loadToLds(__amdgpu_buffer_rsrc_t buffer,
+                                          LdsPtr dst, uint32_t vectorOffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, dst, 16, vectorOffset, 0, 0,
+                                           0);
+#endif
 }
 
 union Vec8 {
@@ -42,60 +73,200 @@ template <> struct StoreVec<float> {
   }
 };
 
-template <class OutT>
-__global__ __launch_bounds__(256) void depthwiseKernel(
-    DepthwiseDesc d, uint64_t total, const __half *__restrict__ in,
-    const __half *__restrict__ w, const OutT *__restrict__ bias,
-    OutT *__restrict__ out) {
-  // Each XCD walks one contiguous range of output pixels (whole images when
-  // the batch divides by 8), so halo rows shared by neighbouring output rows
-  // are re-read from that XCD's L2 rather than from HBM.
-  const uint64_t tid =
-      uint64_t(xcdSwizzle(blockIdx.x, gridDim.x)) * blockDim.x + threadIdx.x;
-  if (tid >= total)
-    return;
-  const uint32_t vecs = d.channels / 8;
-  const uint32_t cv = uint32_t(tid % vecs);
-  uint64_t pix = tid / vecs;
-  const uint32_t ow = uint32_t(pix % d.outW);
-  pix /= d.outW;
-  const uint32_t oh = uint32_t(pix % d.outH);
-  const uint32_t b = uint32_t(pix / d.outH);
+struct DwArgs {
+  DepthwiseDesc d;
+  uint32_t vecs;      // channels / 8
+  uint32_t vecBlock;  // channel vectors per workgroup: vecs if <= 16, else 16
+  uint32_t vecShift;  // log2(vecBlock) when the channels are split in blocks
+  uint32_t vecBlocks; // ceil(vecs / vecBlock)
+  uint32_t tilesH, tilesW;
+  uint32_t patchH, patchW;
+  uint32_t rowElems;  // patchW * vecBlock: 16-byte elements per patch row
+  uint32_t rowPitch;  // rowElems rounded up to a multiple of 64
+  // Compute phase: pixelsPerRound * vecBlock threads are active; a thread
+  // keeps its channel vector and steps pixelsPerRound pixels per round.
+  uint32_t pixelsPerRound, stepY, stepX; // pixelsPerRound = stepY*tileW+stepX
+  uint32_t inBytes;
+};
 
-  float acc[8];
-#pragma unroll
-  for (int i = 0; i != 8; ++i)
-    acc[i] = 0.0f;
-  const __half *inB = in + size_t(b) * d.inH * d.inW * d.channels + cv * 8;
-  const __half *wC = w + cv * 8;
-  for (uint32_t kh = 0; kh != d.kH; ++kh) {
-    const int ih = int(oh * d.strideH + kh * d.dilH) - d.padH;
-    if (ih < int(d.loH) || ih >= int(d.hiH))
-      continue;
-    for (uint32_t kw = 0; kw != d.kW; ++kw) {
-      const int iw = int(ow * d.strideW + kw * d.dilW) - d.padW;
-      if (iw < int(d.loW) || iw >= int(d.hiW))
-        continue;
-      Vec8 x, k;
-      x.raw = *reinterpret_cast<const uint4 *>(
-          inB + (size_t(ih) * d.inW + iw) * d.channels);
-      k.raw = *reinterpret_cast<const uint4 *>(
-          wC + size_t(kh * d.kW + kw) * d.channels);
-#pragma unroll
-      for (int i = 0; i != 4; ++i) {
-        const float2 xf = __half22float2(x.h2[i]);
-        const float2 kf = __half22float2(k.h2[i]);
-        acc[2 * i] = fmaf(xf.x, kf.x, acc[2 * i]);
-        acc[2 * i + 1] = fmaf(xf.y, kf.y, acc[2 * i + 1]);
-      }
+/// KH, KW > 0: kernel extents known at compile time (taps fully unrolled);
+/// 0: taken from the descriptor.
+template <int KH, int KW, class OutT>
+__global__ __launch_bounds__(kThreads) void depthwiseKernel(
+    DwArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
+    const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  extern __shared__ __align__(16) char lds[]; // patchH * rowPitch * 16 bytes
+  const DepthwiseDesc &d = a.d;
+  const uint32_t kH = KH ? KH : d.kH, kW = KW ? KW : d.kW;
+
+  uint32_t tile = xcdSwizzle(blockIdx.x, gridDim.x);
+  const uint32_t cb = tile % a.vecBlocks;
+  tile /= a.vecBlocks;
+  const uint32_t tw = tile % a.tilesW;
+  tile /= a.tilesW;
+  const uint32_t th = tile % a.tilesH;
+  const uint32_t b = tile / a.tilesH;
+
+  const uint32_t oh0 = th * d.tileH, ow0 = tw * d.tileW;
+  const uint32_t cv0 = cb * a.vecBlock;
+  const uint32_t nvec = min(a.vecBlock, a.vecs - cv0); // vectors in this block
+  const int ih0 = int(oh0 * d.strideH) - d.padH; // patch origin in the input
+  const int iw0 = int(ow0 * d.strideW) - d.padW;
+
+  // 1. the whole patch, one burst.  LDS holds patch row ph at byte
+  // 16 * ph * rowPitch, element j = pw * vecBlock + v of the row at + 16 j; a
+  // wave-wide load covers 64 consecutive j of one row.  No division: with all
+  // channels in one block the row is contiguous in memory as well, otherwise
+  // vecBlock is 16 and (pw, v) are a shift and a mask of j.
+  const __amdgpu_buffer_rsrc_t inBuf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<__half *>(in), short(0), int(a.inBytes), 0x00020000);
+  const uint32_t pixelBytes = d.channels * 2;
+  const uint32_t imageOff = b * d.inH * d.inW * pixelBytes;
+  const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint32_t chunksPerRow = a.rowPitch >> 6;
+  const uint32_t chunks = a.patchH * chunksPerRow;
+  // Wave w takes 64-element chunks w, w + 4, ...; (ph, chunk in row) advance
+  // without dividing.
+  uint32_t ph = 0, cr = wave;
+  while (cr >= chunksPerRow) {
+    cr -= chunksPerRow;
+    ++ph;
+  }
+  for (uint32_t chunk = wave; chunk < chunks; chunk += kThreads / 64) {
+    const uint32_t j = cr * 64 + lane;
+    uint32_t pw, v;
+    if (a.vecBlocks == 1) {
+      pw = 0; // row-contiguous: the offset below uses j directly
+      v = j;
+    } else {
+      pw = j >> a.vecShift;
+      v = j & (a.vecBlock - 1);
+    }
+    const int ih = ih0 + int(ph);
+    bool ok = j < a.rowElems && ih >= int(d.loH) && ih < int(d.hiH);
+    uint32_t off = imageOff + uint32_t(ih) * d.inW * pixelBytes;
+    if (a.vecBlocks == 1) {
+      // valid columns [loW, hiW) as a range of j
+      const int jLo = (int(d.loW) - iw0) * int(a.vecBlock);
+      const int jHi = (int(d.hiW) - iw0) * int(a.vecBlock);
+      ok = ok && int(j) >= jLo && int(j) < jHi;
+      off += uint32_t(iw0) * pixelBytes + j * 16;
+    } else {
+      const int iw = iw0 + int(pw);
+      ok = ok && iw >= int(d.loW) && iw < int(d.hiW) && v < nvec;
+      off += uint32_t(iw) * pixelBytes + (cv0 + v) * 16;
+    }
+    loadToLds(inBuf, (LdsPtr)(lds + (ph * a.rowPitch + cr * 64) * 16),
+              ok ? off : kOutOfRange);
+    cr += kThreads / 64;
+    while (cr >= chunksPerRow) {
+      cr -= chunksPerRow;
+      ++ph;
     }
   }
-  if (bias) {
+
+  // This thread's channel vector and first pixel; its kernel taps (3x3:
+  // kept in registers for all its pixels).
+  const uint32_t v = threadIdx.x % a.vecBlock;
+  uint32_t p = threadIdx.x / a.vecBlock;
+  const bool active = p < a.pixelsPerRound && v < nvec;
+  const uint32_t c = (cv0 + (v < nvec ? v : 0)) * 8;
+  const __half *wC = w + c;
+  constexpr bool kTapsInRegs = KH * KW != 0 && KH * KW <= 9;
+  Vec8 taps[kTapsInRegs ? KH * KW : 1];
+  if constexpr (kTapsInRegs) {
 #pragma unroll
-    for (int i = 0; i != 8; ++i)
-      acc[i] += Load<OutT>::at(bias, cv * 8 + i, 0);
+    for (int tap = 0; tap != KH * KW; ++tap)
+      taps[tap].raw =
+          *reinterpret_cast<const uint4 *>(wC + tap * d.channels);
   }
-  StoreVec<OutT>::put(out + tid * 8, acc);
+  float biasV[8];
+#pragma unroll
+  for (int i = 0; i != 8; ++i)
+    biasV[i] = bias ? Load<OutT>::at(bias, c + i, 0) : 0.0f;
+
+  __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's loads landed
+  __syncthreads();
+
+  // 2. + 3.  One item = one output pixel x one channel vector.
+  uint32_t ty = 0, tx = p;
+  while (tx >= d.tileW) {
+    tx -= d.tileW;
+    ++ty;
+  }
+  const uint32_t pixels = d.tileH * d.tileW;
+  if (active)
+    for (; p < pixels; p += a.pixelsPerRound) {
+      const uint32_t oh = oh0 + ty, ow = ow0 + tx;
+      if (oh < d.outH && ow < d.outW) {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i != 8; ++i)
+          acc[i] = biasV[i];
+        const char *patch =
+            lds + (ty * d.strideH * a.rowPitch +
+                   tx * d.strideW * a.vecBlock + v) *
+                      16;
+#pragma unroll
+        for (uint32_t kh = 0; kh < kH; ++kh)
+#pragma unroll
+          for (uint32_t kw = 0; kw < kW; ++kw) {
+            Vec8 x, k;
+            x.raw = *reinterpret_cast<const uint4 *>(
+                patch +
+                (kh * d.dilH * a.rowPitch + kw * d.dilW * a.vecBlock) * 16);
+            if constexpr (kTapsInRegs)
+              k = taps[kh * KW + kw];
+            else
+              k.raw = *reinterpret_cast<const uint4 *>(
+                  wC + (kh * kW + kw) * d.channels);
+#pragma unroll
+            for (int i = 0; i != 4; ++i) {
+              const float2 xf = __half22float2(x.h2[i]);
+              const float2 kf = __half22float2(k.h2[i]);
+              acc[2 * i] = fmaf(xf.x, kf.x, acc[2 * i]);
+              acc[2 * i + 1] = fmaf(xf.y, kf.y, acc[2 * i + 1]);
+            }
+          }
+        StoreVec<OutT>::put(
+            out + ((size_t(b) * d.outH + oh) * d.outW + ow) * d.channels + c,
+            acc);
+      }
+      ty += a.stepY;
+      tx += a.stepX;
+      if (tx >= d.tileW) {
+        tx -= d.tileW;
+        ++ty;
+      }
+    }
+}
+
+template <int KH, int KW, class OutT>
+hipError_t run(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
+               const void *in, const void *w, const void *bias, void *out,
+               hipStream_t stream) {
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void *>(&depthwiseKernel<KH, KW, OutT>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+  if (attr != hipSuccess)
+    return attr;
+  hipLaunchKernelGGL((depthwiseKernel<KH, KW, OutT>), dim3(blocks),
+                     dim3(kThreads), ldsBytes, stream, a,
+                     static_cast<const __half *>(in),
+                     static_cast<const __half *>(w),
+                     static_cast<const OutT *>(bias), static_cast<OutT *>(out));
+  return hipGetLastError();
+}
+
+template <class OutT>
+hipError_t runKernelShape(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
+                          const void *in, const void *w, const void *bias,
+                          void *out, hipStream_t stream) {
+  if (a.d.kH == 3 && a.d.kW == 3)
+    return run<3, 3, OutT>(a, blocks, ldsBytes, in, w, bias, out, stream);
+  if (a.d.kH == 5 && a.d.kW == 5)
+    return run<5, 5, OutT>(a, blocks, ldsBytes, in, w, bias, out, stream);
+  return run<0, 0, OutT>(a, blocks, ldsBytes, in, w, bias, out, stream);
 }
 
 } // namespace
@@ -103,31 +274,39 @@ __global__ __launch_bounds__(256) void depthwiseKernel(
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream) {
-  if (inType != kHalf || d.channels % 8 != 0)
+  if (inType != kHalf || d.channels % 8 != 0 || d.tileH == 0 || d.tileW == 0)
     return hipErrorInvalidValue;
-  const uint64_t total =
-      uint64_t(d.batch) * d.outH * d.outW * (d.channels / 8);
-  if (total == 0)
+  if (uint64_t(d.batch) * d.outH * d.outW * d.channels == 0)
     return hipSuccess;
-  const uint64_t blocks = (total + 255) / 256;
-  if (blocks > 0x7fffffffull)
+  DwArgs a;
+  a.d = d;
+  a.vecs = d.channels / 8;
+  a.vecBlock = a.vecs <= 16 ? a.vecs : 16;
+  a.vecShift = 4;
+  a.vecBlocks = (a.vecs + a.vecBlock - 1) / a.vecBlock;
+  a.tilesH = (d.outH + d.tileH - 1) / d.tileH;
+  a.tilesW = (d.outW + d.tileW - 1) / d.tileW;
+  a.patchH = (d.tileH - 1) * d.strideH + (d.kH - 1) * d.dilH + 1;
+  a.patchW = (d.tileW - 1) * d.strideW + (d.kW - 1) * d.dilW + 1;
+  a.rowElems = a.patchW * a.vecBlock;
+  a.rowPitch = (a.rowElems + 63) / 64 * 64;
+  a.pixelsPerRound = kThreads / a.vecBlock;
+  a.stepY = a.pixelsPerRound / d.tileW;
+  a.stepX = a.pixelsPerRound % d.tileW;
+  const uint64_t inBytes = uint64_t(d.batch) * d.inH * d.inW * d.channels * 2;
+  const uint64_t ldsBytes = uint64_t(a.patchH) * a.rowPitch * 16;
+  const uint64_t blocks =
+      uint64_t(d.batch) * a.tilesH * a.tilesW * a.vecBlocks;
+  if (inBytes >= kOutOfRange || ldsBytes > 64 * 1024 || blocks > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
-  const dim3 grid{uint32_t(blocks)}, block{256};
+  a.inBytes = uint32_t(inBytes);
   if (outType == kHalf)
-    hipLaunchKernelGGL(depthwiseKernel<__half>, grid, block, 0, stream, d,
-                       total, static_cast<const __half *>(in),
-                       static_cast<const __half *>(weightsPacked),
-                       static_cast<const __half *>(bias),
-                       static_cast<__half *>(out));
-  else if (outType == kFloat)
-    hipLaunchKernelGGL(depthwiseKernel<float>, grid, block, 0, stream, d, total,
-                       static_cast<const __half *>(in),
-                       static_cast<const __half *>(weightsPacked),
-                       static_cast<const float *>(bias),
-                       static_cast<float *>(out));
-  else
-    return hipErrorInvalidValue;
-  return hipGetLastError();
+    return runKernelShape<__half>(a, uint32_t(blocks), uint32_t(ldsBytes), in,
+                                  weightsPacked, bias, out, stream);
+  if (outType == kFloat)
+    return runKernelShape<float>(a, uint32_t(blocks), uint32_t(ldsBytes), in,
+                                 weightsPacked, bias, out, stream);
+  return hipErrorInvalidValue;
 }
 
 } // namespace mxk

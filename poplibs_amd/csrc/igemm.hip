@@ -151,66 +151,92 @@ template <int EB> struct Mma;
 /// c ^ (r & 7).  `row` = lane & 31 is the row inside a 32-row block (block
 /// bases are multiples of 8, so r & 7 == lane & 7).
 
-/// fp16: K=16 steps of 32 bytes (two chunks, one per half-wave) per row.
+/// The MFMA operands ("fragments") of one k-step for one consumer wave, and
+/// the two halves of a k-step's work: fetch every fragment from LDS, multiply
+/// sub-steps [S0, S1).  Keeping them apart lets the consumer loop start the
+/// next k-step's LDS reads before the current k-step's last MFMAs.
+
+/// fp16: 4 sub-steps of K=16, 32 bytes (two chunks, one per half-wave) each.
 template <> struct Mma<2> {
-  template <int TN, int FA, int FB>
+  static constexpr int kSubSteps = kRowBytes / 32;
+  template <int TN> struct Frags {
+    half8 a[kSubSteps][2], b[kSubSteps][TN];
+  };
+  template <int TN>
   static __device__ __forceinline__ void
-  step(const char *ldsA, const char *ldsB, int lane, floatx16 (&acc)[2][TN]) {
+  load(const char *ldsA, const char *ldsB, int lane, Frags<TN> &f) {
     const int row = lane & 31;
     const int swz = lane & 7, half = lane >> 5;
 #pragma unroll
-    for (int s = 0; s != kRowBytes / 32; ++s) {
+    for (int s = 0; s != kSubSteps; ++s) {
       const int off = row * kRowBytes + (((s * 2 + half) ^ swz) << 4);
-      half8 a[2], b[TN];
 #pragma unroll
       for (int i = 0; i != 2; ++i)
-        a[i] = *reinterpret_cast<const half8 *>(ldsA + i * 32 * kRowBytes + off);
+        f.a[s][i] =
+            *reinterpret_cast<const half8 *>(ldsA + i * 32 * kRowBytes + off);
 #pragma unroll
       for (int j = 0; j != TN; ++j)
-        b[j] = *reinterpret_cast<const half8 *>(ldsB + j * 32 * kRowBytes + off);
+        f.b[s][j] =
+            *reinterpret_cast<const half8 *>(ldsB + j * 32 * kRowBytes + off);
+    }
+  }
+  template <int S0, int S1, int TN, int FA, int FB>
+  static __device__ __forceinline__ void mul(const Frags<TN> &f,
+                                             floatx16 (&acc)[2][TN]) {
+#pragma unroll
+    for (int s = S0; s != S1; ++s)
 #pragma unroll
       for (int i = 0; i != 2; ++i)
 #pragma unroll
         for (int j = 0; j != TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j],
-                                                             acc[i][j], 0, 0, 0);
-    }
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+              f.a[s][i], f.b[s][j], acc[i][j], 0, 0, 0);
   }
 };
 
-/// fp8: K=64 steps of 64 bytes (four chunks, two per half-wave) per row.
+/// fp8: 2 sub-steps of K=64, 64 bytes (four chunks, two per half-wave) each.
 /// FA / FB: 0 = E4M3, 1 = E5M2 (the cbsz / blgp operand-format fields).
 template <> struct Mma<1> {
-  template <int TN, int FA, int FB>
+  static constexpr int kSubSteps = kRowBytes / 64;
+  template <int TN> struct Frags {
+    intx8 a[kSubSteps][2], b[kSubSteps][TN];
+  };
+  template <int TN>
   static __device__ __forceinline__ void
-  step(const char *ldsA, const char *ldsB, int lane, floatx16 (&acc)[2][TN]) {
+  load(const char *ldsA, const char *ldsB, int lane, Frags<TN> &f) {
     const int row = lane & 31;
     const int swz = lane & 7, half = lane >> 5;
 #pragma unroll
-    for (int s = 0; s != kRowBytes / 64; ++s) {
+    for (int s = 0; s != kSubSteps; ++s) {
       const int c0 = s * 4 + half * 2;
       const int off0 = row * kRowBytes + ((c0 ^ swz) << 4);
       const int off1 = row * kRowBytes + (((c0 + 1) ^ swz) << 4);
+      // 32 bytes per lane: two chunks that the swizzle may have separated.
       auto load32 = [&](const char *p) {
         const uintx4 lo = *reinterpret_cast<const uintx4 *>(p + off0);
         const uintx4 hi = *reinterpret_cast<const uintx4 *>(p + off1);
         return intx8{int(lo.x), int(lo.y), int(lo.z), int(lo.w),
                      int(hi.x), int(hi.y), int(hi.z), int(hi.w)};
       };
-      intx8 a[2], b[TN];
 #pragma unroll
       for (int i = 0; i != 2; ++i)
-        a[i] = load32(ldsA + i * 32 * kRowBytes);
+        f.a[s][i] = load32(ldsA + i * 32 * kRowBytes);
 #pragma unroll
       for (int j = 0; j != TN; ++j)
-        b[j] = load32(ldsB + j * 32 * kRowBytes);
+        f.b[s][j] = load32(ldsB + j * 32 * kRowBytes);
+    }
+  }
+  template <int S0, int S1, int TN, int FA, int FB>
+  static __device__ __forceinline__ void mul(const Frags<TN> &f,
+                                             floatx16 (&acc)[2][TN]) {
+#pragma unroll
+    for (int s = S0; s != S1; ++s)
 #pragma unroll
       for (int i = 0; i != 2; ++i)
 #pragma unroll
         for (int j = 0; j != TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-              a[i], b[j], acc[i][j], FA, FB, 0, 0, 0, 0);
-    }
+              f.a[s][i], f.b[s][j], acc[i][j], FA, FB, 0, 0, 0, 0);
   }
 };
 
@@ -375,17 +401,39 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
 #pragma unroll
         for (int v = 0; v != 16; ++v)
           acc[i][j][v] = 0.0f;
-    stepBarrier(); // barrier 0
-    for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
+    using M = Mma<EB>;
+    constexpr int kLast = M::kSubSteps - 1;
+    typename M::template Frags<TN> f0, f1;
+    auto fetch = [&](uint32_t kt, typename M::template Frags<TN> &f) {
       const char *stage = lds + (kt % NS) * kTileBytes;
-      const char *ldsA = stage + wm * 64 * kRowBytes;
-      const char *ldsB = stage + (kBlockM + wn * (BN / 2)) * kRowBytes;
-      Mma<EB>::template step<TN, FA, FB>(ldsA, ldsB, lane, acc);
-      // The stage may be overwritten after the barrier: its reads must have
-      // returned.
+      M::template load<TN>(stage + wm * 64 * kRowBytes,
+                           stage + (kBlockM + wn * (BN / 2)) * kRowBytes, lane,
+                           f);
+    };
+    // One k-step: multiply all sub-steps but the last, meet the producers
+    // (this stage's LDS reads have all returned by then: the stage may be
+    // refilled), start the next k-step's LDS reads, and only then issue the
+    // last sub-step's MFMAs - the LDS pipe, which is as busy as the matrix
+    // cores with this tile shape, never waits for them.
+    auto step = [&](uint32_t kt, typename M::template Frags<TN> &cur,
+                    typename M::template Frags<TN> &next) {
+      M::template mul<0, kLast, TN, FA, FB>(cur, acc);
       MXK_WAIT_LGKMCNT0();
       stepBarrier(); // barrier kt + 1: step kt + 1 has landed
+      if (kt + 1 != a.kSteps)
+        fetch(kt + 1, next);
+      M::template mul<kLast, kLast + 1, TN, FA, FB>(cur, acc);
+    };
+    stepBarrier(); // barrier 0
+    if (a.kSteps != 0)
+      fetch(0, f0);
+    uint32_t kt = 0;
+    for (; kt + 1 < a.kSteps; kt += 2) {
+      step(kt, f0, f1);
+      step(kt + 1, f1, f0);
     }
+    if (kt < a.kSteps)
+      step(kt, f0, f1);
   }
   // One more meeting point: the producers' trailing loads have landed, so
   // LDS can be reused for the output tile.

@@ -91,6 +91,9 @@ struct DepthwiseDesc {
   int32_t padH, padW; // as in IgemmDesc
   uint32_t strideH, strideW, dilH, dilW;
   uint32_t loH, hiH, loW, hiW;
+  // Output pixels per workgroup tile, chosen by the planner so that the
+  // input patch of a tile fits a third of a CU's LDS.
+  uint32_t tileH, tileW;
 };
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,

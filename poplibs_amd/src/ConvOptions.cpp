@@ -192,6 +192,10 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       pc.blockN = requireUnsigned(sub, m.second);
     } else if (m.first == "blockK") {
       pc.blockK = requireUnsigned(sub, m.second);
+    } else if (m.first == "tileH") {
+      pc.tileH = requireUnsigned(sub, m.second);
+    } else if (m.first == "tileW") {
+      pc.tileW = requireUnsigned(sub, m.second);
     } else {
       throw invalid_option("'" + sub + "': " + m.first +
                            " is not a gfx950 plan constraint");

@@ -107,6 +107,44 @@ Simple2D asSimple2D(const ConvParams &p) {
   return s;
 }
 
+/// Output tile (height, width) of the depthwise kernel: the input patch of a
+/// tile - ((th-1)*stride + (k-1)*dilation + 1 rows, likewise columns, for up
+/// to 16 channel vectors of 16 bytes - has to fit 52 KB so that three
+/// workgroups share the 160 KB of a CU.  Width first: the candidate (at most
+/// 16) that wastes the fewest pixels at the right edge; then the tallest tile
+/// that fits.  {0, 0} when not even one pixel fits.
+std::pair<unsigned, unsigned> chooseDepthwiseTile(const Simple2D &s,
+                                                  std::size_t vecs) {
+  const std::size_t vecBlock = std::min<std::size_t>(vecs, 16);
+  const std::size_t budget = (52 * 1024) / 16; // 16-byte elements
+  auto patch = [](unsigned t, unsigned stride, unsigned k, unsigned dil) {
+    return std::size_t(t - 1) * stride + std::size_t(k - 1) * dil + 1;
+  };
+  for (unsigned maxW = 16; maxW >= 1; maxW /= 2) {
+    unsigned bestW = 0;
+    std::size_t bestWaste = ~std::size_t(0);
+    for (unsigned tw = std::min(maxW, s.outW); tw > maxW / 2; --tw) {
+      const std::size_t waste = (s.outW + tw - 1) / tw * tw - s.outW;
+      if (waste < bestWaste) {
+        bestWaste = waste;
+        bestW = tw;
+      }
+    }
+    if (bestW == 0)
+      continue;
+    const std::size_t pw = patch(bestW, s.strideW, s.kW, s.dilW);
+    unsigned bestH = 0;
+    for (unsigned th = 1; th <= std::min(16u, s.outH); ++th)
+      if (patch(th, s.strideH, s.kH, s.dilH) *
+              ((pw * vecBlock + 63) / 64 * 64) <=
+          budget) // rows are padded to whole 64-element loads
+        bestH = th;
+    if (bestH)
+      return {bestH, bestW};
+  }
+  return {0, 0};
+}
+
 } // namespace
 
 mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
@@ -159,6 +197,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
 
   // Which kernels can take this convolution at all?
   std::string igemmWhyNot, dwWhyNot;
+  std::pair<unsigned, unsigned> dwTile{0, 0};
   if (plan.zeroConv)
     igemmWhyNot = dwWhyNot = "all outputs are zero";
   else if (!s.ok)
@@ -180,6 +219,10 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       dwWhyNot = "not one channel per group";
     else if (p.numConvGroups % 8 != 0)
       dwWhyNot = "channel count not a multiple of 8";
+    else if (plan.inputElems * 2 >= (1ull << 31))
+      dwWhyNot = "tensor too large for 32-bit buffer addressing";
+    else if ((dwTile = chooseDepthwiseTile(s, p.numConvGroups / 8)).first == 0)
+      dwWhyNot = "input patch of a single output pixel exceeds the LDS budget";
   }
 
   // Choose.  PopLibs method names map onto the kernels that take their role:
@@ -264,6 +307,18 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     d.strideH = s.strideH, d.strideW = s.strideW;
     d.dilH = s.dilH, d.dilW = s.dilW;
     d.loH = s.loH, d.hiH = s.hiH, d.loW = s.loW, d.hiW = s.hiW;
+    d.tileH = dwTile.first, d.tileW = dwTile.second;
+    if (pc.tileH || pc.tileW) {
+      d.tileH = pc.tileH ? pc.tileH : d.tileH;
+      d.tileW = pc.tileW ? pc.tileW : d.tileW;
+      const std::size_t vb = std::min<std::size_t>(p.numConvGroups / 8, 16);
+      const std::size_t ph = (d.tileH - 1) * d.strideH + (d.kH - 1) * d.dilH + 1;
+      const std::size_t pw = (d.tileW - 1) * d.strideW + (d.kW - 1) * d.dilW + 1;
+      if (ph * ((pw * vb + 63) / 64 * 64) * 16 > 64 * 1024)
+        throw poplar::invalid_option(
+            "planConstraints gfx950 tileH x tileW: the input patch of such a "
+            "tile does not fit 64 KB of LDS");
+    }
     plan.weightPackedElems = plan.weightElems; // [kH*kW][C]
   } else {
     plan.weightPackedElems = plan.weightElems; // [G][K][Ci][Co]
@@ -313,6 +368,8 @@ std::string mxconv_plan::describe() const {
   } else if (kernel == Kernel::DEPTHWISE) {
     const auto &d = depthwise;
     os << "        channels                   " << d.channels << "\n";
+    os << "        output tile H x W          " << d.tileH << " x " << d.tileW
+       << "\n";
     os << "        packed weights             [" << d.kH * d.kW << "]["
        << d.channels << "]\n";
   } else {
