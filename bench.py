@@ -251,6 +251,10 @@ def main():
                     help="headline workload (c2, c3, c4, c5)")
     ap.add_argument("--only", action="store_true",
                     help="skip the other workloads and the CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 64 MiB device copy, so that a "
+                         "counter run of this command holds a kernel of known "
+                         "HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no "
@@ -262,6 +266,13 @@ def main():
     from poplibs_amd import capi
     pa.lib()
     wls = _workloads(pa)
+    if args.copy_calibration:
+        src = torch.empty(64 * 2 ** 20, dtype=torch.uint8,
+                          device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     def measure(key, steps, warmup):
         wl = wls[key]
