@@ -24,11 +24,15 @@
 // (buffer_load_dwordx4 ... lds): no staging registers, so the depth of the
 // prefetch is set by LDS capacity - all stages but one are in flight while
 // one is being multiplied.  Such a load puts lane l's 16 bytes at LDS base +
-// 16 l, i.e. one instruction fills 8 consecutive 128-byte tile rows.  To keep
-// the consumers' MFMA-operand reads (32 rows, same k) free of bank conflicts
-// the 16-byte chunks of row r are stored at position (chunk ^ (r & 7)); the
-// permutation is applied on the global side, by choosing which chunk each
-// lane fetches, and undone in the LDS read address.
+// 16 l, i.e. one instruction fills 8 consecutive 128-byte tile rows.  LDS has
+// 64 banks of 4 bytes (256 bytes per clock); an MFMA-operand read (32 rows,
+// same k, 16 bytes per lane) runs at that rate only if each run of 16 lanes
+// covers all 64 banks.  So the 16-byte chunks of row r are stored at position
+// (chunk ^ (r & 7)), and in every second 8-row block rows 2i and 2i+1 swap
+// places, which moves that block's chunks to the other 128 bytes of the
+// 256-byte bank period.  The permutation is applied on the global side, by
+// choosing which row and chunk each lane fetches, and undone in the LDS read
+// address.
 // Each consumer wave multiplies its 64 x BN/2 sub-tile with
 // v_mfma_f32_32x32x16_f16 (fp16) or v_mfma_f32_32x32x64_f8f6f4 (fp8),
 // accumulating in fp32.
@@ -147,14 +151,21 @@ __device__ __forceinline__ void loadToLds(__amdgpu_buffer_rsrc_t buffer,
 
 template <int EB> struct Mma;
 
-/// Tile rows in LDS are 128 bytes, chunk c of row r at chunk position
-/// c ^ (r & 7).  `row` = lane & 31 is the row inside a 32-row block (block
-/// bases are multiples of 8, so r & 7 == lane & 7).
+/// Tile rows in LDS are 128 bytes.  Row r sits at row position
+/// r ^ ((r >> 3) & 1), its chunk c at chunk position c ^ (r & 7).  A wave reads
+/// fragments of 32-row blocks whose bases are multiples of 32, so both depend
+/// on the lane only: this is the byte offset of (row lane & 31, chunk 0)
+/// before the chunk XOR.
+__device__ __forceinline__ int fragmentRowOffset(int lane) {
+  return ((lane & 31) ^ ((lane >> 3) & 1)) * kRowBytes;
+}
 
-/// The MFMA operands ("fragments") of one k-step for one consumer wave, and
-/// the two halves of a k-step's work: fetch every fragment from LDS, multiply
-/// sub-steps [S0, S1).  Keeping them apart lets the consumer loop start the
-/// next k-step's LDS reads before the current k-step's last MFMAs.
+/// The MFMA operands ("fragments") of one consumer wave.  A k-step is split
+/// into kSubSteps sub-steps; fragment set s holds what sub-step s multiplies.
+/// load<S> issues the LDS reads of one set, mul<S> the MFMAs that consume it:
+/// the first MFMA, then `between()` (the caller's LDS reads for a later
+/// sub-step, so that they are in flight under the remaining MFMAs), then the
+/// rest.
 
 /// fp16: 4 sub-steps of K=16, 32 bytes (two chunks, one per half-wave) each.
 template <> struct Mma<2> {
@@ -162,35 +173,32 @@ template <> struct Mma<2> {
   template <int TN> struct Frags {
     half8 a[kSubSteps][2], b[kSubSteps][TN];
   };
-  template <int TN>
+  template <int S, int TN>
   static __device__ __forceinline__ void
   load(const char *ldsA, const char *ldsB, int lane, Frags<TN> &f) {
-    const int row = lane & 31;
-    const int swz = lane & 7, half = lane >> 5;
+    const int off = fragmentRowOffset(lane) +
+                    (((S * 2 + (lane >> 5)) ^ (lane & 7)) << 4);
 #pragma unroll
-    for (int s = 0; s != kSubSteps; ++s) {
-      const int off = row * kRowBytes + (((s * 2 + half) ^ swz) << 4);
+    for (int i = 0; i != 2; ++i)
+      f.a[S][i] =
+          *reinterpret_cast<const half8 *>(ldsA + i * 32 * kRowBytes + off);
 #pragma unroll
-      for (int i = 0; i != 2; ++i)
-        f.a[s][i] =
-            *reinterpret_cast<const half8 *>(ldsA + i * 32 * kRowBytes + off);
-#pragma unroll
-      for (int j = 0; j != TN; ++j)
-        f.b[s][j] =
-            *reinterpret_cast<const half8 *>(ldsB + j * 32 * kRowBytes + off);
-    }
+    for (int j = 0; j != TN; ++j)
+      f.b[S][j] =
+          *reinterpret_cast<const half8 *>(ldsB + j * 32 * kRowBytes + off);
   }
-  template <int S0, int S1, int TN, int FA, int FB>
-  static __device__ __forceinline__ void mul(const Frags<TN> &f,
-                                             floatx16 (&acc)[2][TN]) {
+  template <int S, int TN, int FA, int FB, class F>
+  static __device__ __forceinline__ void
+  mul(const Frags<TN> &f, floatx16 (&acc)[2][TN], F &&between) {
 #pragma unroll
-    for (int s = S0; s != S1; ++s)
+    for (int i = 0; i != 2; ++i)
 #pragma unroll
-      for (int i = 0; i != 2; ++i)
-#pragma unroll
-        for (int j = 0; j != TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-              f.a[s][i], f.b[s][j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j != TN; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            f.a[S][i], f.b[S][j], acc[i][j], 0, 0, 0);
+        if (i == 0 && j == 0)
+          between();
+      }
   }
 };
 
@@ -201,42 +209,39 @@ template <> struct Mma<1> {
   template <int TN> struct Frags {
     intx8 a[kSubSteps][2], b[kSubSteps][TN];
   };
-  template <int TN>
+  template <int S, int TN>
   static __device__ __forceinline__ void
   load(const char *ldsA, const char *ldsB, int lane, Frags<TN> &f) {
-    const int row = lane & 31;
-    const int swz = lane & 7, half = lane >> 5;
+    const int rowOff = fragmentRowOffset(lane);
+    const int c0 = S * 4 + (lane >> 5) * 2;
+    const int off0 = rowOff + ((c0 ^ (lane & 7)) << 4);
+    const int off1 = rowOff + (((c0 + 1) ^ (lane & 7)) << 4);
+    // 32 bytes per lane: two chunks that the swizzle may have separated.
+    auto load32 = [&](const char *p) {
+      const uintx4 lo = *reinterpret_cast<const uintx4 *>(p + off0);
+      const uintx4 hi = *reinterpret_cast<const uintx4 *>(p + off1);
+      return intx8{int(lo.x), int(lo.y), int(lo.z), int(lo.w),
+                   int(hi.x), int(hi.y), int(hi.z), int(hi.w)};
+    };
 #pragma unroll
-    for (int s = 0; s != kSubSteps; ++s) {
-      const int c0 = s * 4 + half * 2;
-      const int off0 = row * kRowBytes + ((c0 ^ swz) << 4);
-      const int off1 = row * kRowBytes + (((c0 + 1) ^ swz) << 4);
-      // 32 bytes per lane: two chunks that the swizzle may have separated.
-      auto load32 = [&](const char *p) {
-        const uintx4 lo = *reinterpret_cast<const uintx4 *>(p + off0);
-        const uintx4 hi = *reinterpret_cast<const uintx4 *>(p + off1);
-        return intx8{int(lo.x), int(lo.y), int(lo.z), int(lo.w),
-                     int(hi.x), int(hi.y), int(hi.z), int(hi.w)};
-      };
+    for (int i = 0; i != 2; ++i)
+      f.a[S][i] = load32(ldsA + i * 32 * kRowBytes);
 #pragma unroll
-      for (int i = 0; i != 2; ++i)
-        f.a[s][i] = load32(ldsA + i * 32 * kRowBytes);
-#pragma unroll
-      for (int j = 0; j != TN; ++j)
-        f.b[s][j] = load32(ldsB + j * 32 * kRowBytes);
-    }
+    for (int j = 0; j != TN; ++j)
+      f.b[S][j] = load32(ldsB + j * 32 * kRowBytes);
   }
-  template <int S0, int S1, int TN, int FA, int FB>
-  static __device__ __forceinline__ void mul(const Frags<TN> &f,
-                                             floatx16 (&acc)[2][TN]) {
+  template <int S, int TN, int FA, int FB, class F>
+  static __device__ __forceinline__ void
+  mul(const Frags<TN> &f, floatx16 (&acc)[2][TN], F &&between) {
 #pragma unroll
-    for (int s = S0; s != S1; ++s)
+    for (int i = 0; i != 2; ++i)
 #pragma unroll
-      for (int i = 0; i != 2; ++i)
-#pragma unroll
-        for (int j = 0; j != TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-              f.a[s][i], f.b[s][j], acc[i][j], FA, FB, 0, 0, 0, 0);
+      for (int j = 0; j != TN; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+            f.a[S][i], f.b[S][j], acc[i][j], FA, FB, 0, 0, 0, 0);
+        if (i == 0 && j == 0)
+          between();
+      }
   }
 };
 
@@ -274,9 +279,11 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   if (producer) {
     const int pt = t - (kThreads - kProducers);
     const int pw = pt >> 6; // producer wave
-    // Lane l of a load fills LDS row (l >> 3) of an 8-row block at chunk
-    // position (l & 7); it therefore fetches chunk (l & 7) ^ (row & 7).
-    const int rowInBlock = lane >> 3;
+    // Lane l of a load fills row position (l >> 3) of an 8-row block at chunk
+    // position (l & 7).  This wave's blocks all have the parity of pw: in
+    // odd blocks that position belongs to row (l >> 3) ^ 1; either way the
+    // lane fetches chunk (l & 7) ^ (row & 7).
+    const int rowInBlock = (lane >> 3) ^ (pw & 1);
     const int chunk = (lane & 7) ^ rowInBlock;
     // The buffer starts `shift` bytes before the tensor, as many as the
     // largest amount a padded window reaches above / left of an image, so
@@ -402,38 +409,46 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
         for (int v = 0; v != 16; ++v)
           acc[i][j][v] = 0.0f;
     using M = Mma<EB>;
-    constexpr int kLast = M::kSubSteps - 1;
-    typename M::template Frags<TN> f0, f1;
-    auto fetch = [&](uint32_t kt, typename M::template Frags<TN> &f) {
+    constexpr int SS = M::kSubSteps;
+    constexpr int P = SS / 2; // sub-steps fetched ahead
+    typename M::template Frags<TN> f;
+    // Instructions may not be moved across this point: the order written
+    // here - which LDS reads are in flight under which MFMAs - is the
+    // software pipeline.
+    auto pin = [] { __builtin_amdgcn_sched_barrier(0); };
+    auto fetch = [&](uint32_t kt, auto sub) {
       const char *stage = lds + (kt % NS) * kTileBytes;
-      M::template load<TN>(stage + wm * 64 * kRowBytes,
-                           stage + (kBlockM + wn * (BN / 2)) * kRowBytes, lane,
-                           f);
+      M::template load<decltype(sub)::value, TN>(
+          stage + wm * 64 * kRowBytes,
+          stage + (kBlockM + wn * (BN / 2)) * kRowBytes, lane, f);
     };
-    // One k-step: multiply all sub-steps but the last, meet the producers
-    // (this stage's LDS reads have all returned by then: the stage may be
-    // refilled), start the next k-step's LDS reads, and only then issue the
-    // last sub-step's MFMAs - the LDS pipe, which is as busy as the matrix
-    // cores with this tile shape, never waits for them.
-    auto step = [&](uint32_t kt, typename M::template Frags<TN> &cur,
-                    typename M::template Frags<TN> &next) {
-      M::template mul<0, kLast, TN, FA, FB>(cur, acc);
-      MXK_WAIT_LGKMCNT0();
-      stepBarrier(); // barrier kt + 1: step kt + 1 has landed
-      if (kt + 1 != a.kSteps)
-        fetch(kt + 1, next);
-      M::template mul<kLast, kLast + 1, TN, FA, FB>(cur, acc);
-    };
+    // Sub-steps [0, P) of a k-step are fetched during the previous k-step,
+    // sub-step s + P under the MFMAs of sub-step s.  The workgroup barrier
+    // sits before the last sub-step: every LDS read of this stage has
+    // returned by then (the producers may refill it), the next stage has
+    // landed, and its first reads go out under the last sub-step's MFMAs.
     stepBarrier(); // barrier 0
     if (a.kSteps != 0)
-      fetch(0, f0);
-    uint32_t kt = 0;
-    for (; kt + 1 < a.kSteps; kt += 2) {
-      step(kt, f0, f1);
-      step(kt + 1, f1, f0);
+      staticFor<0, P>([&](auto sub) { fetch(0, sub); });
+    pin();
+    for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
+      staticFor<0, SS - 1>([&](auto sub) {
+        constexpr int S = decltype(sub)::value;
+        M::template mul<S, TN, FA, FB>(f, acc, [&] {
+          if constexpr (S + P < SS)
+            fetch(kt, std::integral_constant<int, S + P>{});
+        });
+        pin();
+      });
+      MXK_WAIT_LGKMCNT0();
+      stepBarrier(); // barrier kt + 1: step kt + 1 has landed
+      pin();
+      M::template mul<SS - 1, TN, FA, FB>(f, acc, [&] {
+        if (kt + 1 != a.kSteps)
+          staticFor<0, P>([&](auto sub) { fetch(kt + 1, sub); });
+      });
+      pin();
     }
-    if (kt < a.kSteps)
-      step(kt, f0, f1);
   }
   // One more meeting point: the producers' trailing loads have landed, so
   // LDS can be reused for the output tile.
