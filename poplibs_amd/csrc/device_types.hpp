@@ -59,5 +59,19 @@ __device__ __forceinline__ void storeOut(__half *p, size_t i, float v) {
   p[i] = __float2half_rn(v);
 }
 
+/// Four consecutive outputs as one vector store; p is aligned to the vector.
+__device__ __forceinline__ void storeOut4(float *p, const float (&v)[4]) {
+  *reinterpret_cast<float4 *>(p) = float4{v[0], v[1], v[2], v[3]};
+}
+__device__ __forceinline__ void storeOut4(__half *p, const float (&v)[4]) {
+  union {
+    __half2 h[2];
+    uint2 u;
+  } pack;
+  pack.h[0] = __floats2half2_rn(v[0], v[1]);
+  pack.h[1] = __floats2half2_rn(v[2], v[3]);
+  *reinterpret_cast<uint2 *>(p) = pack.u;
+}
+
 } // namespace mxk
 #endif

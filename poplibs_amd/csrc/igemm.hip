@@ -37,8 +37,9 @@
 // v_mfma_f32_32x32x16_f16 (fp16) or v_mfma_f32_32x32x64_f8f6f4 (fp8),
 // accumulating in fp32.
 //
-// Addressing.  Everything per-row is computed once, before the loop: a byte
-// offset and a bit mask "kernel tap t reads inside the input".  In the loop
+// Addressing.  Everything per-row is computed once, before the loop, by one
+// thread per row (the result is handed to the producers through a small LDS
+// table): a byte offset and a bit mask "kernel tap t reads inside the input".  In the loop
 // the wave-uniform part of the address (kernel tap, channel block) travels in
 // the scalar offset of the buffer load, and a row whose tap falls on padding
 // gets an out-of-range vector offset, for which the buffer unit delivers
@@ -86,8 +87,28 @@ constexpr int kRowsPerPass = kProducers / kChunks; // rows per producer pass
 constexpr int kLoadBytes = 64 * 16; // LDS bytes one wave-wide load fills
 constexpr uint32_t kOutOfRange = 0x80000000u; // beyond any buffer we accept
 
+/// Division of a 31-bit number by a launch constant: one multiply-high and a
+/// shift (round-up method: mul = ceil(2^(31 + s) / d), s = ceil(log2 d)).
+struct FastDiv {
+  uint32_t mul, shift, one;
+  __device__ __forceinline__ uint32_t operator()(uint32_t n) const {
+    return one ? n : (__umulhi(n, mul) >> shift);
+  }
+};
+
+FastDiv makeFastDiv(uint32_t d) {
+  if (d <= 1)
+    return {0, 0, 1};
+  uint32_t s = 0;
+  while ((1ull << s) < d)
+    ++s;
+  const uint64_t m = ((1ull << (31 + s)) + d - 1) / d;
+  return {uint32_t(m), s - 1, 0};
+}
+
 struct IgemmArgs {
   IgemmDesc d;
+  FastDiv divOutW, divOutH;
   uint32_t M;        // batch * outH * outW
   uint32_t mTiles, nTiles;
   uint32_t kSteps;   // kPadded / elements per k-step
@@ -195,7 +216,7 @@ template <> struct Mma<2> {
 #pragma unroll
       for (int j = 0; j != TN; ++j) {
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-            f.a[S][i], f.b[S][j], acc[i][j], 0, 0, 0);
+            f.b[S][j], f.a[S][i], acc[i][j], 0, 0, 0);
         if (i == 0 && j == 0)
           between();
       }
@@ -238,7 +259,7 @@ template <> struct Mma<1> {
 #pragma unroll
       for (int j = 0; j != TN; ++j) {
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-            f.a[S][i], f.b[S][j], acc[i][j], FA, FB, 0, 0, 0, 0);
+            f.b[S][j], f.a[S][i], acc[i][j], FB, FA, 0, 0, 0, 0);
         if (i == 0 && j == 0)
           between();
       }
@@ -256,7 +277,10 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   constexpr int BROWS = BN / kRowsPerPass;      // B rows loaded per thread
   constexpr int kTileBytes = (kBlockM + BN) * kRowBytes; // one stage
   constexpr int kLoads = AROWS + BROWS; // loads per producer thread and step
-  extern __shared__ __align__(16) char lds[]; // NS * kTileBytes
+  extern __shared__ __align__(16) char lds[]; // NS * kTileBytes + row table
+  // Per tile row: {byte offset of the input element under tap (0, 0), channel
+  // 0 of the group; mask of taps that read inside the input}.
+  uint2 *rowTable = reinterpret_cast<uint2 *>(lds + NS * kTileBytes);
 
   const IgemmDesc &d = a.d;
   const uint32_t tile = xcdSwizzle(blockIdx.x, gridDim.x);
@@ -301,36 +325,9 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
     // Per A row (output pixel) of this thread: the byte offset (from the
     // shifted buffer start) of the input element under kernel tap (0, 0),
     // channel chunk `chunk`, and one bit per kernel tap telling whether that
-    // tap reads inside the input.
+    // tap reads inside the input - read from the row table further down, once
+    // the weight loads, which need none of it, are on their way.
     uint32_t rowOff[AROWS], tapMask[AROWS];
-#pragma unroll
-    for (int r = 0; r != AROWS; ++r) {
-      const uint32_t m = mTile * kBlockM + (r * 4 + pw) * 8 + rowInBlock;
-      const bool rowValid = m < a.M;
-      const uint32_t mm = rowValid ? m : 0;
-      const uint32_t ow = mm % d.outW;
-      const uint32_t oh = (mm / d.outW) % d.outH;
-      const uint32_t b = mm / (d.outW * d.outH);
-      const int ihBase = int(oh * d.strideH) - d.padH;
-      const int iwBase = int(ow * d.strideW) - d.padW;
-      rowOff[r] =
-          shift +
-          ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
-              pixelBytes +
-          g * ciBytes + chunk * 16;
-      uint32_t mask = 0;
-      if (rowValid)
-        for (uint32_t kh = 0, tap = 0; kh != d.kH; ++kh) {
-          const int ih = ihBase + int(kh * d.dilH);
-          const bool hOk = ih >= int(d.loH) && ih < int(d.hiH);
-          for (uint32_t kw = 0; kw != d.kW; ++kw, ++tap) {
-            const int iw = iwBase + int(kw * d.dilW);
-            if (hOk && iw >= int(d.loW) && iw < int(d.hiW))
-              mask |= 1u << tap;
-          }
-        }
-      tapMask[r] = mask;
-    }
 
     // Position inside K of the data loaded next.  UNI: (tap, byte offset of
     // the channel block inside the tap) of the whole k-step, wave-uniform.
@@ -357,10 +354,10 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
                 chunk * 16;
     uint32_t kByte = 0; // byte offset of the next k-step along a B row
 
-    // Issues the loads of the next k-step into LDS stage `stage` and moves on
-    // along K.  Beyond the last k-step every offset is out of range: the
-    // stage is filled with zeros that are never multiplied.
-    auto loadStage = [&](uint32_t stage) {
+    // Issue the A / B loads of the next k-step into LDS stage `stage` and
+    // move on along K.  Beyond the last k-step every offset is out of range:
+    // the stage is filled with zeros that are never multiplied.
+    auto loadA = [&](uint32_t stage) {
       char *base = lds + stage * kTileBytes + pw * kLoadBytes;
       const uint32_t tapOff = (kh * d.dilH * d.inW + kw * d.dilW) * pixelBytes;
       const uint32_t tapBit = tap < taps ? (1u << tap) : 0u;
@@ -375,32 +372,87 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
                     ok ? rowOff[r] - chunk * 16 + tapOff + ciOff : kOutOfRange,
                     0);
       }
+      ciOff += kRowBytes;
+      normalise();
+    };
+    auto loadB = [&](uint32_t stage) {
+      char *base = lds + stage * kTileBytes + pw * kLoadBytes;
       const uint32_t kOff = kByte < a.kPadded * EB ? kByte : kOutOfRange;
 #pragma unroll
       for (int r = 0; r != BROWS; ++r)
         loadToLds(wBuf,
                   (LdsPtr)(base + kBlockM * kRowBytes + r * 4 * kLoadBytes),
                   bOff[r] + kOff, 0);
-      ciOff += kRowBytes;
-      normalise();
       kByte += kRowBytes;
     };
 
     // NS - 1 k-steps in flight; wait for the oldest before each barrier.
+    // Start-up order: all weight loads, then (row table ready) all input
+    // loads; from then on input and weight loads of one k-step together.
 #pragma unroll
     for (int s = 0; s != NS - 1; ++s)
-      loadStage(s);
-    MXK_WAIT_VMCNT((NS - 2) * kLoads);
+      loadB(s);
+    stepBarrier(); // the row table is complete
+#pragma unroll
+    for (int r = 0; r != AROWS; ++r) {
+      const uint2 e = rowTable[(r * 4 + pw) * 8 + rowInBlock];
+      rowOff[r] = e.x + chunk * 16;
+      tapMask[r] = e.y;
+    }
+#pragma unroll
+    for (int s = 0; s != NS - 1; ++s)
+      loadA(s);
+    MXK_WAIT_VMCNT((NS - 2) * AROWS);
     stepBarrier(); // barrier 0: step 0 is in LDS stage 0
     for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
       // Stage (kt - 1) % NS was multiplied before the last barrier: refill it
-      // with step kt + NS - 1, then make sure step kt + 1 has landed.
-      loadStage((kt + NS - 1) % NS);
-      MXK_WAIT_VMCNT((NS - 2) * kLoads);
+      // with step kt + NS - 1, then make sure step kt + 1 has landed.  The
+      // first time round the start-up order still shows in the queue.
+      loadA((kt + NS - 1) % NS);
+      loadB((kt + NS - 1) % NS);
+      if (kt == 0)
+        MXK_WAIT_VMCNT((NS - 3) * AROWS + kLoads);
+      else
+        MXK_WAIT_VMCNT((NS - 2) * kLoads);
       stepBarrier(); // barrier kt + 1
     }
     MXK_WAIT_VMCNT(0); // the trailing zero loads, before LDS is reused
   } else {
+    // While the producers start the weight loads, the first 128 consumer
+    // threads work out the row table, one tile row each.
+    if (t < kBlockM) {
+      const uint32_t m = mTile * kBlockM + t;
+      const bool rowValid = m < a.M;
+      const uint32_t mm = rowValid ? m : 0;
+      const uint32_t q = a.divOutW(mm);
+      const uint32_t ow = mm - q * d.outW;
+      const uint32_t b = a.divOutH(q);
+      const uint32_t oh = q - b * d.outH;
+      const int ihBase = int(oh * d.strideH) - d.padH;
+      const int iwBase = int(ow * d.strideW) - d.padW;
+      const uint32_t shift = (uint32_t(d.padH > 0 ? d.padH : 0) * d.inW +
+                              uint32_t(d.padW > 0 ? d.padW : 0)) *
+                             pixelBytes;
+      uint32_t kwMask = 0, mask = 0;
+      for (uint32_t kw = 0; kw != d.kW; ++kw) {
+        const int iw = iwBase + int(kw * d.dilW);
+        if (iw >= int(d.loW) && iw < int(d.hiW))
+          kwMask |= 1u << kw;
+      }
+      for (uint32_t kh = 0; kh != d.kH; ++kh) {
+        const int ih = ihBase + int(kh * d.dilH);
+        if (ih >= int(d.loH) && ih < int(d.hiH))
+          mask |= kwMask << (kh * d.kW);
+      }
+      rowTable[t] = uint2{
+          shift +
+              ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
+                  pixelBytes +
+              g * ciBytes,
+          rowValid ? mask : 0u};
+    }
+    MXK_WAIT_LGKMCNT0();
+    stepBarrier(); // the row table is complete
 #pragma unroll
     for (int i = 0; i != 2; ++i)
 #pragma unroll
@@ -457,29 +509,38 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   // Epilogue.  All k-steps are consumed and every wave is past the last
   // barrier, so LDS is free: the consumers lay the finished tile out as
   // [128 rows][BN outputs] (+ 16 bytes of padding per row), then everybody
-  // copies it out.  Lane l of a 32x32 accumulator holds column l % 32 and
-  // rows 8 * (v / 4) + 4 * (l / 32) + v % 4 for v = 0..15.
+  // copies it out.  The weights were the MFMA's row operand, so lane l of a
+  // 32x32 accumulator holds output pixel l % 32 and output channels
+  // 8 * (v / 4) + 4 * (l / 32) + v % 4 for v = 0..15: runs of four channels,
+  // contiguous in the channels-last output, that go to LDS as one vector.
   constexpr int kOutRow = BN * int(sizeof(OutT)) + 16;
   static_assert(kBlockM * kOutRow <= NS * kTileBytes, "epilogue tile fits LDS");
   if (!producer) {
-    const uint32_t col = lane & 31, rowOff4 = (lane >> 5) * 4;
+    const uint32_t mRow = lane & 31, nOff4 = (lane >> 5) * 4;
 #pragma unroll
-    for (int j = 0; j != TN; ++j) {
-      const uint32_t nLocal = wn * (BN / 2) + j * 32 + col;
-      const uint32_t n = nTile * BN + nLocal;
-      const float bv = (bias && n < d.outChansPerGroup)
-                           ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
-                           : 0.0f;
+    for (int j = 0; j != TN; ++j)
 #pragma unroll
-      for (int i = 0; i != 2; ++i)
+      for (int q = 0; q != 4; ++q) {
+        const uint32_t nLocal = wn * (BN / 2) + j * 32 + 8 * q + nOff4;
+        float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (bias) {
+          const uint32_t n = nTile * BN + nLocal;
 #pragma unroll
-        for (int v = 0; v != 16; ++v) {
-          const uint32_t mLocal =
-              wm * 64 + i * 32 + 8 * (v / 4) + rowOff4 + (v % 4);
-          storeOut(reinterpret_cast<OutT *>(lds + mLocal * kOutRow), nLocal,
-                   acc[i][j][v] * scale + bv);
+          for (int e = 0; e != 4; ++e)
+            if (n + e < d.outChansPerGroup)
+              bv[e] = Load<OutT>::at(bias, g * d.outChansPerGroup + n + e, 0);
         }
-    }
+#pragma unroll
+        for (int i = 0; i != 2; ++i) {
+          const uint32_t mLocal = wm * 64 + i * 32 + mRow;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e != 4; ++e)
+            v[e] = acc[i][j][q * 4 + e] * scale + bv[e];
+          storeOut4(reinterpret_cast<OutT *>(lds + mLocal * kOutRow) + nLocal,
+                    v);
+        }
+      }
   }
   __syncthreads();
   constexpr int kVecElems = 16 / int(sizeof(OutT));
@@ -514,7 +575,8 @@ hipError_t run(const IgemmArgs &a, const void *in, const void *w,
     return hipSuccess;
   if (blocks > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
-  constexpr int ldsBytes = NS * (kBlockM + BN) * kRowBytes;
+  constexpr int ldsBytes =
+      NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
   // More than the 64 KB a kernel gets by default: raise the limit once.
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void *>(&igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>),
@@ -590,6 +652,8 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
   if (m > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
   a.M = uint32_t(m);
+  a.divOutW = makeFastDiv(d.outW);
+  a.divOutH = makeFastDiv(d.outH);
   a.mTiles = (a.M + kBlockM - 1) / kBlockM;
   a.nTiles = (d.outChansPerGroup + d.blockN - 1) / d.blockN;
   a.coPadded = a.nTiles * d.blockN;
