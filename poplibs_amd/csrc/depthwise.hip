@@ -274,6 +274,9 @@ hipError_t runKernelShape(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream) {
+  if (d.dense3x3)
+    return launchDepthwise3x3(d, inType, outType, in, weightsPacked, bias,
+                                 out, stream);
   if (inType != kHalf || d.channels % 8 != 0 || d.tileH == 0 || d.tileW == 0)
     return hipErrorInvalidValue;
   if (uint64_t(d.batch) * d.outH * d.outW * d.channels == 0)

@@ -59,6 +59,25 @@ __device__ __forceinline__ void storeOut(__half *p, size_t i, float v) {
   p[i] = __float2half_rn(v);
 }
 
+/// Division of a 31-bit number by a launch constant: one multiply-high and a
+/// shift (round-up method: mul = ceil(2^(31 + s) / d), s = ceil(log2 d)).
+struct FastDiv {
+  uint32_t mul, shift, one;
+  __device__ __forceinline__ uint32_t operator()(uint32_t n) const {
+    return one ? n : (__umulhi(n, mul) >> shift);
+  }
+};
+
+inline FastDiv makeFastDiv(uint32_t d) {
+  if (d <= 1)
+    return {0, 0, 1};
+  uint32_t s = 0;
+  while ((1ull << s) < d)
+    ++s;
+  const uint64_t m = ((1ull << (31 + s)) + d - 1) / d;
+  return {uint32_t(m), s - 1, 0};
+}
+
 /// Four consecutive outputs as one vector store; p is aligned to the vector.
 __device__ __forceinline__ void storeOut4(float *p, const float (&v)[4]) {
   *reinterpret_cast<float4 *>(p) = float4{v[0], v[1], v[2], v[3]};

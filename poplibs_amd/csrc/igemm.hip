@@ -87,25 +87,6 @@ constexpr int kRowsPerPass = kProducers / kChunks; // rows per producer pass
 constexpr int kLoadBytes = 64 * 16; // LDS bytes one wave-wide load fills
 constexpr uint32_t kOutOfRange = 0x80000000u; // beyond any buffer we accept
 
-/// Division of a 31-bit number by a launch constant: one multiply-high and a
-/// shift (round-up method: mul = ceil(2^(31 + s) / d), s = ceil(log2 d)).
-struct FastDiv {
-  uint32_t mul, shift, one;
-  __device__ __forceinline__ uint32_t operator()(uint32_t n) const {
-    return one ? n : (__umulhi(n, mul) >> shift);
-  }
-};
-
-FastDiv makeFastDiv(uint32_t d) {
-  if (d <= 1)
-    return {0, 0, 1};
-  uint32_t s = 0;
-  while ((1ull << s) < d)
-    ++s;
-  const uint64_t m = ((1ull << (31 + s)) + d - 1) / d;
-  return {uint32_t(m), s - 1, 0};
-}
-
 struct IgemmArgs {
   IgemmDesc d;
   FastDiv divOutW, divOutH;

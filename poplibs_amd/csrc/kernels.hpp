@@ -94,7 +94,16 @@ struct DepthwiseDesc {
   // Output pixels per workgroup tile, chosen by the planner so that the
   // input patch of a tile fits a third of a CU's LDS.
   uint32_t tileH, tileW;
+  // 1: the dense-loading small-workgroup kernel (3x3 taps, dilation 1,
+  // stride 1 or 2) runs instead of the LDS-tiled one.
+  uint32_t dense3x3;
 };
+/// True for the shapes launchDepthwise3x3 takes.
+bool depthwise3x3Takes(const DepthwiseDesc &d, int inType);
+hipError_t launchDepthwise3x3(const DepthwiseDesc &d, int inType,
+                                 int outType, const void *in,
+                                 const void *weightsPacked, const void *bias,
+                                 void *out, hipStream_t stream);
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream);

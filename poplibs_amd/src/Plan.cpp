@@ -308,6 +308,9 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     d.dilH = s.dilH, d.dilW = s.dilW;
     d.loH = s.loH, d.hiH = s.hiH, d.loW = s.loW, d.hiW = s.hiW;
     d.tileH = dwTile.first, d.tileW = dwTile.second;
+    // An explicit tile asks for the LDS-tiled kernel.
+    d.dense3x3 =
+        !(pc.tileH || pc.tileW) && mxk::depthwise3x3Takes(d, mxk::kHalf);
     if (pc.tileH || pc.tileW) {
       d.tileH = pc.tileH ? pc.tileH : d.tileH;
       d.tileW = pc.tileW ? pc.tileW : d.tileW;
@@ -344,7 +347,10 @@ std::string mxconv_plan::describe() const {
        << " operands, fp32 accumulate)";
     break;
   case Kernel::DEPTHWISE:
-    os << "depthwise direct (vector ALU, LDS halo tiles)";
+    os << (depthwise.dense3x3
+               ? "depthwise direct (vector ALU, dense row loads, small "
+                 "workgroups)"
+               : "depthwise direct (vector ALU, LDS halo tiles)");
     break;
   }
   os << "\n        reason                     " << reason << "\n";
@@ -368,8 +374,9 @@ std::string mxconv_plan::describe() const {
   } else if (kernel == Kernel::DEPTHWISE) {
     const auto &d = depthwise;
     os << "        channels                   " << d.channels << "\n";
-    os << "        output tile H x W          " << d.tileH << " x " << d.tileW
-       << "\n";
+    if (!d.dense3x3)
+      os << "        output tile H x W          " << d.tileH << " x "
+         << d.tileW << "\n";
     os << "        packed weights             [" << d.kH * d.kW << "]["
        << d.channels << "]\n";
   } else {
