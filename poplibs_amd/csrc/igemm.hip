@@ -56,196 +56,10 @@
 // ConvPartialnx1.cpp:52-246), including the quarter (fp8) case whose scale
 // 2^(sIn + sW) is applied once to the fp32 sum
 // (lib/poplin/codelets/inlineAssemblerConv.hpp:28-33).
-#include "device_types.hpp"
-#include "kernels.hpp"
-
-#include <type_traits>
+#include "igemm_common.hpp"
 
 namespace mxk {
 namespace {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef int intx8 __attribute__((ext_vector_type(8)));
-typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
-
-/// Compile-time loop: body(std::integral_constant<int, I>) for I in [0, N).
-template <int I, int N, class F>
-__device__ __forceinline__ void staticFor(F &&body) {
-  if constexpr (I < N) {
-    body(std::integral_constant<int, I>{});
-    staticFor<I + 1, N>(body);
-  }
-}
-
-constexpr int kBlockM = 128;
-constexpr int kRowBytes = 128; // bytes of K per tile row and k-step
-constexpr int kThreads = 512;  // 4 consumer + 4 producer waves
-constexpr int kProducers = 256; // threads that move data
-constexpr int kChunks = kRowBytes / 16; // 16-byte chunks per row
-constexpr int kRowsPerPass = kProducers / kChunks; // rows per producer pass
-constexpr int kLoadBytes = 64 * 16; // LDS bytes one wave-wide load fills
-constexpr uint32_t kOutOfRange = 0x80000000u; // beyond any buffer we accept
-
-struct IgemmArgs {
-  IgemmDesc d;
-  FastDiv divOutW, divOutH;
-  uint32_t M;        // batch * outH * outW
-  uint32_t mTiles, nTiles;
-  uint32_t kSteps;   // kPadded / elements per k-step
-  uint32_t kPadded;  // row length of the packed weights, in elements
-  uint32_t coPadded; // rows per group of the packed weights
-  uint32_t inBytes;  // size of the input tensor
-  uint32_t wBytes;   // size of the packed weights
-};
-
-/// Workgroups are dealt round-robin over the 8 XCDs, each with its own L2.
-/// Give every XCD one contiguous run of tiles so that neighbouring tiles,
-/// which share input halo rows and the weight tile, meet in the same L2.
-__device__ __forceinline__ uint32_t xcdSwizzle(uint32_t bid, uint32_t total) {
-  const uint32_t xcd = bid & 7u, idx = bid >> 3;
-  const uint32_t q = total >> 3, rem = total & 7u;
-  return xcd * q + (xcd < rem ? xcd : rem) + idx;
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t bufferOf(const void *p,
-                                                           uint32_t bytes) {
-  // Raw (stride 0) buffer of `bytes` bytes; 32-bit data format.
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), short(0),
-                                           int(bytes), 0x00020000);
-}
-
-/// `wait until at most n vector-memory operations are outstanding`, leaving
-/// the other counters alone (gfx9 encoding of s_waitcnt).
-#define MXK_WAIT_VMCNT(n)                                                      \
-  __builtin_amdgcn_s_waitcnt(((n)&15) | (((n) >> 4) << 14) | (7 << 4) |       \
-                             (15 << 8))
-
-/// Wait for this wave's LDS reads (and scalar loads) only.
-#define MXK_WAIT_LGKMCNT0() __builtin_amdgcn_s_waitcnt(0xC07F)
-
-/// Workgroup barrier without the release / acquire fences of
-/// __syncthreads().  Those fences would drain every outstanding buffer load
-/// (a load that writes LDS counts as a pending LDS write) at each k-step and
-/// with it the whole prefetch queue.  The callers wait for exactly what the
-/// other side needs - producers: the oldest stage's loads; consumers: their
-/// own LDS reads - before arriving here.
-__device__ __forceinline__ void stepBarrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
-using LdsPtr = __attribute__((address_space(3))) void *;
-
-/// 16 bytes per lane from a buffer straight into LDS: lane l's data lands at
-/// dst + 16 l (dst is wave-uniform).  Out-of-range offsets deliver zeros.
-/// The builtin exists for the GPU target only; the host compilation pass,
-/// which merely needs the kernels' launch stubs, sees an empty body.
-__device__ __forceinline__ void loadToLds(__amdgpu_buffer_rsrc_t buffer,
-                                          LdsPtr dst, uint32_t vectorOffset,
-                                          uint32_t scalarOffset) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, dst, 16, vectorOffset,
-                                           scalarOffset, 0, 0);
-#endif
-}
-
-template <int EB> struct Mma;
-
-/// Tile rows in LDS are 128 bytes.  Row r sits at row position
-/// r ^ ((r >> 3) & 1), its chunk c at chunk position c ^ (r & 7).  A wave reads
-/// fragments of 32-row blocks whose bases are multiples of 32, so both depend
-/// on the lane only: this is the byte offset of (row lane & 31, chunk 0)
-/// before the chunk XOR.
-__device__ __forceinline__ int fragmentRowOffset(int lane) {
-  return ((lane & 31) ^ ((lane >> 3) & 1)) * kRowBytes;
-}
-
-/// The MFMA operands ("fragments") of one consumer wave.  A k-step is split
-/// into kSubSteps sub-steps; fragment set s holds what sub-step s multiplies.
-/// load<S> issues the LDS reads of one set, mul<S> the MFMAs that consume it:
-/// the first MFMA, then `between()` (the caller's LDS reads for a later
-/// sub-step, so that they are in flight under the remaining MFMAs), then the
-/// rest.
-
-/// fp16: 4 sub-steps of K=16, 32 bytes (two chunks, one per half-wave) each.
-template <> struct Mma<2> {
-  static constexpr int kSubSteps = kRowBytes / 32;
-  template <int TN> struct Frags {
-    half8 a[kSubSteps][2], b[kSubSteps][TN];
-  };
-  template <int S, int TN>
-  static __device__ __forceinline__ void
-  load(const char *ldsA, const char *ldsB, int lane, Frags<TN> &f) {
-    const int off = fragmentRowOffset(lane) +
-                    (((S * 2 + (lane >> 5)) ^ (lane & 7)) << 4);
-#pragma unroll
-    for (int i = 0; i != 2; ++i)
-      f.a[S][i] =
-          *reinterpret_cast<const half8 *>(ldsA + i * 32 * kRowBytes + off);
-#pragma unroll
-    for (int j = 0; j != TN; ++j)
-      f.b[S][j] =
-          *reinterpret_cast<const half8 *>(ldsB + j * 32 * kRowBytes + off);
-  }
-  template <int S, int TN, int FA, int FB, class F>
-  static __device__ __forceinline__ void
-  mul(const Frags<TN> &f, floatx16 (&acc)[2][TN], F &&between) {
-#pragma unroll
-    for (int i = 0; i != 2; ++i)
-#pragma unroll
-      for (int j = 0; j != TN; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-            f.b[S][j], f.a[S][i], acc[i][j], 0, 0, 0);
-        if (i == 0 && j == 0)
-          between();
-      }
-  }
-};
-
-/// fp8: 2 sub-steps of K=64, 64 bytes (four chunks, two per half-wave) each.
-/// FA / FB: 0 = E4M3, 1 = E5M2 (the cbsz / blgp operand-format fields).
-template <> struct Mma<1> {
-  static constexpr int kSubSteps = kRowBytes / 64;
-  template <int TN> struct Frags {
-    intx8 a[kSubSteps][2], b[kSubSteps][TN];
-  };
-  template <int S, int TN>
-  static __device__ __forceinline__ void
-  load(const char *ldsA, const char *ldsB, int lane, Frags<TN> &f) {
-    const int rowOff = fragmentRowOffset(lane);
-    const int c0 = S * 4 + (lane >> 5) * 2;
-    const int off0 = rowOff + ((c0 ^ (lane & 7)) << 4);
-    const int off1 = rowOff + (((c0 + 1) ^ (lane & 7)) << 4);
-    // 32 bytes per lane: two chunks that the swizzle may have separated.
-    auto load32 = [&](const char *p) {
-      const uintx4 lo = *reinterpret_cast<const uintx4 *>(p + off0);
-      const uintx4 hi = *reinterpret_cast<const uintx4 *>(p + off1);
-      return intx8{int(lo.x), int(lo.y), int(lo.z), int(lo.w),
-                   int(hi.x), int(hi.y), int(hi.z), int(hi.w)};
-    };
-#pragma unroll
-    for (int i = 0; i != 2; ++i)
-      f.a[S][i] = load32(ldsA + i * 32 * kRowBytes);
-#pragma unroll
-    for (int j = 0; j != TN; ++j)
-      f.b[S][j] = load32(ldsB + j * 32 * kRowBytes);
-  }
-  template <int S, int TN, int FA, int FB, class F>
-  static __device__ __forceinline__ void
-  mul(const Frags<TN> &f, floatx16 (&acc)[2][TN], F &&between) {
-#pragma unroll
-    for (int i = 0; i != 2; ++i)
-#pragma unroll
-      for (int j = 0; j != TN; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-            f.b[S][j], f.a[S][i], acc[i][j], FB, FA, 0, 0, 0, 0);
-        if (i == 0 && j == 0)
-          between();
-      }
-  }
-};
 
 /// UNI: every k-step lies inside one kernel tap (Ci * EB is a multiple of
 /// 128 bytes), so tap and channel block are wave-uniform.
@@ -272,7 +86,6 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   const int t = threadIdx.x;
   const bool producer = t >= kThreads - kProducers; // waves 4-7
   const uint32_t inChans = d.groups * d.inChansPerGroup;
-  const uint32_t outChans = d.groups * d.outChansPerGroup;
   const uint32_t ciBytes = d.inChansPerGroup * EB; // bytes of K per tap
   const uint32_t pixelBytes = inChans * EB;
   const uint32_t taps = d.kH * d.kW;
@@ -449,11 +262,17 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
     // here - which LDS reads are in flight under which MFMAs - is the
     // software pipeline.
     auto pin = [] { __builtin_amdgcn_sched_barrier(0); };
+    const int rowOffset = fragmentRowOffset(lane);
     auto fetch = [&](uint32_t kt, auto sub) {
       const char *stage = lds + (kt % NS) * kTileBytes;
-      M::template load<decltype(sub)::value, TN>(
-          stage + wm * 64 * kRowBytes,
-          stage + (kBlockM + wn * (BN / 2)) * kRowBytes, lane, f);
+      const char *tileA = stage + wm * 64 * kRowBytes + rowOffset;
+      const FragmentAddress at{
+          {tileA, tileA + 32 * kRowBytes},
+          {lane & 7, lane & 7},
+          0,
+          stage + (kBlockM + wn * (BN / 2)) * kRowBytes + rowOffset,
+          lane & 7};
+      M::template load<decltype(sub)::value, TN>(at, lane, f);
     };
     // Sub-steps [0, P) of a k-step are fetched during the previous k-step,
     // sub-step s + P under the MFMAs of sub-step s.  The workgroup barrier
@@ -487,65 +306,10 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   // LDS can be reused for the output tile.
   __syncthreads();
 
-  // Epilogue.  All k-steps are consumed and every wave is past the last
-  // barrier, so LDS is free: the consumers lay the finished tile out as
-  // [128 rows][BN outputs] (+ 16 bytes of padding per row), then everybody
-  // copies it out.  The weights were the MFMA's row operand, so lane l of a
-  // 32x32 accumulator holds output pixel l % 32 and output channels
-  // 8 * (v / 4) + 4 * (l / 32) + v % 4 for v = 0..15: runs of four channels,
-  // contiguous in the channels-last output, that go to LDS as one vector.
-  constexpr int kOutRow = BN * int(sizeof(OutT)) + 16;
-  static_assert(kBlockM * kOutRow <= NS * kTileBytes, "epilogue tile fits LDS");
-  if (!producer) {
-    const uint32_t mRow = lane & 31, nOff4 = (lane >> 5) * 4;
-#pragma unroll
-    for (int j = 0; j != TN; ++j)
-#pragma unroll
-      for (int q = 0; q != 4; ++q) {
-        const uint32_t nLocal = wn * (BN / 2) + j * 32 + 8 * q + nOff4;
-        float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (bias) {
-          const uint32_t n = nTile * BN + nLocal;
-#pragma unroll
-          for (int e = 0; e != 4; ++e)
-            if (n + e < d.outChansPerGroup)
-              bv[e] = Load<OutT>::at(bias, g * d.outChansPerGroup + n + e, 0);
-        }
-#pragma unroll
-        for (int i = 0; i != 2; ++i) {
-          const uint32_t mLocal = wm * 64 + i * 32 + mRow;
-          float v[4];
-#pragma unroll
-          for (int e = 0; e != 4; ++e)
-            v[e] = acc[i][j][q * 4 + e] * scale + bv[e];
-          storeOut4(reinterpret_cast<OutT *>(lds + mLocal * kOutRow) + nLocal,
-                    v);
-        }
-      }
-  }
-  __syncthreads();
-  constexpr int kVecElems = 16 / int(sizeof(OutT));
-  constexpr int kVecsPerRow = BN / kVecElems;
-  // 16-byte stores need the channel count (hence every row start) to be a
-  // multiple of the vector; otherwise fall back to single elements.
-  const bool vectorOk = outChans % kVecElems == 0 &&
-                        d.outChansPerGroup % kVecElems == 0;
-  for (int idx = t; idx < kBlockM * kVecsPerRow; idx += kThreads) {
-    const uint32_t mLocal = idx / kVecsPerRow, vec = idx % kVecsPerRow;
-    const uint32_t m = mTile * kBlockM + mLocal;
-    const uint32_t n = nTile * BN + vec * kVecElems;
-    if (m >= a.M || n >= d.outChansPerGroup)
-      continue;
-    const char *src = lds + mLocal * kOutRow + vec * 16;
-    OutT *dst = out + size_t(m) * outChans + g * d.outChansPerGroup + n;
-    if (vectorOk) {
-      *reinterpret_cast<uintx4 *>(dst) = *reinterpret_cast<const uintx4 *>(src);
-    } else {
-      const OutT *e = reinterpret_cast<const OutT *>(src);
-      for (int k = 0; k != kVecElems && n + k < d.outChansPerGroup; ++k)
-        dst[k] = e[k];
-    }
-  }
+  static_assert(epilogueLdsBytes<BN, OutT>() <= NS * kTileBytes,
+                "epilogue tile fits LDS");
+  igemmEpilogue<BN, OutT>(lds, a, acc, producer, t, lane, wm, wn, mTile, nTile,
+                          g, bias, out, scale);
 }
 
 template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
