@@ -83,6 +83,22 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
                        const void *bias, void *out, const QuarterInfo &q,
                        hipStream_t stream);
 
+/// Pointwise convolution (every kernel extent 1, stride 1, no padding or
+/// truncation, half inputs) with 128, 256 or 512 input channels per group:
+/// a streaming kernel of small workgroups instead of igemm's big tiles.
+struct PointwiseDesc {
+  uint32_t batch, pixels; // pixels per image
+  uint32_t groups, inChansPerGroup, outChansPerGroup;
+};
+bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType);
+/// Elements of the packed weights ([G][32-channel block][k-slice][lane][8]).
+uint64_t pointwisePackedElems(const PointwiseDesc &d);
+hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
+                                      void *dst, hipStream_t stream);
+hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
+                           const void *in, const void *weightsPacked,
+                           const void *bias, void *out, hipStream_t stream);
+
 /// Depthwise (one input and one output channel per group) direct convolution,
 /// 2-D field, stride, zero padding, kernel dilation.
 struct DepthwiseDesc {

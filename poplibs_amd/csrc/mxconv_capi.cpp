@@ -122,6 +122,10 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   switch (plan->kernel) {
   case mxconv_plan::Kernel::IGEMM:
+    if (plan->pointwiseOn)
+      return hipStatus(mxk::launchPointwise(plan->pointwise, inType, outType,
+                                            in, w, bias, out, s),
+                       "pointwise convolution launch");
     return hipStatus(mxk::launchIgemm(plan->igemm, inType, outType, in, w,
                                       bias, out, q, s),
                      "implicit-GEMM convolution launch");
@@ -492,6 +496,10 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
   if (plan->kernel == mxconv_plan::Kernel::IGEMM) {
     if (plan->weightElems != 0)
       REQUIRE_ARG(weights_external);
+    if (plan->pointwiseOn)
+      return hipStatus(mxk::launchPackPointwiseWeights(
+                           plan->pointwise, weights_external, weights_packed, s),
+                       "weight packing");
     return hipStatus(
         mxk::launchPackIgemmWeights(
             weights_external, weights_packed, uint32_t(p.numConvGroups),

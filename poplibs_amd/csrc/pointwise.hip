@@ -1,0 +1,329 @@
+// Pointwise (1x1, stride 1, unpadded) forward convolution with few input
+// channels: a tall, skinny GEMM - M = batch * H * W pixels, K = Ci, N = Co -
+// that is bound by HBM, not by the matrix cores (PopLibs serves it with
+// ConvPartial1x1Out, lib/poplin/codelets/ConvPartial1x1Out.cpp:49-173).
+//
+// igemm.hip's big tiles and deep k-pipeline have nothing to pipeline here:
+// with K = 256 a 128-pixel tile is four k-steps of prologue and epilogue.
+// This kernel streams instead:
+//   * a workgroup is 2 or 4 compute waves + 1 loader wave and owns 64 output
+//     channels; it walks over tiles of 32 or 64 pixels, all of K each;
+//   * the weights never touch LDS: they are packed per (32-channel block,
+//     16-deep k-slice) in MFMA operand order, each compute wave fetches its
+//     block once - one coalesced 16-byte load per lane and slice - and keeps
+//     it in registers for all its tiles.  (Fetching them per tile was
+//     measured to cost as much vector-cache bandwidth as the activations.)
+//   * the loader wave brings the activation rows of a tile (contiguous in
+//     the channels-last tensor) straight into a ring of 3 or 4 LDS buffers
+//     with 1 KB direct-to-LDS loads, 2 or 3 tiles ahead of the compute waves;
+//     row r's 16-byte chunk c is stored at chunk position c ^ (r & 15), so
+//     that an MFMA operand read - 32 rows, one chunk - is spread over all 64
+//     LDS banks (rows are a multiple of 256 bytes).  It issues nothing but
+//     loads, so it can wait for exactly the oldest tile; the compute waves
+//     issue nothing but stores and never wait for memory;
+//   * each compute wave owns one 32 x 32 block of the tile: Ci / 16 MFMAs
+//     (v_mfma_f32_32x32x16_f16, fp32 accumulate), weights as the row operand,
+//     so a lane ends up with runs of 4 consecutive output channels of one
+//     pixel; the block is transposed through a wave-private piece of LDS and
+//     leaves as 16-byte stores, 64 bytes per pixel and store;
+//   * one workgroup barrier per tile: the tile has landed / the buffer before
+//     it has been read.
+#include "igemm_common.hpp"
+
+namespace mxk {
+namespace {
+
+constexpr int kPwChans = 64;         // output channels per workgroup
+constexpr int kPwStageRow = 64 + 16; // staging: 64 bytes of a pixel + padding
+
+struct PwArgs {
+  PointwiseDesc d;
+  uint32_t M;          // batch * pixels per image
+  uint32_t mTiles, nTiles;
+  uint32_t nBlocks;    // 32-channel blocks per group in the packed weights
+  uint32_t walkers;    // workgroups sharing the pixel tiles of one (g, nTile)
+  uint32_t inBytes, wBytes;
+};
+
+/// KS: k-slices of 16 channels (Ci / 16).  TM: pixels per tile (32 or 64);
+/// the workgroup has TM / 16 compute waves and the loader wave.  NB: tile
+/// buffers in LDS; NB - 1 tiles are in flight.
+template <int KS, int TM, int NB, class OutT>
+__global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
+    PwArgs a, const char *__restrict__ in, const char *__restrict__ w,
+    const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  constexpr int kRow = KS * 32;                 // bytes of one activation row
+  constexpr int kChunkBits = KS == 8 ? 4 : KS == 16 ? 5 : 6; // log2(kRow / 16)
+  constexpr int kRowsPerLoad = 1024 / kRow;
+  constexpr int kLoads = TM / kRowsPerLoad; // wave-wide loads per tile
+  constexpr int kTileBytes = TM * kRow;
+  constexpr int kComputeWaves = TM / 16;
+  static_assert((NB - 2) * kLoads <= 63, "wait count fits s_waitcnt");
+  // NB tile buffers | staging
+  extern __shared__ __align__(16) char lds[];
+
+  const PointwiseDesc &d = a.d;
+  const uint32_t walker = blockIdx.x % a.walkers;
+  const uint32_t nTile = (blockIdx.x / a.walkers) % a.nTiles;
+  const uint32_t g = blockIdx.x / (a.walkers * a.nTiles);
+  const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+  const uint32_t pixelBytes = d.groups * d.inChansPerGroup * 2;
+
+  if (wave == kComputeWaves) {
+    // ---- loader.  Load L of a tile fills bytes [1024 L, 1024 L + 1024) of
+    // its buffer, i.e. rows L * kRowsPerLoad ...; lane l holds chunk position
+    // l % (kRow / 16) of row l / (kRow / 16).
+    const __amdgpu_buffer_rsrc_t inBuf = bufferOf(in, a.inBytes);
+    const uint32_t rowInLoad = lane >> kChunkBits;
+    const uint32_t pos = lane & ((1 << kChunkBits) - 1);
+    auto issue = [&](uint32_t mTile, char *buffer) {
+#pragma unroll
+      for (int load = 0; load != kLoads; ++load) {
+        const uint32_t row = load * kRowsPerLoad + rowInLoad;
+        const uint32_t chunk = pos ^ (row & 15u);
+        const uint32_t m = mTile * TM + row;
+        loadToLds(inBuf, (LdsPtr)(buffer + load * 1024),
+                  m < a.M ? m * pixelBytes + g * kRow + chunk * 16
+                          : kOutOfRange,
+                  0);
+      }
+    };
+    // Tiles this walker has no more of are "loaded" all the same, from
+    // beyond the tensor (nothing is fetched): the count of loads in flight
+    // stays what the waits below assume.
+#pragma unroll
+    for (int s = 0; s != NB - 1; ++s)
+      issue(walker + s * a.walkers, lds + s * kTileBytes);
+    uint32_t buffer = NB - 1; // where tile i + NB - 1 goes
+    for (uint32_t mTile = walker; mTile < a.mTiles; mTile += a.walkers) {
+      MXK_WAIT_VMCNT((NB - 2) * kLoads);
+      stepBarrier(); // tile i is in LDS; the buffer before it has been read
+      issue(mTile + (NB - 1) * a.walkers, lds + buffer * kTileBytes);
+      if (++buffer == NB)
+        buffer = 0;
+    }
+    MXK_WAIT_VMCNT(0);
+    return;
+  }
+
+  // ---- compute waves.  This wave's weights -> registers: block nb of the
+  // two 32-channel blocks, every k-slice.
+  const int mb = wave >> 1, nb = wave & 1;
+  half8 wf[KS];
+  {
+    const uintx4 *src =
+        reinterpret_cast<const uintx4 *>(w) +
+        (size_t(g * a.nBlocks + nTile * 2 + nb) * KS) * 64 + lane;
+#pragma unroll
+    for (int ks = 0; ks != KS; ++ks)
+      wf[ks] = __builtin_bit_cast(half8, src[ks * 64]);
+  }
+  // Bias of this lane's channels 8 q + 4 (lane / 32) + e.
+  float biasV[16];
+#pragma unroll
+  for (int v = 0; v != 16; ++v) {
+    const uint32_t n =
+        nTile * kPwChans + nb * 32 + 8 * (v / 4) + 4 * (lane >> 5) + v % 4;
+    biasV[v] = bias && n < d.outChansPerGroup
+                   ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
+                   : 0.0f;
+  }
+  const uint32_t rowLocal = mb * 32 + (lane & 31);
+  const uint32_t swizzle = rowLocal & 15u, half = lane >> 5;
+  char *stage = lds + NB * kTileBytes + wave * 32 * kPwStageRow;
+  const uint32_t outChans = d.groups * d.outChansPerGroup;
+  // Output leaves in passes of 64 bytes per pixel: all 32 channels of the
+  // block (fp16) or 16 of them (fp32).
+  constexpr int kPassChans = 64 / int(sizeof(OutT));
+  constexpr int kVecElems = 16 / int(sizeof(OutT));
+
+  uint32_t buffer = 0;
+  for (uint32_t mTile = walker; mTile < a.mTiles; mTile += a.walkers) {
+    stepBarrier(); // tile i has landed
+    const char *rowPtr = lds + buffer * kTileBytes + rowLocal * kRow;
+    if (++buffer == NB)
+      buffer = 0;
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v != 16; ++v)
+      acc[v] = biasV[v];
+#pragma unroll
+    for (int ks = 0; ks != KS; ++ks) {
+      const half8 x = *reinterpret_cast<const half8 *>(
+          rowPtr + (((ks * 2 + half) ^ swizzle) << 4));
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[ks], x, acc, 0, 0, 0);
+    }
+    // lane = pixel lane % 32, registers = channels 8 (v / 4) + 4 (lane / 32)
+    // + v % 4: transpose through this wave's staging block and store.
+#pragma unroll
+    for (int pass = 0; pass != 32 / kPassChans; ++pass) {
+#pragma unroll
+      for (int q = pass * (kPassChans / 8); q != (pass + 1) * (kPassChans / 8);
+           ++q) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e != 4; ++e)
+          v[e] = acc[q * 4 + e];
+        storeOut4(reinterpret_cast<OutT *>(stage + (lane & 31) * kPwStageRow) +
+                      (8 * q + 4 * half - pass * kPassChans),
+                  v);
+      }
+      // wave-private: only this wave's LDS writes have to be visible
+      MXK_WAIT_LGKMCNT0();
+      const uint32_t vec = lane & 3; // 4 x 16 bytes per pixel and pass
+      const uint32_t n =
+          nTile * kPwChans + nb * 32 + pass * kPassChans + vec * kVecElems;
+#pragma unroll
+      for (int rows = 0; rows != 2; ++rows) {
+        const uint32_t r = rows * 16 + (lane >> 2);
+        const uint32_t m = mTile * TM + mb * 32 + r;
+        const uintx4 data =
+            *reinterpret_cast<const uintx4 *>(stage + r * kPwStageRow + vec * 16);
+        if (m < a.M && n < d.outChansPerGroup)
+          *reinterpret_cast<uintx4 *>(out + size_t(m) * outChans +
+                                      g * d.outChansPerGroup + n) = data;
+      }
+      MXK_WAIT_LGKMCNT0(); // staging is read before the next pass rewrites it
+    }
+  }
+}
+
+/// Weights [G][Co][Ci] -> [G][32-channel block][k-slice][lane][8 halves]:
+/// lane l of a slice holds channel l % 32 of the block, input channels
+/// 16 slice + 8 (l / 32) ... + 8 - the row operand of v_mfma_f32_32x32x16_f16.
+/// Channels past Co are zero.
+__global__ __launch_bounds__(256) void packPointwiseWeightsKernel(
+    const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, uint32_t co,
+    uint32_t ci, uint32_t nBlocks, uint64_t total) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= total)
+    return;
+  const uint32_t e = uint32_t(tid & 7), lane = uint32_t(tid >> 3) & 63;
+  const uint32_t slices = ci / 16;
+  uint64_t r = tid >> 9;
+  const uint32_t ks = uint32_t(r % slices);
+  r /= slices;
+  const uint32_t block = uint32_t(r % nBlocks);
+  const uint64_t g = r / nBlocks;
+  const uint32_t n = block * 32 + (lane & 31);
+  const uint32_t k = ks * 16 + 8 * (lane >> 5) + e;
+  dst[tid] = n < co ? src[(g * co + n) * ci + k] : uint16_t(0);
+}
+
+template <int KS, int TM, int NB, class OutT>
+hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
+               void *out, hipStream_t stream) {
+  constexpr int kComputeWaves = TM / 16;
+  constexpr int ldsBytes =
+      NB * TM * KS * 32 + kComputeWaves * 32 * kPwStageRow;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void *>(&pointwiseKernel<KS, TM, NB, OutT>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+  if (attr != hipSuccess)
+    return attr;
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) !=
+            hipSuccess ||
+        n <= 0)
+      n = 256;
+    return n;
+  }();
+  a.mTiles = (a.M + TM - 1) / TM;
+  // As many workgroups as fit the chip at once (LDS allows 160 KB / ldsBytes
+  // per CU), shared out over the (group, channel tile) pairs.
+  const uint64_t resident = uint64_t(cus) * ((160 * 1024) / ldsBytes);
+  const uint64_t pairs = uint64_t(a.nTiles) * a.d.groups;
+  if (pairs == 0 || a.mTiles == 0)
+    return hipSuccess;
+  uint64_t walkers = resident / pairs;
+  if (walkers < 1)
+    walkers = 1;
+  // ... and no more than give every walker the same number of tiles (to
+  // within one): 3.1 tiles per walker would mean a fourth round at a quarter
+  // of the chip.
+  const uint64_t tilesPerWalker = (a.mTiles + walkers - 1) / walkers;
+  walkers = (a.mTiles + tilesPerWalker - 1) / tilesPerWalker;
+  a.walkers = uint32_t(walkers);
+  const uint64_t blocks = walkers * pairs;
+  // Tile indices up to mTiles + (NB - 1) * walkers are formed in 32 bits.
+  if (blocks > 0x7fffffffull ||
+      uint64_t(a.mTiles) + uint64_t(NB) * walkers > 0x7fffffffull / TM)
+    return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL((pointwiseKernel<KS, TM, NB, OutT>),
+                     dim3(uint32_t(blocks)), dim3(TM * 4 + 64), ldsBytes,
+                     stream, a, static_cast<const char *>(in),
+                     static_cast<const char *>(w),
+                     static_cast<const OutT *>(bias), static_cast<OutT *>(out));
+  return hipGetLastError();
+}
+
+template <class OutT>
+hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
+                     const void *bias, void *out, hipStream_t stream) {
+  // Tiles of 16 KB, three in flight; 32 KB, two in flight, for the widest.
+  switch (a.d.inChansPerGroup) {
+  case 128:
+    return run<8, 64, 4, OutT>(a, in, w, bias, out, stream);
+  case 256:
+    return run<16, 32, 4, OutT>(a, in, w, bias, out, stream);
+  case 512:
+    return run<32, 32, 3, OutT>(a, in, w, bias, out, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+} // namespace
+
+bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType) {
+  const uint32_t ci = d.inChansPerGroup, co = d.outChansPerGroup;
+  const uint64_t m = uint64_t(d.batch) * d.pixels;
+  const uint64_t inBytes = m * d.groups * ci * 2;
+  return inType == kHalf && (outType == kHalf || outType == kFloat) &&
+         (ci == 128 || ci == 256 || ci == 512) && co != 0 &&
+         co % (outType == kHalf ? 8 : 4) == 0 && m != 0 && m < 0x7fffffffull &&
+         inBytes < kOutOfRange &&
+         pointwisePackedElems(d) * 2 < kOutOfRange;
+}
+
+uint64_t pointwisePackedElems(const PointwiseDesc &d) {
+  const uint64_t nBlocks = (d.outChansPerGroup + kPwChans - 1) / kPwChans * 2;
+  return uint64_t(d.groups) * nBlocks * (d.inChansPerGroup / 16) * 512;
+}
+
+hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
+                                      void *dst, hipStream_t stream) {
+  const uint64_t total = pointwisePackedElems(d);
+  if (total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const uint32_t nBlocks = (d.outChansPerGroup + kPwChans - 1) / kPwChans * 2;
+  hipLaunchKernelGGL(packPointwiseWeightsKernel, dim3(uint32_t(blocks)),
+                     dim3(256), 0, stream, static_cast<const uint16_t *>(src),
+                     static_cast<uint16_t *>(dst), d.outChansPerGroup,
+                     d.inChansPerGroup, nBlocks, total);
+  return hipGetLastError();
+}
+
+hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
+                           const void *in, const void *weightsPacked,
+                           const void *bias, void *out, hipStream_t stream) {
+  if (!pointwiseTakes(d, inType, outType))
+    return hipErrorInvalidValue;
+  PwArgs a;
+  a.d = d;
+  a.M = uint32_t(uint64_t(d.batch) * d.pixels);
+  a.mTiles = 0; // set for the tile height of the kernel that runs
+  a.nTiles = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
+  a.nBlocks = a.nTiles * 2;
+  a.inBytes = uint32_t(uint64_t(a.M) * d.groups * d.inChansPerGroup * 2);
+  a.wBytes = uint32_t(pointwisePackedElems(d) * 2);
+  if (outType == kHalf)
+    return runSlices<__half>(a, in, weightsPacked, bias, out, stream);
+  return runSlices<float>(a, in, weightsPacked, bias, out, stream);
+}
+
+} // namespace mxk

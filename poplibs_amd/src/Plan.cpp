@@ -298,6 +298,26 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
     plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;
     plan.weightPackedElems = p.numConvGroups * plan.coPadded * plan.kPadded;
+    // A pointwise convolution with few input channels is bound by HBM, not
+    // by the matrix cores: unless the big tile was asked for explicitly, the
+    // streaming kernel of small workgroups takes it.
+    mxk::PointwiseDesc &pw = plan.pointwise;
+    pw.batch = g.batch, pw.pixels = s.outH * s.outW;
+    pw.groups = g.groups, pw.inChansPerGroup = g.inChansPerGroup;
+    pw.outChansPerGroup = g.outChansPerGroup;
+    const bool unitWindow =
+        s.kH == 1 && s.kW == 1 && s.strideH == 1 && s.strideW == 1 &&
+        s.padH == 0 && s.padW == 0 && s.loH == 0 && s.loW == 0 &&
+        s.hiH == s.inH && s.hiW == s.inW && s.outH == s.inH &&
+        s.outW == s.inW;
+    plan.pointwiseOn =
+        unitWindow && pc.kernel != "igemm" && !pc.blockM && !pc.blockN &&
+        !pc.blockK &&
+        mxk::pointwiseTakes(pw, halfIn ? mxk::kHalf : mxk::kQuarter,
+                            params.outputType == poplar::HALF ? mxk::kHalf
+                                                              : mxk::kFloat);
+    if (plan.pointwiseOn)
+      plan.weightPackedElems = mxk::pointwisePackedElems(pw);
   } else if (chosen == Kernel::DEPTHWISE) {
     mxk::DepthwiseDesc &d = plan.depthwise;
     d.batch = uint32_t(p.batchSize);
@@ -344,7 +364,8 @@ std::string mxconv_plan::describe() const {
   case Kernel::IGEMM:
     os << "implicit GEMM (MFMA, "
        << (params.inputType == poplar::QUARTER ? "fp8" : "fp16")
-       << " operands, fp32 accumulate)";
+       << " operands, fp32 accumulate)"
+       << (pointwiseOn ? ", pointwise streaming variant" : "");
     break;
   case Kernel::DEPTHWISE:
     os << (depthwise.dense3x3
@@ -366,11 +387,21 @@ std::string mxconv_plan::describe() const {
     os << "        gemm M x N x K             " << m << " x "
        << g.outChansPerGroup << " x " << k << " (x " << g.groups
        << " groups)\n";
-    os << "        block M x N x K            " << g.blockM << " x " << g.blockN
-       << " x " << g.blockK << "\n";
-    os << "        workgroups                 " << tiles << "\n";
-    os << "        packed weights             [G=" << g.groups << "]["
-       << coPadded << "][" << kPadded << "]\n";
+    if (pointwiseOn) {
+      const std::size_t nTiles = (g.outChansPerGroup + 63) / 64;
+      os << "        block M x N x K            64 x 64 x " << k << "\n";
+      os << "        workgroups                 "
+         << (m + 63) / 64 * nTiles * g.groups << "\n";
+      os << "        packed weights             [G=" << g.groups << "]["
+         << nTiles * 2 << " blocks of 32][" << k / 16
+         << " slices of 16][64 lanes][8]\n";
+    } else {
+      os << "        block M x N x K            " << g.blockM << " x "
+         << g.blockN << " x " << g.blockK << "\n";
+      os << "        workgroups                 " << tiles << "\n";
+      os << "        packed weights             [G=" << g.groups << "]["
+         << coPadded << "][" << kPadded << "]\n";
+    }
   } else if (kernel == Kernel::DEPTHWISE) {
     const auto &d = depthwise;
     os << "        channels                   " << d.channels << "\n";

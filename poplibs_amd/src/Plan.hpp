@@ -31,6 +31,11 @@ struct mxconv_plan {
 
   mxk::GenericDesc generic{};     // always valid: describes `canonical`
   mxk::IgemmDesc igemm{};         // valid when kernel == IGEMM
+  // kernel == IGEMM and the streaming small-workgroup kernel serves it (1x1,
+  // stride 1, unpadded, few input channels): its descriptor; the packed
+  // weights then have its layout.
+  bool pointwiseOn = false;
+  mxk::PointwiseDesc pointwise{};
   mxk::DepthwiseDesc depthwise{}; // valid when kernel == DEPTHWISE
 
   // Packed weights of the matrix-core kernel: [G][coPadded][kPadded].

@@ -89,6 +89,35 @@ def test_igemm_blockN_override_and_amp_method(oracle):
     _run(oracle, p, 3, 1e-3, "implicit GEMM", options=opts, wscale=0.1)
 
 
+# 1x1, stride 1, unpadded, 128 / 256 / 512 input channels per group: the
+# streaming kernel of small workgroups.  Ragged pixel counts and channel
+# counts against its 64 x 64 tile, groups, 0-D to 2-D fields.
+POINTWISE_CASES = [
+    dict(batch=2, field=(56, 56), kernel=(1, 1), ci=256, co=64),
+    dict(batch=3, field=(7, 11), kernel=(1, 1), ci=128, co=40),
+    dict(batch=1, field=(5, 9), kernel=(1, 1), ci=512, co=136, groups=2),
+    dict(batch=70, field=(), kernel=(), ci=128, co=96),
+    dict(batch=2, field=(33,), kernel=(1,), ci=256, co=8),
+]
+
+
+@pytest.mark.parametrize("kw", POINTWISE_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_pointwise_matches_oracle(oracle, kw, out_type):
+    p = make_params(pa.HALF, out_type, **kw)
+    plan = pa.Plan(p)
+    assert "pointwise streaming variant" in plan.describe(), plan.describe()
+    _run(oracle, p, 8, 1e-3, "implicit GEMM", wscale=0.1)
+
+
+def test_pointwise_pm1_exact_and_big_tile_on_request(oracle):
+    p = make_params(pa.HALF, pa.FLOAT, **POINTWISE_CASES[1])
+    _run(oracle, p, 9, 0, "implicit GEMM", dist="pm1")
+    opts = {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'}
+    assert "pointwise" not in pa.Plan(p, opts).describe()
+    _run(oracle, p, 9, 0, "implicit GEMM", dist="pm1", options=opts)
+
+
 DW_CASES = [
     # BASELINE config 4 shape (3x3 s2 p1, C=96, 112x112), reduced batch
     dict(batch=2, field=(112, 112), kernel=(3, 3), groups=96, stride=2, pad=1),
