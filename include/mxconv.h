@@ -130,6 +130,13 @@ mxconv_status mxconv_params_validate(const mxconv_params *p);
 mxconv_status mxconv_params_canonicalize(const mxconv_params *p,
                                          mxconv_params *canonical);
 
+/* getGradientParams (lib/poplin/ConvUtil.cpp:728-795): the convolution that
+ * turns the gradient w.r.t. the forward output into the gradient w.r.t. the
+ * forward input, given the weights of mxconv_weights_transpose_chans_flip_xy.
+ * The result is canonical. */
+mxconv_status mxconv_get_gradient_params(const mxconv_params *p,
+                                         mxconv_params *gradient);
+
 /* isZeroConvolution (lib/poplin/ConvUtilInternal.cpp:24-38); canonicalizes
  * first, as CanonicalConvParams does. */
 mxconv_status mxconv_params_is_zero_convolution(const mxconv_params *p,
@@ -279,6 +286,17 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
                                  uint8_t weights_metadata, const void *bias,
                                  void *out, void *workspace,
                                  size_t workspace_bytes, mxconv_stream stream);
+
+/* poplin::weightsTransposeChansFlipXY (include/poplin/Convolution.hpp:407-412,
+ * lib/poplin/Convolution.cpp:3262-3388) on device tensors in the external
+ * layout: weights_in [G][Co][Ci][kernel...] -> weights_out
+ * [G][Ci][Co][kernel...] with every spatial axis reversed.  `p` are the
+ * FORWARD parameters (they give G, Co, Ci, the kernel shape and the element
+ * type).  The two buffers must not overlap. */
+mxconv_status mxconv_weights_transpose_chans_flip_xy(const mxconv_params *p,
+                                                     const void *weights_in,
+                                                     void *weights_out,
+                                                     mxconv_stream stream);
 
 /* poplin::addBias (lib/poplin/Convolution.cpp:3637-3648) on a channels-last
  * tensor of `outer_elems` x `channels` elements of `type`. */

@@ -40,6 +40,12 @@ def lib():
             + [pu, pu, pu, pu, pu, pu, pb]       # kernel + transform
             + [pu, pu, pu, pu, pu]               # output transform
             + [u, u, u, u, pd, pd, pd, pd, ctypes.c_size_t, ctypes.c_int])
+        L.oracle_convolution_backward.restype = ctypes.c_int
+        L.oracle_convolution_backward.argtypes = (
+            [u, pu, pu, pu, pu, pu, pu, pb]      # input field + transform
+            + [pu, pu, pu, pu, pu, pu, pb]       # kernel + transform
+            + [pu, pu, pu, pu, pu]               # output transform
+            + [u, u, u, u, pd, pd, pd, ctypes.c_size_t, ctypes.c_int])
         L.oracle_output_field_size.restype = u
         L.oracle_output_field_size.argtypes = [u] * 17
         L.oracle_fp8_decode.restype = ctypes.c_double
@@ -124,6 +130,46 @@ def convolution(p, acts, weights, biases=None, threads=1):
         out.size, int(threads))
     if rc != 0:
         raise RuntimeError(f"oracle_convolution failed with code {rc}")
+    return out
+
+
+def convolution_backward(p, deltas, weights, threads=1):
+    """Gradient of the forward convolution ``p`` with respect to its input.
+
+    ``p`` describes the FORWARD pass.  ``deltas`` has the shape of the forward
+    output [B][G*Co][outField...], ``weights`` are the forward weights
+    [G][Co][Ci][kernel...]; the result has the shape of the forward input
+    [B][G*Ci][field...], dtype float64.
+    """
+    L = lib()
+    nd = len(p.inputFieldShape)
+    G, Ci, Co, B = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                    p.outputChannelsPerConvGroup, p.batchSize)
+    deltas = np.ascontiguousarray(deltas, dtype=np.float64)
+    weights = np.ascontiguousarray(weights, dtype=np.float64)
+    assert deltas.shape == (B, G * Co, *output_field_shape(p)), deltas.shape
+    assert weights.shape == (G, Co, Ci, *p.kernelShape), weights.shape
+    out = np.empty((B, G * Ci, *p.inputFieldShape), dtype=np.float64)
+    it, kt, ot = p.inputTransform, p.kernelTransform, p.outputTransform
+    pd = ctypes.POINTER(ctypes.c_double)
+    spare = np.zeros(1)
+
+    def ptr(a):
+        return (a if a.size else spare).ctypes.data_as(pd)
+
+    rc = L.oracle_convolution_backward(
+        nd, _uarr(p.inputFieldShape), _uarr(it.truncationLower),
+        _uarr(it.truncationUpper), _uarr(it.dilation), _uarr(it.paddingLower),
+        _uarr(it.paddingUpper), _barr(it.flip),
+        _uarr(p.kernelShape), _uarr(kt.truncationLower),
+        _uarr(kt.truncationUpper), _uarr(kt.dilation), _uarr(kt.paddingLower),
+        _uarr(kt.paddingUpper), _barr(kt.flip),
+        _uarr(ot.truncationLower), _uarr(ot.truncationUpper), _uarr(ot.stride),
+        _uarr(ot.paddingLower), _uarr(ot.paddingUpper),
+        B, G, Ci, Co, ptr(deltas), ptr(weights), ptr(out), out.size,
+        int(threads))
+    if rc != 0:
+        raise RuntimeError(f"oracle_convolution_backward failed with code {rc}")
     return out
 
 

@@ -351,6 +351,164 @@ int oracle_convolution(
   return 0;
 }
 
+/*
+ * lib/poplibs_test/Convolution.cpp:577-722: the gradient with respect to the
+ * forward pass's input.  All parameters describe the FORWARD convolution.
+ *   deltas_in   [batch][groups*out_chans_per_group][prod(forward output field)]
+ *   kernel      [groups][out_chans_per_group][in_chans_per_group][prod(kernel)]
+ *   deltas_out  [batch][groups*in_chans_per_group][prod(fwd_input_field_size)]
+ * The reference scatters every (output element, kernel element) product into
+ * the padded forward input and then undoes the input transform.  `threads` > 1
+ * distributes (group, batch) pairs, which touch disjoint rows of the scatter
+ * target; within a row the order of additions is the reference's (oc, oe, ke
+ * ascending).  Returns 0, or -1 size mismatch, -2 rank, -3 allocation.
+ */
+int oracle_convolution_backward(
+    unsigned num_field_dims, const unsigned *fwd_input_field_size,
+    const unsigned *truncation_lower, const unsigned *truncation_upper,
+    const unsigned *input_dilation, const unsigned *padding_lower,
+    const unsigned *padding_upper, const unsigned char *flip_input,
+    const unsigned *kernel_size, const unsigned *kernel_truncation_lower,
+    const unsigned *kernel_truncation_upper, const unsigned *kernel_dilation,
+    const unsigned *kernel_padding_lower, const unsigned *kernel_padding_upper,
+    const unsigned char *flip_kernel, const unsigned *output_truncation_lower,
+    const unsigned *output_truncation_upper, const unsigned *stride,
+    const unsigned *output_padding_lower, const unsigned *output_padding_upper,
+    unsigned batch_size, unsigned num_conv_groups, unsigned in_chans_per_group,
+    unsigned out_chans_per_group, const double *deltas_in, const double *kernel,
+    double *deltas_out, size_t deltas_out_elems, int threads) {
+  const unsigned n = num_field_dims;
+  if (n > ORACLE_MAX_DIMS)
+    return -2;
+  const unsigned fwd_in_chans = num_conv_groups * in_chans_per_group;
+  const unsigned fwd_out_chans = num_conv_groups * out_chans_per_group;
+
+  /* :620-626 */
+  unsigned fwd_output_field_size[ORACLE_MAX_DIMS];
+  for (unsigned d = 0; d != n; ++d)
+    fwd_output_field_size[d] = oracle_output_field_size(
+        fwd_input_field_size[d], kernel_size[d], truncation_lower[d],
+        truncation_upper[d], input_dilation[d], padding_lower[d],
+        padding_upper[d], kernel_truncation_lower[d], kernel_truncation_upper[d],
+        kernel_dilation[d], kernel_padding_lower[d], kernel_padding_upper[d],
+        output_truncation_lower[d], output_truncation_upper[d], stride[d],
+        output_padding_lower[d], output_padding_upper[d]);
+
+  /* :643-647 */
+  unsigned padded_kernel_size[ORACLE_MAX_DIMS];
+  double *padded_kernel = truncate_dilate_pad_flip(
+      kernel, (size_t)num_conv_groups * out_chans_per_group * in_chans_per_group,
+      n, kernel_size, kernel_truncation_lower, kernel_truncation_upper,
+      kernel_dilation, kernel_padding_lower, kernel_padding_upper, flip_kernel,
+      padded_kernel_size);
+  if (!padded_kernel)
+    return -3;
+
+  /* :649-680: the deltas are padded by what the forward pass truncated from
+   * its output, plus the rows a stride > 1 never reached. */
+  unsigned fwd_padded_in_size[ORACLE_MAX_DIMS], fwd_conv_out_size[ORACLE_MAX_DIMS];
+  unsigned deltas_in_padding_upper[ORACLE_MAX_DIMS];
+  for (unsigned d = 0; d != n; ++d) {
+    fwd_padded_in_size[d] =
+        transformed_size(fwd_input_field_size[d], truncation_lower[d],
+                         truncation_upper[d], input_dilation[d],
+                         padding_lower[d], padding_upper[d]);
+    fwd_conv_out_size[d] = fwd_padded_in_size[d] - padded_kernel_size[d] + 1;
+    const unsigned truncated = fwd_conv_out_size[d] - (output_truncation_lower[d] +
+                                                       output_truncation_upper[d]);
+    if (output_padding_lower[d] + (truncated + stride[d] - 1) / stride[d] +
+            output_padding_upper[d] !=
+        fwd_output_field_size[d]) {
+      free(padded_kernel);
+      return -1;
+    }
+    const unsigned striding_ignored =
+        truncated == 0 ? 0 : (truncated - 1) % stride[d];
+    deltas_in_padding_upper[d] = output_truncation_upper[d] + striding_ignored;
+  }
+  /* :681-685 */
+  unsigned char no_flipping[ORACLE_MAX_DIMS] = {0};
+  unsigned padded_deltas_size[ORACLE_MAX_DIMS];
+  double *padded_deltas = truncate_dilate_pad_flip(
+      deltas_in, (size_t)batch_size * fwd_out_chans, n, fwd_output_field_size,
+      output_padding_lower, output_padding_upper, stride,
+      output_truncation_lower, deltas_in_padding_upper, no_flipping,
+      padded_deltas_size);
+  if (!padded_deltas) {
+    free(padded_kernel);
+    return -3;
+  }
+  for (unsigned d = 0; d != n; ++d)
+    if (padded_deltas_size[d] != fwd_conv_out_size[d]) {
+      free(padded_kernel);
+      free(padded_deltas);
+      return -1;
+    }
+
+  /* :693-719 */
+  const size_t fwd_conv_out_elems = product(fwd_conv_out_size, n);
+  const size_t fwd_padded_in_elems = product(fwd_padded_in_size, n);
+  const size_t padded_kernel_elems = product(padded_kernel_size, n);
+  double *conv_out = (double *)calloc(
+      (size_t)batch_size * fwd_in_chans * fwd_padded_in_elems + 1, sizeof(double));
+  if (!conv_out) {
+    free(padded_kernel);
+    free(padded_deltas);
+    return -3;
+  }
+  const long pairs = (long)num_conv_groups * (long)batch_size;
+  if (threads < 1)
+    threads = 1;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+  for (long pair = 0; pair < pairs; ++pair) {
+    const unsigned b = (unsigned)(pair % batch_size);
+    const unsigned gc = (unsigned)(pair / batch_size);
+    for (unsigned oc = 0; oc != out_chans_per_group; ++oc) {
+      const unsigned oc_act = gc * out_chans_per_group + oc;
+      const double *delta_row =
+          padded_deltas + ((size_t)b * fwd_out_chans + oc_act) * fwd_conv_out_elems;
+      const double *kernel_row =
+          padded_kernel + ((size_t)gc * out_chans_per_group + oc) *
+                              in_chans_per_group * padded_kernel_elems;
+      for (size_t oe = 0; oe != fwd_conv_out_elems; ++oe) {
+        unsigned output_indices[ORACLE_MAX_DIMS];
+        unflatten_index(fwd_conv_out_size, n, oe, output_indices);
+        for (size_t ke = 0; ke != padded_kernel_elems; ++ke) {
+          unsigned kernel_indices[ORACLE_MAX_DIMS];
+          unsigned input_indices[ORACLE_MAX_DIMS];
+          unflatten_index(padded_kernel_size, n, ke, kernel_indices);
+          if (get_input_indices(n, fwd_padded_in_size, padded_kernel_size,
+                                output_indices, kernel_indices, input_indices)) {
+            const size_t ie = flatten_index(fwd_padded_in_size, n, input_indices);
+            for (unsigned ic = 0; ic != in_chans_per_group; ++ic) {
+              const unsigned ic_act = gc * in_chans_per_group + ic;
+              conv_out[((size_t)b * fwd_in_chans + ic_act) * fwd_padded_in_elems +
+                       ie] +=
+                  kernel_row[(size_t)ic * padded_kernel_elems + ke] * delta_row[oe];
+            }
+          }
+        }
+      }
+    }
+  }
+
+  /* :720-722 */
+  unsigned size[ORACLE_MAX_DIMS];
+  int rc = truncate_dilate_pad_flip_inverse(
+      conv_out, (size_t)batch_size * fwd_in_chans, n, fwd_padded_in_size,
+      truncation_lower, truncation_upper, input_dilation, padding_lower,
+      padding_upper, flip_input, deltas_out, deltas_out_elems, size);
+  free(conv_out);
+  free(padded_kernel);
+  free(padded_deltas);
+  if (rc != 0)
+    return -1;
+  for (unsigned d = 0; d != n; ++d)
+    if (size[d] != fwd_input_field_size[d])
+      return -1;
+  return 0;
+}
+
 /* ------------------------------------------------------------------------ */
 /* FP8 codec of this build (not Graphcore's): OCP 8-bit floats.
  *   format 1 = E4M3FN: bias 7, no infinities, S.1111.111 is NaN, max 448

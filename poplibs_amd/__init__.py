@@ -8,5 +8,6 @@ a GPU raises.
 """
 from .capi import (  # noqa: F401
     FLOAT, HALF, QUARTER, ConvParams, InputTransform, MxconvError,
-    OutputTransform, Plan, Status, add_bias, build_library, lib, library_path,
-    quarter_metadata, validate_options)
+    OutputTransform, Plan, Status, add_bias, build_library, getGradientParams,
+    lib, library_path, quarter_metadata, validate_options,
+    weightsTransposeChansFlipXY)

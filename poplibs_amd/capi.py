@@ -116,6 +116,9 @@ def lib():
                                        c_uint64, c_uint64, c_uint64]),
         "mxconv_params_validate": (c_int, [P]),
         "mxconv_params_canonicalize": (c_int, [P, P]),
+        "mxconv_get_gradient_params": (c_int, [P, P]),
+        "mxconv_weights_transpose_chans_flip_xy":
+            (c_int, [P, c_void_p, c_void_p, c_void_p]),
         "mxconv_params_is_zero_convolution": (c_int, [P, POINTER(c_int)]),
         "mxconv_params_size": (c_int, [P, c_int32, c_uint32,
                                        POINTER(c_uint64)]),
@@ -342,6 +345,12 @@ class ConvParams:
                                                 byref(out)))
         return ConvParams.from_c(out)
 
+    def getGradientParams(self):
+        """poplin::getGradientParams(params), lib/poplin/ConvUtil.cpp:728-795."""
+        out = CParams()
+        _check(lib().mxconv_get_gradient_params(byref(self.to_c()), byref(out)))
+        return ConvParams.from_c(out)
+
     def _size(self, query, dim):
         v = c_uint64()
         _check(lib().mxconv_params_size(byref(self.to_c()), query, dim,
@@ -539,6 +548,18 @@ class Plan:
                                         weights_packed, weights_metadata, bias,
                                         out, workspace, workspace_bytes,
                                         stream))
+
+
+def getGradientParams(params):
+    """poplin::getGradientParams (lib/poplin/ConvUtil.cpp:728-795)."""
+    return params.getGradientParams()
+
+
+def weightsTransposeChansFlipXY(params, weights_in, weights_out, stream=0):
+    """poplin::weightsTransposeChansFlipXY on device pointers in the external
+    layout; ``params`` are the forward parameters."""
+    _check(lib().mxconv_weights_transpose_chans_flip_xy(
+        byref(params.to_c()), weights_in, weights_out, stream))
 
 
 def add_bias(type_id, acts, bias, outer_elems, channels, stream=0):

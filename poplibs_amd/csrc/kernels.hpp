@@ -52,6 +52,15 @@ hipError_t launchGeneric(const GenericDesc &d, int inType, int outType,
 hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
                           const int perm[4], int elemBytes, hipStream_t stream);
 
+/// dst[g][ci][co][k...] = src[g][co][ci][flipped k...]: channels transposed,
+/// every one of the numDims (<= kMaxDims) kernel axes reversed.
+hipError_t launchWeightsTransposeChansFlipXY(const void *src, void *dst,
+                                             uint64_t groups, uint64_t co,
+                                             uint64_t ci, uint32_t numDims,
+                                             const uint32_t *kernelShape,
+                                             int elemBytes,
+                                             hipStream_t stream);
+
 /// Weights [G][Co][Ci][taps] -> [G][coPadded][kPadded] with k = tap * Ci + ci,
 /// zero-filled beyond Co and beyond taps * Ci: the B operand of the
 /// matrix-core kernel, K contiguous.

@@ -47,6 +47,37 @@ __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
   dst[tid] = v;
 }
 
+struct FlipArgs {
+  uint64_t co, ci, taps, total;
+  uint32_t numDims;
+  uint32_t shape[kMaxDims];
+};
+
+template <class T>
+__global__ __launch_bounds__(256) void transposeChansFlipKernel(
+    FlipArgs a, const T *__restrict__ src, T *__restrict__ dst) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= a.total)
+    return;
+  // tid indexes dst [g][ci][co][k]
+  uint64_t r = tid;
+  const uint64_t k = r % a.taps;
+  r /= a.taps;
+  const uint64_t co = r % a.co;
+  r /= a.co;
+  const uint64_t ci = r % a.ci;
+  const uint64_t g = r / a.ci;
+  // reverse every axis of the row-major tap index
+  uint64_t rem = k, flipped = 0, stride = 1;
+  for (int d = int(a.numDims) - 1; d >= 0; --d) {
+    const uint64_t x = rem % a.shape[d];
+    rem /= a.shape[d];
+    flipped += (a.shape[d] - 1 - x) * stride;
+    stride *= a.shape[d];
+  }
+  dst[tid] = src[((g * a.co + co) * a.ci + ci) * a.taps + flipped];
+}
+
 template <class T>
 __global__ __launch_bounds__(256) void addBiasKernel(T *acts,
                                                      const T *__restrict__ bias,
@@ -124,6 +155,44 @@ hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                        static_cast<const uint16_t *>(src),
                        static_cast<uint16_t *>(dst), co, ci, taps, coPadded,
                        kPadded, total);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launchWeightsTransposeChansFlipXY(const void *src, void *dst,
+                                             uint64_t groups, uint64_t co,
+                                             uint64_t ci, uint32_t numDims,
+                                             const uint32_t *kernelShape,
+                                             int elemBytes,
+                                             hipStream_t stream) {
+  if (numDims > uint32_t(kMaxDims))
+    return hipErrorInvalidValue;
+  FlipArgs a{};
+  a.co = co, a.ci = ci, a.taps = 1, a.numDims = numDims;
+  for (uint32_t d = 0; d != numDims; ++d) {
+    a.shape[d] = kernelShape[d];
+    a.taps *= kernelShape[d];
+  }
+  a.total = groups * co * ci * a.taps;
+  if (a.total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (a.total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  if (elemBytes == 1)
+    hipLaunchKernelGGL(transposeChansFlipKernel<uint8_t>, grid, block, 0,
+                       stream, a, static_cast<const uint8_t *>(src),
+                       static_cast<uint8_t *>(dst));
+  else if (elemBytes == 2)
+    hipLaunchKernelGGL(transposeChansFlipKernel<uint16_t>, grid, block, 0,
+                       stream, a, static_cast<const uint16_t *>(src),
+                       static_cast<uint16_t *>(dst));
+  else if (elemBytes == 4)
+    hipLaunchKernelGGL(transposeChansFlipKernel<uint32_t>, grid, block, 0,
+                       stream, a, static_cast<const uint32_t *>(src),
+                       static_cast<uint32_t *>(dst));
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

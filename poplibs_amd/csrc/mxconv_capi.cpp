@@ -217,6 +217,16 @@ mxconv_status mxconv_params_canonicalize(const mxconv_params *p,
   });
 }
 
+mxconv_status mxconv_get_gradient_params(const mxconv_params *p,
+                                         mxconv_params *gradient) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(gradient);
+  return guarded([&] {
+    poplin::getGradientParams(poplin::ConvParams::fromC(*p)).toC(*gradient);
+    return MXCONV_OK;
+  });
+}
+
 mxconv_status mxconv_params_is_zero_convolution(const mxconv_params *p,
                                                 int *is_zero) {
   REQUIRE_ARG(p);
@@ -595,6 +605,40 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
   return forward(plan, in, weights_packed, bias, out, workspace,
                  workspace_bytes, quarterInfo(in_metadata, weights_metadata),
                  stream);
+}
+
+mxconv_status mxconv_weights_transpose_chans_flip_xy(const mxconv_params *p,
+                                                     const void *weights_in,
+                                                     void *weights_out,
+                                                     mxconv_stream stream) {
+  REQUIRE_ARG(p);
+  lastError.clear();
+  poplin::ConvParams params;
+  const mxconv_status st = guarded([&] {
+    params = poplin::ConvParams::fromC(*p);
+    params.validate();
+    return MXCONV_OK;
+  });
+  if (st != MXCONV_OK)
+    return st;
+  uint64_t elems = params.numConvGroups * params.outputChannelsPerConvGroup *
+                   params.inputChannelsPerConvGroup;
+  uint32_t shape[MXCONV_MAX_FIELD_DIMS] = {};
+  for (std::size_t d = 0; d != params.kernelShape.size(); ++d) {
+    shape[d] = uint32_t(params.kernelShape[d]);
+    elems *= params.kernelShape[d];
+  }
+  if (elems == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(weights_in);
+  REQUIRE_ARG(weights_out);
+  return hipStatus(
+      mxk::launchWeightsTransposeChansFlipXY(
+          weights_in, weights_out, params.numConvGroups,
+          params.outputChannelsPerConvGroup, params.inputChannelsPerConvGroup,
+          uint32_t(params.kernelShape.size()), shape,
+          int(params.inputType.size()), reinterpret_cast<hipStream_t>(stream)),
+      "weight transposition");
 }
 
 mxconv_status mxconv_add_bias(int32_t type, void *acts_internal,

@@ -67,5 +67,12 @@ bool isZeroConvolution(const ConvParams &canonicalParams);
 /// (lib/poplin/ConvUtilInternal.cpp:40-76).
 ConvParams getZeroConv(const ConvParams &params);
 
+/// Parameters of the convolution that computes the gradient with respect
+/// to the forward pass's input from the gradient with respect to its output
+/// and the forward weights with channels transposed and every spatial axis
+/// flipped (weightsTransposeChansFlipXY); canonical
+/// (lib/poplin/ConvUtil.cpp:728-795).
+ConvParams getGradientParams(const ConvParams &params);
+
 } // namespace poplin
 #endif

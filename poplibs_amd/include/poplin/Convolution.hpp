@@ -114,8 +114,10 @@ DeviceTensor createConvOutput(const ConvParams &params,
 
 /// Convolve `in` with `weights`; returns the output tensor.  Tensors in
 /// External layout are converted on the device first.
-/// transposeAndFlipWeights (the backward-pass weight view) is not part of the
-/// forward path and raises poputil::poplibs_error when true.
+/// transposeAndFlipWeights: `weights` are the forward pass's
+/// [G][params.inChans][params.outChans][kernel...] in the external layout and
+/// are passed through weightsTransposeChansFlipXY first - the backward pass
+/// with params = getGradientParams(forward parameters).
 DeviceTensor convolution(const DeviceTensor &in, const DeviceTensor &weights,
                          const ConvParams &params,
                          bool transposeAndFlipWeights, Stream &prog,
@@ -127,6 +129,11 @@ void convolutionWithOutput(const DeviceTensor &in, const DeviceTensor &weights,
                            bool transposeAndFlipWeights, Stream &prog,
                            const poplar::OptionFlags &options = {},
                            PlanningCache *cache = nullptr);
+
+/// weightsOut[g][ci][co][k...] = weightsIn[g][co][ci][flipped k...], both in
+/// the external layout (include/poplin/Convolution.hpp:407-412 of PopLibs).
+void weightsTransposeChansFlipXY(const DeviceTensor &weightsIn,
+                                 const DeviceTensor &weightsOut, Stream &prog);
 
 /// acts[b][c][...] += biases[c].
 void addBias(const DeviceTensor &in, const DeviceTensor &biases, Stream &prog);

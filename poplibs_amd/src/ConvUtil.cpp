@@ -230,6 +230,58 @@ bool isZeroConvolution(const ConvParams &p) {
   return false;
 }
 
+ConvParams getGradientParams(const ConvParams &params) {
+  const ConvParams p = params.canonicalize();
+  const unsigned numFieldDims = unsigned(p.getNumFieldDims());
+  // A "valid" forward convolution is a "full" one going backwards: a valid
+  // one with (kernel size - 1) of padding, on top of what the forward pass
+  // truncated from its output.
+  auto inputPaddingLower = p.outputTransform.truncationLower;
+  auto inputPaddingUpper = p.outputTransform.truncationUpper;
+  for (unsigned d = 0; d != numFieldDims; ++d) {
+    const unsigned k = unsigned(p.getTransformedKernelSize(d));
+    inputPaddingLower[d] += k - 1;
+    inputPaddingUpper[d] += k - 1;
+  }
+  // The caller flips the weights in every spatial axis, which swaps the
+  // kernel's lower and upper truncation / padding.  An input flipped in the
+  // forward pass means an output flipped in the backward pass, i.e. input
+  // and kernel both flipped.
+  std::vector<bool> flipInput(numFieldDims, false);
+  std::vector<bool> flipKernel = p.kernelTransform.flip;
+  for (unsigned d = 0; d != numFieldDims; ++d)
+    if (p.inputTransform.flip[d]) {
+      flipKernel[d] = !flipKernel[d];
+      flipInput[d] = !flipInput[d];
+    }
+  ConvParams::InputTransform inputTransform;
+  inputTransform.truncationLower = p.outputTransform.paddingLower;
+  inputTransform.truncationUpper = p.outputTransform.paddingUpper;
+  inputTransform.dilation = p.outputTransform.stride;
+  inputTransform.paddingLower = inputPaddingLower;
+  inputTransform.paddingUpper = inputPaddingUpper;
+  inputTransform.flip = flipInput;
+  ConvParams::InputTransform kernelTransform;
+  kernelTransform.truncationLower = p.kernelTransform.truncationUpper;
+  kernelTransform.truncationUpper = p.kernelTransform.truncationLower;
+  kernelTransform.dilation = p.kernelTransform.dilation;
+  kernelTransform.paddingLower = p.kernelTransform.paddingUpper;
+  kernelTransform.paddingUpper = p.kernelTransform.paddingLower;
+  kernelTransform.flip = flipKernel;
+  ConvParams::OutputTransform outputTransform;
+  outputTransform.truncationLower = p.inputTransform.paddingLower;
+  outputTransform.truncationUpper = p.inputTransform.paddingUpper;
+  outputTransform.stride = p.inputTransform.dilation;
+  outputTransform.paddingLower = p.inputTransform.truncationLower;
+  outputTransform.paddingUpper = p.inputTransform.truncationUpper;
+  const ConvParams bwd(p.inputType, p.outputType, p.batchSize,
+                       p.getOutputFieldShape(), p.kernelShape,
+                       p.getNumOutputChansPerConvGroup(),
+                       p.getNumInputChansPerConvGroup(), p.getNumConvGroups(),
+                       inputTransform, kernelTransform, outputTransform);
+  return bwd.canonicalize();
+}
+
 ConvParams getZeroConv(const ConvParams &params) {
   // Truncate input and kernel to nothing, pad each back to one zero, convolve
   // to a single element, truncate it away and pad the output to full size.

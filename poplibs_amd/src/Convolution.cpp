@@ -6,6 +6,7 @@
 #include "poplar/exceptions.hpp"
 #include "poputil/exceptions.hpp"
 
+#include <algorithm>
 #include <hip/hip_runtime_api.h>
 
 #include <map>
@@ -310,13 +311,67 @@ void convolutionWithOutput(const DeviceTensor &in, const DeviceTensor &weights,
                            bool transposeAndFlipWeights, Stream &prog,
                            const poplar::OptionFlags &options,
                            PlanningCache *cache) {
-  if (transposeAndFlipWeights)
-    throw poputil::poplibs_error(
-        "transposeAndFlipWeights belongs to the backward pass, which this "
-        "build does not provide");
   auto plan = getPlan(params, options, cache);
-  verify(params, in, weights, &out);
-  run(*plan, params, in, weights, out, prog);
+  if (!transposeAndFlipWeights) {
+    verify(params, in, weights, &out);
+    run(*plan, params, in, weights, out, prog);
+    return;
+  }
+  // Backward pass: `weights` are the forward pass's,
+  // [G][params.inChans][params.outChans][kernel...]; transpose the channel
+  // axes and flip the spatial ones first (lib/poplin/Convolution.cpp:
+  // 3077-3086).
+  if (weights.layout() != DeviceTensor::Layout::External)
+    throw poputil::poplibs_error(
+        "transposeAndFlipWeights needs the weights in the external layout "
+        "(packed weights belong to the plan they were packed for)");
+  std::vector<std::size_t> fwdShape{params.numConvGroups,
+                                    params.inputChannelsPerConvGroup,
+                                    params.outputChannelsPerConvGroup};
+  fwdShape.insert(fwdShape.end(), params.kernelShape.begin(),
+                  params.kernelShape.end());
+  if (weights.shape() != fwdShape)
+    throw poputil::poplibs_error(
+        "Weights tensor shape does not match the convolution parameters "
+        "(expected the forward pass's [G][outChans][inChans][kernel...])");
+  std::vector<std::size_t> bwdShape = fwdShape;
+  std::swap(bwdShape[1], bwdShape[2]);
+  DeviceTensor flipped(weights.elementType(), bwdShape,
+                       DeviceTensor::Layout::External, weights.bytes());
+  flipped.metadata = weights.metadata;
+  weightsTransposeChansFlipXY(weights, flipped, prog);
+  verify(params, in, flipped, &out);
+  run(*plan, params, in, flipped, out, prog);
+  prog.synchronize(); // `flipped` is released on return
+}
+
+void weightsTransposeChansFlipXY(const DeviceTensor &weightsIn,
+                                 const DeviceTensor &weightsOut, Stream &prog) {
+  const auto &si = weightsIn.shape(), &so = weightsOut.shape();
+  if (si.size() < 3 || si.size() - 3 > MXCONV_MAX_FIELD_DIMS ||
+      so.size() != si.size() || so[0] != si[0] || so[1] != si[2] ||
+      so[2] != si[1] ||
+      !std::equal(si.begin() + 3, si.end(), so.begin() + 3))
+    throw poputil::poplibs_error(
+        "weightsTransposeChansFlipXY: weightsOut must be "
+        "[G][inChans][outChans][kernel...] for weightsIn "
+        "[G][outChans][inChans][kernel...]");
+  if (weightsIn.layout() != DeviceTensor::Layout::External ||
+      weightsOut.layout() != DeviceTensor::Layout::External ||
+      weightsIn.elementType() != weightsOut.elementType())
+    throw poputil::poplibs_error(
+        "weightsTransposeChansFlipXY: both tensors must be in the external "
+        "layout and share an element type");
+  // Forward parameters carrying just what the transposition needs.
+  ConvParams fwd(weightsIn.elementType(), 1,
+                 std::vector<std::size_t>(si.begin() + 3, si.end()),
+                 std::vector<std::size_t>(si.begin() + 3, si.end()), si[2],
+                 si[1], si[0]);
+  mxconv_params c;
+  fwd.toC(c);
+  check(mxconv_weights_transpose_chans_flip_xy(&c, weightsIn.data(),
+                                               weightsOut.data(),
+                                               streamOf(prog)));
 }
 
 DeviceTensor convolution(const DeviceTensor &in, const DeviceTensor &weights,

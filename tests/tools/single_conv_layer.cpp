@@ -1,11 +1,12 @@
-// single_conv_layer - command-line harness for one forward convolution.
+// single_conv_layer - command-line harness for one convolution layer: the
+// forward pass and the backward-data pass.
 //
-// Test infrastructure: it runs the convolution through the C++ poplin layer of
-// this build (hence through the C ABI and the gfx950 kernels) and compares the
-// result with the CPU oracle (oracle/conv_oracle.c), exactly as PopLibs'
+// Test infrastructure: it runs the convolutions through the C++ poplin layer
+// of this build (hence through the C ABI and the gfx950 kernels) and compares
+// the results with the CPU oracle (oracle/conv_oracle.c), exactly as PopLibs'
 // tools/single_conv_layer.cpp compares a device run with
-// poplibs_test::conv::convolution.  The forward-pass subset of that tool's
-// options is accepted under the same names (tools/single_conv_layer.cpp:
+// poplibs_test::conv::convolution / convolutionBackward.  The forward- and
+// backward-pass subset of that tool's options is accepted under the same names (tools/single_conv_layer.cpp:
 // 171-430); the same data modes, comparison rule and exit codes apply:
 //   * +-1 "Bernoulli" data with zero tolerance when the sums stay exactly
 //     representable, else uniform random data with tolerances
@@ -16,6 +17,7 @@
 #include "poplar/OptionFlags.hpp"
 #include "poplar/exceptions.hpp"
 #include "poplin/ConvParams.hpp"
+#include "poplin/ConvUtil.hpp"
 #include "poplin/Convolution.hpp"
 #include "poputil/exceptions.hpp"
 
@@ -45,6 +47,14 @@ int oracle_convolution(
     const unsigned *, const unsigned *, const unsigned *, unsigned, unsigned,
     unsigned, unsigned, const double *, const double *, const double *,
     double *, size_t, int);
+int oracle_convolution_backward(
+    unsigned, const unsigned *, const unsigned *, const unsigned *,
+    const unsigned *, const unsigned *, const unsigned *,
+    const unsigned char *, const unsigned *, const unsigned *,
+    const unsigned *, const unsigned *, const unsigned *, const unsigned *,
+    const unsigned char *, const unsigned *, const unsigned *,
+    const unsigned *, const unsigned *, const unsigned *, unsigned, unsigned,
+    unsigned, unsigned, const double *, const double *, double *, size_t, int);
 double oracle_fp8_decode(unsigned code, int format);
 unsigned oracle_fp8_encode(double x, int format);
 }
@@ -247,6 +257,7 @@ int main(int argc, char **argv) try {
       "output-truncation", "output-truncation-upper",
       "output-truncation-lower", "stride", "output-padding",
       "output-padding-upper", "output-padding-lower", "single-phase",
+      "inference-only", "bwd-plan-constraints",
       "plan-only", "inference-only", "tolerance", "absolute-tolerance",
       "batch-size", "conv-groups", "fwd-plan-constraints",
       "fwd-plan-constraints-file", "report-plan", "convolution-options",
@@ -269,9 +280,17 @@ int main(int argc, char **argv) try {
        {"input-channels", "output-channels", "field", "kernel-size"})
     if (!has(required))
       usage(std::string("the option '--") + required + "' is required");
-  const std::string phase = get("single-phase", "fwd");
-  if (phase != "fwd" && phase != "all")
-    usage("only the forward pass is provided (--single-phase fwd)");
+  // Passes (tools/single_conv_layer.cpp:723-735): forward and backward-data
+  // are provided; "all" runs both and says that the weight update is not.
+  const std::string phase = get("single-phase", "all");
+  if (phase != "fwd" && phase != "bwd" && phase != "all")
+    usage("--single-phase must be fwd, bwd or all (the weight-update pass is "
+          "not provided)");
+  const bool inferenceOnly = parseBool(get("inference-only", "false"));
+  const bool doFwdPass = phase == "fwd" || phase == "all";
+  const bool doBwdPass = !inferenceOnly && (phase == "bwd" || phase == "all");
+  if (phase == "all" && !inferenceOnly)
+    std::cout << "Weight-update pass not provided: running fwd and bwd\n";
 
   // ---- parameters (tools/single_conv_layer.cpp:768-790) -------------------
   const Shape field = parseShape(get("field"));
@@ -349,12 +368,32 @@ int main(int argc, char **argv) try {
   }
   poplin::convolutionValidateOptions(options);
 
+  // Backward pass = forward convolution of the output gradient with the
+  // gradient parameters and transposed, flipped weights
+  // (tools/single_conv_layer.cpp:793, 1064-1082).
+  const ConvParams bwdParams = poplin::getGradientParams(params);
+  poplar::OptionFlags bwdOptions = options;
+  if (has("bwd-plan-constraints"))
+    bwdOptions.set("planConstraints", get("bwd-plan-constraints"));
+  else if (has("fwd-plan-constraints"))
+    bwdOptions.set("planConstraints", "");
+  poplin::convolutionValidateOptions(bwdOptions);
   const auto flops = poplin::getFwdFlops(params);
-  std::cout << "Forward FLOPs: " << flops << "\n";
   poplin::PlanningCache cache;
-  if (parseBool(get("report-plan", "false")) || has("plan-only")) {
-    std::cout << "Forward plan:\n";
-    poplin::reportPlanInfo(std::cout, params, options, &cache);
+  const bool reportPlan = parseBool(get("report-plan", "false")) || has("plan-only");
+  if (doFwdPass) {
+    std::cout << "Forward FLOPs: " << flops << "\n";
+    if (reportPlan) {
+      std::cout << "Forward plan:\n";
+      poplin::reportPlanInfo(std::cout, params, options, &cache);
+    }
+  }
+  if (doBwdPass) {
+    std::cout << "Backward FLOPs: " << poplin::getFwdFlops(bwdParams) << "\n";
+    if (reportPlan) {
+      std::cout << "Backward plan:\n";
+      poplin::reportPlanInfo(std::cout, bwdParams, bwdOptions, &cache);
+    }
   }
   if (has("plan-only"))
     return 0;
@@ -425,9 +464,10 @@ int main(int argc, char **argv) try {
     }
   };
   std::vector<double> acts(inElems), weights(wElems),
-      biases(params.getNumOutputChans(), 0.0);
+      biases(params.getNumOutputChans(), 0.0), zDeltas(outElems);
   fill(acts, inputType, -2, 2);
   fill(weights, inputType, -1, 1);
+  fill(zDeltas, inputType, -3, 3);
   if (useBias)
     fill(biases, outputType == poplar::QUARTER ? poplar::HALF : outputType,
          uniformData ? -2 : -1, uniformData ? 6 : 1);
@@ -437,10 +477,13 @@ int main(int argc, char **argv) try {
       x = std::ldexp(x, inMeta.scale);
     for (auto &x : weights)
       x = std::ldexp(x, wMeta.scale);
+    for (auto &x : zDeltas)
+      x = std::ldexp(x, inMeta.scale);
   }
   const auto actBytes = encode(acts, inputType, inMeta);
   const auto weightBytes = encode(weights, inputType, wMeta);
   const auto biasBytes = encode(biases, outputType, {});
+  const auto zDeltaBytes = encode(zDeltas, inputType, inMeta);
 
   // ---- device run ----------------------------------------------------------
   poplin::Stream prog;
@@ -451,7 +494,7 @@ int main(int argc, char **argv) try {
   std::vector<uint8_t> result(outElems * outputType.size());
   std::vector<uint8_t> first;
   const bool ignoreData = has("ignore-data");
-  const unsigned runs = 1 + determinismChecks;
+  const unsigned runs = doFwdPass ? 1 + determinismChecks : 0;
   for (unsigned run = 0; run != runs; ++run) {
     if (!ignoreData) {
       poplin::writeTensor(in, actBytes.data(), prog, params, options, &cache);
@@ -476,7 +519,34 @@ int main(int argc, char **argv) try {
       return 1;
     }
   }
-  if (has("timing-runs")) {
+  // Backward pass: the forward weights, in the external layout, go in with
+  // transposeAndFlipWeights = true.
+  std::vector<uint8_t> bwdResult(inElems * outputType.size());
+  if (doBwdPass) {
+    std::vector<size_t> wShape{params.numConvGroups,
+                               params.outputChannelsPerConvGroup,
+                               params.inputChannelsPerConvGroup};
+    wShape.insert(wShape.end(), kernelShape.begin(), kernelShape.end());
+    poplin::DeviceTensor fwdWeights(inputType, wShape,
+                                    poplin::DeviceTensor::Layout::External,
+                                    std::max<size_t>(weightBytes.size(), 1));
+    fwdWeights.metadata = wMeta;
+    auto deltas = poplin::createInput(bwdParams, bwdOptions, &cache);
+    deltas.metadata = inMeta;
+    if (!ignoreData) {
+      poplin::writeTensor(fwdWeights, weightBytes.data(), prog, params, options,
+                          &cache);
+      poplin::writeTensor(deltas, zDeltaBytes.data(), prog, bwdParams,
+                          bwdOptions, &cache);
+    }
+    auto prevDeltas = poplin::convolution(deltas, fwdWeights, bwdParams, true,
+                                          prog, bwdOptions, &cache);
+    if (!ignoreData)
+      poplin::readTensor(prevDeltas, bwdResult.data(), prog, bwdParams,
+                         bwdOptions, &cache);
+    prog.synchronize();
+  }
+  if (has("timing-runs") && doFwdPass) {
     const unsigned reps = unsigned(std::stoul(get("timing-runs")));
     auto out = poplin::createConvOutput(params, options, &cache);
     poplin::convolutionWithOutput(in, w, out, params, false, prog, options,
@@ -526,48 +596,79 @@ int main(int argc, char **argv) try {
   auto fi = flagsU(inT.flip), fk = flagsU(kT.flip);
   fi.push_back(0);
   fk.push_back(0);
-  std::vector<double> expected(outElems + 1);
   acts.push_back(0);
   weights.push_back(0);
-  const int rc = oracle_convolution(
-      unsigned(n), fs.data(), itl.data(), itu.data(), idl.data(), ipl.data(),
-      ipu.data(), fi.data(), ks.data(), ktl.data(), ktu.data(), kdl.data(),
-      kpl.data(), kpu.data(), fk.data(), otl.data(), otu.data(), ost.data(),
-      opl.data(), opu.data(), unsigned(params.batchSize),
-      unsigned(params.numConvGroups),
-      unsigned(params.inputChannelsPerConvGroup),
-      unsigned(params.outputChannelsPerConvGroup), acts.data(), weights.data(),
-      biases.data(), expected.data(), outElems, 8);
-  if (rc != 0) {
-    std::cerr << "host model failed with code " << rc << "\n";
-    return 1;
-  }
-  expected.resize(outElems);
-  // The host model's result is rounded to the output type before comparing,
-  // as the reference does when it copies the model output into a typed buffer.
-  encode(expected, outputType, {});
-  const auto actual = decode(result, outputType);
-  unsigned mismatches = 0;
-  double num = 0, den = 0;
-  for (size_t i = 0; i != outElems; ++i) {
-    const double a = actual[i], e = expected[i];
-    num += (a - e) * (a - e);
-    den += e * e;
-    const bool bothNan = std::isnan(a) && std::isnan(e);
-    if ((!bothNan && (std::isnan(a) || std::isnan(e))) ||
-        (!isClose(a, e, relTol) && std::fabs(e - a) > absTol)) {
-      if (mismatches++ < 20)
-        std::cerr << "mismatch on element fwd[" << i << "]: expected=" << e
-                  << " actual=" << a << " (abs=" << a - e
-                  << ", rel=" << (a / e - 1.0) * 100.0 << "%)\n";
+  zDeltas.push_back(0);
+  // checkIsClose element by element, plus the relative L2 error.
+  auto compare = [&](const char *name, const std::vector<uint8_t> &bytes,
+                     std::vector<double> &expected, size_t count) {
+    expected.resize(count);
+    // The host model's result is rounded to the output type before
+    // comparing, as the reference does when it copies the model output into
+    // a typed buffer.
+    encode(expected, outputType, {});
+    const auto actual = decode(bytes, outputType);
+    unsigned mismatches = 0;
+    double num = 0, den = 0;
+    for (size_t i = 0; i != count; ++i) {
+      const double a = actual[i], e = expected[i];
+      num += (a - e) * (a - e);
+      den += e * e;
+      const bool bothNan = std::isnan(a) && std::isnan(e);
+      if ((!bothNan && (std::isnan(a) || std::isnan(e))) ||
+          (!isClose(a, e, relTol) && std::fabs(e - a) > absTol)) {
+        if (mismatches++ < 20)
+          std::cerr << "mismatch on element " << name << "[" << i
+                    << "]: expected=" << e << " actual=" << a
+                    << " (abs=" << a - e << ", rel=" << (a / e - 1.0) * 100.0
+                    << "%)\n";
+      }
     }
+    std::cout << "Relative L2 error vs host model (" << name
+              << "): " << (den > 0 ? std::sqrt(num / den) : std::sqrt(num))
+              << "\n";
+    if (mismatches)
+      std::cerr << name << " validation failed (" << mismatches
+                << " mismatches)\n";
+    return mismatches == 0;
+  };
+  bool ok = true;
+  if (doFwdPass) {
+    std::vector<double> expected(outElems + 1);
+    const int rc = oracle_convolution(
+        unsigned(n), fs.data(), itl.data(), itu.data(), idl.data(), ipl.data(),
+        ipu.data(), fi.data(), ks.data(), ktl.data(), ktu.data(), kdl.data(),
+        kpl.data(), kpu.data(), fk.data(), otl.data(), otu.data(), ost.data(),
+        opl.data(), opu.data(), unsigned(params.batchSize),
+        unsigned(params.numConvGroups),
+        unsigned(params.inputChannelsPerConvGroup),
+        unsigned(params.outputChannelsPerConvGroup), acts.data(),
+        weights.data(), biases.data(), expected.data(), outElems, 8);
+    if (rc != 0) {
+      std::cerr << "host model failed with code " << rc << "\n";
+      return 1;
+    }
+    ok = compare("fwd", result, expected, outElems) && ok;
   }
-  std::cout << "Relative L2 error vs host model: "
-            << (den > 0 ? std::sqrt(num / den) : std::sqrt(num)) << "\n";
-  if (mismatches) {
-    std::cerr << "Validation failed (" << mismatches << " mismatches)\n";
+  if (doBwdPass) {
+    std::vector<double> expected(inElems + 1);
+    const int rc = oracle_convolution_backward(
+        unsigned(n), fs.data(), itl.data(), itu.data(), idl.data(), ipl.data(),
+        ipu.data(), fi.data(), ks.data(), ktl.data(), ktu.data(), kdl.data(),
+        kpl.data(), kpu.data(), fk.data(), otl.data(), otu.data(), ost.data(),
+        opl.data(), opu.data(), unsigned(params.batchSize),
+        unsigned(params.numConvGroups),
+        unsigned(params.inputChannelsPerConvGroup),
+        unsigned(params.outputChannelsPerConvGroup), zDeltas.data(),
+        weights.data(), expected.data(), inElems, 8);
+    if (rc != 0) {
+      std::cerr << "host model (backward) failed with code " << rc << "\n";
+      return 1;
+    }
+    ok = compare("bwd", bwdResult, expected, inElems) && ok;
+  }
+  if (!ok)
     return 1;
-  }
   std::cout << "Validation passed\n";
   return 0;
 } catch (const poplar::graph_memory_allocation_error &e) {

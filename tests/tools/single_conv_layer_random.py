@@ -179,7 +179,7 @@ def command(p, binary):
            "--kernel-padding-lower", braces(p.k_pad_lower),
            "--kernel-padding-upper", braces(p.k_pad_upper),
            "--kernel-dilation", braces(p.k_dilation),
-           "--single-phase", "fwd",
+           "--single-phase", "all",
            "--convolution-options",
            '{"partialsType":"%s"}' % p.partials_type]
     if p.data_type == "quarter":
