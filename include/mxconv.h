@@ -287,6 +287,68 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
                                  void *out, void *workspace,
                                  size_t workspace_bytes, mxconv_stream stream);
 
+/* ---- matrix multiplication on the same kernels --------------------------- */
+
+/* getConvParams of lib/poplin/MatMul.cpp:236-272: C[g] = A[g] * B[g] with A
+ * [groups][m][k], B [groups][k][n] is the convolution with batch m, field {1},
+ * kernel {1}, k input and n output channels per group. */
+mxconv_status mxconv_matmul_params(int32_t input_type, int32_t output_type,
+                                   uint64_t groups, uint64_t m, uint64_t k,
+                                   uint64_t n, mxconv_params *p);
+
+/* parseMatMulOptions + getConvOptionFlags (lib/poplin/MatMul.cpp:116-195):
+ * checks matMul option keys / values (partialsType, fullyConnectedPass,
+ * inputRHSIsPreArranged, use128BitConvUnitLoad, enableMultiStageReduce,
+ * enableFastReduce, remapOutputTensor, availableMemoryProportion,
+ * planConstraints, gatherOutput, disableSRForAMPVertices). */
+mxconv_status mxconv_matmul_validate_options(const char *const *keys,
+                                             const char *const *values,
+                                             size_t num_options);
+
+/* mxconv_plan_create for the parameters of mxconv_matmul_params, taking
+ * matMul options (translated as getConvOptionFlags does). */
+mxconv_status mxconv_matmul_plan_create(int32_t input_type, int32_t output_type,
+                                        uint64_t groups, uint64_t m, uint64_t k,
+                                        uint64_t n,
+                                        const char *const *option_keys,
+                                        const char *const *option_values,
+                                        size_t num_options, mxconv_plan **plan);
+
+/* The right-hand side B [groups][k][n] -> the packed weights of a plan made
+ * from mxconv_matmul_params (convWeightsFromMatrix(transpose(B)),
+ * lib/poplin/MatMul.cpp:386). */
+mxconv_status mxconv_matmul_pack_rhs(const mxconv_plan *plan, const void *rhs,
+                                     void *weights_packed,
+                                     mxconv_stream stream);
+
+/* A [groups][m][k] -> the convolution's input [m][groups*k], and its output
+ * [m][groups*n] -> C [groups][m][n] (convActivationsFromMatrix /
+ * matrixFromConvActivations, lib/poplin/MatMul.cpp:197-226).  With one group
+ * both are plain copies and callers may pass the matrices themselves to
+ * mxconv_fwd instead. */
+mxconv_status mxconv_matmul_lhs_to_internal(const mxconv_plan *plan,
+                                            const void *lhs, void *acts_internal,
+                                            mxconv_stream stream);
+mxconv_status mxconv_matmul_out_to_external(const mxconv_plan *plan,
+                                            const void *out_internal,
+                                            void *result, mxconv_stream stream);
+
+/* poplin::transposeGroupedMatrix (include/poplin/MatMul.hpp:612) as a copy:
+ * src [groups][rows][cols] -> dst [groups][cols][rows]; any element type. */
+mxconv_status mxconv_transpose_grouped_matrix(int32_t type, uint64_t groups,
+                                              uint64_t rows, uint64_t cols,
+                                              const void *src, void *dst,
+                                              mxconv_stream stream);
+
+/* c[i] = scale_c * c[i] + scale_product * product[i] over `elems` half or
+ * float elements, evaluated in fp32: the popops::scaledAddTo step of
+ * poplin::matMulAcc / matMulGroupedAcc (lib/poplin/MatMul.cpp:499-519,
+ * 578-597; scale_c = 1 there) and of a general beta * C + alpha * A * B
+ * (tools/general_matrix_multiply.cpp:367). */
+mxconv_status mxconv_scaled_add_to(int32_t type, void *c, float scale_c,
+                                   const void *product, float scale_product,
+                                   uint64_t elems, mxconv_stream stream);
+
 /* poplin::weightsTransposeChansFlipXY (include/poplin/Convolution.hpp:407-412,
  * lib/poplin/Convolution.cpp:3262-3388) on device tensors in the external
  * layout: weights_in [G][Co][Ci][kernel...] -> weights_out

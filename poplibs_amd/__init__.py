@@ -7,7 +7,8 @@ planning are host code), any device call without the built library or without
 a GPU raises.
 """
 from .capi import (  # noqa: F401
-    FLOAT, HALF, QUARTER, ConvParams, InputTransform, MxconvError,
+    FLOAT, HALF, QUARTER, ConvParams, InputTransform, MatMulPlan, MxconvError,
     OutputTransform, Plan, Status, add_bias, build_library, getGradientParams,
-    lib, library_path, quarter_metadata, validate_options,
+    lib, library_path, matMulParams, matMulValidateOptions, quarter_metadata,
+    scaled_add_to, transposeGroupedMatrix, validate_options,
     weightsTransposeChansFlipXY)

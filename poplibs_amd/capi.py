@@ -155,6 +155,28 @@ def lib():
         "mxconv_fwd_quarter": (c_int, [c_void_p, c_void_p, c_uint8, c_void_p,
                                        c_uint8, c_void_p, c_void_p, c_void_p,
                                        c_size_t, c_void_p]),
+        "mxconv_matmul_params": (c_int, [c_int32, c_int32, c_uint64, c_uint64,
+                                         c_uint64, c_uint64, P]),
+        "mxconv_matmul_validate_options": (c_int, [POINTER(c_char_p),
+                                                   POINTER(c_char_p),
+                                                   c_size_t]),
+        "mxconv_matmul_plan_create": (c_int, [c_int32, c_int32, c_uint64,
+                                              c_uint64, c_uint64, c_uint64,
+                                              POINTER(c_char_p),
+                                              POINTER(c_char_p), c_size_t,
+                                              POINTER(c_void_p)]),
+        "mxconv_matmul_pack_rhs": (c_int, [c_void_p, c_void_p, c_void_p,
+                                           c_void_p]),
+        "mxconv_matmul_lhs_to_internal": (c_int, [c_void_p, c_void_p, c_void_p,
+                                                  c_void_p]),
+        "mxconv_matmul_out_to_external": (c_int, [c_void_p, c_void_p, c_void_p,
+                                                  c_void_p]),
+        "mxconv_transpose_grouped_matrix": (c_int, [c_int32, c_uint64, c_uint64,
+                                                    c_uint64, c_void_p,
+                                                    c_void_p, c_void_p]),
+        "mxconv_scaled_add_to": (c_int, [c_int32, c_void_p, ctypes.c_float,
+                                         c_void_p, ctypes.c_float, c_uint64,
+                                         c_void_p]),
         "mxconv_add_bias": (c_int, [c_int32, c_void_p, c_void_p, c_uint64,
                                     c_uint64, c_void_p]),
     }
@@ -550,6 +572,48 @@ class Plan:
                                         stream))
 
 
+def matMulParams(inputType, outputType, groups, m, k, n):
+    """getConvParams of lib/poplin/MatMul.cpp:236-272: the convolution that
+    computes C[g] = A[g] * B[g] for A [groups][m][k], B [groups][k][n]."""
+    out = CParams()
+    _check(lib().mxconv_matmul_params(inputType, outputType, groups, m, k, n,
+                                      byref(out)))
+    return ConvParams.from_c(out)
+
+
+def matMulValidateOptions(options):
+    """Checks matMul option keys and values (lib/poplin/MatMul.cpp:116-160)."""
+    keys, values, n = _option_arrays(options)
+    _check(lib().mxconv_matmul_validate_options(keys, values, n))
+
+
+class MatMulPlan(Plan):
+    """A plan for C[g] = A[g] * B[g], made from matMul options.  The operands
+    are row-major device matrices A [groups][m][k], B [groups][k][n]; with one
+    group A and C are the plan's input and output as they stand."""
+
+    def __init__(self, inputType, outputType, groups, m, k, n, options=None):
+        self.params = matMulParams(inputType, outputType, groups, m, k, n)
+        self.groups, self.m, self.k, self.n = groups, m, k, n
+        keys, values, num = _option_arrays(options)
+        self._h = c_void_p()
+        _check(lib().mxconv_matmul_plan_create(
+            inputType, outputType, groups, m, k, n, keys, values, num,
+            byref(self._h)))
+
+    def pack_rhs(self, rhs, weights_packed, stream=0):
+        _check(lib().mxconv_matmul_pack_rhs(self._h, rhs, weights_packed,
+                                            stream))
+
+    def lhs_to_internal(self, lhs, acts_internal, stream=0):
+        _check(lib().mxconv_matmul_lhs_to_internal(self._h, lhs, acts_internal,
+                                                   stream))
+
+    def out_to_external(self, out_internal, result, stream=0):
+        _check(lib().mxconv_matmul_out_to_external(self._h, out_internal,
+                                                   result, stream))
+
+
 def getGradientParams(params):
     """poplin::getGradientParams (lib/poplin/ConvUtil.cpp:728-795)."""
     return params.getGradientParams()
@@ -560,6 +624,21 @@ def weightsTransposeChansFlipXY(params, weights_in, weights_out, stream=0):
     layout; ``params`` are the forward parameters."""
     _check(lib().mxconv_weights_transpose_chans_flip_xy(
         byref(params.to_c()), weights_in, weights_out, stream))
+
+
+def transposeGroupedMatrix(type_id, groups, rows, cols, src, dst, stream=0):
+    """poplin::transposeGroupedMatrix as a device copy:
+    src [groups][rows][cols] -> dst [groups][cols][rows]."""
+    _check(lib().mxconv_transpose_grouped_matrix(type_id, groups, rows, cols,
+                                                 src, dst, stream))
+
+
+def scaled_add_to(type_id, c, scale_c, product, scale_product, elems,
+                  stream=0):
+    """c = scale_c * c + scale_product * product; poplin::matMulAcc is the
+    case scale_c = 1."""
+    _check(lib().mxconv_scaled_add_to(type_id, c, scale_c, product,
+                                      scale_product, elems, stream))
 
 
 def add_bias(type_id, acts, bias, outer_elems, channels, stream=0):

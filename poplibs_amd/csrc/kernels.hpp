@@ -52,6 +52,11 @@ hipError_t launchGeneric(const GenericDesc &d, int inType, int outType,
 hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
                           const int perm[4], int elemBytes, hipStream_t stream);
 
+/// a[i] = scaleA * a[i] + scaleB * b[i] for half or float arrays, evaluated
+/// in fp32.
+hipError_t launchScaledAdd(int type, void *a, float scaleA, const void *b,
+                           float scaleB, uint64_t total, hipStream_t stream);
+
 /// dst[g][ci][co][k...] = src[g][co][ci][flipped k...]: channels transposed,
 /// every one of the numDims (<= kMaxDims) kernel axes reversed.
 hipError_t launchWeightsTransposeChansFlipXY(const void *src, void *dst,
@@ -67,7 +72,8 @@ hipError_t launchWeightsTransposeChansFlipXY(const void *src, void *dst,
 hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                                   uint32_t co, uint32_t ci, uint32_t taps,
                                   uint32_t coPadded, uint32_t kPadded,
-                                  int elemBytes, hipStream_t stream);
+                                  int elemBytes, hipStream_t stream,
+                                  bool chansTransposed = false);
 
 /// acts[outer][c] += bias[c] for `type` elements (kHalf or kFloat).
 hipError_t launchAddBias(int type, void *acts, const void *bias,
@@ -103,7 +109,8 @@ bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType);
 /// Elements of the packed weights ([G][32-channel block][k-slice][lane][8]).
 uint64_t pointwisePackedElems(const PointwiseDesc &d);
 hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
-                                      void *dst, hipStream_t stream);
+                                      void *dst, hipStream_t stream,
+                                      bool chansTransposed = false);
 hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream);

@@ -32,7 +32,8 @@ __global__ __launch_bounds__(256) void permuteKernel(PermuteArgs a,
 template <class T>
 __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
     const T *__restrict__ src, T *__restrict__ dst, uint32_t co, uint32_t ci,
-    uint32_t taps, uint32_t coPadded, uint32_t kPadded, uint64_t total) {
+    uint32_t taps, uint32_t coPadded, uint32_t kPadded, uint64_t total,
+    bool chansTransposed) {
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
     return;
@@ -42,7 +43,10 @@ __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
   T v = T(0);
   if (n < co && k < taps * ci) {
     const uint32_t tap = k / ci, c = k % ci;
-    v = src[((g * co + n) * ci + c) * taps + tap];
+    // source [G][Co][Ci][taps], or [G][Ci][Co][taps] (a matrix
+    // multiplication's right-hand side)
+    v = chansTransposed ? src[((g * ci + c) * co + n) * taps + tap]
+                        : src[((g * co + n) * ci + c) * taps + tap];
   }
   dst[tid] = v;
 }
@@ -88,6 +92,19 @@ __global__ __launch_bounds__(256) void addBiasKernel(T *acts,
     return;
   const float v = Load<T>::at(acts, tid, 0) + Load<T>::at(bias, tid % channels, 0);
   storeOut(acts, tid, v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void scaledAddKernel(T *a,
+                                                       float scaleA,
+                                                       const T *__restrict__ b,
+                                                       float scaleB,
+                                                       uint64_t total) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= total)
+    return;
+  storeOut(a, tid,
+           scaleA * Load<T>::at(a, tid, 0) + scaleB * Load<T>::at(b, tid, 0));
 }
 
 } // namespace
@@ -137,7 +154,8 @@ hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
 hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                                   uint32_t co, uint32_t ci, uint32_t taps,
                                   uint32_t coPadded, uint32_t kPadded,
-                                  int elemBytes, hipStream_t stream) {
+                                  int elemBytes, hipStream_t stream,
+                                  bool chansTransposed) {
   const uint64_t total = uint64_t(groups) * coPadded * kPadded;
   if (total == 0)
     return hipSuccess;
@@ -149,12 +167,12 @@ hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint8_t>, grid, block, 0, stream,
                        static_cast<const uint8_t *>(src),
                        static_cast<uint8_t *>(dst), co, ci, taps, coPadded,
-                       kPadded, total);
+                       kPadded, total, chansTransposed);
   else if (elemBytes == 2)
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint16_t>, grid, block, 0, stream,
                        static_cast<const uint16_t *>(src),
                        static_cast<uint16_t *>(dst), co, ci, taps, coPadded,
-                       kPadded, total);
+                       kPadded, total, chansTransposed);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
@@ -216,6 +234,27 @@ hipError_t launchAddBias(int type, void *acts, const void *bias,
     hipLaunchKernelGGL(addBiasKernel<__half>, grid, block, 0, stream,
                        static_cast<__half *>(acts),
                        static_cast<const __half *>(bias), total, channels);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launchScaledAdd(int type, void *a, float scaleA, const void *b,
+                           float scaleB, uint64_t total, hipStream_t stream) {
+  if (total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  if (type == kFloat)
+    hipLaunchKernelGGL(scaledAddKernel<float>, grid, block, 0, stream,
+                       static_cast<float *>(a), scaleA,
+                       static_cast<const float *>(b), scaleB, total);
+  else if (type == kHalf)
+    hipLaunchKernelGGL(scaledAddKernel<__half>, grid, block, 0, stream,
+                       static_cast<__half *>(a), scaleA,
+                       static_cast<const __half *>(b), scaleB, total);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

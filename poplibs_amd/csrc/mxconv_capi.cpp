@@ -3,6 +3,7 @@
 #include "mxconv.h"
 
 #include "../src/ConvOptions.hpp"
+#include "../src/MatMulOptions.hpp"
 #include "../src/Plan.hpp"
 #include "kernels.hpp"
 #include "poplar/exceptions.hpp"
@@ -607,6 +608,163 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
                  stream);
 }
 
+// ---- matrix multiplication -------------------------------------------------
+
+} // extern "C"
+
+namespace {
+
+poplin::ConvParams matMulParams(int32_t inputType, int32_t outputType,
+                                uint64_t groups, uint64_t m, uint64_t k,
+                                uint64_t n) {
+  mxconv_params c{};
+  c.input_type = inputType;
+  c.output_type = outputType;
+  const poplin::ConvParams types = poplin::ConvParams::fromC(c); // checks ids
+  return poplin::ConvParams(types.inputType, types.outputType, m, {1}, {1}, k,
+                            n, groups);
+}
+
+/// True when `plan` has the shape mxconv_matmul_params produces.
+bool isMatMulPlan(const mxconv_plan *plan) {
+  const auto &p = plan->params;
+  for (auto s : p.inputFieldShape)
+    if (s != 1)
+      return false;
+  for (auto s : p.kernelShape)
+    if (s != 1)
+      return false;
+  return p == poplin::ConvParams(p.inputType, p.outputType, p.batchSize,
+                                 p.inputFieldShape, p.kernelShape,
+                                 p.inputChannelsPerConvGroup,
+                                 p.outputChannelsPerConvGroup, p.numConvGroups);
+}
+
+} // namespace
+
+extern "C" {
+
+mxconv_status mxconv_matmul_params(int32_t input_type, int32_t output_type,
+                                   uint64_t groups, uint64_t m, uint64_t k,
+                                   uint64_t n, mxconv_params *p) {
+  REQUIRE_ARG(p);
+  return guarded([&] {
+    matMulParams(input_type, output_type, groups, m, k, n).toC(*p);
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_matmul_validate_options(const char *const *keys,
+                                             const char *const *values,
+                                             size_t num_options) {
+  return guarded([&] {
+    poplin::ConvOptions options(poplin::matMulToConvOptions(
+        collectOptions(keys, values, num_options)));
+    (void)options;
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_matmul_plan_create(int32_t input_type, int32_t output_type,
+                                        uint64_t groups, uint64_t m, uint64_t k,
+                                        uint64_t n,
+                                        const char *const *option_keys,
+                                        const char *const *option_values,
+                                        size_t num_options, mxconv_plan **plan) {
+  REQUIRE_ARG(plan);
+  *plan = nullptr;
+  return guarded([&] {
+    poplin::ConvOptions options(poplin::matMulToConvOptions(
+        collectOptions(option_keys, option_values, num_options)));
+    *plan = new mxconv_plan(poplin::makePlan(
+        matMulParams(input_type, output_type, groups, m, k, n), options));
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_matmul_pack_rhs(const mxconv_plan *plan, const void *rhs,
+                                     void *weights_packed,
+                                     mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  if (!isMatMulPlan(plan))
+    return fail(MXCONV_INVALID_PARAMS,
+                "not a matrix-multiplication plan (field and kernel {1}, "
+                "identity transforms)");
+  if (plan->weightPackedElems == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(weights_packed);
+  if (plan->weightElems != 0)
+    REQUIRE_ARG(rhs);
+  const auto &p = plan->params;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int elemBytes = int(p.inputType.size());
+  if (plan->kernel == mxconv_plan::Kernel::IGEMM) {
+    if (plan->pointwiseOn)
+      return hipStatus(mxk::launchPackPointwiseWeights(plan->pointwise, rhs,
+                                                       weights_packed, s, true),
+                       "weight packing");
+    return hipStatus(
+        mxk::launchPackIgemmWeights(
+            rhs, weights_packed, uint32_t(p.numConvGroups),
+            uint32_t(p.outputChannelsPerConvGroup),
+            uint32_t(p.inputChannelsPerConvGroup), 1, uint32_t(plan->coPadded),
+            uint32_t(plan->kPadded), elemBytes, s, true),
+        "weight packing");
+  }
+  // Generic kernel: packed = [G][1][Ci][Co], which is B itself.  Depthwise
+  // kernel (k = n = 1): packed = [1][G], again B itself.
+  return hipStatus(hipMemcpyAsync(weights_packed, rhs, plan->weightBytes(),
+                                  hipMemcpyDeviceToDevice, s),
+                   "weight packing");
+}
+
+} // extern "C"
+
+namespace {
+
+mxconv_status shuffleGroups(const mxconv_plan *plan, const void *src, void *dst,
+                            bool toInternal, mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  if (!isMatMulPlan(plan))
+    return fail(MXCONV_INVALID_PARAMS,
+                "not a matrix-multiplication plan (field and kernel {1}, "
+                "identity transforms)");
+  const auto &p = plan->params;
+  const uint64_t g = p.numConvGroups, m = p.batchSize;
+  const uint64_t c = toInternal ? p.inputChannelsPerConvGroup
+                                : p.outputChannelsPerConvGroup;
+  if (g * m * c == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(src);
+  REQUIRE_ARG(dst);
+  const int elemBytes =
+      int(toInternal ? p.inputType.size() : p.outputType.size());
+  // [G][M][C] -> [M][G][C] or back: swap the two leading axes.
+  const uint64_t dims[4] = {1, toInternal ? g : m, toInternal ? m : g, c};
+  const int perm[4] = {0, 2, 1, 3};
+  return hipStatus(mxk::launchPermute4(src, dst, dims, perm, elemBytes,
+                                       reinterpret_cast<hipStream_t>(stream)),
+                   "matrix group shuffle");
+}
+
+} // namespace
+
+extern "C" {
+
+mxconv_status mxconv_matmul_lhs_to_internal(const mxconv_plan *plan,
+                                            const void *lhs, void *acts_internal,
+                                            mxconv_stream stream) {
+  return shuffleGroups(plan, lhs, acts_internal, true, stream);
+}
+
+mxconv_status mxconv_matmul_out_to_external(const mxconv_plan *plan,
+                                            const void *out_internal,
+                                            void *result, mxconv_stream stream) {
+  return shuffleGroups(plan, out_internal, result, false, stream);
+}
+
 mxconv_status mxconv_weights_transpose_chans_flip_xy(const mxconv_params *p,
                                                      const void *weights_in,
                                                      void *weights_out,
@@ -639,6 +797,42 @@ mxconv_status mxconv_weights_transpose_chans_flip_xy(const mxconv_params *p,
           uint32_t(params.kernelShape.size()), shape,
           int(params.inputType.size()), reinterpret_cast<hipStream_t>(stream)),
       "weight transposition");
+}
+
+mxconv_status mxconv_transpose_grouped_matrix(int32_t type, uint64_t groups,
+                                              uint64_t rows, uint64_t cols,
+                                              const void *src, void *dst,
+                                              mxconv_stream stream) {
+  lastError.clear();
+  if (type != MXCONV_QUARTER && type != MXCONV_HALF && type != MXCONV_FLOAT)
+    return fail(MXCONV_INVALID_PARAMS, "unknown element type");
+  if (groups * rows * cols == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(src);
+  REQUIRE_ARG(dst);
+  const uint64_t dims[4] = {1, groups, rows, cols};
+  const int perm[4] = {0, 1, 3, 2};
+  const int elemBytes = type == MXCONV_FLOAT ? 4 : type == MXCONV_HALF ? 2 : 1;
+  return hipStatus(mxk::launchPermute4(src, dst, dims, perm, elemBytes,
+                                       reinterpret_cast<hipStream_t>(stream)),
+                   "matrix transposition");
+}
+
+mxconv_status mxconv_scaled_add_to(int32_t type, void *c, float scale_c,
+                                   const void *product, float scale_product,
+                                   uint64_t elems, mxconv_stream stream) {
+  lastError.clear();
+  if (type != MXCONV_HALF && type != MXCONV_FLOAT)
+    return fail(MXCONV_INVALID_PARAMS,
+                "scaled add takes half or float tensors");
+  if (elems == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(c);
+  REQUIRE_ARG(product);
+  return hipStatus(mxk::launchScaledAdd(type, c, scale_c, product,
+                                        scale_product, elems,
+                                        reinterpret_cast<hipStream_t>(stream)),
+                   "scaled add");
 }
 
 mxconv_status mxconv_add_bias(int32_t type, void *acts_internal,

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
 /// Channels past Co are zero.
 __global__ __launch_bounds__(256) void packPointwiseWeightsKernel(
     const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, uint32_t co,
-    uint32_t ci, uint32_t nBlocks, uint64_t total) {
+    uint32_t ci, uint32_t nBlocks, uint64_t total, bool chansTransposed) {
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
     return;
@@ -207,7 +207,11 @@ __global__ __launch_bounds__(256) void packPointwiseWeightsKernel(
   const uint64_t g = r / nBlocks;
   const uint32_t n = block * 32 + (lane & 31);
   const uint32_t k = ks * 16 + 8 * (lane >> 5) + e;
-  dst[tid] = n < co ? src[(g * co + n) * ci + k] : uint16_t(0);
+  // source [G][Co][Ci], or [G][Ci][Co] (a matrix multiplication's right-hand
+  // side)
+  dst[tid] = n >= co           ? uint16_t(0)
+             : chansTransposed ? src[(g * ci + k) * co + n]
+                               : src[(g * co + n) * ci + k];
 }
 
 template <int KS, int TM, int NB, class OutT>
@@ -293,7 +297,8 @@ uint64_t pointwisePackedElems(const PointwiseDesc &d) {
 }
 
 hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
-                                      void *dst, hipStream_t stream) {
+                                      void *dst, hipStream_t stream,
+                                      bool chansTransposed) {
   const uint64_t total = pointwisePackedElems(d);
   if (total == 0)
     return hipSuccess;
@@ -304,7 +309,7 @@ hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
   hipLaunchKernelGGL(packPointwiseWeightsKernel, dim3(uint32_t(blocks)),
                      dim3(256), 0, stream, static_cast<const uint16_t *>(src),
                      static_cast<uint16_t *>(dst), d.outChansPerGroup,
-                     d.inChansPerGroup, nBlocks, total);
+                     d.inChansPerGroup, nBlocks, total, chansTransposed);
   return hipGetLastError();
 }
 

@@ -156,6 +156,9 @@ void readTensor(const DeviceTensor &t, void *host, Stream &prog,
                 const ConvParams &params,
                 const poplar::OptionFlags &options = {},
                 PlanningCache *cache = nullptr);
+/// The same for tensors in the External layout, which need no plan.
+void writeTensor(const DeviceTensor &t, const void *host, Stream &prog);
+void readTensor(const DeviceTensor &t, void *host, Stream &prog);
 
 } // namespace poplin
 #endif

@@ -2,6 +2,7 @@
 // memory and host transfers use the HIP runtime directly; every kernel launch
 // goes through an mxconv_* call.
 #include "poplin/Convolution.hpp"
+#include "LayerInternal.hpp"
 #include "mxconv.h"
 #include "poplar/exceptions.hpp"
 #include "poputil/exceptions.hpp"
@@ -17,9 +18,9 @@
 
 namespace poplin {
 
-namespace {
+namespace detail {
 
-[[noreturn]] void raise(mxconv_status s) {
+[[noreturn]] static void raise(mxconv_status s) {
   const std::string message = mxconv_last_error();
   switch (s) {
   case MXCONV_INVALID_OPTION:
@@ -35,7 +36,7 @@ void check(mxconv_status s) {
   if (s != MXCONV_OK)
     raise(s);
 }
-void checkHip(hipError_t e, const char *what) {
+static void checkHip(hipError_t e, const char *what) {
   if (e == hipSuccess)
     return;
   const std::string message = std::string(what) + ": " + hipGetErrorString(e);
@@ -44,15 +45,7 @@ void checkHip(hipError_t e, const char *what) {
   throw poputil::poplibs_error(message);
 }
 
-struct PlanHandle {
-  mxconv_plan *plan = nullptr;
-  explicit PlanHandle(mxconv_plan *p) : plan(p) {}
-  ~PlanHandle() { mxconv_plan_destroy(plan); }
-  PlanHandle(const PlanHandle &) = delete;
-  PlanHandle &operator=(const PlanHandle &) = delete;
-};
-
-std::shared_ptr<PlanHandle> createPlan(const ConvParams &params,
+static std::shared_ptr<PlanHandle> createPlan(const ConvParams &params,
                                        const poplar::OptionFlags &options) {
   mxconv_params c;
   params.toC(c);
@@ -72,7 +65,7 @@ std::size_t bufferBytes(const mxconv_plan *plan, mxconv_buffer which) {
   return bytes;
 }
 
-std::vector<std::size_t> actsShape(std::size_t batch, std::size_t chans,
+static std::vector<std::size_t> actsShape(std::size_t batch, std::size_t chans,
                                    const std::vector<std::size_t> &field) {
   std::vector<std::size_t> shape{batch, chans};
   shape.insert(shape.end(), field.begin(), field.end());
@@ -83,7 +76,8 @@ mxconv_stream streamOf(const Stream &s) {
   return static_cast<mxconv_stream>(s.handle());
 }
 
-} // namespace
+} // namespace detail
+using namespace detail;
 
 // ---- Stream ---------------------------------------------------------------
 
@@ -140,7 +134,7 @@ std::size_t PlanningCache::size() const {
   return impl->plans.size();
 }
 
-namespace {
+namespace detail {
 std::shared_ptr<PlanHandle> getPlan(const ConvParams &params,
                                     const poplar::OptionFlags &options,
                                     PlanningCache *cache) {
@@ -158,7 +152,7 @@ std::shared_ptr<PlanHandle> getPlan(const ConvParams &params,
   cache->impl->plans.emplace(key, plan);
   return plan;
 }
-} // namespace
+} // namespace detail
 
 // ---- entry points ---------------------------------------------------------
 
@@ -487,6 +481,22 @@ void readTensor(const DeviceTensor &t, void *host, Stream &prog,
                             hipMemcpyDeviceToHost, s),
              "hipMemcpyAsync");
   prog.synchronize();
+}
+
+void writeTensor(const DeviceTensor &t, const void *host, Stream &prog) {
+  if (t.layout() != DeviceTensor::Layout::External)
+    throw poputil::poplibs_error(
+        "writeTensor: a tensor in a device layout needs the parameters of "
+        "the plan that laid it out");
+  writeTensor(t, host, prog, ConvParams{});
+}
+
+void readTensor(const DeviceTensor &t, void *host, Stream &prog) {
+  if (t.layout() != DeviceTensor::Layout::External)
+    throw poputil::poplibs_error(
+        "readTensor: a tensor in a device layout needs the parameters of "
+        "the plan that laid it out");
+  readTensor(t, host, prog, ConvParams{});
 }
 
 } // namespace poplin

@@ -169,3 +169,107 @@ def test_conv_random_quarter(seed):
                         "--input-type", "quarter"],
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-3000:])
+
+
+# ---------------------------------------------------------------------------
+# general_matrix_multiply: the reference's cases for its tool of that name
+# (tests/poplin/CMakeLists.txt:515-900).
+
+GEMM = os.path.join(ROOT, "tests", "tools", "general_matrix_multiply")
+
+
+def gemm(*args, timeout=120):
+    if not os.path.exists(GEMM):
+        subprocess.check_call(["make", "-C", os.path.dirname(GEMM)],
+                              stdout=subprocess.DEVNULL)
+    return subprocess.run([GEMM, *args], capture_output=True, text=True,
+                          timeout=timeout)
+
+
+def test_gemm_report_plan_without_a_device():
+    r = gemm("--m", "1024", "--k", "512", "--n", "512", "--report-plan",
+             "--compile-only")
+    assert r.returncode == 0, r.stderr
+    assert "implicit GEMM" in r.stdout
+    assert "batchSize                  1024" in r.stdout
+    # a serial split is an IPU memory device: accepted, and the plan is the
+    # unconstrained one
+    r2 = gemm("--m", "1024", "--k", "512", "--n", "512", "--report-plan",
+              "--compile-only", "--plan-constraints",
+              '{"0":{"partition":{"outChanSplit":{"serial":2}}}}')
+    assert r2.returncode == 0, r2.stderr
+    assert r2.stdout == r.stdout
+
+
+def test_gemm_usage_errors_exit_1():
+    assert gemm("--m", "4", "--k", "4").returncode == 1
+    assert gemm("--m", "4", "--k", "4", "--n", "4", "--bogus").returncode == 1
+    assert gemm("--m", "4", "--k", "4", "--n", "4", "--left-matrix-op",
+                "conjugate").returncode == 1
+    r = gemm("--m", "4", "--k", "4", "--n", "4", "--data-type", "half",
+             "--input-type", "half", "--output-type", "float")
+    assert r.returncode == 1 and "not both" in r.stderr
+    r = gemm("--m", "4", "--k", "4", "--n", "4", "--partials-type", "int",
+             "--compile-only", "--report-plan")
+    assert r.returncode == 1
+
+
+_OPS = [("normal", "normal"), ("transpose", "normal"), ("normal", "transpose"),
+        ("transpose", "transpose")]
+GEMM_GPU_CASES = (
+    [(f"gemm_{m}x{k}x{n}_{a[:2]}A_{b[:2]}B",
+      f"--m {m} --k {k} --n {n} --alpha 1 --beta 1 --tiles-per-ipu=1 "
+      f"--left-matrix-op={a} --right-matrix-op={b}")
+     for (m, k, n) in ((5, 0, 4), (0, 3, 4), (5, 3, 0)) for a, b in _OPS] + [
+        ("gemm_5x0x4_groups3_ignore_data_profile",
+         "--g 3 --m 5 --k 0 --n 4 --tiles-per-ipu=1 --ignore-data --profile "
+         "--report-plan --show-execution-steps --show-var-storage"),
+        ("gemm_1x3x1", "--m 1 --k 3 --n 1 --alpha 1 --beta 1"),
+        ("gemm_1x1000x1", "--m 1 --k 1000 --n 1 --alpha 2 --beta 1"),
+        ("gemm_40x40x40", "--m 40 --k 40 --n 40 --alpha 2 --beta 1"),
+        ("gemm_10x20x30_groups5",
+         "--g 5 --m 10 --k 20 --n 30 --alpha 2 --beta 3"),
+        ("gemm_40x39x38", "--m 40 --k 39 --n 38 --alpha 2 --beta 1"),
+        ("gemm_40x39x38_left_transpose",
+         "--m 40 --k 39 --n 38 --alpha 2 --beta 1 --left-matrix-op=transpose"),
+        ("gemm_40x39x38_right_transpose",
+         "--m 40 --k 39 --n 38 --alpha 2 --beta 1 "
+         "--right-matrix-op=transpose"),
+        ("gemm_40x40x40_halffloat",
+         "--m 40 --k 40 --n 40 --alpha 2 --beta 1 --input-type=half "
+         "--output-type=float"),
+        ("gemm_40x39x38_floathalf",
+         "--m 40 --k 39 --n 38 --alpha 2 --beta 1 --input-type=float "
+         "--output-type=half"),
+        ("gemm_40x39x38_right_transpose_floathalf",
+         "--m 40 --k 39 --n 38 --alpha 2 --beta 1 --right-matrix-op=transpose "
+         "--input-type=float --output-type=half"),
+        ("gemm_100x100x100_serial_split_nx2",
+         "--m 100 --k 100 --n 100 --plan-constraints "
+         '{"0":{"partition":{"outChanSplit":{"serial":2}}}}'),
+        ("gemm_float_40x39x38", "--m 40 --k 39 --n 38 --data-type float"),
+        # matrix-core and streaming kernels, tighter tolerance than the
+        # tool's default 10 % for half
+        ("gemm_1024x512x512_mfma",
+         "--m 1024 --k 512 --n 512 --alpha 1 --beta 0 --tolerance 0.01"),
+        ("gemm_groups4_300x72x136_mfma",
+         "--g 4 --m 300 --k 72 --n 136 --input-type=half --output-type=float "
+         "--tolerance 0.01"),
+        ("gemm_4100x256x64_pointwise",
+         "--m 4100 --k 256 --n 64 --input-type=half --output-type=float "
+         "--tolerance 0.01 --use-create-output=true"),
+        ("gemm_prearranged_rhs_repeated",
+         "--m 700 --k 136 --n 72 --input-type=half --output-type=float "
+         "--tolerance 0.01 --pre-arrange-rhs=true --num-executions 3"),
+        ("gemm_quarter",
+         "--m 200 --k 256 --n 128 --input-type=quarter --output-type=half "
+         "--fp8-format-a quart143 --fp8-format-b quart143 --fp8-scale-b -2"),
+    ])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,args", GEMM_GPU_CASES,
+                         ids=[c[0] for c in GEMM_GPU_CASES])
+def test_gemm_reference_cases(name, args):
+    r = gemm(*args.split())
+    assert r.returncode == 0, (name, r.stdout[-2000:], r.stderr[-2000:])
