@@ -137,6 +137,13 @@ mxconv_status mxconv_params_canonicalize(const mxconv_params *p,
 mxconv_status mxconv_get_gradient_params(const mxconv_params *p,
                                          mxconv_params *gradient);
 
+/* getWeightUpdateParams (include/poplin/ConvUtil.hpp:114,
+ * lib/poplin/Convolution.cpp:3390-3435): the convolution that computes the
+ * gradient w.r.t. the forward weights - batch and input channels exchanged,
+ * the forward output field as kernel.  The result is canonical. */
+mxconv_status mxconv_get_weight_update_params(const mxconv_params *p,
+                                              mxconv_params *weight_update);
+
 /* isZeroConvolution (lib/poplin/ConvUtilInternal.cpp:24-38); canonicalizes
  * first, as CanonicalConvParams does. */
 mxconv_status mxconv_params_is_zero_convolution(const mxconv_params *p,
@@ -332,6 +339,68 @@ mxconv_status mxconv_matmul_lhs_to_internal(const mxconv_plan *plan,
 mxconv_status mxconv_matmul_out_to_external(const mxconv_plan *plan,
                                             const void *out_internal,
                                             void *result, mxconv_stream stream);
+
+/* ---- weight update pass ---------------------------------------------------
+ * poplin::calculateWeightDeltas / convolutionWeightUpdate /
+ * convolutionBiasUpdate (include/poplin/Convolution.hpp:460-563,
+ * lib/poplin/Convolution.cpp:3437-3620).
+ *
+ * The plan of the pass: mxconv_plan_create on
+ * mxconv_get_weight_update_params(fwd) with the forward options, whose `pass`
+ * is replaced as getWeightUpdateOptions does
+ * (lib/poplin/ConvUtilInternal.cpp:941-954).  For
+ * mxconv_convolution_weight_update give forward parameters whose output type
+ * equals the input type, as the reference does (:3535), so that the deltas
+ * come out in the weights' type. */
+mxconv_status mxconv_weight_update_plan_create(const mxconv_params *fwd,
+                                               const char *const *option_keys,
+                                               const char *const *option_values,
+                                               size_t num_options,
+                                               mxconv_plan **plan);
+
+/* Bytes of device scratch the two calls below need for `plan` (the
+ * rearranged operands, the pass's output before it is brought into weight
+ * order and, for the update, the deltas). */
+mxconv_status mxconv_weight_update_workspace_bytes(const mxconv_plan *plan,
+                                                   size_t *bytes);
+
+/* weight_deltas [G][Co][Ci][kernel...] (external layout, the plan's output
+ * type) = gradient w.r.t. the forward weights, from z_deltas
+ * [B][outField...][G*Co] and activations [B][field...][G*Ci], both
+ * channels-last in the forward input type.  Half and float tensors. */
+mxconv_status mxconv_calculate_weight_deltas(const mxconv_plan *plan,
+                                             const void *z_deltas_internal,
+                                             const void *acts_internal,
+                                             void *weight_deltas_external,
+                                             void *workspace,
+                                             size_t workspace_bytes,
+                                             mxconv_stream stream);
+
+/* weights_external += scale * weight deltas (lib/poplin/Convolution.cpp:
+ * 3552-3571); pack the updated weights again for the forward plan. */
+mxconv_status mxconv_convolution_weight_update(const mxconv_plan *plan,
+                                               const void *z_deltas_internal,
+                                               void *weights_external,
+                                               const void *acts_internal,
+                                               float scale, void *workspace,
+                                               size_t workspace_bytes,
+                                               mxconv_stream stream);
+
+/* biases[c] += scale * sum of z_deltas over batch and field
+ * (lib/poplin/Convolution.cpp:3592-3620).  z_deltas is channels-last
+ * [outer_elems][channels]; sums are formed in fp32 in a fixed order.
+ * workspace: mxconv_bias_update_workspace_bytes. */
+mxconv_status mxconv_bias_update_workspace_bytes(uint64_t outer_elems,
+                                                 uint64_t channels,
+                                                 size_t *bytes);
+mxconv_status mxconv_convolution_bias_update(int32_t deltas_type,
+                                             const void *z_deltas_internal,
+                                             uint64_t outer_elems,
+                                             uint64_t channels,
+                                             int32_t bias_type, void *biases,
+                                             float scale, void *workspace,
+                                             size_t workspace_bytes,
+                                             mxconv_stream stream);
 
 /* poplin::transposeGroupedMatrix (include/poplin/MatMul.hpp:612) as a copy:
  * src [groups][rows][cols] -> dst [groups][cols][rows]; any element type. */

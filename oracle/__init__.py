@@ -46,6 +46,12 @@ def lib():
             + [pu, pu, pu, pu, pu, pu, pb]       # kernel + transform
             + [pu, pu, pu, pu, pu]               # output transform
             + [u, u, u, u, pd, pd, pd, ctypes.c_size_t, ctypes.c_int])
+        L.oracle_weight_update.restype = ctypes.c_int
+        L.oracle_weight_update.argtypes = (
+            [u, pu, pu, pu, pu, pu, pu, pb]      # input field + transform
+            + [pu, pu, pu, pu, pu, pu, pb]       # kernel + transform
+            + [pu, pu, pu, pu, pu]               # output transform
+            + [u, u, u, u, pd, pd, pd, ctypes.c_size_t, pd, ctypes.c_int])
         L.oracle_output_field_size.restype = u
         L.oracle_output_field_size.argtypes = [u] * 17
         L.oracle_fp8_decode.restype = ctypes.c_double
@@ -171,6 +177,59 @@ def convolution_backward(p, deltas, weights, threads=1):
     if rc != 0:
         raise RuntimeError(f"oracle_convolution_backward failed with code {rc}")
     return out
+
+
+def weight_deltas(p, activations, deltas, threads=1, with_bias=False):
+    """Gradient of the forward convolution ``p`` with respect to its weights
+    (and, with ``with_bias``, its biases): the deltas that
+    poplibs_test::conv::weightUpdate scales by -learningRate and adds.
+
+    ``activations`` [B][G*Ci][field...] are the forward input, ``deltas``
+    [B][G*Co][outField...] the gradient of the forward output; the result is
+    [G][Co][Ci][kernel...] (and [G*Co]), dtype float64.
+    """
+    L = lib()
+    nd = len(p.inputFieldShape)
+    G, Ci, Co, B = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                    p.outputChannelsPerConvGroup, p.batchSize)
+    activations = np.ascontiguousarray(activations, dtype=np.float64)
+    deltas = np.ascontiguousarray(deltas, dtype=np.float64)
+    assert activations.shape == (B, G * Ci, *p.inputFieldShape), \
+        activations.shape
+    assert deltas.shape == (B, G * Co, *output_field_shape(p)), deltas.shape
+    out = np.empty((G, Co, Ci, *p.kernelShape), dtype=np.float64)
+    bias = np.empty(G * Co, dtype=np.float64)
+    it, kt, ot = p.inputTransform, p.kernelTransform, p.outputTransform
+    pd = ctypes.POINTER(ctypes.c_double)
+    spare = np.zeros(1)
+
+    def ptr(a):
+        return (a if a.size else spare).ctypes.data_as(pd)
+
+    rc = L.oracle_weight_update(
+        nd, _uarr(p.inputFieldShape), _uarr(it.truncationLower),
+        _uarr(it.truncationUpper), _uarr(it.dilation), _uarr(it.paddingLower),
+        _uarr(it.paddingUpper), _barr(it.flip),
+        _uarr(p.kernelShape), _uarr(kt.truncationLower),
+        _uarr(kt.truncationUpper), _uarr(kt.dilation), _uarr(kt.paddingLower),
+        _uarr(kt.paddingUpper), _barr(kt.flip),
+        _uarr(ot.truncationLower), _uarr(ot.truncationUpper), _uarr(ot.stride),
+        _uarr(ot.paddingLower), _uarr(ot.paddingUpper),
+        B, G, Ci, Co, ptr(activations), ptr(deltas), ptr(out), out.size,
+        ptr(bias), int(threads))
+    if rc != 0:
+        raise RuntimeError(f"oracle_weight_update failed with code {rc}")
+    return (out, bias) if with_bias else out
+
+
+def weight_update(p, learning_rate, activations, deltas, kernel, biases,
+                  threads=1):
+    """poplibs_test::conv::weightUpdate: returns the updated (kernel, biases),
+    kernel - learning_rate * weight deltas and likewise for the biases
+    (lib/poplibs_test/Convolution.cpp:870-897)."""
+    dw, db = weight_deltas(p, activations, deltas, threads, with_bias=True)
+    return (np.asarray(kernel, dtype=np.float64) + learning_rate * -dw,
+            np.asarray(biases, dtype=np.float64) + learning_rate * -db)
 
 
 E5M2, E4M3 = 0, 1

@@ -4,6 +4,7 @@
  * CPU restatement, in plain C and double precision, of the host reference
  * model that the PopLibs convolution tests compare against:
  *   poplibs_test::conv::convolution   lib/poplibs_test/Convolution.cpp:455-575
+ * (and of its backward and weight update companions further down)
  * and of the helpers it is built from (cited at each function).  It exists so
  * that the parity tests, the smoke check and the benchmark's CPU-baseline leg
  * have an independent statement of what a forward convolution must produce.
@@ -21,6 +22,11 @@
  *     (lib/poplin/ConvUtil.cpp:234-268),
  *   - slicing invariants (sub-convolution of sliced tensors == slice of the
  *     full result; a split over input channels sums to the full result).
+ * convolutionBackward (:577-722) and weightUpdate (:724-898) are restated
+ * too; they are pinned by torch autograd in float64 on ordinary parameters and,
+ * with every transform, by the adjoint identities
+ *   <conv(x, w), dz> == <x, backward(dz, w)> == <w, weightDeltas(x, dz)>
+ * (tests/test_backward.py, tests/test_weight_update.py).
  * The FP8 codec below is this build's own definition (OCP E4M3FN / E5M2 plus a
  * power-of-two scale); bit-level parity with Graphcore's QUARTER type, whose
  * codec lives in the closed Poplar SDK, is: parity unpinned.
@@ -506,6 +512,188 @@ int oracle_convolution_backward(
   for (unsigned d = 0; d != n; ++d)
     if (size[d] != fwd_input_field_size[d])
       return -1;
+  return 0;
+}
+
+/*
+ * The gradient part of poplibs_test::conv::weightUpdate,
+ * lib/poplibs_test/Convolution.cpp:724-898 (the reference goes on to apply
+ * kernel += learningRate * -weightDeltas and biases += learningRate *
+ * -biasDeltas, :881-897; callers do that on the two arrays returned here).
+ *   activations   [batch][groups*in_chans_per_group][prod(input_field_size)]
+ *   deltas        [batch][groups*out_chans_per_group][prod(output field)]
+ *   weight_deltas [groups][out_chans_per_group][in_chans_per_group]
+ *                 [prod(kernel_size)]       (weight_delta_elems doubles)
+ *   bias_deltas   [groups*out_chans_per_group], may be NULL
+ * Each element's sum runs over the batch outermost and the output positions
+ * innermost, as in the reference (:838-863); threads share out whole
+ * (group, out-channel) rows.  Returns as oracle_convolution.
+ */
+int oracle_weight_update(
+    unsigned num_field_dims, const unsigned *input_field_size,
+    const unsigned *truncation_lower, const unsigned *truncation_upper,
+    const unsigned *input_dilation, const unsigned *padding_lower,
+    const unsigned *padding_upper, const unsigned char *flip_input,
+    const unsigned *kernel_size, const unsigned *kernel_truncation_lower,
+    const unsigned *kernel_truncation_upper, const unsigned *kernel_dilation,
+    const unsigned *kernel_padding_lower, const unsigned *kernel_padding_upper,
+    const unsigned char *flip_kernel, const unsigned *output_truncation_lower,
+    const unsigned *output_truncation_upper, const unsigned *stride,
+    const unsigned *output_padding_lower, const unsigned *output_padding_upper,
+    unsigned batch_size, unsigned num_conv_groups, unsigned in_chans_per_group,
+    unsigned out_chans_per_group, const double *activations,
+    const double *deltas, double *weight_deltas, size_t weight_delta_elems,
+    double *bias_deltas, int threads) {
+  const unsigned n = num_field_dims;
+  if (n > ORACLE_MAX_DIMS)
+    return -2;
+  const unsigned in_chans = num_conv_groups * in_chans_per_group;
+  const unsigned out_chans = num_conv_groups * out_chans_per_group;
+
+  /* :766-771 */
+  unsigned output_field_size[ORACLE_MAX_DIMS];
+  unsigned padded_kernel_size[ORACLE_MAX_DIMS];
+  for (unsigned d = 0; d != n; ++d) {
+    output_field_size[d] = oracle_output_field_size(
+        input_field_size[d], kernel_size[d], truncation_lower[d],
+        truncation_upper[d], input_dilation[d], padding_lower[d],
+        padding_upper[d], kernel_truncation_lower[d], kernel_truncation_upper[d],
+        kernel_dilation[d], kernel_padding_lower[d], kernel_padding_upper[d],
+        output_truncation_lower[d], output_truncation_upper[d], stride[d],
+        output_padding_lower[d], output_padding_upper[d]);
+    /* :778-780 */
+    padded_kernel_size[d] = transformed_size(
+        kernel_size[d], kernel_truncation_lower[d], kernel_truncation_upper[d],
+        kernel_dilation[d], kernel_padding_lower[d], kernel_padding_upper[d]);
+  }
+
+  /* :783-787 */
+  unsigned padded_acts_size[ORACLE_MAX_DIMS];
+  double *padded_acts = truncate_dilate_pad_flip(
+      activations, (size_t)batch_size * in_chans, n, input_field_size,
+      truncation_lower, truncation_upper, input_dilation, padding_lower,
+      padding_upper, flip_input, padded_acts_size);
+  if (!padded_acts)
+    return -3;
+
+  /* :789-808 */
+  unsigned fwd_conv_out_size[ORACLE_MAX_DIMS];
+  unsigned deltas_padding_upper[ORACLE_MAX_DIMS];
+  for (unsigned d = 0; d != n; ++d) {
+    fwd_conv_out_size[d] =
+        absdiff(padded_acts_size[d], padded_kernel_size[d]) + 1;
+    /* The reference adds the truncation here (:796-798) where the backward
+     * pass subtracts it (:663-665); with it the striding term below would be
+     * wrong whenever the output is truncated, and the padded deltas would not
+     * have the size of the forward pass's untruncated output.  The size the
+     * stride sees is the forward convolution output less its truncation. */
+    const unsigned truncated =
+        fwd_conv_out_size[d] -
+        (output_truncation_lower[d] + output_truncation_upper[d]);
+    if (output_padding_lower[d] + (truncated + stride[d] - 1) / stride[d] +
+            output_padding_upper[d] !=
+        output_field_size[d]) {
+      free(padded_acts);
+      return -1;
+    }
+    const unsigned striding_ignored =
+        truncated == 0 ? 0 : (truncated - 1) % stride[d];
+    deltas_padding_upper[d] = output_truncation_upper[d] + striding_ignored;
+  }
+  /* :810-814 */
+  unsigned char no_flipping[ORACLE_MAX_DIMS] = {0};
+  unsigned padded_deltas_size[ORACLE_MAX_DIMS];
+  double *padded_deltas = truncate_dilate_pad_flip(
+      deltas, (size_t)batch_size * out_chans, n, output_field_size,
+      output_padding_lower, output_padding_upper, stride,
+      output_truncation_lower, deltas_padding_upper, no_flipping,
+      padded_deltas_size);
+  if (!padded_deltas) {
+    free(padded_acts);
+    return -3;
+  }
+  for (unsigned d = 0; d != n; ++d)
+    if (padded_deltas_size[d] != fwd_conv_out_size[d]) {
+      free(padded_acts);
+      free(padded_deltas);
+      return -1;
+    }
+
+  /* :830-863 */
+  const size_t padded_kernel_elems = product(padded_kernel_size, n);
+  const size_t padded_deltas_elems = product(fwd_conv_out_size, n);
+  const size_t padded_acts_elems = product(padded_acts_size, n);
+  const size_t rows =
+      (size_t)num_conv_groups * out_chans_per_group * in_chans_per_group;
+  double *padded_weight_deltas =
+      (double *)calloc(rows * padded_kernel_elems + 1, sizeof(double));
+  if (!padded_weight_deltas) {
+    free(padded_acts);
+    free(padded_deltas);
+    return -3;
+  }
+  const long pairs = (long)num_conv_groups * (long)out_chans_per_group;
+  if (threads < 1)
+    threads = 1;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+  for (long pair = 0; pair < pairs; ++pair) {
+    const unsigned oc = (unsigned)(pair % out_chans_per_group);
+    const unsigned gc = (unsigned)(pair / out_chans_per_group);
+    const unsigned oc_act = gc * out_chans_per_group + oc;
+    double *row = padded_weight_deltas + (size_t)pair * in_chans_per_group *
+                                             padded_kernel_elems;
+    for (unsigned b = 0; b != batch_size; ++b) {
+      const double *delta_row =
+          padded_deltas + ((size_t)b * out_chans + oc_act) * padded_deltas_elems;
+      for (size_t oe = 0; oe != padded_deltas_elems; ++oe) {
+        unsigned output_indices[ORACLE_MAX_DIMS];
+        unflatten_index(fwd_conv_out_size, n, oe, output_indices);
+        for (size_t ke = 0; ke != padded_kernel_elems; ++ke) {
+          unsigned kernel_indices[ORACLE_MAX_DIMS];
+          unsigned input_indices[ORACLE_MAX_DIMS];
+          unflatten_index(padded_kernel_size, n, ke, kernel_indices);
+          if (get_input_indices(n, padded_acts_size, padded_kernel_size,
+                                output_indices, kernel_indices, input_indices)) {
+            const size_t ie = flatten_index(padded_acts_size, n, input_indices);
+            for (unsigned ic = 0; ic != in_chans_per_group; ++ic) {
+              const unsigned ic_act = gc * in_chans_per_group + ic;
+              row[(size_t)ic * padded_kernel_elems + ke] +=
+                  padded_acts[((size_t)b * in_chans + ic_act) * padded_acts_elems +
+                              ie] *
+                  delta_row[oe];
+            }
+          }
+        }
+      }
+    }
+  }
+
+  /* :865-868 */
+  unsigned size[ORACLE_MAX_DIMS];
+  int rc = truncate_dilate_pad_flip_inverse(
+      padded_weight_deltas, rows, n, padded_kernel_size, kernel_truncation_lower,
+      kernel_truncation_upper, kernel_dilation, kernel_padding_lower,
+      kernel_padding_upper, flip_kernel, weight_deltas, weight_delta_elems,
+      size);
+  free(padded_weight_deltas);
+  free(padded_acts);
+  free(padded_deltas);
+  if (rc != 0)
+    return -1;
+  for (unsigned d = 0; d != n; ++d)
+    if (size[d] != kernel_size[d])
+      return -1;
+
+  /* :881-891 */
+  if (bias_deltas) {
+    const size_t out_elems = product(output_field_size, n);
+    for (unsigned oc = 0; oc != out_chans; ++oc)
+      bias_deltas[oc] = 0.0;
+    for (unsigned b = 0; b != batch_size; ++b)
+      for (unsigned oc = 0; oc != out_chans; ++oc)
+        for (size_t e = 0; e != out_elems; ++e)
+          bias_deltas[oc] += deltas[((size_t)b * out_chans + oc) * out_elems + e];
+  }
   return 0;
 }
 

@@ -8,7 +8,8 @@ a GPU raises.
 """
 from .capi import (  # noqa: F401
     FLOAT, HALF, QUARTER, ConvParams, InputTransform, MatMulPlan, MxconvError,
-    OutputTransform, Plan, Status, add_bias, build_library, getGradientParams,
-    lib, library_path, matMulParams, matMulValidateOptions, quarter_metadata,
-    scaled_add_to, transposeGroupedMatrix, validate_options,
-    weightsTransposeChansFlipXY)
+    OutputTransform, Plan, Status, WeightUpdatePlan, add_bias,
+    bias_update_workspace_bytes, build_library, convolutionBiasUpdate,
+    getGradientParams, getWeightUpdateParams, lib, library_path, matMulParams,
+    matMulValidateOptions, quarter_metadata, scaled_add_to,
+    transposeGroupedMatrix, validate_options, weightsTransposeChansFlipXY)

@@ -117,6 +117,26 @@ def lib():
         "mxconv_params_validate": (c_int, [P]),
         "mxconv_params_canonicalize": (c_int, [P, P]),
         "mxconv_get_gradient_params": (c_int, [P, P]),
+        "mxconv_get_weight_update_params": (c_int, [P, P]),
+        "mxconv_weight_update_plan_create": (c_int, [P, POINTER(c_char_p),
+                                                     POINTER(c_char_p),
+                                                     c_size_t,
+                                                     POINTER(c_void_p)]),
+        "mxconv_weight_update_workspace_bytes": (c_int, [c_void_p,
+                                                         POINTER(c_size_t)]),
+        "mxconv_calculate_weight_deltas": (c_int, [c_void_p, c_void_p, c_void_p,
+                                                   c_void_p, c_void_p,
+                                                   c_size_t, c_void_p]),
+        "mxconv_convolution_weight_update": (c_int, [c_void_p, c_void_p,
+                                                     c_void_p, c_void_p,
+                                                     ctypes.c_float, c_void_p,
+                                                     c_size_t, c_void_p]),
+        "mxconv_bias_update_workspace_bytes": (c_int, [c_uint64, c_uint64,
+                                                       POINTER(c_size_t)]),
+        "mxconv_convolution_bias_update": (c_int, [c_int32, c_void_p, c_uint64,
+                                                   c_uint64, c_int32, c_void_p,
+                                                   ctypes.c_float, c_void_p,
+                                                   c_size_t, c_void_p]),
         "mxconv_weights_transpose_chans_flip_xy":
             (c_int, [P, c_void_p, c_void_p, c_void_p]),
         "mxconv_params_is_zero_convolution": (c_int, [P, POINTER(c_int)]),
@@ -373,6 +393,13 @@ class ConvParams:
         _check(lib().mxconv_get_gradient_params(byref(self.to_c()), byref(out)))
         return ConvParams.from_c(out)
 
+    def getWeightUpdateParams(self):
+        """poplin::getWeightUpdateParams (lib/poplin/Convolution.cpp:3390)."""
+        out = CParams()
+        _check(lib().mxconv_get_weight_update_params(byref(self.to_c()),
+                                                     byref(out)))
+        return ConvParams.from_c(out)
+
     def _size(self, query, dim):
         v = c_uint64()
         _check(lib().mxconv_params_size(byref(self.to_c()), query, dim,
@@ -612,6 +639,60 @@ class MatMulPlan(Plan):
     def out_to_external(self, out_internal, result, stream=0):
         _check(lib().mxconv_matmul_out_to_external(self._h, out_internal,
                                                    result, stream))
+
+
+class WeightUpdatePlan(Plan):
+    """The plan of the weight update pass of the forward convolution
+    ``fwd_params`` (poplin::calculateWeightDeltas /
+    convolutionWeightUpdate).  Tensors are device pointers: z_deltas and
+    activations channels-last, weights and weight deltas in the external
+    [G][Co][Ci][kernel...] layout."""
+
+    def __init__(self, fwd_params, options=None):
+        self.fwd_params = fwd_params
+        self.params = fwd_params.getWeightUpdateParams()
+        keys, values, n = _option_arrays(options)
+        self._h = c_void_p()
+        _check(lib().mxconv_weight_update_plan_create(
+            byref(fwd_params.to_c()), keys, values, n, byref(self._h)))
+
+    def workspace_bytes(self):
+        v = c_size_t()
+        _check(lib().mxconv_weight_update_workspace_bytes(self._h, byref(v)))
+        return v.value
+
+    def calculate_weight_deltas(self, z_deltas, acts, weight_deltas, workspace,
+                                workspace_bytes, stream=0):
+        _check(lib().mxconv_calculate_weight_deltas(
+            self._h, z_deltas, acts, weight_deltas, workspace, workspace_bytes,
+            stream))
+
+    def weight_update(self, z_deltas, weights, acts, scale, workspace,
+                      workspace_bytes, stream=0):
+        _check(lib().mxconv_convolution_weight_update(
+            self._h, z_deltas, weights, acts, scale, workspace,
+            workspace_bytes, stream))
+
+
+def bias_update_workspace_bytes(outer_elems, channels):
+    v = c_size_t()
+    _check(lib().mxconv_bias_update_workspace_bytes(outer_elems, channels,
+                                                    byref(v)))
+    return v.value
+
+
+def convolutionBiasUpdate(deltas_type, z_deltas, outer_elems, channels,
+                          bias_type, biases, scale, workspace, workspace_bytes,
+                          stream=0):
+    """poplin::convolutionBiasUpdate on a channels-last z_deltas."""
+    _check(lib().mxconv_convolution_bias_update(
+        deltas_type, z_deltas, outer_elems, channels, bias_type, biases, scale,
+        workspace, workspace_bytes, stream))
+
+
+def getWeightUpdateParams(params):
+    """poplin::getWeightUpdateParams (lib/poplin/Convolution.cpp:3390-3435)."""
+    return params.getWeightUpdateParams()
 
 
 def getGradientParams(params):

@@ -52,6 +52,14 @@ hipError_t launchGeneric(const GenericDesc &d, int inType, int outType,
 hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
                           const int perm[4], int elemBytes, hipStream_t stream);
 
+/// biases[c] += scale * sum over rows of zDeltas[row][c] (half or float each),
+/// summed in fp32 in a fixed order: per-split partial sums go to `workspace`
+/// (biasUpdateWorkspaceBytes), a second kernel adds them up split by split.
+size_t biasUpdateWorkspaceBytes(uint64_t rows, uint64_t channels);
+hipError_t launchBiasUpdate(int deltasType, const void *zDeltas, uint64_t rows,
+                            uint64_t channels, int biasType, void *biases,
+                            float scale, void *workspace, hipStream_t stream);
+
 /// a[i] = scaleA * a[i] + scaleB * b[i] for half or float arrays, evaluated
 /// in fp32.
 hipError_t launchScaledAdd(int type, void *a, float scaleA, const void *b,

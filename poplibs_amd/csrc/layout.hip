@@ -107,6 +107,47 @@ __global__ __launch_bounds__(256) void scaledAddKernel(T *a,
            scaleA * Load<T>::at(a, tid, 0) + scaleB * Load<T>::at(b, tid, 0));
 }
 
+constexpr uint32_t kReduceChans = 64, kReduceLanes = 4;
+
+/// partial[split][c] = sum over the rows of `split` of z[row][c], fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void channelSumKernel(
+    const T *__restrict__ z, float *__restrict__ partial, uint64_t rows,
+    uint64_t channels, uint64_t rowsPerSplit) {
+  __shared__ float lanes[kReduceLanes][kReduceChans];
+  const uint32_t cLocal = threadIdx.x % kReduceChans;
+  const uint32_t lane = threadIdx.x / kReduceChans;
+  const uint64_t c = uint64_t(blockIdx.x) * kReduceChans + cLocal;
+  const uint64_t first = uint64_t(blockIdx.y) * rowsPerSplit;
+  const uint64_t last = min(first + rowsPerSplit, rows);
+  float sum = 0.f;
+  if (c < channels)
+    for (uint64_t r = first + lane; r < last; r += kReduceLanes)
+      sum += Load<T>::at(z, r * channels + c, 0);
+  lanes[lane][cLocal] = sum;
+  __syncthreads();
+  if (lane == 0 && c < channels) {
+    float total = lanes[0][cLocal];
+    for (uint32_t l = 1; l != kReduceLanes; ++l)
+      total += lanes[l][cLocal];
+    partial[uint64_t(blockIdx.y) * channels + c] = total;
+  }
+}
+
+/// biases[c] += scale * sum over splits of partial[split][c], splits in order.
+template <typename T>
+__global__ __launch_bounds__(256) void biasUpdateKernel(
+    T *biases, const float *__restrict__ partial, float scale,
+    uint64_t channels, uint32_t splits) {
+  const uint64_t c = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (c >= channels)
+    return;
+  float total = 0.f;
+  for (uint32_t s = 0; s != splits; ++s)
+    total += partial[uint64_t(s) * channels + c];
+  storeOut(biases, c, Load<T>::at(biases, c, 0) + scale * total);
+}
+
 } // namespace
 
 hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
@@ -234,6 +275,51 @@ hipError_t launchAddBias(int type, void *acts, const void *bias,
     hipLaunchKernelGGL(addBiasKernel<__half>, grid, block, 0, stream,
                        static_cast<__half *>(acts),
                        static_cast<const __half *>(bias), total, channels);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+uint32_t biasUpdateSplits(uint64_t rows) {
+  const uint64_t splits = (rows + 127) / 128;
+  return uint32_t(splits < 1 ? 1 : splits > 256 ? 256 : splits);
+}
+
+size_t biasUpdateWorkspaceBytes(uint64_t rows, uint64_t channels) {
+  return size_t(biasUpdateSplits(rows)) * channels * sizeof(float);
+}
+
+hipError_t launchBiasUpdate(int deltasType, const void *zDeltas, uint64_t rows,
+                            uint64_t channels, int biasType, void *biases,
+                            float scale, void *workspace, hipStream_t stream) {
+  if (channels == 0)
+    return hipSuccess;
+  const uint32_t splits = biasUpdateSplits(rows);
+  const uint64_t rowsPerSplit = (rows + splits - 1) / splits;
+  const uint64_t chanBlocks = (channels + kReduceChans - 1) / kReduceChans;
+  if (chanBlocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  float *partial = static_cast<float *>(workspace);
+  const dim3 grid{uint32_t(chanBlocks), splits}, block{256};
+  if (deltasType == kFloat)
+    hipLaunchKernelGGL(channelSumKernel<float>, grid, block, 0, stream,
+                       static_cast<const float *>(zDeltas), partial, rows,
+                       channels, rowsPerSplit);
+  else if (deltasType == kHalf)
+    hipLaunchKernelGGL(channelSumKernel<__half>, grid, block, 0, stream,
+                       static_cast<const __half *>(zDeltas), partial, rows,
+                       channels, rowsPerSplit);
+  else
+    return hipErrorInvalidValue;
+  const dim3 grid2{uint32_t((channels + 255) / 256)};
+  if (biasType == kFloat)
+    hipLaunchKernelGGL(biasUpdateKernel<float>, grid2, block, 0, stream,
+                       static_cast<float *>(biases), partial, scale, channels,
+                       splits);
+  else if (biasType == kHalf)
+    hipLaunchKernelGGL(biasUpdateKernel<__half>, grid2, block, 0, stream,
+                       static_cast<__half *>(biases), partial, scale, channels,
+                       splits);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

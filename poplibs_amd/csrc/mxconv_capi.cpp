@@ -228,6 +228,17 @@ mxconv_status mxconv_get_gradient_params(const mxconv_params *p,
   });
 }
 
+mxconv_status mxconv_get_weight_update_params(const mxconv_params *p,
+                                              mxconv_params *weight_update) {
+  REQUIRE_ARG(p);
+  REQUIRE_ARG(weight_update);
+  return guarded([&] {
+    poplin::getWeightUpdateParams(poplin::ConvParams::fromC(*p))
+        .toC(*weight_update);
+    return MXCONV_OK;
+  });
+}
+
 mxconv_status mxconv_params_is_zero_convolution(const mxconv_params *p,
                                                 int *is_zero) {
   REQUIRE_ARG(p);
@@ -849,6 +860,235 @@ mxconv_status mxconv_add_bias(int32_t type, void *acts_internal,
                                       channels,
                                       reinterpret_cast<hipStream_t>(stream)),
                    "bias add");
+}
+
+} // extern "C"
+
+namespace {
+
+size_t alignUp(size_t v) { return (v + 255) & ~size_t(255); }
+
+/// Where the weight update pass keeps its intermediates in the workspace.
+struct WuWorkspace {
+  size_t input, weightsExternal, weightsPacked, output, deltas, planWorkspace,
+      total;
+};
+
+WuWorkspace wuWorkspace(const mxconv_plan *plan) {
+  WuWorkspace w{};
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t offset = at;
+    at += alignUp(bytes);
+    return offset;
+  };
+  w.input = take(plan->inputBytes());
+  w.weightsExternal = take(plan->weightBytes());
+  w.weightsPacked = take(plan->weightPackedBytes());
+  w.output = take(plan->outputBytes());
+  w.deltas = take(plan->outputBytes());
+  w.planWorkspace = take(plan->workspaceBytes);
+  w.total = at;
+  return w;
+}
+
+uint64_t product(const std::vector<std::size_t> &shape) {
+  uint64_t n = 1;
+  for (auto s : shape)
+    n *= s;
+  return n;
+}
+
+mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
+                           const void *acts, void *deltasOut, char *ws,
+                           mxconv_stream stream) {
+  // The pass's convolution (lib/poplin/Convolution.cpp:3437-3483): batch =
+  // forward input channels, input channels = forward batch, kernel = forward
+  // output field, output field = forward kernel.
+  const auto &p = plan->params;
+  const uint64_t G = p.numConvGroups, Ci = p.batchSize,
+                 B = p.inputChannelsPerConvGroup,
+                 Co = p.outputChannelsPerConvGroup;
+  const uint64_t X = product(p.inputFieldShape), Y = product(p.kernelShape),
+                 K = product(p.getOutputFieldShape());
+  const int inBytes = int(p.inputType.size());
+  const int outBytes = int(p.outputType.size());
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const WuWorkspace w = wuWorkspace(plan);
+  if (G * Co * Ci * K == 0)
+    return MXCONV_OK;
+  mxconv_status st;
+  if (plan->inputElems) {
+    // activations [B][X][G][Ci] -> the pass's input [Ci][X][G][B]
+    const uint64_t dims[4] = {B, X, G, Ci};
+    const int perm[4] = {3, 1, 2, 0};
+    st = hipStatus(mxk::launchPermute4(acts, ws + w.input, dims, perm, inBytes,
+                                       s),
+                   "activation rearrangement");
+    if (st != MXCONV_OK)
+      return st;
+  }
+  if (plan->weightElems) {
+    // deltas [B][Y][G][Co] -> the pass's weights [G][Co][B][Y]
+    const uint64_t dims[4] = {B, Y, G, Co};
+    const int perm[4] = {2, 3, 0, 1};
+    st = hipStatus(mxk::launchPermute4(zDeltas, ws + w.weightsExternal, dims,
+                                       perm, inBytes, s),
+                   "delta rearrangement");
+    if (st != MXCONV_OK)
+      return st;
+  }
+  st = mxconv_pack_weights(plan, ws + w.weightsExternal, ws + w.weightsPacked,
+                           stream);
+  if (st != MXCONV_OK)
+    return st;
+  st = forward(plan, ws + w.input, ws + w.weightsPacked, nullptr,
+               ws + w.output, ws + w.planWorkspace, plan->workspaceBytes,
+               mxk::QuarterInfo{}, stream);
+  if (st != MXCONV_OK)
+    return st;
+  // the pass's output [Ci][K][G][Co] -> weight order [G][Co][Ci][K]
+  const uint64_t dims[4] = {Ci, K, G, Co};
+  const int perm[4] = {2, 3, 0, 1};
+  return hipStatus(mxk::launchPermute4(ws + w.output, deltasOut, dims, perm,
+                                       outBytes, s),
+                   "weight delta rearrangement");
+}
+
+mxconv_status checkWuCall(const mxconv_plan *plan, const void *zDeltas,
+                          const void *acts, const void *result,
+                          const void *workspace, size_t workspaceBytes) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  if (plan->params.inputType == poplar::QUARTER)
+    return fail(MXCONV_UNSUPPORTED,
+                "the weight update pass takes half or float tensors");
+  if (plan->outputElems == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(result);
+  if (plan->inputElems)
+    REQUIRE_ARG(acts);
+  if (plan->weightElems)
+    REQUIRE_ARG(zDeltas);
+  const size_t need = wuWorkspace(plan).total;
+  if (workspaceBytes < need || !workspace)
+    return fail(MXCONV_WORKSPACE_TOO_SMALL,
+                "workspace of " + std::to_string(need) + " bytes required");
+  return MXCONV_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+mxconv_status mxconv_weight_update_plan_create(const mxconv_params *fwd,
+                                               const char *const *option_keys,
+                                               const char *const *option_values,
+                                               size_t num_options,
+                                               mxconv_plan **plan) {
+  REQUIRE_ARG(fwd);
+  REQUIRE_ARG(plan);
+  *plan = nullptr;
+  return guarded([&] {
+    poplin::ConvOptions options(
+        collectOptions(option_keys, option_values, num_options));
+    options = poplin::getWeightUpdateOptions(options);
+    *plan = new mxconv_plan(poplin::makePlan(
+        poplin::getWeightUpdateParams(poplin::ConvParams::fromC(*fwd)),
+        options));
+    return MXCONV_OK;
+  });
+}
+
+mxconv_status mxconv_weight_update_workspace_bytes(const mxconv_plan *plan,
+                                                   size_t *bytes) {
+  REQUIRE_ARG(plan);
+  REQUIRE_ARG(bytes);
+  lastError.clear();
+  *bytes = wuWorkspace(plan).total;
+  return MXCONV_OK;
+}
+
+mxconv_status mxconv_calculate_weight_deltas(const mxconv_plan *plan,
+                                             const void *z_deltas_internal,
+                                             const void *acts_internal,
+                                             void *weight_deltas_external,
+                                             void *workspace,
+                                             size_t workspace_bytes,
+                                             mxconv_stream stream) {
+  const mxconv_status st =
+      checkWuCall(plan, z_deltas_internal, acts_internal,
+                  weight_deltas_external, workspace, workspace_bytes);
+  if (st != MXCONV_OK || plan->outputElems == 0)
+    return st;
+  return weightDeltas(plan, z_deltas_internal, acts_internal,
+                      weight_deltas_external, static_cast<char *>(workspace),
+                      stream);
+}
+
+mxconv_status mxconv_convolution_weight_update(const mxconv_plan *plan,
+                                               const void *z_deltas_internal,
+                                               void *weights_external,
+                                               const void *acts_internal,
+                                               float scale, void *workspace,
+                                               size_t workspace_bytes,
+                                               mxconv_stream stream) {
+  mxconv_status st = checkWuCall(plan, z_deltas_internal, acts_internal,
+                                 weights_external, workspace, workspace_bytes);
+  if (st != MXCONV_OK || plan->outputElems == 0)
+    return st;
+  if (plan->params.outputType != plan->params.inputType)
+    return fail(MXCONV_INVALID_PARAMS,
+                "the weight update needs a plan whose output type is the "
+                "weights' type");
+  char *ws = static_cast<char *>(workspace);
+  char *deltas = ws + wuWorkspace(plan).deltas;
+  st = weightDeltas(plan, z_deltas_internal, acts_internal, deltas, ws, stream);
+  if (st != MXCONV_OK)
+    return st;
+  return hipStatus(mxk::launchScaledAdd(plan->params.outputType.id(),
+                                        weights_external, 1.f, deltas, scale,
+                                        plan->outputElems,
+                                        reinterpret_cast<hipStream_t>(stream)),
+                   "weight update");
+}
+
+mxconv_status mxconv_bias_update_workspace_bytes(uint64_t outer_elems,
+                                                 uint64_t channels,
+                                                 size_t *bytes) {
+  REQUIRE_ARG(bytes);
+  lastError.clear();
+  *bytes = mxk::biasUpdateWorkspaceBytes(outer_elems, channels);
+  return MXCONV_OK;
+}
+
+mxconv_status mxconv_convolution_bias_update(int32_t deltas_type,
+                                             const void *z_deltas_internal,
+                                             uint64_t outer_elems,
+                                             uint64_t channels,
+                                             int32_t bias_type, void *biases,
+                                             float scale, void *workspace,
+                                             size_t workspace_bytes,
+                                             mxconv_stream stream) {
+  lastError.clear();
+  for (int32_t t : {deltas_type, bias_type})
+    if (t != MXCONV_HALF && t != MXCONV_FLOAT)
+      return fail(MXCONV_INVALID_PARAMS,
+                  "the bias update takes half or float tensors");
+  if (channels == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(biases);
+  if (outer_elems)
+    REQUIRE_ARG(z_deltas_internal);
+  const size_t need = mxk::biasUpdateWorkspaceBytes(outer_elems, channels);
+  if (workspace_bytes < need || !workspace)
+    return fail(MXCONV_WORKSPACE_TOO_SMALL,
+                "workspace of " + std::to_string(need) + " bytes required");
+  return hipStatus(mxk::launchBiasUpdate(deltas_type, z_deltas_internal,
+                                         outer_elems, channels, bias_type,
+                                         biases, scale, workspace,
+                                         reinterpret_cast<hipStream_t>(stream)),
+                   "bias update");
 }
 
 } // extern "C"

@@ -74,5 +74,12 @@ ConvParams getZeroConv(const ConvParams &params);
 /// (lib/poplin/ConvUtil.cpp:728-795).
 ConvParams getGradientParams(const ConvParams &params);
 
+/// Parameters of the convolution that computes the gradient with respect to
+/// the forward pass's weights: its input are the forward activations with
+/// batch and channel axes exchanged, its kernel the gradient with respect to
+/// the forward output, its output field the forward kernel; canonical
+/// (include/poplin/ConvUtil.hpp:114, lib/poplin/Convolution.cpp:3390-3435).
+ConvParams getWeightUpdateParams(const ConvParams &params);
+
 } // namespace poplin
 #endif

@@ -71,6 +71,10 @@ public:
   Layout layout() const { return layout_; }
   void *data() const { return buffer_.get(); }
   QuarterMetadata metadata; ///< meaningful for QUARTER tensors only
+  /// For a PackedWeights tensor: the plan whose packing it holds (set by
+  /// createWeights and preArrangeMatMulInputRHS), so that an update of the
+  /// weights can be applied in that packing.
+  std::shared_ptr<const void> packedFor;
 
 private:
   poplar::Type type_;
@@ -92,6 +96,11 @@ public:
 };
 
 std::uint64_t getFwdFlops(const ConvParams &params);
+/// The backward and weight update passes perform the forward pass's number of
+/// operations (lib/poplin/Convolution.cpp:3223-3225); `params` are the
+/// forward parameters.
+std::uint64_t getBwdFlops(const ConvParams &params);
+std::uint64_t getWuFlops(const ConvParams &params);
 
 /// Weights [convGroups][outChansPerGroup][inChansPerGroup][kernel...], held
 /// packed for the plan of (params, options).
@@ -134,6 +143,37 @@ void convolutionWithOutput(const DeviceTensor &in, const DeviceTensor &weights,
 /// the external layout (include/poplin/Convolution.hpp:407-412 of PopLibs).
 void weightsTransposeChansFlipXY(const DeviceTensor &weightsIn,
                                  const DeviceTensor &weightsOut, Stream &prog);
+
+/// Gradient with respect to the forward weights, [G][Co][Ci][kernel...] in the
+/// external layout and the forward output type, from the gradient with
+/// respect to the forward output `zDeltas` and the forward input
+/// `activations` (include/poplin/Convolution.hpp:460-466 of PopLibs).
+/// `params` and `options` are the forward pass's.
+DeviceTensor calculateWeightDeltas(const DeviceTensor &zDeltas,
+                                   const DeviceTensor &activations,
+                                   const ConvParams &params, Stream &prog,
+                                   const poplar::OptionFlags &options = {},
+                                   PlanningCache *cache = nullptr);
+
+/// weights += scale * weight deltas (include/poplin/Convolution.hpp:516-522
+/// of PopLibs).  `weights` are in the external layout or packed (as
+/// createWeights returns them); the deltas are formed in the weights' type.
+void convolutionWeightUpdate(const DeviceTensor &zDeltas,
+                             const DeviceTensor &weights,
+                             const DeviceTensor &activations,
+                             ConvParams params, float scale, Stream &prog,
+                             const poplar::OptionFlags &options = {},
+                             PlanningCache *cache = nullptr);
+
+/// biases[c] += scale * sum of zDeltas[b][c][...] over batch and field
+/// (include/poplin/Convolution.hpp:556-561 of PopLibs).
+void convolutionBiasUpdate(const DeviceTensor &zDeltas,
+                           const DeviceTensor &biases, float scale,
+                           const poplar::OptionFlags &options, Stream &prog);
+
+void reportWeightUpdatePlanInfo(std::ostream &out, const ConvParams &fwdParams,
+                                const poplar::OptionFlags &fwdOptions = {},
+                                PlanningCache *cache = nullptr);
 
 /// acts[b][c][...] += biases[c].
 void addBias(const DeviceTensor &in, const DeviceTensor &biases, Stream &prog);

@@ -279,4 +279,25 @@ std::string ConvOptions::key() const {
   return os.str();
 }
 
+namespace {
+
+bool isFullyConnected(Pass p) {
+  return p == Pass::FC_INFERENCE_FWD || p == Pass::FC_TRAINING_FWD ||
+         p == Pass::FC_TRAINING_BWD || p == Pass::FC_TRAINING_WU;
+}
+
+} // namespace
+
+ConvOptions getWeightUpdateOptions(ConvOptions fwdOptions) {
+  fwdOptions.pass = isFullyConnected(fwdOptions.pass) ? Pass::FC_TRAINING_WU
+                                                      : Pass::TRAINING_WU;
+  return fwdOptions;
+}
+
+ConvOptions getGradientOptions(ConvOptions fwdOptions) {
+  fwdOptions.pass = isFullyConnected(fwdOptions.pass) ? Pass::FC_TRAINING_BWD
+                                                      : Pass::TRAINING_BWD;
+  return fwdOptions;
+}
+
 } // namespace poplin

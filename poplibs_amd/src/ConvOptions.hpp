@@ -59,5 +59,12 @@ public:
   std::string key() const;
 };
 
+/// Options of the weight update / backward pass of a layer whose forward
+/// pass has `fwdOptions`: only `pass` changes, staying within the
+/// fully-connected family if it started there
+/// (lib/poplin/ConvUtilInternal.cpp:941-970).
+ConvOptions getWeightUpdateOptions(ConvOptions fwdOptions);
+ConvOptions getGradientOptions(ConvOptions fwdOptions);
+
 } // namespace poplin
 #endif

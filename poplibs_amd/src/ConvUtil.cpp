@@ -282,6 +282,44 @@ ConvParams getGradientParams(const ConvParams &params) {
   return bwd.canonicalize();
 }
 
+ConvParams getWeightUpdateParams(const ConvParams &params) {
+  const ConvParams p = params.canonicalize();
+  const unsigned numFieldDims = unsigned(p.getNumFieldDims());
+  // The activations keep their transform.  The deltas take the kernel's
+  // place: what the forward pass did to its output is undone on them
+  // (padding <-> truncation, stride -> dilation), and what it did to its
+  // kernel is undone on this convolution's output.
+  ConvParams::InputTransform inputTransform = p.inputTransform;
+  ConvParams::InputTransform kernelTransform;
+  kernelTransform.truncationLower = p.outputTransform.paddingLower;
+  kernelTransform.truncationUpper = p.outputTransform.paddingUpper;
+  kernelTransform.dilation = p.outputTransform.stride;
+  kernelTransform.paddingLower = p.outputTransform.truncationLower;
+  kernelTransform.paddingUpper = p.outputTransform.truncationUpper;
+  kernelTransform.flip.assign(numFieldDims, false);
+  ConvParams::OutputTransform outputTransform;
+  outputTransform.truncationLower = p.kernelTransform.paddingLower;
+  outputTransform.truncationUpper = p.kernelTransform.paddingUpper;
+  outputTransform.stride = p.kernelTransform.dilation;
+  outputTransform.paddingLower = p.kernelTransform.truncationLower;
+  outputTransform.paddingUpper = p.kernelTransform.truncationUpper;
+  // A kernel flipped in the forward pass means this pass's output flipped,
+  // which is the same as flipping both of its operands.
+  for (unsigned d = 0; d != numFieldDims; ++d)
+    if (p.kernelTransform.flip[d]) {
+      inputTransform.flip[d] = !inputTransform.flip[d];
+      kernelTransform.flip[d] = true;
+    }
+  // Batch and input channels change places; the forward output field is the
+  // kernel, the forward kernel the output field.
+  const ConvParams wu(p.inputType, p.outputType,
+                      p.getNumInputChansPerConvGroup(), p.inputFieldShape,
+                      p.getOutputFieldShape(), p.getBatchSize(),
+                      p.getNumOutputChansPerConvGroup(), p.getNumConvGroups(),
+                      inputTransform, kernelTransform, outputTransform);
+  return wu.canonicalize();
+}
+
 ConvParams getZeroConv(const ConvParams &params) {
   // Truncate input and kernel to nothing, pad each back to one zero, convolve
   // to a single element, truncate it away and pad the output to full size.

@@ -173,9 +173,11 @@ DeviceTensor createWeights(const ConvParams &params,
                                  params.inputChannelsPerConvGroup};
   shape.insert(shape.end(), params.kernelShape.begin(),
                params.kernelShape.end());
-  return DeviceTensor(params.inputType, shape,
-                      DeviceTensor::Layout::PackedWeights,
-                      bufferBytes(plan->plan, MXCONV_BUFFER_WEIGHTS_PACKED));
+  DeviceTensor weights(params.inputType, shape,
+                       DeviceTensor::Layout::PackedWeights,
+                       bufferBytes(plan->plan, MXCONV_BUFFER_WEIGHTS_PACKED));
+  weights.packedFor = plan;
+  return weights;
 }
 
 DeviceTensor createBiases(const DeviceTensor &acts) {

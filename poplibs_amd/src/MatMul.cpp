@@ -149,6 +149,7 @@ DeviceTensor preArrange(const std::vector<std::size_t> &aShape,
                       DeviceTensor::Layout::PackedWeights,
                       bufferBytes(plan->plan, MXCONV_BUFFER_WEIGHTS_PACKED));
   packed.metadata = B.metadata;
+  packed.packedFor = plan;
   check(mxconv_matmul_pack_rhs(plan->plan, B.data(), packed.data(),
                                streamOf(prog)));
   return packed;

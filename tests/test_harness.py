@@ -28,6 +28,10 @@ def test_plan_only_reports_flops_and_plan():
     # 3x3 stride 1 "same": going backwards is the same convolution shape
     assert "Backward FLOPs: 7050625024" in r.stdout
     assert "Backward plan:" in r.stdout
+    assert "WU FLOPs: 7050625024" in r.stdout
+    assert "WU plan:" in r.stdout
+    # weight update: batch and input channels exchanged, 28x28 "kernel"
+    assert "kernelShape                {28,28}" in r.stdout
     assert "implicit GEMM" in r.stdout
     assert "inputPaddingLower          {1,1}" in r.stdout
 
@@ -52,7 +56,7 @@ def test_usage_errors_exit_1():
     assert run("--bogus").returncode == 1
     assert run("--input-channels", "1", "--output-channels", "1", "--field",
                "{4}", "--kernel-size", "1", "--single-phase",
-               "wu").returncode == 1
+               "sideways").returncode == 1
 
 
 # name, arguments: modelled on the reference's ctest entries

@@ -1,0 +1,262 @@
+"""Weight update pass: the gradient with respect to the forward weights,
+computed as the reference does - a forward convolution with
+getWeightUpdateParams (lib/poplin/Convolution.cpp:3390-3435) on activations
+and deltas with batch and channel axes exchanged (:3437-3483) - and checked
+against a restatement of poplibs_test::conv::weightUpdate
+(lib/poplibs_test/Convolution.cpp:724-898).
+
+What pins the weight update oracle without running reference code:
+  * ordinary parameters: torch autograd of conv1d/2d/3d in float64;
+  * every transform: the forward pass is linear in its weights, so
+    <conv(x, w), dz> == <w, weightDeltas(x, dz)> for any w, with the forward
+    oracle pinned elsewhere;
+and getWeightUpdateParams by the identity the reference relies on:
+  convolution(getWeightUpdateParams(p), swap(x), swap(dz)) == swap(dW).
+"""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import poplibs_amd as pa
+from helpers import make_params, random_params, rel_l2
+
+from test_backward import TORCH_CASES
+
+
+@pytest.mark.parametrize("kw", TORCH_CASES)
+def test_oracle_weight_deltas_match_torch_autograd(oracle, kw):
+    p = make_params(pa.FLOAT, **kw)
+    nd = len(p.inputFieldShape)
+    rng = np.random.default_rng(4)
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    x = rng.standard_normal((p.batchSize, G * Ci, *p.inputFieldShape))
+    w = rng.standard_normal((G, Co, Ci, *p.kernelShape))
+    it, kt, ot = p.inputTransform, p.kernelTransform, p.outputTransform
+    pads = []
+    for d in reversed(range(nd)):
+        pads += [it.paddingLower[d], it.paddingUpper[d]]
+    xp = torch.nn.functional.pad(torch.tensor(x), pads)
+    wt = torch.tensor(w.reshape(G * Co, Ci, *p.kernelShape),
+                      requires_grad=True)
+    bias = torch.zeros(G * Co, dtype=torch.float64, requires_grad=True)
+    conv = {1: torch.nn.functional.conv1d, 2: torch.nn.functional.conv2d,
+            3: torch.nn.functional.conv3d}[nd]
+    y = conv(xp, wt, bias, stride=tuple(ot.stride),
+             dilation=tuple(kt.dilation), groups=G)
+    dz = rng.standard_normal(tuple(y.shape))
+    y.backward(torch.tensor(dz))
+    dw, db = oracle.weight_deltas(p, x, dz, threads=3, with_bias=True)
+    np.testing.assert_allclose(
+        dw, wt.grad.numpy().reshape(G, Co, Ci, *p.kernelShape), atol=1e-11)
+    np.testing.assert_allclose(db, bias.grad.numpy(), atol=1e-11)
+    # the reference's model applies them as a gradient-descent step
+    w2, b2 = oracle.weight_update(p, 0.25, x, dz, w, np.ones(G * Co))
+    np.testing.assert_allclose(w2, w - 0.25 * dw, atol=1e-12)
+    np.testing.assert_allclose(b2, 1 - 0.25 * db, atol=1e-12)
+
+
+def _random_case(r, rng):
+    p = random_params(r)
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    x = rng.standard_normal((p.batchSize, G * Ci, *p.inputFieldShape))
+    w = rng.standard_normal((G, Co, Ci, *p.kernelShape))
+    dz = rng.standard_normal((p.batchSize, G * Co, *p.getOutputFieldShape()))
+    return p, x, w, dz
+
+
+def test_oracle_weight_deltas_are_the_adjoint_in_the_weights(oracle):
+    r, rng = random.Random(13), np.random.default_rng(13)
+    for _ in range(150):
+        p, x, w, dz = _random_case(r, rng)
+        lhs = np.vdot(oracle.convolution(p, x, w), dz)
+        rhs = np.vdot(w, oracle.weight_deltas(p, x, dz))
+        assert abs(lhs - rhs) <= 1e-9 * (1 + abs(lhs)), p
+
+
+def wu_operands(p, x, dz):
+    """Forward activations and deltas -> the weight update convolution's
+    activations [Ci][G*B][field] and weights [G][Co][B][outField]
+    (lib/poplin/Convolution.cpp:3459-3472)."""
+    G, Ci, Co, B = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                    p.outputChannelsPerConvGroup, p.batchSize)
+    field, out_field = tuple(p.inputFieldShape), tuple(p.getOutputFieldShape())
+    acts = x.reshape(B, G, Ci, *field)
+    acts = np.moveaxis(acts, (0, 1, 2), (2, 1, 0)).reshape(Ci, G * B, *field)
+    weights = dz.reshape(B, G, Co, *out_field)
+    weights = np.moveaxis(weights, (0, 1, 2), (2, 0, 1))
+    return np.ascontiguousarray(acts), np.ascontiguousarray(weights)
+
+
+def wu_result_to_weights(p, out):
+    """The weight update convolution's output [Ci][G*Co][kernel] -> weight
+    deltas [G][Co][Ci][kernel] (:3478-3482)."""
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    out = out.reshape(Ci, G, Co, *p.kernelShape)
+    return np.ascontiguousarray(np.moveaxis(out, (0, 1, 2), (2, 0, 1)))
+
+
+def test_weight_update_params_identity_and_canonical_form(oracle):
+    r, rng = random.Random(14), np.random.default_rng(14)
+    for _ in range(150):
+        p, x, _, dz = _random_case(r, rng)
+        wp = pa.getWeightUpdateParams(p)
+        assert wp == wp.canonicalize()
+        assert wp.getOutputFieldShape() == list(p.kernelShape)
+        assert wp.kernelShape == list(p.getOutputFieldShape())
+        assert wp.batchSize == p.inputChannelsPerConvGroup
+        assert wp.inputChannelsPerConvGroup == p.batchSize
+        assert wp.outputChannelsPerConvGroup == p.outputChannelsPerConvGroup
+        want = oracle.weight_deltas(p, x, dz)
+        acts, weights = wu_operands(p, x, dz)
+        got = wu_result_to_weights(p, oracle.convolution(wp, acts, weights))
+        np.testing.assert_allclose(got, want, atol=1e-10)
+
+
+def test_weight_update_params_known_answer():
+    # 3x3, stride 2, pad 1 on 8x8 -> 4x4: the deltas become a 4x4 kernel
+    # dilated by the stride, sliding over the padded activations with the
+    # forward kernel dilation (1) as stride; the last padding row is never
+    # reached, so the pass truncates it.
+    p = make_params(pa.HALF, batch=4, field=(8, 8), kernel=(3, 3), ci=16,
+                    co=32, stride=2, pad=1)
+    wp = pa.getWeightUpdateParams(p)
+    assert wp.batchSize == 16 and wp.inputChannelsPerConvGroup == 4
+    assert wp.outputChannelsPerConvGroup == 32
+    assert wp.inputFieldShape == [8, 8] and wp.kernelShape == [4, 4]
+    assert wp.kernelTransform.dilation == [2, 2]
+    assert wp.inputTransform.paddingLower == [1, 1]
+    assert wp.inputTransform.paddingUpper == [0, 0]
+    assert wp.outputTransform.stride == [1, 1]
+    assert wp.getOutputFieldShape() == [3, 3]
+
+
+# ---------------------------------------------------------------------------
+# GPU: the same pass through the C ABI.
+
+def run_weight_update(p, x_q, dz_q, options=None, weights_q=None, scale=None):
+    """x_q [B][G*Ci][field...], dz_q [B][G*Co][outField...] in the device
+    element type, external layout.  Returns the weight deltas (or, with
+    weights_q and scale, the updated weights) as float64 and the plan."""
+    from gpu_helpers import _TORCH_DTYPE, device
+    nd = len(p.inputFieldShape)
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    plan = pa.WeightUpdatePlan(p, options)
+    # channels-last device tensors
+    to_cl = (0, *range(2, 2 + nd), 1)
+    x = device(np.ascontiguousarray(x_q.transpose(to_cl)), p.inputType)
+    dz = device(np.ascontiguousarray(dz_q.transpose(to_cl)), p.inputType)
+    ws_bytes = plan.workspace_bytes()
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    if weights_q is None:
+        out = torch.empty((G, Co, Ci, *p.kernelShape),
+                          dtype=_TORCH_DTYPE[p.outputType], device="cuda:0")
+        plan.calculate_weight_deltas(dz.data_ptr(), x.data_ptr(),
+                                     out.data_ptr(), ws.data_ptr(), ws_bytes,
+                                     stream)
+    else:
+        out = device(weights_q, p.inputType)
+        plan.weight_update(dz.data_ptr(), out.data_ptr(), x.data_ptr(), scale,
+                           ws.data_ptr(), ws_bytes, stream)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().astype(np.float64), plan
+
+
+WU_GPU_CASES = [
+    dict(batch=4, field=(14, 14), kernel=(3, 3), ci=32, co=48, pad=1),
+    dict(batch=2, field=(9, 9), kernel=(1, 1), ci=40, co=24),
+    dict(batch=3, field=(9, 10), kernel=(3, 3), ci=8, co=16, stride=2, pad=1),
+    dict(batch=2, field=(12, 13), kernel=(3, 3), groups=16, pad=1),
+    dict(batch=5, field=(17,), kernel=(3,), ci=8, co=8, groups=2, kdil=2,
+         padLower=(2,), padUpper=(1,)),
+    dict(batch=16, field=(8, 8), kernel=(3, 3), ci=64, co=64, pad=1),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kw", WU_GPU_CASES)
+def test_weight_deltas_on_gpu_match_oracle(oracle, kw):
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    rng = np.random.default_rng(22)
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    xq, xd = quantize(
+        rng.standard_normal((p.batchSize, G * Ci, *p.inputFieldShape)), pa.HALF)
+    dq, dd = quantize(
+        rng.standard_normal((p.batchSize, G * Co, *p.getOutputFieldShape()))
+        * 0.1, pa.HALF)
+    got, plan = run_weight_update(p, xq, dq)
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= 1e-5, (rel_l2(got, want), plan.describe())
+
+
+@pytest.mark.gpu
+def test_weight_update_applies_scaled_deltas(oracle):
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, pa.HALF, batch=4, field=(10, 10), kernel=(3, 3),
+                    ci=16, co=32, pad=1)
+    rng = np.random.default_rng(23)
+    xq, xd = quantize(rng.standard_normal((4, 16, 10, 10)), pa.HALF)
+    dq, dd = quantize(rng.standard_normal((4, 32, 10, 10)) * 0.1, pa.HALF)
+    wq, wd = quantize(rng.standard_normal((1, 32, 16, 3, 3)), pa.HALF)
+    got, _ = run_weight_update(p, xq, dq, weights_q=wq, scale=-0.125)
+    want, _ = oracle.weight_update(p, 0.125, xd, dd, wd, np.zeros(32))
+    # deltas rounded to half, then the sum rounded to half
+    assert rel_l2(got, want) <= 2e-3, rel_l2(got, want)
+    # a float-output plan is refused: the deltas must have the weights' type
+    pf = make_params(pa.HALF, pa.FLOAT, batch=4, field=(10, 10), kernel=(3, 3),
+                     ci=16, co=32, pad=1)
+    with pytest.raises(pa.MxconvError) as e:
+        run_weight_update(pf, xq, dq, weights_q=wq, scale=1.0)
+    assert e.value.status == pa.Status.INVALID_PARAMS
+
+
+@pytest.mark.gpu
+def test_weight_update_random_params_on_gpu(oracle):
+    from gpu_helpers import quantize
+    r, rng = random.Random(32), np.random.default_rng(32)
+    for _ in range(25):
+        p, x, _, dz = _random_case(r, rng)
+        p = pa.ConvParams(pa.FLOAT, pa.FLOAT, p.batchSize, p.inputFieldShape,
+                          p.kernelShape, p.inputChannelsPerConvGroup,
+                          p.outputChannelsPerConvGroup, p.numConvGroups,
+                          p.inputTransform, p.kernelTransform,
+                          p.outputTransform)
+        xq, xd = quantize(x, pa.FLOAT)
+        dq, dd = quantize(dz, pa.FLOAT)
+        got, plan = run_weight_update(p, xq, dq)
+        want = oracle.weight_deltas(p, xd, dd)
+        assert got.shape == want.shape
+        if want.size:
+            assert rel_l2(got, want) <= 1e-5, (rel_l2(got, want), p)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,chans,dt,bt", [
+    (1, 1, pa.FLOAT, pa.FLOAT), (1000, 7, pa.HALF, pa.HALF),
+    (25088, 128, pa.HALF, pa.FLOAT), (300, 200, pa.FLOAT, pa.HALF),
+    (0, 5, pa.HALF, pa.HALF)])
+def test_bias_update_on_gpu(rows, chans, dt, bt):
+    from gpu_helpers import device, quantize
+    rng = np.random.default_rng(rows + chans)
+    zq, zd = quantize(rng.standard_normal((rows, chans)), dt)
+    bq, bd = quantize(rng.standard_normal(chans), bt)
+    z, b = device(zq, dt), device(bq, bt)
+    ws_bytes = pa.bias_update_workspace_bytes(rows, chans)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device="cuda:0")
+    pa.convolutionBiasUpdate(dt, z.data_ptr(), rows, chans, bt, b.data_ptr(),
+                             -0.5, ws.data_ptr(), ws_bytes)
+    torch.cuda.synchronize()
+    want = bd - 0.5 * zd.sum(axis=0)
+    got = b.cpu().numpy().astype(np.float64)
+    tol = 2e-3 if bt == pa.HALF else 1e-5
+    np.testing.assert_allclose(got, want, rtol=tol,
+                               atol=tol * max(1.0, np.abs(want).max()))

@@ -1,13 +1,14 @@
 // single_conv_layer - command-line harness for one convolution layer: the
-// forward pass and the backward-data pass.
+// forward, backward-data and weight update passes.
 //
 // Test infrastructure: it runs the convolutions through the C++ poplin layer
 // of this build (hence through the C ABI and the gfx950 kernels) and compares
 // the results with the CPU oracle (oracle/conv_oracle.c), exactly as PopLibs'
 // tools/single_conv_layer.cpp compares a device run with
-// poplibs_test::conv::convolution / convolutionBackward.  The forward- and
-// backward-pass subset of that tool's options is accepted under the same names (tools/single_conv_layer.cpp:
-// 171-430); the same data modes, comparison rule and exit codes apply:
+// poplibs_test::conv::convolution / convolutionBackward / weightUpdate.  That
+// tool's options are accepted under the same names
+// (tools/single_conv_layer.cpp:171-430); the same data modes, comparison rule
+// and exit codes apply:
 //   * +-1 "Bernoulli" data with zero tolerance when the sums stay exactly
 //     representable, else uniform random data with tolerances
 //     (tools/single_conv_layer.cpp:941-1005, lib/poplibs_test/Util.cpp:167-196)
@@ -48,6 +49,21 @@ int oracle_convolution(
     const unsigned *, const unsigned *, const unsigned *, unsigned, unsigned,
     unsigned, unsigned, const double *, const double *, const double *,
     double *, size_t, int);
+int oracle_weight_update(
+    unsigned num_field_dims, const unsigned *input_field_size,
+    const unsigned *truncation_lower, const unsigned *truncation_upper,
+    const unsigned *input_dilation, const unsigned *padding_lower,
+    const unsigned *padding_upper, const unsigned char *flip_input,
+    const unsigned *kernel_size, const unsigned *kernel_truncation_lower,
+    const unsigned *kernel_truncation_upper, const unsigned *kernel_dilation,
+    const unsigned *kernel_padding_lower, const unsigned *kernel_padding_upper,
+    const unsigned char *flip_kernel, const unsigned *output_truncation_lower,
+    const unsigned *output_truncation_upper, const unsigned *stride,
+    const unsigned *output_padding_lower, const unsigned *output_padding_upper,
+    unsigned batch_size, unsigned num_conv_groups, unsigned in_chans_per_group,
+    unsigned out_chans_per_group, const double *activations,
+    const double *deltas, double *weight_deltas, size_t weight_delta_elems,
+    double *bias_deltas, int threads);
 int oracle_convolution_backward(
     unsigned, const unsigned *, const unsigned *, const unsigned *,
     const unsigned *, const unsigned *, const unsigned *,
@@ -124,7 +140,7 @@ int main(int argc, char **argv) try {
       "output-truncation", "output-truncation-upper",
       "output-truncation-lower", "stride", "output-padding",
       "output-padding-upper", "output-padding-lower", "single-phase",
-      "inference-only", "bwd-plan-constraints",
+      "inference-only", "bwd-plan-constraints", "wu-plan-constraints",
       "plan-only", "inference-only", "tolerance", "absolute-tolerance",
       "batch-size", "conv-groups", "fwd-plan-constraints",
       "fwd-plan-constraints-file", "report-plan", "convolution-options",
@@ -147,17 +163,14 @@ int main(int argc, char **argv) try {
        {"input-channels", "output-channels", "field", "kernel-size"})
     if (!has(required))
       usage(std::string("the option '--") + required + "' is required");
-  // Passes (tools/single_conv_layer.cpp:723-735): forward and backward-data
-  // are provided; "all" runs both and says that the weight update is not.
+  // Passes (tools/single_conv_layer.cpp:715-735).
   const std::string phase = get("single-phase", "all");
-  if (phase != "fwd" && phase != "bwd" && phase != "all")
-    usage("--single-phase must be fwd, bwd or all (the weight-update pass is "
-          "not provided)");
+  if (phase != "fwd" && phase != "bwd" && phase != "wu" && phase != "all")
+    usage("--single-phase must be fwd, bwd, wu or all");
   const bool inferenceOnly = parseBool(get("inference-only", "false"));
   const bool doFwdPass = phase == "fwd" || phase == "all";
   const bool doBwdPass = !inferenceOnly && (phase == "bwd" || phase == "all");
-  if (phase == "all" && !inferenceOnly)
-    std::cout << "Weight-update pass not provided: running fwd and bwd\n";
+  bool doWuPass = !inferenceOnly && (phase == "wu" || phase == "all");
 
   // ---- parameters (tools/single_conv_layer.cpp:768-790) -------------------
   const Shape field = parseShape(get("field"));
@@ -212,6 +225,13 @@ int main(int argc, char **argv) try {
       std::stoul(get("output-channels")), std::stoul(get("conv-groups", "1")),
       inT, kT, outT);
   params.validate();
+  if (doWuPass && inputType == poplar::QUARTER) {
+    if (phase == "wu")
+      throw poputil::poplibs_error(
+          "the weight update pass takes half or float tensors");
+    std::cout << "Weight update pass skipped: it takes half or float tensors\n";
+    doWuPass = false;
+  }
 
   // ---- options (tools/single_conv_layer.cpp:803-832) ----------------------
   poplar::OptionFlags options;
@@ -245,6 +265,15 @@ int main(int argc, char **argv) try {
   else if (has("fwd-plan-constraints"))
     bwdOptions.set("planConstraints", "");
   poplin::convolutionValidateOptions(bwdOptions);
+  // Weight update: the forward options with pass TRAINING_WU
+  // (tools/single_conv_layer.cpp:821-824).
+  poplar::OptionFlags wuOptions = options;
+  wuOptions.set("pass", "TRAINING_WU");
+  if (has("wu-plan-constraints"))
+    wuOptions.set("planConstraints", get("wu-plan-constraints"));
+  else if (has("fwd-plan-constraints"))
+    wuOptions.set("planConstraints", "");
+  poplin::convolutionValidateOptions(wuOptions);
   const auto flops = poplin::getFwdFlops(params);
   poplin::PlanningCache cache;
   const bool reportPlan = parseBool(get("report-plan", "false")) || has("plan-only");
@@ -260,6 +289,13 @@ int main(int argc, char **argv) try {
     if (reportPlan) {
       std::cout << "Backward plan:\n";
       poplin::reportPlanInfo(std::cout, bwdParams, bwdOptions, &cache);
+    }
+  }
+  if (doWuPass) {
+    std::cout << "WU FLOPs: " << poplin::getWuFlops(params) << "\n";
+    if (reportPlan) {
+      std::cout << "WU plan:\n";
+      poplin::reportWeightUpdatePlanInfo(std::cout, params, wuOptions, &cache);
     }
   }
   if (has("plan-only"))
@@ -284,7 +320,12 @@ int main(int argc, char **argv) try {
                       : (outputType == poplar::FLOAT ? 1e-6 : 1e-5);
   const unsigned determinismChecks =
       unsigned(std::stoul(get("num-determinism-checks", "0")));
-  const size_t macsPerOut = outElems ? (flops / 2) / outElems : 0;
+  // The longest sum any pass forms (tools/single_conv_layer.cpp:941-975).
+  size_t macsPerOut = outElems ? (flops / 2) / outElems : 0;
+  if (doBwdPass && inElems)
+    macsPerOut = std::max<size_t>(macsPerOut, (flops / 2) / inElems);
+  if (doWuPass && wElems)
+    macsPerOut = std::max<size_t>(macsPerOut, (flops / 2) / wElems);
   const size_t maxInt = std::min(maxContiguousInteger(inputType),
                                  maxContiguousInteger(outputType));
   const bool uniformData = determinismChecks || macsPerOut > 10 * maxInt;
@@ -413,6 +454,47 @@ int main(int argc, char **argv) try {
                          bwdOptions, &cache);
     prog.synchronize();
   }
+  // Weight update: weights += -learningRate * deltas on a copy of the
+  // weights in the external layout, biases likewise
+  // (tools/single_conv_layer.cpp:1056-1094).
+  const double learningRate = uniformData ? 0.05 : 1.0;
+  std::vector<uint8_t> wuWeights(weightBytes.size()),
+      wuBiases(biasBytes.size());
+  if (doWuPass) {
+    std::vector<size_t> wShape{params.numConvGroups,
+                               params.outputChannelsPerConvGroup,
+                               params.inputChannelsPerConvGroup};
+    wShape.insert(wShape.end(), kernelShape.begin(), kernelShape.end());
+    poplin::DeviceTensor master(inputType, wShape,
+                                poplin::DeviceTensor::Layout::External,
+                                std::max<size_t>(weightBytes.size(), 1));
+    // The deltas are held the way a convolution leaves its output and the
+    // backward pass takes its input, whose shape and type they have.
+    auto zIn = poplin::createInput(bwdParams, bwdOptions, &cache);
+    if (!ignoreData) {
+      poplin::writeTensor(master, weightBytes.data(), prog);
+      poplin::writeTensor(zIn, zDeltaBytes.data(), prog, bwdParams, bwdOptions,
+                          &cache);
+      poplin::writeTensor(in, actBytes.data(), prog, params, options, &cache);
+    }
+    poplin::convolutionWeightUpdate(zIn, master, in, params,
+                                    float(-learningRate), prog, wuOptions,
+                                    &cache);
+    if (useBias) {
+      poplin::DeviceTensor b(outputType, {params.getNumOutputChans()},
+                             poplin::DeviceTensor::Layout::External,
+                             std::max<size_t>(biasBytes.size(), 1));
+      if (!ignoreData)
+        poplin::writeTensor(b, biasBytes.data(), prog);
+      poplin::convolutionBiasUpdate(zIn, b, float(-learningRate), options,
+                                    prog);
+      if (!ignoreData)
+        poplin::readTensor(b, wuBiases.data(), prog);
+    }
+    if (!ignoreData)
+      poplin::readTensor(master, wuWeights.data(), prog);
+    prog.synchronize();
+  }
   if (has("timing-runs") && doFwdPass) {
     const unsigned reps = unsigned(std::stoul(get("timing-runs")));
     auto out = poplin::createConvOutput(params, options, &cache);
@@ -468,13 +550,14 @@ int main(int argc, char **argv) try {
   zDeltas.push_back(0);
   // checkIsClose element by element, plus the relative L2 error.
   auto compare = [&](const char *name, const std::vector<uint8_t> &bytes,
-                     std::vector<double> &expected, size_t count) {
+                     std::vector<double> &expected, size_t count,
+                     poplar::Type type) {
     expected.resize(count);
-    // The host model's result is rounded to the output type before
+    // The host model's result is rounded to the tensor's type before
     // comparing, as the reference does when it copies the model output into
     // a typed buffer.
-    encode(expected, outputType, {});
-    const auto actual = decode(bytes, outputType);
+    encode(expected, type, {});
+    const auto actual = decode(bytes, type);
     unsigned mismatches = 0;
     double num = 0, den = 0;
     for (size_t i = 0; i != count; ++i) {
@@ -515,7 +598,7 @@ int main(int argc, char **argv) try {
       std::cerr << "host model failed with code " << rc << "\n";
       return 1;
     }
-    ok = compare("fwd", result, expected, outElems) && ok;
+    ok = compare("fwd", result, expected, outElems, outputType) && ok;
   }
   if (doBwdPass) {
     std::vector<double> expected(inElems + 1);
@@ -532,7 +615,36 @@ int main(int argc, char **argv) try {
       std::cerr << "host model (backward) failed with code " << rc << "\n";
       return 1;
     }
-    ok = compare("bwd", bwdResult, expected, inElems) && ok;
+    ok = compare("bwd", bwdResult, expected, inElems, outputType) && ok;
+  }
+  if (doWuPass) {
+    // tools/single_conv_layer.cpp:1270-1281, 1410-1436
+    std::vector<double> weightDeltas(wElems + 1),
+        biasDeltas(params.getNumOutputChans() + 1);
+    const int rc = oracle_weight_update(
+        unsigned(n), fs.data(), itl.data(), itu.data(), idl.data(), ipl.data(),
+        ipu.data(), fi.data(), ks.data(), ktl.data(), ktu.data(), kdl.data(),
+        kpl.data(), kpu.data(), fk.data(), otl.data(), otu.data(), ost.data(),
+        opl.data(), opu.data(), unsigned(params.batchSize),
+        unsigned(params.numConvGroups),
+        unsigned(params.inputChannelsPerConvGroup),
+        unsigned(params.outputChannelsPerConvGroup), acts.data(),
+        zDeltas.data(), weightDeltas.data(), wElems, biasDeltas.data(), 8);
+    if (rc != 0) {
+      std::cerr << "host model (weight update) failed with code " << rc << "\n";
+      return 1;
+    }
+    std::vector<double> modelWeights(wElems);
+    for (size_t i = 0; i != wElems; ++i)
+      modelWeights[i] = weights[i] + learningRate * -weightDeltas[i];
+    ok = compare("weights", wuWeights, modelWeights, wElems, inputType) && ok;
+    if (useBias) {
+      std::vector<double> modelBiases(params.getNumOutputChans());
+      for (size_t i = 0; i != modelBiases.size(); ++i)
+        modelBiases[i] = biases[i] + learningRate * -biasDeltas[i];
+      ok = compare("biases", wuBiases, modelBiases, modelBiases.size(),
+                   outputType) && ok;
+    }
   }
   if (!ok)
     return 1;
