@@ -294,6 +294,37 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
                                  void *out, void *workspace,
                                  size_t workspace_bytes, mxconv_stream stream);
 
+/* ---- several convolutions at once ---------------------------------------
+ * poplin::multiconv::convolution (include/poplin/MultiConvolution.hpp:
+ * 143-149): `n` independent forward passes, results as if each had been run
+ * by mxconv_fwd / mxconv_fwd_quarter.  PopLibs runs them side by side on
+ * disjoint tile ranges; here, with parallel != 0, they are spread over up to
+ * four HIP streams (the caller's and three of the library's, all at default
+ * priority) that fork from `stream` and join it again before the call
+ * returns, so small convolutions share the chip; with parallel == 0 they run
+ * on `stream` one after another.  Arrays have `n` entries; `bias`,
+ * `workspaces` / `workspace_bytes` and the two metadata arrays may be NULL
+ * (no bias, no workspace, metadata byte 0); metadata is read for plans with
+ * QUARTER inputs only.  Calls on one device are serialised internally. */
+mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
+                               const void *const *in,
+                               const uint8_t *in_metadata,
+                               const void *const *weights_packed,
+                               const uint8_t *weights_metadata,
+                               const void *const *bias, void *const *out,
+                               void *const *workspaces,
+                               const size_t *workspace_bytes, int parallel,
+                               mxconv_stream stream);
+
+/* Checks multi-convolution options (lib/poplin/ConvPlan.cpp:1929-1953):
+ * planType = parallel | serial, perConvReservedTiles (integer), cycleBackOff
+ * (number).  *parallel (may be NULL) receives 1 for planType parallel, the
+ * default, else 0; the other two steer the IPU tile split only. */
+mxconv_status mxconv_multiconv_validate_options(const char *const *keys,
+                                                const char *const *values,
+                                                size_t num_options,
+                                                int *parallel);
+
 /* ---- matrix multiplication on the same kernels --------------------------- */
 
 /* getConvParams of lib/poplin/MatMul.cpp:236-272: C[g] = A[g] * B[g] with A

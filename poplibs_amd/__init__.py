@@ -11,5 +11,6 @@ from .capi import (  # noqa: F401
     OutputTransform, Plan, Status, WeightUpdatePlan, add_bias,
     bias_update_workspace_bytes, build_library, convolutionBiasUpdate,
     getGradientParams, getWeightUpdateParams, lib, library_path, matMulParams,
-    matMulValidateOptions, quarter_metadata, scaled_add_to,
+    matMulValidateOptions, multi_fwd, multiconv_validate_options,
+    quarter_metadata, scaled_add_to,
     transposeGroupedMatrix, validate_options, weightsTransposeChansFlipXY)

@@ -175,6 +175,16 @@ def lib():
         "mxconv_fwd_quarter": (c_int, [c_void_p, c_void_p, c_uint8, c_void_p,
                                        c_uint8, c_void_p, c_void_p, c_void_p,
                                        c_size_t, c_void_p]),
+        "mxconv_multi_fwd": (c_int, [c_size_t, POINTER(c_void_p),
+                                     POINTER(c_void_p), POINTER(c_uint8),
+                                     POINTER(c_void_p), POINTER(c_uint8),
+                                     POINTER(c_void_p), POINTER(c_void_p),
+                                     POINTER(c_void_p), POINTER(c_size_t),
+                                     c_int, c_void_p]),
+        "mxconv_multiconv_validate_options": (c_int, [POINTER(c_char_p),
+                                                      POINTER(c_char_p),
+                                                      c_size_t,
+                                                      POINTER(c_int)]),
         "mxconv_matmul_params": (c_int, [c_int32, c_int32, c_uint64, c_uint64,
                                          c_uint64, c_uint64, P]),
         "mxconv_matmul_validate_options": (c_int, [POINTER(c_char_p),
@@ -688,6 +698,42 @@ def convolutionBiasUpdate(deltas_type, z_deltas, outer_elems, channels,
     _check(lib().mxconv_convolution_bias_update(
         deltas_type, z_deltas, outer_elems, channels, bias_type, biases, scale,
         workspace, workspace_bytes, stream))
+
+
+def multiconv_validate_options(options):
+    """Checks multi-convolution options; True for planType parallel."""
+    keys, values, n = _option_arrays(options)
+    parallel = c_int(1)
+    _check(lib().mxconv_multiconv_validate_options(keys, values, n,
+                                                   byref(parallel)))
+    return bool(parallel.value)
+
+
+def multi_fwd(plans, inputs, weights_packed, outputs, biases=None,
+              in_metadata=None, weights_metadata=None, workspaces=None,
+              workspace_bytes=None, parallel=True, stream=0):
+    """poplin::multiconv::convolution on device pointers: plans[i] run on
+    (inputs[i], weights_packed[i]) into outputs[i]."""
+    n = len(plans)
+
+    def pointers(values):
+        if values is None:
+            return None
+        return (c_void_p * max(n, 1))(*[v or None for v in values])
+
+    def bytes_(values):
+        if values is None:
+            return None
+        return (c_uint8 * max(n, 1))(*values)
+
+    sizes = None
+    if workspace_bytes is not None:
+        sizes = (c_size_t * max(n, 1))(*workspace_bytes)
+    _check(lib().mxconv_multi_fwd(
+        n, pointers([p._h.value for p in plans]), pointers(inputs),
+        bytes_(in_metadata), pointers(weights_packed),
+        bytes_(weights_metadata), pointers(biases), pointers(outputs),
+        pointers(workspaces), sizes, 1 if parallel else 0, stream))
 
 
 def getWeightUpdateParams(params):

@@ -15,6 +15,9 @@
 #include <cstring>
 #include <new>
 #include <sstream>
+#include <map>
+#include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -617,6 +620,157 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
   return forward(plan, in, weights_packed, bias, out, workspace,
                  workspace_bytes, quarterInfo(in_metadata, weights_metadata),
                  stream);
+}
+
+// ---- several convolutions at once -----------------------------------------
+
+} // extern "C"
+
+namespace {
+
+/// The library's worker streams and the events that fork them from, and join
+/// them to, a caller's stream; one set per device, made on first use and kept
+/// for the life of the process.
+struct WorkerStreams {
+  static constexpr int kWorkers = 3;
+  std::mutex mutex;
+  bool ready = false;
+  hipStream_t streams[kWorkers] = {};
+  hipEvent_t fork = nullptr, join[kWorkers] = {};
+};
+
+WorkerStreams *workerStreams(hipError_t *error) {
+  static std::mutex tableMutex;
+  static std::map<int, std::unique_ptr<WorkerStreams>> table;
+  int device = 0;
+  *error = hipGetDevice(&device);
+  if (*error != hipSuccess)
+    return nullptr;
+  std::lock_guard<std::mutex> lock(tableMutex);
+  auto &entry = table[device];
+  if (!entry)
+    entry.reset(new WorkerStreams);
+  if (!entry->ready) {
+    for (auto &s : entry->streams)
+      if ((*error = hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) !=
+          hipSuccess)
+        return nullptr;
+    if ((*error = hipEventCreateWithFlags(&entry->fork,
+                                          hipEventDisableTiming)) != hipSuccess)
+      return nullptr;
+    for (auto &e : entry->join)
+      if ((*error = hipEventCreateWithFlags(&e, hipEventDisableTiming)) !=
+          hipSuccess)
+        return nullptr;
+    entry->ready = true;
+  }
+  return entry.get();
+}
+
+} // namespace
+
+extern "C" {
+
+mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
+                               const void *const *in,
+                               const uint8_t *in_metadata,
+                               const void *const *weights_packed,
+                               const uint8_t *weights_metadata,
+                               const void *const *bias, void *const *out,
+                               void *const *workspaces,
+                               const size_t *workspace_bytes, int parallel,
+                               mxconv_stream stream) {
+  lastError.clear();
+  if (n == 0)
+    return MXCONV_OK;
+  REQUIRE_ARG(plans);
+  REQUIRE_ARG(in);
+  REQUIRE_ARG(weights_packed);
+  REQUIRE_ARG(out);
+  for (size_t i = 0; i != n; ++i)
+    REQUIRE_ARG(plans[i]);
+  auto launch = [&](size_t i, hipStream_t s) {
+    const mxk::QuarterInfo q =
+        plans[i]->params.inputType == poplar::QUARTER
+            ? quarterInfo(in_metadata ? in_metadata[i] : 0,
+                          weights_metadata ? weights_metadata[i] : 0)
+            : mxk::QuarterInfo{};
+    return forward(plans[i], in[i], weights_packed[i], bias ? bias[i] : nullptr,
+                   out[i], workspaces ? workspaces[i] : nullptr,
+                   workspace_bytes ? workspace_bytes[i] : 0, q,
+                   reinterpret_cast<mxconv_stream>(s));
+  };
+  hipStream_t main = reinterpret_cast<hipStream_t>(stream);
+  if (!parallel || n == 1) {
+    for (size_t i = 0; i != n; ++i) {
+      const mxconv_status st = launch(i, main);
+      if (st != MXCONV_OK)
+        return st;
+    }
+    return MXCONV_OK;
+  }
+  hipError_t e = hipSuccess;
+  WorkerStreams *w = workerStreams(&e);
+  if (!w)
+    return hipStatus(e, "worker stream set-up");
+  std::lock_guard<std::mutex> lock(w->mutex);
+  const size_t lanes = std::min<size_t>(n, WorkerStreams::kWorkers + 1);
+  // fork: the workers wait for what `stream` holds so far
+  if ((e = hipEventRecord(w->fork, main)) != hipSuccess)
+    return hipStatus(e, "multi-convolution fork");
+  for (size_t l = 1; l != lanes; ++l)
+    if ((e = hipStreamWaitEvent(w->streams[l - 1], w->fork, 0)) != hipSuccess)
+      return hipStatus(e, "multi-convolution fork");
+  mxconv_status result = MXCONV_OK;
+  for (size_t i = 0; i != n && result == MXCONV_OK; ++i) {
+    const size_t lane = i % lanes;
+    result = launch(i, lane == 0 ? main : w->streams[lane - 1]);
+  }
+  // join, also after a failed launch: `stream` waits for every worker
+  for (size_t l = 1; l != lanes; ++l) {
+    if ((e = hipEventRecord(w->join[l - 1], w->streams[l - 1])) != hipSuccess ||
+        (e = hipStreamWaitEvent(main, w->join[l - 1], 0)) != hipSuccess)
+      return hipStatus(e, "multi-convolution join");
+  }
+  return result;
+}
+
+mxconv_status mxconv_multiconv_validate_options(const char *const *keys,
+                                                const char *const *values,
+                                                size_t num_options,
+                                                int *parallel) {
+  return guarded([&] {
+    int isParallel = 1;
+    for (const auto &kv : collectOptions(keys, values, num_options)) {
+      const std::string &key = kv.first, &value = kv.second;
+      char *end = nullptr;
+      if (key == "planType") {
+        if (value != "parallel" && value != "serial")
+          throw poplar::invalid_option("Invalid value '" + value +
+                                       "' for option 'planType': must be "
+                                       "parallel or serial");
+        isParallel = value == "parallel";
+      } else if (key == "perConvReservedTiles") {
+        const long v = std::strtol(value.c_str(), &end, 10);
+        if (value.empty() || *end != '\0' || v < 0)
+          throw poplar::invalid_option(
+              "Invalid value '" + value +
+              "' for option 'perConvReservedTiles': must be a non-negative "
+              "integer");
+      } else if (key == "cycleBackOff") {
+        (void)std::strtod(value.c_str(), &end);
+        if (value.empty() || *end != '\0')
+          throw poplar::invalid_option("Invalid value '" + value +
+                                       "' for option 'cycleBackOff': must be "
+                                       "a number");
+      } else {
+        throw poplar::invalid_option("Unrecognised option '" + key + "'");
+      }
+    }
+    if (parallel)
+      *parallel = isParallel;
+    return MXCONV_OK;
+  });
 }
 
 // ---- matrix multiplication -------------------------------------------------

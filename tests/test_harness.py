@@ -277,3 +277,80 @@ GEMM_GPU_CASES = (
 def test_gemm_reference_cases(name, args):
     r = gemm(*args.split())
     assert r.returncode == 0, (name, r.stdout[-2000:], r.stderr[-2000:])
+
+
+# ---------------------------------------------------------------------------
+# multi_conv_layer: the reference's cases for its tool of that name
+# (tests/poplin/CMakeLists.txt:4019-4069), --conv arguments from the same JSON
+# documents.
+
+MULTI = os.path.join(ROOT, "tests", "tools", "multi_conv_layer")
+
+
+def _golden(name):
+    with open(os.path.join(ROOT, "tests", "golden", name)) as f:
+        return f.read()
+
+
+def multi(*args, timeout=120):
+    if not os.path.exists(MULTI):
+        subprocess.check_call(["make", "-C", os.path.dirname(MULTI)],
+                              stdout=subprocess.DEVNULL)
+    return subprocess.run([MULTI, *args], capture_output=True, text=True,
+                          timeout=timeout)
+
+
+def test_multi_conv_layer_plans_without_a_device():
+    r = multi("--conv", _golden("depthwise_conv_half.json"), "--conv",
+              _golden("pointwise_conv_float.json"), "--report-plan", "1",
+              "--compile-only")
+    assert r.returncode == 0, r.stderr
+    assert "got 2 convs" in r.stdout
+    assert r.stdout.count("Plan:") == 2
+    assert "depthwise direct" in r.stdout
+    r = multi("--conv", _golden("depthwise_conv_half.json"),
+              "--multiconv-options", '{"planType": "diagonal"}')
+    assert r.returncode == 1 and "planType" in r.stderr
+    assert multi("--conv", "{not json").returncode == 1
+
+
+MULTI_GPU_CASES = [
+    ("multi_conv_different_types",
+     ["depthwise_conv_half.json", "pointwise_conv_float.json"], []),
+    ("multi_conv_different_types_single_tile",
+     ["depthwise_conv_half.json", "depthwise_conv_half.json"],
+     ["--tiles-per-ipu", "1"]),
+    ("multi_conv_different_types_bwd",
+     ["depthwise_conv_half.json", "pointwise_reusable_conv_float.json"],
+     ["--bwd", "1", "--enable-convolution-reuse", "0"]),
+    ("multi_conv_different_types_bwd_reuse",
+     ["depthwise_conv_half.json", "pointwise_reusable_conv_float.json"],
+     ["--bwd", "1", "--enable-convolution-reuse", "1"]),
+    ("multi_conv_quarter_half_fwd",
+     ["depthwise_conv_quarter1.json", "depthwise_conv_quarter2.json"],
+     ["--bwd", "0"]),
+    ("multi_conv_quarter_half_bwd",
+     ["depthwise_conv_quarter1.json", "depthwise_conv_quarter2.json"],
+     ["--bwd", "1"]),
+    ("multi_conv_serial_five",
+     ["depthwise_conv_half.json", "pointwise_conv_float.json",
+      "pointwise_reusable_conv_float.json", "depthwise_conv_half.json",
+      "pointwise_conv_float.json"],
+     ["--multiconv-options", '{"planType": "serial"}']),
+    ("multi_conv_parallel_five",
+     ["depthwise_conv_half.json", "pointwise_conv_float.json",
+      "pointwise_reusable_conv_float.json", "depthwise_conv_half.json",
+      "pointwise_conv_float.json"], []),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,convs,extra", MULTI_GPU_CASES,
+                         ids=[c[0] for c in MULTI_GPU_CASES])
+def test_multi_conv_reference_cases(name, convs, extra):
+    args = []
+    for c in convs:
+        args += ["--conv", _golden(c)]
+    r = multi(*args, *extra)
+    assert r.returncode == 0, (name, r.stdout[-2000:], r.stderr[-2000:])
+    assert "Validation passed" in r.stdout

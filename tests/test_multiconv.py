@@ -1,0 +1,135 @@
+"""Several convolutions handed to the device together
+(poplin::multiconv::convolution, include/poplin/MultiConvolution.hpp:143-149):
+each result must be what the single-convolution entry point gives, whether the
+launches are spread over streams ("parallel") or run in order ("serial")."""
+import numpy as np
+import pytest
+
+import poplibs_amd as pa
+from poplibs_amd import capi
+from helpers import make_params, rel_l2
+
+
+def test_multiconv_options():
+    # lib/poplin/ConvPlan.cpp:1929-1953
+    assert pa.multiconv_validate_options({}) is True
+    assert pa.multiconv_validate_options({"planType": "serial"}) is False
+    assert pa.multiconv_validate_options(
+        {"planType": "parallel", "perConvReservedTiles": "50",
+         "cycleBackOff": "0.1"}) is True
+    for bad in ({"planType": "sideways"}, {"perConvReservedTiles": "many"},
+                {"perConvReservedTiles": "-1"}, {"cycleBackOff": "slow"},
+                {"partialsType": "half"}):
+        with pytest.raises(pa.MxconvError) as e:
+            pa.multiconv_validate_options(bad)
+        assert e.value.status == pa.Status.INVALID_OPTION, bad
+
+
+def test_multi_fwd_of_nothing_is_ok():
+    pa.multi_fwd([], [], [], [])
+
+
+MULTI_CASES = [
+    dict(batch=2, field=(14, 14), kernel=(3, 3), ci=32, co=32, pad=1),
+    dict(batch=1, field=(28, 28), kernel=(5, 5), groups=24),
+    dict(batch=2, field=(17, 32), kernel=(1, 1), ci=16, co=16),
+    dict(batch=3, field=(9, 10), kernel=(3, 3), ci=8, co=16, stride=2, pad=1),
+    dict(batch=2, field=(12, 12), kernel=(1, 1), ci=128, co=64),
+    dict(batch=0, field=(4, 4), kernel=(3, 3), ci=4, co=4),
+    dict(batch=1, field=(7,), kernel=(3,), ci=3, co=5, kdil=2),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("parallel", [True, False])
+def test_multi_fwd_equals_single_convolutions(oracle, parallel):
+    import torch
+    from gpu_helpers import _TORCH_DTYPE, device, quantize, run_conv
+    rng = np.random.default_rng(41)
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    plans, ins, ws, outs, keep, singles, params = [], [], [], [], [], [], []
+    for i, kw in enumerate(MULTI_CASES):
+        t = pa.FLOAT if i % 3 == 2 else pa.HALF
+        p = make_params(t, **kw)
+        G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                     p.outputChannelsPerConvGroup)
+        xq, _ = quantize(rng.standard_normal(
+            (p.batchSize, G * Ci, *p.inputFieldShape)), t)
+        wq, _ = quantize(rng.standard_normal(
+            (G, Co, Ci, *p.kernelShape)) * 0.1, t)
+        plan = pa.Plan(p)
+        singles.append(run_conv(p, xq, wq, plan=plan))
+
+        def buf(which):
+            return torch.empty(max(plan.buffer_bytes(which), 1),
+                               dtype=torch.uint8, device=dev)
+
+        x_ext, w_ext = device(xq, t), device(wq, t)
+        x_int, w_pack, o_int = (buf(capi.BUF_INPUT),
+                                buf(capi.BUF_WEIGHTS_PACKED),
+                                buf(capi.BUF_OUTPUT))
+        plan.acts_to_internal(x_ext.data_ptr(), x_int.data_ptr(), stream)
+        plan.pack_weights(w_ext.data_ptr(), w_pack.data_ptr(), stream)
+        plans.append(plan)
+        ins.append(x_int.data_ptr())
+        ws.append(w_pack.data_ptr())
+        outs.append(o_int.data_ptr())
+        keep += [x_ext, w_ext, x_int, w_pack, o_int]
+        params.append((p, o_int, t))
+    # twice, with work of the caller's stream in between: the fork and join
+    # events are reused from call to call
+    for _ in range(2):
+        pa.multi_fwd(plans, ins, ws, outs, parallel=parallel, stream=stream)
+        torch.cuda.synchronize()
+        for (p, o_int, t), plan, want in zip(params, plans, singles):
+            o_ext = torch.empty(
+                (p.batchSize, p.getNumOutputChans(), *p.getOutputFieldShape()),
+                dtype=_TORCH_DTYPE[t], device=dev)
+            plan.acts_to_external(o_int.data_ptr(), o_ext.data_ptr(), stream)
+            torch.cuda.synchronize()
+            got = o_ext.cpu().numpy().astype(np.float64)
+            np.testing.assert_array_equal(got, want)
+            o_int.zero_()
+
+
+@pytest.mark.gpu
+def test_multi_fwd_quarter_metadata(oracle):
+    import torch
+    from gpu_helpers import device, quantize, run_conv
+    rng = np.random.default_rng(42)
+    dev = torch.device("cuda:0")
+    p = make_params(pa.QUARTER, pa.HALF, batch=2, field=(8, 8), kernel=(3, 3),
+                    ci=32, co=16, pad=1)
+    metas = [(0x81, 0x02), (0x3f, 0x80)]   # (format, scale) pairs differ
+    plans, ins, ws, outs, keep, want = [], [], [], [], [], []
+    for in_meta, w_meta in metas:
+        xq, _ = quantize(rng.standard_normal((2, 32, 8, 8)), pa.QUARTER, oracle)
+        wq, _ = quantize(rng.standard_normal((1, 16, 32, 3, 3)) * 0.2,
+                         pa.QUARTER, oracle)
+        plan = pa.Plan(p)
+        want.append(run_conv(p, xq, wq, plan=plan, in_meta=in_meta,
+                             w_meta=w_meta))
+        x_ext, w_ext = device(xq, pa.QUARTER), device(wq, pa.QUARTER)
+        x_int = torch.empty(plan.buffer_bytes(capi.BUF_INPUT),
+                            dtype=torch.uint8, device=dev)
+        w_pack = torch.empty(plan.buffer_bytes(capi.BUF_WEIGHTS_PACKED),
+                             dtype=torch.uint8, device=dev)
+        o_int = torch.empty(plan.buffer_bytes(capi.BUF_OUTPUT),
+                            dtype=torch.uint8, device=dev)
+        plan.acts_to_internal(x_ext.data_ptr(), x_int.data_ptr())
+        plan.pack_weights(w_ext.data_ptr(), w_pack.data_ptr())
+        plans.append(plan)
+        ins.append(x_int.data_ptr())
+        ws.append(w_pack.data_ptr())
+        outs.append(o_int.data_ptr())
+        keep += [x_ext, w_ext, x_int, w_pack, o_int]
+    pa.multi_fwd(plans, ins, ws, outs, in_metadata=[m[0] for m in metas],
+                 weights_metadata=[m[1] for m in metas])
+    torch.cuda.synchronize()
+    for plan, o_ptr, w in zip(plans, outs, want):
+        o_ext = torch.empty((2, 16, 8, 8), dtype=torch.float16, device=dev)
+        plan.acts_to_external(o_ptr, o_ext.data_ptr())
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(o_ext.cpu().numpy().astype(np.float64),
+                                      w)

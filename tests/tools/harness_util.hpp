@@ -43,7 +43,7 @@ std::map<std::string, std::string> parseCommandLine(int argc, char **argv) {
   return opt;
 }
 
-poplar::Type parseType(const std::string &name) {
+inline poplar::Type parseType(const std::string &name) {
   if (name == "half")
     return poplar::HALF;
   if (name == "float")
@@ -53,7 +53,7 @@ poplar::Type parseType(const std::string &name) {
   usage("unknown type '" + name + "'");
 }
 
-bool parseBool(const std::string &v) {
+inline bool parseBool(const std::string &v) {
   return v == "1" || v == "true" || v == "TRUE" || v == "True";
 }
 
@@ -100,7 +100,7 @@ double fromHalfBits(uint16_t h) {
 }
 
 /// Rounds `values` to `type` in place and returns the device bytes.
-std::vector<uint8_t> encode(std::vector<double> &values, poplar::Type type,
+inline std::vector<uint8_t> encode(std::vector<double> &values, poplar::Type type,
                             const poplin::QuarterMetadata &md) {
   std::vector<uint8_t> bytes(values.size() * type.size());
   for (size_t i = 0; i != values.size(); ++i) {
@@ -123,7 +123,7 @@ std::vector<uint8_t> encode(std::vector<double> &values, poplar::Type type,
   return bytes;
 }
 
-std::vector<double> decode(const std::vector<uint8_t> &bytes,
+inline std::vector<double> decode(const std::vector<uint8_t> &bytes,
                            poplar::Type type) {
   std::vector<double> values(bytes.size() / type.size());
   for (size_t i = 0; i != values.size(); ++i) {
@@ -149,7 +149,7 @@ inline size_t maxContiguousInteger(poplar::Type t) {
 }
 
 /// lib/poplibs_test/Util.cpp:198-217 with boost's strong closeness test.
-bool isClose(double a, double b, double relTol) {
+inline bool isClose(double a, double b, double relTol) {
   if (a == b)
     return true;
   if (std::isnan(a) && std::isnan(b))
