@@ -62,15 +62,18 @@ __device__ __forceinline__ void storeOut(__half *p, size_t i, float v) {
 /// Division of a 31-bit number by a launch constant: one multiply-high and a
 /// shift (round-up method: mul = ceil(2^(31 + s) / d), s = ceil(log2 d)).
 struct FastDiv {
-  uint32_t mul, shift, one;
+  uint32_t mul, shift, one; // one: all bits set when the divisor is 1
   __device__ __forceinline__ uint32_t operator()(uint32_t n) const {
-    return one ? n : (__umulhi(n, mul) >> shift);
+    // a select written with bit operations: no branch, whatever the compiler
+    // knows about `one`
+    const uint32_t q = __umulhi(n, mul) >> shift;
+    return q ^ ((q ^ n) & one);
   }
 };
 
 inline FastDiv makeFastDiv(uint32_t d) {
   if (d <= 1)
-    return {0, 0, 1};
+    return {0, 0, 0xffffffffu};
   uint32_t s = 0;
   while ((1ull << s) < d)
     ++s;

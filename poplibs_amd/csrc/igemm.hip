@@ -46,6 +46,20 @@
 // zeros - no branch and no select on data.  When a k-step spans several
 // kernel taps (fewer than 128 bytes of channels per tap) the tap is per-lane
 // and the offsets are formed in vector registers.
+// Two more ways of addressing serve what the tap mask cannot.  A kernel of
+// more than 32 taps (a weight update pass: its "kernel" is a whole output
+// field) keeps, per row, the ranges of kernel rows and columns that read
+// inside the input - a window is valid on an interval of each - and tests
+// the tap against them.  A dilated (zero-stuffed) input (the backward pass of
+// a strided layer) keeps each row's image offset and window origin, and the
+// producers work out every tap's input position and validity arithmetically.
+// A producer wave gets few issue slots next to a consumer's MFMAs, so both
+// are written to need as few vector instructions per load as they can.
+//
+// Split K.  A convolution with few output tiles but a long K (a weight update
+// pass, a skinny matrix product) is cut along K into `splitK` parts, one
+// workgroup each; every part writes its fp32 partial tile to a workspace
+// [part][pixel][channel] and a second kernel adds the parts in order.
 //
 // Epilogue.  The accumulators are scaled, biased, converted and written to
 // LDS, then all 8 waves copy whole 16-byte vectors to the channels-last
@@ -81,7 +95,11 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   const uint32_t tile = xcdSwizzle(blockIdx.x, gridDim.x);
   const uint32_t nTile = tile % a.nTiles;
   const uint32_t mTile = (tile / a.nTiles) % a.mTiles;
-  const uint32_t g = tile / (a.nTiles * a.mTiles);
+  const uint32_t gs = tile / (a.nTiles * a.mTiles);
+  const uint32_t g = gs % d.groups;
+  const uint32_t part = gs / d.groups; // which part of K
+  out += size_t(part) * a.M * (d.groups * d.outChansPerGroup);
+  const uint32_t mode = a.mode;
 
   const int t = threadIdx.x;
   const bool producer = t >= kThreads - kProducers; // waves 4-7
@@ -95,6 +113,9 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   floatx16 acc[2][TN];
 
   if (producer) {
+    // The producers' address arithmetic shares each SIMD's issue port with a
+    // consumer's MFMAs: let their (short) vector instructions go first.
+    __builtin_amdgcn_s_setprio(3);
     const int pt = t - (kThreads - kProducers);
     const int pw = pt >> 6; // producer wave
     // Lane l of a load fills row position (l >> 3) of an 8-row block at chunk
@@ -108,9 +129,12 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
     // that the per-row offset below is never negative: the buffer unit adds
     // the vector and scalar offsets without wrapping.  Nothing in front of
     // the tensor is ever read (such taps are masked).
-    const uint32_t shift = (uint32_t(d.padH > 0 ? d.padH : 0) * d.inW +
-                            uint32_t(d.padW > 0 ? d.padW : 0)) *
-                           pixelBytes;
+    const uint32_t shift =
+        mode == kDilatedTaps
+            ? 0u
+            : (uint32_t(d.padH > 0 ? d.padH : 0) * d.inW +
+               uint32_t(d.padW > 0 ? d.padW : 0)) *
+                  pixelBytes;
     const __amdgpu_buffer_rsrc_t inBuf =
         bufferOf(in - shift, a.inBytes + shift);
     const __amdgpu_buffer_rsrc_t wBuf = bufferOf(w, a.wBytes);
@@ -122,22 +146,8 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
     // tap reads inside the input - read from the row table further down, once
     // the weight loads, which need none of it, are on their way.
     uint32_t rowOff[AROWS], tapMask[AROWS];
-
-    // Position inside K of the data loaded next.  UNI: (tap, byte offset of
-    // the channel block inside the tap) of the whole k-step, wave-uniform.
-    // Otherwise the same pair for this thread's own 16-byte chunk.
-    uint32_t tap = 0, kh = 0, kw = 0, ciOff = UNI ? 0 : chunk * 16;
-    auto normalise = [&] {
-      while (ciOff >= ciBytes) {
-        ciOff -= ciBytes;
-        ++tap;
-        if (++kw == d.kW) {
-          kw = 0;
-          ++kh;
-        }
-      }
-    };
-    normalise();
+    int originW[AROWS];                       // dilated input only
+    uint32_t khLo[AROWS], khSpan[AROWS], kwLo[AROWS], kwSpan[AROWS]; // ranges
 
     uint32_t bOff[BROWS];
 #pragma unroll
@@ -146,29 +156,10 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
                      a.kPadded) *
                     EB +
                 chunk * 16;
-    uint32_t kByte = 0; // byte offset of the next k-step along a B row
-
-    // Issue the A / B loads of the next k-step into LDS stage `stage` and
-    // move on along K.  Beyond the last k-step every offset is out of range:
-    // the stage is filled with zeros that are never multiplied.
-    auto loadA = [&](uint32_t stage) {
-      char *base = lds + stage * kTileBytes + pw * kLoadBytes;
-      const uint32_t tapOff = (kh * d.dilH * d.inW + kw * d.dilW) * pixelBytes;
-      const uint32_t tapBit = tap < taps ? (1u << tap) : 0u;
-#pragma unroll
-      for (int r = 0; r != AROWS; ++r) {
-        const bool ok = (tapMask[r] & tapBit) != 0;
-        LdsPtr dst = (LdsPtr)(base + r * 4 * kLoadBytes);
-        if constexpr (UNI)
-          loadToLds(inBuf, dst, ok ? rowOff[r] : kOutOfRange, tapOff + ciOff);
-        else
-          loadToLds(inBuf, dst,
-                    ok ? rowOff[r] - chunk * 16 + tapOff + ciOff : kOutOfRange,
-                    0);
-      }
-      ciOff += kRowBytes;
-      normalise();
-    };
+    // Byte offset of the next k-step along a row of the packed weights; this
+    // part of K starts kStart bytes in.
+    const uint32_t kStart = part * a.kSteps * kRowBytes;
+    uint32_t kByte = kStart;
     auto loadB = [&](uint32_t stage) {
       char *base = lds + stage * kTileBytes + pw * kLoadBytes;
       const uint32_t kOff = kByte < a.kPadded * EB ? kByte : kOutOfRange;
@@ -180,36 +171,154 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
       kByte += kRowBytes;
     };
 
-    // NS - 1 k-steps in flight; wait for the oldest before each barrier.
-    // Start-up order: all weight loads, then (row table ready) all input
-    // loads; from then on input and weight loads of one k-step together.
+    // The whole schedule, written once for both ways of addressing the input
+    // (a compile-time choice inside, so that neither loop carries the other's
+    // branches).  NS - 1 k-steps are in flight; the oldest is waited for
+    // before each barrier.  Start-up order: all weight loads, then (row table
+    // ready) all input loads; from then on input and weight loads of one
+    // k-step together.
+    auto produce = [&](auto modeTag) {
+      constexpr int MODE = decltype(modeTag)::value;
+      constexpr bool GEN = MODE == kDilatedTaps;
+      // Position inside K of the input data loaded next.  UNI: (tap, byte
+      // offset of the channel block inside the tap) of the whole k-step,
+      // wave-uniform.  Otherwise the same pair for this thread's own 16-byte
+      // chunk.
+      uint32_t aByte = kStart + (UNI ? 0 : chunk * 16);
+      uint32_t tap = aByte / ciBytes;
+      uint32_t ciOff = aByte - tap * ciBytes;
+      uint32_t kh = tap / d.kW, kw = tap - kh * d.kW;
+      auto advance = [&] {
+        if constexpr (GEN) {
+          // no loop, no branch: everything again from the byte position
+          aByte += kRowBytes;
+          tap = a.divCiBytes(aByte);
+          ciOff = aByte - tap * ciBytes;
+          kh = a.divKW(tap);
+          kw = tap - kh * d.kW;
+        } else {
+          ciOff += kRowBytes;
+          while (ciOff >= ciBytes) {
+            ciOff -= ciBytes;
+            ++tap;
+            if (++kw == d.kW) {
+              kw = 0;
+              ++kh;
+            }
+          }
+        }
+      };
+      auto loadA = [&](uint32_t stage) {
+        char *base = lds + stage * kTileBytes + pw * kLoadBytes;
+        if constexpr (GEN) {
+          // rowOff: the row's image and group; tapMask / originW: its window
+          // origin (row, column) in zero-stuffed input coordinates.  The tap
+          // reads input (origin + tap * dilation) / input dilation when that
+          // is whole and inside [lo, hi).  A producer wave gets to issue a
+          // vector instruction only every few cycles and pays dearly for a
+          // taken branch, so this is straight-line code: selects, 24-bit
+          // multiplies (the launcher checks the ranges), and the division by
+          // the input dilation also when that is 1.
+          const int khd = int(kh * d.dilH), kwd = int(kw * d.dilW);
+          const uint32_t tapOk = tap < taps ? 1u : 0u;
+          const uint32_t lane16 = ciOff + (UNI ? chunk * 16 : 0) - chunk * 16;
+          const uint32_t rowBytes = d.inW * pixelBytes;
+          const uint32_t spanH = d.hiH - d.loH, spanW = d.hiW - d.loW;
+          // One step of the computation for all rows before the next one:
+          // a lone wave waits several cycles for a result it has just
+          // issued, so neighbouring instructions should not depend on each
+          // other.
+          int ihD[AROWS], iwD[AROWS];
+          uint32_t ih[AROWS], iw[AROWS], ok[AROWS], off[AROWS];
+#pragma unroll
+          for (int r = 0; r != AROWS; ++r) {
+            ihD[r] = int(tapMask[r]) + khd;
+            iwD[r] = originW[r] + kwd;
+          }
+#pragma unroll
+          for (int r = 0; r != AROWS; ++r) {
+            ih[r] = a.divInDilH(uint32_t(ihD[r]));
+            iw[r] = a.divInDilW(uint32_t(iwD[r]));
+          }
+#pragma unroll
+          for (int r = 0; r != AROWS; ++r)
+            ok[r] = tapOk & uint32_t((ihD[r] | iwD[r]) >= 0) &
+                    uint32_t(__umul24(ih[r], d.inDilH) == uint32_t(ihD[r])) &
+                    uint32_t(__umul24(iw[r], d.inDilW) == uint32_t(iwD[r])) &
+                    uint32_t(ih[r] - d.loH < spanH) &
+                    uint32_t(iw[r] - d.loW < spanW);
+#pragma unroll
+          for (int r = 0; r != AROWS; ++r)
+            off[r] = rowOff[r] + __umul24(ih[r], rowBytes) +
+                     __umul24(iw[r], pixelBytes) + lane16;
+#pragma unroll
+          for (int r = 0; r != AROWS; ++r) {
+            LdsPtr dst = (LdsPtr)(base + r * 4 * kLoadBytes);
+            loadToLds(inBuf, dst, ok[r] ? off[r] : kOutOfRange, 0);
+          }
+        } else {
+          const uint32_t tapOff =
+              (kh * d.dilH * d.inW + kw * d.dilW) * pixelBytes;
+          const uint32_t tapBit = tap < taps ? (1u << (tap & 31)) : 0u;
+#pragma unroll
+          for (int r = 0; r != AROWS; ++r) {
+            bool ok;
+            if constexpr (MODE == kRangeTaps)
+              ok = (tap < taps) & (kh - khLo[r] < khSpan[r]) &
+                   (kw - kwLo[r] < kwSpan[r]);
+            else
+              ok = (tapMask[r] & tapBit) != 0;
+            LdsPtr dst = (LdsPtr)(base + r * 4 * kLoadBytes);
+            if constexpr (UNI)
+              loadToLds(inBuf, dst, ok ? rowOff[r] : kOutOfRange,
+                        tapOff + ciOff);
+            else
+              loadToLds(inBuf, dst,
+                        ok ? rowOff[r] - chunk * 16 + tapOff + ciOff
+                           : kOutOfRange,
+                        0);
+          }
+        }
+        advance();
+      };
+#pragma unroll
+      for (int r = 0; r != AROWS; ++r) {
+        const uint2 e = rowTable[(r * 4 + pw) * 8 + rowInBlock];
+        rowOff[r] = e.x + chunk * 16;
+        tapMask[r] = GEN ? uint32_t(int(e.y >> 16) - 32768) : e.y;
+        originW[r] = int(e.y & 0xffffu) - 32768;
+        khLo[r] = e.y & 0xffu, khSpan[r] = (e.y >> 8) & 0xffu;
+        kwLo[r] = (e.y >> 16) & 0xffu, kwSpan[r] = e.y >> 24;
+      }
+#pragma unroll
+      for (int s = 0; s != NS - 1; ++s)
+        loadA(s);
+      MXK_WAIT_VMCNT((NS - 2) * AROWS);
+      stepBarrier(); // barrier 0: step 0 is in LDS stage 0
+      for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
+        // Stage (kt - 1) % NS was multiplied before the last barrier: refill
+        // it with step kt + NS - 1, then make sure step kt + 1 has landed.
+        // The first time round the start-up order still shows in the queue.
+        loadA((kt + NS - 1) % NS);
+        loadB((kt + NS - 1) % NS);
+        if (kt == 0)
+          MXK_WAIT_VMCNT((NS - 3) * AROWS + kLoads);
+        else
+          MXK_WAIT_VMCNT((NS - 2) * kLoads);
+        stepBarrier(); // barrier kt + 1
+      }
+    };
+
 #pragma unroll
     for (int s = 0; s != NS - 1; ++s)
       loadB(s);
     stepBarrier(); // the row table is complete
-#pragma unroll
-    for (int r = 0; r != AROWS; ++r) {
-      const uint2 e = rowTable[(r * 4 + pw) * 8 + rowInBlock];
-      rowOff[r] = e.x + chunk * 16;
-      tapMask[r] = e.y;
-    }
-#pragma unroll
-    for (int s = 0; s != NS - 1; ++s)
-      loadA(s);
-    MXK_WAIT_VMCNT((NS - 2) * AROWS);
-    stepBarrier(); // barrier 0: step 0 is in LDS stage 0
-    for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
-      // Stage (kt - 1) % NS was multiplied before the last barrier: refill it
-      // with step kt + NS - 1, then make sure step kt + 1 has landed.  The
-      // first time round the start-up order still shows in the queue.
-      loadA((kt + NS - 1) % NS);
-      loadB((kt + NS - 1) % NS);
-      if (kt == 0)
-        MXK_WAIT_VMCNT((NS - 3) * AROWS + kLoads);
-      else
-        MXK_WAIT_VMCNT((NS - 2) * kLoads);
-      stepBarrier(); // barrier kt + 1
-    }
+    if (mode == kDilatedTaps)
+      produce(std::integral_constant<int, kDilatedTaps>{});
+    else if (mode == kRangeTaps)
+      produce(std::integral_constant<int, kRangeTaps>{});
+    else
+      produce(std::integral_constant<int, kMaskTaps>{});
     MXK_WAIT_VMCNT(0); // the trailing zero loads, before LDS is reused
   } else {
     // While the producers start the weight loads, the first 128 consumer
@@ -227,23 +336,56 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
       const uint32_t shift = (uint32_t(d.padH > 0 ? d.padH : 0) * d.inW +
                               uint32_t(d.padW > 0 ? d.padW : 0)) *
                              pixelBytes;
-      uint32_t kwMask = 0, mask = 0;
-      for (uint32_t kw = 0; kw != d.kW; ++kw) {
-        const int iw = iwBase + int(kw * d.dilW);
-        if (iw >= int(d.loW) && iw < int(d.hiW))
-          kwMask |= 1u << kw;
+      if (mode == kDilatedTaps) {
+        // An invalid row gets the origin (-32768, -32768): no tap of it is
+        // ever inside the input.
+        rowTable[t] = uint2{
+            b * d.inH * d.inW * pixelBytes + g * ciBytes,
+            rowValid ? (uint32_t(ihBase + 32768) << 16) |
+                           uint32_t(iwBase + 32768)
+                     : 0u};
+      } else if (mode == kRangeTaps) {
+        // Kernel rows kh with lo <= base + kh * dilation < hi form an
+        // interval; so do the columns.  {first, length} of each, 8 bits a
+        // piece; an invalid row gets empty ones.
+        auto range = [](int base, int lo, int hi, int dil, int size) {
+          auto ceilDiv = [](int n, int dv) {
+            return n >= 0 ? (n + dv - 1) / dv : -((-n) / dv);
+          };
+          int first = ceilDiv(lo - base, dil), last = ceilDiv(hi - base, dil);
+          first = first < 0 ? 0 : first > size ? size : first;
+          last = last < first ? first : last > size ? size : last;
+          return uint32_t(first) | (uint32_t(last - first) << 8);
+        };
+        const uint32_t ranges =
+            range(ihBase, int(d.loH), int(d.hiH), int(d.dilH), int(d.kH)) |
+            (range(iwBase, int(d.loW), int(d.hiW), int(d.dilW), int(d.kW))
+             << 16);
+        rowTable[t] = uint2{
+            shift +
+                ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
+                    pixelBytes +
+                g * ciBytes,
+            rowValid ? ranges : 0u};
+      } else {
+        uint32_t kwMask = 0, mask = 0;
+        for (uint32_t kw = 0; kw != d.kW; ++kw) {
+          const int iw = iwBase + int(kw * d.dilW);
+          if (iw >= int(d.loW) && iw < int(d.hiW))
+            kwMask |= 1u << kw;
+        }
+        for (uint32_t kh = 0; kh != d.kH; ++kh) {
+          const int ih = ihBase + int(kh * d.dilH);
+          if (ih >= int(d.loH) && ih < int(d.hiH))
+            mask |= kwMask << (kh * d.kW);
+        }
+        rowTable[t] = uint2{
+            shift +
+                ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
+                    pixelBytes +
+                g * ciBytes,
+            rowValid ? mask : 0u};
       }
-      for (uint32_t kh = 0; kh != d.kH; ++kh) {
-        const int ih = ihBase + int(kh * d.dilH);
-        if (ih >= int(d.loH) && ih < int(d.hiH))
-          mask |= kwMask << (kh * d.kW);
-      }
-      rowTable[t] = uint2{
-          shift +
-              ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
-                  pixelBytes +
-              g * ciBytes,
-          rowValid ? mask : 0u};
     }
     MXK_WAIT_LGKMCNT0();
     stepBarrier(); // the row table is complete
@@ -315,7 +457,8 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
 template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
 hipError_t run(const IgemmArgs &a, const void *in, const void *w,
                const void *bias, void *out, float scale, hipStream_t stream) {
-  const uint64_t blocks = uint64_t(a.mTiles) * a.nTiles * a.d.groups;
+  const uint64_t blocks =
+      uint64_t(a.mTiles) * a.nTiles * a.d.groups * a.d.splitK;
   if (blocks == 0)
     return hipSuccess;
   if (blocks > 0x7fffffffull)
@@ -378,21 +521,103 @@ hipError_t runType(const IgemmArgs &a, int inType, int outType, const void *in,
   return runOut<BN, 1, 1, 1>(a, outType, in, w, bias, out, q.scale, stream);
 }
 
+/// out[i] = sum over parts of partial[part][i] (+ bias of i's channel).  The
+/// parts are added in a fixed order: four interleaved running sums (so that
+/// four loads are in flight per lane), combined at the end.
+template <class OutT>
+__global__ __launch_bounds__(64) void splitKReduceKernel(
+    const float *__restrict__ partial, uint32_t parts, uint64_t elems,
+    uint32_t channels, const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  const uint64_t i = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  if (i >= elems)
+    return;
+  // elems and channels are multiples of 4 (checked by the launcher)
+  float4 sum[4] = {};
+  uint32_t p = 0;
+  for (; p + 4 <= parts; p += 4) {
+#pragma unroll
+    for (int u = 0; u != 4; ++u) {
+      const float4 v = *reinterpret_cast<const float4 *>(
+          partial + uint64_t(p + u) * elems + i);
+      sum[u].x += v.x, sum[u].y += v.y, sum[u].z += v.z, sum[u].w += v.w;
+    }
+  }
+  for (; p != parts; ++p) {
+    const float4 v =
+        *reinterpret_cast<const float4 *>(partial + uint64_t(p) * elems + i);
+    sum[0].x += v.x, sum[0].y += v.y, sum[0].z += v.z, sum[0].w += v.w;
+  }
+  float v[4] = {(sum[0].x + sum[1].x) + (sum[2].x + sum[3].x),
+                (sum[0].y + sum[1].y) + (sum[2].y + sum[3].y),
+                (sum[0].z + sum[1].z) + (sum[2].z + sum[3].z),
+                (sum[0].w + sum[1].w) + (sum[2].w + sum[3].w)};
+  if (bias) {
+    const uint32_t c = uint32_t(i % channels);
+#pragma unroll
+    for (int e = 0; e != 4; ++e)
+      v[e] += Load<OutT>::at(bias, c + e, 0);
+  }
+  storeOut4(out + i, v);
+}
+
 } // namespace
+
+int igemmTapAddressing(const IgemmDesc &d) {
+  if (d.inDilH != 1 || d.inDilW != 1)
+    return kDilatedTaps;
+  return d.kH * d.kW > 32 ? kRangeTaps : kMaskTaps;
+}
+
+size_t igemmWorkspaceBytes(const IgemmDesc &d) {
+  if (d.splitK <= 1)
+    return 0;
+  return size_t(d.splitK) * d.batch * d.outH * d.outW * d.groups *
+         d.outChansPerGroup * sizeof(float);
+}
 
 hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
                        const void *in, const void *weightsPacked,
-                       const void *bias, void *out, const QuarterInfo &q,
-                       hipStream_t stream) {
+                       const void *bias, void *out, void *workspace,
+                       const QuarterInfo &q, hipStream_t stream) {
   const uint32_t eb = inType == kHalf ? 2 : 1;
   const uint32_t bke = kRowBytes / eb;
+  const int mode = igemmTapAddressing(d);
+  const bool general = mode == kDilatedTaps;
   // The shapes the kernel is compiled for; the planner only produces these.
   if (d.blockM != kBlockM || (d.blockN != 64 && d.blockN != 128) ||
       d.blockK != bke || d.inChansPerGroup % (16 / eb) != 0 ||
-      (inType != kHalf && inType != kQuarter) || d.kH * d.kW > 32)
+      (inType != kHalf && inType != kQuarter) || d.splitK == 0 ||
+      d.inDilH == 0 || d.inDilW == 0)
+    return hipErrorInvalidValue;
+  // The general addressing keeps window origins as 16-bit offsets from
+  // -32768 and never reaches a tap beyond +32767 of them.
+  if (general &&
+      (uint64_t(d.outH) * d.strideH + uint64_t(d.kH) * d.dilH +
+               uint64_t(d.padH > 0 ? d.padH : -d.padH) >=
+           32768 ||
+       uint64_t(d.outW) * d.strideW + uint64_t(d.kW) * d.dilW +
+               uint64_t(d.padW > 0 ? d.padW : -d.padW) >=
+           32768))
+    return hipErrorInvalidValue;
+  if (d.splitK > 1 &&
+      (!workspace || (d.groups * d.outChansPerGroup) % 4 != 0))
     return hipErrorInvalidValue;
   IgemmArgs a;
   a.d = d;
+  a.mode = uint32_t(mode);
+  // the ranges of valid kernel rows and columns are kept in 8 bits each
+  if (mode == kRangeTaps && (d.kH > 255 || d.kW > 255))
+    return hipErrorInvalidValue;
+  // its multiplications are 24-bit ones
+  if (general && (uint64_t(d.inW) * d.groups * d.inChansPerGroup * eb >=
+                      (1u << 24) ||
+                  d.inH >= (1u << 24) || d.inDilH >= (1u << 24) ||
+                  d.inDilW >= (1u << 24)))
+    return hipErrorInvalidValue;
+  a.divInDilH = makeFastDiv(d.inDilH);
+  a.divInDilW = makeFastDiv(d.inDilW);
+  a.divCiBytes = makeFastDiv(d.inChansPerGroup * eb);
+  a.divKW = makeFastDiv(d.kW);
   const uint64_t m = uint64_t(d.batch) * d.outH * d.outW;
   if (m > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
@@ -404,7 +629,8 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
   a.coPadded = a.nTiles * d.blockN;
   const uint32_t k = d.kH * d.kW * d.inChansPerGroup;
   a.kPadded = (k + bke - 1) / bke * bke;
-  a.kSteps = a.kPadded / bke;
+  // every part runs the same number of k-steps; steps beyond K load zeros
+  a.kSteps = (a.kPadded / bke + d.splitK - 1) / d.splitK;
   // Buffer addressing is 32-bit; the planner keeps larger tensors away.
   const uint64_t inBytes =
       uint64_t(d.batch) * d.inH * d.inW * d.groups * d.inChansPerGroup * eb;
@@ -416,11 +642,43 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
     return hipErrorInvalidConfiguration;
   a.inBytes = uint32_t(inBytes);
   a.wBytes = uint32_t(wBytes);
-  if (d.blockN == 128)
-    return runType<128>(a, inType, outType, in, weightsPacked, bias, out, q,
-                        stream);
-  return runType<64>(a, inType, outType, in, weightsPacked, bias, out, q,
-                     stream);
+  if (d.splitK == 1) {
+    if (d.blockN == 128)
+      return runType<128>(a, inType, outType, in, weightsPacked, bias, out, q,
+                          stream);
+    return runType<64>(a, inType, outType, in, weightsPacked, bias, out, q,
+                       stream);
+  }
+  // fp32 partial tiles per part (scaled, without bias), then their sum.
+  const hipError_t e =
+      d.blockN == 128
+          ? runType<128>(a, inType, kFloat, in, weightsPacked, nullptr,
+                         workspace, q, stream)
+          : runType<64>(a, inType, kFloat, in, weightsPacked, nullptr,
+                        workspace, q, stream);
+  if (e != hipSuccess)
+    return e;
+  const uint32_t channels = d.groups * d.outChansPerGroup;
+  const uint64_t elems = uint64_t(a.M) * channels;
+  if (elems == 0)
+    return hipSuccess;
+  const uint64_t blocks = (elems / 4 + 63) / 64;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const float *partial = static_cast<const float *>(workspace);
+  if (outType == kHalf)
+    hipLaunchKernelGGL(splitKReduceKernel<__half>, dim3(uint32_t(blocks)),
+                       dim3(64), 0, stream, partial, d.splitK, elems,
+                       channels, static_cast<const __half *>(bias),
+                       static_cast<__half *>(out));
+  else if (outType == kFloat)
+    hipLaunchKernelGGL(splitKReduceKernel<float>, dim3(uint32_t(blocks)),
+                       dim3(64), 0, stream, partial, d.splitK, elems,
+                       channels, static_cast<const float *>(bias),
+                       static_cast<float *>(out));
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
 }
 
 } // namespace mxk

@@ -13,9 +13,12 @@ namespace mxk {
 struct IgemmArgs {
   IgemmDesc d;
   FastDiv divOutW, divOutH;
+  FastDiv divInDilH, divInDilW;
+  FastDiv divCiBytes, divKW; // by bytes of K per tap; by kernel width
+  uint32_t mode;     // kMaskTaps, kRangeTaps or kDilatedTaps
   uint32_t M;        // batch * outH * outW
   uint32_t mTiles, nTiles;
-  uint32_t kSteps;   // kPadded / elements per k-step
+  uint32_t kSteps;   // k-steps each workgroup runs (one part of K)
   uint32_t kPadded;  // row length of the packed weights, in elements
   uint32_t coPadded; // rows per group of the packed weights
   uint32_t inBytes;  // size of the input tensor

@@ -52,6 +52,20 @@ hipError_t launchGeneric(const GenericDesc &d, int inType, int outType,
 hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
                           const int perm[4], int elemBytes, hipStream_t stream);
 
+/// dst[g * strideG + c * strideC + p * strideP + b] = src[b][p][g][c]
+/// (strides in elements; elements of 2 or 4 bytes): channels-last activations
+/// with the batch axis moved innermost, as the weight update pass wants both
+/// of its operands.
+hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
+                                uint32_t pixels, uint32_t groups,
+                                uint32_t chans, uint64_t strideG,
+                                uint64_t strideC, uint64_t strideP,
+                                int elemBytes, hipStream_t stream);
+
+/// Zero-fills `bytes` (a multiple of 4) with a kernel, so that the call can
+/// be recorded into a graph.
+hipError_t launchZero(void *dst, uint64_t bytes, hipStream_t stream);
+
 /// biases[c] += scale * sum over rows of zDeltas[row][c] (half or float each),
 /// summed in fp32 in a fixed order: per-split partial sums go to `workspace`
 /// (biasUpdateWorkspaceBytes), a second kernel adds them up split by split.
@@ -100,11 +114,25 @@ struct IgemmDesc {
   uint32_t loH, hiH, loW, hiW;
   // Tile shape chosen by the planner.
   uint32_t blockM, blockN, blockK;
+  // Zeros stuffed between input elements: input row r sits at row r * inDilH
+  // of the field the window slides over (padH, strideH, dilH are in those
+  // coordinates; loH, hiH bound r itself).  1 = none.
+  uint32_t inDilH = 1, inDilW = 1;
+  // Parts K is cut into, one workgroup each; above 1 the launch needs
+  // igemmWorkspaceBytes of scratch and adds the parts up in a second kernel.
+  uint32_t splitK = 1;
 };
+/// How the kernel finds out which kernel taps of an output pixel read inside
+/// the input: a bit mask per pixel (up to 32 taps), ranges of valid kernel
+/// rows and columns per pixel (more taps), or arithmetic per tap (dilated
+/// input).
+enum : int { kMaskTaps = 0, kRangeTaps = 1, kDilatedTaps = 2 };
+int igemmTapAddressing(const IgemmDesc &d);
+size_t igemmWorkspaceBytes(const IgemmDesc &d);
 hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
                        const void *in, const void *weightsPacked,
-                       const void *bias, void *out, const QuarterInfo &q,
-                       hipStream_t stream);
+                       const void *bias, void *out, void *workspace,
+                       const QuarterInfo &q, hipStream_t stream);
 
 /// Pointwise convolution (every kernel extent 1, stride 1, no padding or
 /// truncation, half inputs) with 128, 256 or 512 input channels per group:

@@ -107,6 +107,94 @@ __global__ __launch_bounds__(256) void scaledAddKernel(T *a,
            scaleA * Load<T>::at(a, tid, 0) + scaleB * Load<T>::at(b, tid, 0));
 }
 
+constexpr uint32_t kSwapChans = 64, kSwapRows = 128;
+
+struct SwapArgs {
+  uint32_t batch, pixels, groups, chans; // source [batch][pixels][groups][chans]
+  uint32_t pixelsPerTile, batchPerTile;  // their product is kSwapRows
+  uint64_t strideG, strideC, strideP;    // destination strides; batch has 1
+};
+
+/// dst[g * strideG + c * strideC + p * strideP + b] = src[b][p][g][c]: the
+/// batch axis becomes the innermost one.  A workgroup moves a tile of 128
+/// (pixel, batch) rows by 64 channels through LDS: loads run along the
+/// channels, stores along the batch (and on along the pixels where the
+/// destination keeps them adjacent).
+template <class T, bool VEC>
+__global__ __launch_bounds__(256) void swapBatchChansKernel(
+    SwapArgs a, const T *__restrict__ src, T *__restrict__ dst) {
+  __shared__ uint32_t tile[kSwapRows][kSwapChans + 1];
+  const uint32_t cBlocks = (a.chans + kSwapChans - 1) / kSwapChans;
+  const uint32_t c0 = (blockIdx.x % cBlocks) * kSwapChans;
+  const uint32_t g = blockIdx.x / cBlocks;
+  const uint32_t p0 = blockIdx.y * a.pixelsPerTile;
+  const uint32_t b0 = blockIdx.z * a.batchPerTile;
+  const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  // row = pLocal * batchPerTile + bLocal
+  auto source = [&](uint32_t row, uint32_t c) {
+    const uint32_t p = p0 + row / a.batchPerTile;
+    const uint32_t b = b0 + row % a.batchPerTile;
+    return p < a.pixels && b < a.batch && c < a.chans
+               ? src + ((uint64_t(b) * a.pixels + p) * a.groups + g) * a.chans +
+                     c
+               : nullptr;
+  };
+  if constexpr (VEC) {
+    // 16-byte loads: kVec channels per thread, all loads of a thread issued
+    // before the first is used.  The channel count is a multiple of kVec.
+    constexpr uint32_t kVec = 16 / sizeof(T);
+    constexpr uint32_t kLanesPerRow = kSwapChans / kVec;
+    constexpr uint32_t kRowsPerPass = 256 / kLanesPerRow;
+    constexpr uint32_t kPasses = kSwapRows / kRowsPerPass;
+    const uint32_t cLocal = (threadIdx.x % kLanesPerRow) * kVec;
+    const uint32_t rowInPass = threadIdx.x / kLanesPerRow;
+    uint4 v[kPasses];
+#pragma unroll
+    for (uint32_t i = 0; i != kPasses; ++i) {
+      const T *from = source(i * kRowsPerPass + rowInPass, c0 + cLocal);
+      v[i] = from ? *reinterpret_cast<const uint4 *>(from) : uint4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (uint32_t i = 0; i != kPasses; ++i) {
+      const T *e = reinterpret_cast<const T *>(&v[i]);
+#pragma unroll
+      for (uint32_t k = 0; k != kVec; ++k)
+        tile[i * kRowsPerPass + rowInPass][cLocal + k] = e[k];
+    }
+  } else {
+    constexpr uint32_t kPasses = kSwapRows / 4;
+    T v[kPasses];
+#pragma unroll
+    for (uint32_t i = 0; i != kPasses; ++i) {
+      const T *from = source(i * 4 + wave, c0 + lane);
+      v[i] = from ? *from : T(0);
+    }
+#pragma unroll
+    for (uint32_t i = 0; i != kPasses; ++i)
+      tile[i * 4 + wave][lane] = v[i];
+  }
+  __syncthreads();
+  // 64 lanes = 64 consecutive rows of the tile: consecutive batch entries,
+  // then the next pixel.
+#pragma unroll 4
+  for (uint32_t i = wave; i < kSwapChans * 2; i += 4) {
+    const uint32_t cLocal = i / 2, row = (i % 2) * 64 + lane;
+    const uint32_t p = p0 + row / a.batchPerTile;
+    const uint32_t b = b0 + row % a.batchPerTile;
+    const uint32_t c = c0 + cLocal;
+    if (p < a.pixels && b < a.batch && c < a.chans)
+      dst[g * a.strideG + c * a.strideC + p * a.strideP + b] =
+          T(tile[row][cLocal]);
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void zeroKernel(T *dst, uint64_t total) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid < total)
+    dst[tid] = T(0);
+}
+
 constexpr uint32_t kReduceChans = 64, kReduceLanes = 4;
 
 /// partial[split][c] = sum over the rows of `split` of z[row][c], fp32.
@@ -277,6 +365,68 @@ hipError_t launchAddBias(int type, void *acts, const void *bias,
                        static_cast<const __half *>(bias), total, channels);
   else
     return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
+                                uint32_t pixels, uint32_t groups,
+                                uint32_t chans, uint64_t strideG,
+                                uint64_t strideC, uint64_t strideP,
+                                int elemBytes, hipStream_t stream) {
+  if (uint64_t(batch) * pixels * groups * chans == 0)
+    return hipSuccess;
+  SwapArgs a;
+  a.batch = batch, a.pixels = pixels, a.groups = groups, a.chans = chans;
+  // As much of the batch as a tile takes (a power of two, so that it divides
+  // the 128 rows), the rest of the rows for neighbouring pixels.
+  a.batchPerTile = 1;
+  while (a.batchPerTile < kSwapRows && a.batchPerTile < batch)
+    a.batchPerTile *= 2;
+  a.pixelsPerTile = kSwapRows / a.batchPerTile;
+  a.strideG = strideG, a.strideC = strideC, a.strideP = strideP;
+  const uint64_t gx = uint64_t((chans + kSwapChans - 1) / kSwapChans) * groups;
+  const uint64_t gy = (pixels + a.pixelsPerTile - 1) / a.pixelsPerTile;
+  const uint64_t gz = (batch + a.batchPerTile - 1) / a.batchPerTile;
+  if (gx > 0x7fffffffull || gy > 65535 || gz > 65535)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(gx), uint32_t(gy), uint32_t(gz)}, block{256};
+  // 16-byte loads need every row of channels to start on a 16-byte boundary.
+  const bool vec = chans % uint32_t(16 / elemBytes) == 0 &&
+                   reinterpret_cast<uintptr_t>(src) % 16 == 0;
+  if (elemBytes == 2) {
+    const auto *from = static_cast<const uint16_t *>(src);
+    auto *to = static_cast<uint16_t *>(dst);
+    if (vec)
+      hipLaunchKernelGGL((swapBatchChansKernel<uint16_t, true>), grid, block, 0,
+                         stream, a, from, to);
+    else
+      hipLaunchKernelGGL((swapBatchChansKernel<uint16_t, false>), grid, block,
+                         0, stream, a, from, to);
+  } else if (elemBytes == 4) {
+    const auto *from = static_cast<const uint32_t *>(src);
+    auto *to = static_cast<uint32_t *>(dst);
+    if (vec)
+      hipLaunchKernelGGL((swapBatchChansKernel<uint32_t, true>), grid, block, 0,
+                         stream, a, from, to);
+    else
+      hipLaunchKernelGGL((swapBatchChansKernel<uint32_t, false>), grid, block,
+                         0, stream, a, from, to);
+  } else {
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launchZero(void *dst, uint64_t bytes, hipStream_t stream) {
+  if (bytes == 0)
+    return hipSuccess;
+  if (bytes % 4 != 0)
+    return hipErrorInvalidValue;
+  const uint64_t total = bytes / 4, blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL(zeroKernel<uint32_t>, dim3(uint32_t(blocks)), dim3(256), 0,
+                     stream, static_cast<uint32_t *>(dst), total);
   return hipGetLastError();
 }
 

@@ -131,7 +131,7 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
                                             in, w, bias, out, s),
                        "pointwise convolution launch");
     return hipStatus(mxk::launchIgemm(plan->igemm, inType, outType, in, w,
-                                      bias, out, q, s),
+                                      bias, out, workspace, q, s),
                      "implicit-GEMM convolution launch");
   case mxconv_plan::Kernel::DEPTHWISE:
     return hipStatus(mxk::launchDepthwise(plan->depthwise, inType, outType, in,
@@ -1074,28 +1074,48 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
   mxconv_status st;
   if (plan->inputElems) {
     // activations [B][X][G][Ci] -> the pass's input [Ci][X][G][B]
-    const uint64_t dims[4] = {B, X, G, Ci};
-    const int perm[4] = {3, 1, 2, 0};
-    st = hipStatus(mxk::launchPermute4(acts, ws + w.input, dims, perm, inBytes,
-                                       s),
+    st = hipStatus(mxk::launchSwapBatchChans(acts, ws + w.input, uint32_t(B),
+                                             uint32_t(X), uint32_t(G),
+                                             uint32_t(Ci), B, X * G * B, G * B,
+                                             inBytes, s),
                    "activation rearrangement");
     if (st != MXCONV_OK)
       return st;
   }
-  if (plan->weightElems) {
-    // deltas [B][Y][G][Co] -> the pass's weights [G][Co][B][Y]
-    const uint64_t dims[4] = {B, Y, G, Co};
-    const int perm[4] = {2, 3, 0, 1};
-    st = hipStatus(mxk::launchPermute4(zDeltas, ws + w.weightsExternal, dims,
-                                       perm, inBytes, s),
+  if (plan->kernel == mxconv_plan::Kernel::IGEMM && !plan->pointwiseOn) {
+    // deltas [B][Y][G][Co] -> straight into the matrix-core kernel's packed
+    // weights [G][coPadded][kPadded], k = y * B + b
+    if (plan->coPadded != Co || plan->kPadded != Y * B) {
+      st = hipStatus(mxk::launchZero(ws + w.weightsPacked,
+                                     alignUp(plan->weightPackedBytes()), s),
+                     "delta rearrangement");
+      if (st != MXCONV_OK)
+        return st;
+    }
+    st = hipStatus(mxk::launchSwapBatchChans(
+                       zDeltas, ws + w.weightsPacked, uint32_t(B), uint32_t(Y),
+                       uint32_t(G), uint32_t(Co),
+                       uint64_t(plan->coPadded) * plan->kPadded, plan->kPadded,
+                       B, inBytes, s),
                    "delta rearrangement");
     if (st != MXCONV_OK)
       return st;
+  } else {
+    if (plan->weightElems) {
+      // deltas [B][Y][G][Co] -> the pass's weights [G][Co][B][Y]
+      const uint64_t dims[4] = {B, Y, G, Co};
+      const int perm[4] = {2, 3, 0, 1};
+      st = hipStatus(mxk::launchPermute4(zDeltas, ws + w.weightsExternal, dims,
+                                         perm, inBytes, s),
+                     "delta rearrangement");
+      if (st != MXCONV_OK)
+        return st;
+    }
+    st = mxconv_pack_weights(plan, ws + w.weightsExternal,
+                             ws + w.weightsPacked, stream);
+    if (st != MXCONV_OK)
+      return st;
   }
-  st = mxconv_pack_weights(plan, ws + w.weightsExternal, ws + w.weightsPacked,
-                           stream);
-  if (st != MXCONV_OK)
-    return st;
   st = forward(plan, ws + w.input, ws + w.weightsPacked, nullptr,
                ws + w.output, ws + w.planWorkspace, plan->workspaceBytes,
                mxk::QuarterInfo{}, stream);

@@ -192,6 +192,8 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       pc.blockN = requireUnsigned(sub, m.second);
     } else if (m.first == "blockK") {
       pc.blockK = requireUnsigned(sub, m.second);
+    } else if (m.first == "splitK") {
+      pc.splitK = requireUnsigned(sub, m.second);
     } else if (m.first == "tileH") {
       pc.tileH = requireUnsigned(sub, m.second);
     } else if (m.first == "tileW") {

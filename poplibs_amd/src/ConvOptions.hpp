@@ -35,6 +35,8 @@ struct PlanConstraints {
   /// tile extents; 0 / empty = planner's choice.
   std::string kernel;
   unsigned blockM = 0, blockN = 0, blockK = 0;
+  /// Parts the matrix-core kernel cuts K into; 0 = planner's choice.
+  unsigned splitK = 0;
   /// Output tile of the depthwise kernel; 0 = planner's choice.
   unsigned tileH = 0, tileW = 0;
   std::string text; // the JSON as given, kept for reporting and cache keys

@@ -51,9 +51,10 @@ mxk::GenericDesc makeGenericDesc(const ConvParams &p) {
 }
 
 /// The subset the fast kernels take: up to two field dimensions; input with
-/// truncation and zero padding only; kernel with dilation only; output with
-/// truncation and stride only.  Written as "input row = out*stride +
-/// k*dilation - pad, valid inside [lo, hi)".
+/// truncation, dilation and zero padding; kernel with dilation only; output
+/// with truncation and stride only.  Written as "row of the dilated input =
+/// out*stride + k*dilation - pad; it holds input row r when it equals
+/// r*inDil, valid for r inside [lo, hi)".
 struct Simple2D {
   bool ok = false;
   std::string why;
@@ -61,6 +62,8 @@ struct Simple2D {
   int32_t padH = 0, padW = 0;
   uint32_t strideH = 1, strideW = 1, dilH = 1, dilW = 1;
   uint32_t loH = 0, hiH = 1, loW = 0, hiW = 1;
+  uint32_t inDilH = 1, inDilW = 1;
+  bool inputDilated() const { return inDilH != 1 || inDilW != 1; }
 };
 
 Simple2D asSimple2D(const ConvParams &p) {
@@ -73,8 +76,8 @@ Simple2D asSimple2D(const ConvParams &p) {
   for (unsigned d = 0; d != n; ++d) {
     const auto &it = p.inputTransform, &kt = p.kernelTransform;
     const auto &ot = p.outputTransform;
-    if (it.dilation[d] != 1 || it.flip[d]) {
-      s.why = "input dilation or flip";
+    if (it.flip[d]) {
+      s.why = "input flip";
       return s;
     }
     if (kt.truncationLower[d] || kt.truncationUpper[d] || kt.paddingLower[d] ||
@@ -87,9 +90,10 @@ Simple2D asSimple2D(const ConvParams &p) {
       return s;
     }
     // conv index = o*stride + outTruncLo; padded input = conv + k*dil;
-    // input = padded - padLo + truncLo.
+    // dilated input = padded - padLo; input = dilated / inDil + truncLo when
+    // that is whole.
     const int32_t pad = int32_t(it.paddingLower[d]) -
-                        int32_t(it.truncationLower[d]) -
+                        int32_t(it.truncationLower[d] * it.dilation[d]) -
                         int32_t(ot.truncationLower[d]);
     const uint32_t lo = it.truncationLower[d];
     const uint32_t hi = uint32_t(p.inputFieldShape[d]) - it.truncationUpper[d];
@@ -102,6 +106,7 @@ Simple2D asSimple2D(const ConvParams &p) {
     (isW ? s.dilW : s.dilH) = kt.dilation[d];
     (isW ? s.loW : s.loH) = lo;
     (isW ? s.hiW : s.hiH) = hi;
+    (isW ? s.inDilW : s.inDilH) = it.dilation[d];
   }
   s.ok = true;
   return s;
@@ -208,13 +213,29 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     else if (ci % (halfIn ? 8 : 16) != 0)
       igemmWhyNot = "input channels per group not a multiple of a 16-byte "
                     "vector";
-    else if (std::size_t(s.kH) * s.kW > 32)
-      igemmWhyNot = "more than 32 kernel taps";
+    else if (std::size_t(s.outH) * s.strideH + std::size_t(s.kH) * s.dilH +
+                     std::size_t(std::abs(s.padH)) >=
+                 32768 ||
+             std::size_t(s.outW) * s.strideW + std::size_t(s.kW) * s.dilW +
+                     std::size_t(std::abs(s.padW)) >=
+                 32768)
+      igemmWhyNot = "field too large for 16-bit window origins";
+    else if (s.inputDilated() &&
+             (std::size_t(s.inW) * p.getNumInputChans() *
+                      params.inputType.size() >=
+                  (1u << 24) ||
+              s.inDilH >= (1u << 24) || s.inDilW >= (1u << 24)))
+      igemmWhyNot = "input rows too long for the arithmetic tap addressing";
+    else if (!s.inputDilated() && std::size_t(s.kH) * s.kW > 32 &&
+             (s.kH > 255 || s.kW > 255))
+      igemmWhyNot = "kernel extent above 255";
     else if (plan.inputElems * params.inputType.size() >= (1ull << 30) ||
              plan.weightElems * params.inputType.size() >= (1ull << 30))
       igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     if (!halfIn)
       dwWhyNot = "depthwise kernel takes half inputs";
+    else if (s.inputDilated())
+      dwWhyNot = "input dilation";
     else if (ci != 1 || co != 1)
       dwWhyNot = "not one channel per group";
     else if (p.numConvGroups % 8 != 0)
@@ -282,6 +303,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     g.strideH = s.strideH, g.strideW = s.strideW;
     g.dilH = s.dilH, g.dilW = s.dilW;
     g.loH = s.loH, g.hiH = s.hiH, g.loW = s.loW, g.hiW = s.hiW;
+    g.inDilH = s.inDilH, g.inDilW = s.inDilW;
     // Tile shape.  M = batch * outH * outW pixels, N = out channels of one
     // group, K = kH * kW * in channels.  A 128-pixel tile keeps the A
     // fragment reuse high; N is 128 unless the group has at most 64 output
@@ -298,6 +320,31 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
     plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;
     plan.weightPackedElems = p.numConvGroups * plan.coPadded * plan.kPadded;
+    // Too few output tiles to fill the chip but a long K (a weight update
+    // pass, a skinny matrix product): cut K into parts, one workgroup each,
+    // as many as bring the grid up to about one workgroup per CU while every
+    // part keeps at least 4 k-steps; the fp32 partial tiles go through a
+    // workspace (the role of PopLibs' in-channel split with ReduceAdd,
+    // lib/poplin/ConvReduce.cpp:316-362).
+    {
+      const std::size_t m = p.batchSize * std::size_t(s.outH) * s.outW;
+      const std::size_t tiles = ((m + g.blockM - 1) / g.blockM) *
+                                (plan.coPadded / g.blockN) * p.numConvGroups;
+      const std::size_t kSteps = plan.kPadded / g.blockK;
+      std::size_t parts = 1;
+      if (pc.splitK)
+        parts = pc.splitK;
+      else if (tiles != 0 && tiles * 2 <= gfx950::numCUs && kSteps >= 16)
+        parts = std::min<std::size_t>(gfx950::numCUs / tiles, kSteps / 4);
+      parts = std::max<std::size_t>(1, std::min(parts, kSteps));
+      const std::size_t chans = p.numConvGroups * co;
+      // the reduction reads and writes vectors of four channels; partial
+      // tiles of more than 1 GB are not worth it
+      if (chans % 4 != 0 || parts * m * chans * 4 > (1ull << 30))
+        parts = 1;
+      g.splitK = uint32_t(parts);
+      plan.workspaceBytes = mxk::igemmWorkspaceBytes(g);
+    }
     // A pointwise convolution with few input channels is bound by HBM, not
     // by the matrix cores: unless the big tile was asked for explicitly, the
     // streaming kernel of small workgroups takes it.
@@ -306,7 +353,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     pw.groups = g.groups, pw.inChansPerGroup = g.inChansPerGroup;
     pw.outChansPerGroup = g.outChansPerGroup;
     const bool unitWindow =
-        s.kH == 1 && s.kW == 1 && s.strideH == 1 && s.strideW == 1 &&
+        !s.inputDilated() && g.splitK == 1 && s.kH == 1 && s.kW == 1 &&
+        s.strideH == 1 && s.strideW == 1 &&
         s.padH == 0 && s.padW == 0 && s.loH == 0 && s.loW == 0 &&
         s.hiH == s.inH && s.hiW == s.inW && s.outH == s.inH &&
         s.outW == s.inW;
@@ -398,7 +446,16 @@ std::string mxconv_plan::describe() const {
     } else {
       os << "        block M x N x K            " << g.blockM << " x "
          << g.blockN << " x " << g.blockK << "\n";
-      os << "        workgroups                 " << tiles << "\n";
+      os << "        workgroups                 " << tiles * g.splitK << "\n";
+      if (g.splitK > 1)
+        os << "        K split into parts         " << g.splitK
+           << " (fp32 partial tiles, summed by a second kernel)\n";
+      if (mxk::igemmTapAddressing(g) == mxk::kRangeTaps)
+        os << "        tap addressing             ranges of valid kernel rows "
+              "and columns (more than 32 taps)\n";
+      else if (mxk::igemmTapAddressing(g) == mxk::kDilatedTaps)
+        os << "        tap addressing             arithmetic (dilated "
+              "input)\n";
       os << "        packed weights             [G=" << g.groups << "]["
          << coPadded << "][" << kPadded << "]\n";
     }

@@ -135,9 +135,10 @@ BWD_GPU_CASES = [
     # (64 input channels: the big-tile kernel)
     (dict(batch=2, field=(9, 9), kernel=(1, 1), ci=256, co=64),
      "implicit GEMM"),
-    # forward stride 2: the deltas are dilated going backwards - generic kernel
+    # forward stride 2: the deltas are dilated going backwards - the matrix
+    # cores take it with arithmetic tap addressing
     (dict(batch=2, field=(9, 10), kernel=(3, 3), ci=8, co=16, stride=2, pad=1),
-     "generic direct"),
+     "arithmetic"),
     # depthwise 3x3 stride 1 stays depthwise
     (dict(batch=2, field=(12, 13), kernel=(3, 3), groups=16, pad=1),
      "depthwise direct"),

@@ -389,9 +389,23 @@ def test_planner_choices():
     assert _kernel_of(c2) == "implicit GEMM"
     assert _kernel_of(c4) == "depthwise direct"
     assert _kernel_of(c5) == "implicit GEMM"
+    # a dilated input (what the backward pass of a strided layer brings) and
+    # a kernel of many taps (what a weight update pass brings) stay on the
+    # matrix cores, with other ways of telling which taps read the input
+    dilated = pa.Plan(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
+                                  co=8, idil=2)).describe()
+    assert "implicit GEMM" in dilated and "arithmetic" in dilated
+    many = pa.Plan(make_params(pa.HALF, batch=128, field=(28, 28),
+                               kernel=(28, 28), ci=32, co=128, pad=1))
+    assert "implicit GEMM" in many.describe()
+    assert "ranges of valid kernel rows" in many.describe()
+    # few output tiles, long K: K is cut into parts
+    assert "K split into parts         28" in many.describe()
+    assert many.buffer_bytes(4) == 28 * 128 * 9 * 128 * 4
+    assert "K split" not in pa.Plan(c2).describe()
     # transforms outside the fast subset fall back
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
-                                  co=8, idil=2)) == "generic direct"
+                                  co=8, flipIn=True)) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
                                   co=8, flipK=True)) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),

@@ -345,3 +345,93 @@ def test_baseline_config5_full(oracle):
         # output round: well inside the 3e-2 fp8 budget
         err = rel_l2(got[b], want[0])
         assert err <= 3e-2 and err <= 1e-3, err
+
+
+# Kernels of more than 32 taps (valid-range tap addressing) and dilated
+# (zero-stuffed) inputs (arithmetic tap addressing), the shapes weight update
+# and backward passes bring.
+GENERAL_CASES = [
+    # 7x7 = 49 taps; channel block of a whole k-step per tap (uniform) or less
+    dict(batch=2, field=(20, 19), kernel=(7, 7), ci=64, co=40, pad=3),
+    dict(batch=2, field=(20, 19), kernel=(7, 7), ci=8, co=72, pad=3,
+         stride=2),
+    # backward pass of a stride-2 3x3 layer: input dilated by 2
+    dict(batch=2, field=(14, 15), kernel=(3, 3), ci=64, co=16, idil=2,
+         padLower=(1, 1), padUpper=(2, 2)),
+    dict(batch=3, field=(7, 9), kernel=(3, 2), ci=16, co=136, idil=(3, 2),
+         pad=2, kdil=(1, 2), groups=2),
+    # dilation and truncation together, 1-D
+    dict(batch=2, field=(33,), kernel=(5,), ci=24, co=8, idil=2, itl=(2,),
+         itu=(1,), pad=4, stride=3),
+    # a weight-update-like pass: the "kernel" is a whole 12x12 field, dilated
+    dict(batch=16, field=(26, 26), kernel=(12, 12), ci=8, co=24, kdil=2,
+         padLower=(1, 1), padUpper=(0, 0)),
+]
+
+
+@pytest.mark.parametrize("kw", GENERAL_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_igemm_general_addressing_matches_oracle(oracle, kw, out_type):
+    p = make_params(pa.HALF, out_type, **kw)
+    print("case", p, flush=True)
+    from gpu_helpers import quantize, run_conv
+    acts, weights, biases = random_data(p, 5, "normal")
+    aq, ad = quantize(acts, pa.HALF)
+    wq, wd = quantize(weights * 0.05, pa.HALF)
+    got, plan = run_conv(p, aq, wq, return_plan=True)
+    assert "tap addressing" in plan.describe(), plan.describe()
+    want = oracle.convolution(p, ad, wd, threads=8)
+    assert rel_l2(got, want) <= 1e-3, (rel_l2(got, want), plan.describe())
+
+
+SPLIT_K_CASES = [
+    # (params, forced parts or None for the planner's choice)
+    (dict(batch=1, field=(6, 6), kernel=(3, 3), ci=512, co=128, pad=1), None),
+    (dict(batch=2, field=(9, 7), kernel=(3, 3), ci=64, co=40, pad=1), 3),
+    (dict(batch=2, field=(9, 7), kernel=(3, 3), ci=64, co=40, pad=1), 9),
+    (dict(batch=2, field=(9, 7), kernel=(3, 3), ci=8, co=136, pad=1,
+          groups=2), 2),
+    (dict(batch=16, field=(26, 26), kernel=(12, 12), ci=8, co=24, kdil=2,
+          padLower=(1, 1), padUpper=(0, 0)), None),
+]
+
+
+@pytest.mark.parametrize("kw,parts", SPLIT_K_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_igemm_split_k_matches_oracle(oracle, kw, parts, out_type):
+    p = make_params(pa.HALF, out_type, **kw)
+    print("case", p, parts, flush=True)
+    from gpu_helpers import quantize, run_conv
+    options = None
+    if parts:
+        options = {"planConstraints": '{"gfx950": {"splitK": %d}}' % parts}
+    acts, weights, biases = random_data(p, 6, "normal")
+    aq, ad = quantize(acts, pa.HALF)
+    wq, wd = quantize(weights * 0.05, pa.HALF)
+    bq, bd = quantize(biases, out_type)
+    got, plan = run_conv(p, aq, wq, bq, options, return_plan=True)
+    assert "K split into parts" in plan.describe(), plan.describe()
+    if parts:
+        assert "K split into parts         %d" % parts in plan.describe()
+    want = oracle.convolution(p, ad, wd, bd, threads=8)
+    assert rel_l2(got, want) <= 1e-3, (rel_l2(got, want), plan.describe())
+
+
+def test_igemm_split_k_of_signs_is_exact(oracle):
+    # +-1 data: every partial sum is a small integer, so the parts add up
+    # exactly whatever the cut
+    p = make_params(pa.HALF, pa.FLOAT, batch=1, field=(5, 5), kernel=(3, 3),
+                    ci=128, co=64, pad=1)
+    _run(oracle, p, 9, 0, "implicit GEMM", dist="pm1", bias=False,
+         options={"planConstraints": '{"gfx950": {"splitK": 5}}'})
+
+
+def test_skinny_matmul_is_split_along_k():
+    from test_matmul import run_matmul
+    rng = np.random.default_rng(10)
+    A = rng.standard_normal((1, 48, 4096)).astype(np.float16)
+    B = (rng.standard_normal((1, 4096, 128)) / 64).astype(np.float16)
+    got, plan = run_matmul(A, B, pa.HALF, pa.FLOAT, return_plan=True)
+    assert "K split into parts" in plan.describe(), plan.describe()
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    assert rel_l2(got, want) <= 1e-5
