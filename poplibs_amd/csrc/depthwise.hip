@@ -274,6 +274,9 @@ hipError_t runKernelShape(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream) {
+  if (d.inDilH != 1 || d.inDilW != 1)
+    return launchDepthwiseDirect(d, inType, outType, in, weightsPacked, bias,
+                                 out, stream);
   if (d.dense3x3)
     return launchDepthwise3x3(d, inType, outType, in, weightsPacked, bias,
                                  out, stream);

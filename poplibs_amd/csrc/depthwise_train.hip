@@ -1,0 +1,351 @@
+// Depthwise kernels for the training passes of a depthwise layer (one input
+// and one output channel per group, channels-last, fp16 data, fp32 sums):
+//
+//   depthwiseDirectKernel      a forward convolution that also takes a
+//                              dilated (zero-stuffed) input, which is what
+//                              the backward pass of a strided depthwise layer
+//                              is; one thread per output pixel and vector of
+//                              8 channels, taps that fall between input
+//                              elements skipped.
+//   depthwiseWeightDeltaKernel the gradient with respect to the weights,
+//                              dW[tap][c] = sum over batch and output pixels
+//                              of deltas[pixel][c] * acts[pixel under tap][c];
+//                              one thread per (tap, vector of 8 channels),
+//                              walking a slice of the pixels; the per-slice
+//                              sums go to a workspace and a second kernel
+//                              adds the slices in order.
+//
+// Both are bound by memory: they read each operand from HBM once (re-reads
+// of neighbouring taps hit the caches) and have no matrix-core work.  They
+// take the role of PopLibs' HorizontalMac vertices in the backward and weight
+// update passes (lib/poplin/codelets/ConvPartialHorizontalMac.cpp:34-133).
+#include "device_types.hpp"
+#include "kernels.hpp"
+
+#include <algorithm>
+
+namespace mxk {
+namespace {
+
+union Vec8 {
+  uint4 raw;
+  __half2 h2[4];
+};
+
+__device__ __forceinline__ void fma8(float (&acc)[8], const Vec8 &x,
+                                     const Vec8 &k) {
+#pragma unroll
+  for (int i = 0; i != 4; ++i) {
+    const float2 xf = __half22float2(x.h2[i]);
+    const float2 kf = __half22float2(k.h2[i]);
+    acc[2 * i] = fmaf(xf.x, kf.x, acc[2 * i]);
+    acc[2 * i + 1] = fmaf(xf.y, kf.y, acc[2 * i + 1]);
+  }
+}
+
+__device__ __forceinline__ void store8(__half *p, const float (&v)[8]) {
+  Vec8 o;
+#pragma unroll
+  for (int i = 0; i != 4; ++i)
+    o.h2[i] = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
+  *reinterpret_cast<uint4 *>(p) = o.raw;
+}
+__device__ __forceinline__ void store8(float *p, const float (&v)[8]) {
+  *reinterpret_cast<float4 *>(p) = float4{v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<float4 *>(p + 4) = float4{v[4], v[5], v[6], v[7]};
+}
+
+struct DirectArgs {
+  DepthwiseDesc d;
+  FastDiv divVecs, divOutW, divOutH, divInDilH, divInDilW;
+  uint32_t vecs;
+  uint64_t items; // batch * outH * outW * vecs
+};
+
+template <class OutT>
+__global__ __launch_bounds__(256) void depthwiseDirectKernel(
+    DirectArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
+    const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  const DepthwiseDesc &d = a.d;
+  const uint64_t item = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (item >= a.items)
+    return;
+  // item = ((b * outH + oh) * outW + ow) * vecs + v
+  const uint32_t pixel = a.divVecs(uint32_t(item));
+  const uint32_t v = uint32_t(item) - pixel * a.vecs;
+  const uint32_t row = a.divOutW(pixel);
+  const uint32_t ow = pixel - row * d.outW;
+  const uint32_t b = a.divOutH(row);
+  const uint32_t oh = row - b * d.outH;
+  const uint32_t c = v * 8;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i != 8; ++i)
+    acc[i] = bias ? Load<OutT>::at(bias, c + i, 0) : 0.0f;
+  const int ihBase = int(oh * d.strideH) - d.padH;
+  const int iwBase = int(ow * d.strideW) - d.padW;
+  const __half *image = in + size_t(b) * d.inH * d.inW * d.channels + c;
+  for (uint32_t kh = 0; kh != d.kH; ++kh) {
+    const int ihD = ihBase + int(kh * d.dilH);
+    const uint32_t ih = a.divInDilH(uint32_t(ihD));
+    if (ihD < 0 || ih * d.inDilH != uint32_t(ihD) || ih < d.loH || ih >= d.hiH)
+      continue;
+    for (uint32_t kw = 0; kw != d.kW; ++kw) {
+      const int iwD = iwBase + int(kw * d.dilW);
+      const uint32_t iw = a.divInDilW(uint32_t(iwD));
+      if (iwD < 0 || iw * d.inDilW != uint32_t(iwD) || iw < d.loW ||
+          iw >= d.hiW)
+        continue;
+      Vec8 x, k;
+      x.raw = *reinterpret_cast<const uint4 *>(
+          image + (size_t(ih) * d.inW + iw) * d.channels);
+      k.raw = *reinterpret_cast<const uint4 *>(
+          w + size_t(kh * d.kW + kw) * d.channels + c);
+      fma8(acc, x, k);
+    }
+  }
+  store8(out + size_t(pixel) * d.channels + c, acc);
+}
+
+struct DeltaArgs {
+  DepthwiseDesc d;     // the FORWARD convolution
+  FastDiv divVecs, divOutW, divOutH;
+  uint32_t vecs, taps;
+  uint32_t items;      // taps * vecs
+  uint32_t itemsPerBlock, slots; // itemsPerBlock * slots <= 256 threads
+  uint32_t pixels;     // batch * outH * outW
+  uint32_t pixelsPerSlice, pixelsPerSlot, slices;
+};
+
+/// partial[slice][tap][c] = sum over the slice's output pixels.  A workgroup
+/// takes itemsPerBlock (tap, channel vector) items and one slice of the
+/// pixels; when there are few items, `slots` groups of threads walk a part of
+/// the slice each and their sums meet in LDS.
+__global__ __launch_bounds__(256) void depthwiseWeightDeltaKernel(
+    DeltaArgs a, const __half *__restrict__ acts,
+    const __half *__restrict__ deltas, float *__restrict__ partial) {
+  __shared__ float meet[256][9]; // 8 sums per thread, padded
+  const DepthwiseDesc &d = a.d;
+  const uint32_t slot = threadIdx.x / a.itemsPerBlock;
+  const uint32_t itemLocal = threadIdx.x - slot * a.itemsPerBlock;
+  const uint32_t item = blockIdx.x * a.itemsPerBlock + itemLocal;
+  const bool active = slot < a.slots && item < a.items;
+  // item = tap * vecs + v: neighbouring threads read neighbouring channels
+  const uint32_t tap = a.divVecs(active ? item : 0);
+  const uint32_t c = ((active ? item : 0) - tap * a.vecs) * 8;
+  const uint32_t kh = tap / d.kW, kw = tap - kh * d.kW;
+  const uint32_t slice = blockIdx.y;
+  const uint32_t sliceEnd =
+      min((slice + 1) * a.pixelsPerSlice, a.pixels);
+  const uint32_t first =
+      min(slice * a.pixelsPerSlice + slot * a.pixelsPerSlot, sliceEnd);
+  const uint32_t last = active ? min(first + a.pixelsPerSlot, sliceEnd) : first;
+  // (b, oh, ow) of the first pixel; they advance without dividing
+  uint32_t row = a.divOutW(first);
+  uint32_t ow = first - row * d.outW;
+  uint32_t b = a.divOutH(row);
+  uint32_t oh = row - b * d.outH;
+  const int khd = int(kh * d.dilH) - d.padH, kwd = int(kw * d.dilW) - d.padW;
+  float acc[8] = {};
+  // Four pixels a round: their loads are issued together, so that a wave has
+  // eight of them in flight (the walk is bound by load latency, not by
+  // arithmetic).
+  constexpr int kUnroll = 4;
+  for (uint32_t p = first; p < last; p += kUnroll) {
+    Vec8 x[kUnroll], z[kUnroll];
+#pragma unroll
+    for (int u = 0; u != kUnroll; ++u) {
+      const int ih = int(oh * d.strideH) + khd, iw = int(ow * d.strideW) + kwd;
+      const bool ok = p + u < last && ih >= int(d.loH) && ih < int(d.hiH) &&
+                      iw >= int(d.loW) && iw < int(d.hiW);
+      x[u].raw = uint4{0, 0, 0, 0};
+      z[u].raw = uint4{0, 0, 0, 0};
+      if (ok) {
+        x[u].raw = *reinterpret_cast<const uint4 *>(
+            acts +
+            ((size_t(b) * d.inH + uint32_t(ih)) * d.inW + uint32_t(iw)) *
+                d.channels +
+            c);
+        z[u].raw = *reinterpret_cast<const uint4 *>(
+            deltas + size_t(p + u) * d.channels + c);
+      }
+      if (++ow == d.outW) {
+        ow = 0;
+        if (++oh == d.outH) {
+          oh = 0;
+          ++b;
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u != kUnroll; ++u)
+      fma8(acc, x[u], z[u]);
+  }
+  if (a.slots > 1) {
+#pragma unroll
+    for (int i = 0; i != 8; ++i)
+      meet[threadIdx.x][i] = acc[i];
+    __syncthreads();
+    if (slot == 0)
+      for (uint32_t s2 = 1; s2 != a.slots; ++s2)
+#pragma unroll
+        for (int i = 0; i != 8; ++i)
+          acc[i] += meet[s2 * a.itemsPerBlock + itemLocal][i];
+  }
+  if (!active || slot != 0)
+    return;
+  float *dst = partial + (size_t(slice) * a.taps + tap) * d.channels + c;
+  *reinterpret_cast<float4 *>(dst) = float4{acc[0], acc[1], acc[2], acc[3]};
+  *reinterpret_cast<float4 *>(dst + 4) =
+      float4{acc[4], acc[5], acc[6], acc[7]};
+}
+
+/// out[c][tap] = sum over slices of partial[slice][tap][c], in a fixed order:
+/// a workgroup of 16 waves takes 64 outputs; each wave adds up a contiguous
+/// sixteenth of the slices (four loads in flight per lane), then one thread
+/// per output adds the sixteen sums in order.
+template <class OutT>
+__global__ __launch_bounds__(1024) void depthwiseDeltaSumKernel(
+    const float *__restrict__ partial, uint32_t slices, uint32_t taps,
+    uint32_t channels, OutT *__restrict__ out) {
+  __shared__ float meet[16][64];
+  const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const uint32_t outputs = taps * channels;
+  const uint32_t i = blockIdx.x * 64 + lane; // tap * C + c
+  const uint32_t per = (slices + 15) / 16;
+  const uint32_t from = min(wave * per, slices), to = min(from + per, slices);
+  float sum[4] = {};
+  if (i < outputs) {
+    uint32_t s = from;
+    for (; s + 4 <= to; s += 4)
+#pragma unroll
+      for (int u = 0; u != 4; ++u)
+        sum[u] += partial[size_t(s + u) * outputs + i];
+    for (; s != to; ++s)
+      sum[0] += partial[size_t(s) * outputs + i];
+  }
+  meet[wave][lane] = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+  __syncthreads();
+  if (wave != 0 || i >= outputs)
+    return;
+  float total = meet[0][lane];
+  for (int w = 1; w != 16; ++w)
+    total += meet[w][lane];
+  const uint32_t tap = i / channels, c = i - tap * channels;
+  storeOut(out, size_t(c) * taps + tap, total);
+}
+
+/// Threads of a workgroup: itemsPerBlock items by `slots` parts of a slice.
+void deltaBlockShape(const DepthwiseDesc &d, uint32_t &itemsPerBlock,
+                     uint32_t &slots) {
+  const uint64_t items = uint64_t(d.kH) * d.kW * (d.channels / 8);
+  itemsPerBlock = uint32_t(std::min<uint64_t>(std::max<uint64_t>(items, 1), 256));
+  slots = 256 / itemsPerBlock;
+}
+
+uint32_t deltaSlices(const DepthwiseDesc &d) {
+  // About 4 workgroups per CU in all; a slot walks at least 16 pixels.
+  uint32_t itemsPerBlock, slots;
+  deltaBlockShape(d, itemsPerBlock, slots);
+  const uint64_t pixels = uint64_t(d.batch) * d.outH * d.outW;
+  const uint64_t items = uint64_t(d.kH) * d.kW * (d.channels / 8);
+  const uint64_t itemBlocks = (items + itemsPerBlock - 1) / itemsPerBlock;
+  uint64_t slices = (1024 + itemBlocks - 1) / std::max<uint64_t>(itemBlocks, 1);
+  slices = std::min<uint64_t>(slices, (pixels + 16 * slots - 1) / (16 * slots));
+  slices = std::min<uint64_t>(std::max<uint64_t>(slices, 1), 65535);
+  return uint32_t(slices);
+}
+
+} // namespace
+
+hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
+                                 int outType, const void *in,
+                                 const void *weightsPacked, const void *bias,
+                                 void *out, hipStream_t stream) {
+  if (inType != kHalf || d.channels % 8 != 0 || d.inDilH == 0 || d.inDilW == 0)
+    return hipErrorInvalidValue;
+  DirectArgs a;
+  a.d = d;
+  a.vecs = d.channels / 8;
+  a.items = uint64_t(d.batch) * d.outH * d.outW * a.vecs;
+  if (a.items == 0)
+    return hipSuccess;
+  // item numbers are divided with 31-bit arithmetic
+  if (a.items >= (1ull << 31))
+    return hipErrorInvalidConfiguration;
+  a.divVecs = makeFastDiv(a.vecs);
+  a.divOutW = makeFastDiv(d.outW);
+  a.divOutH = makeFastDiv(d.outH);
+  a.divInDilH = makeFastDiv(d.inDilH);
+  a.divInDilW = makeFastDiv(d.inDilW);
+  const dim3 grid{uint32_t((a.items + 255) / 256)}, block{256};
+  if (outType == kHalf)
+    hipLaunchKernelGGL(depthwiseDirectKernel<__half>, grid, block, 0, stream, a,
+                       static_cast<const __half *>(in),
+                       static_cast<const __half *>(weightsPacked),
+                       static_cast<const __half *>(bias),
+                       static_cast<__half *>(out));
+  else if (outType == kFloat)
+    hipLaunchKernelGGL(depthwiseDirectKernel<float>, grid, block, 0, stream, a,
+                       static_cast<const __half *>(in),
+                       static_cast<const __half *>(weightsPacked),
+                       static_cast<const float *>(bias),
+                       static_cast<float *>(out));
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+size_t depthwiseWeightDeltaWorkspaceBytes(const DepthwiseDesc &d) {
+  return size_t(deltaSlices(d)) * d.kH * d.kW * d.channels * sizeof(float);
+}
+
+hipError_t launchDepthwiseWeightDeltas(const DepthwiseDesc &d, int outType,
+                                       const void *acts, const void *deltas,
+                                       void *workspace, void *weightDeltas,
+                                       hipStream_t stream) {
+  if (d.channels % 8 != 0 || d.inDilH != 1 || d.inDilW != 1)
+    return hipErrorInvalidValue;
+  DeltaArgs a;
+  a.d = d;
+  a.vecs = d.channels / 8;
+  a.taps = d.kH * d.kW;
+  const uint64_t items = uint64_t(a.taps) * a.vecs;
+  const uint64_t pixels = uint64_t(d.batch) * d.outH * d.outW;
+  if (items == 0)
+    return hipSuccess;
+  if (items >= (1ull << 31) || pixels >= (1ull << 31) || !workspace)
+    return hipErrorInvalidConfiguration;
+  a.items = uint32_t(items);
+  a.pixels = uint32_t(pixels);
+  a.slices = deltaSlices(d);
+  deltaBlockShape(d, a.itemsPerBlock, a.slots);
+  a.pixelsPerSlice = uint32_t((pixels + a.slices - 1) / a.slices);
+  a.pixelsPerSlot = (a.pixelsPerSlice + a.slots - 1) / a.slots;
+  a.divVecs = makeFastDiv(a.vecs);
+  a.divOutW = makeFastDiv(d.outW);
+  a.divOutH = makeFastDiv(d.outH);
+  float *partial = static_cast<float *>(workspace);
+  const dim3 grid{uint32_t((items + a.itemsPerBlock - 1) / a.itemsPerBlock),
+                  a.slices},
+      block{256};
+  hipLaunchKernelGGL(depthwiseWeightDeltaKernel, grid, block, 0, stream, a,
+                     static_cast<const __half *>(acts),
+                     static_cast<const __half *>(deltas), partial);
+  const uint32_t outputs = a.taps * d.channels;
+  const dim3 grid2{(outputs + 63) / 64};
+  const dim3 block2{1024};
+  if (outType == kHalf)
+    hipLaunchKernelGGL(depthwiseDeltaSumKernel<__half>, grid2, block2, 0, stream,
+                       partial, a.slices, a.taps, d.channels,
+                       static_cast<__half *>(weightDeltas));
+  else if (outType == kFloat)
+    hipLaunchKernelGGL(depthwiseDeltaSumKernel<float>, grid2, block2, 0, stream,
+                       partial, a.slices, a.taps, d.channels,
+                       static_cast<float *>(weightDeltas));
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+} // namespace mxk

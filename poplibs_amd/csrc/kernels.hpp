@@ -165,6 +165,9 @@ struct DepthwiseDesc {
   // 1: the dense-loading small-workgroup kernel (3x3 taps, dilation 1,
   // stride 1 or 2) runs instead of the LDS-tiled one.
   uint32_t dense3x3;
+  // Zeros stuffed between input elements, as in IgemmDesc; other than 1 the
+  // direct kernel of launchDepthwiseDirect runs.
+  uint32_t inDilH = 1, inDilW = 1;
 };
 /// True for the shapes launchDepthwise3x3 takes.
 bool depthwise3x3Takes(const DepthwiseDesc &d, int inType);
@@ -175,6 +178,23 @@ hipError_t launchDepthwise3x3(const DepthwiseDesc &d, int inType,
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream);
+/// The same convolution by one thread per output vector, reading the input
+/// from global memory; takes a dilated input (d.inDilH, d.inDilW), ignores
+/// the tile fields.
+hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
+                                 int outType, const void *in,
+                                 const void *weightsPacked, const void *bias,
+                                 void *out, hipStream_t stream);
+/// Gradient with respect to the weights of the depthwise FORWARD convolution
+/// `d` (undilated input): weightDeltas [channels][kH * kW] in outType from
+/// acts [batch][inH][inW][channels] and deltas [batch][outH][outW][channels],
+/// both fp16.  Partial sums over slices of the pixels go through `workspace`
+/// and are added in a fixed order.
+size_t depthwiseWeightDeltaWorkspaceBytes(const DepthwiseDesc &d);
+hipError_t launchDepthwiseWeightDeltas(const DepthwiseDesc &d, int outType,
+                                       const void *acts, const void *deltas,
+                                       void *workspace, void *weightDeltas,
+                                       hipStream_t stream);
 
 } // namespace mxk
 #endif

@@ -1036,6 +1036,15 @@ WuWorkspace wuWorkspace(const mxconv_plan *plan) {
     at += alignUp(bytes);
     return offset;
   };
+  if (plan->depthwiseWeightUpdate) {
+    // the depthwise weight-delta kernel reads the layer's tensors as they
+    // are: only its partial sums and, for the update, the deltas
+    w.planWorkspace =
+        take(mxk::depthwiseWeightDeltaWorkspaceBytes(plan->depthwiseForward));
+    w.deltas = take(plan->outputBytes());
+    w.total = at;
+    return w;
+  }
   w.input = take(plan->inputBytes());
   w.weightsExternal = take(plan->weightBytes());
   w.weightsPacked = take(plan->weightPackedBytes());
@@ -1071,6 +1080,11 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
   const WuWorkspace w = wuWorkspace(plan);
   if (G * Co * Ci * K == 0)
     return MXCONV_OK;
+  if (plan->depthwiseWeightUpdate)
+    return hipStatus(mxk::launchDepthwiseWeightDeltas(
+                         plan->depthwiseForward, p.outputType.id(), acts,
+                         zDeltas, ws + w.planWorkspace, deltasOut, s),
+                     "depthwise weight deltas");
   mxconv_status st;
   if (plan->inputElems) {
     // activations [B][X][G][Ci] -> the pass's input [Ci][X][G][B]

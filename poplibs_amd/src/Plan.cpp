@@ -193,6 +193,31 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
 
   using Kernel = mxconv_plan::Kernel;
   using Method = PlanConstraints::Method;
+  // The weight update pass of a depthwise layer (getWeightUpdateParams of
+  // it): one "image" (the layer's single input channel per group), one output
+  // channel per group, the layer's batch as input channels.  Its output field
+  // is the layer's kernel, its kernel the layer's output field, its kernel
+  // dilation the layer's stride and its stride the layer's kernel dilation.
+  {
+    const Simple2D w = asSimple2D(p);
+    if (w.ok && !plan.zeroConv && !w.inputDilated() && p.batchSize == 1 &&
+        p.outputChannelsPerConvGroup == 1 &&
+        params.inputType == poplar::HALF && p.numConvGroups % 8 == 0 &&
+        p.numConvGroups * p.inputChannelsPerConvGroup *
+                std::size_t(w.inH) * w.inW * 2 <
+            (1ull << 31)) {
+      plan.depthwiseWeightUpdate = true;
+      mxk::DepthwiseDesc &f = plan.depthwiseForward;
+      f.batch = uint32_t(p.inputChannelsPerConvGroup);
+      f.channels = uint32_t(p.numConvGroups);
+      f.inH = w.inH, f.inW = w.inW;
+      f.outH = w.kH, f.outW = w.kW, f.kH = w.outH, f.kW = w.outW;
+      f.padH = w.padH, f.padW = w.padW;
+      f.strideH = w.dilH, f.strideW = w.dilW;
+      f.dilH = w.strideH, f.dilW = w.strideW;
+      f.loH = w.loH, f.hiH = w.hiH, f.loW = w.loW, f.hiW = w.hiW;
+    }
+  }
   const auto &pc = options.planConstraints;
   const Simple2D s = asSimple2D(p);
   const bool halfIn = params.inputType == poplar::HALF;
@@ -234,16 +259,17 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     if (!halfIn)
       dwWhyNot = "depthwise kernel takes half inputs";
-    else if (s.inputDilated())
-      dwWhyNot = "input dilation";
     else if (ci != 1 || co != 1)
       dwWhyNot = "not one channel per group";
     else if (p.numConvGroups % 8 != 0)
       dwWhyNot = "channel count not a multiple of 8";
     else if (plan.inputElems * 2 >= (1ull << 31))
       dwWhyNot = "tensor too large for 32-bit buffer addressing";
-    else if ((dwTile = chooseDepthwiseTile(s, p.numConvGroups / 8)).first == 0)
+    else if (!s.inputDilated() &&
+             (dwTile = chooseDepthwiseTile(s, p.numConvGroups / 8)).first == 0)
       dwWhyNot = "input patch of a single output pixel exceeds the LDS budget";
+    else if (s.inputDilated() && plan.outputElems / 8 >= (1ull << 31))
+      dwWhyNot = "tensor too large for 32-bit item numbers";
   }
 
   // Choose.  PopLibs method names map onto the kernels that take their role:
@@ -376,10 +402,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     d.dilH = s.dilH, d.dilW = s.dilW;
     d.loH = s.loH, d.hiH = s.hiH, d.loW = s.loW, d.hiW = s.hiW;
     d.tileH = dwTile.first, d.tileW = dwTile.second;
+    d.inDilH = s.inDilH, d.inDilW = s.inDilW;
     // An explicit tile asks for the LDS-tiled kernel.
-    d.dense3x3 =
-        !(pc.tileH || pc.tileW) && mxk::depthwise3x3Takes(d, mxk::kHalf);
-    if (pc.tileH || pc.tileW) {
+    d.dense3x3 = !s.inputDilated() && !(pc.tileH || pc.tileW) &&
+                 mxk::depthwise3x3Takes(d, mxk::kHalf);
+    if (!s.inputDilated() && (pc.tileH || pc.tileW)) {
       d.tileH = pc.tileH ? pc.tileH : d.tileH;
       d.tileW = pc.tileW ? pc.tileW : d.tileW;
       const std::size_t vb = std::min<std::size_t>(p.numConvGroups / 8, 16);
@@ -416,7 +443,10 @@ std::string mxconv_plan::describe() const {
        << (pointwiseOn ? ", pointwise streaming variant" : "");
     break;
   case Kernel::DEPTHWISE:
-    os << (depthwise.dense3x3
+    os << (depthwise.inDilH != 1 || depthwise.inDilW != 1
+               ? "depthwise direct (vector ALU, one thread per output "
+                 "vector, dilated input)"
+           : depthwise.dense3x3
                ? "depthwise direct (vector ALU, dense row loads, small "
                  "workgroups)"
                : "depthwise direct (vector ALU, LDS halo tiles)");
@@ -470,6 +500,9 @@ std::string mxconv_plan::describe() const {
   } else {
     os << "        packed weights             [G][K][Ci][Co]\n";
   }
+  if (depthwiseWeightUpdate)
+    os << "        as a weight update pass    depthwise weight-delta kernel "
+          "on the layer's own tensors\n";
   os << "        workspaceBytes             " << workspaceBytes << "\n";
   return os.str();
 }

@@ -37,6 +37,13 @@ struct mxconv_plan {
   bool pointwiseOn = false;
   mxk::PointwiseDesc pointwise{};
   mxk::DepthwiseDesc depthwise{}; // valid when kernel == DEPTHWISE
+  // These parameters are the weight update pass of a depthwise layer: the
+  // descriptor of that layer's FORWARD convolution, for the kernel that
+  // forms the weight deltas straight from the layer's tensors
+  // (mxconv_calculate_weight_deltas; the kernel chosen above still serves
+  // the parameters as an ordinary convolution).
+  bool depthwiseWeightUpdate = false;
+  mxk::DepthwiseDesc depthwiseForward{};
 
   // Packed weights of the matrix-core kernel: [G][coPadded][kPadded].
   std::size_t coPadded = 0, kPadded = 0;

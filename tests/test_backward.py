@@ -139,6 +139,11 @@ BWD_GPU_CASES = [
     # cores take it with arithmetic tap addressing
     (dict(batch=2, field=(9, 10), kernel=(3, 3), ci=8, co=16, stride=2, pad=1),
      "arithmetic"),
+    # depthwise 3x3 stride 2: dilated deltas, one thread per output vector
+    (dict(batch=2, field=(13, 12), kernel=(3, 3), groups=24, stride=2, pad=1),
+     "dilated input"),
+    (dict(batch=2, field=(17,), kernel=(5,), groups=8, stride=3, pad=2),
+     "dilated input"),
     # depthwise 3x3 stride 1 stays depthwise
     (dict(batch=2, field=(12, 13), kernel=(3, 3), groups=16, pad=1),
      "depthwise direct"),

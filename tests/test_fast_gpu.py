@@ -435,3 +435,29 @@ def test_skinny_matmul_is_split_along_k():
     assert "K split into parts" in plan.describe(), plan.describe()
     want = A.astype(np.float64) @ B.astype(np.float64)
     assert rel_l2(got, want) <= 1e-5
+
+
+DEPTHWISE_DILATED_CASES = [
+    dict(batch=2, field=(7, 8), kernel=(3, 3), groups=16, idil=2,
+         padLower=(1, 1), padUpper=(2, 2)),
+    dict(batch=1, field=(5, 6), kernel=(4, 3), groups=40, idil=(3, 2), pad=2,
+         kdil=(1, 2), stride=(2, 1)),
+    dict(batch=3, field=(9,), kernel=(5,), groups=8, idil=4, itl=(1,),
+         itu=(2,), pad=3),
+]
+
+
+@pytest.mark.parametrize("kw", DEPTHWISE_DILATED_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_depthwise_dilated_input_matches_oracle(oracle, kw, out_type):
+    p = make_params(pa.HALF, out_type, **kw)
+    print("case", p, flush=True)
+    from gpu_helpers import quantize, run_conv
+    acts, weights, biases = random_data(p, 7, "normal")
+    aq, ad = quantize(acts, pa.HALF)
+    wq, wd = quantize(weights, pa.HALF)
+    bq, bd = quantize(biases, out_type)
+    got, plan = run_conv(p, aq, wq, bq, return_plan=True)
+    assert "dilated input" in plan.describe(), plan.describe()
+    want = oracle.convolution(p, ad, wd, bd, threads=8)
+    assert rel_l2(got, want) <= 1e-3, (rel_l2(got, want), plan.describe())

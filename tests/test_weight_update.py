@@ -198,6 +198,50 @@ def test_weight_deltas_on_gpu_match_oracle(oracle, kw):
     assert rel_l2(got, want) <= 1e-5, (rel_l2(got, want), plan.describe())
 
 
+DEPTHWISE_WU_CASES = [
+    dict(batch=3, field=(20, 21), kernel=(3, 3), groups=24, stride=2, pad=1),
+    dict(batch=2, field=(14, 14), kernel=(5, 5), groups=16, pad=2),
+    dict(batch=4, field=(11, 9), kernel=(3, 2), groups=8, kdil=(2, 1),
+         padLower=(1, 0), padUpper=(2, 1), stride=(1, 2)),
+    dict(batch=2, field=(30,), kernel=(7,), groups=32, stride=3, pad=3),
+    dict(batch=2, field=(12, 12), kernel=(3, 3), groups=40, itl=(1, 0),
+         itu=(0, 2), pad=1),
+    dict(batch=70, field=(6, 6), kernel=(3, 3), groups=8, pad=1),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kw", DEPTHWISE_WU_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_depthwise_weight_deltas_on_gpu(oracle, kw, out_type):
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, out_type, **kw)
+    rng = np.random.default_rng(24)
+    C = p.numConvGroups
+    xq, xd = quantize(
+        rng.standard_normal((p.batchSize, C, *p.inputFieldShape)), pa.HALF)
+    dq, dd = quantize(
+        rng.standard_normal((p.batchSize, C, *p.getOutputFieldShape())) * 0.1,
+        pa.HALF)
+    got, plan = run_weight_update(p, xq, dq)
+    assert "depthwise weight-delta kernel" in plan.describe(), plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert got.shape == want.shape
+    tol = 1e-3 if out_type == pa.HALF else 1e-5
+    assert rel_l2(got, want) <= tol, (rel_l2(got, want), plan.describe())
+
+
+@pytest.mark.gpu
+def test_depthwise_weight_deltas_of_signs_are_exact(oracle):
+    p = make_params(pa.HALF, pa.FLOAT, batch=2, field=(9, 9), kernel=(3, 3),
+                    groups=16, stride=2, pad=1)
+    rng = np.random.default_rng(25)
+    x = rng.choice([-1.0, 1.0], size=(2, 16, 9, 9))
+    dz = rng.choice([-1.0, 1.0], size=(2, 16, 5, 5))
+    got, _ = run_weight_update(p, x.astype(np.float16), dz.astype(np.float16))
+    np.testing.assert_array_equal(got, oracle.weight_deltas(p, x, dz))
+
+
 @pytest.mark.gpu
 def test_weight_update_applies_scaled_deltas(oracle):
     from gpu_helpers import quantize
