@@ -113,6 +113,7 @@ struct SwapArgs {
   uint32_t batch, pixels, groups, chans; // source [batch][pixels][groups][chans]
   uint32_t pixelsPerTile, batchPerTile;  // their product is kSwapRows
   uint64_t strideG, strideC, strideP;    // destination strides; batch has 1
+  uint32_t vectorStores; // 1: 16-byte stores of consecutive batch entries
 };
 
 /// dst[g * strideG + c * strideC + p * strideP + b] = src[b][p][g][c]: the
@@ -174,6 +175,33 @@ __global__ __launch_bounds__(256) void swapBatchChansKernel(
       tile[i * 4 + wave][lane] = v[i];
   }
   __syncthreads();
+  if (a.vectorStores) {
+    // A thread gathers 16 bytes of consecutive batch entries of one channel
+    // (consecutive rows of the tile); consecutive lanes take consecutive
+    // such pieces, then the next channel.  The batch size and every stride
+    // are multiples of the vector length.
+    constexpr uint32_t kVec = 16 / sizeof(T);
+    constexpr uint32_t kPieces = kSwapRows / kVec;
+#pragma unroll 2
+    for (uint32_t i = threadIdx.x; i < kSwapChans * kPieces; i += 256) {
+      const uint32_t cLocal = i / kPieces, row = (i % kPieces) * kVec;
+      const uint32_t p = p0 + row / a.batchPerTile;
+      const uint32_t b = b0 + row % a.batchPerTile;
+      const uint32_t c = c0 + cLocal;
+      if (p < a.pixels && b < a.batch && c < a.chans) {
+        union {
+          uint4 raw;
+          T e[kVec];
+        } v;
+#pragma unroll
+        for (uint32_t k = 0; k != kVec; ++k)
+          v.e[k] = T(tile[row + k][cLocal]);
+        *reinterpret_cast<uint4 *>(dst + g * a.strideG + c * a.strideC +
+                                   p * a.strideP + b) = v.raw;
+      }
+    }
+    return;
+  }
   // 64 lanes = 64 consecutive rows of the tile: consecutive batch entries,
   // then the next pixel.
 #pragma unroll 4
@@ -390,9 +418,15 @@ hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
   if (gx > 0x7fffffffull || gy > 65535 || gz > 65535)
     return hipErrorInvalidConfiguration;
   const dim3 grid{uint32_t(gx), uint32_t(gy), uint32_t(gz)}, block{256};
-  // 16-byte loads need every row of channels to start on a 16-byte boundary.
-  const bool vec = chans % uint32_t(16 / elemBytes) == 0 &&
+  // 16-byte loads need every row of channels to start on a 16-byte boundary;
+  // 16-byte stores, every run of batch entries.
+  const uint32_t perVector = uint32_t(16 / elemBytes);
+  const bool vec = chans % perVector == 0 &&
                    reinterpret_cast<uintptr_t>(src) % 16 == 0;
+  a.vectorStores = batch % perVector == 0 && a.batchPerTile >= perVector &&
+                   strideG % perVector == 0 && strideC % perVector == 0 &&
+                   strideP % perVector == 0 &&
+                   reinterpret_cast<uintptr_t>(dst) % 16 == 0;
   if (elemBytes == 2) {
     const auto *from = static_cast<const uint16_t *>(src);
     auto *to = static_cast<uint16_t *>(dst);
