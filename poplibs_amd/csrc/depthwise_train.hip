@@ -85,23 +85,38 @@ __global__ __launch_bounds__(256) void depthwiseDirectKernel(
   const int ihBase = int(oh * d.strideH) - d.padH;
   const int iwBase = int(ow * d.strideW) - d.padW;
   const __half *image = in + size_t(b) * d.inH * d.inW * d.channels + c;
-  for (uint32_t kh = 0; kh != d.kH; ++kh) {
-    const int ihD = ihBase + int(kh * d.dilH);
-    const uint32_t ih = a.divInDilH(uint32_t(ihD));
-    if (ihD < 0 || ih * d.inDilH != uint32_t(ihD) || ih < d.loH || ih >= d.hiH)
-      continue;
-    for (uint32_t kw = 0; kw != d.kW; ++kw) {
-      const int iwD = iwBase + int(kw * d.dilW);
+  // Validity is separable: the kernel columns that read an input element
+  // are worked out once (a bit each - up to 32 columns at a time), then for
+  // every valid kernel row only those columns are visited.
+  for (uint32_t kw0 = 0; kw0 < d.kW; kw0 += 32) {
+    uint32_t columns = 0;
+    const uint32_t kwEnd = min(d.kW - kw0, 32u);
+    for (uint32_t j = 0; j != kwEnd; ++j) {
+      const int iwD = iwBase + int((kw0 + j) * d.dilW);
       const uint32_t iw = a.divInDilW(uint32_t(iwD));
-      if (iwD < 0 || iw * d.inDilW != uint32_t(iwD) || iw < d.loW ||
-          iw >= d.hiW)
+      if (iwD >= 0 && iw * d.inDilW == uint32_t(iwD) && iw >= d.loW &&
+          iw < d.hiW)
+        columns |= 1u << j;
+    }
+    if (columns == 0)
+      continue;
+    for (uint32_t kh = 0; kh != d.kH; ++kh) {
+      const int ihD = ihBase + int(kh * d.dilH);
+      const uint32_t ih = a.divInDilH(uint32_t(ihD));
+      if (ihD < 0 || ih * d.inDilH != uint32_t(ihD) || ih < d.loH ||
+          ih >= d.hiH)
         continue;
-      Vec8 x, k;
-      x.raw = *reinterpret_cast<const uint4 *>(
-          image + (size_t(ih) * d.inW + iw) * d.channels);
-      k.raw = *reinterpret_cast<const uint4 *>(
-          w + size_t(kh * d.kW + kw) * d.channels + c);
-      fma8(acc, x, k);
+      const __half *row = image + size_t(ih) * d.inW * d.channels;
+      const __half *taps = w + size_t(kh * d.kW + kw0) * d.channels + c;
+      for (uint32_t rest = columns; rest != 0; rest &= rest - 1) {
+        const uint32_t j = uint32_t(__ffs(int(rest))) - 1;
+        const uint32_t iw =
+            a.divInDilW(uint32_t(iwBase + int((kw0 + j) * d.dilW)));
+        Vec8 x, k;
+        x.raw = *reinterpret_cast<const uint4 *>(row + size_t(iw) * d.channels);
+        k.raw = *reinterpret_cast<const uint4 *>(taps + size_t(j) * d.channels);
+        fma8(acc, x, k);
+      }
     }
   }
   store8(out + size_t(pixel) * d.channels + c, acc);
