@@ -298,14 +298,15 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
  * poplin::multiconv::convolution (include/poplin/MultiConvolution.hpp:
  * 143-149): `n` independent forward passes, results as if each had been run
  * by mxconv_fwd / mxconv_fwd_quarter.  PopLibs runs them side by side on
- * disjoint tile ranges; here, with parallel != 0, they are spread over up to
- * four HIP streams (the caller's and three of the library's, all at default
- * priority) that fork from `stream` and join it again before the call
- * returns, so small convolutions share the chip; with parallel == 0 they run
- * on `stream` one after another.  Arrays have `n` entries; `bias`,
+ * disjoint tile ranges; here, with parallel != 0, convolutions that run the
+ * same matrix-core kernel (same tile width, element types, fp8 formats) are
+ * issued as ONE launch whose grid is the concatenation of their tiles, up to
+ * eight at a time, so that convolutions too small to fill the chip share it;
+ * the others, and everything with parallel == 0, run one after another.  All
+ * work is enqueued on `stream`.  Arrays have `n` entries; `bias`,
  * `workspaces` / `workspace_bytes` and the two metadata arrays may be NULL
  * (no bias, no workspace, metadata byte 0); metadata is read for plans with
- * QUARTER inputs only.  Calls on one device are serialised internally. */
+ * QUARTER inputs only. */
 mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
                                const void *const *in,
                                const uint8_t *in_metadata,

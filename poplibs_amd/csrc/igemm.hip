@@ -77,10 +77,13 @@ namespace {
 
 /// UNI: every k-step lies inside one kernel tap (Ci * EB is a multiple of
 /// 128 bytes), so tap and channel block are wave-uniform.
+/// The work of one workgroup: tile number `block` of the `blocks` tiles of
+/// convolution `a`.
 template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
-__global__ __launch_bounds__(kThreads) void igemmKernel(
-    IgemmArgs a, const char *__restrict__ in, const char *__restrict__ w,
-    const OutT *__restrict__ bias, OutT *__restrict__ out, float scale) {
+__device__ __forceinline__ void igemmTile(
+    const IgemmArgs &a, const char *__restrict__ in,
+    const char *__restrict__ w, const OutT *__restrict__ bias,
+    OutT *__restrict__ out, float scale, uint32_t block, uint32_t blocks) {
   constexpr int TN = BN / 64;              // 32-column MFMA tiles per wave
   constexpr int AROWS = kBlockM / kRowsPerPass; // A rows loaded per thread
   constexpr int BROWS = BN / kRowsPerPass;      // B rows loaded per thread
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
   uint2 *rowTable = reinterpret_cast<uint2 *>(lds + NS * kTileBytes);
 
   const IgemmDesc &d = a.d;
-  const uint32_t tile = xcdSwizzle(blockIdx.x, gridDim.x);
+  const uint32_t tile = xcdSwizzle(block, blocks);
   const uint32_t nTile = tile % a.nTiles;
   const uint32_t mTile = (tile / a.nTiles) % a.mTiles;
   const uint32_t gs = tile / (a.nTiles * a.mTiles);
@@ -455,70 +458,160 @@ __global__ __launch_bounds__(kThreads) void igemmKernel(
 }
 
 template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
-hipError_t run(const IgemmArgs &a, const void *in, const void *w,
-               const void *bias, void *out, float scale, hipStream_t stream) {
-  const uint64_t blocks =
-      uint64_t(a.mTiles) * a.nTiles * a.d.groups * a.d.splitK;
-  if (blocks == 0)
-    return hipSuccess;
-  if (blocks > 0x7fffffffull)
-    return hipErrorInvalidConfiguration;
-  constexpr int ldsBytes =
-      NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
-  // More than the 64 KB a kernel gets by default: raise the limit once.
-  static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void *>(&igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>),
-      hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
-  if (attr != hipSuccess)
-    return attr;
-  hipLaunchKernelGGL((igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>),
-                     dim3(uint32_t(blocks)), dim3(kThreads), ldsBytes, stream,
-                     a, static_cast<const char *>(in),
-                     static_cast<const char *>(w),
-                     static_cast<const OutT *>(bias), static_cast<OutT *>(out),
-                     scale);
-  return hipGetLastError();
+__global__ __launch_bounds__(kThreads) void igemmKernel(
+    IgemmArgs a, const char *__restrict__ in, const char *__restrict__ w,
+    const OutT *__restrict__ bias, OutT *__restrict__ out, float scale) {
+  igemmTile<BN, NS, EB, FA, FB, UNI, OutT>(a, in, w, bias, out, scale,
+                                           blockIdx.x, gridDim.x);
 }
 
-template <int BN, int EB, int FA, int FB>
-hipError_t runOut(const IgemmArgs &a, int outType, const void *in,
-                  const void *w, const void *bias, void *out, float scale,
-                  hipStream_t stream) {
-  const bool uni = (a.d.inChansPerGroup * EB) % kRowBytes == 0;
+/// Several convolutions that run the same kernel, in one launch: the grid is
+/// the concatenation of their tiles, so that convolutions too small to fill
+/// the chip share it.  (PopLibs' parallel multi-convolution plan gives each
+/// a disjoint range of tiles, lib/poplin/MultiConvolution.cpp:125-176.)
+constexpr int kMaxFused = int(kIgemmMaxFused);
+struct IgemmFusedArgs {
+  uint32_t count;
+  uint32_t firstBlock[kMaxFused + 1]; // prefix sums of the tile counts
+  IgemmArgs a[kMaxFused];
+  const char *in[kMaxFused];
+  const char *w[kMaxFused];
+  const void *bias[kMaxFused];
+  void *out[kMaxFused];
+  float scale[kMaxFused];
+};
+
+template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
+__global__ __launch_bounds__(kThreads) void igemmFusedKernel(IgemmFusedArgs m) {
+  uint32_t i = 0;
+  while (i + 1 < m.count && blockIdx.x >= m.firstBlock[i + 1])
+    ++i;
+  igemmTile<BN, NS, EB, FA, FB, UNI, OutT>(
+      m.a[i], m.in[i], m.w[i], static_cast<const OutT *>(m.bias[i]),
+      static_cast<OutT *>(m.out[i]), m.scale[i], blockIdx.x - m.firstBlock[i],
+      m.firstBlock[i + 1] - m.firstBlock[i]);
+}
+
+template <class Kernel>
+hipError_t raiseLdsLimit(Kernel kernel, int ldsBytes) {
+  // More than the 64 KB a kernel gets by default.
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                             ldsBytes);
+}
+
+/// What to launch once the kernel's template arguments are known: one
+/// convolution ...
+struct LaunchOne {
+  const IgemmArgs &a;
+  const void *in, *w, *bias;
+  void *out;
+  float scale;
+  hipStream_t stream;
+  template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
+  hipError_t go() const {
+    const uint64_t blocks =
+        uint64_t(a.mTiles) * a.nTiles * a.d.groups * a.d.splitK;
+    if (blocks == 0)
+      return hipSuccess;
+    if (blocks > 0x7fffffffull)
+      return hipErrorInvalidConfiguration;
+    constexpr int ldsBytes =
+        NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
+    static const hipError_t attr = raiseLdsLimit(
+        &igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>, ldsBytes);
+    if (attr != hipSuccess)
+      return attr;
+    hipLaunchKernelGGL((igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>),
+                       dim3(uint32_t(blocks)), dim3(kThreads), ldsBytes,
+                       stream, a, static_cast<const char *>(in),
+                       static_cast<const char *>(w),
+                       static_cast<const OutT *>(bias),
+                       static_cast<OutT *>(out), scale);
+    return hipGetLastError();
+  }
+};
+
+/// ... or several in one grid.
+struct LaunchFused {
+  const IgemmFusedArgs &m;
+  hipStream_t stream;
+  template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
+  hipError_t go() const {
+    const uint32_t blocks = m.firstBlock[m.count];
+    if (blocks == 0)
+      return hipSuccess;
+    constexpr int ldsBytes =
+        NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
+    static const hipError_t attr = raiseLdsLimit(
+        &igemmFusedKernel<BN, NS, EB, FA, FB, UNI, OutT>, ldsBytes);
+    if (attr != hipSuccess)
+      return attr;
+    hipLaunchKernelGGL((igemmFusedKernel<BN, NS, EB, FA, FB, UNI, OutT>),
+                       dim3(blocks), dim3(kThreads), ldsBytes, stream, m);
+    return hipGetLastError();
+  }
+};
+
+/// The kernel instantiation a convolution runs.
+struct KernelKey {
+  int blockN, inType, outType, fa, fb;
+  bool uni;
+  bool operator==(const KernelKey &o) const {
+    return blockN == o.blockN && inType == o.inType && outType == o.outType &&
+           fa == o.fa && fb == o.fb && uni == o.uni;
+  }
+};
+
+KernelKey kernelKey(const IgemmDesc &d, int inType, int outType,
+                    const QuarterInfo &q) {
+  const int eb = inType == kHalf ? 2 : 1;
+  KernelKey k;
+  k.blockN = int(d.blockN), k.inType = inType, k.outType = outType;
+  // Instruction format codes: 0 = E4M3, 1 = E5M2.
+  k.fa = inType == kQuarter && q.inFormat != kE4M3 ? 1 : 0;
+  k.fb = inType == kQuarter && q.weightFormat != kE4M3 ? 1 : 0;
+  k.uni = (d.inChansPerGroup * eb) % kRowBytes == 0;
+  return k;
+}
+
+template <int BN, int EB, int FA, int FB, class Launch>
+hipError_t dispatchOut(const KernelKey &k, const Launch &launch) {
   // Stages of LDS: 4 x 32 KB for the 128-wide tile (one workgroup per CU);
   // 3 x 24 KB for the 64-wide one, so that two workgroups share a CU.
   constexpr int NS = BN == 128 ? 4 : 3;
-  if (outType == kHalf)
-    return uni ? run<BN, NS, EB, FA, FB, true, __half>(a, in, w, bias, out, scale,
-                                                   stream)
-               : run<BN, NS, EB, FA, FB, false, __half>(a, in, w, bias, out, scale,
-                                                    stream);
-  if (outType == kFloat)
-    return uni ? run<BN, NS, EB, FA, FB, true, float>(a, in, w, bias, out, scale,
-                                                  stream)
-               : run<BN, NS, EB, FA, FB, false, float>(a, in, w, bias, out, scale,
-                                                   stream);
+  if (k.outType == kHalf)
+    return k.uni
+               ? launch.template go<BN, NS, EB, FA, FB, true, __half>()
+               : launch.template go<BN, NS, EB, FA, FB, false, __half>();
+  if (k.outType == kFloat)
+    return k.uni ? launch.template go<BN, NS, EB, FA, FB, true, float>()
+                 : launch.template go<BN, NS, EB, FA, FB, false, float>();
   return hipErrorInvalidValue;
 }
 
-template <int BN>
-hipError_t runType(const IgemmArgs &a, int inType, int outType, const void *in,
-                   const void *w, const void *bias, void *out,
-                   const QuarterInfo &q, hipStream_t stream) {
-  if (inType == kHalf)
-    return runOut<BN, 2, 0, 0>(a, outType, in, w, bias, out, 1.0f, stream);
-  if (inType != kQuarter)
+template <int BN, class Launch>
+hipError_t dispatchType(const KernelKey &k, const Launch &launch) {
+  if (k.inType == kHalf)
+    return dispatchOut<BN, 2, 0, 0>(k, launch);
+  if (k.inType != kQuarter)
     return hipErrorInvalidValue;
-  // Instruction format codes: 0 = E4M3, 1 = E5M2.
-  const int fa = q.inFormat == kE4M3 ? 0 : 1;
-  const int fb = q.weightFormat == kE4M3 ? 0 : 1;
-  if (fa == 0 && fb == 0)
-    return runOut<BN, 1, 0, 0>(a, outType, in, w, bias, out, q.scale, stream);
-  if (fa == 0 && fb == 1)
-    return runOut<BN, 1, 0, 1>(a, outType, in, w, bias, out, q.scale, stream);
-  if (fa == 1 && fb == 0)
-    return runOut<BN, 1, 1, 0>(a, outType, in, w, bias, out, q.scale, stream);
-  return runOut<BN, 1, 1, 1>(a, outType, in, w, bias, out, q.scale, stream);
+  if (k.fa == 0 && k.fb == 0)
+    return dispatchOut<BN, 1, 0, 0>(k, launch);
+  if (k.fa == 0 && k.fb == 1)
+    return dispatchOut<BN, 1, 0, 1>(k, launch);
+  if (k.fa == 1 && k.fb == 0)
+    return dispatchOut<BN, 1, 1, 0>(k, launch);
+  return dispatchOut<BN, 1, 1, 1>(k, launch);
+}
+
+template <class Launch>
+hipError_t dispatch(const KernelKey &k, const Launch &launch) {
+  if (k.blockN == 128)
+    return dispatchType<128>(k, launch);
+  if (k.blockN == 64)
+    return dispatchType<64>(k, launch);
+  return hipErrorInvalidValue;
 }
 
 /// out[i] = sum over parts of partial[part][i] (+ bias of i's channel).  The
@@ -575,45 +668,43 @@ size_t igemmWorkspaceBytes(const IgemmDesc &d) {
          d.outChansPerGroup * sizeof(float);
 }
 
-hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
-                       const void *in, const void *weightsPacked,
-                       const void *bias, void *out, void *workspace,
-                       const QuarterInfo &q, hipStream_t stream) {
+namespace {
+
+/// Checks `d` against what the kernels are compiled for (the planner only
+/// produces such shapes) and fills in the kernel's arguments.
+hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
+                   IgemmArgs &a) {
   const uint32_t eb = inType == kHalf ? 2 : 1;
   const uint32_t bke = kRowBytes / eb;
   const int mode = igemmTapAddressing(d);
-  const bool general = mode == kDilatedTaps;
-  // The shapes the kernel is compiled for; the planner only produces these.
+  const bool dilated = mode == kDilatedTaps;
   if (d.blockM != kBlockM || (d.blockN != 64 && d.blockN != 128) ||
       d.blockK != bke || d.inChansPerGroup % (16 / eb) != 0 ||
       (inType != kHalf && inType != kQuarter) || d.splitK == 0 ||
       d.inDilH == 0 || d.inDilW == 0)
     return hipErrorInvalidValue;
-  // The general addressing keeps window origins as 16-bit offsets from
-  // -32768 and never reaches a tap beyond +32767 of them.
-  if (general &&
+  // The arithmetic addressing keeps window origins as 16-bit offsets from
+  // -32768 and never reaches a tap beyond +32767 of them; its
+  // multiplications are 24-bit ones.
+  if (dilated &&
       (uint64_t(d.outH) * d.strideH + uint64_t(d.kH) * d.dilH +
                uint64_t(d.padH > 0 ? d.padH : -d.padH) >=
            32768 ||
        uint64_t(d.outW) * d.strideW + uint64_t(d.kW) * d.dilW +
                uint64_t(d.padW > 0 ? d.padW : -d.padW) >=
-           32768))
+           32768 ||
+       uint64_t(d.inW) * d.groups * d.inChansPerGroup * eb >= (1u << 24) ||
+       d.inH >= (1u << 24) || d.inDilH >= (1u << 24) ||
+       d.inDilW >= (1u << 24)))
     return hipErrorInvalidValue;
-  if (d.splitK > 1 &&
-      (!workspace || (d.groups * d.outChansPerGroup) % 4 != 0))
-    return hipErrorInvalidValue;
-  IgemmArgs a;
-  a.d = d;
-  a.mode = uint32_t(mode);
   // the ranges of valid kernel rows and columns are kept in 8 bits each
   if (mode == kRangeTaps && (d.kH > 255 || d.kW > 255))
     return hipErrorInvalidValue;
-  // its multiplications are 24-bit ones
-  if (general && (uint64_t(d.inW) * d.groups * d.inChansPerGroup * eb >=
-                      (1u << 24) ||
-                  d.inH >= (1u << 24) || d.inDilH >= (1u << 24) ||
-                  d.inDilW >= (1u << 24)))
+  if (d.splitK > 1 &&
+      (!haveWorkspace || (d.groups * d.outChansPerGroup) % 4 != 0))
     return hipErrorInvalidValue;
+  a.d = d;
+  a.mode = uint32_t(mode);
   a.divInDilH = makeFastDiv(d.inDilH);
   a.divInDilW = makeFastDiv(d.inDilW);
   a.divCiBytes = makeFastDiv(d.inChansPerGroup * eb);
@@ -642,20 +733,27 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
     return hipErrorInvalidConfiguration;
   a.inBytes = uint32_t(inBytes);
   a.wBytes = uint32_t(wBytes);
-  if (d.splitK == 1) {
-    if (d.blockN == 128)
-      return runType<128>(a, inType, outType, in, weightsPacked, bias, out, q,
-                          stream);
-    return runType<64>(a, inType, outType, in, weightsPacked, bias, out, q,
-                       stream);
-  }
+  return hipSuccess;
+}
+
+} // namespace
+
+hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
+                       const void *in, const void *weightsPacked,
+                       const void *bias, void *out, void *workspace,
+                       const QuarterInfo &q, hipStream_t stream) {
+  IgemmArgs a;
+  hipError_t e = prepare(d, inType, workspace != nullptr, a);
+  if (e != hipSuccess)
+    return e;
+  const float scale = inType == kQuarter ? q.scale : 1.0f;
+  if (d.splitK == 1)
+    return dispatch(kernelKey(d, inType, outType, q),
+                    LaunchOne{a, in, weightsPacked, bias, out, scale, stream});
   // fp32 partial tiles per part (scaled, without bias), then their sum.
-  const hipError_t e =
-      d.blockN == 128
-          ? runType<128>(a, inType, kFloat, in, weightsPacked, nullptr,
-                         workspace, q, stream)
-          : runType<64>(a, inType, kFloat, in, weightsPacked, nullptr,
-                        workspace, q, stream);
+  e = dispatch(kernelKey(d, inType, kFloat, q),
+               LaunchOne{a, in, weightsPacked, nullptr, workspace, scale,
+                         stream});
   if (e != hipSuccess)
     return e;
   const uint32_t channels = d.groups * d.outChansPerGroup;
@@ -679,6 +777,44 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
+}
+
+bool igemmFusable(const IgemmFusedItem &x, const IgemmFusedItem &y) {
+  return x.d->splitK == 1 && y.d->splitK == 1 &&
+         kernelKey(*x.d, x.inType, x.outType, x.q) ==
+             kernelKey(*y.d, y.inType, y.outType, y.q);
+}
+
+hipError_t launchIgemmFused(const IgemmFusedItem *items, size_t count,
+                            hipStream_t stream) {
+  if (count == 0)
+    return hipSuccess;
+  if (count > size_t(kMaxFused))
+    return hipErrorInvalidValue;
+  IgemmFusedArgs m{};
+  m.count = uint32_t(count);
+  uint64_t blocks = 0;
+  for (size_t i = 0; i != count; ++i) {
+    const IgemmFusedItem &x = items[i];
+    if (!igemmFusable(items[0], x))
+      return hipErrorInvalidValue;
+    const hipError_t e = prepare(*x.d, x.inType, false, m.a[i]);
+    if (e != hipSuccess)
+      return e;
+    m.firstBlock[i] = uint32_t(blocks);
+    blocks += uint64_t(m.a[i].mTiles) * m.a[i].nTiles * x.d->groups;
+    if (blocks > 0x7fffffffull)
+      return hipErrorInvalidConfiguration;
+    m.in[i] = static_cast<const char *>(x.in);
+    m.w[i] = static_cast<const char *>(x.weightsPacked);
+    m.bias[i] = x.bias;
+    m.out[i] = x.out;
+    m.scale[i] = x.inType == kQuarter ? x.q.scale : 1.0f;
+  }
+  m.firstBlock[count] = uint32_t(blocks);
+  return dispatch(kernelKey(*items[0].d, items[0].inType, items[0].outType,
+                            items[0].q),
+                  LaunchFused{m, stream});
 }
 
 } // namespace mxk

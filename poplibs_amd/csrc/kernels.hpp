@@ -134,6 +134,21 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
                        const void *bias, void *out, void *workspace,
                        const QuarterInfo &q, hipStream_t stream);
 
+/// Several convolutions that run the same igemm kernel (same tile width,
+/// types, fp8 formats, channel-block alignment; K not split) as ONE launch
+/// whose grid is the concatenation of their tiles - at most 8 at a time.
+struct IgemmFusedItem {
+  const IgemmDesc *d;
+  int inType, outType;
+  const void *in, *weightsPacked, *bias;
+  void *out;
+  QuarterInfo q;
+};
+constexpr size_t kIgemmMaxFused = 8;
+bool igemmFusable(const IgemmFusedItem &x, const IgemmFusedItem &y);
+hipError_t launchIgemmFused(const IgemmFusedItem *items, size_t count,
+                            hipStream_t stream);
+
 /// Pointwise convolution (every kernel extent 1, stride 1, no padding or
 /// truncation, half inputs) with 128, 256 or 512 input channels per group:
 /// a streaming kernel of small workgroups instead of igemm's big tiles.

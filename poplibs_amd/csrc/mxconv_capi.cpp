@@ -11,13 +11,12 @@
 #include "poplin/ConvUtil.hpp"
 #include "poputil/exceptions.hpp"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <new>
 #include <sstream>
-#include <map>
 #include <memory>
-#include <mutex>
 #include <string>
 #include <vector>
 
@@ -104,10 +103,11 @@ mxk::QuarterInfo quarterInfo(uint8_t inMeta, uint8_t wMeta) {
   return q;
 }
 
-mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
-                      const void *bias, void *out, void *workspace,
-                      size_t workspaceBytes, const mxk::QuarterInfo &q,
-                      mxconv_stream stream) {
+/// The argument checks of a forward pass; MXCONV_OK also when there is
+/// nothing to compute (no output elements).
+mxconv_status checkForward(const mxconv_plan *plan, const void *in,
+                           const void *w, const void *out,
+                           const void *workspace, size_t workspaceBytes) {
   REQUIRE_ARG(plan);
   if (plan->outputElems == 0)
     return MXCONV_OK;
@@ -121,6 +121,17 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
     return fail(MXCONV_WORKSPACE_TOO_SMALL,
                 "workspace of " + std::to_string(plan->workspaceBytes) +
                     " bytes required");
+  return MXCONV_OK;
+}
+
+mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
+                      const void *bias, void *out, void *workspace,
+                      size_t workspaceBytes, const mxk::QuarterInfo &q,
+                      mxconv_stream stream) {
+  const mxconv_status checked =
+      checkForward(plan, in, w, out, workspace, workspaceBytes);
+  if (checked != MXCONV_OK || plan->outputElems == 0)
+    return checked;
   const int inType = plan->params.inputType.id();
   const int outType = plan->params.outputType.id();
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -624,53 +635,6 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
 
 // ---- several convolutions at once -----------------------------------------
 
-} // extern "C"
-
-namespace {
-
-/// The library's worker streams and the events that fork them from, and join
-/// them to, a caller's stream; one set per device, made on first use and kept
-/// for the life of the process.
-struct WorkerStreams {
-  static constexpr int kWorkers = 3;
-  std::mutex mutex;
-  bool ready = false;
-  hipStream_t streams[kWorkers] = {};
-  hipEvent_t fork = nullptr, join[kWorkers] = {};
-};
-
-WorkerStreams *workerStreams(hipError_t *error) {
-  static std::mutex tableMutex;
-  static std::map<int, std::unique_ptr<WorkerStreams>> table;
-  int device = 0;
-  *error = hipGetDevice(&device);
-  if (*error != hipSuccess)
-    return nullptr;
-  std::lock_guard<std::mutex> lock(tableMutex);
-  auto &entry = table[device];
-  if (!entry)
-    entry.reset(new WorkerStreams);
-  if (!entry->ready) {
-    for (auto &s : entry->streams)
-      if ((*error = hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) !=
-          hipSuccess)
-        return nullptr;
-    if ((*error = hipEventCreateWithFlags(&entry->fork,
-                                          hipEventDisableTiming)) != hipSuccess)
-      return nullptr;
-    for (auto &e : entry->join)
-      if ((*error = hipEventCreateWithFlags(&e, hipEventDisableTiming)) !=
-          hipSuccess)
-        return nullptr;
-    entry->ready = true;
-  }
-  return entry.get();
-}
-
-} // namespace
-
-extern "C" {
-
 mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
                                const void *const *in,
                                const uint8_t *in_metadata,
@@ -687,52 +651,108 @@ mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
   REQUIRE_ARG(in);
   REQUIRE_ARG(weights_packed);
   REQUIRE_ARG(out);
-  for (size_t i = 0; i != n; ++i)
-    REQUIRE_ARG(plans[i]);
-  auto launch = [&](size_t i, hipStream_t s) {
-    const mxk::QuarterInfo q =
-        plans[i]->params.inputType == poplar::QUARTER
-            ? quarterInfo(in_metadata ? in_metadata[i] : 0,
-                          weights_metadata ? weights_metadata[i] : 0)
-            : mxk::QuarterInfo{};
-    return forward(plans[i], in[i], weights_packed[i], bias ? bias[i] : nullptr,
-                   out[i], workspaces ? workspaces[i] : nullptr,
-                   workspace_bytes ? workspace_bytes[i] : 0, q,
-                   reinterpret_cast<mxconv_stream>(s));
+  auto quarter = [&](size_t i) {
+    return plans[i]->params.inputType == poplar::QUARTER
+               ? quarterInfo(in_metadata ? in_metadata[i] : 0,
+                             weights_metadata ? weights_metadata[i] : 0)
+               : mxk::QuarterInfo{};
   };
-  hipStream_t main = reinterpret_cast<hipStream_t>(stream);
-  if (!parallel || n == 1) {
-    for (size_t i = 0; i != n; ++i) {
-      const mxconv_status st = launch(i, main);
-      if (st != MXCONV_OK)
-        return st;
+  auto workspace = [&](size_t i) {
+    return workspaces ? workspaces[i] : nullptr;
+  };
+  auto workspaceSize = [&](size_t i) {
+    return workspace_bytes ? workspace_bytes[i] : size_t(0);
+  };
+  // Everything is checked before anything is launched.
+  for (size_t i = 0; i != n; ++i) {
+    const mxconv_status st =
+        checkForward(plans[i], in[i], weights_packed[i], out[i], workspace(i),
+                     workspaceSize(i));
+    if (st != MXCONV_OK)
+      return st;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // A convolution can share a launch when the matrix-core kernel runs it.
+  // A plan that cuts K into parts does so because the convolution alone has
+  // too few tiles for the chip; in company that may no longer hold, so the
+  // shared launch runs it with K in one piece (descriptor copies below) when
+  // that is estimated to be faster than the members one by one as planned
+  // (measured: about 6 us per launch, 0.3 us per k-step of a workgroup, 5 us
+  // for the sum of a split K's parts).
+  mxk::IgemmDesc unsplit[mxk::kIgemmMaxFused];
+  auto tilesOf = [](const mxk::IgemmDesc &d) {
+    const uint64_t m = uint64_t(d.batch) * d.outH * d.outW;
+    return (m + d.blockM - 1) / d.blockM *
+           ((d.outChansPerGroup + d.blockN - 1) / d.blockN) * d.groups;
+  };
+  auto kStepsOf = [](const mxk::IgemmDesc &d) {
+    const uint64_t k = uint64_t(d.kH) * d.kW * d.inChansPerGroup;
+    return (k + d.blockK - 1) / d.blockK;
+  };
+  auto fusedItem = [&](size_t i, size_t slot, mxk::IgemmFusedItem &item) {
+    const mxconv_plan *p = plans[i];
+    if (p->outputElems == 0 || p->kernel != mxconv_plan::Kernel::IGEMM ||
+        p->pointwiseOn)
+      return false;
+    unsplit[slot] = p->igemm;
+    unsplit[slot].splitK = 1;
+    item = {&unsplit[slot],
+            p->params.inputType.id(),
+            p->params.outputType.id(),
+            in[i],
+            weights_packed[i],
+            bias ? bias[i] : nullptr,
+            out[i],
+            quarter(i)};
+    return true;
+  };
+  std::vector<bool> done(n, false);
+  for (size_t i = 0; i != n; ++i) {
+    if (done[i])
+      continue;
+    done[i] = true;
+    mxk::IgemmFusedItem group[mxk::kIgemmMaxFused];
+    size_t member[mxk::kIgemmMaxFused] = {i};
+    size_t members = 0;
+    double alone = 0, together = 0;
+    if (parallel && fusedItem(i, 0, group[0])) {
+      members = 1;
+      for (size_t j = i + 1; j != n && members != mxk::kIgemmMaxFused; ++j) {
+        mxk::IgemmFusedItem item;
+        if (!done[j] && fusedItem(j, members, item) &&
+            mxk::igemmFusable(group[0], item)) {
+          member[members] = j;
+          group[members++] = item;
+        }
+      }
+      uint64_t tiles = 0, longest = 0;
+      for (size_t k = 0; k != members; ++k) {
+        const mxk::IgemmDesc &planned = plans[member[k]]->igemm;
+        const uint64_t steps = kStepsOf(planned), own = tilesOf(planned);
+        const uint64_t rounds = (own * planned.splitK + 255) / 256;
+        alone += 6 + 0.3 * double((steps + planned.splitK - 1) /
+                                  planned.splitK * rounds) +
+                 (planned.splitK != 1 ? 5 : 0);
+        tiles += own;
+        longest = std::max(longest, steps);
+      }
+      together = 6 + 0.3 * double(longest * ((tiles + 255) / 256));
     }
-    return MXCONV_OK;
+    mxconv_status st;
+    if (members >= 2 && together < alone) {
+      for (size_t k = 0; k != members; ++k)
+        done[member[k]] = true;
+      st = hipStatus(mxk::launchIgemmFused(group, members, s),
+                     "fused implicit-GEMM convolution launch");
+    } else {
+      st = forward(plans[i], in[i], weights_packed[i],
+                   bias ? bias[i] : nullptr, out[i], workspace(i),
+                   workspaceSize(i), quarter(i), stream);
+    }
+    if (st != MXCONV_OK)
+      return st;
   }
-  hipError_t e = hipSuccess;
-  WorkerStreams *w = workerStreams(&e);
-  if (!w)
-    return hipStatus(e, "worker stream set-up");
-  std::lock_guard<std::mutex> lock(w->mutex);
-  const size_t lanes = std::min<size_t>(n, WorkerStreams::kWorkers + 1);
-  // fork: the workers wait for what `stream` holds so far
-  if ((e = hipEventRecord(w->fork, main)) != hipSuccess)
-    return hipStatus(e, "multi-convolution fork");
-  for (size_t l = 1; l != lanes; ++l)
-    if ((e = hipStreamWaitEvent(w->streams[l - 1], w->fork, 0)) != hipSuccess)
-      return hipStatus(e, "multi-convolution fork");
-  mxconv_status result = MXCONV_OK;
-  for (size_t i = 0; i != n && result == MXCONV_OK; ++i) {
-    const size_t lane = i % lanes;
-    result = launch(i, lane == 0 ? main : w->streams[lane - 1]);
-  }
-  // join, also after a failed launch: `stream` waits for every worker
-  for (size_t l = 1; l != lanes; ++l) {
-    if ((e = hipEventRecord(w->join[l - 1], w->streams[l - 1])) != hipSuccess ||
-        (e = hipStreamWaitEvent(main, w->join[l - 1], 0)) != hipSuccess)
-      return hipStatus(e, "multi-convolution join");
-  }
-  return result;
+  return MXCONV_OK;
 }
 
 mxconv_status mxconv_multiconv_validate_options(const char *const *keys,

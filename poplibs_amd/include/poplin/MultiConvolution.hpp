@@ -4,10 +4,11 @@
 //
 // Several independent convolutions are handed over together so that they can
 // share the device.  PopLibs gives each a disjoint range of IPU tiles; here
-// the forward passes are spread over HIP streams that fork from, and join,
-// the caller's stream, so that convolutions too small to fill 256 compute
-// units run side by side.  Results are those of the single-convolution
-// functions.
+// forward passes that run the same matrix-core kernel are issued as one
+// launch whose grid is the concatenation of their tiles, so that convolutions
+// too small to fill 256 compute units run side by side.  Results are those
+// of the single-convolution functions (to rounding, where a convolution's K
+// is cut into parts when it runs alone and stays whole in company).
 //
 // Multi-convolution options (lib/poplin/ConvPlan.cpp:1929-1953 of PopLibs):
 // planType = parallel (default) | serial; perConvReservedTiles and

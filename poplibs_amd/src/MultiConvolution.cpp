@@ -1,6 +1,6 @@
 // poplin::multiconv over the C ABI: operands are brought into the device
-// layouts on the caller's stream, then every forward pass goes to the device
-// in one mxconv_multi_fwd call.
+// layouts, then every forward pass goes to the device in one
+// mxconv_multi_fwd call, which fuses what it can into shared launches.
 #include "poplin/MultiConvolution.hpp"
 #include "LayerInternal.hpp"
 #include "poputil/exceptions.hpp"
