@@ -81,7 +81,7 @@ namespace {
 /// convolution `a`.
 template <int BN, int NS, int EB, int FA, int FB, bool UNI, class OutT>
 __device__ __forceinline__ void igemmTile(
-    const IgemmArgs &a, const char *__restrict__ in,
+    const IgemmArgs a, const char *__restrict__ in,
     const char *__restrict__ w, const OutT *__restrict__ bias,
     OutT *__restrict__ out, float scale, uint32_t block, uint32_t blocks) {
   constexpr int TN = BN / 64;              // 32-column MFMA tiles per wave
