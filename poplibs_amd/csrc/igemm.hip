@@ -120,7 +120,9 @@ __device__ __forceinline__ void igemmTile(
     // consumer's MFMAs: let their (short) vector instructions go first.
     __builtin_amdgcn_s_setprio(3);
     const int pt = t - (kThreads - kProducers);
-    const int pw = pt >> 6; // producer wave
+    // producer wave, as a scalar: what depends on it alone (LDS destinations
+    // of the loads) is then formed by scalar instructions
+    const int pw = __builtin_amdgcn_readfirstlane(pt >> 6);
     // Lane l of a load fills row position (l >> 3) of an 8-row block at chunk
     // position (l & 7).  This wave's blocks all have the parity of pw: in
     // odd blocks that position belongs to row (l >> 3) ^ 1; either way the
@@ -165,12 +167,22 @@ __device__ __forceinline__ void igemmTile(
     uint32_t kByte = kStart;
     auto loadB = [&](uint32_t stage) {
       char *base = lds + stage * kTileBytes + pw * kLoadBytes;
-      const uint32_t kOff = kByte < a.kPadded * EB ? kByte : kOutOfRange;
+      // The position along K travels in the scalar offset, which the range
+      // check leaves out: the steps beyond K - whole-wave events - ask for an
+      // out-of-range vector offset instead.
+      if (kByte < a.kPadded * EB) {
 #pragma unroll
-      for (int r = 0; r != BROWS; ++r)
-        loadToLds(wBuf,
-                  (LdsPtr)(base + kBlockM * kRowBytes + r * 4 * kLoadBytes),
-                  bOff[r] + kOff, 0);
+        for (int r = 0; r != BROWS; ++r)
+          loadToLds(wBuf,
+                    (LdsPtr)(base + kBlockM * kRowBytes + r * 4 * kLoadBytes),
+                    bOff[r], kByte);
+      } else {
+#pragma unroll
+        for (int r = 0; r != BROWS; ++r)
+          loadToLds(wBuf,
+                    (LdsPtr)(base + kBlockM * kRowBytes + r * 4 * kLoadBytes),
+                    kOutOfRange, 0);
+      }
       kByte += kRowBytes;
     };
 
@@ -262,6 +274,30 @@ __device__ __forceinline__ void igemmTile(
         } else {
           const uint32_t tapOff =
               (kh * d.dilH * d.inW + kw * d.dilW) * pixelBytes;
+          if constexpr (UNI && MODE == kMaskTaps) {
+            // tapMask holds the complement of the row's mask here: shifted so
+            // that the tap's bit lands on bit 31 and merged into the offset,
+            // it makes the offset out of range exactly when the tap reads
+            // padding - two vector instructions per row.
+            if (tap < taps) {
+              const uint32_t shiftToTop = 31 - tap;
+#pragma unroll
+              for (int r = 0; r != AROWS; ++r) {
+                LdsPtr dst = (LdsPtr)(base + r * 4 * kLoadBytes);
+                loadToLds(inBuf, dst,
+                          (rowOff[r] & 0x7fffffffu) |
+                              ((tapMask[r] << shiftToTop) & 0x80000000u),
+                          tapOff + ciOff);
+              }
+            } else {
+#pragma unroll
+              for (int r = 0; r != AROWS; ++r)
+                loadToLds(inBuf, (LdsPtr)(base + r * 4 * kLoadBytes),
+                          kOutOfRange, 0);
+            }
+            advance();
+            return;
+          }
           const uint32_t tapBit = tap < taps ? (1u << (tap & 31)) : 0u;
 #pragma unroll
           for (int r = 0; r != AROWS; ++r) {
@@ -288,7 +324,9 @@ __device__ __forceinline__ void igemmTile(
       for (int r = 0; r != AROWS; ++r) {
         const uint2 e = rowTable[(r * 4 + pw) * 8 + rowInBlock];
         rowOff[r] = e.x + chunk * 16;
-        tapMask[r] = GEN ? uint32_t(int(e.y >> 16) - 32768) : e.y;
+        tapMask[r] = GEN ? uint32_t(int(e.y >> 16) - 32768)
+                     : UNI && MODE == kMaskTaps ? ~e.y
+                                                : e.y;
         originW[r] = int(e.y & 0xffffu) - 32768;
         khLo[r] = e.y & 0xffu, khSpan[r] = (e.y >> 8) & 0xffu;
         kwLo[r] = (e.y >> 16) & 0xffu, kwSpan[r] = e.y >> 24;
