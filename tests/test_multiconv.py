@@ -113,6 +113,61 @@ def test_multi_fwd_equals_single_convolutions(oracle, parallel):
 
 
 @pytest.mark.gpu
+def test_shared_launch_with_biases_and_groups(oracle):
+    # three convolutions of one kernel instantiation, each with its own bias
+    # (one without), one of them grouped: the shared launch takes each
+    # member's own arguments
+    import torch
+    from gpu_helpers import device, quantize, run_conv
+    rng = np.random.default_rng(43)
+    dev = torch.device("cuda:0")
+    cases = [(dict(batch=2, field=(6, 7), kernel=(3, 3), ci=64, co=72, pad=1),
+              True),
+             (dict(batch=1, field=(9, 9), kernel=(1, 1), ci=128, co=130), False),
+             (dict(batch=2, field=(5, 5), kernel=(2, 2), ci=64, co=80,
+                   groups=2), True)]
+    plans, ins, ws, outs, biases, keep, want, shapes = ([], [], [], [], [], [],
+                                                       [], [])
+    for kw, with_bias in cases:
+        p = make_params(pa.HALF, pa.FLOAT, **kw)
+        G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                     p.outputChannelsPerConvGroup)
+        xq, _ = quantize(rng.standard_normal(
+            (p.batchSize, G * Ci, *p.inputFieldShape)), pa.HALF)
+        wq, _ = quantize(rng.standard_normal(
+            (G, Co, Ci, *p.kernelShape)) * 0.1, pa.HALF)
+        bq, _ = quantize(rng.standard_normal(G * Co), pa.FLOAT)
+        plan = pa.Plan(p)
+        assert "K split" not in plan.describe()
+        want.append(run_conv(p, xq, wq, bq if with_bias else None, plan=plan))
+        x_ext, w_ext = device(xq, pa.HALF), device(wq, pa.HALF)
+        x_int = torch.empty(plan.buffer_bytes(capi.BUF_INPUT),
+                            dtype=torch.uint8, device=dev)
+        w_pack = torch.empty(plan.buffer_bytes(capi.BUF_WEIGHTS_PACKED),
+                             dtype=torch.uint8, device=dev)
+        o_int = torch.empty(plan.buffer_bytes(capi.BUF_OUTPUT),
+                            dtype=torch.uint8, device=dev)
+        b_dev = device(bq, pa.FLOAT)
+        plan.acts_to_internal(x_ext.data_ptr(), x_int.data_ptr())
+        plan.pack_weights(w_ext.data_ptr(), w_pack.data_ptr())
+        plans.append(plan)
+        ins.append(x_int.data_ptr())
+        ws.append(w_pack.data_ptr())
+        outs.append(o_int.data_ptr())
+        biases.append(b_dev.data_ptr() if with_bias else None)
+        keep += [x_ext, w_ext, x_int, w_pack, o_int, b_dev]
+        shapes.append((p.batchSize, G * Co, *p.getOutputFieldShape()))
+    pa.multi_fwd(plans, ins, ws, outs, biases=biases)
+    torch.cuda.synchronize()
+    for plan, o_ptr, w, shape in zip(plans, outs, want, shapes):
+        o_ext = torch.empty(shape, dtype=torch.float32, device=dev)
+        plan.acts_to_external(o_ptr, o_ext.data_ptr())
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(o_ext.cpu().numpy().astype(np.float64),
+                                      w)
+
+
+@pytest.mark.gpu
 def test_multi_fwd_quarter_metadata(oracle):
     import torch
     from gpu_helpers import device, quantize, run_conv
