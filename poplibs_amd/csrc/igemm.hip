@@ -95,12 +95,16 @@ __device__ __forceinline__ void igemmTile(
   uint2 *rowTable = reinterpret_cast<uint2 *>(lds + NS * kTileBytes);
 
   const IgemmDesc &d = a.d;
+  // tile = ((part * groups + g) * mTiles + mTile) * nTiles + nTile, taken
+  // apart with multiply-high divisions: a generic division is some forty
+  // instructions, and every wave would run four of them before anything else.
   const uint32_t tile = xcdSwizzle(block, blocks);
-  const uint32_t nTile = tile % a.nTiles;
-  const uint32_t mTile = (tile / a.nTiles) % a.mTiles;
-  const uint32_t gs = tile / (a.nTiles * a.mTiles);
-  const uint32_t g = gs % d.groups;
-  const uint32_t part = gs / d.groups; // which part of K
+  const uint32_t overN = a.divNTiles(tile);
+  const uint32_t nTile = tile - overN * a.nTiles;
+  const uint32_t gs = a.divMTiles(overN);
+  const uint32_t mTile = overN - gs * a.mTiles;
+  const uint32_t part = a.divGroups(gs); // which part of K
+  const uint32_t g = gs - part * d.groups;
   out += size_t(part) * a.M * (d.groups * d.outChansPerGroup);
   const uint32_t mode = a.mode;
 
@@ -190,8 +194,9 @@ __device__ __forceinline__ void igemmTile(
     // (a compile-time choice inside, so that neither loop carries the other's
     // branches).  NS - 1 k-steps are in flight; the oldest is waited for
     // before each barrier.  Start-up order: all weight loads, then (row table
-    // ready) all input loads; from then on input and weight loads of one
-    // k-step together.
+    // ready) the input loads of step 0, the first barrier, the input loads of
+    // the other stages; from then on input and weight loads of one k-step
+    // together.
     auto produce = [&](auto modeTag) {
       constexpr int MODE = decltype(modeTag)::value;
       constexpr bool GEN = MODE == kDilatedTaps;
@@ -200,9 +205,9 @@ __device__ __forceinline__ void igemmTile(
       // wave-uniform.  Otherwise the same pair for this thread's own 16-byte
       // chunk.
       uint32_t aByte = kStart + (UNI ? 0 : chunk * 16);
-      uint32_t tap = aByte / ciBytes;
+      uint32_t tap = a.divCiBytes(aByte);
       uint32_t ciOff = aByte - tap * ciBytes;
-      uint32_t kh = tap / d.kW, kw = tap - kh * d.kW;
+      uint32_t kh = a.divKW(tap), kw = tap - kh * d.kW;
       auto advance = [&] {
         if constexpr (GEN) {
           // no loop, no branch: everything again from the byte position
@@ -331,11 +336,14 @@ __device__ __forceinline__ void igemmTile(
         khLo[r] = e.y & 0xffu, khSpan[r] = (e.y >> 8) & 0xffu;
         kwLo[r] = (e.y >> 16) & 0xffu, kwSpan[r] = e.y >> 24;
       }
-#pragma unroll
-      for (int s = 0; s != NS - 1; ++s)
-        loadA(s);
-      MXK_WAIT_VMCNT((NS - 2) * AROWS);
+      // The consumers start as soon as step 0 is there; the input loads of
+      // the other stages go out behind their back.
+      loadA(0);
+      MXK_WAIT_VMCNT(0);
       stepBarrier(); // barrier 0: step 0 is in LDS stage 0
+#pragma unroll
+      for (int s = 1; s != NS - 1; ++s)
+        loadA(s);
       for (uint32_t kt = 0; kt != a.kSteps; ++kt) {
         // Stage (kt - 1) % NS was multiplied before the last barrier: refill
         // it with step kt + NS - 1, then make sure step kt + 1 has landed.
@@ -409,16 +417,41 @@ __device__ __forceinline__ void igemmTile(
                 g * ciBytes,
             rowValid ? ranges : 0u};
       } else {
-        uint32_t kwMask = 0, mask = 0;
-        for (uint32_t kw = 0; kw != d.kW; ++kw) {
-          const int iw = iwBase + int(kw * d.dilW);
-          if (iw >= int(d.loW) && iw < int(d.hiW))
-            kwMask |= 1u << kw;
-        }
-        for (uint32_t kh = 0; kh != d.kH; ++kh) {
-          const int ih = ihBase + int(kh * d.dilH);
-          if (ih >= int(d.loH) && ih < int(d.hiH))
-            mask |= kwMask << (kh * d.kW);
+        uint32_t mask = 0;
+        if (d.dilH == 1 && d.dilW == 1) {
+          // Undilated kernel: the valid kernel columns are the interval
+          // [lo - base, hi - base) cut to the kernel, and so are the rows.
+          // Bits [first, last) of a word:
+          auto bitRange = [](int first, int last) {
+            return first < last ? uint32_t(((1ull << last) - 1) &
+                                           ~((1ull << first) - 1))
+                                : 0u;
+          };
+          auto cut = [](int v, int size) {
+            return v < 0 ? 0 : v > size ? size : v;
+          };
+          const int kW = int(d.kW), kH = int(d.kH);
+          const uint32_t kwMask = bitRange(cut(int(d.loW) - iwBase, kW),
+                                           cut(int(d.hiW) - iwBase, kW));
+          // one bit per valid kernel row, at that row's first tap; the
+          // product puts the column mask there (no carries: it is narrower
+          // than the distance between the bits)
+          const uint32_t rowStarts =
+              a.tapRowStarts & bitRange(cut(int(d.loH) - ihBase, kH) * kW,
+                                        cut(int(d.hiH) - ihBase, kH) * kW);
+          mask = kwMask * rowStarts;
+        } else {
+          uint32_t kwMask = 0;
+          for (uint32_t kw = 0; kw != d.kW; ++kw) {
+            const int iw = iwBase + int(kw * d.dilW);
+            if (iw >= int(d.loW) && iw < int(d.hiW))
+              kwMask |= 1u << kw;
+          }
+          for (uint32_t kh = 0; kh != d.kH; ++kh) {
+            const int ih = ihBase + int(kh * d.dilH);
+            if (ih >= int(d.loH) && ih < int(d.hiH))
+              mask |= kwMask << (kh * d.kW);
+          }
         }
         rowTable[t] = uint2{
             shift +
@@ -755,6 +788,14 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
   a.divOutH = makeFastDiv(d.outH);
   a.mTiles = (a.M + kBlockM - 1) / kBlockM;
   a.nTiles = (d.outChansPerGroup + d.blockN - 1) / d.blockN;
+  a.divNTiles = makeFastDiv(a.nTiles);
+  a.divMTiles = makeFastDiv(a.mTiles);
+  a.divGroups = makeFastDiv(d.groups);
+  // bit kh * kW for every kernel row (tap mask mode: at most 32 taps)
+  a.tapRowStarts = 0;
+  if (a.mode == kMaskTaps)
+    for (uint32_t kh = 0; kh != d.kH; ++kh)
+      a.tapRowStarts |= 1u << (kh * d.kW);
   a.coPadded = a.nTiles * d.blockN;
   const uint32_t k = d.kH * d.kW * d.inChansPerGroup;
   a.kPadded = (k + bke - 1) / bke * bke;

@@ -15,6 +15,8 @@ struct IgemmArgs {
   FastDiv divOutW, divOutH;
   FastDiv divInDilH, divInDilW;
   FastDiv divCiBytes, divKW; // by bytes of K per tap; by kernel width
+  FastDiv divNTiles, divMTiles, divGroups; // workgroup number -> tile
+  uint32_t tapRowStarts; // tap mask mode: bit kh * kW for every kernel row
   uint32_t mode;     // kMaskTaps, kRangeTaps or kDilatedTaps
   uint32_t M;        // batch * outH * outW
   uint32_t mTiles, nTiles;
