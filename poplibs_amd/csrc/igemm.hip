@@ -350,7 +350,7 @@ __device__ __forceinline__ void igemmTile(
         // The first time round the start-up order still shows in the queue.
         loadA((kt + NS - 1) % NS);
         loadB((kt + NS - 1) % NS);
-        if (kt == 0)
+        if (kt == 0 && NS > 2)
           MXK_WAIT_VMCNT((NS - 3) * AROWS + kLoads);
         else
           MXK_WAIT_VMCNT((NS - 2) * kLoads);
@@ -522,7 +522,8 @@ __device__ __forceinline__ void igemmTile(
   // LDS can be reused for the output tile.
   __syncthreads();
 
-  static_assert(epilogueLdsBytes<BN, OutT>() <= NS * kTileBytes,
+  static_assert(epilogueLdsBytes<BN, OutT>() <=
+                    igemmLdsBytes<BN, NS, OutT>(),
                 "epilogue tile fits LDS");
   igemmEpilogue<BN, OutT>(lds, a, acc, producer, t, lane, wm, wn, mTile, nTile,
                           g, bias, out, scale);
@@ -587,8 +588,7 @@ struct LaunchOne {
       return hipSuccess;
     if (blocks > 0x7fffffffull)
       return hipErrorInvalidConfiguration;
-    constexpr int ldsBytes =
-        NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
+    constexpr int ldsBytes = igemmLdsBytes<BN, NS, OutT>();
     static const hipError_t attr = raiseLdsLimit(
         &igemmKernel<BN, NS, EB, FA, FB, UNI, OutT>, ldsBytes);
     if (attr != hipSuccess)
@@ -612,8 +612,7 @@ struct LaunchFused {
     const uint32_t blocks = m.firstBlock[m.count];
     if (blocks == 0)
       return hipSuccess;
-    constexpr int ldsBytes =
-        NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
+    constexpr int ldsBytes = igemmLdsBytes<BN, NS, OutT>();
     static const hipError_t attr = raiseLdsLimit(
         &igemmFusedKernel<BN, NS, EB, FA, FB, UNI, OutT>, ldsBytes);
     if (attr != hipSuccess)
@@ -626,11 +625,11 @@ struct LaunchFused {
 
 /// The kernel instantiation a convolution runs.
 struct KernelKey {
-  int blockN, inType, outType, fa, fb;
+  int blockN, stages, inType, outType, fa, fb;
   bool uni;
   bool operator==(const KernelKey &o) const {
-    return blockN == o.blockN && inType == o.inType && outType == o.outType &&
-           fa == o.fa && fb == o.fb && uni == o.uni;
+    return blockN == o.blockN && stages == o.stages && inType == o.inType &&
+           outType == o.outType && fa == o.fa && fb == o.fb && uni == o.uni;
   }
 };
 
@@ -639,6 +638,7 @@ KernelKey kernelKey(const IgemmDesc &d, int inType, int outType,
   const int eb = inType == kHalf ? 2 : 1;
   KernelKey k;
   k.blockN = int(d.blockN), k.inType = inType, k.outType = outType;
+  k.stages = d.blockN == 128 ? int(d.stages) : 3;
   // Instruction format codes: 0 = E4M3, 1 = E5M2.
   k.fa = inType == kQuarter && q.inFormat != kE4M3 ? 1 : 0;
   k.fb = inType == kQuarter && q.weightFormat != kE4M3 ? 1 : 0;
@@ -646,11 +646,8 @@ KernelKey kernelKey(const IgemmDesc &d, int inType, int outType,
   return k;
 }
 
-template <int BN, int EB, int FA, int FB, class Launch>
+template <int BN, int NS, int EB, int FA, int FB, class Launch>
 hipError_t dispatchOut(const KernelKey &k, const Launch &launch) {
-  // Stages of LDS: 4 x 32 KB for the 128-wide tile (one workgroup per CU);
-  // 3 x 24 KB for the 64-wide one, so that two workgroups share a CU.
-  constexpr int NS = BN == 128 ? 4 : 3;
   if (k.outType == kHalf)
     return k.uni
                ? launch.template go<BN, NS, EB, FA, FB, true, __half>()
@@ -661,19 +658,34 @@ hipError_t dispatchOut(const KernelKey &k, const Launch &launch) {
   return hipErrorInvalidValue;
 }
 
+template <int BN, int EB, int FA, int FB, class Launch>
+hipError_t dispatchStages(const KernelKey &k, const Launch &launch) {
+  // Stages of LDS.  128-wide tile: 4 x 32 KB (one workgroup per CU) or
+  // 2 x 32 KB (two per CU); 64-wide tile: 3 x 24 KB (two per CU).
+  if constexpr (BN == 128) {
+    if (k.stages == 4)
+      return dispatchOut<BN, 4, EB, FA, FB>(k, launch);
+    if (k.stages == 2)
+      return dispatchOut<BN, 2, EB, FA, FB>(k, launch);
+    return hipErrorInvalidValue;
+  } else {
+    return dispatchOut<BN, 3, EB, FA, FB>(k, launch);
+  }
+}
+
 template <int BN, class Launch>
 hipError_t dispatchType(const KernelKey &k, const Launch &launch) {
   if (k.inType == kHalf)
-    return dispatchOut<BN, 2, 0, 0>(k, launch);
+    return dispatchStages<BN, 2, 0, 0>(k, launch);
   if (k.inType != kQuarter)
     return hipErrorInvalidValue;
   if (k.fa == 0 && k.fb == 0)
-    return dispatchOut<BN, 1, 0, 0>(k, launch);
+    return dispatchStages<BN, 1, 0, 0>(k, launch);
   if (k.fa == 0 && k.fb == 1)
-    return dispatchOut<BN, 1, 0, 1>(k, launch);
+    return dispatchStages<BN, 1, 0, 1>(k, launch);
   if (k.fa == 1 && k.fb == 0)
-    return dispatchOut<BN, 1, 1, 0>(k, launch);
-  return dispatchOut<BN, 1, 1, 1>(k, launch);
+    return dispatchStages<BN, 1, 1, 0>(k, launch);
+  return dispatchStages<BN, 1, 1, 1>(k, launch);
 }
 
 template <class Launch>

@@ -219,6 +219,15 @@ template <int BN, class OutT> constexpr int epilogueLdsBytes() {
   return kBlockM * (BN * int(sizeof(OutT)) + 16);
 }
 
+/// LDS of a workgroup: the stages and the row table - or the output tile, if
+/// that is larger (two stages and fp32 outputs).
+template <int BN, int NS, class OutT> constexpr int igemmLdsBytes() {
+  constexpr int loop =
+      NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
+  return loop > epilogueLdsBytes<BN, OutT>() ? loop
+                                             : epilogueLdsBytes<BN, OutT>();
+}
+
 /// Writes the workgroup's finished 128 x BN tile.  Call with every wave past
 /// its last use of LDS (a workgroup barrier behind it): LDS is reused from
 /// offset 0.

@@ -121,6 +121,11 @@ struct IgemmDesc {
   // Parts K is cut into, one workgroup each; above 1 the launch needs
   // igemmWorkspaceBytes of scratch and adds the parts up in a second kernel.
   uint32_t splitK = 1;
+  // LDS stages of the 128-wide tile: 4 (one workgroup per CU, deep prefetch)
+  // or 2 (two workgroups per CU, which cover each other's start-up, barriers
+  // and epilogue: for grids of more workgroups than CUs).  The 64-wide tile
+  // always runs 3.
+  uint32_t stages = 4;
 };
 /// How the kernel finds out which kernel taps of an output pixel read inside
 /// the input: a bit mask per pixel (up to 32 taps), ranges of valid kernel

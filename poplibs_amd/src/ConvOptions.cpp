@@ -194,6 +194,8 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       pc.blockK = requireUnsigned(sub, m.second);
     } else if (m.first == "splitK") {
       pc.splitK = requireUnsigned(sub, m.second);
+    } else if (m.first == "stages") {
+      pc.stages = requireUnsigned(sub, m.second);
     } else if (m.first == "tileH") {
       pc.tileH = requireUnsigned(sub, m.second);
     } else if (m.first == "tileW") {

@@ -37,6 +37,7 @@ struct PlanConstraints {
   unsigned blockM = 0, blockN = 0, blockK = 0;
   /// Parts the matrix-core kernel cuts K into; 0 = planner's choice.
   unsigned splitK = 0;
+  unsigned stages = 0; // LDS stages of the 128-wide igemm tile: 2 or 4
   /// Output tile of the depthwise kernel; 0 = planner's choice.
   unsigned tileH = 0, tileW = 0;
   std::string text; // the JSON as given, kept for reporting and cache keys

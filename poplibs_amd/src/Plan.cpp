@@ -370,6 +370,16 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         parts = 1;
       g.splitK = uint32_t(parts);
       plan.workspaceBytes = mxk::igemmWorkspaceBytes(g);
+      // More workgroups than CUs: run the 128-wide tile with two LDS stages
+      // instead of four, so that two workgroups share a CU and one's
+      // start-up, barriers and epilogue are covered by the other's MFMAs.
+      // With one workgroup per CU or fewer the deeper prefetch is worth
+      // more.
+      g.stages = pc.stages ? pc.stages
+                           : (tiles * parts > gfx950::numCUs ? 2 : 4);
+      if (g.stages != 2 && g.stages != 4)
+        throw poplar::invalid_option(
+            "planConstraints gfx950 stages must be 2 or 4");
     }
     // A pointwise convolution with few input channels is bound by HBM, not
     // by the matrix cores: unless the big tile was asked for explicitly, the
@@ -477,6 +487,10 @@ std::string mxconv_plan::describe() const {
       os << "        block M x N x K            " << g.blockM << " x "
          << g.blockN << " x " << g.blockK << "\n";
       os << "        workgroups                 " << tiles * g.splitK << "\n";
+      if (g.blockN == 128)
+        os << "        LDS stages                 " << g.stages
+           << (g.stages == 2 ? " (two workgroups per CU)\n"
+                             : " (one workgroup per CU)\n");
       if (g.splitK > 1)
         os << "        K split into parts         " << g.splitK
            << " (fp32 partial tiles, summed by a second kernel)\n";

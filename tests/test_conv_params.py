@@ -403,6 +403,16 @@ def test_planner_choices():
     assert "K split into parts         28" in many.describe()
     assert many.buffer_bytes(4) == 28 * 128 * 9 * 128 * 4
     assert "K split" not in pa.Plan(c2).describe()
+    # one workgroup per CU or fewer: four LDS stages; more workgroups than
+    # CUs: two stages, two workgroups per CU
+    assert "LDS stages                 4" in pa.Plan(c2).describe()
+    c2_large = make_params(pa.HALF, batch=256, field=(28, 28), kernel=(3, 3),
+                           ci=128, co=128, pad=1)
+    assert "LDS stages                 2" in pa.Plan(c2_large).describe()
+    forced = pa.Plan(c2, {"planConstraints": '{"gfx950": {"stages": 2}}'})
+    assert "LDS stages                 2" in forced.describe()
+    with pytest.raises(MxconvError):
+        pa.Plan(c2, {"planConstraints": '{"gfx950": {"stages": 3}}'})
     # transforms outside the fast subset fall back
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
                                   co=8, flipIn=True)) == "generic direct"

@@ -179,7 +179,7 @@ def test_depthwise_fp32_out_pm1_exact(oracle):
     _run(oracle, p, 5, 0, "depthwise direct", dist="pm1")
 
 
-def _fp8_case(oracle, p, seed, fmt_a, fmt_w):
+def _fp8_case(oracle, p, seed, fmt_a, fmt_w, options=None):
     """values ~N(0,1) (weights scaled), per-tensor power-of-two scale chosen
     so the largest magnitude lands below the format's maximum."""
     from gpu_helpers import quantize, run_conv
@@ -195,7 +195,7 @@ def _fp8_case(oracle, p, seed, fmt_a, fmt_w):
     sa, sw = scale_for(acts, fmt_a), scale_for(weights, fmt_w)
     aq, ad = quantize(acts, pa.QUARTER, oracle, fmt_a, sa)
     wq, wd = quantize(weights, pa.QUARTER, oracle, fmt_w, sw)
-    got, plan = run_conv(p, aq, wq, None, None,
+    got, plan = run_conv(p, aq, wq, None, options,
                          in_meta=pa.quarter_metadata(fmt_a, sa),
                          w_meta=pa.quarter_metadata(fmt_w, sw),
                          return_plan=True)
@@ -414,6 +414,45 @@ def test_igemm_split_k_matches_oracle(oracle, kw, parts, out_type):
     if parts:
         assert "K split into parts         %d" % parts in plan.describe()
     want = oracle.convolution(p, ad, wd, bd, threads=8)
+    assert rel_l2(got, want) <= 1e-3, (rel_l2(got, want), plan.describe())
+
+
+STAGES_CASES = [
+    # (params, input type, forced stages or None for the planner's choice)
+    (dict(batch=3, field=(9, 11), kernel=(3, 3), ci=128, co=130, pad=1),
+     pa.HALF, 2),
+    (dict(batch=2, field=(7, 7), kernel=(3, 3), ci=40, co=72, pad=1),
+     pa.HALF, 2),
+    (dict(batch=2, field=(9, 11), kernel=(2, 3), ci=128, co=96, pad=1),
+     pa.QUARTER, 2),
+    # more workgroups than CUs: two stages are the planner's own choice
+    (dict(batch=24, field=(40, 40), kernel=(1, 3), ci=16, co=128,
+          padLower=(0, 1), padUpper=(0, 1)), pa.HALF, None),
+]
+
+
+@pytest.mark.parametrize("kw,in_type,stages", STAGES_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_igemm_two_stage_variant_matches_oracle(oracle, kw, in_type, stages,
+                                                out_type):
+    if in_type == pa.QUARTER and out_type == pa.FLOAT:
+        pytest.skip("quarter inputs give half outputs")
+    p = make_params(in_type, out_type, **kw)
+    print("case", p, stages, flush=True)
+    from gpu_helpers import quantize, run_conv
+    options = None
+    if stages:
+        options = {"planConstraints": '{"gfx950": {"stages": %d}}' % stages}
+    if in_type == pa.QUARTER:
+        got, want, plan = _fp8_case(oracle, p, 12, 1, 0, options)
+    else:
+        acts, weights, biases = random_data(p, 12, "normal")
+        aq, ad = quantize(acts, in_type)
+        wq, wd = quantize(weights * 0.05, in_type)
+        bq, bd = quantize(biases, out_type)
+        got, plan = run_conv(p, aq, wq, bq, options, return_plan=True)
+        want = oracle.convolution(p, ad, wd, bd, threads=8)
+    assert "LDS stages                 2" in plan.describe(), plan.describe()
     assert rel_l2(got, want) <= 1e-3, (rel_l2(got, want), plan.describe())
 
 
