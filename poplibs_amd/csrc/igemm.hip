@@ -635,7 +635,7 @@ struct KernelKey {
 
 KernelKey kernelKey(const IgemmDesc &d, int inType, int outType,
                     const QuarterInfo &q) {
-  const int eb = inType == kHalf ? 2 : 1;
+  const int eb = inType == kFloat ? 4 : inType == kHalf ? 2 : 1;
   KernelKey k;
   k.blockN = int(d.blockN), k.inType = inType, k.outType = outType;
   k.stages = d.blockN == 128 ? int(d.stages) : 3;
@@ -677,6 +677,8 @@ template <int BN, class Launch>
 hipError_t dispatchType(const KernelKey &k, const Launch &launch) {
   if (k.inType == kHalf)
     return dispatchStages<BN, 2, 0, 0>(k, launch);
+  if (k.inType == kFloat)
+    return dispatchStages<BN, 4, 0, 0>(k, launch);
   if (k.inType != kQuarter)
     return hipErrorInvalidValue;
   if (k.fa == 0 && k.fb == 0)
@@ -757,13 +759,14 @@ namespace {
 /// produces such shapes) and fills in the kernel's arguments.
 hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
                    IgemmArgs &a) {
-  const uint32_t eb = inType == kHalf ? 2 : 1;
+  const uint32_t eb = inType == kFloat ? 4 : inType == kHalf ? 2 : 1;
   const uint32_t bke = kRowBytes / eb;
   const int mode = igemmTapAddressing(d);
   const bool dilated = mode == kDilatedTaps;
   if (d.blockM != kBlockM || (d.blockN != 64 && d.blockN != 128) ||
       d.blockK != bke || d.inChansPerGroup % (16 / eb) != 0 ||
-      (inType != kHalf && inType != kQuarter) || d.splitK == 0 ||
+      (inType != kHalf && inType != kQuarter && inType != kFloat) ||
+      d.splitK == 0 ||
       d.inDilH == 0 || d.inDilW == 0)
     return hipErrorInvalidValue;
   // The arithmetic addressing keeps window origins as 16-bit offsets from

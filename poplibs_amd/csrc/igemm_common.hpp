@@ -31,6 +31,7 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef int intx8 __attribute__((ext_vector_type(8)));
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
@@ -169,6 +170,47 @@ template <> struct Mma<2> {
         if (i == 0 && j == 0)
           between();
       }
+  }
+};
+
+/// fp32: 4 sub-steps of 8 values, 32 bytes (two chunks, one per half-wave)
+/// each.  The fp32 MFMA takes one value per lane (K = 2: one from either
+/// half-wave), so the four values of a lane's chunk feed four MFMAs; which
+/// k meets which is the same for both operands, and that is all that counts.
+template <> struct Mma<4> {
+  static constexpr int kSubSteps = kRowBytes / 32;
+  template <int TN> struct Frags {
+    floatx4 a[kSubSteps][2], b[kSubSteps][TN];
+  };
+  template <int S, int TN>
+  static __device__ __forceinline__ void load(const FragmentAddress &at,
+                                              int lane, Frags<TN> &f) {
+    const int c = S * 2 + (lane >> 5);
+#pragma unroll
+    for (int i = 0; i != 2; ++i)
+      f.a[S][i] = *reinterpret_cast<const floatx4 *>(
+          at.a[i] + (((at.chunkBase + c) ^ at.swizzleA[i]) << 4));
+#pragma unroll
+    for (int j = 0; j != TN; ++j)
+      f.b[S][j] = *reinterpret_cast<const floatx4 *>(
+          at.b + j * 32 * kRowBytes + ((c ^ at.swizzleB) << 4));
+  }
+  template <int S, int TN, int FA, int FB, class F>
+  static __device__ __forceinline__ void
+  mul(const Frags<TN> &f, floatx16 (&acc)[2][TN], F &&between) {
+    // the four MFMAs into one accumulator depend on each other: the other
+    // accumulators' go in between
+#pragma unroll
+    for (int e = 0; e != 4; ++e)
+#pragma unroll
+      for (int i = 0; i != 2; ++i)
+#pragma unroll
+        for (int j = 0; j != TN; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+              f.b[S][j][e], f.a[S][i][e], acc[i][j], 0, 0, 0);
+          if (e == 0 && i == 0 && j == 0)
+            between();
+        }
   }
 };
 

@@ -330,6 +330,11 @@ hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                        static_cast<const uint16_t *>(src),
                        static_cast<uint16_t *>(dst), co, ci, taps, coPadded,
                        kPadded, total, chansTransposed);
+  else if (elemBytes == 4)
+    hipLaunchKernelGGL(packIgemmWeightsKernel<uint32_t>, grid, block, 0, stream,
+                       static_cast<const uint32_t *>(src),
+                       static_cast<uint32_t *>(dst), co, ci, taps, coPadded,
+                       kPadded, total, chansTransposed);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

@@ -222,6 +222,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   const Simple2D s = asSimple2D(p);
   const bool halfIn = params.inputType == poplar::HALF;
   const bool quarterIn = params.inputType == poplar::QUARTER;
+  const bool floatIn = params.inputType == poplar::FLOAT;
   const std::size_t ci = p.inputChannelsPerConvGroup;
   const std::size_t co = p.outputChannelsPerConvGroup;
 
@@ -233,9 +234,9 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   else if (!s.ok)
     igemmWhyNot = dwWhyNot = s.why;
   else {
-    if (!(halfIn || quarterIn))
-      igemmWhyNot = "matrix-core kernel takes half or quarter inputs";
-    else if (ci % (halfIn ? 8 : 16) != 0)
+    if (!(halfIn || quarterIn || floatIn))
+      igemmWhyNot = "matrix-core kernel takes float, half or quarter inputs";
+    else if (ci % (16 / params.inputType.size()) != 0)
       igemmWhyNot = "input channels per group not a multiple of a 16-byte "
                     "vector";
     else if (std::size_t(s.outH) * s.strideH + std::size_t(s.kH) * s.dilH +
@@ -336,12 +337,13 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     // channels, when a narrower tile avoids computing padding.
     g.blockM = pc.blockM ? pc.blockM : 128;
     g.blockN = pc.blockN ? pc.blockN : (co <= 64 ? 64 : 128);
-    g.blockK = pc.blockK ? pc.blockK : (halfIn ? 64 : 128);
+    const unsigned stepElems = unsigned(128 / params.inputType.size());
+    g.blockK = pc.blockK ? pc.blockK : stepElems;
     if (g.blockM != 128 || (g.blockN != 64 && g.blockN != 128) ||
-        g.blockK != (halfIn ? 64u : 128u))
+        g.blockK != stepElems)
       throw poplar::invalid_option(
           "planConstraints gfx950 tile not available: blockM must be 128, "
-          "blockN 64 or 128, blockK 64 (half) or 128 (quarter)");
+          "blockN 64 or 128, blockK 32 (float), 64 (half) or 128 (quarter)");
     const std::size_t k = std::size_t(s.kH) * s.kW * ci;
     plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
     plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;
@@ -397,7 +399,10 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     plan.pointwiseOn =
         unitWindow && pc.kernel != "igemm" && !pc.blockM && !pc.blockN &&
         !pc.blockK &&
-        mxk::pointwiseTakes(pw, halfIn ? mxk::kHalf : mxk::kQuarter,
+        mxk::pointwiseTakes(pw,
+                            halfIn    ? mxk::kHalf
+                            : floatIn ? mxk::kFloat
+                                      : mxk::kQuarter,
                             params.outputType == poplar::HALF ? mxk::kHalf
                                                               : mxk::kFloat);
     if (plan.pointwiseOn)
@@ -448,7 +453,9 @@ std::string mxconv_plan::describe() const {
     break;
   case Kernel::IGEMM:
     os << "implicit GEMM (MFMA, "
-       << (params.inputType == poplar::QUARTER ? "fp8" : "fp16")
+       << (params.inputType == poplar::QUARTER ? "fp8"
+           : params.inputType == poplar::FLOAT ? "fp32"
+                                               : "fp16")
        << " operands, fp32 accumulate)"
        << (pointwiseOn ? ", pointwise streaming variant" : "");
     break;

@@ -385,7 +385,7 @@ def test_planner_choices():
                      groups=96, stride=2, pad=1)
     c5 = make_params(pa.QUARTER, pa.HALF, batch=64, field=(14, 14),
                      kernel=(3, 3), ci=256, co=256, pad=1)
-    assert _kernel_of(c1) == "generic direct"      # fp32 inputs
+    assert _kernel_of(c1) == "implicit GEMM"       # fp32 MFMA
     assert _kernel_of(c2) == "implicit GEMM"
     assert _kernel_of(c4) == "depthwise direct"
     assert _kernel_of(c5) == "implicit GEMM"
@@ -429,8 +429,10 @@ def test_planner_choices():
                            '{"method": {"type": "AMP"}}'}) == "depthwise direct"
     forced = {"planConstraints": '{"gfx950": {"kernel": "generic"}}'}
     assert _kernel_of(c2, forced) == "generic direct"
+    odd = make_params(pa.FLOAT, field=(8, 8), kernel=(3, 3), ci=6, co=8)
+    assert _kernel_of(odd) == "generic direct"  # 6 floats: no 16-byte vector
     with pytest.raises(MxconvError) as e:
-        pa.Plan(c1, {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'})
+        pa.Plan(odd, {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'})
     assert e.value.status == Status.INVALID_OPTION
     with pytest.raises(MxconvError):
         pa.Plan(c2, {"planConstraints": '{"gfx950": {"blockM": 96}}'})

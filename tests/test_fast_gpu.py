@@ -417,6 +417,56 @@ def test_igemm_split_k_matches_oracle(oracle, kw, parts, out_type):
     assert rel_l2(got, want) <= 1e-3, (rel_l2(got, want), plan.describe())
 
 
+FP32_CASES = [
+    # the reference's own CPU-runnable configuration: 3x3, 16 -> 16, 32x32
+    dict(batch=1, field=(32, 32), kernel=(3, 3), ci=16, co=16, pad=1),
+    # a k-step inside one tap (32 floats of channels) ...
+    dict(batch=2, field=(14, 14), kernel=(3, 3), ci=64, co=128, pad=1),
+    # ... and k-steps that span taps, ragged against the tile
+    dict(batch=3, field=(9, 7), kernel=(3, 3), ci=4, co=40, pad=1),
+    dict(batch=1, field=(5, 5), kernel=(2, 3), ci=12, co=130,
+         padLower=(1, 0), padUpper=(0, 2)),
+    dict(batch=2, field=(17, 15), kernel=(3, 3), ci=8, co=24, groups=3,
+         stride=(2, 1), kdil=(1, 2), pad=2),
+    # dilated input, many taps, a plain matrix product
+    dict(batch=2, field=(6, 5), kernel=(3, 3), ci=8, co=16, idil=(2, 3),
+         pad=2),
+    dict(batch=1, field=(13, 13), kernel=(7, 7), ci=4, co=8, pad=3),
+    dict(batch=70, field=(), kernel=(), ci=96, co=64),
+]
+
+
+@pytest.mark.parametrize("kw", FP32_CASES)
+@pytest.mark.parametrize("out_type", [pa.FLOAT, pa.HALF])
+def test_igemm_fp32_matches_oracle(oracle, kw, out_type):
+    p = make_params(pa.FLOAT, out_type, **kw)
+    print("case", p, flush=True)
+    # fp32 products and sums: the fp16 output rounding is the only other error
+    _run(oracle, p, 21, 2e-6 if out_type == pa.FLOAT else 5e-4,
+         "implicit GEMM", wscale=0.1)
+
+
+def test_igemm_fp32_of_signs_is_exact(oracle):
+    p = make_params(pa.FLOAT, pa.FLOAT, batch=2, field=(9, 9), kernel=(3, 3),
+                    ci=32, co=72, pad=1)
+    _run(oracle, p, 22, 0, "implicit GEMM", dist="pm1")
+
+
+def test_igemm_fp32_split_k(oracle):
+    p = make_params(pa.FLOAT, pa.FLOAT, batch=1, field=(6, 6), kernel=(3, 3),
+                    ci=256, co=128, pad=1)
+    from gpu_helpers import quantize, run_conv
+    acts, weights, biases = random_data(p, 23, "normal")
+    aq, ad = quantize(acts, pa.FLOAT)
+    wq, wd = quantize(weights * 0.05, pa.FLOAT)
+    bq, bd = quantize(biases, pa.FLOAT)
+    got, plan = run_conv(p, aq, wq, bq, None, return_plan=True)
+    assert "fp32 operands" in plan.describe(), plan.describe()
+    assert "K split into parts" in plan.describe(), plan.describe()
+    want = oracle.convolution(p, ad, wd, bd, threads=8)
+    assert rel_l2(got, want) <= 2e-6
+
+
 STAGES_CASES = [
     # (params, input type, forced stages or None for the planner's choice)
     (dict(batch=3, field=(9, 11), kernel=(3, 3), ci=128, co=130, pad=1),

@@ -73,7 +73,8 @@ PLAN_CASES = [
     (pa.HALF, 1, 1024, 512, 512, None, "implicit GEMM"),
     (pa.HALF, 1, 4096, 256, 64, None, "pointwise streaming"),
     (pa.HALF, 1, 7, 5, 3, None, "generic direct"),
-    (pa.FLOAT, 1, 64, 64, 64, None, "generic direct"),
+    (pa.FLOAT, 1, 64, 64, 64, None, "implicit GEMM (MFMA, fp32"),
+    (pa.FLOAT, 1, 64, 62, 64, None, "generic direct"),
     (pa.HALF, 1, 64, 64, 64,
      {"planConstraints": '{"gfx950": {"kernel": "generic"}}'}, "generic direct"),
     (pa.HALF, 4, 256, 64, 64, None, "implicit GEMM"),
