@@ -88,14 +88,22 @@ hipError_t launchWeightsTransposeChansFlipXY(const void *src, void *dst,
                                              int elemBytes,
                                              hipStream_t stream);
 
+/// [pixels][groups][ci] -> [pixels][groups][ciPadded], the new channels zero;
+/// ciPadded * elemBytes is a multiple of 16.
+hipError_t launchPadChans(const void *src, void *dst, uint64_t pixels,
+                          uint32_t groups, uint32_t ci, uint32_t ciPadded,
+                          int elemBytes, hipStream_t stream);
+
 /// Weights [G][Co][Ci][taps] -> [G][coPadded][kPadded] with k = tap * Ci + ci,
 /// zero-filled beyond Co and beyond taps * Ci: the B operand of the
-/// matrix-core kernel, K contiguous.
+/// matrix-core kernel, K contiguous.  With ciPadded (not 0) every tap takes
+/// ciPadded places of k, the ones beyond Ci zero.
 hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                                   uint32_t co, uint32_t ci, uint32_t taps,
                                   uint32_t coPadded, uint32_t kPadded,
                                   int elemBytes, hipStream_t stream,
-                                  bool chansTransposed = false);
+                                  bool chansTransposed = false,
+                                  uint32_t ciPadded = 0);
 
 /// acts[outer][c] += bias[c] for `type` elements (kHalf or kFloat).
 hipError_t launchAddBias(int type, void *acts, const void *bias,

@@ -32,8 +32,8 @@ __global__ __launch_bounds__(256) void permuteKernel(PermuteArgs a,
 template <class T>
 __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
     const T *__restrict__ src, T *__restrict__ dst, uint32_t co, uint32_t ci,
-    uint32_t taps, uint32_t coPadded, uint32_t kPadded, uint64_t total,
-    bool chansTransposed) {
+    uint32_t ciPadded, uint32_t taps, uint32_t coPadded, uint32_t kPadded,
+    uint64_t total, bool chansTransposed) {
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
     return;
@@ -41,14 +41,37 @@ __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
   const uint32_t n = uint32_t((tid / kPadded) % coPadded);
   const uint64_t g = tid / (uint64_t(kPadded) * coPadded);
   T v = T(0);
-  if (n < co && k < taps * ci) {
-    const uint32_t tap = k / ci, c = k % ci;
+  if (n < co && k < taps * ciPadded) {
+    const uint32_t tap = k / ciPadded, c = k % ciPadded;
     // source [G][Co][Ci][taps], or [G][Ci][Co][taps] (a matrix
     // multiplication's right-hand side)
-    v = chansTransposed ? src[((g * ci + c) * co + n) * taps + tap]
-                        : src[((g * co + n) * ci + c) * taps + tap];
+    if (c < ci)
+      v = chansTransposed ? src[((g * ci + c) * co + n) * taps + tap]
+                          : src[((g * co + n) * ci + c) * taps + tap];
   }
   dst[tid] = v;
+}
+
+/// One 16-byte vector of the padded tensor per thread.
+template <class T>
+__global__ __launch_bounds__(256) void padChansKernel(
+    const T *__restrict__ src, T *__restrict__ dst, uint64_t vectors,
+    uint32_t ci, uint32_t ciPadded) {
+  constexpr uint32_t kVec = 16 / sizeof(T);
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= vectors)
+    return;
+  const uint32_t perGroup = ciPadded / kVec;
+  const uint64_t pg = tid / perGroup; // pixel * groups + group
+  const uint32_t c0 = uint32_t(tid - pg * perGroup) * kVec;
+  union {
+    T e[kVec];
+    uint4 u;
+  } v;
+#pragma unroll
+  for (uint32_t i = 0; i != kVec; ++i)
+    v.e[i] = c0 + i < ci ? src[pg * ci + c0 + i] : T(0);
+  reinterpret_cast<uint4 *>(dst)[tid] = v.u;
 }
 
 struct FlipArgs {
@@ -312,7 +335,11 @@ hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                                   uint32_t co, uint32_t ci, uint32_t taps,
                                   uint32_t coPadded, uint32_t kPadded,
                                   int elemBytes, hipStream_t stream,
-                                  bool chansTransposed) {
+                                  bool chansTransposed, uint32_t ciPadded) {
+  if (ciPadded == 0)
+    ciPadded = ci;
+  if (ciPadded < ci)
+    return hipErrorInvalidValue;
   const uint64_t total = uint64_t(groups) * coPadded * kPadded;
   if (total == 0)
     return hipSuccess;
@@ -323,20 +350,49 @@ hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
   if (elemBytes == 1)
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint8_t>, grid, block, 0, stream,
                        static_cast<const uint8_t *>(src),
-                       static_cast<uint8_t *>(dst), co, ci, taps, coPadded,
-                       kPadded, total, chansTransposed);
+                       static_cast<uint8_t *>(dst), co, ci, ciPadded, taps,
+                       coPadded, kPadded, total, chansTransposed);
   else if (elemBytes == 2)
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint16_t>, grid, block, 0, stream,
                        static_cast<const uint16_t *>(src),
-                       static_cast<uint16_t *>(dst), co, ci, taps, coPadded,
-                       kPadded, total, chansTransposed);
+                       static_cast<uint16_t *>(dst), co, ci, ciPadded, taps,
+                       coPadded, kPadded, total, chansTransposed);
   else if (elemBytes == 4)
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint32_t>, grid, block, 0, stream,
                        static_cast<const uint32_t *>(src),
-                       static_cast<uint32_t *>(dst), co, ci, taps, coPadded,
-                       kPadded, total, chansTransposed);
+                       static_cast<uint32_t *>(dst), co, ci, ciPadded, taps,
+                       coPadded, kPadded, total, chansTransposed);
   else
     return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launchPadChans(const void *src, void *dst, uint64_t pixels,
+                          uint32_t groups, uint32_t ci, uint32_t ciPadded,
+                          int elemBytes, hipStream_t stream) {
+  if ((elemBytes != 1 && elemBytes != 2 && elemBytes != 4) || ciPadded < ci ||
+      (uint64_t(ciPadded) * elemBytes) % 16 != 0)
+    return hipErrorInvalidValue;
+  const uint64_t vectors =
+      pixels * groups * (uint64_t(ciPadded) * elemBytes / 16);
+  if (vectors == 0)
+    return hipSuccess;
+  const uint64_t blocks = (vectors + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  if (elemBytes == 1)
+    hipLaunchKernelGGL(padChansKernel<uint8_t>, grid, block, 0, stream,
+                       static_cast<const uint8_t *>(src),
+                       static_cast<uint8_t *>(dst), vectors, ci, ciPadded);
+  else if (elemBytes == 2)
+    hipLaunchKernelGGL(padChansKernel<uint16_t>, grid, block, 0, stream,
+                       static_cast<const uint16_t *>(src),
+                       static_cast<uint16_t *>(dst), vectors, ci, ciPadded);
+  else
+    hipLaunchKernelGGL(padChansKernel<uint32_t>, grid, block, 0, stream,
+                       static_cast<const uint32_t *>(src),
+                       static_cast<uint32_t *>(dst), vectors, ci, ciPadded);
   return hipGetLastError();
 }
 

@@ -141,6 +141,21 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
       return hipStatus(mxk::launchPointwise(plan->pointwise, inType, outType,
                                             in, w, bias, out, s),
                        "pointwise convolution launch");
+    if (plan->paddedInputChans) {
+      // the kernel reads whole 16-byte vectors of channels: give it a copy
+      // with the channels of every group filled up with zeros
+      const mxk::IgemmDesc &g = plan->igemm;
+      char *padded = static_cast<char *>(workspace) + plan->paddedInputOffset;
+      const mxconv_status st = hipStatus(
+          mxk::launchPadChans(
+              in, padded, uint64_t(g.batch) * g.inH * g.inW, g.groups,
+              uint32_t(plan->params.inputChannelsPerConvGroup),
+              g.inChansPerGroup, int(plan->params.inputType.size()), s),
+          "channel padding launch");
+      if (st != MXCONV_OK)
+        return st;
+      in = padded;
+    }
     return hipStatus(mxk::launchIgemm(plan->igemm, inType, outType, in, w,
                                       bias, out, workspace, q, s),
                      "implicit-GEMM convolution launch");
@@ -541,7 +556,8 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
             weights_external, weights_packed, uint32_t(p.numConvGroups),
             uint32_t(p.outputChannelsPerConvGroup),
             uint32_t(p.inputChannelsPerConvGroup), uint32_t(taps),
-            uint32_t(plan->coPadded), uint32_t(plan->kPadded), elemBytes, s),
+            uint32_t(plan->coPadded), uint32_t(plan->kPadded), elemBytes, s,
+            false, uint32_t(plan->paddedInputChans)),
         "weight packing");
   }
   REQUIRE_ARG(weights_external);
@@ -691,8 +707,9 @@ mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
   };
   auto fusedItem = [&](size_t i, size_t slot, mxk::IgemmFusedItem &item) {
     const mxconv_plan *p = plans[i];
+    // (a plan that pads its input channels runs a copy first: on its own)
     if (p->outputElems == 0 || p->kernel != mxconv_plan::Kernel::IGEMM ||
-        p->pointwiseOn)
+        p->pointwiseOn || p->paddedInputChans)
       return false;
     unsplit[slot] = p->igemm;
     unsplit[slot].splitK = 1;
@@ -894,7 +911,8 @@ mxconv_status mxconv_matmul_pack_rhs(const mxconv_plan *plan, const void *rhs,
             rhs, weights_packed, uint32_t(p.numConvGroups),
             uint32_t(p.outputChannelsPerConvGroup),
             uint32_t(p.inputChannelsPerConvGroup), 1, uint32_t(plan->coPadded),
-            uint32_t(plan->kPadded), elemBytes, s, true),
+            uint32_t(plan->kPadded), elemBytes, s, true,
+            uint32_t(plan->paddedInputChans)),
         "weight packing");
   }
   // Generic kernel: packed = [G][1][Ci][Co], which is B itself.  Depthwise

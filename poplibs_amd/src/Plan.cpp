@@ -225,6 +225,13 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   const bool floatIn = params.inputType == poplar::FLOAT;
   const std::size_t ci = p.inputChannelsPerConvGroup;
   const std::size_t co = p.outputChannelsPerConvGroup;
+  // The matrix-core kernel reads whole 16-byte vectors of channels; other
+  // channel counts are padded with zeros (input: a copy per launch; weights:
+  // when they are packed).
+  const std::size_t vecElems = 16 / params.inputType.size();
+  const std::size_t ciPadded = (ci + vecElems - 1) / vecElems * vecElems;
+  const bool weightUpdatePass = options.pass == Pass::TRAINING_WU ||
+                                options.pass == Pass::FC_TRAINING_WU;
 
   // Which kernels can take this convolution at all?
   std::string igemmWhyNot, dwWhyNot;
@@ -236,9 +243,23 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   else {
     if (!(halfIn || quarterIn || floatIn))
       igemmWhyNot = "matrix-core kernel takes float, half or quarter inputs";
-    else if (ci % (16 / params.inputType.size()) != 0)
+    else if (ciPadded != ci &&
+             (weightUpdatePass || ci == 0 || (ci == 1 && co == 1)))
+      // (a weight update pass writes the kernel's operands itself, in the
+      // unpadded arrangement; one channel per group is vector-ALU work)
       igemmWhyNot = "input channels per group not a multiple of a 16-byte "
                     "vector";
+    else if (ciPadded != ci &&
+             p.batchSize * std::size_t(s.inH) * s.inW * p.numConvGroups *
+                     ciPadded * params.inputType.size() >=
+                 (1ull << 30))
+      igemmWhyNot = "tensor too large for 32-bit buffer addressing";
+    else if (ciPadded != ci && pc.kernel != "igemm" &&
+             2.0 * double(p.batchSize) * s.outH * s.outW * s.kH * s.kW * ci *
+                     co * p.numConvGroups <
+                 double(1u << 22))
+      igemmWhyNot = "too little work to pay for a padded copy of the input "
+                    "(channels per group not a multiple of a 16-byte vector)";
     else if (std::size_t(s.outH) * s.strideH + std::size_t(s.kH) * s.dilH +
                      std::size_t(std::abs(s.padH)) >=
                  32768 ||
@@ -323,7 +344,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     mxk::IgemmDesc &g = plan.igemm;
     g.batch = uint32_t(p.batchSize);
     g.groups = uint32_t(p.numConvGroups);
-    g.inChansPerGroup = uint32_t(ci);
+    g.inChansPerGroup = uint32_t(ciPadded);
     g.outChansPerGroup = uint32_t(co);
     g.inH = s.inH, g.inW = s.inW, g.outH = s.outH, g.outW = s.outW;
     g.kH = s.kH, g.kW = s.kW, g.padH = s.padH, g.padW = s.padW;
@@ -344,7 +365,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       throw poplar::invalid_option(
           "planConstraints gfx950 tile not available: blockM must be 128, "
           "blockN 64 or 128, blockK 32 (float), 64 (half) or 128 (quarter)");
-    const std::size_t k = std::size_t(s.kH) * s.kW * ci;
+    const std::size_t k = std::size_t(s.kH) * s.kW * ciPadded;
     plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
     plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;
     plan.weightPackedElems = p.numConvGroups * plan.coPadded * plan.kPadded;
@@ -372,6 +393,14 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         parts = 1;
       g.splitK = uint32_t(parts);
       plan.workspaceBytes = mxk::igemmWorkspaceBytes(g);
+      if (ciPadded != ci) {
+        plan.paddedInputChans = ciPadded;
+        plan.paddedInputOffset = (plan.workspaceBytes + 255) / 256 * 256;
+        plan.workspaceBytes = plan.paddedInputOffset +
+                              p.batchSize * std::size_t(s.inH) * s.inW *
+                                  p.numConvGroups * ciPadded *
+                                  params.inputType.size();
+      }
       // More workgroups than CUs: run the 128-wide tile with two LDS stages
       // instead of four, so that two workgroups share a CU and one's
       // start-up, barriers and epilogue are covered by the other's MFMAs.
@@ -397,7 +426,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         s.hiH == s.inH && s.hiW == s.inW && s.outH == s.inH &&
         s.outW == s.inW;
     plan.pointwiseOn =
-        unitWindow && pc.kernel != "igemm" && !pc.blockM && !pc.blockN &&
+        unitWindow && ciPadded == ci && pc.kernel != "igemm" && !pc.blockM && !pc.blockN &&
         !pc.blockK &&
         mxk::pointwiseTakes(pw,
                             halfIn    ? mxk::kHalf
@@ -509,6 +538,11 @@ std::string mxconv_plan::describe() const {
               "input)\n";
       os << "        packed weights             [G=" << g.groups << "]["
          << coPadded << "][" << kPadded << "]\n";
+      if (paddedInputChans)
+        os << "        input channels padded      "
+           << params.inputChannelsPerConvGroup << " -> " << paddedInputChans
+           << " per group (zero-filled copy in the workspace, every "
+              "launch)\n";
     }
   } else if (kernel == Kernel::DEPTHWISE) {
     const auto &d = depthwise;

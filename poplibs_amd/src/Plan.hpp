@@ -47,6 +47,11 @@ struct mxconv_plan {
 
   // Packed weights of the matrix-core kernel: [G][coPadded][kPadded].
   std::size_t coPadded = 0, kPadded = 0;
+  // Input channels per group as the matrix-core kernel sees them, when that
+  // is more than the parameters say (0 otherwise): the channels are padded
+  // with zeros to a whole 16-byte vector by a copy into the workspace, at
+  // byte offset paddedInputOffset, before every launch.
+  std::size_t paddedInputChans = 0, paddedInputOffset = 0;
 
   std::size_t inputElems = 0, outputElems = 0, weightElems = 0,
               weightPackedElems = 0, biasElems = 0;

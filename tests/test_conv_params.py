@@ -420,6 +420,19 @@ def test_planner_choices():
                                   co=8, flipK=True)) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
                                   ci=8, co=8)) == "generic direct"
+    # channel counts that are no whole 16-byte vector are padded for the
+    # matrix cores (a zero-filled copy in the workspace) ...
+    few = pa.Plan(make_params(pa.HALF, batch=2, field=(32, 32), kernel=(3, 3),
+                              ci=3, co=64))
+    assert "implicit GEMM" in few.describe()
+    assert "input channels padded      3 -> 8" in few.describe()
+    assert few.buffer_bytes(4) == 2 * 32 * 32 * 8 * 2
+    assert few.buffer_bytes(0) == 2 * 32 * 32 * 3 * 2   # the caller's input
+    # ... except in a weight update pass, which forms the operands itself,
+    # and when there is too little work to pay for the copy
+    assert _kernel_of(make_params(pa.HALF, batch=2, field=(32, 32),
+                                  kernel=(3, 3), ci=3, co=64),
+                      {"pass": "TRAINING_WU"}) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=4,
                                   co=8)) == "generic direct"
     # method names of the reference steer the choice
@@ -429,10 +442,10 @@ def test_planner_choices():
                            '{"method": {"type": "AMP"}}'}) == "depthwise direct"
     forced = {"planConstraints": '{"gfx950": {"kernel": "generic"}}'}
     assert _kernel_of(c2, forced) == "generic direct"
-    odd = make_params(pa.FLOAT, field=(8, 8), kernel=(3, 3), ci=6, co=8)
-    assert _kernel_of(odd) == "generic direct"  # 6 floats: no 16-byte vector
+    flipped = make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8, co=8,
+                          flipK=True)
     with pytest.raises(MxconvError) as e:
-        pa.Plan(odd, {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'})
+        pa.Plan(flipped, {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'})
     assert e.value.status == Status.INVALID_OPTION
     with pytest.raises(MxconvError):
         pa.Plan(c2, {"planConstraints": '{"gfx950": {"blockM": 96}}'})

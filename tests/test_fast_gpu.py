@@ -467,6 +467,43 @@ def test_igemm_fp32_split_k(oracle):
     assert rel_l2(got, want) <= 2e-6
 
 
+PADDED_CHANNEL_CASES = [
+    # a first layer: 3 input channels, 7x7 stride 2
+    (pa.HALF, dict(batch=2, field=(40, 40), kernel=(7, 7), ci=3, co=64,
+                   stride=2, pad=3)),
+    # groups, each padded by itself; ragged outputs
+    (pa.HALF, dict(batch=4, field=(20, 20), kernel=(3, 3), ci=4, co=12,
+                   groups=5, pad=1)),
+    (pa.HALF, dict(batch=6, field=(16, 18), kernel=(3, 3), ci=13, co=40,
+                   pad=1, stride=(1, 2))),
+    (pa.FLOAT, dict(batch=8, field=(24, 24), kernel=(3, 3), ci=3, co=32,
+                    pad=1)),
+    (pa.FLOAT, dict(batch=2, field=(24, 24), kernel=(3, 3), ci=6, co=16,
+                    groups=2, idil=2, pad=2)),
+    (pa.QUARTER, dict(batch=4, field=(24, 24), kernel=(3, 3), ci=5, co=32,
+                      pad=1)),
+]
+
+
+@pytest.mark.parametrize("in_type,kw", PADDED_CHANNEL_CASES)
+def test_igemm_pads_odd_channel_counts(oracle, in_type, kw):
+    out_type = pa.FLOAT if in_type == pa.FLOAT else pa.HALF
+    p = make_params(in_type, out_type, **kw)
+    print("case", p, flush=True)
+    if in_type == pa.QUARTER:
+        got, want, plan = _fp8_case(oracle, p, 31, 1, 1)
+    else:
+        from gpu_helpers import quantize, run_conv
+        acts, weights, biases = random_data(p, 31, "normal")
+        aq, ad = quantize(acts, in_type)
+        wq, wd = quantize(weights * 0.1, in_type)
+        bq, bd = quantize(biases, out_type)
+        got, plan = run_conv(p, aq, wq, bq, None, return_plan=True)
+        want = oracle.convolution(p, ad, wd, bd, threads=8)
+    assert "input channels padded" in plan.describe(), plan.describe()
+    assert rel_l2(got, want) <= (2e-6 if in_type == pa.FLOAT else 1e-3)
+
+
 STAGES_CASES = [
     # (params, input type, forced stages or None for the planner's choice)
     (dict(batch=3, field=(9, 11), kernel=(3, 3), ci=128, co=130, pad=1),

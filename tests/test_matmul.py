@@ -75,6 +75,7 @@ PLAN_CASES = [
     (pa.HALF, 1, 7, 5, 3, None, "generic direct"),
     (pa.FLOAT, 1, 64, 64, 64, None, "implicit GEMM (MFMA, fp32"),
     (pa.FLOAT, 1, 64, 62, 64, None, "generic direct"),
+    (pa.FLOAT, 1, 256, 62, 256, None, "input channels padded      62 -> 64"),
     (pa.HALF, 1, 64, 64, 64,
      {"planConstraints": '{"gfx950": {"kernel": "generic"}}'}, "generic direct"),
     (pa.HALF, 4, 256, 64, 64, None, "implicit GEMM"),
