@@ -113,7 +113,7 @@ __device__ __forceinline__ void igemmTile(
   const uint32_t inChans = d.groups * d.inChansPerGroup;
   const uint32_t ciBytes = d.inChansPerGroup * EB; // bytes of K per tap
   const uint32_t pixelBytes = inChans * EB;
-  const uint32_t taps = d.kH * d.kW;
+  const uint32_t taps = d.kD * d.kH * d.kW;
 
   const int wave = (t >> 6) & 3, lane = t & 63;
   const int wm = wave >> 1, wn = wave & 1;
@@ -141,7 +141,9 @@ __device__ __forceinline__ void igemmTile(
     const uint32_t shift =
         mode == kDilatedTaps
             ? 0u
-            : (uint32_t(d.padH > 0 ? d.padH : 0) * d.inW +
+            : ((uint32_t(d.padD > 0 ? d.padD : 0) * d.inH +
+                uint32_t(d.padH > 0 ? d.padH : 0)) *
+                   d.inW +
                uint32_t(d.padW > 0 ? d.padW : 0)) *
                   pixelBytes;
     const __amdgpu_buffer_rsrc_t inBuf =
@@ -207,14 +209,16 @@ __device__ __forceinline__ void igemmTile(
       uint32_t aByte = kStart + (UNI ? 0 : chunk * 16);
       uint32_t tap = a.divCiBytes(aByte);
       uint32_t ciOff = aByte - tap * ciBytes;
-      uint32_t kh = a.divKW(tap), kw = tap - kh * d.kW;
+      // tap = (kd * kH + kh) * kW + kw
+      uint32_t kRow = a.divKW(tap), kw = tap - kRow * d.kW;
+      uint32_t kd = a.divKH(kRow), kh = kRow - kd * d.kH;
       auto advance = [&] {
         if constexpr (GEN) {
           // no loop, no branch: everything again from the byte position
           aByte += kRowBytes;
           tap = a.divCiBytes(aByte);
           ciOff = aByte - tap * ciBytes;
-          kh = a.divKW(tap);
+          kh = a.divKW(tap); // (no depth with a dilated input)
           kw = tap - kh * d.kW;
         } else {
           ciOff += kRowBytes;
@@ -223,7 +227,10 @@ __device__ __forceinline__ void igemmTile(
             ++tap;
             if (++kw == d.kW) {
               kw = 0;
-              ++kh;
+              if (++kh == d.kH) {
+                kh = 0;
+                ++kd;
+              }
             }
           }
         }
@@ -278,7 +285,8 @@ __device__ __forceinline__ void igemmTile(
           }
         } else {
           const uint32_t tapOff =
-              (kh * d.dilH * d.inW + kw * d.dilW) * pixelBytes;
+              ((kd * d.dilD * d.inH + kh * d.dilH) * d.inW + kw * d.dilW) *
+              pixelBytes;
           if constexpr (UNI && MODE == kMaskTaps) {
             // tapMask holds the complement of the row's mask here: shifted so
             // that the tap's bit lands on bit 31 and merged into the offset,
@@ -378,13 +386,28 @@ __device__ __forceinline__ void igemmTile(
       const uint32_t mm = rowValid ? m : 0;
       const uint32_t q = a.divOutW(mm);
       const uint32_t ow = mm - q * d.outW;
-      const uint32_t b = a.divOutH(q);
-      const uint32_t oh = q - b * d.outH;
+      const uint32_t q2 = a.divOutH(q);
+      const uint32_t oh = q - q2 * d.outH;
+      const uint32_t b = a.divOutD(q2);
+      const uint32_t od = q2 - b * d.outD;
+      const int idBase = int(od * d.strideD) - d.padD;
       const int ihBase = int(oh * d.strideH) - d.padH;
       const int iwBase = int(ow * d.strideW) - d.padW;
-      const uint32_t shift = (uint32_t(d.padH > 0 ? d.padH : 0) * d.inW +
+      const uint32_t shift = ((uint32_t(d.padD > 0 ? d.padD : 0) * d.inH +
+                               uint32_t(d.padH > 0 ? d.padH : 0)) *
+                                  d.inW +
                               uint32_t(d.padW > 0 ? d.padW : 0)) *
                              pixelBytes;
+      // byte offset of the input element under tap (0, 0, 0) from the
+      // (shifted) buffer start; the additions wrap where a window starts
+      // above or left of the image and come right again with the shift
+      const uint32_t originOffset =
+          shift +
+          (((b * d.inD + uint32_t(idBase)) * d.inH + uint32_t(ihBase)) *
+               d.inW +
+           uint32_t(iwBase)) *
+              pixelBytes +
+          g * ciBytes;
       if (mode == kDilatedTaps) {
         // An invalid row gets the origin (-32768, -32768): no tap of it is
         // ever inside the input.
@@ -410,15 +433,10 @@ __device__ __forceinline__ void igemmTile(
             range(ihBase, int(d.loH), int(d.hiH), int(d.dilH), int(d.kH)) |
             (range(iwBase, int(d.loW), int(d.hiW), int(d.dilW), int(d.kW))
              << 16);
-        rowTable[t] = uint2{
-            shift +
-                ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
-                    pixelBytes +
-                g * ciBytes,
-            rowValid ? ranges : 0u};
+        rowTable[t] = uint2{originOffset, rowValid ? ranges : 0u};
       } else {
         uint32_t mask = 0;
-        if (d.dilH == 1 && d.dilW == 1) {
+        if (d.dilD == 1 && d.dilH == 1 && d.dilW == 1) {
           // Undilated kernel: the valid kernel columns are the interval
           // [lo - base, hi - base) cut to the kernel, and so are the rows.
           // Bits [first, last) of a word:
@@ -430,7 +448,7 @@ __device__ __forceinline__ void igemmTile(
           auto cut = [](int v, int size) {
             return v < 0 ? 0 : v > size ? size : v;
           };
-          const int kW = int(d.kW), kH = int(d.kH);
+          const int kW = int(d.kW), kH = int(d.kH), kD = int(d.kD);
           const uint32_t kwMask = bitRange(cut(int(d.loW) - iwBase, kW),
                                            cut(int(d.hiW) - iwBase, kW));
           // one bit per valid kernel row, at that row's first tap; the
@@ -439,7 +457,12 @@ __device__ __forceinline__ void igemmTile(
           const uint32_t rowStarts =
               a.tapRowStarts & bitRange(cut(int(d.loH) - ihBase, kH) * kW,
                                         cut(int(d.hiH) - ihBase, kH) * kW);
-          mask = kwMask * rowStarts;
+          // likewise one bit per valid kernel plane, at its first tap
+          const uint32_t planeStarts =
+              a.tapPlaneStarts &
+              bitRange(cut(int(d.loD) - idBase, kD) * kH * kW,
+                       cut(int(d.hiD) - idBase, kD) * kH * kW);
+          mask = kwMask * rowStarts * planeStarts;
         } else {
           uint32_t kwMask = 0;
           for (uint32_t kw = 0; kw != d.kW; ++kw) {
@@ -447,18 +470,19 @@ __device__ __forceinline__ void igemmTile(
             if (iw >= int(d.loW) && iw < int(d.hiW))
               kwMask |= 1u << kw;
           }
+          uint32_t planeMask = 0;
           for (uint32_t kh = 0; kh != d.kH; ++kh) {
             const int ih = ihBase + int(kh * d.dilH);
             if (ih >= int(d.loH) && ih < int(d.hiH))
-              mask |= kwMask << (kh * d.kW);
+              planeMask |= kwMask << (kh * d.kW);
+          }
+          for (uint32_t kd = 0; kd != d.kD; ++kd) {
+            const int id = idBase + int(kd * d.dilD);
+            if (id >= int(d.loD) && id < int(d.hiD))
+              mask |= planeMask << (kd * d.kH * d.kW);
           }
         }
-        rowTable[t] = uint2{
-            shift +
-                ((b * d.inH + uint32_t(ihBase)) * d.inW + uint32_t(iwBase)) *
-                    pixelBytes +
-                g * ciBytes,
-            rowValid ? mask : 0u};
+        rowTable[t] = uint2{originOffset, rowValid ? mask : 0u};
       }
     }
     MXK_WAIT_LGKMCNT0();
@@ -743,13 +767,13 @@ __global__ __launch_bounds__(64) void splitKReduceKernel(
 int igemmTapAddressing(const IgemmDesc &d) {
   if (d.inDilH != 1 || d.inDilW != 1)
     return kDilatedTaps;
-  return d.kH * d.kW > 32 ? kRangeTaps : kMaskTaps;
+  return d.kD * d.kH * d.kW > 32 ? kRangeTaps : kMaskTaps;
 }
 
 size_t igemmWorkspaceBytes(const IgemmDesc &d) {
   if (d.splitK <= 1)
     return 0;
-  return size_t(d.splitK) * d.batch * d.outH * d.outW * d.groups *
+  return size_t(d.splitK) * d.batch * d.outD * d.outH * d.outW * d.groups *
          d.outChansPerGroup * sizeof(float);
 }
 
@@ -786,6 +810,11 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
   // the ranges of valid kernel rows and columns are kept in 8 bits each
   if (mode == kRangeTaps && (d.kH > 255 || d.kW > 255))
     return hipErrorInvalidValue;
+  // a depth dimension goes with the tap mask only
+  if (mode != kMaskTaps && (d.inD != 1 || d.outD != 1 || d.kD != 1))
+    return hipErrorInvalidValue;
+  if (d.kD == 0 || d.kH == 0 || d.kW == 0)
+    return hipErrorInvalidValue;
   if (d.splitK > 1 &&
       (!haveWorkspace || (d.groups * d.outChansPerGroup) % 4 != 0))
     return hipErrorInvalidValue;
@@ -795,32 +824,40 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
   a.divInDilW = makeFastDiv(d.inDilW);
   a.divCiBytes = makeFastDiv(d.inChansPerGroup * eb);
   a.divKW = makeFastDiv(d.kW);
-  const uint64_t m = uint64_t(d.batch) * d.outH * d.outW;
+  a.divKH = makeFastDiv(d.kH);
+  const uint64_t m = uint64_t(d.batch) * d.outD * d.outH * d.outW;
   if (m > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
   a.M = uint32_t(m);
   a.divOutW = makeFastDiv(d.outW);
   a.divOutH = makeFastDiv(d.outH);
+  a.divOutD = makeFastDiv(d.outD);
   a.mTiles = (a.M + kBlockM - 1) / kBlockM;
   a.nTiles = (d.outChansPerGroup + d.blockN - 1) / d.blockN;
   a.divNTiles = makeFastDiv(a.nTiles);
   a.divMTiles = makeFastDiv(a.mTiles);
   a.divGroups = makeFastDiv(d.groups);
   // bit kh * kW for every kernel row (tap mask mode: at most 32 taps)
-  a.tapRowStarts = 0;
-  if (a.mode == kMaskTaps)
+  a.tapRowStarts = a.tapPlaneStarts = 0;
+  if (a.mode == kMaskTaps) {
     for (uint32_t kh = 0; kh != d.kH; ++kh)
       a.tapRowStarts |= 1u << (kh * d.kW);
+    for (uint32_t kd = 0; kd != d.kD; ++kd)
+      a.tapPlaneStarts |= 1u << (kd * d.kH * d.kW);
+  }
   a.coPadded = a.nTiles * d.blockN;
-  const uint32_t k = d.kH * d.kW * d.inChansPerGroup;
+  const uint32_t k = d.kD * d.kH * d.kW * d.inChansPerGroup;
   a.kPadded = (k + bke - 1) / bke * bke;
   // every part runs the same number of k-steps; steps beyond K load zeros
   a.kSteps = (a.kPadded / bke + d.splitK - 1) / d.splitK;
   // Buffer addressing is 32-bit; the planner keeps larger tensors away.
   const uint64_t inBytes =
-      uint64_t(d.batch) * d.inH * d.inW * d.groups * d.inChansPerGroup * eb;
+      uint64_t(d.batch) * d.inD * d.inH * d.inW * d.groups *
+      d.inChansPerGroup * eb;
   const uint64_t wBytes = uint64_t(d.groups) * a.coPadded * a.kPadded * eb;
-  const uint64_t shift = (uint64_t(d.padH > 0 ? d.padH : 0) * d.inW +
+  const uint64_t shift = ((uint64_t(d.padD > 0 ? d.padD : 0) * d.inH +
+                           uint64_t(d.padH > 0 ? d.padH : 0)) *
+                              d.inW +
                           uint64_t(d.padW > 0 ? d.padW : 0)) *
                          d.groups * d.inChansPerGroup * eb;
   if (inBytes + shift >= kOutOfRange || wBytes >= kOutOfRange)

@@ -16,7 +16,9 @@ struct IgemmArgs {
   FastDiv divInDilH, divInDilW;
   FastDiv divCiBytes, divKW; // by bytes of K per tap; by kernel width
   FastDiv divNTiles, divMTiles, divGroups; // workgroup number -> tile
+  FastDiv divOutD, divKH;
   uint32_t tapRowStarts; // tap mask mode: bit kh * kW for every kernel row
+  uint32_t tapPlaneStarts; // ... and bit kd * kH * kW for every kernel plane
   uint32_t mode;     // kMaskTaps, kRangeTaps or kDilatedTaps
   uint32_t M;        // batch * outH * outW
   uint32_t mTiles, nTiles;

@@ -122,6 +122,12 @@ struct IgemmDesc {
   uint32_t loH, hiH, loW, hiW;
   // Tile shape chosen by the planner.
   uint32_t blockM, blockN, blockK;
+  // A third, outermost field dimension (depth), with the same meaning of its
+  // members; 1 / 0 where a field has none.  Kernels of at most 32 taps on
+  // undilated inputs only.
+  uint32_t inD = 1, outD = 1, kD = 1;
+  int32_t padD = 0;
+  uint32_t strideD = 1, dilD = 1, loD = 0, hiD = 1;
   // Zeros stuffed between input elements: input row r sits at row r * inDilH
   // of the field the window slides over (padH, strideH, dilH are in those
   // coordinates; loH, hiH bound r itself).  1 = none.

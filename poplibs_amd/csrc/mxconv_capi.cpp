@@ -148,7 +148,7 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
       char *padded = static_cast<char *>(workspace) + plan->paddedInputOffset;
       const mxconv_status st = hipStatus(
           mxk::launchPadChans(
-              in, padded, uint64_t(g.batch) * g.inH * g.inW, g.groups,
+              in, padded, uint64_t(g.batch) * g.inD * g.inH * g.inW, g.groups,
               uint32_t(plan->params.inputChannelsPerConvGroup),
               g.inChansPerGroup, int(plan->params.inputType.size()), s),
           "channel padding launch");
@@ -697,12 +697,12 @@ mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
   // for the sum of a split K's parts).
   mxk::IgemmDesc unsplit[mxk::kIgemmMaxFused];
   auto tilesOf = [](const mxk::IgemmDesc &d) {
-    const uint64_t m = uint64_t(d.batch) * d.outH * d.outW;
+    const uint64_t m = uint64_t(d.batch) * d.outD * d.outH * d.outW;
     return (m + d.blockM - 1) / d.blockM *
            ((d.outChansPerGroup + d.blockN - 1) / d.blockN) * d.groups;
   };
   auto kStepsOf = [](const mxk::IgemmDesc &d) {
-    const uint64_t k = uint64_t(d.kH) * d.kW * d.inChansPerGroup;
+    const uint64_t k = uint64_t(d.kD) * d.kH * d.kW * d.inChansPerGroup;
     return (k + d.blockK - 1) / d.blockK;
   };
   auto fusedItem = [&](size_t i, size_t slot, mxk::IgemmFusedItem &item) {

@@ -63,16 +63,27 @@ struct Simple2D {
   uint32_t strideH = 1, strideW = 1, dilH = 1, dilW = 1;
   uint32_t loH = 0, hiH = 1, loW = 0, hiW = 1;
   uint32_t inDilH = 1, inDilW = 1;
-  bool inputDilated() const { return inDilH != 1 || inDilW != 1; }
+  // A third, outermost dimension (depth).  One that the window does not
+  // slide over in any interesting way (kernel 1, stride 1, nothing padded,
+  // truncated or dilated) is folded into the batch instead.
+  uint32_t inD = 1, outD = 1, kD = 1;
+  int32_t padD = 0;
+  uint32_t strideD = 1, dilD = 1, loD = 0, hiD = 1, inDilD = 1;
+  std::size_t batch = 0; // the batch size times the folded depth
+  bool hasDepth() const { return inD != 1 || outD != 1 || kD != 1; }
+  bool inputDilated() const {
+    return inDilH != 1 || inDilW != 1 || inDilD != 1;
+  }
 };
 
 Simple2D asSimple2D(const ConvParams &p) {
   Simple2D s;
   const unsigned n = unsigned(p.getNumFieldDims());
-  if (n > 2) {
-    s.why = "more than two field dimensions";
+  if (n > 3) {
+    s.why = "more than three field dimensions";
     return s;
   }
+  s.batch = p.batchSize;
   for (unsigned d = 0; d != n; ++d) {
     const auto &it = p.inputTransform, &kt = p.kernelTransform;
     const auto &ot = p.outputTransform;
@@ -97,16 +108,25 @@ Simple2D asSimple2D(const ConvParams &p) {
                         int32_t(ot.truncationLower[d]);
     const uint32_t lo = it.truncationLower[d];
     const uint32_t hi = uint32_t(p.inputFieldShape[d]) - it.truncationUpper[d];
-    const bool isW = (d + 1 == n);
-    (isW ? s.inW : s.inH) = uint32_t(p.inputFieldShape[d]);
-    (isW ? s.outW : s.outH) = uint32_t(p.getOutputSize(d));
-    (isW ? s.kW : s.kH) = uint32_t(p.kernelShape[d]);
-    (isW ? s.padW : s.padH) = pad;
-    (isW ? s.strideW : s.strideH) = ot.stride[d];
-    (isW ? s.dilW : s.dilH) = kt.dilation[d];
-    (isW ? s.loW : s.loH) = lo;
-    (isW ? s.hiW : s.hiH) = hi;
-    (isW ? s.inDilW : s.inDilH) = it.dilation[d];
+    // which of depth, height, width: the innermost dimension is the width
+    const unsigned which = d + 3 - n;
+    auto pick = [which](auto &dd, auto &hh, auto &ww) -> auto & {
+      return which == 0 ? dd : which == 1 ? hh : ww;
+    };
+    pick(s.inD, s.inH, s.inW) = uint32_t(p.inputFieldShape[d]);
+    pick(s.outD, s.outH, s.outW) = uint32_t(p.getOutputSize(d));
+    pick(s.kD, s.kH, s.kW) = uint32_t(p.kernelShape[d]);
+    pick(s.padD, s.padH, s.padW) = pad;
+    pick(s.strideD, s.strideH, s.strideW) = ot.stride[d];
+    pick(s.dilD, s.dilH, s.dilW) = kt.dilation[d];
+    pick(s.loD, s.loH, s.loW) = lo;
+    pick(s.hiD, s.hiH, s.hiW) = hi;
+    pick(s.inDilD, s.inDilH, s.inDilW) = it.dilation[d];
+  }
+  if (s.kD == 1 && s.strideD == 1 && s.padD == 0 && s.loD == 0 &&
+      s.hiD == s.inD && s.inDilD == 1 && s.outD == s.inD) {
+    s.batch *= s.inD;
+    s.inD = s.outD = s.hiD = 1;
   }
   s.ok = true;
   return s;
@@ -200,7 +220,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   // dilation the layer's stride and its stride the layer's kernel dilation.
   {
     const Simple2D w = asSimple2D(p);
-    if (w.ok && !plan.zeroConv && !w.inputDilated() && p.batchSize == 1 &&
+    if (w.ok && !w.hasDepth() && w.batch == 1 && !plan.zeroConv &&
+        !w.inputDilated() && p.batchSize == 1 &&
         p.outputChannelsPerConvGroup == 1 &&
         params.inputType == poplar::HALF && p.numConvGroups % 8 == 0 &&
         p.numConvGroups * p.inputChannelsPerConvGroup *
@@ -250,13 +271,13 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       igemmWhyNot = "input channels per group not a multiple of a 16-byte "
                     "vector";
     else if (ciPadded != ci &&
-             p.batchSize * std::size_t(s.inH) * s.inW * p.numConvGroups *
-                     ciPadded * params.inputType.size() >=
+             s.batch * s.inD * s.inH * s.inW * p.numConvGroups * ciPadded *
+                     params.inputType.size() >=
                  (1ull << 30))
       igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     else if (ciPadded != ci && pc.kernel != "igemm" &&
-             2.0 * double(p.batchSize) * s.outH * s.outW * s.kH * s.kW * ci *
-                     co * p.numConvGroups <
+             2.0 * double(s.batch) * s.outD * s.outH * s.outW * s.kD * s.kH *
+                     s.kW * ci * co * p.numConvGroups <
                  double(1u << 22))
       igemmWhyNot = "too little work to pay for a padded copy of the input "
                     "(channels per group not a multiple of a 16-byte vector)";
@@ -267,6 +288,10 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                      std::size_t(std::abs(s.padW)) >=
                  32768)
       igemmWhyNot = "field too large for 16-bit window origins";
+    else if (s.hasDepth() &&
+             (s.inputDilated() || std::size_t(s.kD) * s.kH * s.kW > 32))
+      igemmWhyNot = "three field dimensions with a dilated input or more "
+                    "than 32 kernel taps";
     else if (s.inputDilated() &&
              (std::size_t(s.inW) * p.getNumInputChans() *
                       params.inputType.size() >=
@@ -279,7 +304,9 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     else if (plan.inputElems * params.inputType.size() >= (1ull << 30) ||
              plan.weightElems * params.inputType.size() >= (1ull << 30))
       igemmWhyNot = "tensor too large for 32-bit buffer addressing";
-    if (!halfIn)
+    if (s.hasDepth())
+      dwWhyNot = "three field dimensions";
+    else if (!halfIn)
       dwWhyNot = "depthwise kernel takes half inputs";
     else if (ci != 1 || co != 1)
       dwWhyNot = "not one channel per group";
@@ -342,9 +369,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
 
   if (chosen == Kernel::IGEMM) {
     mxk::IgemmDesc &g = plan.igemm;
-    g.batch = uint32_t(p.batchSize);
+    g.batch = uint32_t(s.batch);
     g.groups = uint32_t(p.numConvGroups);
     g.inChansPerGroup = uint32_t(ciPadded);
+    g.inD = s.inD, g.outD = s.outD, g.kD = s.kD, g.padD = s.padD;
+    g.strideD = s.strideD, g.dilD = s.dilD, g.loD = s.loD, g.hiD = s.hiD;
     g.outChansPerGroup = uint32_t(co);
     g.inH = s.inH, g.inW = s.inW, g.outH = s.outH, g.outW = s.outW;
     g.kH = s.kH, g.kW = s.kW, g.padH = s.padH, g.padW = s.padW;
@@ -365,7 +394,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       throw poplar::invalid_option(
           "planConstraints gfx950 tile not available: blockM must be 128, "
           "blockN 64 or 128, blockK 32 (float), 64 (half) or 128 (quarter)");
-    const std::size_t k = std::size_t(s.kH) * s.kW * ciPadded;
+    const std::size_t k = std::size_t(s.kD) * s.kH * s.kW * ciPadded;
     plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
     plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;
     plan.weightPackedElems = p.numConvGroups * plan.coPadded * plan.kPadded;
@@ -376,7 +405,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     // workspace (the role of PopLibs' in-channel split with ReduceAdd,
     // lib/poplin/ConvReduce.cpp:316-362).
     {
-      const std::size_t m = p.batchSize * std::size_t(s.outH) * s.outW;
+      const std::size_t m = s.batch * s.outD * s.outH * s.outW;
       const std::size_t tiles = ((m + g.blockM - 1) / g.blockM) *
                                 (plan.coPadded / g.blockN) * p.numConvGroups;
       const std::size_t kSteps = plan.kPadded / g.blockK;
@@ -397,7 +426,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         plan.paddedInputChans = ciPadded;
         plan.paddedInputOffset = (plan.workspaceBytes + 255) / 256 * 256;
         plan.workspaceBytes = plan.paddedInputOffset +
-                              p.batchSize * std::size_t(s.inH) * s.inW *
+                              s.batch * s.inD * s.inH * s.inW *
                                   p.numConvGroups * ciPadded *
                                   params.inputType.size();
       }
@@ -420,14 +449,15 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     pw.groups = g.groups, pw.inChansPerGroup = g.inChansPerGroup;
     pw.outChansPerGroup = g.outChansPerGroup;
     const bool unitWindow =
-        !s.inputDilated() && g.splitK == 1 && s.kH == 1 && s.kW == 1 &&
+        !s.hasDepth() && !s.inputDilated() && g.splitK == 1 && s.kH == 1 &&
+        s.kW == 1 &&
         s.strideH == 1 && s.strideW == 1 &&
         s.padH == 0 && s.padW == 0 && s.loH == 0 && s.loW == 0 &&
         s.hiH == s.inH && s.hiW == s.inW && s.outH == s.inH &&
         s.outW == s.inW;
     plan.pointwiseOn =
-        unitWindow && ciPadded == ci && pc.kernel != "igemm" && !pc.blockM && !pc.blockN &&
-        !pc.blockK &&
+        unitWindow && ciPadded == ci && pc.kernel != "igemm" && !pc.blockM &&
+        !pc.blockN && !pc.blockK &&
         mxk::pointwiseTakes(pw,
                             halfIn    ? mxk::kHalf
                             : floatIn ? mxk::kFloat
@@ -438,7 +468,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       plan.weightPackedElems = mxk::pointwisePackedElems(pw);
   } else if (chosen == Kernel::DEPTHWISE) {
     mxk::DepthwiseDesc &d = plan.depthwise;
-    d.batch = uint32_t(p.batchSize);
+    d.batch = uint32_t(s.batch);
     d.channels = uint32_t(p.numConvGroups);
     d.inH = s.inH, d.inW = s.inW, d.outH = s.outH, d.outW = s.outW;
     d.kH = s.kH, d.kW = s.kW, d.padH = s.padH, d.padW = s.padW;
@@ -504,8 +534,9 @@ std::string mxconv_plan::describe() const {
   os << "        partialsType               float\n";
   if (kernel == Kernel::IGEMM) {
     const auto &g = igemm;
-    const std::size_t m = std::size_t(g.batch) * g.outH * g.outW;
-    const std::size_t k = std::size_t(g.kH) * g.kW * g.inChansPerGroup;
+    const std::size_t m = std::size_t(g.batch) * g.outD * g.outH * g.outW;
+    const std::size_t k =
+        std::size_t(g.kD) * g.kH * g.kW * g.inChansPerGroup;
     const std::size_t tiles = (m + g.blockM - 1) / g.blockM *
                               (coPadded / g.blockN) * g.groups;
     os << "        gemm M x N x K             " << m << " x "

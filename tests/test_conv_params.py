@@ -418,8 +418,21 @@ def test_planner_choices():
                                   co=8, flipIn=True)) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
                                   co=8, flipK=True)) == "generic direct"
+    # three field dimensions: the matrix cores take kernels of up to 32 taps
+    # on undilated inputs; a depth the window does not slide over is batch
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
+                                  ci=8, co=8)) == "implicit GEMM"
+    assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 4),
                                   ci=8, co=8)) == "generic direct"
+    assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
+                                  ci=8, co=8, idil=(1, 2, 1))) == \
+        "generic direct"
+    folded = pa.Plan(make_params(pa.HALF, batch=2, field=(5, 9, 9),
+                                 kernel=(1, 7, 7), ci=8, co=8))
+    assert "gemm M x N x K             90 x 8 x 392" in folded.describe()
+    assert _kernel_of(make_params(pa.HALF, field=(4, 8, 8, 8),
+                                  kernel=(1, 3, 3, 3), ci=8, co=8)) == \
+        "generic direct"
     # channel counts that are no whole 16-byte vector are padded for the
     # matrix cores (a zero-filled copy in the workspace) ...
     few = pa.Plan(make_params(pa.HALF, batch=2, field=(32, 32), kernel=(3, 3),

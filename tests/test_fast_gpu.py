@@ -504,6 +504,49 @@ def test_igemm_pads_odd_channel_counts(oracle, in_type, kw):
     assert rel_l2(got, want) <= (2e-6 if in_type == pa.FLOAT else 1e-3)
 
 
+DEPTH_CASES = [
+    # a 3-D UNet style layer
+    (pa.HALF, dict(batch=2, field=(6, 10, 9), kernel=(3, 3, 3), ci=16, co=24,
+                   pad=1)),
+    # stride, padding and kernel dilation different in every dimension
+    (pa.HALF, dict(batch=2, field=(9, 8, 11), kernel=(2, 3, 3), ci=8, co=40,
+                   stride=(2, 1, 2), kdil=(2, 1, 1), padLower=(1, 0, 2),
+                   padUpper=(2, 1, 0), groups=2)),
+    (pa.HALF, dict(batch=1, field=(5, 7, 6), kernel=(3, 1, 2), ci=64, co=130,
+                   padLower=(2, 0, 1), padUpper=(0, 0, 0))),
+    # truncation in depth; few channels (padded)
+    (pa.HALF, dict(batch=2, field=(8, 12, 12), kernel=(3, 3, 3), ci=3, co=32,
+                   itl=(1, 0, 0), itu=(0, 1, 0), pad=1)),
+    (pa.FLOAT, dict(batch=2, field=(5, 6, 7), kernel=(3, 3, 3), ci=8, co=16,
+                    pad=1)),
+    (pa.QUARTER, dict(batch=2, field=(5, 6, 7), kernel=(3, 3, 3), ci=16,
+                      co=16, pad=1)),
+    # a depth the window does not slide over: folded into the batch
+    (pa.HALF, dict(batch=2, field=(5, 9, 9), kernel=(1, 7, 7), ci=8, co=16,
+                   padLower=(0, 3, 3), padUpper=(0, 3, 3))),
+]
+
+
+@pytest.mark.parametrize("in_type,kw", DEPTH_CASES)
+def test_igemm_three_field_dimensions(oracle, in_type, kw):
+    out_type = pa.FLOAT if in_type == pa.FLOAT else pa.HALF
+    p = make_params(in_type, out_type, **kw)
+    print("case", p, flush=True)
+    if in_type == pa.QUARTER:
+        got, want, plan = _fp8_case(oracle, p, 41, 1, 1)
+        assert _plan_kernel(plan) == "implicit GEMM", plan.describe()
+        assert rel_l2(got, want) <= 1e-3
+    else:
+        _run(oracle, p, 41, 2e-6 if in_type == pa.FLOAT else 1e-3,
+             "implicit GEMM", wscale=0.1)
+
+
+def test_igemm_three_dimensions_of_signs_is_exact(oracle):
+    p = make_params(pa.HALF, pa.FLOAT, batch=2, field=(4, 6, 5),
+                    kernel=(3, 3, 3), ci=16, co=24, pad=1, stride=(1, 2, 1))
+    _run(oracle, p, 42, 0, "implicit GEMM", dist="pm1")
+
+
 STAGES_CASES = [
     # (params, input type, forced stages or None for the planner's choice)
     (dict(batch=3, field=(9, 11), kernel=(3, 3), ci=128, co=130, pad=1),
