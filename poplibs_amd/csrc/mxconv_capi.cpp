@@ -1134,7 +1134,8 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
     if (st != MXCONV_OK)
       return st;
   }
-  if (plan->kernel == mxconv_plan::Kernel::IGEMM && !plan->pointwiseOn) {
+  if (plan->kernel == mxconv_plan::Kernel::IGEMM && !plan->pointwiseOn &&
+      !plan->paddedInputChans) {
     // deltas [B][Y][G][Co] -> straight into the matrix-core kernel's packed
     // weights [G][coPadded][kPadded], k = y * B + b
     if (plan->coPadded != Co || plan->kPadded != Y * B) {

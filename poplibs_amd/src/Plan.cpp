@@ -251,8 +251,6 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   // when they are packed).
   const std::size_t vecElems = 16 / params.inputType.size();
   const std::size_t ciPadded = (ci + vecElems - 1) / vecElems * vecElems;
-  const bool weightUpdatePass = options.pass == Pass::TRAINING_WU ||
-                                options.pass == Pass::FC_TRAINING_WU;
 
   // Which kernels can take this convolution at all?
   std::string igemmWhyNot, dwWhyNot;
@@ -264,10 +262,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   else {
     if (!(halfIn || quarterIn || floatIn))
       igemmWhyNot = "matrix-core kernel takes float, half or quarter inputs";
-    else if (ciPadded != ci &&
-             (weightUpdatePass || ci == 0 || (ci == 1 && co == 1)))
-      // (a weight update pass writes the kernel's operands itself, in the
-      // unpadded arrangement; one channel per group is vector-ALU work)
+    else if (ciPadded != ci && (ci == 0 || (ci == 1 && co == 1)))
+      // (one channel per group is vector-ALU work)
       igemmWhyNot = "input channels per group not a multiple of a 16-byte "
                     "vector";
     else if (ciPadded != ci &&

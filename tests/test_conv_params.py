@@ -441,11 +441,7 @@ def test_planner_choices():
     assert "input channels padded      3 -> 8" in few.describe()
     assert few.buffer_bytes(4) == 2 * 32 * 32 * 8 * 2
     assert few.buffer_bytes(0) == 2 * 32 * 32 * 3 * 2   # the caller's input
-    # ... except in a weight update pass, which forms the operands itself,
-    # and when there is too little work to pay for the copy
-    assert _kernel_of(make_params(pa.HALF, batch=2, field=(32, 32),
-                                  kernel=(3, 3), ci=3, co=64),
-                      {"pass": "TRAINING_WU"}) == "generic direct"
+    # ... except when there is too little work to pay for the copy
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=4,
                                   co=8)) == "generic direct"
     # method names of the reference steer the choice

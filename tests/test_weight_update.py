@@ -198,6 +198,22 @@ def test_weight_deltas_on_gpu_match_oracle(oracle, kw):
     assert rel_l2(got, want) <= 1e-5, (rel_l2(got, want), plan.describe())
 
 
+@pytest.mark.gpu
+def test_weight_deltas_of_a_small_batch_run_on_the_matrix_cores(oracle):
+    # the pass's input channels are the layer's batch: 4 of them are padded
+    # to a whole vector and the pass stays on the matrix cores
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, pa.FLOAT, batch=4, field=(14, 14), kernel=(3, 3),
+                    ci=32, co=48, pad=1)
+    rng = np.random.default_rng(26)
+    xq, xd = quantize(rng.standard_normal((4, 32, 14, 14)), pa.HALF)
+    dq, dd = quantize(rng.standard_normal((4, 48, 14, 14)) * 0.1, pa.HALF)
+    got, plan = run_weight_update(p, xq, dq)
+    assert "implicit GEMM" in plan.describe(), plan.describe()
+    assert "input channels padded      4 -> 8" in plan.describe()
+    assert rel_l2(got, oracle.weight_deltas(p, xd, dd, threads=8)) <= 1e-5
+
+
 DEPTHWISE_WU_CASES = [
     dict(batch=3, field=(20, 21), kernel=(3, 3), groups=24, stride=2, pad=1),
     dict(batch=2, field=(14, 14), kernel=(5, 5), groups=16, pad=2),
