@@ -107,6 +107,11 @@ __device__ __forceinline__ void igemmTile(
   const uint32_t g = gs - part * d.groups;
   out += size_t(part) * a.M * (d.groups * d.outChansPerGroup);
   const uint32_t mode = a.mode;
+  // The input is addressed with 32-bit offsets from the first image the
+  // tile reads - a tile's rows span few images, the whole tensor may be far
+  // larger than 2^31 bytes.
+  const uint32_t firstImage =
+      a.divOutD(a.divOutH(a.divOutW(mTile * kBlockM)));
 
   const int t = threadIdx.x;
   const bool producer = t >= kThreads - kProducers; // waves 4-7
@@ -146,8 +151,11 @@ __device__ __forceinline__ void igemmTile(
                    d.inW +
                uint32_t(d.padW > 0 ? d.padW : 0)) *
                   pixelBytes;
+    const uint64_t skipped = uint64_t(firstImage) * a.imageBytes;
+    const uint64_t left = a.inBytes - skipped + shift;
     const __amdgpu_buffer_rsrc_t inBuf =
-        bufferOf(in - shift, a.inBytes + shift);
+        bufferOf(in + skipped - shift,
+                 uint32_t(left < kOutOfRange - 1 ? left : kOutOfRange - 1));
     const __amdgpu_buffer_rsrc_t wBuf = bufferOf(w, a.wBytes);
 
     // Load r of this wave fills the 8-row block (r * 4 + pw) of the A tile.
@@ -388,8 +396,9 @@ __device__ __forceinline__ void igemmTile(
       const uint32_t ow = mm - q * d.outW;
       const uint32_t q2 = a.divOutH(q);
       const uint32_t oh = q - q2 * d.outH;
-      const uint32_t b = a.divOutD(q2);
-      const uint32_t od = q2 - b * d.outD;
+      const uint32_t image = a.divOutD(q2);
+      const uint32_t od = q2 - image * d.outD;
+      const uint32_t b = image - firstImage; // (0 for an invalid row: unused)
       const int idBase = int(od * d.strideD) - d.padD;
       const int ihBase = int(oh * d.strideH) - d.padH;
       const int iwBase = int(ow * d.strideW) - d.padW;
@@ -770,6 +779,26 @@ int igemmTapAddressing(const IgemmDesc &d) {
   return d.kD * d.kH * d.kW > 32 ? kRangeTaps : kMaskTaps;
 }
 
+bool igemmAddressable(const IgemmDesc &d, int inType) {
+  const uint64_t eb = inType == kFloat ? 4 : inType == kHalf ? 2 : 1;
+  const uint64_t imageBytes =
+      uint64_t(d.inD) * d.inH * d.inW * d.groups * d.inChansPerGroup * eb;
+  const uint64_t shift = ((uint64_t(d.padD > 0 ? d.padD : 0) * d.inH +
+                           uint64_t(d.padH > 0 ? d.padH : 0)) *
+                              d.inW +
+                          uint64_t(d.padW > 0 ? d.padW : 0)) *
+                         d.groups * d.inChansPerGroup * eb;
+  // images a tile of 128 output rows can touch: its rows' own, one more when
+  // it starts inside an image
+  const uint64_t rowsPerImage = uint64_t(d.outD) * d.outH * d.outW;
+  if (rowsPerImage == 0)
+    return true;
+  uint64_t images = (kBlockM - 1) / rowsPerImage + 2;
+  if (images > d.batch)
+    images = d.batch;
+  return images * imageBytes + shift < kOutOfRange - (1u << 20);
+}
+
 size_t igemmWorkspaceBytes(const IgemmDesc &d) {
   if (d.splitK <= 1)
     return 0;
@@ -850,19 +879,15 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
   a.kPadded = (k + bke - 1) / bke * bke;
   // every part runs the same number of k-steps; steps beyond K load zeros
   a.kSteps = (a.kPadded / bke + d.splitK - 1) / d.splitK;
-  // Buffer addressing is 32-bit; the planner keeps larger tensors away.
-  const uint64_t inBytes =
-      uint64_t(d.batch) * d.inD * d.inH * d.inW * d.groups *
-      d.inChansPerGroup * eb;
+  // Buffer addressing is 32-bit: the weights as a whole, the input from the
+  // first image a tile reads (igemmAddressable; the planner keeps other
+  // shapes away).
   const uint64_t wBytes = uint64_t(d.groups) * a.coPadded * a.kPadded * eb;
-  const uint64_t shift = ((uint64_t(d.padD > 0 ? d.padD : 0) * d.inH +
-                           uint64_t(d.padH > 0 ? d.padH : 0)) *
-                              d.inW +
-                          uint64_t(d.padW > 0 ? d.padW : 0)) *
-                         d.groups * d.inChansPerGroup * eb;
-  if (inBytes + shift >= kOutOfRange || wBytes >= kOutOfRange)
+  if (!igemmAddressable(d, inType) || wBytes >= kOutOfRange)
     return hipErrorInvalidConfiguration;
-  a.inBytes = uint32_t(inBytes);
+  a.imageBytes = uint32_t(uint64_t(d.inD) * d.inH * d.inW * d.groups *
+                          d.inChansPerGroup * eb);
+  a.inBytes = uint64_t(d.batch) * a.imageBytes;
   a.wBytes = uint32_t(wBytes);
   return hipSuccess;
 }

@@ -25,7 +25,8 @@ struct IgemmArgs {
   uint32_t kSteps;   // k-steps each workgroup runs (one part of K)
   uint32_t kPadded;  // row length of the packed weights, in elements
   uint32_t coPadded; // rows per group of the packed weights
-  uint32_t inBytes;  // size of the input tensor
+  uint64_t inBytes;    // size of the input tensor
+  uint32_t imageBytes; // ... and of one image (batch element) of it
   uint32_t wBytes;   // size of the packed weights
 };
 

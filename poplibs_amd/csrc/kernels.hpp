@@ -146,6 +146,10 @@ struct IgemmDesc {
 /// rows and columns per pixel (more taps), or arithmetic per tap (dilated
 /// input).
 enum : int { kMaskTaps = 0, kRangeTaps = 1, kDilatedTaps = 2 };
+/// Whether the kernel can address the input: it uses 32-bit offsets from the
+/// first image (batch element) a tile of 128 output rows reads, so those few
+/// images - not the tensor - have to stay under 2^31 bytes.
+bool igemmAddressable(const IgemmDesc &d, int inType);
 int igemmTapAddressing(const IgemmDesc &d);
 size_t igemmWorkspaceBytes(const IgemmDesc &d);
 hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,

@@ -252,6 +252,20 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   const std::size_t vecElems = 16 / params.inputType.size();
   const std::size_t ciPadded = (ci + vecElems - 1) / vecElems * vecElems;
 
+  // The matrix-core kernel addresses its input with 32-bit offsets from the
+  // first image a tile reads.
+  auto inputAddressable = [&] {
+    mxk::IgemmDesc g{};
+    g.batch = uint32_t(s.batch), g.groups = uint32_t(p.numConvGroups);
+    g.inChansPerGroup = uint32_t(ciPadded);
+    g.inD = s.inD, g.inH = s.inH, g.inW = s.inW;
+    g.outD = s.outD, g.outH = s.outH, g.outW = s.outW;
+    g.padD = s.padD, g.padH = s.padH, g.padW = s.padW;
+    return s.batch < (1ull << 31) &&
+           mxk::igemmAddressable(
+               g, halfIn ? mxk::kHalf : floatIn ? mxk::kFloat : mxk::kQuarter);
+  };
+
   // Which kernels can take this convolution at all?
   std::string igemmWhyNot, dwWhyNot;
   std::pair<unsigned, unsigned> dwTile{0, 0};
@@ -266,11 +280,6 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       // (one channel per group is vector-ALU work)
       igemmWhyNot = "input channels per group not a multiple of a 16-byte "
                     "vector";
-    else if (ciPadded != ci &&
-             s.batch * s.inD * s.inH * s.inW * p.numConvGroups * ciPadded *
-                     params.inputType.size() >=
-                 (1ull << 30))
-      igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     else if (ciPadded != ci && pc.kernel != "igemm" &&
              2.0 * double(s.batch) * s.outD * s.outH * s.outW * s.kD * s.kH *
                      s.kW * ci * co * p.numConvGroups <
@@ -297,8 +306,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     else if (!s.inputDilated() && std::size_t(s.kH) * s.kW > 32 &&
              (s.kH > 255 || s.kW > 255))
       igemmWhyNot = "kernel extent above 255";
-    else if (plan.inputElems * params.inputType.size() >= (1ull << 30) ||
-             plan.weightElems * params.inputType.size() >= (1ull << 30))
+    else if (!inputAddressable() ||
+             s.batch * s.outD * s.outH * s.outW >= (1ull << 31) ||
+             p.numConvGroups * ((co + 127) / 128 * 128) * s.kD * s.kH * s.kW *
+                     (ciPadded + vecElems * 8) * params.inputType.size() >=
+                 (1ull << 31))
       igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     if (s.hasDepth())
       dwWhyNot = "three field dimensions";

@@ -547,6 +547,45 @@ def test_igemm_three_dimensions_of_signs_is_exact(oracle):
     _run(oracle, p, 42, 0, "implicit GEMM", dist="pm1")
 
 
+def test_igemm_input_beyond_two_gigabytes(oracle):
+    """The input is addressed with 32-bit offsets from the first image a tile
+    reads, so the tensor itself may exceed 2^31 bytes: every image of such a
+    batch must come out exactly as it does alone."""
+    import torch
+    from poplibs_amd import capi
+    kw = dict(field=(512, 512), kernel=(3, 3), ci=256, co=16, pad=1)
+    big = make_params(pa.HALF, pa.HALF, batch=18, **kw)
+    one = make_params(pa.HALF, pa.HALF, batch=1, **kw)
+    plan_big, plan_one = pa.Plan(big), pa.Plan(one)
+    assert _plan_kernel(plan_big) == "implicit GEMM", plan_big.describe()
+    assert plan_big.buffer_bytes(capi.BUF_INPUT) > 2 ** 31
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn((18, 512, 512, 256), generator=g, device=dev,
+                    dtype=torch.float16)           # channels-last, as documented
+    w = (torch.randn((1, 16, 256, 3, 3), generator=g, device=dev,
+                     dtype=torch.float16) * 0.02)
+
+    def buf(plan, which):
+        return torch.empty(max(plan.buffer_bytes(which), 16),
+                           dtype=torch.uint8, device=dev)
+
+    def run(plan, x_part):
+        wp, out = buf(plan, capi.BUF_WEIGHTS_PACKED), buf(plan, capi.BUF_OUTPUT)
+        ws = buf(plan, capi.BUF_WORKSPACE)
+        plan.pack_weights(w.data_ptr(), wp.data_ptr())
+        plan.fwd(x_part.data_ptr(), wp.data_ptr(), out.data_ptr(), None,
+                 ws.data_ptr(), ws.numel())
+        torch.cuda.synchronize()
+        return out.view(torch.float16)
+
+    got = run(plan_big, x).view(18, 512, 512, 16)
+    for image in (0, 7, 8, 17):
+        alone = run(plan_one, x[image].contiguous()).view(512, 512, 16)
+        assert torch.equal(got[image], alone), image
+    assert torch.isfinite(got).all() and got.abs().max() > 0
+
+
 STAGES_CASES = [
     # (params, input type, forced stages or None for the planner's choice)
     (dict(batch=3, field=(9, 11), kernel=(3, 3), ci=128, co=130, pad=1),
