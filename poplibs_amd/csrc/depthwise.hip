@@ -274,6 +274,30 @@ hipError_t runKernelShape(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream) {
+  // The kernels address a launch's tensors with 32-bit offsets.  Images are
+  // independent: a batch whose input or output exceeds that goes out as
+  // several launches of as many images as fit.
+  {
+    const uint64_t outBytes = outType == kHalf ? 2 : 4;
+    const uint64_t inImage = uint64_t(d.inH) * d.inW * d.channels * 2;
+    const uint64_t outImage = uint64_t(d.outH) * d.outW * d.channels * outBytes;
+    const uint64_t limit = kOutOfRange / 2;
+    const uint64_t image = inImage > outImage ? inImage : outImage;
+    if (image != 0 && image < limit && uint64_t(d.batch) * image >= limit) {
+      const uint32_t perLaunch = uint32_t(limit / image);
+      for (uint32_t first = 0; first < d.batch; first += perLaunch) {
+        DepthwiseDesc part = d;
+        part.batch = d.batch - first < perLaunch ? d.batch - first : perLaunch;
+        const hipError_t e = launchDepthwise(
+            part, inType, outType,
+            static_cast<const char *>(in) + first * inImage, weightsPacked,
+            bias, static_cast<char *>(out) + first * outImage, stream);
+        if (e != hipSuccess)
+          return e;
+      }
+      return hipSuccess;
+    }
+  }
   if (d.inDilH != 1 || d.inDilW != 1)
     return launchDepthwiseDirect(d, inType, outType, in, weightsPacked, bias,
                                  out, stream);

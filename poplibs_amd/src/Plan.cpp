@@ -320,13 +320,15 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       dwWhyNot = "not one channel per group";
     else if (p.numConvGroups % 8 != 0)
       dwWhyNot = "channel count not a multiple of 8";
-    else if (plan.inputElems * 2 >= (1ull << 31))
-      dwWhyNot = "tensor too large for 32-bit buffer addressing";
+    else if (std::size_t(s.inH) * s.inW * p.numConvGroups * 2 >=
+                 (1ull << 30) ||
+             std::size_t(s.outH) * s.outW * p.numConvGroups * 4 >=
+                 (1ull << 30))
+      dwWhyNot = "image too large for 32-bit buffer addressing";
     else if (!s.inputDilated() &&
              (dwTile = chooseDepthwiseTile(s, p.numConvGroups / 8)).first == 0)
       dwWhyNot = "input patch of a single output pixel exceeds the LDS budget";
-    else if (s.inputDilated() && plan.outputElems / 8 >= (1ull << 31))
-      dwWhyNot = "tensor too large for 32-bit item numbers";
+
   }
 
   // Choose.  PopLibs method names map onto the kernels that take their role:

@@ -586,6 +586,41 @@ def test_igemm_input_beyond_two_gigabytes(oracle):
     assert torch.isfinite(got).all() and got.abs().max() > 0
 
 
+def test_depthwise_batch_beyond_one_launch(oracle):
+    """A depthwise batch too large for one launch's 32-bit offsets goes out
+    in several launches: every image as it comes out alone."""
+    import torch
+    from poplibs_amd import capi
+    kw = dict(field=(112, 112), kernel=(3, 3), groups=96, stride=2, pad=1)
+    big = make_params(pa.HALF, pa.HALF, batch=520, **kw)
+    one = make_params(pa.HALF, pa.HALF, batch=1, **kw)
+    plan_big, plan_one = pa.Plan(big), pa.Plan(one)
+    assert _plan_kernel(plan_big) == "depthwise direct", plan_big.describe()
+    assert plan_big.buffer_bytes(capi.BUF_INPUT) > 2 ** 30
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(6)
+    x = torch.randn((520, 112, 112, 96), generator=g, device=dev,
+                    dtype=torch.float16)
+    w = torch.randn((96, 1, 1, 3, 3), generator=g, device=dev,
+                    dtype=torch.float16)
+
+    def buf(plan, which):
+        return torch.empty(max(plan.buffer_bytes(which), 16),
+                           dtype=torch.uint8, device=dev)
+
+    def run(plan, x_part):
+        wp, out = buf(plan, capi.BUF_WEIGHTS_PACKED), buf(plan, capi.BUF_OUTPUT)
+        plan.pack_weights(w.data_ptr(), wp.data_ptr())
+        plan.fwd(x_part.data_ptr(), wp.data_ptr(), out.data_ptr())
+        torch.cuda.synchronize()
+        return out.view(torch.float16)
+
+    got = run(plan_big, x).view(520, 56, 56, 96)
+    for image in (0, 221, 222, 443, 444, 519):
+        alone = run(plan_one, x[image].contiguous()).view(56, 56, 96)
+        assert torch.equal(got[image], alone), image
+
+
 STAGES_CASES = [
     # (params, input type, forced stages or None for the planner's choice)
     (dict(batch=3, field=(9, 11), kernel=(3, 3), ci=128, co=130, pad=1),
