@@ -844,11 +844,19 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
     return hipErrorInvalidValue;
   if (d.kD == 0 || d.kH == 0 || d.kW == 0)
     return hipErrorInvalidValue;
+  // outputs mapped into a larger field: plain 2-D convolutions, K not split
+  const bool outMapped = d.outFullH != 0 || d.outFullW != 0;
+  if (outMapped &&
+      (d.outD != 1 || d.splitK != 1 || d.outStepH == 0 || d.outStepW == 0 ||
+       (d.outH != 0 && (d.outH - 1) * d.outStepH + d.outOffH >= d.outFullH) ||
+       (d.outW != 0 && (d.outW - 1) * d.outStepW + d.outOffW >= d.outFullW)))
+    return hipErrorInvalidValue;
   if (d.splitK > 1 &&
       (!haveWorkspace || (d.groups * d.outChansPerGroup) % 4 != 0))
     return hipErrorInvalidValue;
   a.d = d;
   a.mode = uint32_t(mode);
+  a.outMapped = outMapped ? 1u : 0u;
   a.divInDilH = makeFastDiv(d.inDilH);
   a.divInDilW = makeFastDiv(d.inDilW);
   a.divCiBytes = makeFastDiv(d.inChansPerGroup * eb);
@@ -878,7 +886,7 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
   const uint32_t k = d.kD * d.kH * d.kW * d.inChansPerGroup;
   a.kPadded = (k + bke - 1) / bke * bke;
   // every part runs the same number of k-steps; steps beyond K load zeros
-  a.kSteps = (a.kPadded / bke + d.splitK - 1) / d.splitK;
+  a.kSteps = d.noTaps ? 0 : (a.kPadded / bke + d.splitK - 1) / d.splitK;
   // Buffer addressing is 32-bit: the weights as a whole, the input from the
   // first image a tile reads (igemmAddressable; the planner keeps other
   // shapes away).

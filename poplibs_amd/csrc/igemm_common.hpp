@@ -19,6 +19,7 @@ struct IgemmArgs {
   FastDiv divOutD, divKH;
   uint32_t tapRowStarts; // tap mask mode: bit kh * kW for every kernel row
   uint32_t tapPlaneStarts; // ... and bit kd * kH * kW for every kernel plane
+  uint32_t outMapped; // outputs go to every outStep-th pixel of a larger field
   uint32_t mode;     // kMaskTaps, kRangeTaps or kDilatedTaps
   uint32_t M;        // batch * outH * outW
   uint32_t mTiles, nTiles;
@@ -334,7 +335,17 @@ igemmEpilogue(char *lds, const IgemmArgs &a, floatx16 (&acc)[2][BN / 64],
     if (m >= a.M || n >= d.outChansPerGroup)
       continue;
     const char *src = lds + mLocal * kOutRow + vec * 16;
-    OutT *dst = out + size_t(m) * outChans + g * d.outChansPerGroup + n;
+    // the output pixel of row m: m itself, or - one phase of a convolution
+    // over a zero-stuffed input - every outStep-th pixel of a larger field
+    size_t pixel = m;
+    if (a.outMapped) {
+      const uint32_t q = a.divOutW(m), ow = m - q * d.outW;
+      const uint32_t image = a.divOutH(q), oh = q - image * d.outH;
+      pixel = (size_t(image) * d.outFullH + oh * d.outStepH + d.outOffH) *
+                  d.outFullW +
+              ow * d.outStepW + d.outOffW;
+    }
+    OutT *dst = out + pixel * outChans + g * d.outChansPerGroup + n;
     if (vectorOk) {
       *reinterpret_cast<uintx4 *>(dst) = *reinterpret_cast<const uintx4 *>(src);
     } else {

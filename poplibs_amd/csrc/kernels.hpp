@@ -65,6 +65,15 @@ hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
 /// Zero-fills `bytes` (a multiple of 4) with a kernel, so that the call can
 /// be recorded into a graph.
 hipError_t launchZero(void *dst, uint64_t bytes, hipStream_t stream);
+/// out[image][fullH][fullW][chans] (kHalf or kFloat): every element outside
+/// rows [offH, offH + insideH) x columns [offW, offW + insideW) becomes
+/// bias[channel], or 0 without a bias; the inside is not touched.
+hipError_t launchFillOutputPadding(int type, void *out, const void *bias,
+                                   uint64_t images, uint32_t fullH,
+                                   uint32_t fullW, uint32_t offH,
+                                   uint32_t offW, uint32_t insideH,
+                                   uint32_t insideW, uint32_t chans,
+                                   hipStream_t stream);
 
 /// biases[c] += scale * sum over rows of zDeltas[row][c] (half or float each),
 /// summed in fp32 in a fixed order: per-split partial sums go to `workspace`
@@ -98,12 +107,21 @@ hipError_t launchPadChans(const void *src, void *dst, uint64_t pixels,
 /// zero-filled beyond Co and beyond taps * Ci: the B operand of the
 /// matrix-core kernel, K contiguous.  With ciPadded (not 0) every tap takes
 /// ciPadded places of k, the ones beyond Ci zero.
+/// `select` (optional) packs a sub-kernel: of a kH x kW kernel the taps
+/// (firstH + i * stepH, firstW + j * stepW), i < countH, j < countW, in that
+/// order; `taps` is then kH * kW of the source and K holds countH * countW of
+/// them (none: all zeros).
+struct IgemmTapSelection {
+  uint32_t kW;
+  uint32_t firstH, stepH, countH, firstW, stepW, countW;
+};
 hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                                   uint32_t co, uint32_t ci, uint32_t taps,
                                   uint32_t coPadded, uint32_t kPadded,
                                   int elemBytes, hipStream_t stream,
                                   bool chansTransposed = false,
-                                  uint32_t ciPadded = 0);
+                                  uint32_t ciPadded = 0,
+                                  const IgemmTapSelection *select = nullptr);
 
 /// acts[outer][c] += bias[c] for `type` elements (kHalf or kFloat).
 hipError_t launchAddBias(int type, void *acts, const void *bias,
@@ -128,6 +146,18 @@ struct IgemmDesc {
   uint32_t inD = 1, outD = 1, kD = 1;
   int32_t padD = 0;
   uint32_t strideD = 1, dilD = 1, loD = 0, hiD = 1;
+  // Where the outputs go: pixel (oh, ow) of this convolution is pixel
+  // (oh * outStepH + outOffH, ow * outStepW + outOffW) of an output tensor
+  // with outFullH x outFullW pixels per image (0: the convolution's own
+  // field).  That is how one phase of a convolution over a zero-stuffed input
+  // - the outputs whose windows meet the same residue of real input rows and
+  // columns - writes its share of the whole output.  No depth with it.
+  uint32_t outFullH = 0, outFullW = 0;
+  uint32_t outStepH = 1, outStepW = 1, outOffH = 0, outOffW = 0;
+  // No tap of the kernel ever reads real input (a phase of a zero-stuffed
+  // input that only meets stuffed zeros): the outputs are the bias, or zero,
+  // and the workgroups run no k-step at all.
+  uint32_t noTaps = 0;
   // Zeros stuffed between input elements: input row r sits at row r * inDilH
   // of the field the window slides over (padH, strideH, dilH are in those
   // coordinates; loH, hiH bound r itself).  1 = none.

@@ -33,7 +33,8 @@ template <class T>
 __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
     const T *__restrict__ src, T *__restrict__ dst, uint32_t co, uint32_t ci,
     uint32_t ciPadded, uint32_t taps, uint32_t coPadded, uint32_t kPadded,
-    uint64_t total, bool chansTransposed) {
+    uint64_t total, bool chansTransposed, bool selected,
+    IgemmTapSelection select) {
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
     return;
@@ -41,8 +42,16 @@ __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
   const uint32_t n = uint32_t((tid / kPadded) % coPadded);
   const uint64_t g = tid / (uint64_t(kPadded) * coPadded);
   T v = T(0);
-  if (n < co && k < taps * ciPadded) {
-    const uint32_t tap = k / ciPadded, c = k % ciPadded;
+  const uint32_t packedTaps =
+      selected ? select.countH * select.countW : taps;
+  if (n < co && k < packedTaps * ciPadded) {
+    uint32_t tap = k / ciPadded;
+    const uint32_t c = k % ciPadded;
+    if (selected) {
+      const uint32_t i = tap / select.countW, j = tap % select.countW;
+      tap = (select.firstH + i * select.stepH) * select.kW + select.firstW +
+            j * select.stepW;
+    }
     // source [G][Co][Ci][taps], or [G][Ci][Co][taps] (a matrix
     // multiplication's right-hand side)
     if (c < ci)
@@ -335,7 +344,9 @@ hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                                   uint32_t co, uint32_t ci, uint32_t taps,
                                   uint32_t coPadded, uint32_t kPadded,
                                   int elemBytes, hipStream_t stream,
-                                  bool chansTransposed, uint32_t ciPadded) {
+                                  bool chansTransposed, uint32_t ciPadded,
+                                  const IgemmTapSelection *select) {
+  const IgemmTapSelection chosen = select ? *select : IgemmTapSelection{};
   if (ciPadded == 0)
     ciPadded = ci;
   if (ciPadded < ci)
@@ -351,17 +362,20 @@ hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint8_t>, grid, block, 0, stream,
                        static_cast<const uint8_t *>(src),
                        static_cast<uint8_t *>(dst), co, ci, ciPadded, taps,
-                       coPadded, kPadded, total, chansTransposed);
+                       coPadded, kPadded, total, chansTransposed,
+                       select != nullptr, chosen);
   else if (elemBytes == 2)
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint16_t>, grid, block, 0, stream,
                        static_cast<const uint16_t *>(src),
                        static_cast<uint16_t *>(dst), co, ci, ciPadded, taps,
-                       coPadded, kPadded, total, chansTransposed);
+                       coPadded, kPadded, total, chansTransposed,
+                       select != nullptr, chosen);
   else if (elemBytes == 4)
     hipLaunchKernelGGL(packIgemmWeightsKernel<uint32_t>, grid, block, 0, stream,
                        static_cast<const uint32_t *>(src),
                        static_cast<uint32_t *>(dst), co, ci, ciPadded, taps,
-                       coPadded, kPadded, total, chansTransposed);
+                       coPadded, kPadded, total, chansTransposed,
+                       select != nullptr, chosen);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
@@ -522,6 +536,105 @@ hipError_t launchZero(void *dst, uint64_t bytes, hipStream_t stream) {
     return hipErrorInvalidConfiguration;
   hipLaunchKernelGGL(zeroKernel<uint32_t>, dim3(uint32_t(blocks)), dim3(256), 0,
                      stream, static_cast<uint32_t *>(dst), total);
+  return hipGetLastError();
+}
+
+namespace {
+/// One element of the padded output field per thread; those inside the
+/// convolution's own outputs are left alone.
+template <class T>
+__global__ __launch_bounds__(256) void fillOutputPaddingKernel(
+    T *__restrict__ out, const T *__restrict__ bias, uint64_t total,
+    uint32_t fullH, uint32_t fullW, uint32_t offH, uint32_t offW,
+    uint32_t insideH, uint32_t insideW, uint32_t chans) {
+  const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= total)
+    return;
+  const uint64_t pixel = tid / chans;
+  const uint32_t c = uint32_t(tid - pixel * chans);
+  const uint32_t w = uint32_t(pixel % fullW);
+  const uint32_t h = uint32_t((pixel / fullW) % fullH);
+  if (h - offH < insideH && w - offW < insideW)
+    return;
+  out[tid] = bias ? bias[c] : T(0);
+}
+} // namespace
+
+namespace {
+/// The same with one 16-byte vector per thread and 32-bit arithmetic inside
+/// an image (blockIdx.y, .z: the image); channel counts that are whole
+/// vectors.
+template <class T>
+__global__ __launch_bounds__(256) void fillOutputPaddingVectorKernel(
+    T *__restrict__ out, const T *__restrict__ bias, uint32_t imageVectors,
+    uint32_t fullW, uint32_t offH, uint32_t offW, uint32_t insideH,
+    uint32_t insideW, uint32_t vecsPerPixel) {
+  constexpr uint32_t kVec = 16 / sizeof(T);
+  const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= imageVectors)
+    return;
+  const uint32_t pixel = idx / vecsPerPixel, vec = idx - pixel * vecsPerPixel;
+  const uint32_t h = pixel / fullW, w = pixel - h * fullW;
+  if (h - offH < insideH && w - offW < insideW)
+    return;
+  const uint64_t image = uint64_t(blockIdx.z) * gridDim.y + blockIdx.y;
+  uint4 v{0, 0, 0, 0};
+  if (bias)
+    v = *reinterpret_cast<const uint4 *>(bias + vec * kVec);
+  reinterpret_cast<uint4 *>(out)[image * imageVectors + idx] = v;
+}
+} // namespace
+
+hipError_t launchFillOutputPadding(int type, void *out, const void *bias,
+                                   uint64_t images, uint32_t fullH,
+                                   uint32_t fullW, uint32_t offH,
+                                   uint32_t offW, uint32_t insideH,
+                                   uint32_t insideW, uint32_t chans,
+                                   hipStream_t stream) {
+  const uint64_t total = images * fullH * fullW * chans;
+  if (total == 0)
+    return hipSuccess;
+  const uint32_t vecElems = type == kHalf ? 8 : 4;
+  const uint64_t imageVectors = uint64_t(fullH) * fullW * (chans / vecElems);
+  if ((type == kHalf || type == kFloat) && chans % vecElems == 0 &&
+      imageVectors < (1ull << 31) &&
+      (bias == nullptr || reinterpret_cast<uintptr_t>(bias) % 16 == 0) &&
+      reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    // images as grid y (and z beyond 32768 of them)
+    const uint32_t gy = uint32_t(images < 32768 ? images : 32768);
+    if (images % gy == 0 && images / gy < 65536) {
+      const dim3 grid{uint32_t((imageVectors + 255) / 256), gy,
+                      uint32_t(images / gy)};
+      if (type == kHalf)
+        hipLaunchKernelGGL(fillOutputPaddingVectorKernel<__half>, grid,
+                           dim3(256), 0, stream, static_cast<__half *>(out),
+                           static_cast<const __half *>(bias),
+                           uint32_t(imageVectors), fullW, offH, offW, insideH,
+                           insideW, chans / vecElems);
+      else
+        hipLaunchKernelGGL(fillOutputPaddingVectorKernel<float>, grid,
+                           dim3(256), 0, stream, static_cast<float *>(out),
+                           static_cast<const float *>(bias),
+                           uint32_t(imageVectors), fullW, offH, offW, insideH,
+                           insideW, chans / vecElems);
+      return hipGetLastError();
+    }
+  }
+  const uint64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull)
+    return hipErrorInvalidConfiguration;
+  if (type == kHalf)
+    hipLaunchKernelGGL(fillOutputPaddingKernel<__half>, dim3(uint32_t(blocks)),
+                       dim3(256), 0, stream, static_cast<__half *>(out),
+                       static_cast<const __half *>(bias), total, fullH, fullW,
+                       offH, offW, insideH, insideW, chans);
+  else if (type == kFloat)
+    hipLaunchKernelGGL(fillOutputPaddingKernel<float>, dim3(uint32_t(blocks)),
+                       dim3(256), 0, stream, static_cast<float *>(out),
+                       static_cast<const float *>(bias), total, fullH, fullW,
+                       offH, offW, insideH, insideW, chans);
+  else
+    return hipErrorInvalidValue;
   return hipGetLastError();
 }
 

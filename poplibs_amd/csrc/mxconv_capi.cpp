@@ -137,6 +137,22 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   switch (plan->kernel) {
   case mxconv_plan::Kernel::IGEMM:
+    if (plan->outputPadded) {
+      // zeros (the bias) around the convolution's own outputs
+      const mxk::IgemmDesc &g = plan->igemm;
+      const uint32_t insideH = g.outFullH - plan->outputPadLoH -
+                               plan->outputPadHiH,
+                     insideW = g.outFullW - plan->outputPadLoW -
+                               plan->outputPadHiW;
+      const mxconv_status st = hipStatus(
+          mxk::launchFillOutputPadding(
+              outType, out, bias, g.batch, g.outFullH, g.outFullW,
+              plan->outputPadLoH, plan->outputPadLoW, insideH, insideW,
+              uint32_t(plan->params.getNumOutputChans()), s),
+          "output padding fill");
+      if (st != MXCONV_OK)
+        return st;
+    }
     if (plan->pointwiseOn)
       return hipStatus(mxk::launchPointwise(plan->pointwise, inType, outType,
                                             in, w, bias, out, s),
@@ -155,6 +171,24 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
       if (st != MXCONV_OK)
         return st;
       in = padded;
+    }
+    if (!plan->igemmPhases.empty()) {
+      // one convolution per phase of the zero-stuffed input, in one launch
+      mxk::IgemmFusedItem items[mxk::kIgemmMaxFused];
+      size_t count = 0;
+      const size_t elemBytes = plan->params.inputType.size();
+      for (const auto &phase : plan->igemmPhases)
+        items[count++] = {&phase.d,
+                          inType,
+                          outType,
+                          in,
+                          static_cast<const char *>(w) +
+                              phase.packedOffset * elemBytes,
+                          bias,
+                          out,
+                          q};
+      return hipStatus(mxk::launchIgemmFused(items, count, s),
+                       "implicit-GEMM convolution launch (phases)");
     }
     return hipStatus(mxk::launchIgemm(plan->igemm, inType, outType, in, w,
                                       bias, out, workspace, q, s),
@@ -551,6 +585,22 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
       return hipStatus(mxk::launchPackPointwiseWeights(
                            plan->pointwise, weights_external, weights_packed, s),
                        "weight packing");
+    for (const auto &phase : plan->igemmPhases) {
+      const mxconv_status st = hipStatus(
+          mxk::launchPackIgemmWeights(
+              weights_external,
+              static_cast<char *>(weights_packed) +
+                  phase.packedOffset * elemBytes,
+              uint32_t(p.numConvGroups), uint32_t(p.outputChannelsPerConvGroup),
+              uint32_t(p.inputChannelsPerConvGroup), uint32_t(taps),
+              uint32_t(plan->coPadded), uint32_t(phase.kPadded), elemBytes, s,
+              false, uint32_t(plan->paddedInputChans), &phase.taps),
+          "weight packing");
+      if (st != MXCONV_OK)
+        return st;
+    }
+    if (!plan->igemmPhases.empty())
+      return MXCONV_OK;
     return hipStatus(
         mxk::launchPackIgemmWeights(
             weights_external, weights_packed, uint32_t(p.numConvGroups),
@@ -709,7 +759,7 @@ mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
     const mxconv_plan *p = plans[i];
     // (a plan that pads its input channels runs a copy first: on its own)
     if (p->outputElems == 0 || p->kernel != mxconv_plan::Kernel::IGEMM ||
-        p->pointwiseOn || p->paddedInputChans)
+        p->pointwiseOn || p->paddedInputChans || !p->igemmPhases.empty())
       return false;
     unsplit[slot] = p->igemm;
     unsplit[slot].splitK = 1;
@@ -1135,7 +1185,7 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
       return st;
   }
   if (plan->kernel == mxconv_plan::Kernel::IGEMM && !plan->pointwiseOn &&
-      !plan->paddedInputChans) {
+      !plan->paddedInputChans && plan->igemmPhases.empty()) {
     // deltas [B][Y][G][Co] -> straight into the matrix-core kernel's packed
     // weights [G][coPadded][kPadded], k = y * B + b
     if (plan->coPadded != Co || plan->kPadded != Y * B) {

@@ -70,6 +70,11 @@ struct Simple2D {
   int32_t padD = 0;
   uint32_t strideD = 1, dilD = 1, loD = 0, hiD = 1, inDilD = 1;
   std::size_t batch = 0; // the batch size times the folded depth
+  // Zeros around the output field (outH, outW are the convolution's own).
+  uint32_t outPadLoH = 0, outPadHiH = 0, outPadLoW = 0, outPadHiW = 0;
+  bool outputPadded() const {
+    return outPadLoH || outPadHiH || outPadLoW || outPadHiW;
+  }
   bool hasDepth() const { return inD != 1 || outD != 1 || kD != 1; }
   bool inputDilated() const {
     return inDilH != 1 || inDilW != 1 || inDilD != 1;
@@ -96,8 +101,8 @@ Simple2D asSimple2D(const ConvParams &p) {
       s.why = "kernel truncation, padding or flip";
       return s;
     }
-    if (ot.paddingLower[d] || ot.paddingUpper[d]) {
-      s.why = "output padding";
+    if ((ot.paddingLower[d] || ot.paddingUpper[d]) && n == 3 && d == 0) {
+      s.why = "output padding in the depth dimension";
       return s;
     }
     // conv index = o*stride + outTruncLo; padded input = conv + k*dil;
@@ -114,7 +119,12 @@ Simple2D asSimple2D(const ConvParams &p) {
       return which == 0 ? dd : which == 1 ? hh : ww;
     };
     pick(s.inD, s.inH, s.inW) = uint32_t(p.inputFieldShape[d]);
-    pick(s.outD, s.outH, s.outW) = uint32_t(p.getOutputSize(d));
+    pick(s.outD, s.outH, s.outW) = uint32_t(
+        p.getOutputSize(d) - ot.paddingLower[d] - ot.paddingUpper[d]);
+    if (which != 0) {
+      (which == 1 ? s.outPadLoH : s.outPadLoW) = ot.paddingLower[d];
+      (which == 1 ? s.outPadHiH : s.outPadHiW) = ot.paddingUpper[d];
+    }
     pick(s.kD, s.kH, s.kW) = uint32_t(p.kernelShape[d]);
     pick(s.padD, s.padH, s.padW) = pad;
     pick(s.strideD, s.strideH, s.strideW) = ot.stride[d];
@@ -220,7 +230,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   // dilation the layer's stride and its stride the layer's kernel dilation.
   {
     const Simple2D w = asSimple2D(p);
-    if (w.ok && !w.hasDepth() && w.batch == 1 && !plan.zeroConv &&
+    if (w.ok && !w.hasDepth() && !w.outputPadded() && w.batch == 1 &&
+        !plan.zeroConv &&
         !w.inputDilated() && p.batchSize == 1 &&
         p.outputChannelsPerConvGroup == 1 &&
         params.inputType == poplar::HALF && p.numConvGroups % 8 == 0 &&
@@ -294,9 +305,10 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                  32768)
       igemmWhyNot = "field too large for 16-bit window origins";
     else if (s.hasDepth() &&
-             (s.inputDilated() || std::size_t(s.kD) * s.kH * s.kW > 32))
-      igemmWhyNot = "three field dimensions with a dilated input or more "
-                    "than 32 kernel taps";
+             (s.inputDilated() || s.outputPadded() ||
+              std::size_t(s.kD) * s.kH * s.kW > 32))
+      igemmWhyNot = "three field dimensions with a dilated input, a padded "
+                    "output or more than 32 kernel taps";
     else if (s.inputDilated() &&
              (std::size_t(s.inW) * p.getNumInputChans() *
                       params.inputType.size() >=
@@ -314,6 +326,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     if (s.hasDepth())
       dwWhyNot = "three field dimensions";
+    else if (s.outputPadded())
+      dwWhyNot = "output padding";
     else if (!halfIn)
       dwWhyNot = "depthwise kernel takes half inputs";
     else if (ci != 1 || co != 1)
@@ -391,6 +405,16 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     g.dilH = s.dilH, g.dilW = s.dilW;
     g.loH = s.loH, g.hiH = s.hiH, g.loW = s.loW, g.hiW = s.hiW;
     g.inDilH = s.inDilH, g.inDilW = s.inDilW;
+    if (s.outputPadded()) {
+      // the convolution writes the inside of the padded field; the launch
+      // fills the field with zeros (or the bias) first
+      g.outFullH = s.outH + s.outPadLoH + s.outPadHiH;
+      g.outFullW = s.outW + s.outPadLoW + s.outPadHiW;
+      g.outOffH = s.outPadLoH, g.outOffW = s.outPadLoW;
+      plan.outputPadded = true;
+      plan.outputPadLoH = s.outPadLoH, plan.outputPadHiH = s.outPadHiH;
+      plan.outputPadLoW = s.outPadLoW, plan.outputPadHiW = s.outPadHiW;
+    }
     // Tile shape.  M = batch * outH * outW pixels, N = out channels of one
     // group, K = kH * kW * in channels.  A 128-pixel tile keeps the A
     // fragment reuse high; N is 128 unless the group has at most 64 output
@@ -430,6 +454,10 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       // tiles of more than 1 GB are not worth it
       if (chans % 4 != 0 || parts * m * chans * 4 > (1ull << 30))
         parts = 1;
+      // (the sum of the parts is written pixel after pixel: not into a
+      // padded output field)
+      if (s.outputPadded())
+        parts = 1;
       g.splitK = uint32_t(parts);
       plan.workspaceBytes = mxk::igemmWorkspaceBytes(g);
       if (ciPadded != ci) {
@@ -451,6 +479,101 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         throw poplar::invalid_option(
             "planConstraints gfx950 stages must be 2 or 4");
     }
+    // Zero-stuffed input, window moving by single pixels: one ordinary
+    // convolution per phase instead of arithmetic on every tap - no MACs on
+    // the stuffed zeros, and the fast tap-mask addressing.
+    if (s.inputDilated() && !s.hasDepth() && g.splitK == 1 &&
+        (s.inDilH == 1 || s.strideH == 1) &&
+        (s.inDilW == 1 || s.strideW == 1) &&
+        std::size_t(s.inDilH) * s.inDilW <= mxk::kIgemmMaxFused) {
+      // One dimension of one phase.  The window of output o = q * inDil +
+      // phase meets real input under kernel tap k when phase - pad + k * dil
+      // is a multiple of inDil - taps first, first + step, ... - and reads
+      // input q + (phase - pad + k * dil) / inDil there.
+      struct Dim {
+        uint32_t out = 0, first = 0, step = 1, count = 0;
+        int32_t pad = 0;
+        uint32_t dil = 1;
+        bool dead = false; // no tap ever meets real input: all zeros
+      };
+      auto dimOf = [](uint32_t phase, uint32_t inDil, uint32_t out,
+                      uint32_t k, int32_t pad, uint32_t dil) {
+        Dim r;
+        r.out = out > phase ? (out - phase + inDil - 1) / inDil : 0;
+        int64_t firstOffset = 0;
+        for (uint32_t t = 0; t != k; ++t) {
+          const int64_t x = int64_t(phase) - pad + int64_t(t) * dil;
+          if (x % int64_t(inDil) != 0)
+            continue;
+          if (r.count == 0)
+            r.first = t, firstOffset = x / int64_t(inDil);
+          else if (r.count == 1)
+            r.step = t - r.first;
+          ++r.count;
+        }
+        if (r.count == 0) {
+          r.dead = true, r.count = 1;
+          return r;
+        }
+        r.pad = int32_t(-firstOffset);
+        r.dil = r.count > 1 ? r.step * dil / inDil : 1;
+        return r;
+      };
+      std::size_t offset = 0;
+      for (uint32_t ph = 0; ph != s.inDilH; ++ph)
+        for (uint32_t pw = 0; pw != s.inDilW; ++pw) {
+          // a dimension that is not dilated keeps its stride and geometry
+          const Dim h = s.inDilH == 1
+                            ? Dim{s.outH, 0, 1, s.kH, s.padH, s.dilH, false}
+                            : dimOf(ph, s.inDilH, s.outH, s.kH, s.padH, s.dilH);
+          const Dim w = s.inDilW == 1
+                            ? Dim{s.outW, 0, 1, s.kW, s.padW, s.dilW, false}
+                            : dimOf(pw, s.inDilW, s.outW, s.kW, s.padW, s.dilW);
+          if (h.out == 0 || w.out == 0)
+            continue;
+          mxconv_plan::IgemmPhase phase;
+          mxk::IgemmDesc &q = phase.d;
+          q = g;
+          q.inDilH = q.inDilW = 1;
+          q.outH = h.out, q.outW = w.out, q.kH = h.count, q.kW = w.count;
+          q.padH = h.pad, q.padW = w.pad, q.dilH = h.dil, q.dilW = w.dil;
+          if (s.inDilH != 1)
+            q.strideH = 1;
+          if (s.inDilW != 1)
+            q.strideW = 1;
+          if (h.dead)
+            q.loH = q.hiH = 0;
+          if (w.dead)
+            q.loW = q.hiW = 0;
+          q.outFullH = s.outH + s.outPadLoH + s.outPadHiH;
+          q.outFullW = s.outW + s.outPadLoW + s.outPadHiW;
+          q.outStepH = s.inDilH, q.outStepW = s.inDilW;
+          q.outOffH = ph + s.outPadLoH, q.outOffW = pw + s.outPadLoW;
+          const bool dead = h.dead || w.dead;
+          q.noTaps = dead ? 1 : 0;
+          phase.taps = {s.kW,
+                        h.first, h.step, dead ? 0u : h.count,
+                        w.first, w.step, dead ? 0u : w.count};
+          const std::size_t kk = std::size_t(q.kH) * q.kW * ciPadded;
+          phase.kPadded = (kk + g.blockK - 1) / g.blockK * g.blockK;
+          phase.packedOffset = offset;
+          offset += p.numConvGroups * plan.coPadded * phase.kPadded;
+          plan.igemmPhases.push_back(phase);
+        }
+      // (kernel of more than 32 taps per phase: the ranges take over inside
+      // the kernel, as for any convolution)
+      plan.weightPackedElems = offset;
+      std::size_t phaseTiles = 0;
+      for (const auto &ph : plan.igemmPhases)
+        phaseTiles += (std::size_t(ph.d.batch) * ph.d.outH * ph.d.outW +
+                       g.blockM - 1) /
+                      g.blockM * (plan.coPadded / g.blockN) * g.groups;
+      const uint32_t stages =
+          pc.stages ? pc.stages : (phaseTiles > gfx950::numCUs ? 2 : 4);
+      for (auto &ph : plan.igemmPhases)
+        ph.d.stages = stages;
+      g.stages = stages;
+    }
     // A pointwise convolution with few input channels is bound by HBM, not
     // by the matrix cores: unless the big tile was asked for explicitly, the
     // streaming kernel of small workgroups takes it.
@@ -459,7 +582,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     pw.groups = g.groups, pw.inChansPerGroup = g.inChansPerGroup;
     pw.outChansPerGroup = g.outChansPerGroup;
     const bool unitWindow =
-        !s.hasDepth() && !s.inputDilated() && g.splitK == 1 && s.kH == 1 &&
+        !s.hasDepth() && !s.outputPadded() && !s.inputDilated() &&
+        g.splitK == 1 && s.kH == 1 &&
         s.kW == 1 &&
         s.strideH == 1 && s.strideW == 1 &&
         s.padH == 0 && s.padW == 0 && s.loH == 0 && s.loW == 0 &&
@@ -574,6 +698,10 @@ std::string mxconv_plan::describe() const {
       if (mxk::igemmTapAddressing(g) == mxk::kRangeTaps)
         os << "        tap addressing             ranges of valid kernel rows "
               "and columns (more than 32 taps)\n";
+      else if (!igemmPhases.empty())
+        os << "        dilated input              " << igemmPhases.size()
+           << " phases, one convolution of the undilated input each, in "
+              "one launch\n";
       else if (mxk::igemmTapAddressing(g) == mxk::kDilatedTaps)
         os << "        tap addressing             arithmetic (dilated "
               "input)\n";

@@ -10,6 +10,7 @@
 #include "poplin/ConvParams.hpp"
 #include <cstddef>
 #include <string>
+#include <vector>
 
 /// Fixed properties of the one target this library is written for.
 namespace gfx950 {
@@ -47,6 +48,26 @@ struct mxconv_plan {
 
   // Packed weights of the matrix-core kernel: [G][coPadded][kPadded].
   std::size_t coPadded = 0, kPadded = 0;
+  // A convolution over a zero-stuffed input (the backward pass of a strided
+  // layer), taken apart: the outputs whose windows meet the same residue of
+  // real input rows and columns form one ordinary convolution of the
+  // UNdilated input with a sub-kernel - one "phase" each, all in one launch.
+  // Empty when the convolution is not run that way.  Each phase's packed
+  // weights [G][coPadded][kPadded of the phase] start packedOffset elements
+  // into the packed buffer.
+  struct IgemmPhase {
+    mxk::IgemmDesc d;
+    mxk::IgemmTapSelection taps;
+    std::size_t packedOffset = 0, kPadded = 0;
+  };
+  std::vector<IgemmPhase> igemmPhases;
+  // The output field has zero padding around the convolution's own outputs:
+  // the launch fills it with zeros (or the bias) before the kernel writes
+  // the inside.
+  bool outputPadded = false;
+  uint32_t outputPadLoH = 0, outputPadHiH = 0, outputPadLoW = 0,
+           outputPadHiW = 0;
+
   // Input channels per group as the matrix-core kernel sees them, when that
   // is more than the parameters say (0 otherwise): the channels are padded
   // with zeros to a whole 16-byte vector by a copy into the workspace, at

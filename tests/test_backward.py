@@ -136,9 +136,12 @@ BWD_GPU_CASES = [
     (dict(batch=2, field=(9, 9), kernel=(1, 1), ci=256, co=64),
      "implicit GEMM"),
     # forward stride 2: the deltas are dilated going backwards - the matrix
-    # cores take it with arithmetic tap addressing
+    # cores take it as one convolution per phase of the stuffed zeros
     (dict(batch=2, field=(9, 10), kernel=(3, 3), ci=8, co=16, stride=2, pad=1),
-     "arithmetic"),
+     "4 phases"),
+    # ... also a strided 1x1 shortcut, three of whose four phases are zeros
+    (dict(batch=2, field=(9, 10), kernel=(1, 1), ci=16, co=24, stride=2),
+     "4 phases"),
     # depthwise 3x3 stride 2: dilated deltas, one thread per output vector
     (dict(batch=2, field=(13, 12), kernel=(3, 3), groups=24, stride=2, pad=1),
      "dilated input"),

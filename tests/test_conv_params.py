@@ -394,7 +394,12 @@ def test_planner_choices():
     # matrix cores, with other ways of telling which taps read the input
     dilated = pa.Plan(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
                                   co=8, idil=2)).describe()
-    assert "implicit GEMM" in dilated and "arithmetic" in dilated
+    assert "implicit GEMM" in dilated and "4 phases" in dilated
+    # ... with a window that moves by more than one pixel over the stuffed
+    # input there are no such phases: every tap's position is worked out
+    strided = pa.Plan(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
+                                  co=8, idil=2, stride=2)).describe()
+    assert "implicit GEMM" in strided and "arithmetic" in strided
     many = pa.Plan(make_params(pa.HALF, batch=128, field=(28, 28),
                                kernel=(28, 28), ci=32, co=128, pad=1))
     assert "implicit GEMM" in many.describe()
@@ -426,6 +431,9 @@ def test_planner_choices():
                                   ci=8, co=8)) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
                                   ci=8, co=8, idil=(1, 2, 1))) == \
+        "generic direct"
+    assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
+                                  ci=8, co=8, opu=(0, 1, 0))) == \
         "generic direct"
     folded = pa.Plan(make_params(pa.HALF, batch=2, field=(5, 9, 9),
                                  kernel=(1, 7, 7), ci=8, co=8))

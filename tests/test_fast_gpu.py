@@ -363,6 +363,9 @@ GENERAL_CASES = [
     # dilation and truncation together, 1-D
     dict(batch=2, field=(33,), kernel=(5,), ci=24, co=8, idil=2, itl=(2,),
          itu=(1,), pad=4, stride=3),
+    # a window that strides over a dilated input: arithmetic on every tap
+    dict(batch=2, field=(11, 12), kernel=(3, 3), ci=64, co=24, idil=2,
+         stride=(2, 3), pad=2),
     # a weight-update-like pass: the "kernel" is a whole 12x12 field, dilated
     dict(batch=16, field=(26, 26), kernel=(12, 12), ci=8, co=24, kdil=2,
          padLower=(1, 1), padUpper=(0, 0)),
@@ -379,7 +382,8 @@ def test_igemm_general_addressing_matches_oracle(oracle, kw, out_type):
     aq, ad = quantize(acts, pa.HALF)
     wq, wd = quantize(weights * 0.05, pa.HALF)
     got, plan = run_conv(p, aq, wq, return_plan=True)
-    assert "tap addressing" in plan.describe(), plan.describe()
+    assert ("tap addressing" in plan.describe()
+            or "phases" in plan.describe()), plan.describe()
     want = oracle.convolution(p, ad, wd, threads=8)
     assert rel_l2(got, want) <= 1e-3, (rel_l2(got, want), plan.describe())
 
@@ -619,6 +623,86 @@ def test_depthwise_batch_beyond_one_launch(oracle):
     for image in (0, 221, 222, 443, 444, 519):
         alone = run(plan_one, x[image].contiguous()).view(56, 56, 96)
         assert torch.equal(got[image], alone), image
+
+
+PHASE_CASES = [
+    # (input type, params, phases expected)
+    # backward of 3x3 stride 2: phases of 1, 2, 2 and 4 taps
+    (pa.HALF, dict(batch=2, field=(14, 15), kernel=(3, 3), ci=64, co=40,
+                   idil=2, padLower=(1, 1), padUpper=(2, 2)), 4),
+    # backward of 1x1 stride 2: one phase carries everything, three are zero
+    (pa.HALF, dict(batch=2, field=(9, 10), kernel=(1, 1), ci=64, co=16,
+                   idil=2, padUpper=(1, 1)), 4),
+    # 7x7, dilated by 2 in both dimensions: 16 taps in the largest phase
+    (pa.HALF, dict(batch=1, field=(12, 11), kernel=(7, 7), ci=8, co=24,
+                   idil=2, pad=3), 4),
+    # one dimension only; the other strides and has a dilated kernel
+    (pa.HALF, dict(batch=2, field=(8, 13), kernel=(3, 3), ci=16, co=72,
+                   idil=(3, 1), stride=(1, 2), kdil=(1, 2), pad=2, groups=2),
+     3),
+    # dilation 3 x 2, kernel dilation 2: phases without any tap in a dimension
+    (pa.HALF, dict(batch=2, field=(7, 9), kernel=(3, 2), ci=16, co=136,
+                   idil=(3, 2), pad=2, kdil=(2, 2)), 6),
+    # truncation of the input under the dilation, negative effective padding
+    (pa.HALF, dict(batch=2, field=(12, 12), kernel=(3, 3), ci=8, co=8, idil=2,
+                   itl=(1, 2), itu=(2, 0), padLower=(0, 0),
+                   padUpper=(0, 0)), 4),
+    # few channels (padded copy), float and quarter operands
+    (pa.HALF, dict(batch=4, field=(16, 16), kernel=(3, 3), ci=3, co=32,
+                   idil=2, pad=1), 4),
+    (pa.FLOAT, dict(batch=2, field=(9, 8), kernel=(3, 3), ci=8, co=16, idil=2,
+                    pad=2), 4),
+    (pa.QUARTER, dict(batch=2, field=(9, 8), kernel=(3, 3), ci=32, co=16,
+                      idil=2, pad=2), 4),
+]
+
+
+@pytest.mark.parametrize("in_type,kw,phases", PHASE_CASES)
+def test_igemm_phases_of_a_dilated_input(oracle, in_type, kw, phases):
+    out_type = pa.FLOAT if in_type == pa.FLOAT else pa.HALF
+    p = make_params(in_type, out_type, **kw)
+    print("case", p, flush=True)
+    if in_type == pa.QUARTER:
+        got, want, plan = _fp8_case(oracle, p, 51, 1, 1)
+    else:
+        from gpu_helpers import quantize, run_conv
+        acts, weights, biases = random_data(p, 51, "normal")
+        aq, ad = quantize(acts, in_type)
+        wq, wd = quantize(weights * 0.1, in_type)
+        bq, bd = quantize(biases, out_type)
+        got, plan = run_conv(p, aq, wq, bq, None, return_plan=True)
+        want = oracle.convolution(p, ad, wd, bd, threads=8)
+    assert "%d phases" % phases in plan.describe(), plan.describe()
+    assert rel_l2(got, want) <= (2e-6 if in_type == pa.FLOAT else 1e-3), \
+        (rel_l2(got, want), plan.describe())
+
+
+OUTPUT_PADDING_CASES = [
+    dict(batch=2, field=(9, 8), kernel=(3, 3), ci=16, co=24, pad=1,
+         opl=(1, 0), opu=(2, 3)),
+    dict(batch=2, field=(12, 12), kernel=(3, 3), ci=8, co=40, stride=2,
+         otl=(1, 0), opl=(0, 2), opu=(1, 0), groups=2),
+    # what the backward pass of a strided 1x1 layer on an even field is: the
+    # forward pass never read the last row and column
+    dict(batch=2, field=(5, 5), kernel=(1, 1), ci=64, co=32, idil=2,
+         opu=(1, 1)),
+    dict(batch=2, field=(6, 7), kernel=(3, 3), ci=16, co=16, idil=2, pad=2,
+         opl=(1, 1), opu=(0, 2)),
+]
+
+
+@pytest.mark.parametrize("kw", OUTPUT_PADDING_CASES)
+@pytest.mark.parametrize("bias", [False, True])
+def test_igemm_output_padding(oracle, kw, bias):
+    p = make_params(pa.HALF, pa.HALF, **kw)
+    print("case", p, flush=True)
+    _run(oracle, p, 53, 1e-3, "implicit GEMM", wscale=0.1, bias=bias)
+
+
+def test_igemm_phases_of_signs_are_exact(oracle):
+    p = make_params(pa.HALF, pa.FLOAT, batch=2, field=(9, 9), kernel=(3, 3),
+                    ci=32, co=24, idil=2, pad=2)
+    _run(oracle, p, 52, 0, "implicit GEMM", dist="pm1")
 
 
 STAGES_CASES = [

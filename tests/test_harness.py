@@ -175,6 +175,19 @@ def test_conv_random_quarter(seed):
     assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-3000:])
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(1086, 1106))
+def test_conv_random_float(seed):
+    # float inputs run on the matrix cores too; these seeds include three
+    # field dimensions with output padding and dilated inputs
+    import sys
+    print("conv_random_float seed", seed, flush=True)
+    r = subprocess.run([sys.executable, RANDOM, "--seed", str(seed),
+                        "--input-type", "float"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-3000:])
+
+
 # ---------------------------------------------------------------------------
 # general_matrix_multiply: the reference's cases for its tool of that name
 # (tests/poplin/CMakeLists.txt:515-900).
