@@ -757,9 +757,11 @@ mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
   };
   auto fusedItem = [&](size_t i, size_t slot, mxk::IgemmFusedItem &item) {
     const mxconv_plan *p = plans[i];
-    // (a plan that pads its input channels runs a copy first: on its own)
+    // (a plan with more to a launch than its one kernel - a padded copy of
+    // the input, several phases, an output border to fill - runs on its own)
     if (p->outputElems == 0 || p->kernel != mxconv_plan::Kernel::IGEMM ||
-        p->pointwiseOn || p->paddedInputChans || !p->igemmPhases.empty())
+        p->pointwiseOn || p->paddedInputChans || !p->igemmPhases.empty() ||
+        p->outputPadded)
       return false;
     unsplit[slot] = p->igemm;
     unsplit[slot].splitK = 1;

@@ -46,6 +46,13 @@ MULTI_CASES = [
     # and two with the narrow tile and per-lane taps
     dict(batch=2, field=(8, 8), kernel=(3, 3), ci=8, co=24, pad=1),
     dict(batch=1, field=(10, 4), kernel=(1, 3), ci=24, co=40),
+    # launches with more to them than one kernel - a padded copy of the
+    # input, phases of a dilated input, a padded output field - run on their
+    # own inside the set
+    dict(batch=4, field=(16, 16), kernel=(3, 3), ci=3, co=128, pad=1),
+    dict(batch=2, field=(9, 8), kernel=(3, 3), ci=64, co=136, idil=2, pad=2),
+    dict(batch=2, field=(9, 8), kernel=(3, 3), ci=64, co=136, pad=1,
+         opl=(1, 0), opu=(0, 2)),
 ]
 
 
@@ -91,6 +98,8 @@ def test_multi_fwd_equals_single_convolutions(oracle, parallel):
         keep += [x_ext, w_ext, x_int, w_pack, o_int, scratch]
         params.append((p, o_int, t))
     assert any("K split" in p.describe() for p in plans)
+    assert any("input channels padded" in p.describe() for p in plans)
+    assert any("phases" in p.describe() for p in plans)
     # twice, with work of the caller's stream in between
     for _ in range(2):
         pa.multi_fwd(plans, ins, ws, outs, workspaces=wss,
