@@ -203,7 +203,7 @@ hipError_t launchIgemmFused(const IgemmFusedItem *items, size_t count,
                             hipStream_t stream);
 
 /// Pointwise convolution (every kernel extent 1, stride 1, no padding or
-/// truncation, half inputs) with 128, 256 or 512 input channels per group:
+/// truncation, half inputs) with 64, 128, 256 or 512 input channels per group:
 /// a streaming kernel of small workgroups instead of igemm's big tiles.
 struct PointwiseDesc {
   uint32_t batch, pixels; // pixels per image

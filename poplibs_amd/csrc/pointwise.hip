@@ -53,7 +53,10 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
     PwArgs a, const char *__restrict__ in, const char *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
   constexpr int kRow = KS * 32;                 // bytes of one activation row
-  constexpr int kChunkBits = KS == 8 ? 4 : KS == 16 ? 5 : 6; // log2(kRow / 16)
+  constexpr int kChunkBits =
+      KS == 4 ? 3 : KS == 8 ? 4 : KS == 16 ? 5 : 6; // log2(kRow / 16)
+  // chunk c of row r sits at chunk position c ^ (r & kSwizzle)
+  constexpr uint32_t kSwizzle = KS == 4 ? 7u : 15u;
   constexpr int kRowsPerLoad = 1024 / kRow;
   constexpr int kLoads = TM / kRowsPerLoad; // wave-wide loads per tile
   constexpr int kTileBytes = TM * kRow;
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
 #pragma unroll
       for (int load = 0; load != kLoads; ++load) {
         const uint32_t row = load * kRowsPerLoad + rowInLoad;
-        const uint32_t chunk = pos ^ (row & 15u);
+        const uint32_t chunk = pos ^ (row & kSwizzle);
         const uint32_t m = mTile * TM + row;
         loadToLds(inBuf, (LdsPtr)(buffer + load * 1024),
                   m < a.M ? m * pixelBytes + g * kRow + chunk * 16
@@ -129,7 +132,7 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
                    : 0.0f;
   }
   const uint32_t rowLocal = mb * 32 + (lane & 31);
-  const uint32_t swizzle = rowLocal & 15u, half = lane >> 5;
+  const uint32_t swizzle = rowLocal & kSwizzle, half = lane >> 5;
   char *stage = lds + NB * kTileBytes + wave * 32 * kPwStageRow;
   const uint32_t outChans = d.groups * d.outChansPerGroup;
   // Output leaves in passes of 64 bytes per pixel: all 32 channels of the
@@ -268,6 +271,8 @@ hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
                      const void *bias, void *out, hipStream_t stream) {
   // Tiles of 16 KB, three in flight; 32 KB, two in flight, for the widest.
   switch (a.d.inChansPerGroup) {
+  case 64:
+    return run<4, 64, 4, OutT>(a, in, w, bias, out, stream);
   case 128:
     return run<8, 64, 4, OutT>(a, in, w, bias, out, stream);
   case 256:
@@ -285,7 +290,7 @@ bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType) {
   const uint64_t m = uint64_t(d.batch) * d.pixels;
   const uint64_t inBytes = m * d.groups * ci * 2;
   return inType == kHalf && (outType == kHalf || outType == kFloat) &&
-         (ci == 128 || ci == 256 || ci == 512) && co != 0 &&
+         (ci == 64 || ci == 128 || ci == 256 || ci == 512) && co != 0 &&
          co % (outType == kHalf ? 8 : 4) == 0 && m != 0 && m < 0x7fffffffull &&
          inBytes < kOutOfRange &&
          pointwisePackedElems(d) * 2 < kOutOfRange;

@@ -89,7 +89,7 @@ def test_igemm_blockN_override_and_amp_method(oracle):
     _run(oracle, p, 3, 1e-3, "implicit GEMM", options=opts, wscale=0.1)
 
 
-# 1x1, stride 1, unpadded, 128 / 256 / 512 input channels per group: the
+# 1x1, stride 1, unpadded, 64 / 128 / 256 / 512 input channels per group: the
 # streaming kernel of small workgroups.  Ragged pixel counts and channel
 # counts against its 64 x 64 tile, groups, 0-D to 2-D fields.
 POINTWISE_CASES = [
@@ -98,6 +98,9 @@ POINTWISE_CASES = [
     dict(batch=1, field=(5, 9), kernel=(1, 1), ci=512, co=136, groups=2),
     dict(batch=70, field=(), kernel=(), ci=128, co=96),
     dict(batch=2, field=(33,), kernel=(1,), ci=256, co=8),
+    # 64 channels: rows of 128 bytes (the backward pass of a 256 -> 64 layer)
+    dict(batch=2, field=(28, 29), kernel=(1, 1), ci=64, co=256),
+    dict(batch=3, field=(7, 11), kernel=(1, 1), ci=64, co=72, groups=3),
 ]
 
 
