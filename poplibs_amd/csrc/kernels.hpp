@@ -61,6 +61,17 @@ hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
                                 uint32_t chans, uint64_t strideG,
                                 uint64_t strideC, uint64_t strideP,
                                 int elemBytes, hipStream_t stream);
+/// Two of them (same element size) in one launch where both take the vector
+/// path; otherwise one after the other.
+struct SwapBatchChans {
+  const void *src;
+  void *dst;
+  uint32_t batch, pixels, groups, chans;
+  uint64_t strideG, strideC, strideP;
+};
+hipError_t launchSwapBatchChansPair(const SwapBatchChans &first,
+                                    const SwapBatchChans &second,
+                                    int elemBytes, hipStream_t stream);
 
 /// Zero-fills `bytes` (a multiple of 4) with a kernel, so that the call can
 /// be recorded into a graph.

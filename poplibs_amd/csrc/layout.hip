@@ -154,14 +154,16 @@ struct SwapArgs {
 /// channels, stores along the batch (and on along the pixels where the
 /// destination keeps them adjacent).
 template <class T, bool VEC>
-__global__ __launch_bounds__(256) void swapBatchChansKernel(
-    SwapArgs a, const T *__restrict__ src, T *__restrict__ dst) {
+__device__ __forceinline__ void
+swapBatchChansTile(const SwapArgs &a, const T *__restrict__ src,
+                   T *__restrict__ dst, uint32_t blockX, uint32_t blockY,
+                   uint32_t blockZ) {
   __shared__ uint32_t tile[kSwapRows][kSwapChans + 1];
   const uint32_t cBlocks = (a.chans + kSwapChans - 1) / kSwapChans;
-  const uint32_t c0 = (blockIdx.x % cBlocks) * kSwapChans;
-  const uint32_t g = blockIdx.x / cBlocks;
-  const uint32_t p0 = blockIdx.y * a.pixelsPerTile;
-  const uint32_t b0 = blockIdx.z * a.batchPerTile;
+  const uint32_t c0 = (blockX % cBlocks) * kSwapChans;
+  const uint32_t g = blockX / cBlocks;
+  const uint32_t p0 = blockY * a.pixelsPerTile;
+  const uint32_t b0 = blockZ * a.batchPerTile;
   const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   // row = pLocal * batchPerTile + bLocal
   auto source = [&](uint32_t row, uint32_t c) {
@@ -246,6 +248,34 @@ __global__ __launch_bounds__(256) void swapBatchChansKernel(
       dst[g * a.strideG + c * a.strideC + p * a.strideP + b] =
           T(tile[row][cLocal]);
   }
+}
+
+template <class T, bool VEC>
+__global__ __launch_bounds__(256) void swapBatchChansKernel(
+    SwapArgs a, const T *__restrict__ src, T *__restrict__ dst) {
+  swapBatchChansTile<T, VEC>(a, src, dst, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+/// Two such rearrangements in one launch (the two operands of a weight update
+/// pass): the grid's z extent is the sum of theirs, x and y cover the larger;
+/// workgroups outside their tensor's own grid have nothing to do.
+struct SwapPairArgs {
+  SwapArgs a[2];
+  uint32_t gridX[2], gridY[2], gridZ0; // z blocks of the first
+};
+template <class T>
+__global__ __launch_bounds__(256) void swapBatchChansPairKernel(
+    SwapPairArgs m, const T *__restrict__ src0, T *__restrict__ dst0,
+    const T *__restrict__ src1, T *__restrict__ dst1) {
+  const uint32_t which = blockIdx.z < m.gridZ0 ? 0 : 1;
+  if (blockIdx.x >= m.gridX[which] || blockIdx.y >= m.gridY[which])
+    return;
+  if (which == 0)
+    swapBatchChansTile<T, true>(m.a[0], src0, dst0, blockIdx.x, blockIdx.y,
+                                blockIdx.z);
+  else
+    swapBatchChansTile<T, true>(m.a[1], src1, dst1, blockIdx.x, blockIdx.y,
+                                blockIdx.z - m.gridZ0);
 }
 
 template <class T>
@@ -471,14 +501,21 @@ hipError_t launchAddBias(int type, void *acts, const void *bias,
   return hipGetLastError();
 }
 
-hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
-                                uint32_t pixels, uint32_t groups,
-                                uint32_t chans, uint64_t strideG,
-                                uint64_t strideC, uint64_t strideP,
-                                int elemBytes, hipStream_t stream) {
-  if (uint64_t(batch) * pixels * groups * chans == 0)
-    return hipSuccess;
+namespace {
+struct SwapLaunch {
   SwapArgs a;
+  dim3 grid;
+  bool vectorLoads;
+};
+
+/// Tile shape, grid and vector widths of one rearrangement.
+hipError_t prepareSwap(const void *src, const void *dst, uint32_t batch,
+                       uint32_t pixels, uint32_t groups, uint32_t chans,
+                       uint64_t strideG, uint64_t strideC, uint64_t strideP,
+                       int elemBytes, SwapLaunch &l) {
+  if (elemBytes != 2 && elemBytes != 4)
+    return hipErrorInvalidValue;
+  SwapArgs &a = l.a;
   a.batch = batch, a.pixels = pixels, a.groups = groups, a.chans = chans;
   // As much of the batch as a tile takes (a power of two, so that it divides
   // the 128 rows), the rest of the rows for neighbouring pixels.
@@ -492,16 +529,35 @@ hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
   const uint64_t gz = (batch + a.batchPerTile - 1) / a.batchPerTile;
   if (gx > 0x7fffffffull || gy > 65535 || gz > 65535)
     return hipErrorInvalidConfiguration;
-  const dim3 grid{uint32_t(gx), uint32_t(gy), uint32_t(gz)}, block{256};
+  l.grid = dim3{uint32_t(gx), uint32_t(gy), uint32_t(gz)};
   // 16-byte loads need every row of channels to start on a 16-byte boundary;
   // 16-byte stores, every run of batch entries.
   const uint32_t perVector = uint32_t(16 / elemBytes);
-  const bool vec = chans % perVector == 0 &&
-                   reinterpret_cast<uintptr_t>(src) % 16 == 0;
+  l.vectorLoads = chans % perVector == 0 &&
+                  reinterpret_cast<uintptr_t>(src) % 16 == 0;
   a.vectorStores = batch % perVector == 0 && a.batchPerTile >= perVector &&
                    strideG % perVector == 0 && strideC % perVector == 0 &&
                    strideP % perVector == 0 &&
                    reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+  return hipSuccess;
+}
+} // namespace
+
+hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
+                                uint32_t pixels, uint32_t groups,
+                                uint32_t chans, uint64_t strideG,
+                                uint64_t strideC, uint64_t strideP,
+                                int elemBytes, hipStream_t stream) {
+  if (uint64_t(batch) * pixels * groups * chans == 0)
+    return hipSuccess;
+  SwapLaunch l;
+  const hipError_t e = prepareSwap(src, dst, batch, pixels, groups, chans,
+                                   strideG, strideC, strideP, elemBytes, l);
+  if (e != hipSuccess)
+    return e;
+  const SwapArgs &a = l.a;
+  const dim3 grid = l.grid, block{256};
+  const bool vec = l.vectorLoads;
   if (elemBytes == 2) {
     const auto *from = static_cast<const uint16_t *>(src);
     auto *to = static_cast<uint16_t *>(dst);
@@ -511,7 +567,7 @@ hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
     else
       hipLaunchKernelGGL((swapBatchChansKernel<uint16_t, false>), grid, block,
                          0, stream, a, from, to);
-  } else if (elemBytes == 4) {
+  } else {
     const auto *from = static_cast<const uint32_t *>(src);
     auto *to = static_cast<uint32_t *>(dst);
     if (vec)
@@ -520,9 +576,57 @@ hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
     else
       hipLaunchKernelGGL((swapBatchChansKernel<uint32_t, false>), grid, block,
                          0, stream, a, from, to);
-  } else {
-    return hipErrorInvalidValue;
   }
+  return hipGetLastError();
+}
+
+hipError_t launchSwapBatchChansPair(const SwapBatchChans &first,
+                                    const SwapBatchChans &second,
+                                    int elemBytes, hipStream_t stream) {
+  auto alone = [&](const SwapBatchChans &x) {
+    return launchSwapBatchChans(x.src, x.dst, x.batch, x.pixels, x.groups,
+                                x.chans, x.strideG, x.strideC, x.strideP,
+                                elemBytes, stream);
+  };
+  auto empty = [](const SwapBatchChans &x) {
+    return uint64_t(x.batch) * x.pixels * x.groups * x.chans == 0;
+  };
+  SwapLaunch l[2];
+  bool together = !empty(first) && !empty(second);
+  if (together) {
+    const SwapBatchChans *both[2] = {&first, &second};
+    for (int i = 0; i != 2 && together; ++i) {
+      const SwapBatchChans &x = *both[i];
+      together = prepareSwap(x.src, x.dst, x.batch, x.pixels, x.groups,
+                             x.chans, x.strideG, x.strideC, x.strideP,
+                             elemBytes, l[i]) == hipSuccess &&
+                 l[i].vectorLoads;
+    }
+    together = together && l[0].grid.z + l[1].grid.z <= 65535;
+  }
+  if (!together) {
+    const hipError_t e = alone(first);
+    return e != hipSuccess ? e : alone(second);
+  }
+  SwapPairArgs m;
+  for (int i = 0; i != 2; ++i)
+    m.a[i] = l[i].a, m.gridX[i] = l[i].grid.x, m.gridY[i] = l[i].grid.y;
+  m.gridZ0 = l[0].grid.z;
+  const dim3 grid{l[0].grid.x > l[1].grid.x ? l[0].grid.x : l[1].grid.x,
+                  l[0].grid.y > l[1].grid.y ? l[0].grid.y : l[1].grid.y,
+                  l[0].grid.z + l[1].grid.z};
+  if (elemBytes == 2)
+    hipLaunchKernelGGL(swapBatchChansPairKernel<uint16_t>, grid, dim3{256}, 0,
+                       stream, m, static_cast<const uint16_t *>(first.src),
+                       static_cast<uint16_t *>(first.dst),
+                       static_cast<const uint16_t *>(second.src),
+                       static_cast<uint16_t *>(second.dst));
+  else
+    hipLaunchKernelGGL(swapBatchChansPairKernel<uint32_t>, grid, dim3{256}, 0,
+                       stream, m, static_cast<const uint32_t *>(first.src),
+                       static_cast<uint32_t *>(first.dst),
+                       static_cast<const uint32_t *>(second.src),
+                       static_cast<uint32_t *>(second.dst));
   return hipGetLastError();
 }
 

@@ -1176,20 +1176,17 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
                          zDeltas, ws + w.planWorkspace, deltasOut, s),
                      "depthwise weight deltas");
   mxconv_status st;
-  if (plan->inputElems) {
-    // activations [B][X][G][Ci] -> the pass's input [Ci][X][G][B]
-    st = hipStatus(mxk::launchSwapBatchChans(acts, ws + w.input, uint32_t(B),
-                                             uint32_t(X), uint32_t(G),
-                                             uint32_t(Ci), B, X * G * B, G * B,
-                                             inBytes, s),
-                   "activation rearrangement");
-    if (st != MXCONV_OK)
-      return st;
-  }
-  if (plan->kernel == mxconv_plan::Kernel::IGEMM && !plan->pointwiseOn &&
-      !plan->paddedInputChans && plan->igemmPhases.empty()) {
+  // activations [B][X][G][Ci] -> the pass's input [Ci][X][G][B]
+  const mxk::SwapBatchChans actsSwap{
+      acts,        ws + w.input, uint32_t(B), uint32_t(X), uint32_t(G),
+      uint32_t(Ci), B,           X * G * B,   G * B};
+  const bool direct = plan->kernel == mxconv_plan::Kernel::IGEMM &&
+                      !plan->pointwiseOn && !plan->paddedInputChans &&
+                      plan->igemmPhases.empty();
+  if (direct) {
     // deltas [B][Y][G][Co] -> straight into the matrix-core kernel's packed
-    // weights [G][coPadded][kPadded], k = y * B + b
+    // weights [G][coPadded][kPadded], k = y * B + b; both rearrangements in
+    // one launch
     if (plan->coPadded != Co || plan->kPadded != Y * B) {
       st = hipStatus(mxk::launchZero(ws + w.weightsPacked,
                                      alignUp(plan->weightPackedBytes()), s),
@@ -1197,15 +1194,30 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
       if (st != MXCONV_OK)
         return st;
     }
-    st = hipStatus(mxk::launchSwapBatchChans(
-                       zDeltas, ws + w.weightsPacked, uint32_t(B), uint32_t(Y),
-                       uint32_t(G), uint32_t(Co),
-                       uint64_t(plan->coPadded) * plan->kPadded, plan->kPadded,
-                       B, inBytes, s),
-                   "delta rearrangement");
+    const mxk::SwapBatchChans deltasSwap{
+        zDeltas,
+        ws + w.weightsPacked,
+        uint32_t(B),
+        uint32_t(Y),
+        uint32_t(G),
+        uint32_t(Co),
+        uint64_t(plan->coPadded) * plan->kPadded,
+        plan->kPadded,
+        B};
+    st = hipStatus(
+        mxk::launchSwapBatchChansPair(actsSwap, deltasSwap, inBytes, s),
+        "activation and delta rearrangement");
     if (st != MXCONV_OK)
       return st;
   } else {
+    st = hipStatus(mxk::launchSwapBatchChans(
+                       actsSwap.src, actsSwap.dst, actsSwap.batch,
+                       actsSwap.pixels, actsSwap.groups, actsSwap.chans,
+                       actsSwap.strideG, actsSwap.strideC, actsSwap.strideP,
+                       inBytes, s),
+                   "activation rearrangement");
+    if (st != MXCONV_OK)
+      return st;
     if (plan->weightElems) {
       // deltas [B][Y][G][Co] -> the pass's weights [G][Co][B][Y]
       const uint64_t dims[4] = {B, Y, G, Co};
