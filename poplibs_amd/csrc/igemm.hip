@@ -738,7 +738,8 @@ hipError_t dispatch(const KernelKey &k, const Launch &launch) {
 template <class OutT>
 __global__ __launch_bounds__(64) void splitKReduceKernel(
     const float *__restrict__ partial, uint32_t parts, uint64_t elems,
-    uint32_t channels, const OutT *__restrict__ bias, OutT *__restrict__ out) {
+    uint32_t channels, const OutT *__restrict__ bias, OutT *__restrict__ out,
+    bool transposed) {
   const uint64_t i = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
   if (i >= elems)
     return;
@@ -762,11 +763,19 @@ __global__ __launch_bounds__(64) void splitKReduceKernel(
                 (sum[0].y + sum[1].y) + (sum[2].y + sum[3].y),
                 (sum[0].z + sum[1].z) + (sum[2].z + sum[3].z),
                 (sum[0].w + sum[1].w) + (sum[2].w + sum[3].w)};
+  const uint32_t c = uint32_t(i % channels);
   if (bias) {
-    const uint32_t c = uint32_t(i % channels);
 #pragma unroll
     for (int e = 0; e != 4; ++e)
       v[e] += Load<OutT>::at(bias, c + e, 0);
+  }
+  if (transposed) {
+    // [channel][pixel]
+    const uint64_t pixels = elems / channels, pixel = i / channels;
+#pragma unroll
+    for (int e = 0; e != 4; ++e)
+      storeOut(out, (c + e) * pixels + pixel, v[e]);
+    return;
   }
   storeOut4(out + i, v);
 }
@@ -857,6 +866,11 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
   a.d = d;
   a.mode = uint32_t(mode);
   a.outMapped = outMapped ? 1u : 0u;
+  if (d.outTransposed && outMapped)
+    return hipErrorInvalidValue;
+  // (with K split the workgroups write partial tiles, [pixel][channel] as
+  // ever; the kernel that adds them up transposes)
+  a.outTransposed = d.outTransposed && d.splitK == 1 ? 1u : 0u;
   a.divInDilH = makeFastDiv(d.inDilH);
   a.divInDilW = makeFastDiv(d.inDilW);
   a.divCiBytes = makeFastDiv(d.inChansPerGroup * eb);
@@ -932,12 +946,12 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
     hipLaunchKernelGGL(splitKReduceKernel<__half>, dim3(uint32_t(blocks)),
                        dim3(64), 0, stream, partial, d.splitK, elems,
                        channels, static_cast<const __half *>(bias),
-                       static_cast<__half *>(out));
+                       static_cast<__half *>(out), d.outTransposed != 0);
   else if (outType == kFloat)
     hipLaunchKernelGGL(splitKReduceKernel<float>, dim3(uint32_t(blocks)),
                        dim3(64), 0, stream, partial, d.splitK, elems,
                        channels, static_cast<const float *>(bias),
-                       static_cast<float *>(out));
+                       static_cast<float *>(out), d.outTransposed != 0);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

@@ -20,6 +20,7 @@ struct IgemmArgs {
   uint32_t tapRowStarts; // tap mask mode: bit kh * kW for every kernel row
   uint32_t tapPlaneStarts; // ... and bit kd * kH * kW for every kernel plane
   uint32_t outMapped; // outputs go to every outStep-th pixel of a larger field
+  uint32_t outTransposed; // the final result as [channel][pixel]
   uint32_t mode;     // kMaskTaps, kRangeTaps or kDilatedTaps
   uint32_t M;        // batch * outH * outW
   uint32_t mTiles, nTiles;
@@ -344,6 +345,13 @@ igemmEpilogue(char *lds, const IgemmArgs &a, floatx16 (&acc)[2][BN / 64],
       pixel = (size_t(image) * d.outFullH + oh * d.outStepH + d.outOffH) *
                   d.outFullW +
               ow * d.outStepW + d.outOffW;
+    }
+    if (a.outTransposed) {
+      // [channel][pixel]: element stores, for small outputs
+      const OutT *e = reinterpret_cast<const OutT *>(src);
+      for (int k = 0; k != kVecElems && n + k < d.outChansPerGroup; ++k)
+        out[size_t(g * d.outChansPerGroup + n + k) * a.M + m] = e[k];
+      continue;
     }
     OutT *dst = out + pixel * outChans + g * d.outChansPerGroup + n;
     if (vectorOk) {

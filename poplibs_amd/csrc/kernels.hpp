@@ -169,6 +169,10 @@ struct IgemmDesc {
   // input that only meets stuffed zeros): the outputs are the bias, or zero,
   // and the workgroups run no k-step at all.
   uint32_t noTaps = 0;
+  // Write the result as [channel][pixel] instead of [pixel][channel]: a
+  // weight update pass's result in weight order.  Element stores - for small
+  // outputs.  Not together with the output mapping above.
+  uint32_t outTransposed = 0;
   // Zeros stuffed between input elements: input row r sits at row r * inDilH
   // of the field the window slides over (padH, strideH, dilH are in those
   // coordinates; loH, hiH bound r itself).  1 = none.

@@ -1209,6 +1209,17 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
         "activation and delta rearrangement");
     if (st != MXCONV_OK)
       return st;
+    // The pass's output [Ci][K][G][Co] is wanted in weight order
+    // [G][Co][Ci][K] - its transpose as a matrix: the kernel (or, with K
+    // split, the sum of the parts) writes it that way.
+    mxk::IgemmDesc transposed = plan->igemm;
+    transposed.outTransposed = 1;
+    return hipStatus(
+        mxk::launchIgemm(transposed, p.inputType.id(), p.outputType.id(),
+                         ws + w.input, ws + w.weightsPacked, nullptr,
+                         deltasOut, ws + w.planWorkspace, mxk::QuarterInfo{},
+                         s),
+        "weight delta convolution launch");
   } else {
     st = hipStatus(mxk::launchSwapBatchChans(
                        actsSwap.src, actsSwap.dst, actsSwap.batch,
