@@ -93,6 +93,9 @@ __device__ __forceinline__ void igemmTile(
   // Per tile row: {byte offset of the input element under tap (0, 0), channel
   // 0 of the group; mask of taps that read inside the input}.
   uint2 *rowTable = reinterpret_cast<uint2 *>(lds + NS * kTileBytes);
+  // ... and, where kernel taps are told apart by ranges and the field has a
+  // depth, the range of valid kernel planes.
+  uint32_t *depthTable = reinterpret_cast<uint32_t *>(rowTable + kBlockM);
 
   const IgemmDesc &d = a.d;
   // tile = ((part * groups + g) * mTiles + mTile) * nTiles + nTile, taken
@@ -167,6 +170,7 @@ __device__ __forceinline__ void igemmTile(
     uint32_t rowOff[AROWS], tapMask[AROWS];
     int originW[AROWS];                       // dilated input only
     uint32_t khLo[AROWS], khSpan[AROWS], kwLo[AROWS], kwSpan[AROWS]; // ranges
+    uint32_t kdLo[AROWS], kdSpan[AROWS];
 
     uint32_t bOff[BROWS];
 #pragma unroll
@@ -325,7 +329,7 @@ __device__ __forceinline__ void igemmTile(
             bool ok;
             if constexpr (MODE == kRangeTaps)
               ok = (tap < taps) & (kh - khLo[r] < khSpan[r]) &
-                   (kw - kwLo[r] < kwSpan[r]);
+                   (kw - kwLo[r] < kwSpan[r]) & (kd - kdLo[r] < kdSpan[r]);
             else
               ok = (tapMask[r] & tapBit) != 0;
             LdsPtr dst = (LdsPtr)(base + r * 4 * kLoadBytes);
@@ -351,6 +355,12 @@ __device__ __forceinline__ void igemmTile(
         originW[r] = int(e.y & 0xffffu) - 32768;
         khLo[r] = e.y & 0xffu, khSpan[r] = (e.y >> 8) & 0xffu;
         kwLo[r] = (e.y >> 16) & 0xffu, kwSpan[r] = e.y >> 24;
+        if constexpr (MODE == kRangeTaps) {
+          const uint32_t planes = depthTable[(r * 4 + pw) * 8 + rowInBlock];
+          kdLo[r] = planes & 0xffu, kdSpan[r] = planes >> 8;
+        } else {
+          kdLo[r] = 0, kdSpan[r] = 1;
+        }
       }
       // The consumers start as soon as step 0 is there; the input loads of
       // the other stages go out behind their back.
@@ -443,6 +453,8 @@ __device__ __forceinline__ void igemmTile(
             (range(iwBase, int(d.loW), int(d.hiW), int(d.dilW), int(d.kW))
              << 16);
         rowTable[t] = uint2{originOffset, rowValid ? ranges : 0u};
+        depthTable[t] =
+            range(idBase, int(d.loD), int(d.hiD), int(d.dilD), int(d.kD));
       } else {
         uint32_t mask = 0;
         if (d.dilD == 1 && d.dilH == 1 && d.dilW == 1) {
@@ -848,8 +860,10 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
   // the ranges of valid kernel rows and columns are kept in 8 bits each
   if (mode == kRangeTaps && (d.kH > 255 || d.kW > 255))
     return hipErrorInvalidValue;
-  // a depth dimension goes with the tap mask only
-  if (mode != kMaskTaps && (d.inD != 1 || d.outD != 1 || d.kD != 1))
+  // a depth dimension goes with the tap mask and the ranges
+  if (mode == kDilatedTaps && (d.inD != 1 || d.outD != 1 || d.kD != 1))
+    return hipErrorInvalidValue;
+  if (mode == kRangeTaps && d.kD > 255)
     return hipErrorInvalidValue;
   if (d.kD == 0 || d.kH == 0 || d.kW == 0)
     return hipErrorInvalidValue;

@@ -270,7 +270,8 @@ template <int BN, class OutT> constexpr int epilogueLdsBytes() {
 /// that is larger (two stages and fp32 outputs).
 template <int BN, int NS, class OutT> constexpr int igemmLdsBytes() {
   constexpr int loop =
-      NS * (kBlockM + BN) * kRowBytes + kBlockM * int(sizeof(uint2));
+      NS * (kBlockM + BN) * kRowBytes +
+      kBlockM * int(sizeof(uint2) + sizeof(uint32_t));
   return loop > epilogueLdsBytes<BN, OutT>() ? loop
                                              : epilogueLdsBytes<BN, OutT>();
 }

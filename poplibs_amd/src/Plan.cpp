@@ -304,19 +304,17 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                      std::size_t(std::abs(s.padW)) >=
                  32768)
       igemmWhyNot = "field too large for 16-bit window origins";
-    else if (s.hasDepth() &&
-             (s.inputDilated() || s.outputPadded() ||
-              std::size_t(s.kD) * s.kH * s.kW > 32))
-      igemmWhyNot = "three field dimensions with a dilated input, a padded "
-                    "output or more than 32 kernel taps";
+    else if (s.hasDepth() && (s.inputDilated() || s.outputPadded()))
+      igemmWhyNot = "three field dimensions with a dilated input or a "
+                    "padded output";
     else if (s.inputDilated() &&
              (std::size_t(s.inW) * p.getNumInputChans() *
                       params.inputType.size() >=
                   (1u << 24) ||
               s.inDilH >= (1u << 24) || s.inDilW >= (1u << 24)))
       igemmWhyNot = "input rows too long for the arithmetic tap addressing";
-    else if (!s.inputDilated() && std::size_t(s.kH) * s.kW > 32 &&
-             (s.kH > 255 || s.kW > 255))
+    else if (!s.inputDilated() && std::size_t(s.kD) * s.kH * s.kW > 32 &&
+             (s.kD > 255 || s.kH > 255 || s.kW > 255))
       igemmWhyNot = "kernel extent above 255";
     else if (!inputAddressable() ||
              s.batch * s.outD * s.outH * s.outW >= (1ull << 31) ||

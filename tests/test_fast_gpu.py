@@ -531,6 +531,13 @@ DEPTH_CASES = [
     # a depth the window does not slide over: folded into the batch
     (pa.HALF, dict(batch=2, field=(5, 9, 9), kernel=(1, 7, 7), ci=8, co=16,
                    padLower=(0, 3, 3), padUpper=(0, 3, 3))),
+    # more than 32 taps in three dimensions: ranges of valid planes, rows and
+    # columns (what a weight update pass of a 3-D layer brings)
+    (pa.HALF, dict(batch=2, field=(6, 7, 8), kernel=(3, 3, 4), ci=16, co=24,
+                   pad=1)),
+    (pa.HALF, dict(batch=2, field=(9, 8, 7), kernel=(5, 5, 5), ci=64, co=40,
+                   padLower=(2, 1, 3), padUpper=(1, 2, 2), stride=(1, 2, 1),
+                   kdil=(2, 1, 1))),
 ]
 
 

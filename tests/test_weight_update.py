@@ -176,6 +176,10 @@ WU_GPU_CASES = [
     dict(batch=5, field=(17,), kernel=(3,), ci=8, co=8, groups=2, kdil=2,
          padLower=(2,), padUpper=(1,)),
     dict(batch=16, field=(8, 8), kernel=(3, 3), ci=64, co=64, pad=1),
+    # three field dimensions: the pass's kernel is the layer's output volume
+    dict(batch=8, field=(6, 7, 5), kernel=(3, 3, 3), ci=16, co=24, pad=1),
+    dict(batch=8, field=(6, 8, 8), kernel=(3, 3, 3), ci=8, co=16, pad=1,
+         stride=(1, 2, 2)),
 ]
 
 
