@@ -869,8 +869,11 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
     return hipErrorInvalidValue;
   // outputs mapped into a larger field: plain 2-D convolutions, K not split
   const bool outMapped = d.outFullH != 0 || d.outFullW != 0;
+  const uint32_t fullD = d.outFullD ? d.outFullD : d.outD;
   if (outMapped &&
-      (d.outD != 1 || d.splitK != 1 || d.outStepH == 0 || d.outStepW == 0 ||
+      (d.splitK != 1 || d.outStepH == 0 || d.outStepW == 0 ||
+       d.outStepD == 0 ||
+       (d.outD != 0 && (d.outD - 1) * d.outStepD + d.outOffD >= fullD) ||
        (d.outH != 0 && (d.outH - 1) * d.outStepH + d.outOffH >= d.outFullH) ||
        (d.outW != 0 && (d.outW - 1) * d.outStepW + d.outOffW >= d.outFullW)))
     return hipErrorInvalidValue;
@@ -878,6 +881,7 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
       (!haveWorkspace || (d.groups * d.outChansPerGroup) % 4 != 0))
     return hipErrorInvalidValue;
   a.d = d;
+  a.d.outFullD = fullD;
   a.mode = uint32_t(mode);
   a.outMapped = outMapped ? 1u : 0u;
   if (d.outTransposed && outMapped)

@@ -342,8 +342,11 @@ igemmEpilogue(char *lds, const IgemmArgs &a, floatx16 (&acc)[2][BN / 64],
     size_t pixel = m;
     if (a.outMapped) {
       const uint32_t q = a.divOutW(m), ow = m - q * d.outW;
-      const uint32_t image = a.divOutH(q), oh = q - image * d.outH;
-      pixel = (size_t(image) * d.outFullH + oh * d.outStepH + d.outOffH) *
+      const uint32_t q2 = a.divOutH(q), oh = q - q2 * d.outH;
+      const uint32_t image = a.divOutD(q2), od = q2 - image * d.outD;
+      pixel = ((size_t(image) * d.outFullD + od * d.outStepD + d.outOffD) *
+                   d.outFullH +
+               oh * d.outStepH + d.outOffH) *
                   d.outFullW +
               ow * d.outStepW + d.outOffW;
     }

@@ -125,6 +125,9 @@ hipError_t launchPadChans(const void *src, void *dst, uint64_t pixels,
 struct IgemmTapSelection {
   uint32_t kW;
   uint32_t firstH, stepH, countH, firstW, stepW, countW;
+  // the same along a depth: planes firstD + a * stepD, a < countD, of a
+  // kernel of kH rows per plane (1 plane, unselected, by default)
+  uint32_t kH = 1, firstD = 0, stepD = 1, countD = 1;
 };
 hipError_t launchPackIgemmWeights(const void *src, void *dst, uint32_t groups,
                                   uint32_t co, uint32_t ci, uint32_t taps,
@@ -162,9 +165,11 @@ struct IgemmDesc {
   // with outFullH x outFullW pixels per image (0: the convolution's own
   // field).  That is how one phase of a convolution over a zero-stuffed input
   // - the outputs whose windows meet the same residue of real input rows and
-  // columns - writes its share of the whole output.  No depth with it.
+  // columns - writes its share of the whole output.  The same along the
+  // depth (outFullD 0: the convolution's own).
   uint32_t outFullH = 0, outFullW = 0;
   uint32_t outStepH = 1, outStepW = 1, outOffH = 0, outOffW = 0;
+  uint32_t outFullD = 0, outStepD = 1, outOffD = 0;
   // No tap of the kernel ever reads real input (a phase of a zero-stuffed
   // input that only meets stuffed zeros): the outputs are the bias, or zero,
   // and the workgroups run no k-step at all.

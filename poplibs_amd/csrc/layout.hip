@@ -43,14 +43,17 @@ __global__ __launch_bounds__(256) void packIgemmWeightsKernel(
   const uint64_t g = tid / (uint64_t(kPadded) * coPadded);
   T v = T(0);
   const uint32_t packedTaps =
-      selected ? select.countH * select.countW : taps;
+      selected ? select.countD * select.countH * select.countW : taps;
   if (n < co && k < packedTaps * ciPadded) {
     uint32_t tap = k / ciPadded;
     const uint32_t c = k % ciPadded;
     if (selected) {
-      const uint32_t i = tap / select.countW, j = tap % select.countW;
-      tap = (select.firstH + i * select.stepH) * select.kW + select.firstW +
-            j * select.stepW;
+      const uint32_t j = tap % select.countW, rest = tap / select.countW;
+      const uint32_t i = rest % select.countH, plane = rest / select.countH;
+      tap = ((select.firstD + plane * select.stepD) * select.kH +
+             select.firstH + i * select.stepH) *
+                select.kW +
+            select.firstW + j * select.stepW;
     }
     // source [G][Co][Ci][taps], or [G][Ci][Co][taps] (a matrix
     // multiplication's right-hand side)

@@ -304,9 +304,16 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                      std::size_t(std::abs(s.padW)) >=
                  32768)
       igemmWhyNot = "field too large for 16-bit window origins";
-    else if (s.hasDepth() && (s.inputDilated() || s.outputPadded()))
-      igemmWhyNot = "three field dimensions with a dilated input or a "
-                    "padded output";
+    else if (s.hasDepth() &&
+             (s.outputPadded() ||
+              (s.inputDilated() &&
+               !((s.inDilD == 1 || s.strideD == 1) &&
+                 (s.inDilH == 1 || s.strideH == 1) &&
+                 (s.inDilW == 1 || s.strideW == 1) &&
+                 std::size_t(s.inDilD) * s.inDilH * s.inDilW <=
+                     mxk::kIgemmMaxFused))))
+      igemmWhyNot = "three field dimensions with a padded output or a "
+                    "dilated input that does not come apart into phases";
     else if (s.inputDilated() &&
              (std::size_t(s.inW) * p.getNumInputChans() *
                       params.inputType.size() >=
@@ -456,6 +463,9 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       // padded output field)
       if (s.outputPadded())
         parts = 1;
+      // (three dimensions over a dilated input run as phases only)
+      if (s.hasDepth() && s.inputDilated())
+        parts = 1;
       g.splitK = uint32_t(parts);
       plan.workspaceBytes = mxk::igemmWorkspaceBytes(g);
       if (ciPadded != ci) {
@@ -480,10 +490,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     // Zero-stuffed input, window moving by single pixels: one ordinary
     // convolution per phase instead of arithmetic on every tap - no MACs on
     // the stuffed zeros, and the fast tap-mask addressing.
-    if (s.inputDilated() && !s.hasDepth() && g.splitK == 1 &&
+    if (s.inputDilated() && g.splitK == 1 &&
+        (s.inDilD == 1 || s.strideD == 1) &&
         (s.inDilH == 1 || s.strideH == 1) &&
         (s.inDilW == 1 || s.strideW == 1) &&
-        std::size_t(s.inDilH) * s.inDilW <= mxk::kIgemmMaxFused) {
+        std::size_t(s.inDilD) * s.inDilH * s.inDilW <= mxk::kIgemmMaxFused) {
       // One dimension of one phase.  The window of output o = q * inDil +
       // phase meets real input under kernel tap k when phase - pad + k * dil
       // is a multiple of inDil - taps first, first + step, ... - and reads
@@ -518,16 +529,21 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         return r;
       };
       std::size_t offset = 0;
+      for (uint32_t pd = 0; pd != s.inDilD; ++pd)
       for (uint32_t ph = 0; ph != s.inDilH; ++ph)
         for (uint32_t pw = 0; pw != s.inDilW; ++pw) {
           // a dimension that is not dilated keeps its stride and geometry
+          const Dim dd = s.inDilD == 1
+                             ? Dim{s.outD, 0, 1, s.kD, s.padD, s.dilD, false}
+                             : dimOf(pd, s.inDilD, s.outD, s.kD, s.padD,
+                                     s.dilD);
           const Dim h = s.inDilH == 1
                             ? Dim{s.outH, 0, 1, s.kH, s.padH, s.dilH, false}
                             : dimOf(ph, s.inDilH, s.outH, s.kH, s.padH, s.dilH);
           const Dim w = s.inDilW == 1
                             ? Dim{s.outW, 0, 1, s.kW, s.padW, s.dilW, false}
                             : dimOf(pw, s.inDilW, s.outW, s.kW, s.padW, s.dilW);
-          if (h.out == 0 || w.out == 0)
+          if (dd.out == 0 || h.out == 0 || w.out == 0)
             continue;
           mxconv_plan::IgemmPhase phase;
           mxk::IgemmDesc &q = phase.d;
@@ -535,6 +551,12 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
           q.inDilH = q.inDilW = 1;
           q.outH = h.out, q.outW = w.out, q.kH = h.count, q.kW = w.count;
           q.padH = h.pad, q.padW = w.pad, q.dilH = h.dil, q.dilW = w.dil;
+          q.outD = dd.out, q.kD = dd.count, q.padD = dd.pad, q.dilD = dd.dil;
+          if (s.inDilD != 1)
+            q.strideD = 1;
+          if (dd.dead)
+            q.loD = q.hiD = 0;
+          q.outFullD = s.outD, q.outStepD = s.inDilD, q.outOffD = pd;
           if (s.inDilH != 1)
             q.strideH = 1;
           if (s.inDilW != 1)
@@ -547,12 +569,14 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
           q.outFullW = s.outW + s.outPadLoW + s.outPadHiW;
           q.outStepH = s.inDilH, q.outStepW = s.inDilW;
           q.outOffH = ph + s.outPadLoH, q.outOffW = pw + s.outPadLoW;
-          const bool dead = h.dead || w.dead;
+          const bool dead = dd.dead || h.dead || w.dead;
           q.noTaps = dead ? 1 : 0;
           phase.taps = {s.kW,
                         h.first, h.step, dead ? 0u : h.count,
-                        w.first, w.step, dead ? 0u : w.count};
-          const std::size_t kk = std::size_t(q.kH) * q.kW * ciPadded;
+                        w.first, w.step, dead ? 0u : w.count,
+                        s.kH, dd.first, dd.step, dead ? 0u : dd.count};
+          const std::size_t kk =
+              std::size_t(q.kD) * q.kH * q.kW * ciPadded;
           phase.kPadded = (kk + g.blockK - 1) / g.blockK * g.blockK;
           phase.packedOffset = offset;
           offset += p.numConvGroups * plan.coPadded * phase.kPadded;
@@ -563,7 +587,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       plan.weightPackedElems = offset;
       std::size_t phaseTiles = 0;
       for (const auto &ph : plan.igemmPhases)
-        phaseTiles += (std::size_t(ph.d.batch) * ph.d.outH * ph.d.outW +
+        phaseTiles += (std::size_t(ph.d.batch) * ph.d.outD * ph.d.outH *
+                           ph.d.outW +
                        g.blockM - 1) /
                       g.blockM * (plan.coPadded / g.blockN) * g.groups;
       const uint32_t stages =

@@ -430,9 +430,12 @@ def test_planner_choices():
     many3d = pa.Plan(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 4),
                                  ci=8, co=8)).describe()
     assert "implicit GEMM" in many3d and "ranges of valid kernel" in many3d
+    assert "2 phases" in pa.Plan(make_params(
+        pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3), ci=8, co=8,
+        idil=(1, 2, 1))).describe()
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
-                                  ci=8, co=8, idil=(1, 2, 1))) == \
-        "generic direct"
+                                  ci=8, co=8, idil=(1, 2, 1),
+                                  stride=(1, 2, 1))) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
                                   ci=8, co=8, opu=(0, 1, 0))) == \
         "generic direct"

@@ -664,6 +664,12 @@ PHASE_CASES = [
                     pad=2), 4),
     (pa.QUARTER, dict(batch=2, field=(9, 8), kernel=(3, 3), ci=32, co=16,
                       idil=2, pad=2), 4),
+    # three field dimensions: backward of a 3x3x3 stride-2 layer, and one
+    # that strides in two of the three
+    (pa.HALF, dict(batch=2, field=(4, 5, 6), kernel=(3, 3, 3), ci=16, co=24,
+                   idil=2, padLower=(1, 1, 1), padUpper=(2, 2, 2)), 8),
+    (pa.HALF, dict(batch=2, field=(5, 4, 6), kernel=(2, 3, 3), ci=8, co=40,
+                   idil=(1, 2, 2), stride=(2, 1, 1), pad=1), 4),
 ]
 
 
