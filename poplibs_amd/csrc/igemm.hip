@@ -8,10 +8,12 @@
 //             (zero outside the valid input window: padding is never stored)
 //   B[k][n] = packed weights [g][n][k]  (K contiguous, zero padded)
 // Both operands are therefore contiguous along K in memory, which is how an
-// MFMA lane wants them: 16 bytes = 8 halves (or 16 fp8) of consecutive k.
+// MFMA lane wants them: 16 bytes = 8 halves (16 fp8, 4 floats) of
+// consecutive k.  A field with a depth adds od / kd to pixels and taps in the
+// same way.
 //
 // Workgroup: 512 threads = 8 wave64, tile 128 (M) x BN (N), BN = 64 or 128,
-// K step of 128 bytes per row (64 halves / 128 fp8).
+// K step of 128 bytes per row (64 halves / 128 fp8 / 32 floats).
 //
 // Producer / consumer waves.  Waves 4-7 only move data; waves 0-3 only feed
 // the matrix cores (and run the epilogue); each SIMD holds one of each kind,
@@ -64,6 +66,10 @@
 // Epilogue.  The accumulators are scaled, biased, converted and written to
 // LDS, then all 8 waves copy whole 16-byte vectors to the channels-last
 // output, so that every store instruction covers full rows of the tile.
+// Row m of the GEMM is output pixel m - or, for the caller that runs one
+// convolution per phase of a zero-stuffed input or has a padded output field,
+// every outStep-th pixel of a larger field from an offset; a weight update
+// pass asks for the transposed result, [channel][pixel].
 //
 // This takes the role of PopLibs' AMP vertices ConvPartial1x1Out /
 // ConvPartialnx1 (lib/poplin/codelets/ConvPartial1x1Out.cpp:49-173,

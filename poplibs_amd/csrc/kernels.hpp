@@ -142,8 +142,10 @@ hipError_t launchAddBias(int type, void *acts, const void *bias,
                          uint64_t outerElems, uint64_t channels,
                          hipStream_t stream);
 
-/// Implicit-GEMM forward convolution on the matrix cores (2-D field, stride,
-/// zero padding and kernel dilation only).
+/// Implicit-GEMM forward convolution on the matrix cores: float, half or
+/// quarter operands; a field of up to three dimensions with stride, zero
+/// padding, truncation and kernel dilation; a dilated (zero-stuffed) input in
+/// two dimensions.
 struct IgemmDesc {
   uint32_t batch, groups, inChansPerGroup, outChansPerGroup;
   uint32_t inH, inW, outH, outW, kH, kW;
