@@ -607,7 +607,8 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
             uint32_t(p.outputChannelsPerConvGroup),
             uint32_t(p.inputChannelsPerConvGroup), uint32_t(taps),
             uint32_t(plan->coPadded), uint32_t(plan->kPadded), elemBytes, s,
-            false, uint32_t(plan->paddedInputChans)),
+            false, uint32_t(plan->paddedInputChans),
+            plan->kernelSelected ? &plan->igemmTaps : nullptr),
         "weight packing");
   }
   REQUIRE_ARG(weights_external);
@@ -1182,7 +1183,7 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
       uint32_t(Ci), B,           X * G * B,   G * B};
   const bool direct = plan->kernel == mxconv_plan::Kernel::IGEMM &&
                       !plan->pointwiseOn && !plan->paddedInputChans &&
-                      plan->igemmPhases.empty();
+                      plan->igemmPhases.empty() && !plan->kernelSelected;
   if (direct) {
     // deltas [B][Y][G][Co] -> straight into the matrix-core kernel's packed
     // weights [G][coPadded][kPadded], k = y * B + b; both rearrangements in

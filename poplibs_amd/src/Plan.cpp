@@ -70,6 +70,15 @@ struct Simple2D {
   int32_t padD = 0;
   uint32_t strideD = 1, dilD = 1, loD = 0, hiD = 1, inDilD = 1;
   std::size_t batch = 0; // the batch size times the folded depth
+  // Kernel truncation, padding and flips: the kernel the window applies
+  // (kD, kH, kW) is a selection of the taps of the stored one - tap j of it
+  // is stored tap first + j * step (step 1, or -1 for a flipped dimension) -
+  // and kernel padding only moves the window (folded into pad).  fullK*: the
+  // stored extents.
+  bool kernelSelected = false;
+  uint32_t fullKD = 1, fullKH = 1, fullKW = 1;
+  uint32_t selFirstD = 0, selFirstH = 0, selFirstW = 0;
+  uint32_t selStepD = 1, selStepH = 1, selStepW = 1; // 1 or uint32_t(-1)
   // Zeros around the output field (outH, outW are the convolution's own).
   uint32_t outPadLoH = 0, outPadHiH = 0, outPadLoW = 0, outPadHiW = 0;
   bool outputPadded() const {
@@ -96,9 +105,12 @@ Simple2D asSimple2D(const ConvParams &p) {
       s.why = "input flip";
       return s;
     }
-    if (kt.truncationLower[d] || kt.truncationUpper[d] || kt.paddingLower[d] ||
-        kt.paddingUpper[d] || kt.flip[d]) {
-      s.why = "kernel truncation, padding or flip";
+    const bool kernelTransformed =
+        kt.truncationLower[d] || kt.truncationUpper[d] || kt.paddingLower[d] ||
+        kt.paddingUpper[d] || kt.flip[d];
+    if (kt.truncationLower[d] + kt.truncationUpper[d] >= p.kernelShape[d] &&
+        kernelTransformed) {
+      s.why = "kernel truncated to nothing";
       return s;
     }
     if ((ot.paddingLower[d] || ot.paddingUpper[d]) && n == 3 && d == 0) {
@@ -108,9 +120,15 @@ Simple2D asSimple2D(const ConvParams &p) {
     // conv index = o*stride + outTruncLo; padded input = conv + k*dil;
     // dilated input = padded - padLo; input = dilated / inDil + truncLo when
     // that is whole.
-    const int32_t pad = int32_t(it.paddingLower[d]) -
-                        int32_t(it.truncationLower[d] * it.dilation[d]) -
-                        int32_t(ot.truncationLower[d]);
+    // (kernel padding shifts where the taps sit in the window: the lower
+    // one, or - the flip comes last - the upper one of a flipped kernel)
+    const int32_t pad =
+        int32_t(it.paddingLower[d]) -
+        int32_t(it.truncationLower[d] * it.dilation[d]) -
+        int32_t(ot.truncationLower[d]) -
+        int32_t(kt.flip[d] ? kt.paddingUpper[d] : kt.paddingLower[d]);
+    const uint32_t kept = uint32_t(p.kernelShape[d] - kt.truncationLower[d] -
+                                   kt.truncationUpper[d]);
     const uint32_t lo = it.truncationLower[d];
     const uint32_t hi = uint32_t(p.inputFieldShape[d]) - it.truncationUpper[d];
     // which of depth, height, width: the innermost dimension is the width
@@ -125,7 +143,13 @@ Simple2D asSimple2D(const ConvParams &p) {
       (which == 1 ? s.outPadLoH : s.outPadLoW) = ot.paddingLower[d];
       (which == 1 ? s.outPadHiH : s.outPadHiW) = ot.paddingUpper[d];
     }
-    pick(s.kD, s.kH, s.kW) = uint32_t(p.kernelShape[d]);
+    pick(s.kD, s.kH, s.kW) = kept;
+    pick(s.fullKD, s.fullKH, s.fullKW) = uint32_t(p.kernelShape[d]);
+    pick(s.selFirstD, s.selFirstH, s.selFirstW) =
+        kt.flip[d] ? uint32_t(kt.truncationLower[d]) + kept - 1
+                   : uint32_t(kt.truncationLower[d]);
+    pick(s.selStepD, s.selStepH, s.selStepW) = kt.flip[d] ? ~0u : 1u;
+    s.kernelSelected = s.kernelSelected || kernelTransformed;
     pick(s.padD, s.padH, s.padW) = pad;
     pick(s.strideD, s.strideH, s.strideW) = ot.stride[d];
     pick(s.dilD, s.dilH, s.dilW) = kt.dilation[d];
@@ -230,7 +254,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   // dilation the layer's stride and its stride the layer's kernel dilation.
   {
     const Simple2D w = asSimple2D(p);
-    if (w.ok && !w.hasDepth() && !w.outputPadded() && w.batch == 1 &&
+    if (w.ok && !w.hasDepth() && !w.outputPadded() && !w.kernelSelected &&
+        w.batch == 1 &&
         !plan.zeroConv &&
         !w.inputDilated() && p.batchSize == 1 &&
         p.outputChannelsPerConvGroup == 1 &&
@@ -331,6 +356,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       igemmWhyNot = "tensor too large for 32-bit buffer addressing";
     if (s.hasDepth())
       dwWhyNot = "three field dimensions";
+    else if (s.kernelSelected)
+      dwWhyNot = "kernel truncation, padding or flip";
     else if (s.outputPadded())
       dwWhyNot = "output padding";
     else if (!halfIn)
@@ -410,6 +437,13 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     g.dilH = s.dilH, g.dilW = s.dilW;
     g.loH = s.loH, g.hiH = s.hiH, g.loW = s.loW, g.hiW = s.hiW;
     g.inDilH = s.inDilH, g.inDilW = s.inDilW;
+    if (s.kernelSelected) {
+      plan.kernelSelected = true;
+      plan.igemmTaps = {s.fullKW,
+                        s.selFirstH, s.selStepH, s.kH,
+                        s.selFirstW, s.selStepW, s.kW,
+                        s.fullKH, s.selFirstD, s.selStepD, s.kD};
+    }
     if (s.outputPadded()) {
       // the convolution writes the inside of the padded field; the launch
       // fills the field with zeros (or the bias) first
@@ -571,10 +605,19 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
           q.outOffH = ph + s.outPadLoH, q.outOffW = pw + s.outPadLoW;
           const bool dead = dd.dead || h.dead || w.dead;
           q.noTaps = dead ? 1 : 0;
-          phase.taps = {s.kW,
-                        h.first, h.step, dead ? 0u : h.count,
-                        w.first, w.step, dead ? 0u : w.count,
-                        s.kH, dd.first, dd.step, dead ? 0u : dd.count};
+          // (tap j of the phase is tap first + j * step of the applied
+          // kernel, which is a selection of the stored one itself)
+          phase.taps = {s.fullKW,
+                        s.selFirstH + s.selStepH * h.first,
+                        s.selStepH * h.step,
+                        dead ? 0u : h.count,
+                        s.selFirstW + s.selStepW * w.first,
+                        s.selStepW * w.step,
+                        dead ? 0u : w.count,
+                        s.fullKH,
+                        s.selFirstD + s.selStepD * dd.first,
+                        s.selStepD * dd.step,
+                        dead ? 0u : dd.count};
           const std::size_t kk =
               std::size_t(q.kD) * q.kH * q.kW * ciPadded;
           phase.kPadded = (kk + g.blockK - 1) / g.blockK * g.blockK;
@@ -605,7 +648,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     pw.groups = g.groups, pw.inChansPerGroup = g.inChansPerGroup;
     pw.outChansPerGroup = g.outChansPerGroup;
     const bool unitWindow =
-        !s.hasDepth() && !s.outputPadded() && !s.inputDilated() &&
+        !s.hasDepth() && !s.outputPadded() && !s.kernelSelected &&
+        !s.inputDilated() &&
         g.splitK == 1 && s.kH == 1 &&
         s.kW == 1 &&
         s.strideH == 1 && s.strideW == 1 &&

@@ -61,6 +61,10 @@ struct mxconv_plan {
     std::size_t packedOffset = 0, kPadded = 0;
   };
   std::vector<IgemmPhase> igemmPhases;
+  // The kernel the window applies is a selection of the stored taps (kernel
+  // truncation, flips): what the weight packing picks.
+  bool kernelSelected = false;
+  mxk::IgemmTapSelection igemmTaps{};
   // The output field has zero padding around the convolution's own outputs:
   // the launch fills it with zeros (or the bias) before the kernel writes
   // the inside.

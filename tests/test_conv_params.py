@@ -421,8 +421,10 @@ def test_planner_choices():
     # transforms outside the fast subset fall back
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
                                   co=8, flipIn=True)) == "generic direct"
+    # (a flipped, truncated or padded kernel is the stored one with its taps
+    # picked in another order: the weight packing's business)
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8,
-                                  co=8, flipK=True)) == "generic direct"
+                                  co=8, flipK=True)) == "implicit GEMM"
     # three field dimensions: the matrix cores take undilated inputs; a
     # depth the window does not slide over is batch
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
@@ -464,7 +466,7 @@ def test_planner_choices():
     forced = {"planConstraints": '{"gfx950": {"kernel": "generic"}}'}
     assert _kernel_of(c2, forced) == "generic direct"
     flipped = make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=8, co=8,
-                          flipK=True)
+                          flipIn=True)
     with pytest.raises(MxconvError) as e:
         pa.Plan(flipped, {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'})
     assert e.value.status == Status.INVALID_OPTION

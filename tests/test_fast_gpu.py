@@ -721,6 +721,37 @@ def test_igemm_phases_of_signs_are_exact(oracle):
     _run(oracle, p, 52, 0, "implicit GEMM", dist="pm1")
 
 
+KERNEL_TRANSFORM_CASES = [
+    # flipped in one dimension, in both; with a dilated kernel
+    dict(batch=2, field=(9, 10), kernel=(3, 3), ci=16, co=24, pad=1,
+         flipK=(True, False)),
+    dict(batch=2, field=(9, 10), kernel=(3, 2), ci=64, co=72, pad=1,
+         flipK=True, kdil=(1, 2)),
+    # truncated (taps dropped at either end), truncated and flipped
+    dict(batch=2, field=(12, 11), kernel=(5, 4), ci=8, co=40, pad=2,
+         ktl=(1, 0), ktu=(1, 2)),
+    dict(batch=2, field=(12, 11), kernel=(5, 4), ci=8, co=40, pad=2,
+         ktl=(2, 1), ktu=(0, 1), flipK=(True, True), stride=2),
+    # padded (the window is larger than the taps), padded and flipped
+    dict(batch=2, field=(10, 10), kernel=(3, 3), ci=16, co=16, pad=2,
+         kpl=(1, 0), kpu=(0, 2)),
+    dict(batch=2, field=(10, 10), kernel=(3, 3), ci=16, co=16, pad=2,
+         kpl=(1, 0), kpu=(0, 2), flipK=(True, True), kdil=2, groups=2),
+    # together with a dilated input (phases) and with three dimensions
+    dict(batch=2, field=(7, 8), kernel=(3, 3), ci=16, co=24, idil=2, pad=2,
+         flipK=True, ktu=(1, 0)),
+    dict(batch=2, field=(5, 6, 7), kernel=(3, 3, 3), ci=8, co=16, pad=1,
+         flipK=(True, False, True), ktl=(0, 1, 0)),
+]
+
+
+@pytest.mark.parametrize("kw", KERNEL_TRANSFORM_CASES)
+def test_igemm_kernel_truncation_padding_flip(oracle, kw):
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    print("case", p, flush=True)
+    _run(oracle, p, 71, 1e-3, "implicit GEMM", wscale=0.1)
+
+
 STAGES_CASES = [
     # (params, input type, forced stages or None for the planner's choice)
     (dict(batch=3, field=(9, 11), kernel=(3, 3), ci=128, co=130, pad=1),
