@@ -76,15 +76,17 @@ hipError_t launchSwapBatchChansPair(const SwapBatchChans &first,
 /// Zero-fills `bytes` (a multiple of 4) with a kernel, so that the call can
 /// be recorded into a graph.
 hipError_t launchZero(void *dst, uint64_t bytes, hipStream_t stream);
-/// out[image][fullH][fullW][chans] (kHalf or kFloat): every element outside
-/// rows [offH, offH + insideH) x columns [offW, offW + insideW) becomes
-/// bias[channel], or 0 without a bias; the inside is not touched.
+/// out[image][fullD][fullH][fullW][chans] (kHalf or kFloat): every element
+/// outside planes [offD, offD + insideD) x rows [offH, offH + insideH) x
+/// columns [offW, offW + insideW) becomes bias[channel], or 0 without a bias;
+/// the inside is not touched.
 hipError_t launchFillOutputPadding(int type, void *out, const void *bias,
-                                   uint64_t images, uint32_t fullH,
-                                   uint32_t fullW, uint32_t offH,
-                                   uint32_t offW, uint32_t insideH,
-                                   uint32_t insideW, uint32_t chans,
-                                   hipStream_t stream);
+                                   uint64_t images, uint32_t fullD,
+                                   uint32_t fullH, uint32_t fullW,
+                                   uint32_t offD, uint32_t offH,
+                                   uint32_t offW, uint32_t insideD,
+                                   uint32_t insideH, uint32_t insideW,
+                                   uint32_t chans, hipStream_t stream);
 
 /// biases[c] += scale * sum over rows of zDeltas[row][c] (half or float each),
 /// summed in fp32 in a fixed order: per-split partial sums go to `workspace`

@@ -652,8 +652,9 @@ namespace {
 template <class T>
 __global__ __launch_bounds__(256) void fillOutputPaddingKernel(
     T *__restrict__ out, const T *__restrict__ bias, uint64_t total,
-    uint32_t fullH, uint32_t fullW, uint32_t offH, uint32_t offW,
-    uint32_t insideH, uint32_t insideW, uint32_t chans) {
+    uint32_t fullD, uint32_t fullH, uint32_t fullW, uint32_t offD,
+    uint32_t offH, uint32_t offW, uint32_t insideD, uint32_t insideH,
+    uint32_t insideW, uint32_t chans) {
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
     return;
@@ -661,7 +662,8 @@ __global__ __launch_bounds__(256) void fillOutputPaddingKernel(
   const uint32_t c = uint32_t(tid - pixel * chans);
   const uint32_t w = uint32_t(pixel % fullW);
   const uint32_t h = uint32_t((pixel / fullW) % fullH);
-  if (h - offH < insideH && w - offW < insideW)
+  const uint32_t z = uint32_t((pixel / fullW / fullH) % fullD);
+  if (z - offD < insideD && h - offH < insideH && w - offW < insideW)
     return;
   out[tid] = bias ? bias[c] : T(0);
 }
@@ -674,15 +676,17 @@ namespace {
 template <class T>
 __global__ __launch_bounds__(256) void fillOutputPaddingVectorKernel(
     T *__restrict__ out, const T *__restrict__ bias, uint32_t imageVectors,
-    uint32_t fullW, uint32_t offH, uint32_t offW, uint32_t insideH,
-    uint32_t insideW, uint32_t vecsPerPixel) {
+    uint32_t fullH, uint32_t fullW, uint32_t offD, uint32_t offH,
+    uint32_t offW, uint32_t insideD, uint32_t insideH, uint32_t insideW,
+    uint32_t vecsPerPixel) {
   constexpr uint32_t kVec = 16 / sizeof(T);
   const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= imageVectors)
     return;
   const uint32_t pixel = idx / vecsPerPixel, vec = idx - pixel * vecsPerPixel;
-  const uint32_t h = pixel / fullW, w = pixel - h * fullW;
-  if (h - offH < insideH && w - offW < insideW)
+  const uint32_t row = pixel / fullW, w = pixel - row * fullW;
+  const uint32_t z = row / fullH, h = row - z * fullH;
+  if (z - offD < insideD && h - offH < insideH && w - offW < insideW)
     return;
   const uint64_t image = uint64_t(blockIdx.z) * gridDim.y + blockIdx.y;
   uint4 v{0, 0, 0, 0};
@@ -693,16 +697,18 @@ __global__ __launch_bounds__(256) void fillOutputPaddingVectorKernel(
 } // namespace
 
 hipError_t launchFillOutputPadding(int type, void *out, const void *bias,
-                                   uint64_t images, uint32_t fullH,
-                                   uint32_t fullW, uint32_t offH,
-                                   uint32_t offW, uint32_t insideH,
-                                   uint32_t insideW, uint32_t chans,
-                                   hipStream_t stream) {
-  const uint64_t total = images * fullH * fullW * chans;
+                                   uint64_t images, uint32_t fullD,
+                                   uint32_t fullH, uint32_t fullW,
+                                   uint32_t offD, uint32_t offH,
+                                   uint32_t offW, uint32_t insideD,
+                                   uint32_t insideH, uint32_t insideW,
+                                   uint32_t chans, hipStream_t stream) {
+  const uint64_t total = images * fullD * fullH * fullW * chans;
   if (total == 0)
     return hipSuccess;
   const uint32_t vecElems = type == kHalf ? 8 : 4;
-  const uint64_t imageVectors = uint64_t(fullH) * fullW * (chans / vecElems);
+  const uint64_t imageVectors =
+      uint64_t(fullD) * fullH * fullW * (chans / vecElems);
   if ((type == kHalf || type == kFloat) && chans % vecElems == 0 &&
       imageVectors < (1ull << 31) &&
       (bias == nullptr || reinterpret_cast<uintptr_t>(bias) % 16 == 0) &&
@@ -716,14 +722,14 @@ hipError_t launchFillOutputPadding(int type, void *out, const void *bias,
         hipLaunchKernelGGL(fillOutputPaddingVectorKernel<__half>, grid,
                            dim3(256), 0, stream, static_cast<__half *>(out),
                            static_cast<const __half *>(bias),
-                           uint32_t(imageVectors), fullW, offH, offW, insideH,
-                           insideW, chans / vecElems);
+                           uint32_t(imageVectors), fullH, fullW, offD, offH,
+                           offW, insideD, insideH, insideW, chans / vecElems);
       else
         hipLaunchKernelGGL(fillOutputPaddingVectorKernel<float>, grid,
                            dim3(256), 0, stream, static_cast<float *>(out),
                            static_cast<const float *>(bias),
-                           uint32_t(imageVectors), fullW, offH, offW, insideH,
-                           insideW, chans / vecElems);
+                           uint32_t(imageVectors), fullH, fullW, offD, offH,
+                           offW, insideD, insideH, insideW, chans / vecElems);
       return hipGetLastError();
     }
   }
@@ -733,13 +739,15 @@ hipError_t launchFillOutputPadding(int type, void *out, const void *bias,
   if (type == kHalf)
     hipLaunchKernelGGL(fillOutputPaddingKernel<__half>, dim3(uint32_t(blocks)),
                        dim3(256), 0, stream, static_cast<__half *>(out),
-                       static_cast<const __half *>(bias), total, fullH, fullW,
-                       offH, offW, insideH, insideW, chans);
+                       static_cast<const __half *>(bias), total, fullD, fullH,
+                       fullW, offD, offH, offW, insideD, insideH, insideW,
+                       chans);
   else if (type == kFloat)
     hipLaunchKernelGGL(fillOutputPaddingKernel<float>, dim3(uint32_t(blocks)),
                        dim3(256), 0, stream, static_cast<float *>(out),
-                       static_cast<const float *>(bias), total, fullH, fullW,
-                       offH, offW, insideH, insideW, chans);
+                       static_cast<const float *>(bias), total, fullD, fullH,
+                       fullW, offD, offH, offW, insideD, insideH, insideW,
+                       chans);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

@@ -140,14 +140,17 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
     if (plan->outputPadded) {
       // zeros (the bias) around the convolution's own outputs
       const mxk::IgemmDesc &g = plan->igemm;
-      const uint32_t insideH = g.outFullH - plan->outputPadLoH -
+      const uint32_t fullD = g.outFullD ? g.outFullD : g.outD;
+      const uint32_t insideD = fullD - plan->outputPadLoD - plan->outputPadHiD,
+                     insideH = g.outFullH - plan->outputPadLoH -
                                plan->outputPadHiH,
                      insideW = g.outFullW - plan->outputPadLoW -
                                plan->outputPadHiW;
       const mxconv_status st = hipStatus(
           mxk::launchFillOutputPadding(
-              outType, out, bias, g.batch, g.outFullH, g.outFullW,
-              plan->outputPadLoH, plan->outputPadLoW, insideH, insideW,
+              outType, out, bias, g.batch, fullD, g.outFullH, g.outFullW,
+              plan->outputPadLoD, plan->outputPadLoH, plan->outputPadLoW,
+              insideD, insideH, insideW,
               uint32_t(plan->params.getNumOutputChans()), s),
           "output padding fill");
       if (st != MXCONV_OK)

@@ -81,8 +81,10 @@ struct Simple2D {
   uint32_t selStepD = 1, selStepH = 1, selStepW = 1; // 1 or uint32_t(-1)
   // Zeros around the output field (outH, outW are the convolution's own).
   uint32_t outPadLoH = 0, outPadHiH = 0, outPadLoW = 0, outPadHiW = 0;
+  uint32_t outPadLoD = 0, outPadHiD = 0;
   bool outputPadded() const {
-    return outPadLoH || outPadHiH || outPadLoW || outPadHiW;
+    return outPadLoH || outPadHiH || outPadLoW || outPadHiW || outPadLoD ||
+           outPadHiD;
   }
   bool hasDepth() const { return inD != 1 || outD != 1 || kD != 1; }
   bool inputDilated() const {
@@ -113,10 +115,6 @@ Simple2D asSimple2D(const ConvParams &p) {
       s.why = "kernel truncated to nothing";
       return s;
     }
-    if ((ot.paddingLower[d] || ot.paddingUpper[d]) && n == 3 && d == 0) {
-      s.why = "output padding in the depth dimension";
-      return s;
-    }
     // conv index = o*stride + outTruncLo; padded input = conv + k*dil;
     // dilated input = padded - padLo; input = dilated / inDil + truncLo when
     // that is whole.
@@ -139,10 +137,8 @@ Simple2D asSimple2D(const ConvParams &p) {
     pick(s.inD, s.inH, s.inW) = uint32_t(p.inputFieldShape[d]);
     pick(s.outD, s.outH, s.outW) = uint32_t(
         p.getOutputSize(d) - ot.paddingLower[d] - ot.paddingUpper[d]);
-    if (which != 0) {
-      (which == 1 ? s.outPadLoH : s.outPadLoW) = ot.paddingLower[d];
-      (which == 1 ? s.outPadHiH : s.outPadHiW) = ot.paddingUpper[d];
-    }
+    pick(s.outPadLoD, s.outPadLoH, s.outPadLoW) = ot.paddingLower[d];
+    pick(s.outPadHiD, s.outPadHiH, s.outPadHiW) = ot.paddingUpper[d];
     pick(s.kD, s.kH, s.kW) = kept;
     pick(s.fullKD, s.fullKH, s.fullKW) = uint32_t(p.kernelShape[d]);
     pick(s.selFirstD, s.selFirstH, s.selFirstW) =
@@ -158,7 +154,8 @@ Simple2D asSimple2D(const ConvParams &p) {
     pick(s.inDilD, s.inDilH, s.inDilW) = it.dilation[d];
   }
   if (s.kD == 1 && s.strideD == 1 && s.padD == 0 && s.loD == 0 &&
-      s.hiD == s.inD && s.inDilD == 1 && s.outD == s.inD) {
+      s.hiD == s.inD && s.inDilD == 1 && s.outD == s.inD &&
+      s.outPadLoD == 0 && s.outPadHiD == 0) {
     s.batch *= s.inD;
     s.inD = s.outD = s.hiD = 1;
   }
@@ -330,15 +327,14 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                  32768)
       igemmWhyNot = "field too large for 16-bit window origins";
     else if (s.hasDepth() &&
-             (s.outputPadded() ||
-              (s.inputDilated() &&
+             ((s.inputDilated() &&
                !((s.inDilD == 1 || s.strideD == 1) &&
                  (s.inDilH == 1 || s.strideH == 1) &&
                  (s.inDilW == 1 || s.strideW == 1) &&
                  std::size_t(s.inDilD) * s.inDilH * s.inDilW <=
                      mxk::kIgemmMaxFused))))
-      igemmWhyNot = "three field dimensions with a padded output or a "
-                    "dilated input that does not come apart into phases";
+      igemmWhyNot = "three field dimensions with a dilated input that does "
+                    "not come apart into phases";
     else if (s.inputDilated() &&
              (std::size_t(s.inW) * p.getNumInputChans() *
                       params.inputType.size() >=
@@ -449,10 +445,13 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       // fills the field with zeros (or the bias) first
       g.outFullH = s.outH + s.outPadLoH + s.outPadHiH;
       g.outFullW = s.outW + s.outPadLoW + s.outPadHiW;
+      g.outFullD = s.outD + s.outPadLoD + s.outPadHiD;
       g.outOffH = s.outPadLoH, g.outOffW = s.outPadLoW;
+      g.outOffD = s.outPadLoD;
       plan.outputPadded = true;
       plan.outputPadLoH = s.outPadLoH, plan.outputPadHiH = s.outPadHiH;
       plan.outputPadLoW = s.outPadLoW, plan.outputPadHiW = s.outPadHiW;
+      plan.outputPadLoD = s.outPadLoD, plan.outputPadHiD = s.outPadHiD;
     }
     // Tile shape.  M = batch * outH * outW pixels, N = out channels of one
     // group, K = kH * kW * in channels.  A 128-pixel tile keeps the A
@@ -590,7 +589,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
             q.strideD = 1;
           if (dd.dead)
             q.loD = q.hiD = 0;
-          q.outFullD = s.outD, q.outStepD = s.inDilD, q.outOffD = pd;
+          q.outFullD = s.outD + s.outPadLoD + s.outPadHiD;
+          q.outStepD = s.inDilD, q.outOffD = pd + s.outPadLoD;
           if (s.inDilH != 1)
             q.strideH = 1;
           if (s.inDilW != 1)

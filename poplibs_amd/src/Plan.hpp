@@ -70,7 +70,7 @@ struct mxconv_plan {
   // the inside.
   bool outputPadded = false;
   uint32_t outputPadLoH = 0, outputPadHiH = 0, outputPadLoW = 0,
-           outputPadHiW = 0;
+           outputPadHiW = 0, outputPadLoD = 0, outputPadHiD = 0;
 
   // Input channels per group as the matrix-core kernel sees them, when that
   // is more than the parameters say (0 otherwise): the channels are padded

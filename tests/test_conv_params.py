@@ -440,7 +440,7 @@ def test_planner_choices():
                                   stride=(1, 2, 1))) == "generic direct"
     assert _kernel_of(make_params(pa.HALF, field=(8, 8, 8), kernel=(3, 3, 3),
                                   ci=8, co=8, opu=(0, 1, 0))) == \
-        "generic direct"
+        "implicit GEMM"
     folded = pa.Plan(make_params(pa.HALF, batch=2, field=(5, 9, 9),
                                  kernel=(1, 7, 7), ci=8, co=8))
     assert "gemm M x N x K             90 x 8 x 392" in folded.describe()

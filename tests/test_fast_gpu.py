@@ -704,6 +704,12 @@ OUTPUT_PADDING_CASES = [
          opu=(1, 1)),
     dict(batch=2, field=(6, 7), kernel=(3, 3), ci=16, co=16, idil=2, pad=2,
          opl=(1, 1), opu=(0, 2)),
+    # three field dimensions, padded in all of them; the backward pass of a
+    # strided 1x1x1 layer on an even volume
+    dict(batch=2, field=(4, 5, 6), kernel=(3, 3, 3), ci=8, co=16, pad=1,
+         opl=(1, 0, 2), opu=(0, 1, 1)),
+    dict(batch=2, field=(3, 3, 3), kernel=(1, 1, 1), ci=64, co=32, idil=2,
+         opu=(1, 1, 1)),
 ]
 
 
