@@ -257,25 +257,12 @@ class TrainingRunner:
             self.result.data_ptr(), self.ws.data_ptr(), self.ws_bytes, s)
 
 
-def parity(runner, images, tol):
-    import oracle
-    runner.launch(0)
-    got = runner.output_external(0)
-    acts, weights = runner.oracle_inputs(images)
-    one = runner.pa.ConvParams.from_c(runner.p.to_c())
-    one.batchSize = len(images)
-    want = oracle.convolution(one, acts, weights, threads=os.cpu_count() or 1)
-    err = (np.linalg.norm((got[images] - want).ravel())
-           / np.linalg.norm(want.ravel()))
-    if not err <= tol:
-        raise SystemExit(f"parity check failed: rel-L2 {err} > {tol}")
-    return float(err)
-
-
-def cpu_baseline(runner, budget_s=12.0):
+def cpu_baseline(runner, tol, budget_s=12.0):
     """Times the single-threaded CPU oracle (a port of the reference's
     poplibs_test::conv::convolution) on a bounded sample of the same
-    workload: the first n images of the batch."""
+    workload: the first n images of the batch.  The sample's result also
+    checks the GPU's output for those images; this is the only place where
+    this program runs the oracle."""
     import oracle
     p = runner.p
     one = runner.pa.ConvParams.from_c(p.to_c())
@@ -288,13 +275,25 @@ def cpu_baseline(runner, budget_s=12.0):
     sample = runner.pa.ConvParams.from_c(p.to_c())
     sample.batchSize = n
     acts, weights = runner.oracle_inputs(list(range(n)))
+    # A workload the oracle finishes early is repeated, so that the figure
+    # rests on about budget_s of CPU work either way.
+    reps = int(min(16, max(1, round(budget_s / max(t1 * n, 1e-3))))) \
+        if n == p.batchSize else 1
     t0 = time.perf_counter()
-    oracle.convolution(sample, acts, weights, threads=1)
-    t = time.perf_counter() - t0
+    for _ in range(reps):
+        want = oracle.convolution(sample, acts, weights, threads=1)
+    t = (time.perf_counter() - t0) / reps
+    runner.launch(0)
+    got = runner.output_external(0)[:n]
+    err = float(np.linalg.norm((got - want).ravel())
+                / np.linalg.norm(want.ravel()))
+    if not err <= tol:
+        raise SystemExit(f"parity check failed: rel-L2 {err} > {tol}")
     return {"value": round(sample.getFwdFlops() / t / 1e12, 6),
             "unit": "TFLOP/s", "cores": 1, "kind": "port",
             "sample": f"first {n} of {p.batchSize} images of the same "
-                      f"workload, {t:.2f} s, double precision, 1 thread"}
+                      f"workload, {reps} x {t:.2f} s, double precision, 1 thread",
+            "gpu_rel_l2_vs_sample": err, "tolerance": tol}
 
 
 def measured_traffic(key):
@@ -348,8 +347,6 @@ def main():
         if wl["bound"] == "hbm":
             sets = max(1, -(-300 * 2 ** 20 // probe.bytes))
         runner = probe if sets == 1 else Runner(pa, capi, torch, wl, sets=sets)
-        tol = 3e-2 if wl["dtype"] == "fp8" else 1e-3
-        err = parity(runner, [0, wl["params"].batchSize - 1], tol)
         wall, kernel, mode = time_steps(torch, runner, steps, warmup)
         if wl["bound"] == "mfma":
             achieved = runner.flops / kernel / 1e12
@@ -358,7 +355,7 @@ def main():
             achieved = runner.bytes / kernel / 1e9
             peak, unit = PEAK_HBM_GBS, "GB/s"
         return dict(
-            runner=runner, wall=wall, kernel=kernel, mode=mode, err=err,
+            runner=runner, wall=wall, kernel=kernel, mode=mode,
             sets=sets,
             roofline={"bound": wl["bound"], "achieved": round(achieved, 3),
                       "peak": peak, "unit": unit,
@@ -382,8 +379,7 @@ def main():
         "dtype": wl["dtype"], "data": "synthetic",
         "config": {"workload": wl["name"], "flops_per_step": runner.flops,
                    "bytes_per_step": runner.bytes,
-                   "issue": head["mode"], "buffer_sets": head["sets"],
-                   "parity_rel_l2_vs_oracle": head["err"]},
+                   "issue": head["mode"], "buffer_sets": head["sets"]},
         "roofline": head["roofline"],
     }
     if not args.only:
@@ -400,7 +396,6 @@ def main():
                 "gbytes_per_s": round(r.bytes * args.steps / m["wall"] / 1e9,
                                       1),
                 "buffer_sets": m["sets"],
-                "parity_rel_l2_vs_oracle": m["err"],
                 "roofline": m["roofline"]}
             del m, r
             torch.cuda.empty_cache()
@@ -423,7 +418,8 @@ def main():
                 del r
                 torch.cuda.empty_cache()
         line["training_passes"] = passes
-        line["cpu_baseline"] = cpu_baseline(runner)
+        line["cpu_baseline"] = cpu_baseline(
+            runner, 3e-2 if wl["dtype"] == "fp8" else 1e-3)
     print(json.dumps(line), flush=True)
 
 
