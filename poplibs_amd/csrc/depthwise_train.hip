@@ -122,6 +122,137 @@ __global__ __launch_bounds__(256) void depthwiseDirectKernel(
   store8(out + size_t(pixel) * d.channels + c, acc);
 }
 
+struct BlockArgs {
+  DepthwiseDesc d;
+  FastDiv divVecs, divBlocksW, divStrips;
+  uint32_t vecs, blocksW, strips;
+  int32_t firstBlockH, firstBlockW;
+  uint64_t items; // batch * strips * blocksW * vecs
+};
+
+/// The same convolution for an input dilated by S in both dimensions with
+/// unit stride and unit kernel dilation (the backward pass of a layer of
+/// stride S), K x K taps.  With oh - padH = S q + r (0 <= r < S) the taps
+/// that read an input element are those with (r + kh) % S == 0, and they read
+/// row q + (r + kh) / S: the same for every output of phase r.  So a thread
+/// takes S x S blocks of outputs (one output of every phase), R blocks below
+/// each other, for one vector of 8 channels: it loads the (R + ND - 1) x ND
+/// input vectors they need (ND = (K + S - 2) / S + 1) and all K x K taps
+/// once, and every output then takes exactly its own taps - no tests, no
+/// divergence between neighbouring outputs, each input vector loaded once per
+/// thread.
+template <int S, int K, int R, class OutT>
+__global__ __launch_bounds__(256) void depthwiseDilatedBlockKernel(
+    BlockArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
+    const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  const DepthwiseDesc &d = a.d;
+  const uint64_t item = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (item >= a.items)
+    return;
+  // item = ((b * strips + strip) * blocksW + block column) * vecs + v
+  const uint32_t col = a.divVecs(uint32_t(item));
+  const uint32_t v = uint32_t(item) - col * a.vecs;
+  const uint32_t t = a.divBlocksW(col);
+  const uint32_t bw = col - t * a.blocksW;
+  const uint32_t b = a.divStrips(t);
+  const uint32_t strip = t - b * a.strips;
+  const int qw = a.firstBlockW + int(bw);
+  const int qh0 = a.firstBlockH + int(strip) * R;
+  const uint32_t c = v * 8;
+  constexpr int ND = (K + S - 2) / S + 1;
+  constexpr int ROWS = R + ND - 1;
+
+  const __half *image = in + size_t(b) * d.inH * d.inW * d.channels + c;
+  Vec8 x[ROWS][ND];
+#pragma unroll
+  for (int i = 0; i != ROWS; ++i)
+#pragma unroll
+    for (int j = 0; j != ND; ++j) {
+      const int ih = qh0 + i, iw = qw + j;
+      x[i][j].raw = uint4{0, 0, 0, 0};
+      if (ih >= int(d.loH) && ih < int(d.hiH) && iw >= int(d.loW) &&
+          iw < int(d.hiW))
+        x[i][j].raw = *reinterpret_cast<const uint4 *>(
+            image + (size_t(ih) * d.inW + size_t(iw)) * d.channels);
+    }
+  Vec8 k[K * K];
+#pragma unroll
+  for (int tap = 0; tap != K * K; ++tap)
+    k[tap].raw =
+        *reinterpret_cast<const uint4 *>(w + size_t(tap) * d.channels + c);
+  float biasV[8];
+#pragma unroll
+  for (int i = 0; i != 8; ++i)
+    biasV[i] = bias ? Load<OutT>::at(bias, c + i, 0) : 0.0f;
+
+  OutT *outImage = out + size_t(b) * d.outH * d.outW * d.channels + c;
+#pragma unroll
+  for (int i = 0; i != R; ++i)
+#pragma unroll
+    for (int rh = 0; rh != S; ++rh) {
+      const int oh = S * (qh0 + i) + rh + d.padH;
+      if (oh < 0 || oh >= int(d.outH))
+        continue;
+#pragma unroll
+      for (int rw = 0; rw != S; ++rw) {
+        const int ow = S * qw + rw + d.padW;
+        if (ow < 0 || ow >= int(d.outW))
+          continue;
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e != 8; ++e)
+          acc[e] = biasV[e];
+#pragma unroll
+        for (int kh = 0; kh != K; ++kh)
+#pragma unroll
+          for (int kw = 0; kw != K; ++kw)
+            if ((rh + kh) % S == 0 && (rw + kw) % S == 0)
+              fma8(acc, x[i + (rh + kh) / S][(rw + kw) / S], k[kh * K + kw]);
+        store8(outImage + (size_t(oh) * d.outW + size_t(ow)) * d.channels,
+               acc);
+      }
+    }
+}
+
+inline int floorDiv(int n, int d) { return n >= 0 ? n / d : -((-n + d - 1) / d); }
+
+/// Launches depthwiseDilatedBlockKernel<S, K, R> on a shape it is built for.
+template <int S, int K, int R>
+hipError_t launchDilatedBlock(const DepthwiseDesc &d, int outType,
+                              const void *in, const void *w, const void *bias,
+                              void *out, hipStream_t stream) {
+  BlockArgs a;
+  a.d = d;
+  a.vecs = d.channels / 8;
+  a.firstBlockH = floorDiv(-d.padH, S);
+  a.firstBlockW = floorDiv(-d.padW, S);
+  const uint32_t blocksH =
+      uint32_t(floorDiv(int(d.outH) - 1 - d.padH, S) - a.firstBlockH + 1);
+  a.blocksW =
+      uint32_t(floorDiv(int(d.outW) - 1 - d.padW, S) - a.firstBlockW + 1);
+  a.strips = (blocksH + R - 1) / R;
+  a.items = uint64_t(d.batch) * a.strips * a.blocksW * a.vecs;
+  if (a.items >= (1ull << 31))
+    return hipErrorInvalidConfiguration;
+  a.divVecs = makeFastDiv(a.vecs);
+  a.divBlocksW = makeFastDiv(a.blocksW);
+  a.divStrips = makeFastDiv(a.strips);
+  const dim3 grid{uint32_t((a.items + 255) / 256)}, block{256};
+  if (outType == kHalf)
+    hipLaunchKernelGGL((depthwiseDilatedBlockKernel<S, K, R, __half>), grid,
+                       block, 0, stream, a, static_cast<const __half *>(in),
+                       static_cast<const __half *>(w),
+                       static_cast<const __half *>(bias),
+                       static_cast<__half *>(out));
+  else
+    hipLaunchKernelGGL((depthwiseDilatedBlockKernel<S, K, R, float>), grid,
+                       block, 0, stream, a, static_cast<const __half *>(in),
+                       static_cast<const __half *>(w),
+                       static_cast<const float *>(bias),
+                       static_cast<float *>(out));
+  return hipGetLastError();
+}
+
 struct DeltaArgs {
   DepthwiseDesc d;     // the FORWARD convolution
   FastDiv divVecs, divOutW, divOutH;
@@ -273,6 +404,13 @@ uint32_t deltaSlices(const DepthwiseDesc &d) {
 
 } // namespace
 
+bool depthwiseDirectInBlocks(const DepthwiseDesc &d) {
+  return d.inDilH == 2 && d.inDilW == 2 && d.strideH == 1 && d.strideW == 1 &&
+         d.dilH == 1 && d.dilW == 1 && d.kH == d.kW &&
+         (d.kH == 3 || d.kH == 5) && d.outH < (1u << 30) &&
+         d.outW < (1u << 30);
+}
+
 hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
                                  int outType, const void *in,
                                  const void *weightsPacked, const void *bias,
@@ -288,6 +426,14 @@ hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
   // item numbers are divided with 31-bit arithmetic
   if (a.items >= (1ull << 31))
     return hipErrorInvalidConfiguration;
+  if ((outType == kHalf || outType == kFloat) && depthwiseDirectInBlocks(d)) {
+    if (d.kH == 3)
+      return launchDilatedBlock<2, 3, 4>(d, outType, in, weightsPacked, bias,
+                                         out, stream);
+    if (d.kH == 5)
+      return launchDilatedBlock<2, 5, 2>(d, outType, in, weightsPacked, bias,
+                                         out, stream);
+  }
   a.divVecs = makeFastDiv(a.vecs);
   a.divOutW = makeFastDiv(d.outW);
   a.divOutH = makeFastDiv(d.outH);

@@ -277,6 +277,11 @@ hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
                                  int outType, const void *in,
                                  const void *weightsPacked, const void *bias,
                                  void *out, hipStream_t stream);
+/// True when launchDepthwiseDirect serves `d` with its kernel of one thread
+/// per block of outputs (input dilated by 2 in both dimensions, unit stride
+/// and kernel dilation, 3x3 or 5x5 taps: the backward pass of a stride-2
+/// layer), which loads every input vector and tap once per thread.
+bool depthwiseDirectInBlocks(const DepthwiseDesc &d);
 /// Gradient with respect to the weights of the depthwise FORWARD convolution
 /// `d` (undilated input): weightDeltas [channels][kH * kW] in outType from
 /// acts [batch][inH][inW][channels] and deltas [batch][outH][outW][channels],

@@ -720,7 +720,10 @@ std::string mxconv_plan::describe() const {
        << (pointwiseOn ? ", pointwise streaming variant" : "");
     break;
   case Kernel::DEPTHWISE:
-    os << (depthwise.inDilH != 1 || depthwise.inDilW != 1
+    os << (mxk::depthwiseDirectInBlocks(depthwise)
+               ? "depthwise direct (vector ALU, one thread per 2x2 block of "
+                 "outputs, dilated input)"
+           : depthwise.inDilH != 1 || depthwise.inDilW != 1
                ? "depthwise direct (vector ALU, one thread per output "
                  "vector, dilated input)"
            : depthwise.dense3x3

@@ -147,6 +147,19 @@ BWD_GPU_CASES = [
      "dilated input"),
     (dict(batch=2, field=(17,), kernel=(5,), groups=8, stride=3, pad=2),
      "dilated input"),
+    # ... stride 2 with 3x3 or 5x5 taps: a thread per 2x2 block of outputs.
+    # No padding, even and odd fields, a channel count that is no power of
+    # two, asymmetric padding, more rows than one thread's strip, 5x5
+    (dict(batch=2, field=(13, 11), kernel=(3, 3), groups=8, stride=2),
+     "dilated input"),
+    (dict(batch=3, field=(14, 14), kernel=(3, 3), groups=40, stride=2, pad=1),
+     "dilated input"),
+    (dict(batch=1, field=(37, 12), kernel=(3, 3), groups=16, stride=2,
+          padLower=(0, 1), padUpper=(1, 0)), "dilated input"),
+    (dict(batch=2, field=(15, 14), kernel=(5, 5), groups=16, stride=2, pad=2),
+     "dilated input"),
+    (dict(batch=1, field=(10, 21), kernel=(5, 5), groups=8, stride=2,
+          padLower=(1, 2), padUpper=(2, 0)), "dilated input"),
     # depthwise 3x3 stride 1 stays depthwise
     (dict(batch=2, field=(12, 13), kernel=(3, 3), groups=16, pad=1),
      "depthwise direct"),
