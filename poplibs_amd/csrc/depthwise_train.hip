@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256) void depthwiseWeightDeltaKernel(
 
 /// out[c][tap] = sum over slices of partial[slice][tap][c], in a fixed order:
 /// a workgroup of 16 waves takes 64 outputs; each wave adds up a contiguous
-/// sixteenth of the slices (four loads in flight per lane), then one thread
+/// sixteenth of the slices (sixteen loads in flight per lane), then one thread
 /// per output adds the sixteen sums in order.
 template <class OutT>
 __global__ __launch_bounds__(1024) void depthwiseDeltaSumKernel(
@@ -360,17 +360,25 @@ __global__ __launch_bounds__(1024) void depthwiseDeltaSumKernel(
   const uint32_t i = blockIdx.x * 64 + lane; // tap * C + c
   const uint32_t per = (slices + 15) / 16;
   const uint32_t from = min(wave * per, slices), to = min(from + per, slices);
-  float sum[4] = {};
+  // Sixteen loads in flight per lane: the walk is a chain of memory
+  // latencies, and there are only a few workgroups of it.
+  constexpr int kInFlight = 16;
+  float sum[kInFlight] = {};
   if (i < outputs) {
     uint32_t s = from;
-    for (; s + 4 <= to; s += 4)
+    for (; s + kInFlight <= to; s += kInFlight)
 #pragma unroll
-      for (int u = 0; u != 4; ++u)
+      for (int u = 0; u != kInFlight; ++u)
         sum[u] += partial[size_t(s + u) * outputs + i];
     for (; s != to; ++s)
       sum[0] += partial[size_t(s) * outputs + i];
   }
-  meet[wave][lane] = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+#pragma unroll
+  for (int width = kInFlight / 2; width != 0; width /= 2)
+#pragma unroll
+    for (int u = 0; u != width; ++u)
+      sum[u] += sum[u + width];
+  meet[wave][lane] = sum[0];
   __syncthreads();
   if (wave != 0 || i >= outputs)
     return;
