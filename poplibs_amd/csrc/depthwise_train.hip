@@ -347,21 +347,23 @@ __global__ __launch_bounds__(256) void depthwiseWeightDeltaKernel(
 }
 
 /// out[c][tap] = sum over slices of partial[slice][tap][c], in a fixed order:
-/// a workgroup of 16 waves takes 64 outputs; each wave adds up a contiguous
-/// sixteenth of the slices (sixteen loads in flight per lane), then one thread
-/// per output adds the sixteen sums in order.
+/// a workgroup of 16 waves takes 16 outputs and cuts the slices into 64
+/// contiguous parts, a quarter of a wave (16 lanes, 64 contiguous bytes per
+/// slice) to each; a lane adds up its part with sixteen loads in flight, then
+/// one thread per output adds the 64 sums in order.  Few outputs per
+/// workgroup, because the outputs are few (taps x channels) and the walk over
+/// the slices is a chain of memory latencies: this way there are four times
+/// the workgroups and a quarter of the chain.
 template <class OutT>
 __global__ __launch_bounds__(1024) void depthwiseDeltaSumKernel(
     const float *__restrict__ partial, uint32_t slices, uint32_t taps,
     uint32_t channels, OutT *__restrict__ out) {
-  __shared__ float meet[16][64];
-  const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  __shared__ float meet[64][16];
+  const uint32_t column = threadIdx.x % 16, part = threadIdx.x / 16;
   const uint32_t outputs = taps * channels;
-  const uint32_t i = blockIdx.x * 64 + lane; // tap * C + c
-  const uint32_t per = (slices + 15) / 16;
-  const uint32_t from = min(wave * per, slices), to = min(from + per, slices);
-  // Sixteen loads in flight per lane: the walk is a chain of memory
-  // latencies, and there are only a few workgroups of it.
+  const uint32_t i = blockIdx.x * 16 + column; // tap * C + c
+  const uint32_t per = (slices + 63) / 64;
+  const uint32_t from = min(part * per, slices), to = min(from + per, slices);
   constexpr int kInFlight = 16;
   float sum[kInFlight] = {};
   if (i < outputs) {
@@ -370,21 +372,23 @@ __global__ __launch_bounds__(1024) void depthwiseDeltaSumKernel(
 #pragma unroll
       for (int u = 0; u != kInFlight; ++u)
         sum[u] += partial[size_t(s + u) * outputs + i];
-    for (; s != to; ++s)
-      sum[0] += partial[size_t(s) * outputs + i];
+#pragma unroll
+    for (int u = 0; u != kInFlight - 1; ++u)
+      if (s + u < to)
+        sum[u] += partial[size_t(s + u) * outputs + i];
   }
 #pragma unroll
   for (int width = kInFlight / 2; width != 0; width /= 2)
 #pragma unroll
     for (int u = 0; u != width; ++u)
       sum[u] += sum[u + width];
-  meet[wave][lane] = sum[0];
+  meet[part][column] = sum[0];
   __syncthreads();
-  if (wave != 0 || i >= outputs)
+  if (part != 0 || i >= outputs)
     return;
-  float total = meet[0][lane];
-  for (int w = 1; w != 16; ++w)
-    total += meet[w][lane];
+  float total = meet[0][column];
+  for (int w = 1; w != 64; ++w)
+    total += meet[w][column];
   const uint32_t tap = i / channels, c = i - tap * channels;
   storeOut(out, size_t(c) * taps + tap, total);
 }
@@ -502,7 +506,7 @@ hipError_t launchDepthwiseWeightDeltas(const DepthwiseDesc &d, int outType,
                      static_cast<const __half *>(acts),
                      static_cast<const __half *>(deltas), partial);
   const uint32_t outputs = a.taps * d.channels;
-  const dim3 grid2{(outputs + 63) / 64};
+  const dim3 grid2{(outputs + 15) / 16};
   const dim3 block2{1024};
   if (outType == kHalf)
     hipLaunchKernelGGL(depthwiseDeltaSumKernel<__half>, grid2, block2, 0, stream,
