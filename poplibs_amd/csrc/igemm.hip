@@ -238,6 +238,16 @@ __device__ __forceinline__ void igemmTile(
           ciOff = aByte - tap * ciBytes;
           kh = a.divKW(tap); // (no depth with a dilated input)
           kw = tap - kh * d.kW;
+        } else if constexpr (!UNI) {
+          // Per thread, so a loop would diverge; straight-line code instead,
+          // as above, with the depth
+          aByte += kRowBytes;
+          tap = a.divCiBytes(aByte);
+          ciOff = aByte - tap * ciBytes;
+          kRow = a.divKW(tap);
+          kw = tap - kRow * d.kW;
+          kd = a.divKH(kRow);
+          kh = kRow - kd * d.kH;
         } else {
           ciOff += kRowBytes;
           while (ciOff >= ciBytes) {
