@@ -160,6 +160,9 @@ BWD_GPU_CASES = [
      "dilated input"),
     (dict(batch=1, field=(10, 21), kernel=(5, 5), groups=8, stride=2,
           padLower=(1, 2), padUpper=(2, 0)), "dilated input"),
+    # ... the forward output was padded: those deltas are cut off again
+    (dict(batch=2, field=(13, 12), kernel=(3, 3), groups=16, stride=2, pad=1,
+          opl=(1, 0), opu=(0, 2)), "dilated input"),
     # depthwise 3x3 stride 1 stays depthwise
     (dict(batch=2, field=(12, 13), kernel=(3, 3), groups=16, pad=1),
      "depthwise direct"),
