@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0                            # MI355X HBM3E
 
 
 def _workloads(pa):
-    """The BASELINE configurations 2-5 as ConvParams + data recipe."""
+    """The benchmark configurations 2-5 as ConvParams + data recipe."""
     def params(t_in, t_out, batch, field, kernel, ci, co, groups, stride, pad):
         p = pa.ConvParams(t_in, t_out, batch, list(field), list(kernel), ci,
                           co, groups)

@@ -3,7 +3,7 @@ the CPU oracle, through the C ABI.
 
 Tolerances (relative L2 error against the double-precision oracle fed the same
 rounded inputs): fp16 in / fp32 accumulate <= 1e-3; fp8 in / fp32 accumulate
-<= 3e-2; +-1 data with fp32 output: exact.  The BASELINE configurations are
+<= 3e-2; +-1 data with fp32 output: exact.  The benchmark configurations are
 run at full size and checked on a subset of batch images (the convolution is
 independent per image) plus size-independent properties."""
 import numpy as np
@@ -46,9 +46,9 @@ def _run(oracle, p, seed, tol, expect_kernel, dist="normal", bias=True,
 
 
 IGEMM_CASES = [
-    # BASELINE config 2 shape (3x3 s1 p1, 128->128, 28x28), reduced batch
+    # benchmark config 2 shape (3x3 s1 p1, 128->128, 28x28), reduced batch
     dict(batch=2, field=(28, 28), kernel=(3, 3), ci=128, co=128, pad=1),
-    # BASELINE config 3 shape (1x1, 256->64, 56x56), reduced batch
+    # benchmark config 3 shape (1x1, 256->64, 56x56), reduced batch
     dict(batch=1, field=(56, 56), kernel=(1, 1), ci=256, co=64),
     # M, N, K all ragged against the 128 x {64,128} x 64 tile
     dict(batch=3, field=(9, 7), kernel=(3, 3), ci=8, co=40, pad=1),
@@ -122,7 +122,7 @@ def test_pointwise_pm1_exact_and_big_tile_on_request(oracle):
 
 
 DW_CASES = [
-    # BASELINE config 4 shape (3x3 s2 p1, C=96, 112x112), reduced batch
+    # benchmark config 4 shape (3x3 s2 p1, C=96, 112x112), reduced batch
     dict(batch=2, field=(112, 112), kernel=(3, 3), groups=96, stride=2, pad=1),
     dict(batch=3, field=(9, 11), kernel=(3, 3), groups=8, pad=1),
     dict(batch=1, field=(13, 7), kernel=(5, 2), groups=24, stride=(1, 2),
@@ -208,7 +208,7 @@ def _fp8_case(oracle, p, seed, fmt_a, fmt_w, options=None):
 
 @pytest.mark.parametrize("fmt_a,fmt_w", [(1, 1), (1, 0), (0, 1), (0, 0)])
 def test_igemm_fp8_matches_oracle(oracle, fmt_a, fmt_w):
-    # BASELINE config 5 shape (3x3 s1 p1, 256->256, 14x14), reduced batch
+    # benchmark config 5 shape (3x3 s1 p1, 256->256, 14x14), reduced batch
     p = make_params(pa.QUARTER, pa.HALF, batch=2, field=(14, 14),
                     kernel=(3, 3), ci=256, co=256, pad=1)
     got, want, plan = _fp8_case(oracle, p, 6, fmt_a, fmt_w)
@@ -265,7 +265,7 @@ def test_quarter_small_integer_data_is_exact(oracle):
     np.testing.assert_array_equal(got3, want / 8.0)
 
 
-# ---- BASELINE configurations at full size ---------------------------------
+# ---- benchmark configurations at full size ---------------------------------
 
 def _full_size(oracle, p, seed, tol, kernel, act_fn=None, w_std=1.0,
                images=(0, -1)):

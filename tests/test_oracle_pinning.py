@@ -42,7 +42,7 @@ CASES_TORCH = [
          stride=(1, 2, 1), kdil=(2, 1, 1)),
     dict(field=(12, 12), kernel=(3, 3), groups=6, stride=2, pad=1, batch=2),
     dict(field=(6, 6), kernel=(1, 1), ci=5, co=7, batch=2),
-    # BASELINE config 1 shape class (N1 32x32 16->16 3x3 p1), reduced field
+    # benchmark config 1 shape class (N1 32x32 16->16 3x3 p1), reduced field
     dict(field=(16, 16), kernel=(3, 3), ci=16, co=16, pad=1),
 ]
 
