@@ -194,6 +194,10 @@ struct IgemmDesc {
   // and epilogue: for grids of more workgroups than CUs).  The 64-wide tile
   // always runs 3.
   uint32_t stages = 4;
+  // 1: the kernel that keeps a tile's input patch in LDS runs (unit stride,
+  // channels in whole 128-byte slices; igemmPatchTakes); the packed weights
+  // then have its layout (launchPackIgemmPatchWeights).  blockM 64 or 128.
+  uint32_t patch = 0;
 };
 /// How the kernel finds out which kernel taps of an output pixel read inside
 /// the input: a bit mask per pixel (up to 32 taps), ranges of valid kernel
@@ -210,6 +214,26 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
                        const void *in, const void *weightsPacked,
                        const void *bias, void *out, void *workspace,
                        const QuarterInfo &q, hipStream_t stream);
+
+/// The same convolution by the kernel that loads the input rows a tile reads
+/// into LDS once and forms every tap's operand by LDS addressing: unit stride,
+/// undilated input, two field dimensions, half or quarter inputs whose
+/// channels per group fill whole 128-byte slices, K not split.
+bool igemmPatchTakes(const IgemmDesc &d, int inType, int outType);
+/// Elements of its packed weights:
+/// [G][32-channel block][K half][k-step][operand][lane][16 bytes].
+uint64_t igemmPatchPackedElems(const IgemmDesc &d, int inType);
+/// src as for launchPackIgemmWeights; sourceTaps: taps of the stored kernel.
+hipError_t launchPackIgemmPatchWeights(const IgemmDesc &d, int inType,
+                                       const void *src, void *dst,
+                                       uint32_t sourceTaps, hipStream_t stream,
+                                       bool chansTransposed = false,
+                                       const IgemmTapSelection *select =
+                                           nullptr);
+hipError_t launchIgemmPatch(const IgemmDesc &d, int inType, int outType,
+                            const void *in, const void *weightsPacked,
+                            const void *bias, void *out, const QuarterInfo &q,
+                            hipStream_t stream);
 
 /// Several convolutions that run the same igemm kernel (same tile width,
 /// types, fp8 formats, channel-block alignment; K not split) as ONE launch

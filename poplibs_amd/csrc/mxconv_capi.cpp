@@ -175,6 +175,10 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
         return st;
       in = padded;
     }
+    if (plan->igemm.patch)
+      return hipStatus(mxk::launchIgemmPatch(plan->igemm, inType, outType, in,
+                                             w, bias, out, q, s),
+                       "implicit-GEMM convolution launch (resident patch)");
     if (!plan->igemmPhases.empty()) {
       // one convolution per phase of the zero-stuffed input, in one launch
       mxk::IgemmFusedItem items[mxk::kIgemmMaxFused];
@@ -604,6 +608,13 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
     }
     if (!plan->igemmPhases.empty())
       return MXCONV_OK;
+    if (plan->igemm.patch)
+      return hipStatus(
+          mxk::launchPackIgemmPatchWeights(
+              plan->igemm, p.inputType.id(), weights_external, weights_packed,
+              uint32_t(taps), s, false,
+              plan->kernelSelected ? &plan->igemmTaps : nullptr),
+          "weight packing");
     return hipStatus(
         mxk::launchPackIgemmWeights(
             weights_external, weights_packed, uint32_t(p.numConvGroups),
@@ -765,7 +776,7 @@ mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
     // the input, several phases, an output border to fill - runs on its own)
     if (p->outputElems == 0 || p->kernel != mxconv_plan::Kernel::IGEMM ||
         p->pointwiseOn || p->paddedInputChans || !p->igemmPhases.empty() ||
-        p->outputPadded)
+        p->outputPadded || p->igemm.patch)
       return false;
     unsplit[slot] = p->igemm;
     unsplit[slot].splitK = 1;
@@ -961,6 +972,11 @@ mxconv_status mxconv_matmul_pack_rhs(const mxconv_plan *plan, const void *rhs,
     if (plan->pointwiseOn)
       return hipStatus(mxk::launchPackPointwiseWeights(plan->pointwise, rhs,
                                                        weights_packed, s, true),
+                       "weight packing");
+    if (plan->igemm.patch)
+      return hipStatus(mxk::launchPackIgemmPatchWeights(
+                           plan->igemm, p.inputType.id(), rhs, weights_packed,
+                           1, s, true),
                        "weight packing");
     return hipStatus(
         mxk::launchPackIgemmWeights(
@@ -1186,7 +1202,8 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
       uint32_t(Ci), B,           X * G * B,   G * B};
   const bool direct = plan->kernel == mxconv_plan::Kernel::IGEMM &&
                       !plan->pointwiseOn && !plan->paddedInputChans &&
-                      plan->igemmPhases.empty() && !plan->kernelSelected;
+                      plan->igemmPhases.empty() && !plan->kernelSelected &&
+                      !plan->igemm.patch;
   if (direct) {
     // deltas [B][Y][G][Co] -> straight into the matrix-core kernel's packed
     // weights [G][coPadded][kPadded], k = y * B + b; both rearrangements in

@@ -196,6 +196,11 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       pc.splitK = requireUnsigned(sub, m.second);
     } else if (m.first == "stages") {
       pc.stages = requireUnsigned(sub, m.second);
+    } else if (m.first == "patch") {
+      const unsigned v = requireUnsigned(sub, m.second);
+      if (v > 1)
+        throw invalid_option("'" + sub + "': Must be 0 or 1");
+      pc.patch = int(v);
     } else if (m.first == "tileH") {
       pc.tileH = requireUnsigned(sub, m.second);
     } else if (m.first == "tileW") {

@@ -38,6 +38,9 @@ struct PlanConstraints {
   /// Parts the matrix-core kernel cuts K into; 0 = planner's choice.
   unsigned splitK = 0;
   unsigned stages = 0; // LDS stages of the 128-wide igemm tile: 2 or 4
+  /// The matrix-core kernel that keeps the input patch in LDS: -1 planner's
+  /// choice, 0 never, 1 whenever it can take the convolution.
+  int patch = -1;
   /// Output tile of the depthwise kernel; 0 = planner's choice.
   unsigned tileH = 0, tileW = 0;
   std::string text; // the JSON as given, kept for reporting and cache keys

@@ -461,7 +461,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     g.blockN = pc.blockN ? pc.blockN : (co <= 64 ? 64 : 128);
     const unsigned stepElems = unsigned(128 / params.inputType.size());
     g.blockK = pc.blockK ? pc.blockK : stepElems;
-    if (g.blockM != 128 || (g.blockN != 64 && g.blockN != 128) ||
+    if ((g.blockM != 128 && g.blockM != 64) ||
+        (g.blockN != 64 && g.blockN != 128) ||
         g.blockK != stepElems)
       throw poplar::invalid_option(
           "planConstraints gfx950 tile not available: blockM must be 128, "
@@ -657,7 +658,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         s.hiH == s.inH && s.hiW == s.inW && s.outH == s.inH &&
         s.outW == s.inW;
     plan.pointwiseOn =
-        unitWindow && ciPadded == ci && pc.kernel != "igemm" && !pc.blockM &&
+        unitWindow && ciPadded == ci && pc.kernel != "igemm" &&
+        pc.patch != 1 && !pc.blockM &&
         !pc.blockN && !pc.blockK &&
         mxk::pointwiseTakes(pw,
                             halfIn    ? mxk::kHalf
@@ -667,6 +669,40 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                                                               : mxk::kFloat);
     if (plan.pointwiseOn)
       plan.weightPackedElems = mxk::pointwisePackedElems(pw);
+    // Unit stride and whole 128-byte slices of channels: the kernel that
+    // keeps the tile's input patch in LDS reads every input element once
+    // instead of once per tap.
+    if (!plan.pointwiseOn && plan.igemmPhases.empty() &&
+        !plan.paddedInputChans &&
+        (g.splitK == 1 || (pc.patch == 1 && !pc.splitK)) && pc.patch != 0 &&
+        !pc.blockN && !pc.blockK && !pc.stages) {
+      mxk::IgemmDesc trial = g;
+      trial.patch = 1;
+      trial.splitK = 1; // (asked for by name, it runs K whole)
+      const int inId = halfIn ? mxk::kHalf : floatIn ? mxk::kFloat
+                                                     : mxk::kQuarter;
+      const int outId =
+          params.outputType == poplar::HALF ? mxk::kHalf : mxk::kFloat;
+      // It wins where the launch is one round of workgroups or less (its
+      // workgroup fills a CU's LDS, so two never share a CU and cover each
+      // other's start-up the way the streaming kernel's do).
+      const std::size_t patchTiles =
+          (std::size_t(s.batch) * s.outH * s.outW + trial.blockM - 1) /
+          trial.blockM * ((co + 127) / 128) * p.numConvGroups;
+      if (mxk::igemmPatchTakes(trial, inId, outId) &&
+          (pc.patch == 1 || (co > 64 && s.kH * s.kW > 1 &&
+                             patchTiles <= gfx950::numCUs))) {
+        g = trial;
+        g.blockN = 128;
+        plan.workspaceBytes = 0;
+        plan.coPadded = (co + 127) / 128 * 128;
+        plan.weightPackedElems = mxk::igemmPatchPackedElems(g, inId);
+      }
+    }
+    if (!g.patch && g.blockM != 128)
+      throw poplar::invalid_option(
+          "planConstraints gfx950 blockM 64 goes with the resident-patch "
+          "kernel only");
   } else if (chosen == Kernel::DEPTHWISE) {
     mxk::DepthwiseDesc &d = plan.depthwise;
     d.batch = uint32_t(s.batch);
@@ -717,7 +753,8 @@ std::string mxconv_plan::describe() const {
            : params.inputType == poplar::FLOAT ? "fp32"
                                                : "fp16")
        << " operands, fp32 accumulate)"
-       << (pointwiseOn ? ", pointwise streaming variant" : "");
+       << (pointwiseOn ? ", pointwise streaming variant" : "")
+       << (igemm.patch ? ", input patch resident in LDS" : "");
     break;
   case Kernel::DEPTHWISE:
     os << (mxk::depthwiseDirectInBlocks(depthwise)
