@@ -661,10 +661,17 @@ bool patchShape(const IgemmDesc &d, int inType, int outType, PatchShape &s) {
   const uint64_t tile =
       32 * s.rb * (kPatchBN * (outType == kHalf ? 2 : 4) + 16);
   const uint64_t patchEnd = (patch + 1023) / 1024 * 1024;
+  // Beside the patch where there is room (the waves then hand over their
+  // sums as they finish, without waiting for the others to leave the patch);
+  // the output tile, written once all have, goes over the patch if it ends
+  // before the exchange area, else behind that.
   uint64_t bytes;
-  if (patchEnd + exchange <= uint64_t(kLdsLimit)) {
-    s.exchangeByte = uint32_t(patchEnd), s.tileByte = 0;
-    bytes = std::max(patchEnd + exchange, tile);
+  if (patchEnd + exchange <= uint64_t(kLdsLimit) &&
+      (tile <= patchEnd ||
+       patchEnd + exchange + tile <= uint64_t(kLdsLimit))) {
+    s.exchangeByte = uint32_t(patchEnd);
+    s.tileByte = tile <= patchEnd ? 0 : uint32_t(patchEnd + exchange);
+    bytes = patchEnd + exchange + (tile <= patchEnd ? 0 : tile);
   } else {
     s.exchangeByte = 0, s.tileByte = uint32_t(exchange);
     bytes = std::max(patch, exchange + tile);

@@ -145,3 +145,19 @@ def test_patch_twice_in_a_row_is_bit_identical(oracle):
     first = run_conv(p, aq, wq, None, FORCED)
     second = run_conv(p, aq, wq, None, FORCED)
     np.testing.assert_array_equal(first, second)
+
+
+def test_patch_small_patch_float_output_repeats(oracle):
+    """A patch smaller than the fp32 output tile: the epilogue's exchange area
+    and the output tile must not share LDS (waves leave the exchange at
+    different times).  Many runs, all equal to the oracle's +-1 result."""
+    p = make_params(pa.HALF, pa.FLOAT, batch=2, field=(6, 7), kernel=(3, 3),
+                    ci=64, co=72, pad=1)
+    first = _run(oracle, p, 41, 0, dist="pm1")
+    from gpu_helpers import quantize, run_conv
+    acts, weights, biases = random_data(p, 41, "pm1")
+    aq, _ = quantize(acts, p.inputType)
+    wq, _ = quantize(weights, p.inputType)
+    bq, _ = quantize(biases, p.outputType)
+    for _ in range(20):
+        np.testing.assert_array_equal(run_conv(p, aq, wq, bq, FORCED), first)
