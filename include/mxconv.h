@@ -281,6 +281,21 @@ mxconv_status mxconv_fwd(const mxconv_plan *plan, const void *in,
                          void *out, void *workspace, size_t workspace_bytes,
                          mxconv_stream stream);
 
+/* mxconv_fwd for callers that cannot allocate device memory or carry a
+ * workspace around (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the scratch memory a plan needs - fp32
+ * partial tiles when K is split, the zero-filled copy of an input whose
+ * channels are padded - comes from a buffer of 32 MiB built into the library,
+ * one per GPU.  No counterpart in the reference (Poplar owns all memory
+ * there).  Returns MXCONV_WORKSPACE_TOO_SMALL for a plan whose workspace
+ * exceeds the buffer; allocates nothing.  All calls on one GPU share the
+ * buffer: calls that overlap in time on one GPU race. */
+mxconv_status mxconv_fwd_static_scratch(const mxconv_plan *plan,
+                                        const void *in,
+                                        const void *weights_packed,
+                                        const void *bias, void *out,
+                                        mxconv_stream stream);
+
 /* The same for QUARTER inputs.  Each metadata byte is
  * (format << 7) | (scale & 0x3f): format 1 = E4M3 ("F143"), 0 = E5M2
  * ("F152"); scale is a signed 6-bit power of two, value = fp8 * 2^scale (bit

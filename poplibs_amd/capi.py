@@ -172,6 +172,8 @@ def lib():
                                             c_void_p]),
         "mxconv_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_size_t, c_void_p]),
+        "mxconv_fwd_static_scratch": (c_int, [c_void_p, c_void_p, c_void_p,
+                                              c_void_p, c_void_p, c_void_p]),
         "mxconv_fwd_quarter": (c_int, [c_void_p, c_void_p, c_uint8, c_void_p,
                                        c_uint8, c_void_p, c_void_p, c_void_p,
                                        c_size_t, c_void_p]),
@@ -599,6 +601,11 @@ class Plan:
             workspace_bytes=0, stream=0):
         _check(lib().mxconv_fwd(self._h, inp, weights_packed, bias, out,
                                 workspace, workspace_bytes, stream))
+
+    def fwd_static_scratch(self, inp, weights_packed, out, bias=None,
+                           stream=0):
+        _check(lib().mxconv_fwd_static_scratch(self._h, inp, weights_packed,
+                                               bias, out, stream))
 
     def fwd_quarter(self, inp, in_metadata, weights_packed, weights_metadata,
                     out, bias=None, workspace=None, workspace_bytes=0,

@@ -2,6 +2,8 @@
 // exceptions into status codes, and dispatch to the kernel launchers.
 #include "mxconv.h"
 
+#include <hip/hip_runtime.h>
+
 #include "../src/ConvOptions.hpp"
 #include "../src/MatMulOptions.hpp"
 #include "../src/Plan.hpp"
@@ -17,6 +19,7 @@
 #include <new>
 #include <sstream>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -712,6 +715,74 @@ mxconv_status mxconv_fwd_quarter(const mxconv_plan *plan, const void *in,
   return forward(plan, in, weights_packed, bias, out, workspace,
                  workspace_bytes, quarterInfo(in_metadata, weights_metadata),
                  stream);
+}
+
+// ---- forward pass that allocates nothing ----------------------------------
+
+namespace {
+
+// Scratch memory of the allocation-free entry point: one array per GPU, part
+// of the loaded code object, held until the process ends.
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxScratchDevices = 64;
+std::mutex scratchMutex;
+void *scratchOfDevice[kMaxScratchDevices] = {};
+
+/// The address of `scratch` on the current device (every GPU holds its own
+/// copy at its own address; the array's name is no device address in host
+/// code), looked up once per device.
+mxconv_status staticScratch(void **ptr) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess)
+    return hipStatus(e, "hipGetDevice");
+  if (device < 0 || device >= kMaxScratchDevices)
+    return fail(MXCONV_UNSUPPORTED, "device ordinal beyond " +
+                                        std::to_string(kMaxScratchDevices));
+  std::lock_guard<std::mutex> lock(scratchMutex);
+  if (!scratchOfDevice[device]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return hipStatus(e != hipSuccess ? e : hipErrorInvalidSymbol,
+                       "hipGetSymbolAddress(scratch)");
+    scratchOfDevice[device] = p;
+  }
+  *ptr = scratchOfDevice[device];
+  return MXCONV_OK;
+}
+
+} // namespace
+
+mxconv_status mxconv_fwd_static_scratch(const mxconv_plan *plan,
+                                        const void *in,
+                                        const void *weights_packed,
+                                        const void *bias, void *out,
+                                        mxconv_stream stream) {
+  REQUIRE_ARG(plan);
+  lastError.clear();
+  if (plan->params.inputType == poplar::QUARTER)
+    return fail(MXCONV_INVALID_PARAMS,
+                "quarter inputs carry metadata: call mxconv_fwd_quarter");
+  if (plan->workspaceBytes > kStaticScratchBytes)
+    return fail(MXCONV_WORKSPACE_TOO_SMALL,
+                "the plan needs " + std::to_string(plan->workspaceBytes) +
+                    " bytes of scratch memory, the built-in buffer holds " +
+                    std::to_string(kStaticScratchBytes) +
+                    ": call mxconv_fwd with a workspace");
+  void *ws = nullptr;
+  if (plan->workspaceBytes) {
+    // (every byte a launch reads from its scratch memory it has written
+    // before: partial sums and padded copies are stored whole, so nothing has
+    // to be cleared between calls)
+    const mxconv_status st = staticScratch(&ws);
+    if (st != MXCONV_OK)
+      return st;
+  }
+  return forward(plan, in, weights_packed, bias, out, ws,
+                 plan->workspaceBytes, mxk::QuarterInfo{}, stream);
 }
 
 // ---- several convolutions at once -----------------------------------------
