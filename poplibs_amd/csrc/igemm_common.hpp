@@ -102,12 +102,16 @@ using LdsPtr = __attribute__((address_space(3))) void *;
 /// dst + 16 l (dst is wave-uniform).  Out-of-range offsets deliver zeros.
 /// The builtin exists for the GPU target only; the host compilation pass,
 /// which merely needs the kernels' launch stubs, sees an empty body.
+/// POLICY: the load's cache policy bits - 0, or kStreamingLoad for data that
+/// is read once.
+constexpr int kStreamingLoad = 2;
+template <int POLICY = 0>
 __device__ __forceinline__ void loadToLds(__amdgpu_buffer_rsrc_t buffer,
                                           LdsPtr dst, uint32_t vectorOffset,
                                           uint32_t scalarOffset) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, dst, 16, vectorOffset,
-                                           scalarOffset, 0, 0);
+                                           scalarOffset, 0, POLICY);
 #endif
 }
 

@@ -182,9 +182,14 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
         const uint32_t m = mTile * TM + mb * 32 + r;
         const uintx4 data =
             *reinterpret_cast<const uintx4 *>(stage + r * kPwStageRow + vec * 16);
-        if (m < a.M && n < d.outChansPerGroup)
-          *reinterpret_cast<uintx4 *>(out + size_t(m) * outChans +
-                                      g * d.outChansPerGroup + n) = data;
+        if (m < a.M && n < d.outChansPerGroup) {
+          uintx4 *dst = reinterpret_cast<uintx4 *>(
+              out + size_t(m) * outChans + g * d.outChansPerGroup + n);
+          // streaming store (the output is not read again here): 15.2 ->
+          // 12.4 us on the 56 x 56, 256 -> 64 layer.  The same hint on the
+          // loads loses a microsecond of that.
+          __builtin_nontemporal_store(data, dst);
+        }
       }
       MXK_WAIT_LGKMCNT0(); // staging is read before the next pass rewrites it
     }
