@@ -513,6 +513,8 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
     __syncthreads();
     // 16-byte stores, whole rows of the tile per instruction, through a
     // buffer that ends with the last valid row: rows beyond M go nowhere.
+    // (Streaming cache policy - the same bit as for loads: the tile is not
+    // read again here.)
     constexpr int kVecsPerRow = kPatchBN * int(sizeof(OutT)) / 16;
     constexpr int kRowsPerPass = kPatchThreads / kVecsPerRow;
     const uint32_t outRowBytes = a.outChans * sizeof(OutT);
@@ -533,7 +535,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
       __builtin_amdgcn_raw_buffer_store_b128(
           *reinterpret_cast<const uintx4 *>(from +
                                             pass * kRowsPerPass * kOutRow),
-          outBuf, to, pass * kRowsPerPass * outRowBytes, 0);
+          outBuf, to, pass * kRowsPerPass * outRowBytes, kStreamingLoad);
   }
 }
 
