@@ -236,6 +236,15 @@ void mxconv_plan_destroy(mxconv_plan *plan);
 mxconv_status mxconv_plan_describe(const mxconv_plan *plan, char *buffer,
                                    size_t capacity, size_t *needed);
 
+/* Whether weights packed for `packed_for` are laid out as `plan` reads them
+ * (*same = 1) or not (0).  In the reference the options given to
+ * createWeights only decide a tensor layout and convolution() rearranges a
+ * tensor laid out otherwise (lib/poplin/Convolution.cpp:2569-2628); here a
+ * packed buffer carries no description of itself, so the caller has to ask. */
+mxconv_status mxconv_plans_pack_alike(const mxconv_plan *plan,
+                                      const mxconv_plan *packed_for,
+                                      int32_t *same);
+
 /* Sizes, in bytes, of the device buffers mxconv_fwd works on; what
  * createInput / createWeights / createConvOutput / createBiases allocate in
  * the reference (lib/poplin/Convolution.cpp:1563-1577, 1713-1728, 1813-1825,

@@ -164,6 +164,8 @@ def lib():
                                          POINTER(c_size_t)]),
         "mxconv_plan_buffer_bytes": (c_int, [c_void_p, c_int32,
                                              POINTER(c_size_t)]),
+        "mxconv_plans_pack_alike": (c_int, [c_void_p, c_void_p,
+                                            POINTER(c_int32)]),
         "mxconv_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p,
                                         c_void_p]),
         "mxconv_acts_to_internal": (c_int, [c_void_p, c_void_p, c_void_p,
@@ -579,6 +581,13 @@ class Plan:
         _check(lib().mxconv_plan_describe(self._h, buf, need.value,
                                           byref(need)))
         return buf.value.decode()
+
+    def packs_like(self, other):
+        """Whether weights packed for `other` are laid out as this plan
+        reads them."""
+        same = c_int32()
+        _check(lib().mxconv_plans_pack_alike(self._h, other._h, byref(same)))
+        return bool(same.value)
 
     def buffer_bytes(self, which):
         v = c_size_t()

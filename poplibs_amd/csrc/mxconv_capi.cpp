@@ -574,6 +574,44 @@ mxconv_status mxconv_plan_buffer_bytes(const mxconv_plan *plan, int32_t which,
   return fail(MXCONV_INVALID_PARAMS, "unknown buffer id");
 }
 
+namespace {
+/// Everything the layout of a plan's packed weights depends on.
+std::string packingSignature(const mxconv_plan &p) {
+  std::ostringstream os;
+  os << int(p.kernel) << '/' << p.params.inputType.toString() << '/'
+     << p.weightElems << '/' << p.weightPackedElems;
+  if (p.kernel == mxconv_plan::Kernel::IGEMM) {
+    os << "/pw" << p.pointwiseOn << "/patch" << p.igemm.patch << "/co"
+       << p.coPadded << "/k" << p.kPadded << "/ci" << p.paddedInputChans
+       << "/sel" << p.kernelSelected;
+    auto taps = [&](const mxk::IgemmTapSelection &t) {
+      os << '[' << t.kW << ',' << t.firstH << ',' << t.stepH << ','
+         << t.countH << ',' << t.firstW << ',' << t.stepW << ',' << t.countW
+         << ',' << t.kH << ',' << t.firstD << ',' << t.stepD << ','
+         << t.countD << ']';
+    };
+    if (p.kernelSelected)
+      taps(p.igemmTaps);
+    for (const auto &phase : p.igemmPhases) {
+      os << "/ph" << phase.packedOffset << ':' << phase.kPadded;
+      taps(phase.taps);
+    }
+  }
+  return os.str();
+}
+} // namespace
+
+mxconv_status mxconv_plans_pack_alike(const mxconv_plan *plan,
+                                      const mxconv_plan *packed_for,
+                                      int32_t *same) {
+  REQUIRE_ARG(plan);
+  REQUIRE_ARG(packed_for);
+  REQUIRE_ARG(same);
+  lastError.clear();
+  *same = packingSignature(*plan) == packingSignature(*packed_for) ? 1 : 0;
+  return MXCONV_OK;
+}
+
 mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
                                   const void *weights_external,
                                   void *weights_packed, mxconv_stream stream) {
@@ -1274,7 +1312,10 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
   const bool direct = plan->kernel == mxconv_plan::Kernel::IGEMM &&
                       !plan->pointwiseOn && !plan->paddedInputChans &&
                       plan->igemmPhases.empty() && !plan->kernelSelected &&
-                      !plan->igemm.patch;
+                      !plan->igemm.patch &&
+                      // (a padded output field - the forward kernel was
+                      // truncated - is filled by the general path)
+                      !plan->outputPadded;
   if (direct) {
     // deltas [B][Y][G][Co] -> straight into the matrix-core kernel's packed
     // weights [G][coPadded][kPadded], k = y * B + b; both rearrangements in
@@ -1365,7 +1406,7 @@ mxconv_status checkWuCall(const mxconv_plan *plan, const void *zDeltas,
   if (plan->weightElems)
     REQUIRE_ARG(zDeltas);
   const size_t need = wuWorkspace(plan).total;
-  if (workspaceBytes < need || !workspace)
+  if (workspaceBytes < need || (need && !workspace))
     return fail(MXCONV_WORKSPACE_TOO_SMALL,
                 "workspace of " + std::to_string(need) + " bytes required");
   return MXCONV_OK;

@@ -267,6 +267,22 @@ void run(const PlanHandle &plan, const ConvParams &params,
     check(mxconv_acts_to_internal(plan.plan, in.data(), inCl.data(),
                                   streamOf(prog)));
   }
+  if (weights.layout() == DeviceTensor::Layout::PackedWeights) {
+    // A packed buffer is only good for plans that pack the same way (kernel,
+    // tile padding, phases ...): another plan would read it wrongly, possibly
+    // beyond its end.  (PopLibs would rearrange such a tensor,
+    // lib/poplin/Convolution.cpp:2569-2628; packing cannot be undone here.)
+    const auto *packing =
+        static_cast<const PlanHandle *>(weights.packedFor.get());
+    int32_t same = 0;
+    if (packing)
+      check(mxconv_plans_pack_alike(plan.plan, packing->plan, &same));
+    if (!same)
+      throw poputil::poplibs_error(
+          "The weights were arranged (createWeights) for another plan than "
+          "the one these parameters and options give: pass them in the "
+          "external layout or create them with the same options");
+  }
   if (weights.layout() == DeviceTensor::Layout::External) {
     wPacked = DeviceTensor(weights.elementType(), weights.shape(),
                            DeviceTensor::Layout::PackedWeights,

@@ -218,6 +218,32 @@ def test_weight_deltas_of_a_small_batch_run_on_the_matrix_cores(oracle):
     assert rel_l2(got, oracle.weight_deltas(p, xd, dd, threads=8)) <= 1e-5
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch", [8, 16])
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_weight_deltas_of_a_truncated_kernel(oracle, batch, out_type):
+    # Kernel truncation of the layer is output padding of its weight update
+    # pass (the deltas of the truncated taps are zero): with a batch that is
+    # a whole vector the pass runs on the matrix cores, and the padded rows
+    # of the deltas have to be written all the same.
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, out_type, batch=batch, field=(8, 8),
+                    kernel=(3, 3), ci=16, co=16, ktl=(1, 0), pad=1)
+    rng = np.random.default_rng(27)
+    xq, xd = quantize(rng.standard_normal((batch, 16, 8, 8)), pa.HALF)
+    dq, dd = quantize(
+        rng.standard_normal((batch, 16, *p.getOutputFieldShape())) * 0.1,
+        pa.HALF)
+    got, plan = run_weight_update(p, xq, dq)
+    assert "implicit GEMM" in plan.describe(), plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert got.shape == want.shape
+    assert not want[:, :, :, 0, :].any()  # the truncated kernel row
+    tol = 1e-3 if out_type == pa.HALF else 1e-5
+    assert rel_l2(got, want) <= tol, (rel_l2(got, want), plan.describe())
+    np.testing.assert_array_equal(got[:, :, :, 0, :], 0)
+
+
 DEPTHWISE_WU_CASES = [
     dict(batch=3, field=(20, 21), kernel=(3, 3), groups=24, stride=2, pad=1),
     dict(batch=2, field=(14, 14), kernel=(5, 5), groups=16, pad=2),
