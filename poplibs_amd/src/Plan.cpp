@@ -4,6 +4,8 @@
 #include "poputil/exceptions.hpp"
 
 #include <algorithm>
+#include <cmath>
+#include <cstdio>
 #include <sstream>
 
 namespace poplin {
@@ -199,6 +201,54 @@ std::pair<unsigned, unsigned> chooseDepthwiseTile(const Simple2D &s,
       return {bestH, bestW};
   }
   return {0, 0};
+}
+
+} // namespace
+
+namespace {
+
+// Cost model of the matrix-core kernels, in microseconds, from kernel traces
+// and in-kernel cycle stamps on MI355X at the ~2.0 GHz the chip holds under
+// MFMA load.  A k-step is 128 bytes of K per tile row.
+constexpr double kLaunchUs = 2.0; // dispatch + drain of any kernel
+
+/// Rounds of workgroups a launch makes with `perCU` workgroups per CU: whole
+/// ones where one workgroup owns a CU (equal tiles all end together), softer
+/// where two share it.
+double roundsOf(std::size_t workgroups, std::size_t perCU) {
+  const double slots = double(gfx950::numCUs) * double(perCU);
+  if (double(workgroups) <= slots)
+    return 1.0;
+  const double whole = std::ceil(double(workgroups) / slots);
+  return perCU == 1 ? whole : std::min(whole, double(workgroups) / slots + 0.5);
+}
+
+/// igemmKernel: 1.45 us start-up + 1.5 us epilogue, 0.345 us per k-step of a
+/// 128 x 128 tile (0.24 for 128 x 64); further rounds on a CU pay another
+/// 1.5 us (nothing overlaps the next workgroup's start-up); two workgroups
+/// sharing a CU take 2.1 times one's time between them; K split adds the
+/// second kernel's 5 us.
+double estimateStreaming(std::size_t workgroups, std::size_t kSteps,
+                         std::size_t perCU, unsigned blockN, unsigned splitK) {
+  const double rounds = roundsOf(workgroups, perCU);
+  const double step = blockN == 128 ? 0.345 : 0.24;
+  double tile = 2.95 + step * double(kSteps);
+  if (perCU == 1 && rounds > 1)
+    tile += 1.5;
+  if (perCU == 2)
+    tile *= double(workgroups) > double(gfx950::numCUs) ? 2.1 : 1.0;
+  return kLaunchUs + rounds * tile + (splitK > 1 ? 5.0 : 0.0);
+}
+
+/// igemmPatchKernel: 1.9 us to the first MFMA + 0.5 us reduction and stores,
+/// 0.333 us per k-step of 128 pixels (half of that for 64); one workgroup per
+/// CU, so further rounds pay their start-up in full (4.5 us instead of 2.4).
+double estimatePatch(std::size_t workgroups, std::size_t kSteps,
+                     unsigned blockM) {
+  const double rounds = roundsOf(workgroups, 1);
+  const double step = blockM == 128 ? 0.333 : 0.167;
+  const double fixed = rounds > 1 ? 4.5 : 2.4;
+  return kLaunchUs + rounds * (fixed + step * double(kSteps));
 }
 
 } // namespace
@@ -683,15 +733,92 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                                                      : mxk::kQuarter;
       const int outId =
           params.outputType == poplar::HALF ? mxk::kHalf : mxk::kFloat;
-      // It wins where the launch is one round of workgroups or less (its
-      // workgroup fills a CU's LDS, so two never share a CU and cover each
-      // other's start-up the way the streaming kernel's do).
-      const std::size_t patchTiles =
-          (std::size_t(s.batch) * s.outH * s.outW + trial.blockM - 1) /
-          trial.blockM * ((co + 127) / 128) * p.numConvGroups;
-      if (mxk::igemmPatchTakes(trial, inId, outId) &&
-          (pc.patch == 1 || (co > 64 && s.kH * s.kW > 1 &&
-                             patchTiles <= gfx950::numCUs))) {
+      // Weigh the tilings: the streaming kernel as planned above against
+      // this kernel with 128- and 64-pixel tiles, by estimated time.
+      const bool takes = mxk::igemmPatchTakes(trial, inId, outId);
+      const std::size_t m = std::size_t(s.batch) * s.outH * s.outW;
+      const std::size_t nTiles128 = (co + 127) / 128 * p.numConvGroups;
+      const std::size_t stepBytes = 128;
+      const std::size_t patchSteps =
+          ciPadded * params.inputType.size() / stepBytes * s.kH * s.kW;
+      auto add = [&](const std::string &name, std::size_t workgroups,
+                     std::size_t perCU, std::size_t kSteps, double us,
+                     double rounds) {
+        mxconv_plan::Candidate c;
+        c.name = name, c.workgroups = workgroups, c.perCU = perCU;
+        c.kSteps = kSteps, c.estimateUs = us, c.rounds = rounds;
+        plan.candidates.push_back(c);
+        return plan.candidates.size() - 1;
+      };
+      const std::size_t streamTiles =
+          (m + 127) / 128 * (plan.coPadded / g.blockN) * p.numConvGroups *
+          g.splitK;
+      const std::size_t streamSteps =
+          (plan.kPadded / g.blockK + g.splitK - 1) / g.splitK;
+      const std::size_t streamPerCU = g.blockN == 64 || g.stages == 2 ? 2 : 1;
+      const std::size_t iStream =
+          add("streaming " + std::to_string(g.blockM) + " x " +
+                  std::to_string(g.blockN) + ", " +
+                  std::to_string(g.blockN == 128 ? g.stages : 3) + " stages" +
+                  (g.splitK > 1 ? ", K in " + std::to_string(g.splitK) +
+                                      " parts"
+                                : ""),
+              streamTiles, streamPerCU, streamSteps,
+              estimateStreaming(streamTiles, streamSteps, streamPerCU,
+                                g.blockN, g.splitK),
+              roundsOf(streamTiles, streamPerCU));
+      std::size_t best = iStream;
+      if (takes && s.kH * s.kW > 1 && co > 64) {
+        for (unsigned bm : {128u, 64u}) {
+          mxk::IgemmDesc t2 = trial;
+          t2.blockM = bm;
+          if (!mxk::igemmPatchTakes(t2, inId, outId))
+            continue;
+          const std::size_t tiles = (m + bm - 1) / bm * nTiles128;
+          const std::size_t i =
+              add("resident patch " + std::to_string(bm) + " x 128", tiles, 1,
+                  patchSteps, estimatePatch(tiles, patchSteps, bm),
+                  roundsOf(tiles, 1));
+          if (plan.candidates[i].estimateUs <
+              plan.candidates[best].estimateUs)
+            best = i;
+        }
+      }
+      // planConstraints: patch 1 = whenever it can, with the tile asked for
+      // (128 by default)
+      bool usePatch = takes && best != iStream;
+      if (pc.patch == 1 && takes) {
+        usePatch = true;
+        best = plan.candidates.size();
+        for (std::size_t i = 0; i != plan.candidates.size(); ++i)
+          if (plan.candidates[i].name ==
+              "resident patch " + std::to_string(trial.blockM) + " x 128")
+            best = i;
+        if (best == plan.candidates.size()) {
+          const std::size_t tiles =
+              (m + trial.blockM - 1) / trial.blockM * nTiles128;
+          best = add("resident patch " + std::to_string(trial.blockM) +
+                         " x 128",
+                     tiles, 1, patchSteps,
+                     estimatePatch(tiles, patchSteps, trial.blockM),
+                     roundsOf(tiles, 1));
+        }
+      } else if (pc.blockM && usePatch) {
+        // a forced tile height picks among the patch tilings only
+        usePatch = false;
+        for (std::size_t i = 0; i != plan.candidates.size(); ++i)
+          if (plan.candidates[i].name ==
+              "resident patch " + std::to_string(pc.blockM) + " x 128")
+            usePatch = true, best = i;
+        if (!usePatch)
+          best = iStream;
+      }
+      plan.candidates[best].chosen = true;
+      if (usePatch) {
+        trial.blockM = plan.candidates[best].name.find(" 64 x") !=
+                               std::string::npos
+                           ? 64
+                           : 128;
         g = trial;
         g.blockN = 128;
         plan.workspaceBytes = 0;
@@ -794,8 +921,17 @@ std::string mxconv_plan::describe() const {
     } else {
       os << "        block M x N x K            " << g.blockM << " x "
          << g.blockN << " x " << g.blockK << "\n";
-      os << "        workgroups                 " << tiles * g.splitK << "\n";
-      if (g.blockN == 128)
+      os << "        workgroups                 " << tiles * g.splitK
+         << " on " << gfx950::numCUs << " CUs ("
+         << std::min<std::size_t>(tiles * g.splitK, gfx950::numCUs)
+         << " busy, "
+         << (tiles * g.splitK + gfx950::numCUs - 1) / gfx950::numCUs
+         << " round(s) of tiles)\n";
+      if (g.patch)
+        os << "        data path                  input rows of the tile "
+              "resident in LDS, weights straight to registers; 8 waves, one "
+              "workgroup per CU\n";
+      else if (g.blockN == 128)
         os << "        LDS stages                 " << g.stages
            << (g.stages == 2 ? " (two workgroups per CU)\n"
                              : " (one workgroup per CU)\n");
@@ -812,8 +948,25 @@ std::string mxconv_plan::describe() const {
       else if (mxk::igemmTapAddressing(g) == mxk::kDilatedTaps)
         os << "        tap addressing             arithmetic (dilated "
               "input)\n";
-      os << "        packed weights             [G=" << g.groups << "]["
-         << coPadded << "][" << kPadded << "]\n";
+      if (g.patch)
+        os << "        packed weights             [G=" << g.groups << "]["
+           << coPadded / 32 << " blocks of 32][" << k * params.inputType.size() / 128
+           << " k-steps][2 halves][2][64 lanes][16 bytes]\n";
+      else
+        os << "        packed weights             [G=" << g.groups << "]["
+           << coPadded << "][" << kPadded << "]\n";
+      if (!candidates.empty()) {
+        os << "        tilings weighed            workgroups  per CU  rounds  "
+              "k-steps  estimate\n";
+        for (const auto &c : candidates) {
+          char line[160];
+          std::snprintf(line, sizeof line,
+                        "          %c %-34s %8zu  %6zu  %6.2f  %7zu  %7.1f us\n",
+                        c.chosen ? '*' : ' ', c.name.c_str(), c.workgroups,
+                        c.perCU, c.rounds, c.kSteps, c.estimateUs);
+          os << line;
+        }
+      }
       if (paddedInputChans)
         os << "        input channels padded      "
            << params.inputChannelsPerConvGroup << " -> " << paddedInputChans

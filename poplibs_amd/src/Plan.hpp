@@ -29,6 +29,17 @@ struct mxconv_plan {
   bool zeroConv = false;
   Kernel kernel = Kernel::GENERIC;
   std::string reason; // why this kernel was chosen
+  // The tilings of the matrix-core kernels the planner weighed for this
+  // convolution, with the time each was estimated to take (the role of the
+  // reference's per-candidate cost estimates, lib/poplin/ConvPlan.cpp:502-565,
+  // reportPlanEstimatedCosts).
+  struct Candidate {
+    std::string name;
+    std::size_t workgroups = 0, perCU = 1, kSteps = 0;
+    double rounds = 0, estimateUs = 0;
+    bool chosen = false;
+  };
+  std::vector<Candidate> candidates;
 
   mxk::GenericDesc generic{};     // always valid: describes `canonical`
   mxk::IgemmDesc igemm{};         // valid when kernel == IGEMM

@@ -410,7 +410,10 @@ def test_planner_choices():
     assert "K split" not in pa.Plan(c2).describe()
     # one workgroup per CU or fewer: four LDS stages; more workgroups than
     # CUs: two stages, two workgroups per CU
-    assert "LDS stages                 4" in pa.Plan(c2).describe()
+    # (c2 itself goes to the kernel with the input patch resident in LDS)
+    streaming = {"planConstraints": '{"gfx950": {"patch": 0}}'}
+    assert "LDS stages                 4" in pa.Plan(c2, streaming).describe()
+    assert "input rows of the tile resident" in pa.Plan(c2).describe()
     c2_large = make_params(pa.HALF, batch=256, field=(28, 28), kernel=(3, 3),
                            ci=128, co=128, pad=1)
     assert "LDS stages                 2" in pa.Plan(c2_large).describe()
@@ -498,3 +501,40 @@ def test_plan_buffers_and_type_rules():
     with pytest.raises(MxconvError) as e:
         q.fwd(1, 1, 1)
     assert "mxconv_fwd_quarter" in e.value.message
+
+
+def test_planner_weighs_tilings_and_reports_them():
+    """The matrix-core plan lists the tilings it weighed with their estimated
+    times, picks the cheapest, and says how many CUs the launch occupies;
+    planConstraints force each of them (role of choosePlan,
+    lib/poplin/ConvPlan.cpp:502-565, and of reportPlanEstimatedCosts)."""
+    import json
+    import re
+    p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                    co=128, pad=1)
+    text = pa.Plan(p).describe()
+    assert "196 on 256 CUs (196 busy, 1 round(s) of tiles)" in text
+    rows = re.findall(r"^\s+(\*?)\s*(streaming|resident patch) (.*?)\s+(\d+)"
+                      r"\s+(\d+)\s+([\d.]+)\s+(\d+)\s+([\d.]+) us$", text,
+                      re.M)
+    assert len(rows) == 3, text
+    chosen = [r for r in rows if r[0] == "*"]
+    assert len(chosen) == 1 and chosen[0][1] == "resident patch"
+    assert float(chosen[0][7]) == min(float(r[7]) for r in rows)
+    # a layer of many tiles: two streaming workgroups per CU win
+    big = make_params(pa.HALF, batch=256, field=(14, 14), kernel=(3, 3),
+                      ci=256, co=256, pad=1)
+    text = pa.Plan(big).describe()
+    assert "* streaming 128 x 128, 2 stages" in text
+    assert "784 on 256 CUs (256 busy, 4 round(s) of tiles)" in text
+
+    def forced(**kw):
+        return pa.Plan(p, {"planConstraints":
+                           json.dumps({"gfx950": kw})}).describe()
+    assert "resident" not in forced(patch=0)
+    assert "LDS stages                 4" in forced(patch=0)
+    assert "* resident patch 64 x 128" in forced(patch=1, blockM=64)
+    assert "392 on 256 CUs (256 busy, 2 round(s)" in forced(patch=1,
+                                                             blockM=64)
+    assert "* resident patch 128 x 128" in forced(patch=1)
+    assert "LDS stages                 2" in forced(stages=2)
