@@ -297,8 +297,11 @@ mxconv_status mxconv_fwd(const mxconv_plan *plan, const void *in,
  * channels are padded - comes from a buffer of 32 MiB built into the library,
  * one per GPU.  No counterpart in the reference (Poplar owns all memory
  * there).  Returns MXCONV_WORKSPACE_TOO_SMALL for a plan whose workspace
- * exceeds the buffer; allocates nothing.  All calls on one GPU share the
- * buffer: calls that overlap in time on one GPU race. */
+ * exceeds the buffer; allocates nothing.  The first call on a GPU looks up
+ * the buffer's address there, at which point the HIP runtime may load the
+ * library's device data: make that call once at set-up, outside any capture.
+ * All calls on one GPU share the buffer: calls that overlap in time on one
+ * GPU race. */
 mxconv_status mxconv_fwd_static_scratch(const mxconv_plan *plan,
                                         const void *in,
                                         const void *weights_packed,

@@ -58,6 +58,7 @@ constexpr uint32_t kInvalid = 0x40000000u;
 
 struct PatchArgs {
   uint32_t M, mTiles, nTiles, groups;
+  uint32_t tileM; // output pixels per tile
   uint32_t outW, outH;
   uint32_t rowsPerImage; // patch rows per image: outH + (kH - 1) * dilH
   uint32_t inH;
@@ -82,6 +83,156 @@ struct PatchArgs {
 template <int RB, class OutT> constexpr int patchEpilogueBytes() {
   return kPatchWaves * (RB / 2) * kTN * 4 * 1024 +
          32 * RB * (kPatchBN * int(sizeof(OutT)) + 16);
+}
+
+/// The output pixels [m0, mLast] of a tile and the patch rows they read: rows
+/// [firstRow, firstRow + rows) of the sequence "image 0's rowsPerImage padded
+/// rows, image 1's, ...".
+struct TileSpan {
+  uint32_t m0, mLast, image0, firstRow, rows;
+};
+
+__device__ __forceinline__ TileSpan tileSpan(const PatchArgs &a,
+                                             uint32_t mTile) {
+  TileSpan s;
+  s.m0 = mTile * a.tileM;
+  s.mLast = (s.m0 + a.tileM < a.M ? s.m0 + a.tileM : a.M) - 1;
+  const uint32_t q0 = a.divOutW(s.m0);
+  s.image0 = a.divOutH(q0);
+  s.firstRow = s.image0 * a.rowsPerImage + (q0 - s.image0 * a.outH);
+  const uint32_t qL = a.divOutW(s.mLast), imageL = a.divOutH(qL);
+  s.rows = imageL * a.rowsPerImage + (qL - imageL * a.outH) +
+           (a.rowsPerImage - a.outH) + 1 - s.firstRow;
+  return s;
+}
+
+/// LDS byte of output pixel m's tap (0, 0) in slice 0 of the patch.
+__device__ __forceinline__ uint32_t patchByteOf(const PatchArgs &a,
+                                                const TileSpan &s, uint32_t m) {
+  m = m < s.mLast ? m : s.mLast;
+  const uint32_t q = a.divOutW(m), ow = m - q * a.outW;
+  const uint32_t image = a.divOutH(q), oh = q - image * a.outH;
+  return (image * a.rowsPerImage + oh - s.firstRow) * a.rowPitch +
+         ow * kPixelPitch;
+}
+
+/// Loads the patch of a tile, all waves together.  Column blocks of all
+/// slices, slice 0 first, are dealt out to the waves in turn.  Slice 0 is what
+/// the k loop waits for: its loads go out before anything else, then
+/// `between()` runs (the first weight loads - WEIGHT_LOADS of them per wave -
+/// and address arithmetic, which fill the wait), then the wave waits for its
+/// part of slice 0 and meets the others at a barrier; the later slices' loads
+/// follow and are waited for inside the k loop.
+template <int WEIGHT_LOADS, class Between, class Behind>
+__device__ __forceinline__ void
+loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
+          int lane, uint32_t g, const TileSpan &span, Between &&between,
+          Behind &&behind) {
+  // Patch row `lane`: where its input row starts, from the first image the
+  // tile reads (32-bit offsets), or kInvalid for a row of padding.  A load
+  // adds the lane's own offset, itself kInvalid for padding columns: any sum
+  // with a kInvalid in it lies beyond the buffer, which the range check
+  // limits to kInvalid bytes, and reads as zeros.
+  uint32_t rowBase;
+  {
+    const uint32_t r = span.firstRow + lane;
+    const uint32_t image = a.divRowsPerImage(r);
+    const uint32_t ih = r - image * a.rowsPerImage - uint32_t(a.padH);
+    rowBase = ih - a.loH < a.spanH
+                  ? ((image - span.image0) * a.inH + ih) * a.inRowBytes +
+                        g * a.ciBytes
+                  : kInvalid;
+  }
+  const uint64_t skipped = uint64_t(span.image0) * a.imageBytes;
+  const uint64_t left = a.inBytes - skipped;
+  const __amdgpu_buffer_rsrc_t inBuf =
+      bufferOf(in + skipped, uint32_t(left < kInvalid ? left : kInvalid));
+  const uint32_t rows = span.rows;
+  // One wave loads column block q (units 64 q .. 64 q + 63 of every patch
+  // row: chunk u % 9 of the pixel in padded column u / 9) of a slice.
+  auto loadColumns = [&](uint32_t slice, uint32_t q) {
+    const uint32_t u = q * 64 + lane;
+    const uint32_t col = u / kPixelUnits, c = u - col * kPixelUnits;
+    const uint32_t iw = col - uint32_t(a.padW);
+    const uint32_t laneOff =
+        c < 8 && iw - a.loW < a.spanW ? iw * a.pixelBytes + c * 16 : kInvalid;
+    // (the last block of a row is a partial one: lanes beyond it write
+    // nothing)
+    if (u < a.rowUnits) {
+      char *dst = lds + slice * a.sliceBytes + q * 1024;
+      auto loadRow = [&](uint32_t row) {
+        const uint32_t base = __builtin_amdgcn_readlane(rowBase, row);
+        loadToLds(inBuf, (LdsPtr)dst, laneOff + base, slice * 128);
+        dst += a.rowPitch;
+      };
+      // (four at a time: a taken branch costs as much as a load)
+      uint32_t row = 0;
+      for (; row + 4 <= rows; row += 4) {
+        loadRow(row), loadRow(row + 1), loadRow(row + 2), loadRow(row + 3);
+      }
+      for (; row < rows; ++row)
+        loadRow(row);
+    }
+  };
+  // A wave with no block of slice 0 issues its first block of a later slice
+  // right away (behind `between`, so that slice 0 gets ahead); the others do
+  // so after the barrier.
+  const uint32_t blocks = a.slices * a.rowLoads;
+  uint32_t next = wave;
+  for (; next < a.rowLoads; next += kPatchWaves)
+    loadColumns(0, next);
+  const bool early = uint32_t(wave) >= a.rowLoads;
+  between();
+  if (early) {
+    if (next < blocks) {
+      const uint32_t s = a.divRowLoads(next);
+      loadColumns(s, next - s * a.rowLoads);
+      next += kPatchWaves;
+    }
+  } else {
+    // slice 0 is in LDS once all but the weight loads have landed
+    MXK_WAIT_VMCNT(WEIGHT_LOADS);
+  }
+  __builtin_amdgcn_s_barrier();
+  behind();
+  for (; next < blocks; next += kPatchWaves) {
+    const uint32_t s = a.divRowLoads(next);
+    loadColumns(s, next - s * a.rowLoads);
+  }
+}
+
+/// The finished tile, [row][128 channels] at a pitch of kOutRow bytes in LDS,
+/// goes out as 16-byte stores, whole rows per instruction, through a buffer
+/// that ends with the last valid row: rows beyond it go nowhere.  (Streaming
+/// cache policy - the same bit as for loads: the tile is not read again
+/// here.)  ROWS: rows the tile has room for in LDS.
+template <int ROWS, class OutT>
+__device__ __forceinline__ void
+storeTile(const PatchArgs &a, const char *tileOut, OutT *__restrict__ out,
+          int t, uint32_t g, uint32_t nTile, const TileSpan &span) {
+  constexpr int kOutRow = kPatchBN * int(sizeof(OutT)) + 16;
+  constexpr int kVecsPerRow = kPatchBN * int(sizeof(OutT)) / 16;
+  constexpr int kRowsPerPass = kPatchThreads / kVecsPerRow;
+  static_assert(ROWS % kRowsPerPass == 0, "whole passes");
+  const uint32_t outRowBytes = a.outChans * sizeof(OutT);
+  const uint32_t validRows = span.mLast + 1 - span.m0;
+  const uint32_t nLeft = a.outChansPerGroup - nTile * kPatchBN;
+  const uint32_t validBytes =
+      (nLeft < uint32_t(kPatchBN) ? nLeft : kPatchBN) * sizeof(OutT);
+  const __amdgpu_buffer_rsrc_t outBuf = bufferOf(
+      out + size_t(span.m0) * a.outChans + g * a.outChansPerGroup +
+          nTile * kPatchBN,
+      (validRows - 1) * outRowBytes + validBytes);
+  const uint32_t row = t / kVecsPerRow, vecByte = (t % kVecsPerRow) * 16;
+  const uint32_t to =
+      vecByte < validBytes ? row * outRowBytes + vecByte : kOutOfRange;
+  const char *from = tileOut + row * kOutRow + vecByte;
+#pragma unroll
+  for (int pass = 0; pass != ROWS / kRowsPerPass; ++pass)
+    __builtin_amdgcn_raw_buffer_store_b128(
+        *reinterpret_cast<const uintx4 *>(from +
+                                          pass * kRowsPerPass * kOutRow),
+        outBuf, to, pass * kRowsPerPass * outRowBytes, kStreamingLoad);
 }
 
 template <int EB> struct PatchMma;
@@ -147,8 +298,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
   const uint32_t nTile = tile - overN * a.nTiles;
   const uint32_t g = a.divMTiles(overN);
   const uint32_t mTile = overN - g * a.mTiles;
-  const uint32_t m0 = mTile * BM;
-  const uint32_t mLast = (m0 + BM < a.M ? m0 + BM : a.M) - 1;
+  const TileSpan span = tileSpan(a, mTile);
 
   // The weights of this wave's 32 kTN channels: per k-step and K half 2 KB per
   // 32 channels, lane l's two 16-byte operands at 16 l and 1024 + 16 l; the
@@ -172,108 +322,23 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
     wOff += kStepBytes;
   };
 
-  // The patch: rows [firstRow, firstRow + rows) of the sequence "image 0's
-  // rowsPerImage padded rows, image 1's, ...".
-  const uint32_t q0 = a.divOutW(m0), image0 = a.divOutH(q0);
-  const uint32_t firstRow = image0 * a.rowsPerImage + (q0 - image0 * a.outH);
-  const uint32_t qL = a.divOutW(mLast), imageL = a.divOutH(qL);
-  const uint32_t rows = imageL * a.rowsPerImage + (qL - imageL * a.outH) +
-                        (a.rowsPerImage - a.outH) + 1 - firstRow;
-  // Per row block: the LDS byte of the lane's pixel (tap (0, 0), slice 0) and
-  // of the first chunk this lane reads of a k-step.  (Worked out while the
-  // first loads are in flight.)
+  // Per row block: the LDS byte of the first chunk this lane reads of a
+  // k-step, at tap (0, 0) of slice 0.  (Worked out while the first loads are
+  // in flight.)
   uint32_t pixelByte[RB];
-  auto pixelBytes = [&] {
-#pragma unroll
-    for (int i = 0; i != RB; ++i) {
-      uint32_t m = m0 + i * 32 + (lane & 31);
-      m = m < a.M ? m : a.M - 1;
-      const uint32_t q = a.divOutW(m), ow = m - q * a.outW;
-      const uint32_t image = a.divOutH(q), oh = q - image * a.outH;
-      pixelByte[i] = (image * a.rowsPerImage + oh - firstRow) * a.rowPitch +
-                     ow * kPixelPitch + Mma::laneByte(grp, lane >> 5);
-    }
-  };
-  {
-    // Patch row `lane`: where its input row starts, from the first image the
-    // tile reads (32-bit offsets), or kInvalid for a row of padding.  A load
-    // adds the lane's own offset, itself kInvalid for padding columns: any
-    // sum with a kInvalid in it lies beyond the buffer, which the range check
-    // limits to kInvalid bytes, and reads as zeros.
-    uint32_t rowBase;
-    {
-      const uint32_t r = firstRow + lane;
-      const uint32_t image = a.divRowsPerImage(r);
-      const uint32_t ih = r - image * a.rowsPerImage - uint32_t(a.padH);
-      rowBase = ih - a.loH < a.spanH
-                    ? ((image - image0) * a.inH + ih) * a.inRowBytes +
-                          g * a.ciBytes
-                    : kInvalid;
-    }
-    const uint64_t skipped = uint64_t(image0) * a.imageBytes;
-    const uint64_t left = a.inBytes - skipped;
-    const __amdgpu_buffer_rsrc_t inBuf =
-        bufferOf(in + skipped, uint32_t(left < kInvalid ? left : kInvalid));
-    // One wave loads column block q (units 64 q .. 64 q + 63 of every patch
-    // row: chunk u % 9 of the pixel in padded column u / 9) of a slice.
-    auto loadColumns = [&](uint32_t slice, uint32_t q) {
-      const uint32_t u = q * 64 + lane;
-      const uint32_t col = u / kPixelUnits, c = u - col * kPixelUnits;
-      const uint32_t iw = col - uint32_t(a.padW);
-      const uint32_t laneOff =
-          c < 8 && iw - a.loW < a.spanW ? iw * a.pixelBytes + c * 16 : kInvalid;
-      // (the last block of a row is a partial one: lanes beyond it write
-      // nothing)
-      if (u < a.rowUnits) {
-        char *dst = lds + slice * a.sliceBytes + q * 1024;
-        auto loadRow = [&](uint32_t row) {
-          const uint32_t base = __builtin_amdgcn_readlane(rowBase, row);
-          loadToLds(inBuf, (LdsPtr)dst, laneOff + base, slice * 128);
-          dst += a.rowPitch;
-        };
-        // (four at a time: a taken branch costs as much as a load)
-        uint32_t row = 0;
-        for (; row + 4 <= rows; row += 4) {
-          loadRow(row), loadRow(row + 1), loadRow(row + 2), loadRow(row + 3);
-        }
-        for (; row < rows; ++row)
-          loadRow(row);
-      }
-    };
-    // Column blocks of all slices, slice 0 first, are dealt out to the waves
-    // in turn.  Slice 0 is what the loop waits for: its loads go out before
-    // anything else.  A wave with none of them issues its first blocks of
-    // later slices right away, too (behind the arithmetic, so that slice 0
-    // gets ahead); the others do so after the barrier.
-    const uint32_t blocks = a.slices * a.rowLoads;
-    uint32_t next = wave;
-    for (; next < a.rowLoads; next += kPatchWaves)
-      loadColumns(0, next);
-    const bool early = uint32_t(wave) >= a.rowLoads;
+  loadPatch<2 * kTN * D>(a, in, lds, wave, lane, g, span, [&] {
 #pragma unroll
     for (int u = 0; u != D; ++u)
       loadB(bf[u]);
-    pixelBytes();
+#pragma unroll
+    for (int i = 0; i != RB; ++i)
+      pixelByte[i] = patchByteOf(a, span, span.m0 + i * 32 + (lane & 31)) +
+                     Mma::laneByte(grp, lane >> 5);
     // (keeps the arithmetic above this point: it fills the wait)
 #pragma unroll
     for (int i = 0; i != RB; ++i)
       asm volatile("" ::"v"(pixelByte[i]));
-    if (early) {
-      if (next < blocks) {
-        const uint32_t s = a.divRowLoads(next);
-        loadColumns(s, next - s * a.rowLoads);
-        next += kPatchWaves;
-      }
-    } else {
-      // slice 0 is in LDS once all but the weight loads have landed
-      MXK_WAIT_VMCNT(2 * kTN * D);
-    }
-    __builtin_amdgcn_s_barrier();
-    for (; next < blocks; next += kPatchWaves) {
-      const uint32_t s = a.divRowLoads(next);
-      loadColumns(s, next - s * a.rowLoads);
-    }
-  }
+  }, [] {});
 
   floatx16 acc[RB][kTN];
 #pragma unroll
@@ -511,43 +576,382 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
         keep(std::integral_constant<int, 1>{}, std::false_type{});
     }
     __syncthreads();
-    // 16-byte stores, whole rows of the tile per instruction, through a
-    // buffer that ends with the last valid row: rows beyond M go nowhere.
-    // (Streaming cache policy - the same bit as for loads: the tile is not
-    // read again here.)
-    constexpr int kVecsPerRow = kPatchBN * int(sizeof(OutT)) / 16;
-    constexpr int kRowsPerPass = kPatchThreads / kVecsPerRow;
-    const uint32_t outRowBytes = a.outChans * sizeof(OutT);
-    const uint32_t validRows = (a.M - m0 < uint32_t(BM) ? a.M - m0 : BM);
-    const uint32_t nLeft = a.outChansPerGroup - nTile * kPatchBN;
-    const uint32_t validBytes =
-        (nLeft < uint32_t(kPatchBN) ? nLeft : kPatchBN) * sizeof(OutT);
-    const __amdgpu_buffer_rsrc_t outBuf = bufferOf(
-        out + size_t(m0) * a.outChans + g * a.outChansPerGroup +
-            nTile * kPatchBN,
-        (validRows - 1) * outRowBytes + validBytes);
-    const uint32_t row = t / kVecsPerRow, vecByte = (t % kVecsPerRow) * 16;
-    const uint32_t to =
-        vecByte < validBytes ? row * outRowBytes + vecByte : kOutOfRange;
-    const char *from = tileOut + row * kOutRow + vecByte;
+    storeTile<BM>(a, tileOut, out, t, g, nTile, span);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The same kernel on 16-pixel MFMA blocks, for tiles of any height up to 112
+// pixels: a layer of M pixels is cut into as many equal tiles as there are
+// CUs (the 25 088 pixels of a 32 x 28 x 28 layer: 256 tiles of 98 instead of
+// 196 of 128), and seven 16-row blocks cover the tile with less padding than
+// four 32-row ones would.  Differences from the kernel above:
+//   - MFMA 16x16x32 (fp16) / 16x16x128 (fp8): a wave's 32 channels are two
+//     column blocks, so an A operand read from LDS feeds two MFMAs;
+//   - the two waves of a SIMD split K by k-step parity (wave grp takes steps
+//     grp, grp + 2, ...) - an fp8 MFMA spans a whole 128-byte k-step;
+//   - packed weights: [group][32 channels][k-step][4 operands][lane][16 B],
+//     operand (u, c) = K unit u (64 bytes of K), column block c for fp16;
+//     (c, r) = column block c, 16-byte half r of the lane's 32 bytes for fp8;
+//     lane l holds channel 16 c + l % 16 and the K bytes the A side's lane l
+//     reads (16 (l / 16) of the unit; 32 (l / 16) + 16 r of the step).
+// ---------------------------------------------------------------------------
+constexpr int kAhead16 = 2; // own k-steps the weight loads run ahead
+constexpr int kBlocks16 = 7;              // 16-row blocks per tile
+constexpr int kRows16 = 16 * kBlocks16;   // pixels a tile has room for
+constexpr int kKeep16 = (kBlocks16 + 1) / 2; // blocks K half 0's wave finishes
+
+template <int EB> struct PatchMma16;
+template <> struct PatchMma16<2> {
+  static constexpr int kUnits = 2; // MFMA K = 32 halves: two per k-step
+  static constexpr int kReads = 1; // 16-byte operands per lane and MFMA
+  static __device__ __forceinline__ int laneByte(int quarter) {
+    return quarter * 16;
+  }
+  template <int FA, int FB>
+  static __device__ __forceinline__ void
+  mul(const uintx4 (&b)[kReads], const uintx4 (&x)[kReads], floatx4 &acc) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+        __builtin_bit_cast(half8, b[0]), __builtin_bit_cast(half8, x[0]), acc,
+        0, 0, 0);
+  }
+};
+template <> struct PatchMma16<1> {
+  static constexpr int kUnits = 1; // MFMA K = 128 bytes: the k-step
+  static constexpr int kReads = 2;
+  static __device__ __forceinline__ int laneByte(int quarter) {
+    return quarter * 32;
+  }
+  template <int FA, int FB>
+  static __device__ __forceinline__ void
+  mul(const uintx4 (&b)[kReads], const uintx4 (&x)[kReads], floatx4 &acc) {
+    const intx8 bb{int(b[0].x), int(b[0].y), int(b[0].z), int(b[0].w),
+                   int(b[1].x), int(b[1].y), int(b[1].z), int(b[1].w)};
+    const intx8 xx{int(x[0].x), int(x[0].y), int(x[0].z), int(x[0].w),
+                   int(x[1].x), int(x[1].y), int(x[1].z), int(x[1].w)};
+    acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bb, xx, acc, FB, FA,
+                                                           0, 0, 0, 0);
+  }
+};
+
+/// D: k-steps of its own (every second one) a wave's weight loads run ahead.
+template <int EB, int FA, int FB, int D, class OutT>
+__global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
+    const PatchArgs a, const char *__restrict__ in, const char *__restrict__ w,
+    const OutT *__restrict__ bias, OutT *__restrict__ out, float scale) {
+  static_assert(kTN == 1 && D % 2 == 0 && 64 % D == 0, "");
+  constexpr int RB = kBlocks16;
+  extern __shared__ __align__(16) char lds[];
+  using Mma = PatchMma16<EB>;
+  constexpr int kUnits = Mma::kUnits, kReads = Mma::kReads;
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int grp = wave / kWavesN, wn = wave % kWavesN;
+
+  const uint32_t tile = xcdSwizzle(blockIdx.x, gridDim.x);
+  const uint32_t overN = a.divNTiles(tile);
+  const uint32_t nTile = tile - overN * a.nTiles;
+  const uint32_t g = a.divMTiles(overN);
+  const uint32_t mTile = overN - g * a.mTiles;
+  const TileSpan span = tileSpan(a, mTile);
+
+  // This wave's k-steps: grp, grp + 2, ... - `own` of them (at least one: the
+  // kernel has two taps or more).  Their weights: 4 KB per step, lane l's four
+  // operands 1 KB apart; the buffer ends with the wave's last step, so the
+  // loads that run ahead beyond it read zeros.
+  const uint32_t own = (a.kSteps + 1 - grp) >> 1;
+  const uint32_t waveBlock = (g * a.nTiles + nTile) * kWavesN + wn;
+  const __amdgpu_buffer_rsrc_t wBuf =
+      bufferOf(w + (size_t(waveBlock) * a.kSteps + grp) * 4096,
+               (own - 1) * 8192 + 4096);
+  uint32_t wOff = lane * 16;
+  uintx4 bf[D][kUnits][2][kReads];
+  auto loadB = [&](uintx4(&dst)[kUnits][2][kReads]) {
 #pragma unroll
-    for (int pass = 0; pass != BM / kRowsPerPass; ++pass)
-      __builtin_amdgcn_raw_buffer_store_b128(
-          *reinterpret_cast<const uintx4 *>(from +
-                                            pass * kRowsPerPass * kOutRow),
-          outBuf, to, pass * kRowsPerPass * outRowBytes, kStreamingLoad);
+    for (int u = 0; u != kUnits; ++u)
+#pragma unroll
+      for (int c = 0; c != 2; ++c)
+#pragma unroll
+        for (int r = 0; r != kReads; ++r)
+          dst[u][c][r] = __builtin_bit_cast(
+              uintx4,
+              __builtin_amdgcn_raw_buffer_load_b128(
+                  wBuf, wOff + ((u * 2 + c) * kReads + r) * 1024, 0, 0));
+    wOff += 8192;
+  };
+
+  // Per row block: the LDS byte of the first chunk this lane reads of a
+  // k-step, at tap (0, 0) of slice 0.
+  uint32_t pixelByte[RB];
+  // (the first step's weights before the barrier, the others behind it: the
+  // vector memory path is what bounds the time to the barrier)
+  constexpr int kFirst = 1;
+  loadPatch<4 * kFirst>(a, in, lds, wave, lane, g, span, [&] {
+#pragma unroll
+    for (int u = 0; u != kFirst; ++u)
+      loadB(bf[u]);
+#pragma unroll
+    for (int i = 0; i != RB; ++i)
+      pixelByte[i] = patchByteOf(a, span, span.m0 + i * 16 + (lane & 15)) +
+                     Mma::laneByte(lane >> 4);
+#pragma unroll
+    for (int i = 0; i != RB; ++i)
+      asm volatile("" ::"v"(pixelByte[i]));
+  }, [&] {
+#pragma unroll
+    for (int u = kFirst; u != D; ++u)
+      loadB(bf[u]);
+  });
+
+  floatx4 acc[RB][2];
+#pragma unroll
+  for (int i = 0; i != RB; ++i)
+#pragma unroll
+    for (int c = 0; c != 2; ++c)
+      acc[i][c] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // Own step j is k-step kt = 2 j + grp = slice * taps + tap; its A operands
+  // sit at pixelByte + tapByte.  The offsets of 64 own steps at a time are
+  // kept one per lane: lane l holds own step tableBase + 1 + l's, with bit 31
+  // set on the wave's first step in a slice (tap 0 or 1).
+  uint32_t tapTable = 0, tableBase = 0;
+  auto fillTable = [&] {
+    const uint32_t kt = 2 * (tableBase + 1 + lane) + grp;
+    const uint32_t slice = a.divTaps(kt), tap = kt - slice * a.taps;
+    const uint32_t kh = a.divKW(tap), kw = tap - kh * a.kW;
+    tapTable = (slice * a.sliceBytes + kh * a.tapRowBytes +
+                kw * a.tapColBytes) |
+               (tap < 2 ? 0x80000000u : 0u);
+  };
+  fillTable();
+  // (own step 0 is tap `grp` of slice 0)
+  uint32_t tapByte;
+  {
+    const uint32_t kh = a.divKW(uint32_t(grp)), kw = uint32_t(grp) - kh * a.kW;
+    tapByte = kh * a.tapRowBytes + kw * a.tapColBytes;
+  }
+  struct Operands {
+    uintx4 x[RB][kReads];
+  };
+  auto readA = [&](Operands &o, uint32_t at) {
+#pragma unroll
+    for (int i = 0; i != RB; ++i)
+#pragma unroll
+      for (int r = 0; r != kReads; ++r)
+        o.x[i][r] = *reinterpret_cast<const uintx4 *>(lds + pixelByte[i] + at +
+                                                      16 * r);
+  };
+  auto multiply = [&](const uintx4(&b)[2][kReads], const Operands &o) {
+#pragma unroll
+    for (int i = 0; i != RB; ++i)
+#pragma unroll
+      for (int c = 0; c != 2; ++c)
+        Mma::template mul<FA, FB>(b[c], o.x[i], acc[i][c]);
+  };
+  // MFMAs and the LDS reads of the next unit in turn (a wave issues in order
+  // and an MFMA behind another waits for the pipe: what stands between two
+  // of them costs nothing).
+  auto interleave = [&] {
+    __builtin_amdgcn_sched_group_barrier(0x002, RB, 0);
+#pragma unroll
+    for (int k = 0; k != RB * kReads; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 / kReads, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+  };
+  // One own step: kUnits units of MFMAs; `first` holds unit 0's operands and
+  // gets the next step's on the way out when the step has two units, else
+  // `second` does.  GUARD: the steps behind the last whole group of D.
+  auto step = [&](auto guard, uintx4(&b)[kUnits][2][kReads], Operands &first,
+                  Operands &second, uint32_t j) {
+    constexpr bool GUARD = decltype(guard)::value;
+    const bool more = !GUARD || j + 1 < own;
+    uint32_t nextTap = 0;
+    if (more) {
+      const uint32_t entry = __builtin_amdgcn_readlane(tapTable, j - tableBase);
+      nextTap = entry & 0x7fffffffu;
+      if (entry & 0x80000000u) {
+        // A new slice: its loads were issued before the loop, so they are
+        // older than the weight loads of the last D steps (loads complete in
+        // order); the barrier tells that the other waves' have landed too.
+        if (j >= uint32_t(D))
+          MXK_WAIT_VMCNT(4 * (D - 1));
+        else
+          MXK_WAIT_VMCNT(0);
+        __builtin_amdgcn_s_barrier();
+      }
+    }
+    if constexpr (!GUARD) {
+      if constexpr (kUnits == 2) {
+        readA(second, tapByte + 64);
+        multiply(b[0], first);
+        interleave();
+        readA(first, nextTap);
+        multiply(b[1], second);
+        interleave();
+      } else {
+        readA(second, nextTap);
+        multiply(b[0], first);
+        interleave();
+      }
+      loadB(b);
+      __builtin_amdgcn_sched_group_barrier(0x020, 4, 0);
+    } else {
+      if (j < own) {
+        if constexpr (kUnits == 2) {
+          readA(second, tapByte + 64);
+          multiply(b[0], first);
+          if (more)
+            readA(first, nextTap);
+          multiply(b[1], second);
+        } else {
+          if (more)
+            readA(second, nextTap);
+          multiply(b[0], first);
+        }
+      }
+    }
+    tapByte = nextTap;
+  };
+  Operands even, odd;
+  // (nothing but these LDS reads pending at the head of the loop, so that
+  // the waits inside it count reads)
+  MXK_WAIT_LGKMCNT0();
+  readA(even, tapByte);
+  uint32_t j = 0;
+  auto group = [&](auto guard) {
+    if (j - tableBase == 64) {
+      tableBase = j;
+      fillTable();
+    }
+#pragma unroll
+    for (int u = 0; u != D; u += 2) {
+      if constexpr (kUnits == 2) {
+        step(guard, bf[u], even, odd, j + u);
+        step(guard, bf[u + 1], even, odd, j + u + 1);
+      } else {
+        step(guard, bf[u], even, odd, j + u);
+        step(guard, bf[u + 1], odd, even, j + u + 1);
+      }
+    }
+  };
+  // (every step of a whole group has a successor to fetch for: the last
+  // steps, at least one, are left to the guarded group)
+  for (; j + D < own; j += D)
+    group(std::false_type{});
+  group(std::true_type{});
+
+  // Sum the two waves' halves of K: wave grp 0 finishes row blocks
+  // [0, kKeep16), wave grp 1 the others; each hands the other its sums of the
+  // blocks it does not finish, through LDS - beside the patch where there is
+  // room, else in its place, once everybody is done with it.
+  if (a.exchangeByte == 0)
+    __syncthreads();
+  {
+    uintx4 *exchange = reinterpret_cast<uintx4 *>(lds + a.exchangeByte);
+    constexpr int kOutRow = kPatchBN * int(sizeof(OutT)) + 16;
+    constexpr int kSlot = kKeep16 * 2; // 1 KB vectors a wave may be handed
+    char *tileOut = lds + a.tileByte;
+    auto give = [&](auto half) {
+      constexpr int G = decltype(half)::value;
+      constexpr int kFrom = G == 0 ? kKeep16 : 0;
+      constexpr int kTo = G == 0 ? RB : kKeep16;
+#pragma unroll
+      for (int i = kFrom; i != kTo; ++i)
+#pragma unroll
+        for (int c = 0; c != 2; ++c)
+          exchange[((wn * 2 + (1 - G)) * kSlot + (i - kFrom) * 2 + c) * 64 +
+                   lane] = __builtin_bit_cast(uintx4, acc[i][c]);
+    };
+    if (grp == 0)
+      give(std::integral_constant<int, 0>{});
+    else
+      give(std::integral_constant<int, 1>{});
+    __syncthreads();
+    // the lane's channels of the tile: nLane + 16 c + e, e < 4
+    const uint32_t nLane = wn * 32 + (lane >> 4) * 4;
+    char *laneOut = tileOut + (lane & 15) * kOutRow + nLane * sizeof(OutT);
+    auto keep = [&](auto half, auto biased) {
+      constexpr int G = decltype(half)::value;
+      constexpr int kFrom = G == 0 ? 0 : kKeep16;
+      constexpr int kTo = G == 0 ? kKeep16 : RB;
+      float bv[2][4] = {};
+      if constexpr (decltype(biased)::value) {
+        // (the channel count is a multiple of the output vector, so a run of
+        // four channels is inside it or outside)
+#pragma unroll
+        for (int c = 0; c != 2; ++c) {
+          const uint32_t n = nTile * kPatchBN + nLane + 16 * c;
+          const OutT *b = bias + g * a.outChansPerGroup +
+                          (n < a.outChansPerGroup ? n : 0);
+          if constexpr (sizeof(OutT) == 2) {
+            const uint2 raw = *reinterpret_cast<const uint2 *>(b);
+            const __half2 lo = __builtin_bit_cast(__half2, raw.x),
+                          hi = __builtin_bit_cast(__half2, raw.y);
+            bv[c][0] = __low2float(lo), bv[c][1] = __high2float(lo);
+            bv[c][2] = __low2float(hi), bv[c][3] = __high2float(hi);
+          } else {
+            const float4 raw = *reinterpret_cast<const float4 *>(b);
+            bv[c][0] = raw.x, bv[c][1] = raw.y, bv[c][2] = raw.z,
+            bv[c][3] = raw.w;
+          }
+        }
+      }
+      floatx4 other[kTo - kFrom][2];
+#pragma unroll
+      for (int i = kFrom; i != kTo; ++i)
+#pragma unroll
+        for (int c = 0; c != 2; ++c)
+          other[i - kFrom][c] = __builtin_bit_cast(
+              floatx4,
+              exchange[((wn * 2 + G) * kSlot + (i - kFrom) * 2 + c) * 64 +
+                       lane]);
+#pragma unroll
+      for (int i = kFrom; i != kTo; ++i)
+#pragma unroll
+        for (int c = 0; c != 2; ++c) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e != 4; ++e) {
+            v[e] = acc[i][c][e] + other[i - kFrom][c][e];
+            if constexpr (EB == 1)
+              v[e] *= scale;
+            if constexpr (decltype(biased)::value)
+              v[e] += bv[c][e];
+          }
+          storeOut4(reinterpret_cast<OutT *>(laneOut + i * 16 * kOutRow) +
+                        16 * c,
+                    v);
+        }
+    };
+    if (bias) {
+      if (grp == 0)
+        keep(std::integral_constant<int, 0>{}, std::true_type{});
+      else
+        keep(std::integral_constant<int, 1>{}, std::true_type{});
+    } else {
+      if (grp == 0)
+        keep(std::integral_constant<int, 0>{}, std::false_type{});
+      else
+        keep(std::integral_constant<int, 1>{}, std::false_type{});
+    }
+    __syncthreads();
+    storeTile<128>(a, tileOut, out, t, g, nTile, span);
   }
 }
 
 /// One element of the packed weights per thread:
 /// [group][block of kTN x 32 channels][k-step][K half][32 channels][operand j]
-/// [lane][16 bytes].
+/// [lane][16 bytes], or igemmPatch16Kernel's order of the same 4 KB per step
+/// and 32 channels.
 template <class T>
 __global__ __launch_bounds__(256) void packPatchWeightsKernel(
     const T *__restrict__ src, T *__restrict__ dst, uint32_t co, uint32_t ci,
     uint32_t taps, uint32_t blocks, uint32_t kSteps, uint32_t packedTaps,
     uint64_t total, bool chansTransposed, bool selected,
-    IgemmTapSelection select) {
+    IgemmTapSelection select, bool blocks16) {
   constexpr uint32_t kVec = 16 / sizeof(T), kSlice = 128 / sizeof(T);
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
@@ -562,9 +966,21 @@ __global__ __launch_bounds__(256) void packPatchWeightsKernel(
   const uint32_t block =
       uint32_t(rest / kSteps % (blocks / kTN)) * kTN + c32;
   const uint64_t g = rest / kSteps / (blocks / kTN);
-  const uint32_t n = block * 32 + (lane & 31), h = lane >> 5;
-  const uint32_t within = sizeof(T) == 2 ? half * 32 + j * 16 + h * 8 + e
-                                         : half * 64 + h * 32 + j * 16 + e;
+  uint32_t n, within;
+  if (blocks16) {
+    // igemmPatch16Kernel: operand `half * 2 + j` of the step is (K unit,
+    // column block) for fp16 and (column block, half of the lane's 32 bytes)
+    // for fp8; lane = (K quarter, channel of the column block)
+    const uint32_t quarter = lane >> 4;
+    n = block * 32 + (sizeof(T) == 2 ? j : half) * 16 + (lane & 15);
+    within = sizeof(T) == 2 ? half * 32 + quarter * 8 + e
+                            : quarter * 32 + j * 16 + e;
+  } else {
+    const uint32_t h = lane >> 5;
+    n = block * 32 + (lane & 31);
+    within = sizeof(T) == 2 ? half * 32 + j * 16 + h * 8 + e
+                            : half * 64 + h * 32 + j * 16 + e;
+  }
   const uint32_t slice = kt / packedTaps;
   uint32_t tap = kt % packedTaps;
   const uint32_t c = slice * kSlice + within;
@@ -627,9 +1043,12 @@ bool patchShape(const IgemmDesc &d, int inType, int outType, PatchShape &s) {
       d.strideW != 1 || d.inDilH != 1 || d.inDilW != 1 || d.outFullH != 0 ||
       d.outFullW != 0 || d.outTransposed || d.noTaps || d.splitK != 1)
     return false;
-  if (d.blockM != 128 && d.blockM != 64)
+  const bool blocks16 = d.patch == 2;
+  if (blocks16 ? d.blockM == 0 || d.blockM > uint32_t(kRows16) ||
+                     uint64_t(d.kH) * d.kW < 2 || kTN != 1
+               : d.blockM != 128 && d.blockM != 64)
     return false;
-  s.rb = d.blockM / 32;
+  s.rb = blocks16 ? 0 : d.blockM / 32;
   const uint64_t M = uint64_t(d.batch) * d.outH * d.outW;
   if (M == 0 || M > 0x7fffffffull || d.kH == 0 || d.kW == 0 ||
       d.inChansPerGroup == 0)
@@ -659,9 +1078,11 @@ bool patchShape(const IgemmDesc &d, int inType, int outType, PatchShape &s) {
   if (patch > uint64_t(kLdsLimit))
     return false;
   s.rowPitch = uint32_t(pitch);
-  const uint64_t exchange = uint64_t(kPatchWaves) * (s.rb / 2) * kTN * 4 * 1024;
-  const uint64_t tile =
-      32 * s.rb * (kPatchBN * (outType == kHalf ? 2 : 4) + 16);
+  const uint64_t exchange =
+      blocks16 ? uint64_t(kPatchWaves) * kKeep16 * 2 * 1024
+               : uint64_t(kPatchWaves) * (s.rb / 2) * kTN * 4 * 1024;
+  const uint64_t tile = (blocks16 ? 128 : 32 * s.rb) *
+                        (kPatchBN * (outType == kHalf ? 2 : 4) + 16);
   const uint64_t patchEnd = (patch + 1023) / 1024 * 1024;
   // Beside the patch where there is room (the waves then hand over their
   // sums as they finish, without waiting for the others to leave the patch);
@@ -720,6 +1141,21 @@ template <int EB, int FA, int FB, class OutT>
 hipError_t dispatchPatchShape(const PatchShape &s, const PatchArgs &a,
                               const void *in, const void *w, const void *bias,
                               void *out, float scale, hipStream_t stream) {
+  if (s.rb == 0) {
+    auto kernel = &igemmPatch16Kernel<EB, FA, FB, kAhead16, OutT>;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(kernel),
+        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
+    if (attr != hipSuccess)
+      return attr;
+    hipLaunchKernelGGL(kernel, dim3(a.mTiles * a.nTiles * a.groups),
+                       dim3(kPatchThreads), s.ldsBytes, stream, a,
+                       static_cast<const char *>(in),
+                       static_cast<const char *>(w),
+                       static_cast<const OutT *>(bias),
+                       static_cast<OutT *>(out), scale);
+    return hipGetLastError();
+  }
   if (s.rb == 4)
     return launchPatchKernel<EB, FA, FB, 4, 4, OutT>(a, s.ldsBytes, in, w,
                                                      bias, out, scale, stream);
@@ -780,14 +1216,14 @@ hipError_t launchPackIgemmPatchWeights(const IgemmDesc &d, int inType,
                        static_cast<uint16_t *>(dst), d.outChansPerGroup,
                        d.inChansPerGroup, sourceTaps, blocks32, kSteps,
                        packedTaps, total, chansTransposed, select != nullptr,
-                       chosen);
+                       chosen, d.patch == 2);
   else
     hipLaunchKernelGGL(packPatchWeightsKernel<uint8_t>, dim3(uint32_t(blocks)),
                        dim3(256), 0, stream, static_cast<const uint8_t *>(src),
                        static_cast<uint8_t *>(dst), d.outChansPerGroup,
                        d.inChansPerGroup, sourceTaps, blocks32, kSteps,
                        packedTaps, total, chansTransposed, select != nullptr,
-                       chosen);
+                       chosen, d.patch == 2);
   return hipGetLastError();
 }
 
@@ -800,6 +1236,7 @@ hipError_t launchIgemmPatch(const IgemmDesc &d, int inType, int outType,
     return hipErrorInvalidValue;
   PatchArgs a{};
   a.M = d.batch * d.outH * d.outW;
+  a.tileM = d.blockM;
   a.mTiles = (a.M + d.blockM - 1) / d.blockM;
   a.nTiles = (d.outChansPerGroup + 127) / 128;
   a.groups = d.groups;

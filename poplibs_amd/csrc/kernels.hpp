@@ -194,9 +194,11 @@ struct IgemmDesc {
   // and epilogue: for grids of more workgroups than CUs).  The 64-wide tile
   // always runs 3.
   uint32_t stages = 4;
-  // 1: the kernel that keeps a tile's input patch in LDS runs (unit stride,
-  // channels in whole 128-byte slices; igemmPatchTakes); the packed weights
-  // then have its layout (launchPackIgemmPatchWeights).  blockM 64 or 128.
+  // 1 or 2: the kernel that keeps a tile's input patch in LDS runs (unit
+  // stride, channels in whole 128-byte slices; igemmPatchTakes); the packed
+  // weights then have its layout (launchPackIgemmPatchWeights).  1: 32-pixel
+  // MFMA blocks, blockM 64 or 128; 2: 16-pixel MFMA blocks, blockM = pixels
+  // per tile, any number up to 112.
   uint32_t patch = 0;
 };
 /// How the kernel finds out which kernel taps of an output pixel read inside

@@ -39,7 +39,10 @@ struct PlanConstraints {
   unsigned splitK = 0;
   unsigned stages = 0; // LDS stages of the 128-wide igemm tile: 2 or 4
   /// The matrix-core kernel that keeps the input patch in LDS: -1 planner's
-  /// choice, 0 never, 1 whenever it can take the convolution.
+  /// choice, 0 never, 1 / 2 whenever it can take the convolution (1: tiles of
+  /// 128 or 64 pixels in 32-pixel MFMA blocks; 2: tiles of up to 112 pixels
+  /// in 16-pixel blocks, as many equal ones as there are CUs unless blockM
+  /// names the height).
   int patch = -1;
   /// Output tile of the depthwise kernel; 0 = planner's choice.
   unsigned tileH = 0, tileW = 0;

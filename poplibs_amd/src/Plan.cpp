@@ -7,6 +7,7 @@
 #include <cmath>
 #include <cstdio>
 #include <sstream>
+#include <vector>
 
 namespace poplin {
 
@@ -240,12 +241,19 @@ double estimateStreaming(std::size_t workgroups, std::size_t kSteps,
   return kLaunchUs + rounds * tile + (splitK > 1 ? 5.0 : 0.0);
 }
 
-/// igemmPatchKernel: 1.9 us to the first MFMA + 0.5 us reduction and stores,
-/// 0.333 us per k-step of 128 pixels (half of that for 64); one workgroup per
-/// CU, so further rounds pay their start-up in full (4.5 us instead of 2.4).
-double estimatePatch(std::size_t workgroups, std::size_t kSteps,
+/// igemmPatchKernel (mode 1): 1.9 us to the first MFMA + 0.5 us reduction and
+/// stores, 0.333 us per k-step of 128 pixels (half of that for 64); one
+/// workgroup per CU, so further rounds pay their start-up in full (4.5 us
+/// instead of 2.4).  igemmPatch16Kernel (mode 2): seven blocks of 16 pixels
+/// whatever the tile's height, 0.34 us per k-step, 1.5 us around them (2.6 us
+/// in further rounds).  Measured: 9.6 us for 256 tiles of 18 k-steps, 20.5 us
+/// for 50 k-steps, 128.6 us for 14 rounds of 18, 60 us for 4 rounds of 36.
+double estimatePatch(std::size_t workgroups, std::size_t kSteps, unsigned mode,
                      unsigned blockM) {
   const double rounds = roundsOf(workgroups, 1);
+  if (mode == 2)
+    return kLaunchUs +
+           rounds * ((rounds > 1 ? 2.6 : 1.5) + 0.34 * double(kSteps));
   const double step = blockM == 128 ? 0.333 : 0.167;
   const double fixed = rounds > 1 ? 4.5 : 2.4;
   return kLaunchUs + rounds * (fixed + step * double(kSteps));
@@ -511,12 +519,14 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     g.blockN = pc.blockN ? pc.blockN : (co <= 64 ? 64 : 128);
     const unsigned stepElems = unsigned(128 / params.inputType.size());
     g.blockK = pc.blockK ? pc.blockK : stepElems;
-    if ((g.blockM != 128 && g.blockM != 64) ||
+    const bool anyHeight = pc.patch == 2 && g.blockM >= 1 && g.blockM <= 112;
+    if ((g.blockM != 128 && g.blockM != 64 && !anyHeight) ||
         (g.blockN != 64 && g.blockN != 128) ||
         g.blockK != stepElems)
       throw poplar::invalid_option(
-          "planConstraints gfx950 tile not available: blockM must be 128, "
-          "blockN 64 or 128, blockK 32 (float), 64 (half) or 128 (quarter)");
+          "planConstraints gfx950 tile not available: blockM must be 128 (64 "
+          "with patch 1, 1 to 112 with patch 2), blockN 64 or 128, blockK 32 "
+          "(float), 64 (half) or 128 (quarter)");
     const std::size_t k = std::size_t(s.kD) * s.kH * s.kW * ciPadded;
     plan.coPadded = (co + g.blockN - 1) / g.blockN * g.blockN;
     plan.kPadded = (k + g.blockK - 1) / g.blockK * g.blockK;
@@ -709,7 +719,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         s.outW == s.inW;
     plan.pointwiseOn =
         unitWindow && ciPadded == ci && pc.kernel != "igemm" &&
-        pc.patch != 1 && !pc.blockM &&
+        pc.patch < 1 && !pc.blockM &&
         !pc.blockN && !pc.blockK &&
         mxk::pointwiseTakes(pw,
                             halfIn    ? mxk::kHalf
@@ -724,32 +734,57 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     // instead of once per tap.
     if (!plan.pointwiseOn && plan.igemmPhases.empty() &&
         !plan.paddedInputChans &&
-        (g.splitK == 1 || (pc.patch == 1 && !pc.splitK)) && pc.patch != 0 &&
+        (g.splitK == 1 || (pc.patch >= 1 && !pc.splitK)) && pc.patch != 0 &&
         !pc.blockN && !pc.blockK && !pc.stages) {
-      mxk::IgemmDesc trial = g;
-      trial.patch = 1;
-      trial.splitK = 1; // (asked for by name, it runs K whole)
       const int inId = halfIn ? mxk::kHalf : floatIn ? mxk::kFloat
                                                      : mxk::kQuarter;
       const int outId =
           params.outputType == poplar::HALF ? mxk::kHalf : mxk::kFloat;
-      // Weigh the tilings: the streaming kernel as planned above against
-      // this kernel with 128- and 64-pixel tiles, by estimated time.
-      const bool takes = mxk::igemmPatchTakes(trial, inId, outId);
       const std::size_t m = std::size_t(s.batch) * s.outH * s.outW;
       const std::size_t nTiles128 = (co + 127) / 128 * p.numConvGroups;
       const std::size_t stepBytes = 128;
       const std::size_t patchSteps =
           ciPadded * params.inputType.size() / stepBytes * s.kH * s.kW;
-      auto add = [&](const std::string &name, std::size_t workgroups,
-                     std::size_t perCU, std::size_t kSteps, double us,
-                     double rounds) {
+      // Weigh the tilings by estimated time: the streaming kernel as planned
+      // above against this kernel with tiles of 128 and 64 pixels (32-pixel
+      // MFMA blocks) and with the layer cut into as many equal tiles of at
+      // most 112 pixels as there are CUs (16-pixel blocks).
+      struct Tiling {
+        uint32_t patch, blockM;
+      };
+      std::vector<Tiling> tilings;
+      auto add = [&](const std::string &name, Tiling tiling,
+                     std::size_t workgroups, std::size_t perCU,
+                     std::size_t kSteps, double us, double rounds) {
         mxconv_plan::Candidate c;
         c.name = name, c.workgroups = workgroups, c.perCU = perCU;
         c.kSteps = kSteps, c.estimateUs = us, c.rounds = rounds;
         plan.candidates.push_back(c);
+        tilings.push_back(tiling);
         return plan.candidates.size() - 1;
       };
+      const std::size_t none = ~std::size_t(0);
+      auto addPatch = [&](uint32_t mode, uint32_t bm) -> std::size_t {
+        mxk::IgemmDesc t = g;
+        t.patch = mode, t.blockM = bm;
+        t.splitK = 1; // (asked for by name, it runs K whole)
+        if (!mxk::igemmPatchTakes(t, inId, outId))
+          return none;
+        const std::size_t tiles = (m + bm - 1) / bm * nTiles128;
+        return add("resident patch " + std::to_string(bm) + " x 128" +
+                       (mode == 2 ? ", 16-pixel blocks" : ""),
+                   Tiling{mode, bm}, tiles, 1, patchSteps,
+                   estimatePatch(tiles, patchSteps, mode, bm),
+                   roundsOf(tiles, 1));
+      };
+      // Equal tiles, one per CU; 112 pixels where that takes several rounds.
+      const std::size_t across = gfx950::numCUs / std::max<std::size_t>(
+                                                      1, nTiles128);
+      const uint32_t equalM =
+          across == 0 ? 112u
+                      : uint32_t(std::min<std::size_t>(
+                            112, std::max<std::size_t>(
+                                     16, (m + across - 1) / across)));
       const std::size_t streamTiles =
           (m + 127) / 128 * (plan.coPadded / g.blockN) * p.numConvGroups *
           g.splitK;
@@ -757,69 +792,39 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
           (plan.kPadded / g.blockK + g.splitK - 1) / g.splitK;
       const std::size_t streamPerCU = g.blockN == 64 || g.stages == 2 ? 2 : 1;
       const std::size_t iStream =
-          add("streaming " + std::to_string(g.blockM) + " x " +
-                  std::to_string(g.blockN) + ", " +
+          add("streaming 128 x " + std::to_string(g.blockN) + ", " +
                   std::to_string(g.blockN == 128 ? g.stages : 3) + " stages" +
                   (g.splitK > 1 ? ", K in " + std::to_string(g.splitK) +
                                       " parts"
                                 : ""),
-              streamTiles, streamPerCU, streamSteps,
+              Tiling{0, 128}, streamTiles, streamPerCU, streamSteps,
               estimateStreaming(streamTiles, streamSteps, streamPerCU,
                                 g.blockN, g.splitK),
               roundsOf(streamTiles, streamPerCU));
       std::size_t best = iStream;
-      if (takes && s.kH * s.kW > 1 && co > 64) {
-        for (unsigned bm : {128u, 64u}) {
-          mxk::IgemmDesc t2 = trial;
-          t2.blockM = bm;
-          if (!mxk::igemmPatchTakes(t2, inId, outId))
+      if (pc.patch >= 1) {
+        // planConstraints: whenever the kernel can, with the tile asked for
+        const uint32_t bm = pc.blockM ? pc.blockM
+                                      : pc.patch == 2 ? equalM : 128u;
+        const std::size_t i = addPatch(uint32_t(pc.patch), bm);
+        if (i != none)
+          best = i;
+      } else if (g.splitK == 1 && s.kH * s.kW > 1 && co > 64) {
+        for (Tiling t : {Tiling{1, 128}, Tiling{1, 64}, Tiling{2, equalM}}) {
+          // (a forced tile height picks among the patch tilings only)
+          if (pc.blockM && pc.blockM != t.blockM)
             continue;
-          const std::size_t tiles = (m + bm - 1) / bm * nTiles128;
-          const std::size_t i =
-              add("resident patch " + std::to_string(bm) + " x 128", tiles, 1,
-                  patchSteps, estimatePatch(tiles, patchSteps, bm),
-                  roundsOf(tiles, 1));
-          if (plan.candidates[i].estimateUs <
-              plan.candidates[best].estimateUs)
+          const std::size_t i = addPatch(t.patch, t.blockM);
+          if (i != none && plan.candidates[i].estimateUs <
+                               plan.candidates[best].estimateUs)
             best = i;
         }
-      }
-      // planConstraints: patch 1 = whenever it can, with the tile asked for
-      // (128 by default)
-      bool usePatch = takes && best != iStream;
-      if (pc.patch == 1 && takes) {
-        usePatch = true;
-        best = plan.candidates.size();
-        for (std::size_t i = 0; i != plan.candidates.size(); ++i)
-          if (plan.candidates[i].name ==
-              "resident patch " + std::to_string(trial.blockM) + " x 128")
-            best = i;
-        if (best == plan.candidates.size()) {
-          const std::size_t tiles =
-              (m + trial.blockM - 1) / trial.blockM * nTiles128;
-          best = add("resident patch " + std::to_string(trial.blockM) +
-                         " x 128",
-                     tiles, 1, patchSteps,
-                     estimatePatch(tiles, patchSteps, trial.blockM),
-                     roundsOf(tiles, 1));
-        }
-      } else if (pc.blockM && usePatch) {
-        // a forced tile height picks among the patch tilings only
-        usePatch = false;
-        for (std::size_t i = 0; i != plan.candidates.size(); ++i)
-          if (plan.candidates[i].name ==
-              "resident patch " + std::to_string(pc.blockM) + " x 128")
-            usePatch = true, best = i;
-        if (!usePatch)
-          best = iStream;
       }
       plan.candidates[best].chosen = true;
-      if (usePatch) {
-        trial.blockM = plan.candidates[best].name.find(" 64 x") !=
-                               std::string::npos
-                           ? 64
-                           : 128;
-        g = trial;
+      if (best != iStream) {
+        g.patch = tilings[best].patch;
+        g.blockM = tilings[best].blockM;
+        g.splitK = 1;
         g.blockN = 128;
         plan.workspaceBytes = 0;
         plan.coPadded = (co + 127) / 128 * 128;
@@ -930,7 +935,12 @@ std::string mxconv_plan::describe() const {
       if (g.patch)
         os << "        data path                  input rows of the tile "
               "resident in LDS, weights straight to registers; 8 waves, one "
-              "workgroup per CU\n";
+              "workgroup per CU; MFMA blocks of "
+           << (g.patch == 2
+                   ? "16 pixels, k-steps taken in turn by the two waves of a "
+                     "SIMD\n"
+                   : "32 pixels, each k-step halved between the two waves of "
+                     "a SIMD\n");
       else if (g.blockN == 128)
         os << "        LDS stages                 " << g.stages
            << (g.stages == 2 ? " (two workgroups per CU)\n"
@@ -951,7 +961,9 @@ std::string mxconv_plan::describe() const {
       if (g.patch)
         os << "        packed weights             [G=" << g.groups << "]["
            << coPadded / 32 << " blocks of 32][" << k * params.inputType.size() / 128
-           << " k-steps][2 halves][2][64 lanes][16 bytes]\n";
+           << " k-steps]"
+           << (g.patch == 2 ? "[4 operands]" : "[2 halves][2]")
+           << "[64 lanes][16 bytes]\n";
       else
         os << "        packed weights             [G=" << g.groups << "]["
            << coPadded << "][" << kPadded << "]\n";

@@ -416,7 +416,9 @@ def test_planner_choices():
     assert "input rows of the tile resident" in pa.Plan(c2).describe()
     c2_large = make_params(pa.HALF, batch=256, field=(28, 28), kernel=(3, 3),
                            ci=128, co=128, pad=1)
-    assert "LDS stages                 2" in pa.Plan(c2_large).describe()
+    assert "LDS stages                 2" in \
+        pa.Plan(c2_large, streaming).describe()
+    assert "MFMA blocks of 16 pixels" in pa.Plan(c2_large).describe()
     forced = pa.Plan(c2, {"planConstraints": '{"gfx950": {"stages": 2}}'})
     assert "LDS stages                 2" in forced.describe()
     with pytest.raises(MxconvError):
@@ -513,20 +515,25 @@ def test_planner_weighs_tilings_and_reports_them():
     p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
                     co=128, pad=1)
     text = pa.Plan(p).describe()
-    assert "196 on 256 CUs (196 busy, 1 round(s) of tiles)" in text
+    # 25 088 pixels: 256 equal tiles of 98 rather than 196 of 128
+    assert "256 on 256 CUs (256 busy, 1 round(s) of tiles)" in text
+    assert "block M x N x K            98 x 128 x 64" in text
     rows = re.findall(r"^\s+(\*?)\s*(streaming|resident patch) (.*?)\s+(\d+)"
                       r"\s+(\d+)\s+([\d.]+)\s+(\d+)\s+([\d.]+) us$", text,
                       re.M)
-    assert len(rows) == 3, text
+    assert len(rows) == 4, text
     chosen = [r for r in rows if r[0] == "*"]
     assert len(chosen) == 1 and chosen[0][1] == "resident patch"
+    assert "16-pixel blocks" in chosen[0][2]
     assert float(chosen[0][7]) == min(float(r[7]) for r in rows)
-    # a layer of many tiles: two streaming workgroups per CU win
+    # a layer of many tiles: rounds of 112-pixel tiles (measured 60 us against
+    # 68 us for two streaming workgroups per CU)
     big = make_params(pa.HALF, batch=256, field=(14, 14), kernel=(3, 3),
                       ci=256, co=256, pad=1)
     text = pa.Plan(big).describe()
-    assert "* streaming 128 x 128, 2 stages" in text
-    assert "784 on 256 CUs (256 busy, 4 round(s) of tiles)" in text
+    assert "* resident patch 112 x 128, 16-pixel blocks" in text
+    assert "896 on 256 CUs (256 busy, 4 round(s) of tiles)" in text
+    assert "streaming 128 x 128, 2 stages" in text
 
     def forced(**kw):
         return pa.Plan(p, {"planConstraints":
@@ -537,4 +544,10 @@ def test_planner_weighs_tilings_and_reports_them():
     assert "392 on 256 CUs (256 busy, 2 round(s)" in forced(patch=1,
                                                              blockM=64)
     assert "* resident patch 128 x 128" in forced(patch=1)
+    assert "196 on 256 CUs (196 busy, 1 round(s)" in forced(patch=1)
+    assert "* resident patch 98 x 128, 16-pixel blocks" in forced(patch=2)
+    assert "* resident patch 112 x 128, 16-pixel blocks" in \
+        forced(patch=2, blockM=112)
+    with pytest.raises(MxconvError):
+        forced(patch=2, blockM=113)
     assert "LDS stages                 2" in forced(stages=2)

@@ -20,11 +20,13 @@ pytestmark = pytest.mark.gpu
 FORCED = {"planConstraints": json.dumps({"gfx950": {"patch": 1}})}
 FORCED64 = {"planConstraints":
             json.dumps({"gfx950": {"patch": 1, "blockM": 64}})}
+FORCED16 = {"planConstraints": json.dumps({"gfx950": {"patch": 2}})}
 PATCH = "input patch resident in LDS"
+BLOCKS16 = "MFMA blocks of 16 pixels"
 
 
 def _run(oracle, p, seed, tol, dist="normal", bias=True, options=FORCED,
-         wscale=0.1):
+         wscale=0.1, return_plan=False):
     from gpu_helpers import quantize, run_conv
     acts, weights, biases = random_data(p, seed, dist)
     weights = weights * (1.0 if dist == "pm1" else wscale)
@@ -41,7 +43,7 @@ def _run(oracle, p, seed, tol, dist="normal", bias=True, options=FORCED,
     else:
         err = rel_l2(got, want)
         assert err <= tol, (err, p)
-    return got
+    return (got, plan) if return_plan else got
 
 
 CASES = [
@@ -91,6 +93,43 @@ def test_patch_64_row_tiles(oracle, kw):
     _run(oracle, p, 13, 1e-3, options=FORCED64, bias=False)
 
 
+def _forced16(tile_pixels):
+    return {"planConstraints": json.dumps(
+        {"gfx950": {"patch": 2, "blockM": tile_pixels}})}
+
+
+# (the pointwise case has one tap: the wave pairs of this variant take turns
+# by k-step, which wants two)
+@pytest.mark.parametrize("kw", [c for c in CASES if c["kernel"] != (1, 1)])
+def test_patch_16_pixel_blocks(oracle, kw):
+    p = make_params(pa.HALF, **kw)
+    print("case", p, flush=True)
+    _, plan = _run(oracle, p, 14, 1e-3, options=FORCED16, return_plan=True)
+    assert BLOCKS16 in plan.describe()
+
+
+@pytest.mark.parametrize("tile_pixels", [112, 98, 37, 16, 5])
+def test_patch_16_pixel_blocks_tile_heights(oracle, tile_pixels):
+    p = make_params(pa.HALF, pa.FLOAT, **CASES[1])
+    print("case", p, tile_pixels, flush=True)
+    _, plan = _run(oracle, p, 15, 0, dist="pm1",
+                   options=_forced16(tile_pixels), return_plan=True)
+    assert BLOCKS16 in plan.describe()
+    assert "block M x N x K            %d x" % tile_pixels in plan.describe()
+
+
+@pytest.mark.parametrize("kw", CASES[2:7])
+def test_patch_16_pixel_blocks_pm1_exact(oracle, kw):
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    print("case", p, flush=True)
+    _run(oracle, p, 16, 0, dist="pm1", options=FORCED16)
+
+
+def test_patch_16_pixel_blocks_refuse_one_tap():
+    p = make_params(pa.HALF, **CASES[7])
+    assert PATCH not in pa.Plan(p, FORCED16).describe()
+
+
 def test_patch_is_the_planners_choice_for_the_benchmark_layers():
     p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
                     co=128, pad=1)
@@ -98,8 +137,13 @@ def test_patch_is_the_planners_choice_for_the_benchmark_layers():
     p = make_params(pa.QUARTER, pa.HALF, batch=64, field=(14, 14),
                     kernel=(3, 3), ci=256, co=256, pad=1)
     assert PATCH in pa.Plan(p).describe()
-    # more workgroups than CUs: the streaming kernel, two workgroups per CU
+    # more workgroups than CUs: tiles of 112 pixels, several rounds of them
     p = make_params(pa.HALF, batch=256, field=(28, 28), kernel=(3, 3), ci=128,
+                    co=128, pad=1)
+    text = pa.Plan(p).describe()
+    assert BLOCKS16 in text and "block M x N x K            112 x" in text
+    # channels that do not come in whole 128-byte slices: the streaming kernel
+    p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=96,
                     co=128, pad=1)
     assert PATCH not in pa.Plan(p).describe()
     off = {"planConstraints": json.dumps({"gfx950": {"patch": 0}})}
@@ -115,23 +159,25 @@ def test_patch_forced_on_a_strided_layer_is_refused_quietly():
     assert PATCH not in pa.Plan(p, FORCED).describe()
 
 
+@pytest.mark.parametrize("options", [FORCED, FORCED16])
 @pytest.mark.parametrize("fmt_a,fmt_w", [(1, 1), (1, 0), (0, 1), (0, 0)])
-def test_patch_fp8_matches_oracle(oracle, fmt_a, fmt_w):
+def test_patch_fp8_matches_oracle(oracle, fmt_a, fmt_w, options):
     from test_fast_gpu import _fp8_case
     p = make_params(pa.QUARTER, pa.HALF, batch=5, field=(14, 14),
                     kernel=(3, 3), ci=256, co=256, pad=1)
-    got, want, plan = _fp8_case(oracle, p, 6, fmt_a, fmt_w, options=FORCED)
+    got, want, plan = _fp8_case(oracle, p, 6, fmt_a, fmt_w, options=options)
     assert PATCH in plan.describe()
     err = rel_l2(got, want)
     assert err <= 3e-2, err
     assert err <= 1e-3, err
 
 
-def test_patch_fp8_ragged(oracle):
+@pytest.mark.parametrize("options", [FORCED, FORCED16])
+def test_patch_fp8_ragged(oracle, options):
     from test_fast_gpu import _fp8_case
     p = make_params(pa.QUARTER, pa.HALF, batch=3, field=(7, 9), kernel=(3, 2),
                     ci=128, co=40, groups=2, pad=1)
-    got, want, plan = _fp8_case(oracle, p, 7, 1, 1, options=FORCED)
+    got, want, plan = _fp8_case(oracle, p, 7, 1, 1, options=options)
     assert PATCH in plan.describe()
     assert rel_l2(got, want) <= 1e-3
 
