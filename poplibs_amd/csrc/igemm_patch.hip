@@ -49,8 +49,12 @@ constexpr int kTN = PATCH_TN;
 constexpr int kWavesN = 4 / kTN;
 constexpr int kPatchWaves = 2 * kWavesN;
 constexpr int kPatchThreads = 64 * kPatchWaves;
-constexpr int kPixelUnits = 9;      // 16-byte units per pixel in the patch
-constexpr int kPixelPitch = 16 * kPixelUnits;
+// 16-byte units per pixel in the patch: 8 of channels and padding that keeps
+// the MFMA operand reads free of bank conflicts - 144 bytes from pixel to
+// pixel where 32 lanes read 32 pixels (igemmPatchKernel), 160 bytes where 16
+// lanes read 16 (igemmPatch16Kernel; measured: 246 bytes per clock against
+// 171 at 144).
+constexpr int kPixelUnits = 9, kPixelUnits16 = 10;
 constexpr int kPatchBN = 128;
 constexpr int kLdsLimit = 160 * 1024;
 // An offset no buffer the kernel makes reaches: marks padding rows / columns.
@@ -107,13 +111,14 @@ __device__ __forceinline__ TileSpan tileSpan(const PatchArgs &a,
 }
 
 /// LDS byte of output pixel m's tap (0, 0) in slice 0 of the patch.
+template <int UNITS>
 __device__ __forceinline__ uint32_t patchByteOf(const PatchArgs &a,
                                                 const TileSpan &s, uint32_t m) {
   m = m < s.mLast ? m : s.mLast;
   const uint32_t q = a.divOutW(m), ow = m - q * a.outW;
   const uint32_t image = a.divOutH(q), oh = q - image * a.outH;
   return (image * a.rowsPerImage + oh - s.firstRow) * a.rowPitch +
-         ow * kPixelPitch;
+         ow * (16 * UNITS);
 }
 
 /// Loads the patch of a tile, all waves together.  Column blocks of all
@@ -123,7 +128,7 @@ __device__ __forceinline__ uint32_t patchByteOf(const PatchArgs &a,
 /// and address arithmetic, which fill the wait), then the wave waits for its
 /// part of slice 0 and meets the others at a barrier; the later slices' loads
 /// follow and are waited for inside the k loop.
-template <int WEIGHT_LOADS, class Between, class Behind>
+template <int WEIGHT_LOADS, int UNITS, class Between, class Behind>
 __device__ __forceinline__ void
 loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
           int lane, uint32_t g, const TileSpan &span, Between &&between,
@@ -149,10 +154,11 @@ loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
       bufferOf(in + skipped, uint32_t(left < kInvalid ? left : kInvalid));
   const uint32_t rows = span.rows;
   // One wave loads column block q (units 64 q .. 64 q + 63 of every patch
-  // row: chunk u % 9 of the pixel in padded column u / 9) of a slice.
+  // row: chunk u % UNITS of the pixel in padded column u / UNITS) of a
+  // slice.
   auto loadColumns = [&](uint32_t slice, uint32_t q) {
     const uint32_t u = q * 64 + lane;
-    const uint32_t col = u / kPixelUnits, c = u - col * kPixelUnits;
+    const uint32_t col = u / UNITS, c = u - col * UNITS;
     const uint32_t iw = col - uint32_t(a.padW);
     const uint32_t laneOff =
         c < 8 && iw - a.loW < a.spanW ? iw * a.pixelBytes + c * 16 : kInvalid;
@@ -326,13 +332,14 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
   // k-step, at tap (0, 0) of slice 0.  (Worked out while the first loads are
   // in flight.)
   uint32_t pixelByte[RB];
-  loadPatch<2 * kTN * D>(a, in, lds, wave, lane, g, span, [&] {
+  loadPatch<2 * kTN * D, kPixelUnits>(a, in, lds, wave, lane, g, span, [&] {
 #pragma unroll
     for (int u = 0; u != D; ++u)
       loadB(bf[u]);
 #pragma unroll
     for (int i = 0; i != RB; ++i)
-      pixelByte[i] = patchByteOf(a, span, span.m0 + i * 32 + (lane & 31)) +
+      pixelByte[i] =
+          patchByteOf<kPixelUnits>(a, span, span.m0 + i * 32 + (lane & 31)) +
                      Mma::laneByte(grp, lane >> 5);
     // (keeps the arithmetic above this point: it fills the wait)
 #pragma unroll
@@ -594,7 +601,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
 //     operand (u, c) = K unit u (64 bytes of K), column block c for fp16;
 //     (c, r) = column block c, 16-byte half r of the lane's 32 bytes for fp8;
 //     lane l holds channel 16 c + l % 16 and the K bytes the A side's lane l
-//     reads (16 (l / 16) of the unit; 32 (l / 16) + 16 r of the step).
+//     reads (16 (l / 16) of the unit; 64 r + 16 (l / 16) of the step).
 // ---------------------------------------------------------------------------
 constexpr int kAhead16 = 2; // own k-steps the weight loads run ahead
 constexpr int kBlocks16 = 7;              // 16-row blocks per tile
@@ -618,9 +625,12 @@ template <> struct PatchMma16<2> {
 };
 template <> struct PatchMma16<1> {
   static constexpr int kUnits = 1; // MFMA K = 128 bytes: the k-step
+  // Two 16-byte reads per lane, 64 bytes apart: each of them then has the
+  // fp16 read's pattern (which K bytes a lane multiplies does not matter as
+  // long as the weights are packed alike).
   static constexpr int kReads = 2;
   static __device__ __forceinline__ int laneByte(int quarter) {
-    return quarter * 32;
+    return quarter * 16;
   }
   template <int FA, int FB>
   static __device__ __forceinline__ void
@@ -688,13 +698,14 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
   // (the first step's weights before the barrier, the others behind it: the
   // vector memory path is what bounds the time to the barrier)
   constexpr int kFirst = 1;
-  loadPatch<4 * kFirst>(a, in, lds, wave, lane, g, span, [&] {
+  loadPatch<4 * kFirst, kPixelUnits16>(a, in, lds, wave, lane, g, span, [&] {
 #pragma unroll
     for (int u = 0; u != kFirst; ++u)
       loadB(bf[u]);
 #pragma unroll
     for (int i = 0; i != RB; ++i)
-      pixelByte[i] = patchByteOf(a, span, span.m0 + i * 16 + (lane & 15)) +
+      pixelByte[i] = patchByteOf<kPixelUnits16>(
+                         a, span, span.m0 + i * 16 + (lane & 15)) +
                      Mma::laneByte(lane >> 4);
 #pragma unroll
     for (int i = 0; i != RB; ++i)
@@ -741,7 +752,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
 #pragma unroll
       for (int r = 0; r != kReads; ++r)
         o.x[i][r] = *reinterpret_cast<const uintx4 *>(lds + pixelByte[i] + at +
-                                                      16 * r);
+                                                      64 * r);
   };
   auto multiply = [&](const uintx4(&b)[2][kReads], const Operands &o) {
 #pragma unroll
@@ -974,7 +985,7 @@ __global__ __launch_bounds__(256) void packPatchWeightsKernel(
     const uint32_t quarter = lane >> 4;
     n = block * 32 + (sizeof(T) == 2 ? j : half) * 16 + (lane & 15);
     within = sizeof(T) == 2 ? half * 32 + quarter * 8 + e
-                            : quarter * 32 + j * 16 + e;
+                            : j * 64 + quarter * 16 + e;
   } else {
     const uint32_t h = lane >> 5;
     n = block * 32 + (lane & 31);
@@ -1062,14 +1073,15 @@ bool patchShape(const IgemmDesc &d, int inType, int outType, PatchShape &s) {
   s.taps = d.kH * d.kW;
   s.kSteps = s.slices * s.taps;
   const uint64_t cols = uint64_t(d.outW) + uint64_t(d.kW - 1) * d.dilW;
-  s.rowLoads = uint32_t((cols * kPixelUnits + 63) / 64);
-  // Consecutive pixels sit 144 bytes apart, which spreads the 16-byte reads
-  // of 16 lanes over all 64 banks; the pitch of the rows continues that
+  const uint64_t units = blocks16 ? kPixelUnits16 : kPixelUnits;
+  s.rowLoads = uint32_t((cols * units + 63) / 64);
+  // The pitch from pixel to pixel spreads the 16-byte reads of an MFMA
+  // operand over all 64 banks; the pitch of the rows continues that
   // progression (modulo the 256 bytes of the banks) from the last pixel of an
   // output row to the first of the next.
   const uint64_t pitch =
-      uint64_t(d.outW) * kPixelPitch +
-      ((cols - d.outW) * kPixelPitch + 255) / 256 * 256;
+      uint64_t(d.outW) * 16 * units +
+      ((cols - d.outW) * 16 * units + 255) / 256 * 256;
   s.maxRows = maxPatchRows(d);
   // (a lane per patch row works out where the rows start)
   if (s.maxRows > 64)
@@ -1250,8 +1262,9 @@ hipError_t launchIgemmPatch(const IgemmDesc &d, int inType, int outType,
   a.rowLoads = s.rowLoads;
   a.rowPitch = s.rowPitch;
   a.tapRowBytes = d.dilH * s.rowPitch;
-  a.tapColBytes = d.dilW * kPixelPitch;
-  a.rowUnits = (d.outW + (d.kW - 1) * d.dilW) * kPixelUnits;
+  const uint32_t units = d.patch == 2 ? kPixelUnits16 : kPixelUnits;
+  a.tapColBytes = d.dilW * 16 * units;
+  a.rowUnits = (d.outW + (d.kW - 1) * d.dilW) * units;
   a.sliceBytes = s.maxRows * s.rowPitch;
   a.exchangeByte = s.exchangeByte, a.tileByte = s.tileByte;
   a.pixelBytes = d.groups * d.inChansPerGroup * s.eb;
