@@ -308,6 +308,32 @@ hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
 /// and kernel dilation, 3x3 or 5x5 taps: the backward pass of a stride-2
 /// layer), which loads every input vector and tap once per thread.
 bool depthwiseDirectInBlocks(const DepthwiseDesc &d);
+/// The FORWARD convolution of a dense layer whose weight deltas
+/// launchWuTap forms from the layer's own tensors: two field dimensions, unit
+/// stride, nothing dilated, truncated or flipped, fp16 tensors, channels in
+/// whole 16-byte vectors.  An input pixel of output (y, x) and tap (kh, kw) is
+/// (y + kh - padH, x + kw - padW), read when it lies in [loH, hiH) x
+/// [loW, hiW), else zero.
+struct WuTapDesc {
+  uint32_t batch, inH, inW, outH, outW, kH, kW;
+  int32_t padH, padW;
+  uint32_t loH, hiH, loW, hiW;
+  uint32_t groups, ci, co;
+  // pixels (batch, y, x flattened) a workgroup sums over: a multiple of 64
+  uint32_t chunkPixels;
+};
+bool wuTapTakes(const WuTapDesc &d);
+/// Pixels per workgroup that give about one workgroup per compute unit.
+uint32_t wuTapChunkPixels(const WuTapDesc &d, uint32_t computeUnits);
+uint64_t wuTapWorkspaceBytes(const WuTapDesc &d);
+/// weightDeltas [groups][co][ci][kH][kW] in outType (half or float) from acts
+/// [batch][inH][inW][groups][ci] and deltas [batch][outH][outW][groups][co],
+/// both fp16; fp32 partial tiles of the pixel chunks go through `workspace`
+/// and are added in a fixed order.
+hipError_t launchWuTap(const WuTapDesc &d, int outType, const void *acts,
+                       const void *deltas, void *workspace, void *out,
+                       hipStream_t stream);
+
 /// Gradient with respect to the weights of the depthwise FORWARD convolution
 /// `d` (undilated input): weightDeltas [channels][kH * kW] in outType from
 /// acts [batch][inH][inW][channels] and deltas [batch][outH][outW][channels],

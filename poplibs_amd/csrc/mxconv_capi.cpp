@@ -1264,6 +1264,12 @@ WuWorkspace wuWorkspace(const mxconv_plan *plan) {
     w.total = at;
     return w;
   }
+  if (plan->denseWeightUpdate) {
+    w.planWorkspace = take(mxk::wuTapWorkspaceBytes(plan->denseForward));
+    w.deltas = take(plan->outputBytes());
+    w.total = at;
+    return w;
+  }
   w.input = take(plan->inputBytes());
   w.weightsExternal = take(plan->weightBytes());
   w.weightsPacked = take(plan->weightPackedBytes());
@@ -1304,6 +1310,11 @@ mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
                          plan->depthwiseForward, p.outputType.id(), acts,
                          zDeltas, ws + w.planWorkspace, deltasOut, s),
                      "depthwise weight deltas");
+  if (plan->denseWeightUpdate)
+    return hipStatus(mxk::launchWuTap(plan->denseForward, p.outputType.id(),
+                                      acts, zDeltas, ws + w.planWorkspace,
+                                      deltasOut, s),
+                     "matrix-core weight deltas");
   mxconv_status st;
   // activations [B][X][G][Ci] -> the pass's input [Ci][X][G][B]
   const mxk::SwapBatchChans actsSwap{

@@ -330,6 +330,35 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       f.loH = w.loH, f.hiH = w.hiH, f.loW = w.loW, f.hiW = w.hiW;
     }
   }
+  // The weight update pass of a dense layer with unit stride and nothing
+  // dilated: batch = the layer's input channels, input channels = its batch,
+  // kernel = its output field, output field = its kernel.  (Opt out:
+  // planConstraints gfx950 kernel names one.)
+  {
+    const Simple2D w = asSimple2D(p);
+    if (w.ok && !w.hasDepth() && !w.outputPadded() && !w.kernelSelected &&
+        !plan.zeroConv && !plan.depthwiseWeightUpdate && !w.inputDilated() &&
+        w.batch == p.batchSize && w.strideH == 1 && w.strideW == 1 &&
+        w.dilH == 1 && w.dilW == 1 && params.inputType == poplar::HALF &&
+        options.planConstraints.kernel.empty() &&
+        options.planConstraints.method == PlanConstraints::Method::ANY) {
+      mxk::WuTapDesc &f = plan.denseForward;
+      f.batch = uint32_t(p.inputChannelsPerConvGroup);
+      f.inH = w.inH, f.inW = w.inW;
+      f.outH = w.kH, f.outW = w.kW, f.kH = w.outH, f.kW = w.outW;
+      f.padH = w.padH, f.padW = w.padW;
+      f.loH = w.loH, f.hiH = w.hiH, f.loW = w.loW, f.hiW = w.hiW;
+      f.groups = uint32_t(p.numConvGroups);
+      f.ci = uint32_t(p.batchSize);
+      f.co = uint32_t(p.outputChannelsPerConvGroup);
+      f.chunkPixels = mxk::wuTapChunkPixels(f, gfx950::numCUs);
+      // (enough pixels to be worth the matrix cores: a kernel-sized field
+      // of a tiny batch stays with the general path)
+      const std::size_t pixels = std::size_t(f.batch) * f.outH * f.outW;
+      plan.denseWeightUpdate = pixels >= 1024 && f.ci >= 16 && f.co >= 16 &&
+                               mxk::wuTapTakes(f);
+    }
+  }
   const auto &pc = options.planConstraints;
   const Simple2D s = asSimple2D(p);
   const bool halfIn = params.inputType == poplar::HALF;
@@ -999,6 +1028,18 @@ std::string mxconv_plan::describe() const {
   if (depthwiseWeightUpdate)
     os << "        as a weight update pass    depthwise weight-delta kernel "
           "on the layer's own tensors\n";
+  if (denseWeightUpdate) {
+    const auto &f = denseForward;
+    const std::size_t m = std::size_t(f.batch) * f.outH * f.outW;
+    const std::size_t chunks = (m + f.chunkPixels - 1) / f.chunkPixels;
+    const std::size_t tiles = std::size_t(f.groups) * f.kH * f.kW *
+                              ((f.ci + 127) / 128) * ((f.co + 127) / 128);
+    os << "        as a weight update pass    matrix-core weight-delta kernel "
+          "on the layer's own tensors (transposing LDS reads): "
+       << tiles << " tap x channel tiles x " << chunks << " chunks of "
+       << f.chunkPixels << " pixels = " << tiles * chunks
+       << " workgroups, fp32 partial tiles summed in order\n";
+  }
   os << "        workspaceBytes             " << workspaceBytes << "\n";
   return os.str();
 }

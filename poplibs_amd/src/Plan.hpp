@@ -56,6 +56,10 @@ struct mxconv_plan {
   // the parameters as an ordinary convolution).
   bool depthwiseWeightUpdate = false;
   mxk::DepthwiseDesc depthwiseForward{};
+  // ... or of a dense unit-stride layer: the matrix-core kernel that reads
+  // the layer's tensors as they are (mxk::launchWuTap).
+  bool denseWeightUpdate = false;
+  mxk::WuTapDesc denseForward{};
 
   // Packed weights of the matrix-core kernel: [G][coPadded][kPadded].
   std::size_t coPadded = 0, kPadded = 0;

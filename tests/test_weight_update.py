@@ -202,6 +202,92 @@ def test_weight_deltas_on_gpu_match_oracle(oracle, kw):
     assert rel_l2(got, want) <= 1e-5, (rel_l2(got, want), plan.describe())
 
 
+DENSE_WU = "matrix-core weight-delta kernel on the layer's own tensors"
+DENSE_WU_CASES = [
+    # the ResNet-style 3x3 layer at a small batch: 9 taps x 12 chunks
+    dict(batch=4, field=(28, 28), kernel=(3, 3), ci=128, co=128, pad=1),
+    # channels ragged against the 128 x 128 tile, groups, pixels no multiple
+    # of 64, a 3 x 2 kernel with asymmetric padding
+    dict(batch=9, field=(13, 11), kernel=(3, 2), ci=72, co=40, groups=2,
+         padLower=(1, 0), padUpper=(1, 1)),
+    # more channels than one tile
+    dict(batch=6, field=(14, 14), kernel=(3, 3), ci=136, co=264, pad=1),
+    # pointwise: one tap
+    dict(batch=8, field=(12, 12), kernel=(1, 1), ci=64, co=32),
+    # a 5 x 5 kernel, more padding than the window needs
+    dict(batch=8, field=(12, 12), kernel=(5, 5), ci=16, co=24, pad=3),
+    # input truncation (negative padding)
+    dict(batch=8, field=(16, 14), kernel=(3, 3), ci=32, co=32, itl=(1, 0),
+         itu=(0, 2), pad=1),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+@pytest.mark.parametrize("kw", DENSE_WU_CASES)
+def test_dense_weight_deltas_from_the_layers_own_tensors(oracle, kw, out_type):
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, out_type, **kw)
+    print("case", p, flush=True)
+    rng = np.random.default_rng(61)
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    xq, xd = quantize(
+        rng.standard_normal((p.batchSize, G * Ci, *p.inputFieldShape)), pa.HALF)
+    dq, dd = quantize(
+        rng.standard_normal((p.batchSize, G * Co, *p.getOutputFieldShape()))
+        * 0.1, pa.HALF)
+    got, plan = run_weight_update(p, xq, dq)
+    assert DENSE_WU in plan.describe(), plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert got.shape == want.shape
+    # fp32 accumulation; a half result is rounded once
+    tol = 1e-5 if out_type == pa.FLOAT else 1e-3
+    assert rel_l2(got, want) <= tol, (rel_l2(got, want), plan.describe())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kw", DENSE_WU_CASES[:3])
+def test_dense_weight_deltas_of_signs_are_exact(oracle, kw):
+    # +-1 tensors: every product and every partial sum is a small integer
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    print("case", p, flush=True)
+    rng = np.random.default_rng(62)
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    x = rng.choice([-1.0, 1.0], (p.batchSize, G * Ci, *p.inputFieldShape))
+    dz = rng.choice([-1.0, 1.0],
+                    (p.batchSize, G * Co, *p.getOutputFieldShape()))
+    got, plan = run_weight_update(p, x.astype(np.float16),
+                                  dz.astype(np.float16))
+    assert DENSE_WU in plan.describe()
+    np.testing.assert_array_equal(got, oracle.weight_deltas(p, x, dz,
+                                                            threads=8))
+
+
+def test_dense_weight_update_plan_choice():
+    big = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3),
+                      ci=128, co=128, pad=1)
+    text = pa.WeightUpdatePlan(big).describe()
+    assert DENSE_WU in text
+    assert "9 tap x channel tiles x 28 chunks of 896 pixels = 252 workgroups" \
+        in text
+    # strided layers, tiny pixel counts and fp32 tensors stay with the pass's
+    # own convolution
+    for kw in (dict(batch=32, field=(28, 28), kernel=(3, 3), ci=128, co=128,
+                    pad=1, stride=2),
+               dict(batch=1, field=(8, 8), kernel=(3, 3), ci=128, co=128,
+                    pad=1)):
+        assert DENSE_WU not in pa.WeightUpdatePlan(
+            make_params(pa.HALF, **kw)).describe()
+    assert DENSE_WU not in pa.WeightUpdatePlan(
+        make_params(pa.FLOAT, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                    co=128, pad=1)).describe()
+    # ... and a kernel named in planConstraints is honoured
+    opts = {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'}
+    assert DENSE_WU not in pa.WeightUpdatePlan(big, opts).describe()
+
+
 @pytest.mark.gpu
 def test_weight_deltas_of_a_small_batch_run_on_the_matrix_cores(oracle):
     # the pass's input channels are the layer's batch: 4 of them are padded
