@@ -268,17 +268,23 @@ __global__ __launch_bounds__(kWuThreads) void wuTapKernel(
   }
 }
 
-/// deltas[g][co][ci][tap] = sum over the chunks, in order; four running sums
-/// keep four loads in flight per lane.  (Measured alternatives, both slower:
-/// two outputs per thread with eight sums; a workgroup per input channel that
-/// gathers each output channel's taps in LDS and writes them together.)
+/// deltas[g][co][ci][tap] = sum over the chunks in a fixed order.  Four
+/// neighbouring lanes share an output vector of four channels: lane part p
+/// adds the chunks p, p + 4, ... (two running sums, two loads in flight), and
+/// the four meet as (s0 + s1) + (s2 + s3) - four times the threads of a lane
+/// per output, which is what a 16 MB stream needs to keep HBM busy.
+/// (Measured alternatives, all slower: one lane per output vector with four
+/// running sums - 6.3 us; two outputs per thread with eight sums; a workgroup
+/// per input channel that gathers each output channel's taps in LDS and
+/// writes them together.)
 template <class OutT>
 __global__ __launch_bounds__(256) void wuTapSumKernel(
     const float *__restrict__ partial, OutT *__restrict__ out, uint32_t chunks,
     uint32_t groups, uint32_t taps, uint32_t ci, uint32_t co,
     uint32_t ciTiles, uint32_t coTiles) {
-  // thread -> (group, tap, ci, 4 co), co fastest
-  const uint64_t id = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  // thread -> (group, tap, ci, 4 co, part), part fastest
+  const uint64_t id = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) >> 2;
+  const uint32_t part = threadIdx.x & 3;
   const uint32_t co4 = (coTiles * 128) / 4;
   const uint32_t c = uint32_t(id % co4) * 4;
   uint64_t rest = id / co4;
@@ -286,6 +292,7 @@ __global__ __launch_bounds__(256) void wuTapSumKernel(
   rest /= ciTiles * 128;
   const uint32_t tap = uint32_t(rest % taps);
   const uint32_t g = uint32_t(rest / taps);
+  // (whole groups of four lanes leave together)
   if (g >= groups || i >= ci || c >= co)
     return;
   const size_t tile = 128 * 128;
@@ -295,28 +302,30 @@ __global__ __launch_bounds__(256) void wuTapSumKernel(
                       c / 128) *
                          tile +
                      (i % 128) * 128 + c % 128;
-  float4 sum[4] = {};
-  uint32_t p = 0;
-  for (; p + 4 <= chunks; p += 4) {
-#pragma unroll
-    for (int u = 0; u != 4; ++u) {
-      const float4 v =
-          *reinterpret_cast<const float4 *>(src + size_t(p + u) * perChunk);
-      sum[u].x += v.x, sum[u].y += v.y, sum[u].z += v.z, sum[u].w += v.w;
-    }
+  float4 sum[2] = {};
+  uint32_t p = part;
+  for (; p + 4 < chunks; p += 8) {
+    const float4 v0 = *reinterpret_cast<const float4 *>(src + size_t(p) * perChunk);
+    const float4 v1 =
+        *reinterpret_cast<const float4 *>(src + size_t(p + 4) * perChunk);
+    sum[0].x += v0.x, sum[0].y += v0.y, sum[0].z += v0.z, sum[0].w += v0.w;
+    sum[1].x += v1.x, sum[1].y += v1.y, sum[1].z += v1.z, sum[1].w += v1.w;
   }
-  for (; p != chunks; ++p) {
-    const float4 v = *reinterpret_cast<const float4 *>(src + size_t(p) * perChunk);
-    sum[0].x += v.x, sum[0].y += v.y, sum[0].z += v.z, sum[0].w += v.w;
+  if (p < chunks) {
+    const float4 v0 = *reinterpret_cast<const float4 *>(src + size_t(p) * perChunk);
+    sum[0].x += v0.x, sum[0].y += v0.y, sum[0].z += v0.z, sum[0].w += v0.w;
   }
-  const float v[4] = {(sum[0].x + sum[1].x) + (sum[2].x + sum[3].x),
-                      (sum[0].y + sum[1].y) + (sum[2].y + sum[3].y),
-                      (sum[0].z + sum[1].z) + (sum[2].z + sum[3].z),
-                      (sum[0].w + sum[1].w) + (sum[2].w + sum[3].w)};
-  // (co is a multiple of 8: the planner's condition)
+  float v[4] = {sum[0].x + sum[1].x, sum[0].y + sum[1].y, sum[0].z + sum[1].z,
+                sum[0].w + sum[1].w};
 #pragma unroll
-  for (int e = 0; e != 4; ++e)
-    storeOut(out, ((size_t(g) * co + c + e) * ci + i) * taps + tap, v[e]);
+  for (int e = 0; e != 4; ++e) {
+    v[e] += __shfl_xor(v[e], 1); // s0 + s1, s2 + s3
+    v[e] += __shfl_xor(v[e], 2);
+  }
+  // (co is a multiple of 8: the planner's condition); lane part p stores
+  // channel c + p
+  storeOut(out, ((size_t(g) * co + c + part) * ci + i) * taps + tap,
+           part == 0 ? v[0] : part == 1 ? v[1] : part == 2 ? v[2] : v[3]);
 }
 
 uint64_t tilesOf(const WuTapDesc &d) {
@@ -403,7 +412,7 @@ hipError_t launchWuTap(const WuTapDesc &d, int outType, const void *acts,
   if (e != hipSuccess)
     return e;
   const uint64_t threads =
-      uint64_t(d.groups) * a.taps * a.ciTiles * 128 * (a.coTiles * 128 / 4);
+      uint64_t(d.groups) * a.taps * a.ciTiles * 128 * (a.coTiles * 128 / 4) * 4;
   const uint32_t sumBlocks = uint32_t((threads + 255) / 256);
   if (outType == kHalf)
     hipLaunchKernelGGL(wuTapSumKernel<__half>, dim3(sumBlocks), dim3(256), 0,
