@@ -15,19 +15,23 @@
 // producer waves and no LDS writes, and the vector cache carries the weights
 // only.
 //
-// Workgroup: 8 waves, tile 32*RB pixels x 128 channels.  Wave (grp, wn):
+// Two kernels share this data path.  igemmPatchKernel (first in this file):
+// MFMA 32x32, tiles of 32*RB pixels x 128 channels; wave (grp, wn) takes
 // channels 32 wn .. 32 wn + 31 of all pixels, and of every k-step (128 bytes
 // of K: one tap, one channel slice) the half `grp` - two waves per SIMD that
-// cover each other's LDS latency.  The two halves are summed through LDS at
-// the end.
+// cover each other's LDS latency, their sums meeting in LDS at the end.
+// igemmPatch16Kernel (further down, with its own notes): MFMA 16x16, tiles of
+// any height up to 112 pixels, the two waves of a SIMD taking k-steps in
+// turn - what the planner picks.
 //
-// LDS patch: [slice][patch row][unit], a unit = 16 bytes, a pixel = 9 units
-// (8 of channels + 1 unused): at a pitch of 144 bytes the 16-byte reads of
-// 16 neighbouring pixels cover all 64 banks without any swizzle, so a tap is
-// a plain byte offset.  A patch row = the input row of one image with its
-// zero padding left and right, rounded up to whole 1 KB wave loads; patch
-// rows are the rows, padding rows included, of consecutive images that the
-// tile's pixels read.
+// LDS patch: [slice][patch row][unit], a unit = 16 bytes, a pixel = 8 units
+// of channels + 1 or 2 unused: at a pitch of 144 bytes (32-pixel MFMA blocks)
+// or 160 bytes (16-pixel blocks) the 16-byte operand reads of neighbouring
+// pixels cover all 64 banks without any swizzle, so a tap is a plain byte
+// offset.  A patch row = the input row of one image with its zero padding
+// left and right; the pitch of the rows continues the pixels' progression
+// through the banks (modulo 256 bytes).  Patch rows are the rows, padding
+// rows included, of consecutive images that the tile's pixels read.
 //
 // Takes the role of PopLibs' AMP vertex ConvPartialnx1
 // (lib/poplin/codelets/ConvPartialnx1.cpp:52-246) for these shapes; the fp8

@@ -130,6 +130,16 @@ def test_patch_16_pixel_blocks_refuse_one_tap():
     assert PATCH not in pa.Plan(p, FORCED16).describe()
 
 
+@pytest.mark.parametrize("options", [FORCED, FORCED16])
+def test_patch_that_leaves_no_room_beside_it(oracle, options):
+    """Four channel slices of a 28-wide field: the patch takes 140 KB of the
+    160, so the waves' sums meet in its place once everybody has left it."""
+    p = make_params(pa.HALF, batch=2, field=(28, 28), kernel=(3, 3), ci=256,
+                    co=136, pad=1)
+    print("case", p, flush=True)
+    _run(oracle, p, 17, 1e-3, options=options)
+
+
 def test_patch_is_the_planners_choice_for_the_benchmark_layers():
     p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
                     co=128, pad=1)
