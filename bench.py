@@ -254,6 +254,9 @@ class TrainingRunner:
                        if l.strip().startswith("kernel ")][0]
         if which == "wu" and "depthwise weight-delta kernel" in text:
             self.kernel = "depthwise weight-delta kernel (vector ALU)"
+        if which == "wu" and "matrix-core weight-delta kernel" in text:
+            self.kernel = ("matrix-core weight-delta kernel on the layer's own "
+                           "tensors (MFMA, transposing LDS reads) + ordered sum")
 
     def _bwd(self, i=0):
         s = self.torch.cuda.current_stream().cuda_stream
