@@ -265,6 +265,29 @@ def test_dense_weight_deltas_of_signs_are_exact(oracle, kw):
                                                             threads=8))
 
 
+@pytest.mark.gpu
+def test_dense_weight_deltas_at_the_benchmark_layers_full_size(oracle):
+    """configs[1] whole (N=32 28x28 128->128 3x3): 252 workgroups, 28 chunks
+    of 896 pixels.  Against the oracle, and - independent of it - against the
+    sum of the deltas of the two halves of the batch (the pass is linear in
+    the pixels it sums over)."""
+    from gpu_helpers import quantize
+    kw = dict(field=(28, 28), kernel=(3, 3), ci=128, co=128, pad=1)
+    p = make_params(pa.HALF, pa.FLOAT, batch=32, **kw)
+    rng = np.random.default_rng(63)
+    xq, xd = quantize(rng.standard_normal((32, 128, 28, 28)), pa.HALF)
+    dq, dd = quantize(rng.standard_normal((32, 128, 28, 28)) * 0.05, pa.HALF)
+    got, plan = run_weight_update(p, xq, dq)
+    assert DENSE_WU in plan.describe()
+    assert "28 chunks of 896 pixels = 252 workgroups" in plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert rel_l2(got, want) <= 1e-5, rel_l2(got, want)
+    half = make_params(pa.HALF, pa.FLOAT, batch=16, **kw)
+    lo, _ = run_weight_update(half, xq[:16], dq[:16])
+    hi, _ = run_weight_update(half, xq[16:], dq[16:])
+    assert rel_l2(lo + hi, got) <= 1e-6
+
+
 def test_dense_weight_update_plan_choice():
     big = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3),
                       ci=128, co=128, pad=1)
