@@ -53,6 +53,8 @@ struct WuTapArgs {
   uint32_t taps, ciTiles, coTiles;
   uint32_t chunks, tilesPerChunk;
   uint32_t actPixelBytes, deltaPixelBytes; // groups * channels * 2
+  uint32_t actImageBytes;                  // inH * inW * actPixelBytes
+  uint32_t stepX, stepY, stepImages;       // 64 pixels as columns, rows, images
   uint64_t actBytes, deltaBytes;
   FastDiv divOutW, divOutH, divTaps, divCiTiles, divCoTiles, divKW;
   FastDiv divTilesPerChunk;
@@ -113,20 +115,33 @@ __global__ __launch_bounds__(kWuThreads) void wuTapKernel(
   const uint32_t actLane = actChan < d.ci ? (g * d.ci + actChan) * 2 : kWuInvalid;
   const uint32_t deltaLane =
       deltaChan < d.co ? (g * d.co + deltaChan) * 2 : kWuInvalid;
-  auto load = [&](uint32_t step, char *__restrict__ into) {
+  // Steps are loaded in order, so each lane keeps where its two pixels of the
+  // next step are (column, row, image) and moves them on by 64 pixels with
+  // two carries instead of taking the pixel number apart every time.
+  struct Walker {
+    uint32_t x, y, imageAt, deltaAt, p;
+  } at[2];
+#pragma unroll
+  for (int h = 0; h != 2; ++h) {
+    const uint32_t p = p0 + h * 32 + row;
+    const uint32_t pr = a.divOutW(p), b = a.divOutH(pr);
+    at[h].x = p - pr * d.outW, at[h].y = pr - b * d.outH;
+    at[h].imageAt = b * a.actImageBytes;
+    at[h].deltaAt = p * a.deltaPixelBytes;
+    at[h].p = p;
+  }
+  const uint32_t tapY = kh - uint32_t(d.padH), tapX = kw - uint32_t(d.padW);
+  auto load = [&](char *__restrict__ into) {
     char *stage = into + wave * 1024;
 #pragma unroll
     for (int h = 0; h != 2; ++h) {
-      const uint32_t p = p0 + step * 64 + h * 32 + row;
-      const uint32_t pr = a.divOutW(p), x = p - pr * d.outW;
-      const uint32_t b = a.divOutH(pr), y = pr - b * d.outH;
-      const uint32_t iy = y + kh - uint32_t(d.padH),
-                     ix = x + kw - uint32_t(d.padW);
-      const bool inside = p < p1;
-      const uint32_t deltaAt = inside ? p * a.deltaPixelBytes : kWuInvalid;
+      Walker &w = at[h];
+      const uint32_t iy = w.y + tapY, ix = w.x + tapX;
+      const bool inside = w.p < p1;
+      const uint32_t deltaAt = inside ? w.deltaAt : kWuInvalid;
       const uint32_t actAt =
           inside && iy - d.loH < d.hiH - d.loH && ix - d.loW < d.hiW - d.loW
-              ? ((b * d.inH + iy) * d.inW + ix) * a.actPixelBytes
+              ? w.imageAt + (iy * d.inW + ix) * a.actPixelBytes
               : kWuInvalid;
       // (any sum with a kWuInvalid in it lies beyond the buffer and reads
       // as zeros)
@@ -134,6 +149,16 @@ __global__ __launch_bounds__(kWuThreads) void wuTapKernel(
                 deltaAt + deltaLane, 0);
       loadToLds(actBuf, (LdsPtr)(stage + (2 * h + 1) * kWuTileBytes),
                 actAt + actLane, 0);
+      // 64 pixels on: stepX columns, stepY rows, stepImages images, with the
+      // carries (a single one each: x < outW and stepX < outW, likewise y)
+      w.p += 64, w.deltaAt += 64 * a.deltaPixelBytes;
+      w.x += a.stepX;
+      const uint32_t carryX = w.x >= d.outW ? 1u : 0u;
+      w.x -= carryX ? d.outW : 0u;
+      w.y += a.stepY + carryX;
+      const uint32_t carryY = w.y >= d.outH ? 1u : 0u;
+      w.y -= carryY ? d.outH : 0u;
+      w.imageAt += (a.stepImages + carryY) * a.actImageBytes;
     }
   };
 
@@ -201,14 +226,14 @@ __global__ __launch_bounds__(kWuThreads) void wuTapKernel(
     MXK_WAIT_VMCNT(8);
     stepBarrier();
     // (everybody's reads of step's stage finished an iteration ago)
-    load(step + kWuStages, into);
+    load(into);
     read(next, from);
     multiply(cur);
     MXK_WAIT_LGKMCNT0();
   };
 #pragma unroll
   for (int s = 0; s != kWuStages; ++s)
-    load(s, lds + s * kWuStageBytes);
+    load(lds + s * kWuStageBytes);
   Operands even, odd;
   MXK_WAIT_VMCNT(12);
   stepBarrier();
@@ -386,7 +411,11 @@ hipError_t launchWuTap(const WuTapDesc &d, int outType, const void *acts,
   a.ciTiles = (d.ci + 127) / 128, a.coTiles = (d.co + 127) / 128;
   a.actPixelBytes = d.groups * d.ci * 2;
   a.deltaPixelBytes = d.groups * d.co * 2;
-  a.actBytes = uint64_t(d.batch) * d.inH * d.inW * a.actPixelBytes;
+  a.actImageBytes = d.inH * d.inW * a.actPixelBytes;
+  a.actBytes = uint64_t(d.batch) * a.actImageBytes;
+  a.stepX = 64 % d.outW;
+  a.stepY = 64 / d.outW % d.outH;
+  a.stepImages = 64 / d.outW / d.outH;
   a.deltaBytes = uint64_t(a.M) * a.deltaPixelBytes;
   a.divOutW = makeFastDiv(d.outW), a.divOutH = makeFastDiv(d.outH);
   a.divTaps = makeFastDiv(a.taps), a.divCiTiles = makeFastDiv(a.ciTiles);
