@@ -426,6 +426,11 @@ def main():
         runner = probe if sets == 1 else Runner(pa, capi, torch, wl, sets=sets)
         wall, kernel, mode, fastest = time_steps(torch, runner, steps,
                                                  warmup)
+        # ... and, labelled as such, the figure with one buffer set (tensors
+        # in the Infinity Cache from the launch before)
+        hot = None
+        if sets != 1:
+            _, hot, _, _ = time_steps(torch, probe, steps, warmup)
         if wl["bound"] == "mfma":
             achieved = runner.flops / kernel / 1e12
             peak, unit = PEAK_TFLOPS[wl["dtype"]], "TFLOP/s"
@@ -442,6 +447,8 @@ def main():
                       "traffic": traffic, "traffic_stale": stale,
                       "kernel_us": round(kernel * 1e6, 3),
                       "kernel_us_fastest_pass": round(fastest * 1e6, 3),
+                      **({"kernel_us_one_buffer_set_cache_hot":
+                          round(hot * 1e6, 3)} if hot else {}),
                       "algorithmic_per_launch":
                           runner.flops if wl["bound"] == "mfma"
                           else runner.bytes})
