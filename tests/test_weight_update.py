@@ -219,6 +219,13 @@ DENSE_WU_CASES = [
     # input truncation (negative padding)
     dict(batch=8, field=(16, 14), kernel=(3, 3), ci=32, co=32, itl=(1, 0),
          itu=(0, 2), pad=1),
+    # a 1-D field, a kernel wider than 64 pixels' worth of columns is not
+    # needed: rows of 40 pixels, so 64 pixels span rows and images
+    dict(batch=30, field=(40,), kernel=(5,), ci=24, co=16, pad=2),
+    # tiny images: 64 pixels span several of them
+    dict(batch=70, field=(4, 4), kernel=(3, 3), ci=16, co=16, pad=1),
+    # one image
+    dict(batch=1, field=(40, 36), kernel=(3, 3), ci=16, co=48, pad=1),
 ]
 
 
