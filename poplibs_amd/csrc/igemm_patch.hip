@@ -706,11 +706,20 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
 #pragma unroll
     for (int u = 0; u != kFirst; ++u)
       loadB(bf[u]);
+    // Lane l works out where pixels l and 64 + l of the tile sit in the
+    // patch (two divisions by the field's width and height instead of seven
+    // per lane: a lone wave issues an instruction every 5 to 8 cycles, and
+    // the workgroup's first MFMA waits for its slowest wave); a lane then
+    // fetches the pixels of its row blocks from the lanes that hold them.
+    const uint32_t first = patchByteOf<kPixelUnits16>(a, span, span.m0 + lane);
+    const uint32_t second =
+        patchByteOf<kPixelUnits16>(a, span, span.m0 + 64 + lane);
 #pragma unroll
-    for (int i = 0; i != RB; ++i)
-      pixelByte[i] = patchByteOf<kPixelUnits16>(
-                         a, span, span.m0 + i * 16 + (lane & 15)) +
+    for (int i = 0; i != RB; ++i) {
+      const int from = (16 * i + (lane & 15)) & 63;
+      pixelByte[i] = uint32_t(__shfl(int(i < 4 ? first : second), from)) +
                      Mma::laneByte(lane >> 4);
+    }
 #pragma unroll
     for (int i = 0; i != RB; ++i)
       asm volatile("" ::"v"(pixelByte[i]));
