@@ -665,6 +665,11 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
   const int grp = wave / kWavesN, wn = wave % kWavesN;
 
   const uint32_t tile = xcdSwizzle(blockIdx.x, gridDim.x);
+  // (Arguments the compiler would otherwise fetch where they are first used,
+  // each fetch a round trip of the scalar cache on the way to the first MFMA:
+  // naming them here puts them into the one fetch at the kernel's start.)
+  asm volatile("" ::"s"(w), "s"(out), "s"(bias), "s"(a.inH), "s"(a.ciBytes),
+               "s"(a.inRowBytes), "s"(a.outChans), "s"(a.outChansPerGroup));
   const uint32_t overN = a.divNTiles(tile);
   const uint32_t nTile = tile - overN * a.nTiles;
   const uint32_t g = a.divMTiles(overN);
