@@ -213,9 +213,9 @@ loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
 
 /// The finished tile, [row][128 channels] at a pitch of kOutRow bytes in LDS,
 /// goes out as 16-byte stores, whole rows per instruction, through a buffer
-/// that ends with the last valid row: rows beyond it go nowhere.  (Streaming
-/// cache policy - the same bit as for loads: the tile is not read again
-/// here.)  ROWS: rows the tile has room for in LDS.
+/// that ends with the last valid row: rows beyond it go nowhere.  (Written
+/// through the L2: nothing is left to write back when the kernel ends.)
+/// ROWS: rows the tile has room for in LDS.
 template <int ROWS, class OutT>
 __device__ __forceinline__ void
 storeTile(const PatchArgs &a, const char *tileOut, OutT *__restrict__ out,
@@ -242,7 +242,7 @@ storeTile(const PatchArgs &a, const char *tileOut, OutT *__restrict__ out,
     __builtin_amdgcn_raw_buffer_store_b128(
         *reinterpret_cast<const uintx4 *>(from +
                                           pass * kRowsPerPass * kOutRow),
-        outBuf, to, pass * kRowsPerPass * outRowBytes, kStreamingLoad);
+        outBuf, to, pass * kRowsPerPass * outRowBytes, kWriteThroughStore);
 }
 
 template <int EB> struct PatchMma;
