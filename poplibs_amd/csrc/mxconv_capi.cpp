@@ -1527,7 +1527,7 @@ mxconv_status mxconv_convolution_bias_update(int32_t deltas_type,
   if (outer_elems)
     REQUIRE_ARG(z_deltas_internal);
   const size_t need = mxk::biasUpdateWorkspaceBytes(outer_elems, channels);
-  if (workspace_bytes < need || !workspace)
+  if (workspace_bytes < need || (need && !workspace))
     return fail(MXCONV_WORKSPACE_TOO_SMALL,
                 "workspace of " + std::to_string(need) + " bytes required");
   return hipStatus(mxk::launchBiasUpdate(deltas_type, z_deltas_internal,
