@@ -189,8 +189,10 @@ __global__ __launch_bounds__(kWuThreads) void wuTapKernel(
   // Software pipeline.  Iteration `step`: wait for step + 1's tiles, issue
   // the loads of step + kWuStages into the stage that step's operands were
   // read from (in the iteration before), read step + 1's operands, and only
-  // then multiply step's - the transposing reads, at about 10 cycles each for
-  // the whole CU, are what bounds the loop, and they run under the MFMAs.
+  // then multiply step's, so that the reads run under the MFMAs.  (What the
+  // loop waits for is the loads: the nine taps of a chunk read the same
+  // pixels on nine XCDs, nine in ten L2 requests miss, and an XCD's link to
+  // memory delivers about 1.3 TB/s.)
   // (`__restrict__` on the stage written and the stage read, so that the
   // compiler does not make the reads wait for the loads just issued: a load
   // that writes LDS is a pending LDS write to it.)
@@ -385,8 +387,8 @@ uint32_t wuTapChunkPixels(const WuTapDesc &d, uint32_t computeUnits) {
   // About one workgroup per CU; chunks of whole super-steps of 64 pixels, not
   // so short that start-up and the tile's way out outweigh the products.
   // (Dealing the workgroups of a chunk to one XCD, for its L2 to fetch the
-  // chunk's pixels once, gains nothing: the loop is bound by the transposing
-  // LDS reads.)
+  // chunk's pixels once, shortens the loop by a quarter, but the partial
+  // tiles' stores, all at the same moment then, take longer than that gains.)
   const uint64_t M = uint64_t(d.batch) * d.outH * d.outW;
   const uint64_t tiles = std::max<uint64_t>(1, tilesOf(d));
   const uint64_t chunks = std::max<uint64_t>(1, computeUnits / tiles);
