@@ -265,6 +265,14 @@ uint64_t pointwisePackedElems(const PointwiseDesc &d);
 hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
                                       void *dst, hipStream_t stream,
                                       bool chansTransposed = false);
+/// How launchPointwise runs a layer on a chip of `cus` compute units:
+/// persistent workgroups, each taking tiles of `tilePixels` pixels in turn
+/// through a ring of `ring` LDS buffers filled by `loaderWaves` waves.
+struct PointwiseLaunch {
+  uint32_t tilePixels, ring, loaderWaves, tilesPerWorkgroup;
+  uint64_t workgroups;
+};
+PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus);
 hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream);

@@ -45,11 +45,12 @@ struct PwArgs {
   uint32_t inBytes, wBytes;
 };
 
-/// KS: k-slices of 16 channels (Ci / 16).  TM: pixels per tile (32 or 64);
-/// the workgroup has TM / 16 compute waves and the loader wave.  NB: tile
-/// buffers in LDS; NB - 1 tiles are in flight.
-template <int KS, int TM, int NB, class OutT>
-__global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
+/// KS: k-slices of 16 channels (Ci / 16).  TM: pixels per tile (32, 64, 128);
+/// the workgroup has TM / 16 compute waves and LW loader waves, which take
+/// the loads of a tile in turn.  NB: tile buffers in LDS; NB - 1 tiles are in
+/// flight.
+template <int KS, int TM, int NB, int LW, class OutT>
+__global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
     PwArgs a, const char *__restrict__ in, const char *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
   constexpr int kRow = KS * 32;                 // bytes of one activation row
@@ -61,7 +62,9 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
   constexpr int kLoads = TM / kRowsPerLoad; // wave-wide loads per tile
   constexpr int kTileBytes = TM * kRow;
   constexpr int kComputeWaves = TM / 16;
-  static_assert((NB - 2) * kLoads <= 63, "wait count fits s_waitcnt");
+  static_assert(kLoads % LW == 0, "the loader waves share a tile evenly");
+  constexpr int kOwnLoads = kLoads / LW; // ... per loader wave
+  static_assert((NB - 2) * kOwnLoads <= 63, "wait count fits s_waitcnt");
   // NB tile buffers | staging
   extern __shared__ __align__(16) char lds[];
 
@@ -72,7 +75,8 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
   const uint32_t pixelBytes = d.groups * d.inChansPerGroup * 2;
 
-  if (wave == kComputeWaves) {
+  if (wave >= kComputeWaves) {
+    const int loader = wave - kComputeWaves;
     // ---- loader.  Load L of a tile fills bytes [1024 L, 1024 L + 1024) of
     // its buffer, i.e. rows L * kRowsPerLoad ...; lane l holds chunk position
     // l % (kRow / 16) of row l / (kRow / 16).
@@ -81,7 +85,8 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
     const uint32_t pos = lane & ((1 << kChunkBits) - 1);
     auto issue = [&](uint32_t mTile, char *buffer) {
 #pragma unroll
-      for (int load = 0; load != kLoads; ++load) {
+      for (int own = 0; own != kOwnLoads; ++own) {
+        const uint32_t load = own * LW + loader;
         const uint32_t row = load * kRowsPerLoad + rowInLoad;
         const uint32_t chunk = pos ^ (row & kSwizzle);
         const uint32_t m = mTile * TM + row;
@@ -99,7 +104,7 @@ __global__ __launch_bounds__(TM * 4 + 64) void pointwiseKernel(
       issue(walker + s * a.walkers, lds + s * kTileBytes);
     uint32_t buffer = NB - 1; // where tile i + NB - 1 goes
     for (uint32_t mTile = walker; mTile < a.mTiles; mTile += a.walkers) {
-      MXK_WAIT_VMCNT((NB - 2) * kLoads);
+      MXK_WAIT_VMCNT((NB - 2) * kOwnLoads);
       stepBarrier(); // tile i is in LDS; the buffer before it has been read
       issue(mTile + (NB - 1) * a.walkers, lds + buffer * kTileBytes);
       if (++buffer == NB)
@@ -222,14 +227,49 @@ __global__ __launch_bounds__(256) void packPointwiseWeightsKernel(
                                : src[(g * co + n) * ci + k];
 }
 
-template <int KS, int TM, int NB, class OutT>
+/// Workgroups that share the pixel tiles of one (group, channel tile) pair:
+/// as many workgroups as fit the chip at once (LDS allows 160 KB / ldsBytes
+/// per CU), shared out over the pairs - and no more than give every walker
+/// the same number of tiles (to within one): 3.1 tiles per walker would mean
+/// a fourth round at a quarter of the chip.
+uint64_t walkersFor(uint64_t mTiles, uint64_t pairs, uint32_t ldsBytes,
+                    uint32_t cus) {
+  const uint64_t resident = uint64_t(cus) * ((160 * 1024) / ldsBytes);
+  uint64_t walkers = resident / pairs;
+  if (walkers < 1)
+    walkers = 1;
+  const uint64_t tilesPerWalker = (mTiles + walkers - 1) / walkers;
+  return (mTiles + tilesPerWalker - 1) / tilesPerWalker;
+}
+
+/// Tile height, ring depth and loader waves by input channels per group.
+/// Tiles of 16 to 32 KB, a ring of three (one workgroup per CU), two or four
+/// loader waves.  Measured on N = 32 layers of 56 x 56 (28 x 28 for 512
+/// channels), against one loader wave and a ring of four (three for 512):
+/// 64 -> 256 channels 15.9 against 19.3 us, 128 -> 128 10.1 against 11.2,
+/// 256 -> 64 11.65 against 13.1, 512 -> 128 9.4 against 13.9.  One loader wave
+/// does not issue a tile's loads - ten instructions each - as fast as HBM
+/// delivers them; a deeper ring, or 128-pixel tiles where 64 are listed, is
+/// slower.
+struct PwShape {
+  int tm, nb, lw;
+};
+constexpr PwShape kShape64{128, 3, 2}, kShape128{128, 3, 4},
+    kShape256{64, 3, 2}, kShape512{32, 3, 4};
+constexpr PwShape shapeFor(uint32_t ci) {
+  return ci == 64 ? kShape64 : ci == 128 ? kShape128 : ci == 256 ? kShape256
+                                                                 : kShape512;
+}
+constexpr uint32_t ldsBytesOf(PwShape s, uint32_t ci) {
+  return uint32_t(s.nb * s.tm * (ci / 16) * 32 + (s.tm / 16) * 32 * kPwStageRow);
+}
+
+template <int KS, int TM, int NB, int LW, class OutT>
 hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
                void *out, hipStream_t stream) {
-  constexpr int kComputeWaves = TM / 16;
-  constexpr int ldsBytes =
-      NB * TM * KS * 32 + kComputeWaves * 32 * kPwStageRow;
+  constexpr int ldsBytes = ldsBytesOf(PwShape{TM, NB, LW}, KS * 16);
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void *>(&pointwiseKernel<KS, TM, NB, OutT>),
+      reinterpret_cast<const void *>(&pointwiseKernel<KS, TM, NB, LW, OutT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
   if (attr != hipSuccess)
     return attr;
@@ -243,28 +283,18 @@ hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
     return n;
   }();
   a.mTiles = (a.M + TM - 1) / TM;
-  // As many workgroups as fit the chip at once (LDS allows 160 KB / ldsBytes
-  // per CU), shared out over the (group, channel tile) pairs.
-  const uint64_t resident = uint64_t(cus) * ((160 * 1024) / ldsBytes);
   const uint64_t pairs = uint64_t(a.nTiles) * a.d.groups;
   if (pairs == 0 || a.mTiles == 0)
     return hipSuccess;
-  uint64_t walkers = resident / pairs;
-  if (walkers < 1)
-    walkers = 1;
-  // ... and no more than give every walker the same number of tiles (to
-  // within one): 3.1 tiles per walker would mean a fourth round at a quarter
-  // of the chip.
-  const uint64_t tilesPerWalker = (a.mTiles + walkers - 1) / walkers;
-  walkers = (a.mTiles + tilesPerWalker - 1) / tilesPerWalker;
+  const uint64_t walkers = walkersFor(a.mTiles, pairs, ldsBytes, cus);
   a.walkers = uint32_t(walkers);
   const uint64_t blocks = walkers * pairs;
   // Tile indices up to mTiles + (NB - 1) * walkers are formed in 32 bits.
   if (blocks > 0x7fffffffull ||
       uint64_t(a.mTiles) + uint64_t(NB) * walkers > 0x7fffffffull / TM)
     return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((pointwiseKernel<KS, TM, NB, OutT>),
-                     dim3(uint32_t(blocks)), dim3(TM * 4 + 64), ldsBytes,
+  hipLaunchKernelGGL((pointwiseKernel<KS, TM, NB, LW, OutT>),
+                     dim3(uint32_t(blocks)), dim3(TM * 4 + 64 * LW), ldsBytes,
                      stream, a, static_cast<const char *>(in),
                      static_cast<const char *>(w),
                      static_cast<const OutT *>(bias), static_cast<OutT *>(out));
@@ -274,16 +304,19 @@ hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
 template <class OutT>
 hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
                      const void *bias, void *out, hipStream_t stream) {
-  // Tiles of 16 KB, three in flight; 32 KB, two in flight, for the widest.
   switch (a.d.inChansPerGroup) {
   case 64:
-    return run<4, 64, 4, OutT>(a, in, w, bias, out, stream);
+    return run<4, kShape64.tm, kShape64.nb, kShape64.lw, OutT>(a, in, w, bias,
+                                                              out, stream);
   case 128:
-    return run<8, 64, 4, OutT>(a, in, w, bias, out, stream);
+    return run<8, kShape128.tm, kShape128.nb, kShape128.lw, OutT>(
+        a, in, w, bias, out, stream);
   case 256:
-    return run<16, 32, 4, OutT>(a, in, w, bias, out, stream);
+    return run<16, kShape256.tm, kShape256.nb, kShape256.lw, OutT>(
+        a, in, w, bias, out, stream);
   case 512:
-    return run<32, 32, 3, OutT>(a, in, w, bias, out, stream);
+    return run<32, kShape512.tm, kShape512.nb, kShape512.lw, OutT>(
+        a, in, w, bias, out, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -321,6 +354,23 @@ hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
                      static_cast<uint16_t *>(dst), d.outChansPerGroup,
                      d.inChansPerGroup, nBlocks, total, chansTransposed);
   return hipGetLastError();
+}
+
+PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus) {
+  const PwShape s = shapeFor(d.inChansPerGroup);
+  PointwiseLaunch l{};
+  l.tilePixels = uint32_t(s.tm), l.ring = uint32_t(s.nb);
+  l.loaderWaves = uint32_t(s.lw);
+  const uint64_t mTiles = (uint64_t(d.batch) * d.pixels + s.tm - 1) / s.tm;
+  const uint64_t pairs =
+      uint64_t((d.outChansPerGroup + kPwChans - 1) / kPwChans) * d.groups;
+  if (mTiles == 0 || pairs == 0)
+    return l;
+  const uint64_t walkers =
+      walkersFor(mTiles, pairs, ldsBytesOf(s, d.inChansPerGroup), cus);
+  l.workgroups = walkers * pairs;
+  l.tilesPerWorkgroup = uint32_t((mTiles + walkers - 1) / walkers);
+  return l;
 }
 
 hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,

@@ -946,9 +946,14 @@ std::string mxconv_plan::describe() const {
        << " groups)\n";
     if (pointwiseOn) {
       const std::size_t nTiles = (g.outChansPerGroup + 63) / 64;
-      os << "        block M x N x K            64 x 64 x " << k << "\n";
-      os << "        workgroups                 "
-         << (m + 63) / 64 * nTiles * g.groups << "\n";
+      const mxk::PointwiseLaunch l =
+          mxk::pointwiseLaunchShape(pointwise, gfx950::numCUs);
+      os << "        block M x N x K            " << l.tilePixels
+         << " x 64 x " << k << "\n";
+      os << "        workgroups                 " << l.workgroups << " on "
+         << gfx950::numCUs << " CUs, each taking " << l.tilesPerWorkgroup
+         << " tiles in turn through a ring of " << l.ring
+         << " LDS buffers filled by " << l.loaderWaves << " loader waves\n";
       os << "        packed weights             [G=" << g.groups << "]["
          << nTiles * 2 << " blocks of 32][" << k / 16
          << " slices of 16][64 lanes][8]\n";
