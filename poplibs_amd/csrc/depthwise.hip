@@ -301,6 +301,9 @@ hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
   if (d.inDilH != 1 || d.inDilW != 1)
     return launchDepthwiseDirect(d, inType, outType, in, weightsPacked, bias,
                                  out, stream);
+  if (d.dense3x3 == 2)
+    return launchDepthwiseRows(d, inType, outType, in, weightsPacked, bias,
+                               out, stream);
   if (d.dense3x3)
     return launchDepthwise3x3(d, inType, outType, in, weightsPacked, bias,
                                  out, stream);

@@ -1,0 +1,309 @@
+// Depthwise 3x3 forward convolution (dilation 1, stride 1 or 2) by persistent
+// workgroups that stream input rows through a ring in LDS: the same role as
+// depthwise3x3.hip (PopLibs' HorizontalMac vertices,
+// lib/poplin/codelets/ConvPartialHorizontalMac.cpp:34-133), for layers large
+// enough to give every CU a band of rows.
+//
+// A workgroup owns a band of output rows of one column strip of one image
+// and walks down it.  Loader waves bring the strip's input rows, one after
+// the other, into a ring of row slots with dense 1 KB loads that write LDS
+// directly (no registers, so many rows are in flight); every input row is
+// fetched once per band - the two (stride 2) or one (stride 1) new rows an
+// output row needs, not the three it reads.  Compute waves - one thread per
+// output pixel and channel vector of the current output row - read their nine
+// input vectors from the ring, multiply by taps they keep in registers for
+// the whole band, and store 16 bytes each, a whole output row of the strip as
+// one contiguous run.  One barrier per output row.  Several loader waves,
+// because one wave does not issue loads as fast as HBM delivers them (ten
+// instructions per load).
+#include "igemm_common.hpp"
+
+namespace mxk {
+namespace {
+
+constexpr int kRowLoads = 12;           // 1 KB loads per input row slot
+constexpr int kSlotBytes = kRowLoads * 1024;
+constexpr int kLoaderWaves = 4;
+constexpr int kComputeWaves = 6;
+constexpr int kComputeThreads = 64 * kComputeWaves;
+constexpr int kRowsThreads = 64 * (kComputeWaves + kLoaderWaves);
+constexpr int kOwnLoads = kRowLoads / kLoaderWaves; // per loader wave and row
+constexpr uint32_t kNoByte = 0x80000000u;           // beyond any buffer here
+
+/// Steps (output rows) the loads run ahead, and row slots of the ring, by
+/// stride: a step needs rows [j S, j S + 2], so `ahead` steps on the way take
+/// ahead * S + 3 slots.  Six rows on the way (108 KB of LDS): on N = 32,
+/// 112 x 112, 96 channels, stride 2 that takes 17.7 us, eight rows 18.0, ten
+/// 18.3, four 17.85, two 18.9; two loader waves 18.2, six as four.
+template <int S> struct Ring {
+  static constexpr int kAhead = 6 / S;
+  static constexpr int kSlots = kAhead * S + 3;
+};
+
+struct RowsArgs {
+  DepthwiseDesc d;
+  uint32_t vecs;              // channels / 8
+  uint32_t strips, colsOut;   // column strips per image, output columns each
+  uint32_t bands, rowsOut;    // row bands per strip, output rows each
+  uint32_t colsIn;            // input columns of a strip: (colsOut-1)*S + 3
+  uint32_t inBytes;
+  FastDiv divVecs, divStrips, divBands;
+};
+
+union Vec8 {
+  uintx4 raw;
+  __half2 h2[4];
+};
+
+template <class OutT> struct PutVec;
+template <> struct PutVec<__half> {
+  static __device__ __forceinline__ void put(__half *p, const float (&v)[8]) {
+    Vec8 o;
+#pragma unroll
+    for (int i = 0; i != 4; ++i)
+      o.h2[i] = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
+    __builtin_nontemporal_store(o.raw, reinterpret_cast<uintx4 *>(p));
+  }
+};
+template <> struct PutVec<float> {
+  static __device__ __forceinline__ void put(float *p, const float (&v)[8]) {
+    __builtin_nontemporal_store(floatx4{v[0], v[1], v[2], v[3]},
+                                reinterpret_cast<floatx4 *>(p));
+    __builtin_nontemporal_store(floatx4{v[4], v[5], v[6], v[7]},
+                                reinterpret_cast<floatx4 *>(p + 4));
+  }
+};
+
+template <int S, class OutT>
+__global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
+    RowsArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
+    const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  constexpr int kAhead = Ring<S>::kAhead, kSlots = Ring<S>::kSlots;
+  extern __shared__ __align__(16) char lds[];
+  const DepthwiseDesc &d = a.d;
+  const uint32_t t = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(int(t >> 6));
+  const uint32_t lane = t & 63;
+
+  // Workgroup -> (image, band, strip), strip fastest; each XCD, which takes
+  // workgroups round-robin, gets a contiguous run: neighbouring bands share
+  // their halo rows in its L2.
+  const uint32_t walker = xcdSwizzle(blockIdx.x, gridDim.x);
+  uint32_t q = a.divStrips(walker);
+  const uint32_t strip = walker - q * a.strips;
+  const uint32_t b = a.divBands(q);
+  const uint32_t band = q - b * a.bands;
+  const uint32_t oh0 = band * a.rowsOut, ow0 = strip * a.colsOut;
+  const uint32_t steps =
+      oh0 + a.rowsOut <= d.outH ? a.rowsOut : d.outH - oh0;
+  const int ih0 = int(oh0 * S) - d.padH, iw0 = int(ow0 * S) - d.padW;
+  const uint32_t pixelBytes = d.channels * 2;
+  // relative input rows [0, rowsIn) are what the band reads
+  const uint32_t rowsIn = (steps - 1) * S + 3;
+
+  if (wave >= kComputeWaves) {
+    // ---- loaders.  Load L of a row fills bytes [1024 L, 1024 L + 1024) of
+    // its slot: 16-byte unit u = 64 L + lane is channel vector u % vecs of
+    // strip column u / vecs.  Loader l takes L = l, l + kLoaderWaves, ...
+    const int loader = wave - kComputeWaves;
+    const __amdgpu_buffer_rsrc_t inBuf = bufferOf(in, a.inBytes);
+    uint32_t unitByte[kOwnLoads]; // from the strip's first column, or kNoByte
+#pragma unroll
+    for (int own = 0; own != kOwnLoads; ++own) {
+      const uint32_t u = (own * kLoaderWaves + loader) * 64 + lane;
+      const uint32_t col = a.divVecs(u);
+      const int iw = iw0 + int(col);
+      unitByte[own] = col < a.colsIn && iw >= int(d.loW) && iw < int(d.hiW)
+                          ? uint32_t(iw) * pixelBytes + (u - col * a.vecs) * 16
+                          : kNoByte;
+    }
+    const uint32_t imageByte = b * d.inH * d.inW * pixelBytes;
+    const uint32_t rowBytes = d.inW * pixelBytes;
+    uint32_t next = 0; // the relative row loaded next
+    auto loadRow = [&] {
+      const int ih = ih0 + int(next);
+      const bool ok = next < rowsIn && ih >= int(d.loH) && ih < int(d.hiH);
+      const uint32_t rowByte =
+          ok ? imageByte + uint32_t(ih) * rowBytes : kNoByte;
+      char *slot = lds + (next % kSlots) * kSlotBytes;
+#pragma unroll
+      for (int own = 0; own != kOwnLoads; ++own)
+        // (a sum with kNoByte in it lies beyond the buffer: zeros)
+        loadToLds<kStreamingLoad>(
+            inBuf, (LdsPtr)(slot + (own * kLoaderWaves + loader) * 1024),
+            (rowByte | unitByte[own]) >= kNoByte ? kNoByte
+                                                 : rowByte + unitByte[own],
+            0);
+      ++next;
+    };
+    // rows of steps 0 .. kAhead - 1
+#pragma unroll 1
+    for (int r = 0; r != (kAhead - 1) * S + 3; ++r)
+      loadRow();
+    for (uint32_t j = 0; j < steps; ++j) {
+      // step j's rows have landed when all but the rows of the kAhead - 1
+      // steps behind it have
+      MXK_WAIT_VMCNT((kAhead - 1) * S * kOwnLoads);
+      stepBarrier();
+      // (the rows before step j's are free: everybody is through step j - 1)
+#pragma unroll
+      for (int r = 0; r != S; ++r)
+        loadRow();
+    }
+    MXK_WAIT_VMCNT(0);
+    return;
+  }
+
+  // ---- compute waves.  Thread t: strip column t / vecs, channel vector
+  // t % vecs.
+  const uint32_t col = a.divVecs(t), v = t - col * a.vecs;
+  const uint32_t ow = ow0 + col;
+  const bool active = col < a.colsOut && ow < d.outW;
+  const uint32_t c = (active ? v : 0) * 8;
+  Vec8 taps[9];
+#pragma unroll
+  for (int tap = 0; tap != 9; ++tap)
+    taps[tap].raw =
+        *reinterpret_cast<const uintx4 *>(w + tap * d.channels + c);
+  float biasV[8];
+#pragma unroll
+  for (int e = 0; e != 8; ++e)
+    biasV[e] = bias ? Load<OutT>::at(bias, c + e, 0) : 0.0f;
+  // the thread's window in a row slot: columns col * S .. + 2
+  const uint32_t windowByte = ((active ? col : 0) * S * a.vecs + v) * 16;
+  OutT *dst = out + ((size_t(b) * d.outH + oh0) * d.outW + ow) * d.channels + c;
+  const size_t outRow = size_t(d.outW) * d.channels;
+  uint32_t slot = 0; // slot of relative row j * S
+  for (uint32_t j = 0; j < steps; ++j) {
+    stepBarrier(); // step j's rows are in the ring
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e != 8; ++e)
+      acc[e] = biasV[e];
+    uint32_t rowSlot = slot;
+#pragma unroll
+    for (int kh = 0; kh != 3; ++kh) {
+      const char *row = lds + rowSlot * kSlotBytes + windowByte;
+#pragma unroll
+      for (int kw = 0; kw != 3; ++kw) {
+        Vec8 x;
+        x.raw = *reinterpret_cast<const uintx4 *>(row + kw * a.vecs * 16);
+        const Vec8 &k = taps[kh * 3 + kw];
+#pragma unroll
+        for (int e = 0; e != 4; ++e) {
+          const float2 xf = __half22float2(x.h2[e]);
+          const float2 kf = __half22float2(k.h2[e]);
+          acc[2 * e] = fmaf(xf.x, kf.x, acc[2 * e]);
+          acc[2 * e + 1] = fmaf(xf.y, kf.y, acc[2 * e + 1]);
+        }
+      }
+      rowSlot = rowSlot + 1 == kSlots ? 0 : rowSlot + 1;
+    }
+    // (the reads are done - their values were used - before the next
+    // barrier lets the loaders overwrite the rows)
+    if (active)
+      PutVec<OutT>::put(dst, acc);
+    dst += outRow;
+    slot += S;
+    slot -= slot >= kSlots ? kSlots : 0;
+  }
+}
+
+/// Strips, bands and their sizes for a chip of `cus` compute units; false
+/// when the kernel does not take the layer.
+bool shapeFor(const DepthwiseDesc &d, uint32_t cus, RowsArgs &a) {
+  if (d.kH != 3 || d.kW != 3 || d.dilH != 1 || d.dilW != 1 ||
+      d.strideH != d.strideW || (d.strideH != 1 && d.strideH != 2) ||
+      d.channels % 8 != 0 || d.channels == 0 || d.inDilH != 1 ||
+      d.inDilW != 1 || d.batch == 0 || d.outH == 0 || d.outW == 0)
+    return false;
+  const uint32_t s = d.strideH;
+  a.vecs = d.channels / 8;
+  // a strip's input row fits a slot, its output row the compute threads
+  const uint32_t unitsPerSlot = kSlotBytes / 16;
+  if (a.vecs * 3 > unitsPerSlot || a.vecs > uint32_t(kComputeThreads))
+    return false;
+  const uint32_t maxColsIn = unitsPerSlot / a.vecs;
+  uint32_t maxColsOut = (maxColsIn - 3) / s + 1;
+  if (maxColsOut > kComputeThreads / a.vecs)
+    maxColsOut = kComputeThreads / a.vecs;
+  a.strips = (d.outW + maxColsOut - 1) / maxColsOut;
+  a.colsOut = (d.outW + a.strips - 1) / a.strips;
+  a.colsIn = (a.colsOut - 1) * s + 3;
+  // about one workgroup per CU
+  const uint64_t columns = uint64_t(d.batch) * a.strips;
+  uint64_t bands = cus / columns;
+  if (bands < 1)
+    bands = 1;
+  if (bands > d.outH)
+    bands = d.outH;
+  a.rowsOut = uint32_t((d.outH + bands - 1) / bands);
+  a.bands = (d.outH + a.rowsOut - 1) / a.rowsOut;
+  return true;
+}
+
+template <int S, class OutT>
+hipError_t run(const RowsArgs &a, const void *in, const void *w,
+               const void *bias, void *out, hipStream_t stream) {
+  constexpr int ldsBytes = Ring<S>::kSlots * kSlotBytes;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void *>(&depthwiseRowsKernel<S, OutT>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+  if (attr != hipSuccess)
+    return attr;
+  const uint32_t blocks = a.d.batch * a.strips * a.bands;
+  hipLaunchKernelGGL((depthwiseRowsKernel<S, OutT>), dim3(blocks),
+                     dim3(kRowsThreads), ldsBytes, stream, a,
+                     static_cast<const __half *>(in),
+                     static_cast<const __half *>(w),
+                     static_cast<const OutT *>(bias), static_cast<OutT *>(out));
+  return hipGetLastError();
+}
+
+} // namespace
+
+bool depthwiseRowsTakes(const DepthwiseDesc &d, int inType) {
+  RowsArgs a;
+  if (inType != kHalf || d.cus == 0 || !shapeFor(d, d.cus, a))
+    return false;
+  const uint64_t inBytes = uint64_t(d.batch) * d.inH * d.inW * d.channels * 2;
+  const uint64_t blocks = uint64_t(d.batch) * a.strips * a.bands;
+  return inBytes < kNoByte && blocks < 0x7fffffffull;
+}
+
+DepthwiseRowsLaunch depthwiseRowsLaunchShape(const DepthwiseDesc &d) {
+  RowsArgs a{};
+  DepthwiseRowsLaunch l{};
+  if (d.cus == 0 || !shapeFor(d, d.cus, a))
+    return l;
+  l.strips = a.strips, l.colsOut = a.colsOut;
+  l.bands = a.bands, l.rowsOut = a.rowsOut;
+  l.workgroups = uint64_t(d.batch) * a.strips * a.bands;
+  l.ringRows = d.strideH == 2 ? Ring<2>::kSlots : Ring<1>::kSlots;
+  l.loaderWaves = kLoaderWaves;
+  return l;
+}
+
+hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
+                               const void *in, const void *weightsPacked,
+                               const void *bias, void *out,
+                               hipStream_t stream) {
+  if (!depthwiseRowsTakes(d, inType) ||
+      (outType != kHalf && outType != kFloat))
+    return hipErrorInvalidValue;
+  RowsArgs a{};
+  shapeFor(d, d.cus, a);
+  a.d = d;
+  a.inBytes = uint32_t(uint64_t(d.batch) * d.inH * d.inW * d.channels * 2);
+  a.divVecs = makeFastDiv(a.vecs);
+  a.divStrips = makeFastDiv(a.strips);
+  a.divBands = makeFastDiv(a.bands);
+  const bool s1 = d.strideH == 1;
+  if (outType == kHalf)
+    return s1 ? run<1, __half>(a, in, weightsPacked, bias, out, stream)
+              : run<2, __half>(a, in, weightsPacked, bias, out, stream);
+  return s1 ? run<1, float>(a, in, weightsPacked, bias, out, stream)
+            : run<2, float>(a, in, weightsPacked, bias, out, stream);
+}
+
+} // namespace mxk

@@ -288,9 +288,12 @@ struct DepthwiseDesc {
   // Output pixels per workgroup tile, chosen by the planner so that the
   // input patch of a tile fits a third of a CU's LDS.
   uint32_t tileH, tileW;
-  // 1: the dense-loading small-workgroup kernel (3x3 taps, dilation 1,
-  // stride 1 or 2) runs instead of the LDS-tiled one.
+  // 3x3 taps, dilation 1, stride 1 or 2 - 1: the dense-loading
+  // small-workgroup kernel, 2: the persistent kernel with a ring of input rows
+  // in LDS (launchDepthwiseRows), instead of the LDS-tiled one.
   uint32_t dense3x3;
+  // Compute units the persistent kernel spreads its workgroups over.
+  uint32_t cus = 0;
   // Zeros stuffed between input elements, as in IgemmDesc; other than 1 the
   // direct kernel of launchDepthwiseDirect runs.
   uint32_t inDilH = 1, inDilW = 1;
@@ -301,6 +304,19 @@ hipError_t launchDepthwise3x3(const DepthwiseDesc &d, int inType,
                                  int outType, const void *in,
                                  const void *weightsPacked, const void *bias,
                                  void *out, hipStream_t stream);
+/// The same layers (3x3 taps, dilation 1, stride 1 or 2) by persistent
+/// workgroups, about one per compute unit (d.cus), each walking down a band
+/// of output rows of a column strip with the input rows in an LDS ring.
+bool depthwiseRowsTakes(const DepthwiseDesc &d, int inType);
+struct DepthwiseRowsLaunch {
+  uint32_t strips, colsOut, bands, rowsOut, ringRows, loaderWaves;
+  uint64_t workgroups;
+};
+DepthwiseRowsLaunch depthwiseRowsLaunchShape(const DepthwiseDesc &d);
+hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
+                               const void *in, const void *weightsPacked,
+                               const void *bias, void *out,
+                               hipStream_t stream);
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream);

@@ -201,6 +201,11 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       if (v > 2)
         throw invalid_option("'" + sub + "': Must be 0, 1 or 2");
       pc.patch = int(v);
+    } else if (m.first == "rowRing") {
+      const unsigned v = requireUnsigned(sub, m.second);
+      if (v > 1)
+        throw invalid_option("'" + sub + "': Must be 0 or 1");
+      pc.rowRing = int(v);
     } else if (m.first == "tileH") {
       pc.tileH = requireUnsigned(sub, m.second);
     } else if (m.first == "tileW") {

@@ -46,6 +46,10 @@ struct PlanConstraints {
   int patch = -1;
   /// Output tile of the depthwise kernel; 0 = planner's choice.
   unsigned tileH = 0, tileW = 0;
+  /// The depthwise 3x3 kernel whose persistent workgroups keep a ring of
+  /// input rows in LDS: -1 planner's choice, 0 never, 1 whenever it can take
+  /// the layer.
+  int rowRing = -1;
   std::string text; // the JSON as given, kept for reporting and cache keys
 };
 

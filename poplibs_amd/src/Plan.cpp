@@ -878,6 +878,26 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     // An explicit tile asks for the LDS-tiled kernel.
     d.dense3x3 = !s.inputDilated() && !(pc.tileH || pc.tileW) &&
                  mxk::depthwise3x3Takes(d, mxk::kHalf);
+    // Layers that give every CU a band of at least four output rows go to
+    // the persistent kernel with a ring of input rows in LDS: its start-up
+    // (seven rows before the first output) wants rows to spread over.
+    if (d.dense3x3 && pc.rowRing != 0) {
+      d.cus = gfx950::numCUs;
+      const mxk::DepthwiseRowsLaunch l = mxk::depthwiseRowsLaunchShape(d);
+      const bool takes = mxk::depthwiseRowsTakes(d, mxk::kHalf);
+      if (pc.rowRing == 1 && !takes)
+        throw poplar::invalid_option(
+            "planConstraints gfx950 rowRing: that kernel takes 3x3 taps, "
+            "stride 1 or 2, channels in vectors of 8, at most 256 to a "
+            "pixel");
+      if (takes && (pc.rowRing == 1 ||
+                    (l.workgroups * 2 >= gfx950::numCUs && l.rowsOut >= 4)))
+        d.dense3x3 = 2;
+    } else if (pc.rowRing == 1) {
+      throw poplar::invalid_option(
+          "planConstraints gfx950 rowRing: the layer is not one the "
+          "depthwise 3x3 kernels take");
+    }
     if (!s.inputDilated() && (pc.tileH || pc.tileW)) {
       d.tileH = pc.tileH ? pc.tileH : d.tileH;
       d.tileW = pc.tileW ? pc.tileW : d.tileW;
@@ -924,6 +944,9 @@ std::string mxconv_plan::describe() const {
            : depthwise.inDilH != 1 || depthwise.inDilW != 1
                ? "depthwise direct (vector ALU, one thread per output "
                  "vector, dilated input)"
+           : depthwise.dense3x3 == 2
+               ? "depthwise direct (vector ALU, input rows streamed through "
+                 "an LDS ring by persistent workgroups)"
            : depthwise.dense3x3
                ? "depthwise direct (vector ALU, dense row loads, small "
                  "workgroups)"
@@ -1025,6 +1048,15 @@ std::string mxconv_plan::describe() const {
     if (!d.dense3x3)
       os << "        output tile H x W          " << d.tileH << " x "
          << d.tileW << "\n";
+    if (d.dense3x3 == 2) {
+      const mxk::DepthwiseRowsLaunch l = mxk::depthwiseRowsLaunchShape(d);
+      os << "        workgroups                 " << l.workgroups << " on "
+         << d.cus << " CUs: per image " << l.strips << " strips of "
+         << l.colsOut << " output columns x " << l.bands << " bands of "
+         << l.rowsOut << " output rows; ring of " << l.ringRows
+         << " input rows in LDS filled by " << l.loaderWaves
+         << " loader waves\n";
+    }
     os << "        packed weights             [" << d.kH * d.kW << "]["
        << d.channels << "]\n";
   } else {

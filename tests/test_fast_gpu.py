@@ -177,6 +177,55 @@ def test_depthwise_3x3_plan_reports_its_kernel_and_tile_override(oracle):
     _run(oracle, p, 7, 1e-3, "depthwise direct", options=opts)
 
 
+ROW_RING = {"planConstraints": '{"gfx950": {"rowRing": 1}}'}
+RING = "input rows streamed through an LDS ring"
+
+
+# The persistent kernel with a ring of input rows in LDS, forced onto the same
+# shapes (the planner keeps it for layers that fill the chip): bands of one
+# row, strips narrower than the image and wider, images smaller than a ring.
+@pytest.mark.parametrize("kw", DW3X3_CASES + [
+    # several strips (28 channel vectors per pixel: 13 output columns each)
+    # and bands of more than one row
+    dict(batch=48, field=(40, 60), kernel=(3, 3), groups=224, stride=2,
+         pad=1),
+    # stride 1, rows longer than a strip
+    dict(batch=40, field=(30, 150), kernel=(3, 3), groups=64, stride=1,
+         pad=1),
+])
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_depthwise_row_ring_matches_oracle(oracle, kw, out_type):
+    p = make_params(pa.HALF, out_type, **kw)
+    print("case", p, flush=True)
+    assert RING in pa.Plan(p, ROW_RING).describe()
+    _run(oracle, p, 8, 1e-3, "depthwise direct", options=ROW_RING)
+
+
+def test_depthwise_row_ring_pm1_exact(oracle):
+    for kw in (DW3X3_CASES[0], DW3X3_CASES[3], DW3X3_CASES[6]):
+        p = make_params(pa.HALF, pa.FLOAT, **kw)
+        _run(oracle, p, 9, 0, "depthwise direct", dist="pm1",
+             options=ROW_RING)
+
+
+def test_depthwise_row_ring_plan_choice():
+    big = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                      groups=96, stride=2, pad=1)
+    text = pa.Plan(big).describe()
+    assert RING in text, text
+    assert ("256 on 256 CUs: per image 2 strips of 28 output columns x 4 "
+            "bands of 14 output rows") in text, text
+    off = pa.Plan(big, {"planConstraints": '{"gfx950": {"rowRing": 0}}'})
+    assert "dense row loads" in off.describe()
+    # few rows per CU: the small workgroups stay
+    small = make_params(pa.HALF, **DW3X3_CASES[0])
+    assert "dense row loads" in pa.Plan(small).describe()
+    # not a 3x3 kernel: the constraint cannot be met
+    with pytest.raises(pa.MxconvError):
+        pa.Plan(make_params(pa.HALF, batch=2, field=(20, 20), kernel=(5, 5),
+                            groups=32, pad=2), ROW_RING)
+
+
 def test_depthwise_fp32_out_pm1_exact(oracle):
     p = make_params(pa.HALF, pa.FLOAT, **DW_CASES[1])
     _run(oracle, p, 5, 0, "depthwise direct", dist="pm1")
