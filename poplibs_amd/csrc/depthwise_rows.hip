@@ -16,6 +16,16 @@
 // one contiguous run.  One barrier per output row.  Several loader waves,
 // because one wave does not issue loads as fast as HBM delivers them (ten
 // instructions per load).
+//
+// depthwiseRowsDeltaKernel is the same walk for the layer's weight deltas,
+//   dW[kh][kw][c] = sum over b, oh, ow of
+//       deltas[b][oh][ow][c] * acts[b][oh S + kh - padH][ow S + kw - padW][c]
+// (the pass PopLibs runs as a convolution of its own,
+// lib/poplin/Convolution.cpp:3437-3483 calculateWeightDeltas): a second,
+// smaller ring holds the rows of the deltas, a thread keeps the 9 x 8 sums of
+// its output column and channel vector in registers down the band, the
+// columns meet in LDS at the end, and every workgroup leaves one [9][C] fp32
+// tile, which depthwiseDeltaSumKernel adds in order.
 #include "igemm_common.hpp"
 
 namespace mxk {
@@ -74,6 +84,42 @@ template <> struct PutVec<float> {
   }
 };
 
+/// What a loader wave knows of a strip's rows of one tensor: per own load,
+/// the byte of its 16-byte unit from the row's first pixel, or kNoByte.
+/// LOADS: loads per row and loader wave; row slots are LOADS * kLoaderWaves KB.
+template <int LOADS> struct StripRow {
+  uint32_t unitByte[LOADS];
+  /// Columns [first, first + cols) of rows whose valid columns are [lo, hi).
+  __device__ __forceinline__ void setup(int first, uint32_t cols, int lo,
+                                        int hi, uint32_t pixelBytes,
+                                        uint32_t vecs, const FastDiv &divVecs,
+                                        int loader, uint32_t lane) {
+#pragma unroll
+    for (int own = 0; own != LOADS; ++own) {
+      const uint32_t u = (own * kLoaderWaves + loader) * 64 + lane;
+      const uint32_t col = divVecs(u);
+      const int at = first + int(col);
+      unitByte[own] = col < cols && at >= lo && at < hi
+                          ? uint32_t(at) * pixelBytes + (u - col * vecs) * 16
+                          : kNoByte;
+    }
+  }
+  /// The row that starts at rowByte of the buffer (kNoByte: a row of zeros)
+  /// into `slot`.
+  __device__ __forceinline__ void load(const __amdgpu_buffer_rsrc_t &buf,
+                                       char *slot, uint32_t rowByte,
+                                       int loader) const {
+#pragma unroll
+    for (int own = 0; own != LOADS; ++own)
+      // (anything with kNoByte in it lies beyond the buffer: zeros)
+      loadToLds<kStreamingLoad>(
+          buf, (LdsPtr)(slot + (own * kLoaderWaves + loader) * 1024),
+          (rowByte | unitByte[own]) >= kNoByte ? kNoByte
+                                               : rowByte + unitByte[own],
+          0);
+  }
+};
+
 template <int S, class OutT>
 __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
     RowsArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
@@ -107,16 +153,9 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
     // strip column u / vecs.  Loader l takes L = l, l + kLoaderWaves, ...
     const int loader = wave - kComputeWaves;
     const __amdgpu_buffer_rsrc_t inBuf = bufferOf(in, a.inBytes);
-    uint32_t unitByte[kOwnLoads]; // from the strip's first column, or kNoByte
-#pragma unroll
-    for (int own = 0; own != kOwnLoads; ++own) {
-      const uint32_t u = (own * kLoaderWaves + loader) * 64 + lane;
-      const uint32_t col = a.divVecs(u);
-      const int iw = iw0 + int(col);
-      unitByte[own] = col < a.colsIn && iw >= int(d.loW) && iw < int(d.hiW)
-                          ? uint32_t(iw) * pixelBytes + (u - col * a.vecs) * 16
-                          : kNoByte;
-    }
+    StripRow<kOwnLoads> strip;
+    strip.setup(iw0, a.colsIn, int(d.loW), int(d.hiW), pixelBytes, a.vecs,
+                a.divVecs, loader, lane);
     const uint32_t imageByte = b * d.inH * d.inW * pixelBytes;
     const uint32_t rowBytes = d.inW * pixelBytes;
     uint32_t next = 0; // the relative row loaded next
@@ -125,15 +164,7 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
       const bool ok = next < rowsIn && ih >= int(d.loH) && ih < int(d.hiH);
       const uint32_t rowByte =
           ok ? imageByte + uint32_t(ih) * rowBytes : kNoByte;
-      char *slot = lds + (next % kSlots) * kSlotBytes;
-#pragma unroll
-      for (int own = 0; own != kOwnLoads; ++own)
-        // (a sum with kNoByte in it lies beyond the buffer: zeros)
-        loadToLds<kStreamingLoad>(
-            inBuf, (LdsPtr)(slot + (own * kLoaderWaves + loader) * 1024),
-            (rowByte | unitByte[own]) >= kNoByte ? kNoByte
-                                                 : rowByte + unitByte[own],
-            0);
+      strip.load(inBuf, lds + (next % kSlots) * kSlotBytes, rowByte, loader);
       ++next;
     };
     // rows of steps 0 .. kAhead - 1
@@ -206,6 +237,178 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
     dst += outRow;
     slot += S;
     slot -= slot >= kSlots ? kSlots : 0;
+  }
+}
+
+
+// ---- weight deltas
+
+constexpr int kDeltaLoads = 8; // 1 KB loads per slot of a row of deltas
+constexpr int kDeltaSlotBytes = kDeltaLoads * 1024;
+constexpr int kOwnDeltaLoads = kDeltaLoads / kLoaderWaves;
+constexpr int kSumRow = 73; // floats a thread leaves for the columns' meeting
+
+/// Rings of the weight-delta kernel: rows of activations as in the forward
+/// kernel, one row of deltas per step; four steps' rows on the way at stride
+/// 1, three at stride 2 (140 / 124 KB of LDS).
+template <int S> struct DeltaRing {
+  static constexpr int kAhead = S == 2 ? 3 : 4;
+  static constexpr int kSlots = kAhead * S + 3;
+  static constexpr int kDeltaSlots = kAhead + 1;
+  static constexpr int kBytes =
+      kSlots * kSlotBytes + kDeltaSlots * kDeltaSlotBytes;
+  static_assert(kBytes >= kComputeThreads * kSumRow * 4, "the sums fit");
+  static_assert(kBytes <= 160 * 1024, "LDS of a CU");
+};
+
+/// partial[walker][tap][c] = the walker's band's sum.
+template <int S>
+__global__ __launch_bounds__(kRowsThreads) void depthwiseRowsDeltaKernel(
+    RowsArgs a, const __half *__restrict__ acts,
+    const __half *__restrict__ deltas, uint32_t deltaBytes,
+    float *__restrict__ partial) {
+  using R = DeltaRing<S>;
+  constexpr int kAhead = R::kAhead, kSlots = R::kSlots;
+  constexpr int kDeltaSlots = R::kDeltaSlots;
+  extern __shared__ __align__(16) char lds[];
+  char *deltaRing = lds + kSlots * kSlotBytes;
+  const DepthwiseDesc &d = a.d;
+  const uint32_t t = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(int(t >> 6));
+  const uint32_t lane = t & 63;
+
+  const uint32_t walker = xcdSwizzle(blockIdx.x, gridDim.x);
+  uint32_t q = a.divStrips(walker);
+  const uint32_t strip = walker - q * a.strips;
+  const uint32_t b = a.divBands(q);
+  const uint32_t band = q - b * a.bands;
+  const uint32_t oh0 = band * a.rowsOut, ow0 = strip * a.colsOut;
+  const uint32_t steps =
+      oh0 + a.rowsOut <= d.outH ? a.rowsOut : d.outH - oh0;
+  const int ih0 = int(oh0 * S) - d.padH, iw0 = int(ow0 * S) - d.padW;
+  const uint32_t pixelBytes = d.channels * 2;
+  const uint32_t rowsIn = (steps - 1) * S + 3;
+
+  if (wave >= kComputeWaves) {
+    // ---- loaders: per step the new rows of activations, then the step's
+    // row of deltas (output columns [ow0, ow0 + colsOut) of row oh0 + j).
+    const int loader = wave - kComputeWaves;
+    const __amdgpu_buffer_rsrc_t actBuf = bufferOf(acts, a.inBytes);
+    const __amdgpu_buffer_rsrc_t deltaBuf = bufferOf(deltas, deltaBytes);
+    StripRow<kOwnLoads> actStrip;
+    actStrip.setup(iw0, a.colsIn, int(d.loW), int(d.hiW), pixelBytes, a.vecs,
+                   a.divVecs, loader, lane);
+    StripRow<kOwnDeltaLoads> deltaStrip;
+    deltaStrip.setup(int(ow0), a.colsOut, 0, int(d.outW), pixelBytes, a.vecs,
+                     a.divVecs, loader, lane);
+    const uint32_t imageByte = b * d.inH * d.inW * pixelBytes;
+    const uint32_t rowBytes = d.inW * pixelBytes;
+    const uint32_t deltaImageByte = b * d.outH * d.outW * pixelBytes;
+    const uint32_t deltaRowBytes = d.outW * pixelBytes;
+    uint32_t next = 0, nextStep = 0;
+    auto loadStep = [&](int rows) {
+      for (int r = 0; r != rows; ++r) {
+        const int ih = ih0 + int(next);
+        const bool ok = next < rowsIn && ih >= int(d.loH) && ih < int(d.hiH);
+        actStrip.load(actBuf, lds + (next % kSlots) * kSlotBytes,
+                      ok ? imageByte + uint32_t(ih) * rowBytes : kNoByte,
+                      loader);
+        ++next;
+      }
+      deltaStrip.load(deltaBuf,
+                      deltaRing + (nextStep % kDeltaSlots) * kDeltaSlotBytes,
+                      nextStep < steps ? deltaImageByte +
+                                             (oh0 + nextStep) * deltaRowBytes
+                                       : kNoByte,
+                      loader);
+      ++nextStep;
+    };
+    // steps 0 .. kAhead - 1, in the order the loop goes on in: the counts
+    // below rely on it
+    loadStep(3);
+#pragma unroll 1
+    for (int s = 1; s != kAhead; ++s)
+      loadStep(S);
+    for (uint32_t j = 0; j < steps; ++j) {
+      MXK_WAIT_VMCNT((kAhead - 1) * (S * kOwnLoads + kOwnDeltaLoads));
+      stepBarrier();
+      loadStep(S);
+    }
+    MXK_WAIT_VMCNT(0);
+    // (the rings are the columns' meeting place next: nothing of these
+    // loads' may land later)
+    stepBarrier();
+    return;
+  }
+
+  // ---- compute waves.  Thread t: strip column t / vecs, channel vector
+  // t % vecs; a thread beyond the strip's columns reads zeros for deltas.
+  const uint32_t colOf = a.divVecs(t), v = t - colOf * a.vecs;
+  const bool inStrip = colOf < a.colsOut;
+  const uint32_t col = inStrip ? colOf : 0;
+  const uint32_t windowByte = (col * S * a.vecs + v) * 16;
+  // (8 KB hold 512 units: any t has a unit, of zeros beyond the strip)
+  const uint32_t deltaByte = t * 16;
+  float acc[9][8];
+#pragma unroll
+  for (int tap = 0; tap != 9; ++tap)
+#pragma unroll
+    for (int e = 0; e != 8; ++e)
+      acc[tap][e] = 0.0f;
+  uint32_t slot = 0, deltaSlot = 0;
+  for (uint32_t j = 0; j < steps; ++j) {
+    stepBarrier();
+    Vec8 dz;
+    dz.raw = *reinterpret_cast<const uintx4 *>(
+        deltaRing + deltaSlot * kDeltaSlotBytes + deltaByte);
+    float dzf[8];
+#pragma unroll
+    for (int e = 0; e != 4; ++e) {
+      const float2 f = __half22float2(dz.h2[e]);
+      dzf[2 * e] = f.x, dzf[2 * e + 1] = f.y;
+    }
+    uint32_t rowSlot = slot;
+#pragma unroll
+    for (int kh = 0; kh != 3; ++kh) {
+      const char *row = lds + rowSlot * kSlotBytes + windowByte;
+#pragma unroll
+      for (int kw = 0; kw != 3; ++kw) {
+        Vec8 x;
+        x.raw = *reinterpret_cast<const uintx4 *>(row + kw * a.vecs * 16);
+#pragma unroll
+        for (int e = 0; e != 4; ++e) {
+          const float2 xf = __half22float2(x.h2[e]);
+          acc[kh * 3 + kw][2 * e] =
+              fmaf(xf.x, dzf[2 * e], acc[kh * 3 + kw][2 * e]);
+          acc[kh * 3 + kw][2 * e + 1] =
+              fmaf(xf.y, dzf[2 * e + 1], acc[kh * 3 + kw][2 * e + 1]);
+        }
+      }
+      rowSlot = rowSlot + 1 == kSlots ? 0 : rowSlot + 1;
+    }
+    slot += S;
+    slot -= slot >= kSlots ? kSlots : 0;
+    deltaSlot = deltaSlot + 1 == kDeltaSlots ? 0 : deltaSlot + 1;
+  }
+  // The columns meet: every thread leaves its 72 sums, then thread o adds
+  // those of output o = (tap, channel) over the strip's columns, in order.
+  stepBarrier(); // the loaders' last (zero) rows have landed, all reads done
+  float *sums = reinterpret_cast<float *>(lds);
+#pragma unroll
+  for (int tap = 0; tap != 9; ++tap)
+#pragma unroll
+    for (int e = 0; e != 8; ++e)
+      sums[t * kSumRow + tap * 8 + e] = inStrip ? acc[tap][e] : 0.0f;
+  __syncthreads();
+  const uint32_t outputs = 9 * d.channels;
+  float *dst = partial + size_t(walker) * outputs;
+  for (uint32_t o = t; o < outputs; o += kComputeThreads) {
+    const uint32_t tap = o / d.channels, c = o - tap * d.channels;
+    const float *from = sums + (c >> 3) * kSumRow + tap * 8 + (c & 7);
+    float sum = 0.0f;
+    for (uint32_t k = 0; k != a.colsOut; ++k)
+      sum += from[k * a.vecs * kSumRow];
+    dst[o] = sum;
   }
 }
 
@@ -304,6 +507,51 @@ hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
               : run<2, __half>(a, in, weightsPacked, bias, out, stream);
   return s1 ? run<1, float>(a, in, weightsPacked, bias, out, stream)
             : run<2, float>(a, in, weightsPacked, bias, out, stream);
+}
+
+bool depthwiseRowsDeltaTakes(const DepthwiseDesc &d) {
+  const uint64_t deltaBytes =
+      uint64_t(d.batch) * d.outH * d.outW * d.channels * 2;
+  return depthwiseRowsTakes(d, kHalf) && deltaBytes < kNoByte;
+}
+
+size_t depthwiseRowsDeltaWorkspaceBytes(const DepthwiseDesc &d) {
+  const DepthwiseRowsLaunch l = depthwiseRowsLaunchShape(d);
+  return size_t(l.workgroups) * 9 * d.channels * sizeof(float);
+}
+
+hipError_t launchDepthwiseRowsDeltas(const DepthwiseDesc &d, const void *acts,
+                                     const void *deltas, void *partial,
+                                     uint32_t *walkers, hipStream_t stream) {
+  if (!depthwiseRowsDeltaTakes(d) || !partial)
+    return hipErrorInvalidValue;
+  RowsArgs a{};
+  shapeFor(d, d.cus, a);
+  a.d = d;
+  a.inBytes = uint32_t(uint64_t(d.batch) * d.inH * d.inW * d.channels * 2);
+  a.divVecs = makeFastDiv(a.vecs);
+  a.divStrips = makeFastDiv(a.strips);
+  a.divBands = makeFastDiv(a.bands);
+  const uint32_t deltaBytes =
+      uint32_t(uint64_t(d.batch) * d.outH * d.outW * d.channels * 2);
+  const uint32_t blocks = d.batch * a.strips * a.bands;
+  *walkers = blocks;
+  auto run = [&](auto stride) -> hipError_t {
+    constexpr int S = decltype(stride)::value;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&depthwiseRowsDeltaKernel<S>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, DeltaRing<S>::kBytes);
+    if (attr != hipSuccess)
+      return attr;
+    hipLaunchKernelGGL(depthwiseRowsDeltaKernel<S>, dim3(blocks),
+                       dim3(kRowsThreads), DeltaRing<S>::kBytes, stream, a,
+                       static_cast<const __half *>(acts),
+                       static_cast<const __half *>(deltas), deltaBytes,
+                       static_cast<float *>(partial));
+    return hipGetLastError();
+  };
+  return d.strideH == 1 ? run(std::integral_constant<int, 1>{})
+                        : run(std::integral_constant<int, 2>{});
 }
 
 } // namespace mxk

@@ -470,6 +470,8 @@ hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
 }
 
 size_t depthwiseWeightDeltaWorkspaceBytes(const DepthwiseDesc &d) {
+  if (d.dense3x3 == 2)
+    return depthwiseRowsDeltaWorkspaceBytes(d);
   return size_t(deltaSlices(d)) * d.kH * d.kW * d.channels * sizeof(float);
 }
 
@@ -491,20 +493,28 @@ hipError_t launchDepthwiseWeightDeltas(const DepthwiseDesc &d, int outType,
     return hipErrorInvalidConfiguration;
   a.items = uint32_t(items);
   a.pixels = uint32_t(pixels);
-  a.slices = deltaSlices(d);
-  deltaBlockShape(d, a.itemsPerBlock, a.slots);
-  a.pixelsPerSlice = uint32_t((pixels + a.slices - 1) / a.slices);
-  a.pixelsPerSlot = (a.pixelsPerSlice + a.slots - 1) / a.slots;
-  a.divVecs = makeFastDiv(a.vecs);
-  a.divOutW = makeFastDiv(d.outW);
-  a.divOutH = makeFastDiv(d.outH);
   float *partial = static_cast<float *>(workspace);
-  const dim3 grid{uint32_t((items + a.itemsPerBlock - 1) / a.itemsPerBlock),
-                  a.slices},
-      block{256};
-  hipLaunchKernelGGL(depthwiseWeightDeltaKernel, grid, block, 0, stream, a,
-                     static_cast<const __half *>(acts),
-                     static_cast<const __half *>(deltas), partial);
+  if (d.dense3x3 == 2) {
+    // persistent workgroups with the rows in LDS rings: one tile each
+    const hipError_t e = launchDepthwiseRowsDeltas(d, acts, deltas, partial,
+                                                   &a.slices, stream);
+    if (e != hipSuccess)
+      return e;
+  } else {
+    a.slices = deltaSlices(d);
+    deltaBlockShape(d, a.itemsPerBlock, a.slots);
+    a.pixelsPerSlice = uint32_t((pixels + a.slices - 1) / a.slices);
+    a.pixelsPerSlot = (a.pixelsPerSlice + a.slots - 1) / a.slots;
+    a.divVecs = makeFastDiv(a.vecs);
+    a.divOutW = makeFastDiv(d.outW);
+    a.divOutH = makeFastDiv(d.outH);
+    const dim3 grid{uint32_t((items + a.itemsPerBlock - 1) / a.itemsPerBlock),
+                    a.slices},
+        block{256};
+    hipLaunchKernelGGL(depthwiseWeightDeltaKernel, grid, block, 0, stream, a,
+                       static_cast<const __half *>(acts),
+                       static_cast<const __half *>(deltas), partial);
+  }
   const uint32_t outputs = a.taps * d.channels;
   const dim3 grid2{(outputs + 15) / 16};
   const dim3 block2{1024};

@@ -317,6 +317,14 @@ hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
                                const void *in, const void *weightsPacked,
                                const void *bias, void *out,
                                hipStream_t stream);
+/// The weight deltas of such a layer the same way: one fp32 tile [9][C] per
+/// workgroup at partial[workgroup], to be added in order; *walkers = their
+/// count.
+bool depthwiseRowsDeltaTakes(const DepthwiseDesc &d);
+size_t depthwiseRowsDeltaWorkspaceBytes(const DepthwiseDesc &d);
+hipError_t launchDepthwiseRowsDeltas(const DepthwiseDesc &d, const void *acts,
+                                     const void *deltas, void *partial,
+                                     uint32_t *walkers, hipStream_t stream);
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
                            const void *bias, void *out, hipStream_t stream);

@@ -328,6 +328,15 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       f.strideH = w.dilH, f.strideW = w.dilW;
       f.dilH = w.strideH, f.dilW = w.strideW;
       f.loH = w.loH, f.hiH = w.hiH, f.loW = w.loW, f.hiW = w.hiW;
+      // 3x3 layers that give every CU a band of rows: the persistent kernel
+      // with the rows of both tensors in LDS rings (as for the forward pass)
+      f.cus = gfx950::numCUs;
+      const mxk::DepthwiseRowsLaunch l = mxk::depthwiseRowsLaunchShape(f);
+      if (options.planConstraints.rowRing != 0 &&
+          mxk::depthwiseRowsDeltaTakes(f) &&
+          (options.planConstraints.rowRing == 1 ||
+           (l.workgroups * 2 >= gfx950::numCUs && l.rowsOut >= 4)))
+        f.dense3x3 = 2;
     }
   }
   // The weight update pass of a dense layer with unit stride and nothing
@@ -1062,9 +1071,18 @@ std::string mxconv_plan::describe() const {
   } else {
     os << "        packed weights             [G][K][Ci][Co]\n";
   }
-  if (depthwiseWeightUpdate)
+  if (depthwiseWeightUpdate) {
     os << "        as a weight update pass    depthwise weight-delta kernel "
-          "on the layer's own tensors\n";
+          "on the layer's own tensors";
+    if (depthwiseForward.dense3x3 == 2) {
+      const mxk::DepthwiseRowsLaunch l =
+          mxk::depthwiseRowsLaunchShape(depthwiseForward);
+      os << ", rows of both streamed through LDS rings by " << l.workgroups
+         << " persistent workgroups (" << l.strips << " strips x " << l.bands
+         << " bands of " << l.rowsOut << " rows per image)";
+    }
+    os << "\n";
+  }
   if (denseWeightUpdate) {
     const auto &f = denseForward;
     const std::size_t m = std::size_t(f.batch) * f.outH * f.outW;

@@ -404,6 +404,76 @@ def test_depthwise_weight_deltas_of_signs_are_exact(oracle):
     np.testing.assert_array_equal(got, oracle.weight_deltas(p, x, dz))
 
 
+ROW_RING = {"planConstraints": '{"gfx950": {"rowRing": 1}}'}
+RING_WU = "rows of both streamed through LDS rings"
+RING_WU_CASES = [
+    # stride 2: strips narrower than the image, bands of one row
+    dict(batch=3, field=(20, 21), kernel=(3, 3), groups=24, stride=2, pad=1),
+    # stride 1, asymmetric padding, several strips (28 vectors per pixel)
+    dict(batch=5, field=(17, 40), kernel=(3, 3), groups=224, stride=1,
+         padLower=(2, 0), padUpper=(0, 1)),
+    # input truncation (negative padding), ragged last strip and band
+    dict(batch=2, field=(29, 71), kernel=(3, 3), groups=40, stride=2,
+         itl=(1, 0), itu=(0, 2), pad=1),
+    # bands of several rows
+    dict(batch=40, field=(36, 30), kernel=(3, 3), groups=16, stride=2, pad=1),
+    # tiny images
+    dict(batch=70, field=(3, 3), kernel=(3, 3), groups=8, pad=1),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kw", RING_WU_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_depthwise_weight_deltas_row_rings(oracle, kw, out_type):
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, out_type, **kw)
+    print("case", p, flush=True)
+    rng = np.random.default_rng(26)
+    C = p.numConvGroups
+    xq, xd = quantize(
+        rng.standard_normal((p.batchSize, C, *p.inputFieldShape)), pa.HALF)
+    dq, dd = quantize(
+        rng.standard_normal((p.batchSize, C, *p.getOutputFieldShape())) * 0.1,
+        pa.HALF)
+    got, plan = run_weight_update(p, xq, dq, options=ROW_RING)
+    assert RING_WU in plan.describe(), plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert got.shape == want.shape
+    tol = 1e-3 if out_type == pa.HALF else 1e-5
+    assert rel_l2(got, want) <= tol, (rel_l2(got, want), plan.describe())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kw", RING_WU_CASES[:3])
+def test_depthwise_weight_deltas_row_rings_of_signs_are_exact(oracle, kw):
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    rng = np.random.default_rng(27)
+    C = p.numConvGroups
+    x = rng.choice([-1.0, 1.0], (p.batchSize, C, *p.inputFieldShape))
+    dz = rng.choice([-1.0, 1.0], (p.batchSize, C, *p.getOutputFieldShape()))
+    got, plan = run_weight_update(p, x.astype(np.float16),
+                                  dz.astype(np.float16), options=ROW_RING)
+    assert RING_WU in plan.describe()
+    np.testing.assert_array_equal(got, oracle.weight_deltas(p, x, dz,
+                                                            threads=8))
+
+
+def test_depthwise_weight_update_row_rings_plan_choice():
+    big = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                      groups=96, stride=2, pad=1)
+    text = pa.WeightUpdatePlan(big).describe()
+    assert RING_WU in text and "256 persistent workgroups" in text, text
+    off = pa.WeightUpdatePlan(
+        big, {"planConstraints": '{"gfx950": {"rowRing": 0}}'}).describe()
+    assert "depthwise weight-delta kernel" in off and RING_WU not in off
+    small = make_params(pa.HALF, **DEPTHWISE_WU_CASES[0])
+    assert RING_WU not in pa.WeightUpdatePlan(small).describe()
+    # a 5 x 5 kernel stays with the slices whatever is asked
+    five = make_params(pa.HALF, **DEPTHWISE_WU_CASES[1])
+    assert RING_WU not in pa.WeightUpdatePlan(five, ROW_RING).describe()
+
+
 @pytest.mark.gpu
 def test_weight_update_applies_scaled_deltas(oracle):
     from gpu_helpers import quantize
