@@ -254,6 +254,10 @@ class TrainingRunner:
                        if l.strip().startswith("kernel ")][0]
         if which == "wu" and "depthwise weight-delta kernel" in text:
             self.kernel = "depthwise weight-delta kernel (vector ALU)"
+            if "streamed through LDS rings" in text:
+                self.kernel = ("depthwise weight-delta kernel (vector ALU, "
+                               "rows of both tensors streamed through LDS "
+                               "rings by persistent workgroups) + ordered sum")
         if which == "wu" and "matrix-core weight-delta kernel" in text:
             self.kernel = ("matrix-core weight-delta kernel on the layer's own "
                            "tensors (MFMA, transposing LDS reads) + ordered sum")
