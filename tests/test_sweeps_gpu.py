@@ -173,3 +173,43 @@ def test_weight_deltas_random_dense_layers(oracle):
         dense += is_dense
         other += not is_dense
     assert dense >= 40 and other >= 20, (dense, other)
+
+
+def test_depthwise_row_rings_random_layers(oracle):
+    """The persistent depthwise 3x3 kernels (forward and weight deltas),
+    forced onto random layers: strips and bands of every raggedness."""
+    from test_weight_update import run_weight_update
+    rng = random.Random(20250614)
+    options = {"planConstraints": json.dumps({"gfx950": {"rowRing": 1}})}
+    fwd = wu = 0
+    for case in range(160):
+        s = rng.choice([1, 2])
+        lo, hi = _pads(rng, (0, 0), 2)
+        kw = dict(batch=rng.randint(1, 9),
+                  field=(rng.randint(3, 45), rng.randint(3, 90)),
+                  kernel=(3, 3), ci=1, co=1, groups=8 * rng.randint(1, 28),
+                  padLower=lo, padUpper=hi, stride=(s, s))
+        if rng.random() < 0.15:
+            kw["itl"] = (rng.randint(0, 1), rng.randint(0, 1))
+        try:
+            p = make_params(pa.HALF, pa.FLOAT, **kw)
+            plan = pa.Plan(p, options)
+        except pa.MxconvError:
+            continue  # no valid convolution
+        print("case", case, kw, flush=True)
+        assert "LDS ring" in plan.describe(), plan.describe()
+        _exact(oracle, p, options, 9000 + case)
+        fwd += 1
+        if case % 2:
+            continue
+        r = np.random.default_rng(9500 + case)
+        C = p.numConvGroups
+        x = r.choice([-1.0, 1.0], (p.batchSize, C, *p.inputFieldShape))
+        dz = r.choice([-1.0, 1.0], (p.batchSize, C, *p.getOutputFieldShape()))
+        got, wplan = run_weight_update(p, x.astype(np.float16),
+                                       dz.astype(np.float16), options=options)
+        assert "LDS rings" in wplan.describe(), wplan.describe()
+        np.testing.assert_array_equal(
+            got, oracle.weight_deltas(p, x, dz, threads=8))
+        wu += 1
+    assert fwd >= 100 and wu >= 50, (fwd, wu)
