@@ -515,9 +515,10 @@ def test_planner_weighs_tilings_and_reports_them():
     p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
                     co=128, pad=1)
     text = pa.Plan(p).describe()
-    # 25 088 pixels: 256 equal tiles of 98 rather than 196 of 128
-    assert "256 on 256 CUs (256 busy, 1 round(s) of tiles)" in text
-    assert "block M x N x K            98 x 128 x 64" in text
+    # 25 088 pixels: 224 tiles of 112 (seven whole 16-pixel blocks; 256 equal
+    # tiles of 98 cost each workgroup the same seven) rather than 196 of 128
+    assert "224 on 256 CUs (224 busy, 1 round(s) of tiles)" in text
+    assert "block M x N x K            112 x 128 x 64" in text
     rows = re.findall(r"^\s+(\*?)\s*(streaming|resident patch) (.*?)\s+(\d+)"
                       r"\s+(\d+)\s+([\d.]+)\s+(\d+)\s+([\d.]+) us$", text,
                       re.M)
@@ -545,7 +546,9 @@ def test_planner_weighs_tilings_and_reports_them():
                                                              blockM=64)
     assert "* resident patch 128 x 128" in forced(patch=1)
     assert "196 on 256 CUs (196 busy, 1 round(s)" in forced(patch=1)
-    assert "* resident patch 98 x 128, 16-pixel blocks" in forced(patch=2)
+    assert "* resident patch 112 x 128, 16-pixel blocks" in forced(patch=2)
+    assert "* resident patch 98 x 128, 16-pixel blocks" in \
+        forced(patch=2, blockM=98)
     assert "* resident patch 112 x 128, 16-pixel blocks" in \
         forced(patch=2, blockM=112)
     with pytest.raises(MxconvError):
