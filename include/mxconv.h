@@ -236,6 +236,17 @@ void mxconv_plan_destroy(mxconv_plan *plan);
 mxconv_status mxconv_plan_describe(const mxconv_plan *plan, char *buffer,
                                    size_t capacity, size_t *needed);
 
+/* reportPlanEstimatedCosts (include/poplin/Convolution.hpp:590-611,
+ * lib/poplin/Convolution.cpp:3923-3936): the planner's estimate for one
+ * launch of the plan.  *cycles: shader-clock cycles at 2.1 GHz from the cost
+ * model the tilings were weighed with, or MXCONV_COST_UNKNOWN where the model
+ * does not cover the kernel (the generic one).  *memory_bytes: the temporary
+ * device memory of a launch (the workspace).  Touches no GPU. */
+#define MXCONV_COST_UNKNOWN UINT64_MAX
+mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
+                                          uint64_t *cycles,
+                                          uint64_t *memory_bytes);
+
 /* Whether weights packed for `packed_for` are laid out as `plan` reads them
  * (*same = 1) or not (0).  In the reference the options given to
  * createWeights only decide a tensor layout and convolution() rearranges a

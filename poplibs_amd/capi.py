@@ -164,6 +164,8 @@ def lib():
                                          POINTER(c_size_t)]),
         "mxconv_plan_buffer_bytes": (c_int, [c_void_p, c_int32,
                                              POINTER(c_size_t)]),
+        "mxconv_plan_estimated_costs": (c_int, [c_void_p, POINTER(c_uint64),
+                                                POINTER(c_uint64)]),
         "mxconv_plans_pack_alike": (c_int, [c_void_p, c_void_p,
                                             POINTER(c_int32)]),
         "mxconv_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p,
@@ -581,6 +583,18 @@ class Plan:
         _check(lib().mxconv_plan_describe(self._h, buf, need.value,
                                           byref(need)))
         return buf.value.decode()
+
+    COST_UNKNOWN = 2 ** 64 - 1
+
+    def estimated_costs(self):
+        """(cycles, memory bytes) the planner estimates for one launch:
+        reportPlanEstimatedCosts (include/poplin/Convolution.hpp:590-611).
+        cycles is COST_UNKNOWN where the cost model does not cover the
+        kernel."""
+        cycles, memory = c_uint64(), c_uint64()
+        _check(lib().mxconv_plan_estimated_costs(self._h, byref(cycles),
+                                                 byref(memory)))
+        return cycles.value, memory.value
 
     def packs_like(self, other):
         """Whether weights packed for `other` are laid out as this plan

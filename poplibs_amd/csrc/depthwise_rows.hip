@@ -40,15 +40,30 @@ constexpr int kRowsThreads = 64 * (kComputeWaves + kLoaderWaves);
 constexpr int kOwnLoads = kRowLoads / kLoaderWaves; // per loader wave and row
 constexpr uint32_t kNoByte = 0x80000000u;           // beyond any buffer here
 
-/// Steps (output rows) the loads run ahead, and row slots of the ring, by
-/// stride: a step needs rows [j S, j S + 2], so `ahead` steps on the way take
-/// ahead * S + 3 slots.  Six rows on the way (108 KB of LDS): on N = 32,
-/// 112 x 112, 96 channels, stride 2 that takes 17.7 us, eight rows 18.0, ten
-/// 18.3, four 17.85, two 18.9; two loader waves 18.2, six as four.
+/// The forward kernel's ring by stride.  kAhead: steps (output rows) the
+/// loads run ahead; a step needs rows [j S, j S + 2], so `ahead` steps on the
+/// way take ahead * S + 3 slots.  Six rows on the way: on N = 32, 112 x 112,
+/// 96 channels, stride 2 that takes 17.7 us, eight rows 18.0, ten 18.3, four
+/// 17.85, two 18.9; two loader waves 18.2, six as four.
+/// At stride 1 a step adds one row to the two the step before it used: the
+/// compute waves keep the window in registers and read the row the NEXT step
+/// adds while they multiply (kEarlyRows = 1: that row has landed a step
+/// early, one more slot), and eight compute waves, two on every SIMD, take
+/// wider strips (N = 32, 56 x 56, 144 channels: 16.5 us with six waves
+/// reading nine vectors per step, 13.8 with eight, 13.1 with the register
+/// window as well).  At stride 2 both cost time (17.8 -> 18.0 and 18.2 us).
 template <int S> struct Ring {
   static constexpr int kAhead = 6 / S;
-  static constexpr int kSlots = kAhead * S + 3;
+  static constexpr int kEarlyRows = S == 1 ? 1 : 0;
+  static constexpr int kWindow = 3 + kEarlyRows; // rows landed at a barrier
+  static constexpr int kSlots = kAhead * S + kWindow;
+  static constexpr int kComputeWaves = S == 1 ? 8 : 6;
+  static constexpr int kComputeThreads = 64 * kComputeWaves;
+  static constexpr int kThreads = 64 * (kComputeWaves + kLoaderWaves);
 };
+constexpr uint32_t fwdComputeThreads(uint32_t stride) {
+  return stride == 1 ? Ring<1>::kComputeThreads : Ring<2>::kComputeThreads;
+}
 
 struct RowsArgs {
   DepthwiseDesc d;
@@ -71,7 +86,7 @@ template <> struct PutVec<__half> {
     Vec8 o;
 #pragma unroll
     for (int i = 0; i != 4; ++i)
-      o.h2[i] = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
+      o.h2[i] = roundPairToHalf(v[2 * i], v[2 * i + 1]);
     __builtin_nontemporal_store(o.raw, reinterpret_cast<uintx4 *>(p));
   }
 };
@@ -121,7 +136,7 @@ template <int LOADS> struct StripRow {
 };
 
 template <int S, class OutT>
-__global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
+__global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
     RowsArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
   constexpr int kAhead = Ring<S>::kAhead, kSlots = Ring<S>::kSlots;
@@ -147,11 +162,11 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
   // relative input rows [0, rowsIn) are what the band reads
   const uint32_t rowsIn = (steps - 1) * S + 3;
 
-  if (wave >= kComputeWaves) {
+  if (wave >= Ring<S>::kComputeWaves) {
     // ---- loaders.  Load L of a row fills bytes [1024 L, 1024 L + 1024) of
     // its slot: 16-byte unit u = 64 L + lane is channel vector u % vecs of
     // strip column u / vecs.  Loader l takes L = l, l + kLoaderWaves, ...
-    const int loader = wave - kComputeWaves;
+    const int loader = wave - Ring<S>::kComputeWaves;
     const __amdgpu_buffer_rsrc_t inBuf = bufferOf(in, a.inBytes);
     StripRow<kOwnLoads> strip;
     strip.setup(iw0, a.colsIn, int(d.loW), int(d.hiW), pixelBytes, a.vecs,
@@ -169,10 +184,10 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
     };
     // rows of steps 0 .. kAhead - 1
 #pragma unroll 1
-    for (int r = 0; r != (kAhead - 1) * S + 3; ++r)
+    for (int r = 0; r != (kAhead - 1) * S + Ring<S>::kWindow; ++r)
       loadRow();
     for (uint32_t j = 0; j < steps; ++j) {
-      // step j's rows have landed when all but the rows of the kAhead - 1
+      // step j's window has landed when all but the rows of the kAhead - 1
       // steps behind it have
       MXK_WAIT_VMCNT((kAhead - 1) * S * kOwnLoads);
       stepBarrier();
@@ -204,21 +219,27 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
   const uint32_t windowByte = ((active ? col : 0) * S * a.vecs + v) * 16;
   OutT *dst = out + ((size_t(b) * d.outH + oh0) * d.outW + ow) * d.channels + c;
   const size_t outRow = size_t(d.outW) * d.channels;
-  uint32_t slot = 0; // slot of relative row j * S
-  for (uint32_t j = 0; j < steps; ++j) {
-    stepBarrier(); // step j's rows are in the ring
+  auto rowOf = [&](uint32_t slot) {
+    return lds + slot * kSlotBytes + windowByte;
+  };
+  auto readRow = [&](Vec8(&row)[3], const char *from) {
+#pragma unroll
+    for (int kw = 0; kw != 3; ++kw)
+      row[kw].raw =
+          *reinterpret_cast<const uintx4 *>(from + kw * a.vecs * 16);
+  };
+  // out row = bias + the nine taps over three window rows, kh then kw
+  auto multiply = [&](const Vec8(&r0)[3], const Vec8(&r1)[3],
+                      const Vec8(&r2)[3]) {
     float acc[8];
 #pragma unroll
     for (int e = 0; e != 8; ++e)
       acc[e] = biasV[e];
-    uint32_t rowSlot = slot;
 #pragma unroll
-    for (int kh = 0; kh != 3; ++kh) {
-      const char *row = lds + rowSlot * kSlotBytes + windowByte;
+    for (int kh = 0; kh != 3; ++kh)
 #pragma unroll
       for (int kw = 0; kw != 3; ++kw) {
-        Vec8 x;
-        x.raw = *reinterpret_cast<const uintx4 *>(row + kw * a.vecs * 16);
+        const Vec8 &x = kh == 0 ? r0[kw] : kh == 1 ? r1[kw] : r2[kw];
         const Vec8 &k = taps[kh * 3 + kw];
 #pragma unroll
         for (int e = 0; e != 4; ++e) {
@@ -228,15 +249,65 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsKernel(
           acc[2 * e + 1] = fmaf(xf.y, kf.y, acc[2 * e + 1]);
         }
       }
-      rowSlot = rowSlot + 1 == kSlots ? 0 : rowSlot + 1;
-    }
-    // (the reads are done - their values were used - before the next
-    // barrier lets the loaders overwrite the rows)
     if (active)
       PutVec<OutT>::put(dst, acc);
     dst += outRow;
-    slot += S;
-    slot -= slot >= kSlots ? kSlots : 0;
+  };
+  auto next = [&](uint32_t slot) {
+    return slot + 1 == uint32_t(kSlots) ? 0u : slot + 1;
+  };
+
+  if constexpr (Ring<S>::kEarlyRows == 0) {
+    // A step reads its three rows behind its barrier.  (The reads are done -
+    // their values were used - before the next barrier lets the loaders
+    // overwrite the rows.)
+    uint32_t slot = 0; // slot of relative row j * S
+    for (uint32_t j = 0; j < steps; ++j) {
+      stepBarrier(); // step j's rows are in the ring
+      Vec8 win[3][3];
+      uint32_t rowSlot = slot;
+#pragma unroll
+      for (int kh = 0; kh != 3; ++kh) {
+        readRow(win[kh], rowOf(rowSlot));
+        rowSlot = next(rowSlot);
+      }
+      multiply(win[0], win[1], win[2]);
+      slot += S;
+      slot -= slot >= uint32_t(kSlots) ? kSlots : 0;
+    }
+  } else {
+    // Stride 1.  The window lives in four register rows: a step multiplies
+    // the three it holds from earlier steps and reads the one the next step
+    // adds into the fourth, so every row is read from LDS once and that read
+    // hides behind the multiplications.  A row's slot is loaded into again
+    // only after the barrier of the step behind the one that used the row.
+    static_assert(S == 1 && Ring<S>::kEarlyRows == 1, "one row per step");
+    Vec8 win[4][3];
+    uint32_t readSlot = 0; // slot of the next row to read
+    auto step = [&](auto off, bool first) {
+      constexpr int OFF = decltype(off)::value;
+      stepBarrier(); // the step's rows and the next step's are in the ring
+      if (first) {
+#pragma unroll
+        for (int r = 0; r != 3; ++r) {
+          readRow(win[r], rowOf(readSlot));
+          readSlot = next(readSlot);
+        }
+      }
+      readRow(win[(OFF + 3) % 4], rowOf(readSlot));
+      readSlot = next(readSlot);
+      multiply(win[OFF], win[(OFF + 1) % 4], win[(OFF + 2) % 4]);
+    };
+    // the register rows come round every four steps
+    for (uint32_t j = 0; j < steps; j += 4) {
+      step(std::integral_constant<int, 0>{}, j == 0);
+      if (j + 1 < steps)
+        step(std::integral_constant<int, 1>{}, false);
+      if (j + 2 < steps)
+        step(std::integral_constant<int, 2>{}, false);
+      if (j + 3 < steps)
+        step(std::integral_constant<int, 3>{}, false);
+    }
   }
 }
 
@@ -414,7 +485,8 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsDeltaKernel(
 
 /// Strips, bands and their sizes for a chip of `cus` compute units; false
 /// when the kernel does not take the layer.
-bool shapeFor(const DepthwiseDesc &d, uint32_t cus, RowsArgs &a) {
+bool shapeFor(const DepthwiseDesc &d, uint32_t cus, RowsArgs &a,
+              uint32_t computeThreads = kComputeThreads) {
   if (d.kH != 3 || d.kW != 3 || d.dilH != 1 || d.dilW != 1 ||
       d.strideH != d.strideW || (d.strideH != 1 && d.strideH != 2) ||
       d.channels % 8 != 0 || d.channels == 0 || d.inDilH != 1 ||
@@ -424,12 +496,12 @@ bool shapeFor(const DepthwiseDesc &d, uint32_t cus, RowsArgs &a) {
   a.vecs = d.channels / 8;
   // a strip's input row fits a slot, its output row the compute threads
   const uint32_t unitsPerSlot = kSlotBytes / 16;
-  if (a.vecs * 3 > unitsPerSlot || a.vecs > uint32_t(kComputeThreads))
+  if (a.vecs * 3 > unitsPerSlot || a.vecs > computeThreads)
     return false;
   const uint32_t maxColsIn = unitsPerSlot / a.vecs;
   uint32_t maxColsOut = (maxColsIn - 3) / s + 1;
-  if (maxColsOut > kComputeThreads / a.vecs)
-    maxColsOut = kComputeThreads / a.vecs;
+  if (maxColsOut > computeThreads / a.vecs)
+    maxColsOut = computeThreads / a.vecs;
   a.strips = (d.outW + maxColsOut - 1) / maxColsOut;
   a.colsOut = (d.outW + a.strips - 1) / a.strips;
   a.colsIn = (a.colsOut - 1) * s + 3;
@@ -456,7 +528,7 @@ hipError_t run(const RowsArgs &a, const void *in, const void *w,
     return attr;
   const uint32_t blocks = a.d.batch * a.strips * a.bands;
   hipLaunchKernelGGL((depthwiseRowsKernel<S, OutT>), dim3(blocks),
-                     dim3(kRowsThreads), ldsBytes, stream, a,
+                     dim3(Ring<S>::kThreads), ldsBytes, stream, a,
                      static_cast<const __half *>(in),
                      static_cast<const __half *>(w),
                      static_cast<const OutT *>(bias), static_cast<OutT *>(out));
@@ -465,26 +537,38 @@ hipError_t run(const RowsArgs &a, const void *in, const void *w,
 
 } // namespace
 
-bool depthwiseRowsTakes(const DepthwiseDesc &d, int inType) {
+namespace {
+bool takes(const DepthwiseDesc &d, int inType, uint32_t computeThreads) {
   RowsArgs a;
-  if (inType != kHalf || d.cus == 0 || !shapeFor(d, d.cus, a))
+  if (inType != kHalf || d.cus == 0 || !shapeFor(d, d.cus, a, computeThreads))
     return false;
   const uint64_t inBytes = uint64_t(d.batch) * d.inH * d.inW * d.channels * 2;
   const uint64_t blocks = uint64_t(d.batch) * a.strips * a.bands;
   return inBytes < kNoByte && blocks < 0x7fffffffull;
 }
 
-DepthwiseRowsLaunch depthwiseRowsLaunchShape(const DepthwiseDesc &d) {
+DepthwiseRowsLaunch launchShapeOf(const DepthwiseDesc &d,
+                                  uint32_t computeThreads) {
   RowsArgs a{};
   DepthwiseRowsLaunch l{};
-  if (d.cus == 0 || !shapeFor(d, d.cus, a))
+  if (d.cus == 0 || !shapeFor(d, d.cus, a, computeThreads))
     return l;
   l.strips = a.strips, l.colsOut = a.colsOut;
   l.bands = a.bands, l.rowsOut = a.rowsOut;
   l.workgroups = uint64_t(d.batch) * a.strips * a.bands;
   l.ringRows = d.strideH == 2 ? Ring<2>::kSlots : Ring<1>::kSlots;
   l.loaderWaves = kLoaderWaves;
+  l.computeWaves = computeThreads / 64;
   return l;
+}
+} // namespace
+
+bool depthwiseRowsTakes(const DepthwiseDesc &d, int inType) {
+  return takes(d, inType, fwdComputeThreads(d.strideH));
+}
+
+DepthwiseRowsLaunch depthwiseRowsLaunchShape(const DepthwiseDesc &d) {
+  return launchShapeOf(d, fwdComputeThreads(d.strideH));
 }
 
 hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
@@ -495,7 +579,7 @@ hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
       (outType != kHalf && outType != kFloat))
     return hipErrorInvalidValue;
   RowsArgs a{};
-  shapeFor(d, d.cus, a);
+  shapeFor(d, d.cus, a, fwdComputeThreads(d.strideH));
   a.d = d;
   a.inBytes = uint32_t(uint64_t(d.batch) * d.inH * d.inW * d.channels * 2);
   a.divVecs = makeFastDiv(a.vecs);
@@ -512,11 +596,17 @@ hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
 bool depthwiseRowsDeltaTakes(const DepthwiseDesc &d) {
   const uint64_t deltaBytes =
       uint64_t(d.batch) * d.outH * d.outW * d.channels * 2;
-  return depthwiseRowsTakes(d, kHalf) && deltaBytes < kNoByte;
+  return takes(d, kHalf, kComputeThreads) && deltaBytes < kNoByte;
+}
+
+DepthwiseRowsLaunch depthwiseRowsDeltaLaunchShape(const DepthwiseDesc &d) {
+  DepthwiseRowsLaunch l = launchShapeOf(d, kComputeThreads);
+  l.ringRows = d.strideH == 2 ? DeltaRing<2>::kSlots : DeltaRing<1>::kSlots;
+  return l;
 }
 
 size_t depthwiseRowsDeltaWorkspaceBytes(const DepthwiseDesc &d) {
-  const DepthwiseRowsLaunch l = depthwiseRowsLaunchShape(d);
+  const DepthwiseRowsLaunch l = depthwiseRowsDeltaLaunchShape(d);
   return size_t(l.workgroups) * 9 * d.channels * sizeof(float);
 }
 

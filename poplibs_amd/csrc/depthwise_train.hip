@@ -47,7 +47,7 @@ __device__ __forceinline__ void store8(__half *p, const float (&v)[8]) {
   Vec8 o;
 #pragma unroll
   for (int i = 0; i != 4; ++i)
-    o.h2[i] = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
+    o.h2[i] = roundPairToHalf(v[2 * i], v[2 * i + 1]);
   *reinterpret_cast<uint4 *>(p) = o.raw;
 }
 __device__ __forceinline__ void store8(float *p, const float (&v)[8]) {

@@ -51,11 +51,24 @@ template <> struct Load<uint8_t> {
   }
 };
 
+/// Two fp32 sums rounded to half, to nearest even, as fp32 values: the empty
+/// asm keeps the compiler from folding the multiply-add that produced a sum
+/// into the conversion (v_fma_mixlo_f16 rounds once, from the exact result),
+/// which it does for some of a kernel's sums and not for others.  Every
+/// vector-ALU kernel rounds through here, so that a layer's output does not
+/// depend on which of them ran it - and is the fp32 partial cast to half that
+/// the reference's partialsType float produces.
+__device__ __forceinline__ __half2 roundPairToHalf(float a, float b) {
+  asm("" : "+v"(a), "+v"(b));
+  return __floats2half2_rn(a, b);
+}
+
 /// fp32 -> output element, round to nearest even.
 __device__ __forceinline__ void storeOut(float *p, size_t i, float v) {
   p[i] = v;
 }
 __device__ __forceinline__ void storeOut(__half *p, size_t i, float v) {
+  asm("" : "+v"(v)); // (as in roundPairToHalf)
   p[i] = __float2half_rn(v);
 }
 
@@ -90,8 +103,8 @@ __device__ __forceinline__ void storeOut4(__half *p, const float (&v)[4]) {
     __half2 h[2];
     uint2 u;
   } pack;
-  pack.h[0] = __floats2half2_rn(v[0], v[1]);
-  pack.h[1] = __floats2half2_rn(v[2], v[3]);
+  pack.h[0] = roundPairToHalf(v[0], v[1]);
+  pack.h[1] = roundPairToHalf(v[2], v[3]);
   *reinterpret_cast<uint2 *>(p) = pack.u;
 }
 

@@ -310,6 +310,7 @@ hipError_t launchDepthwise3x3(const DepthwiseDesc &d, int inType,
 bool depthwiseRowsTakes(const DepthwiseDesc &d, int inType);
 struct DepthwiseRowsLaunch {
   uint32_t strips, colsOut, bands, rowsOut, ringRows, loaderWaves;
+  uint32_t computeWaves;
   uint64_t workgroups;
 };
 DepthwiseRowsLaunch depthwiseRowsLaunchShape(const DepthwiseDesc &d);
@@ -321,6 +322,7 @@ hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
 /// workgroup at partial[workgroup], to be added in order; *walkers = their
 /// count.
 bool depthwiseRowsDeltaTakes(const DepthwiseDesc &d);
+DepthwiseRowsLaunch depthwiseRowsDeltaLaunchShape(const DepthwiseDesc &d);
 size_t depthwiseRowsDeltaWorkspaceBytes(const DepthwiseDesc &d);
 hipError_t launchDepthwiseRowsDeltas(const DepthwiseDesc &d, const void *acts,
                                      const void *deltas, void *partial,

@@ -546,6 +546,20 @@ mxconv_status mxconv_plan_describe(const mxconv_plan *plan, char *buffer,
   });
 }
 
+mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
+                                          uint64_t *cycles,
+                                          uint64_t *memory_bytes) {
+  REQUIRE_ARG(plan);
+  REQUIRE_ARG(cycles);
+  REQUIRE_ARG(memory_bytes);
+  lastError.clear();
+  const double us = plan->estimatedMicroseconds();
+  *cycles = us < 0 ? MXCONV_COST_UNKNOWN
+                   : uint64_t(us * mxconv_plan::kEstimateClockMHz + 0.5);
+  *memory_bytes = plan->workspaceBytes;
+  return MXCONV_OK;
+}
+
 mxconv_status mxconv_plan_buffer_bytes(const mxconv_plan *plan, int32_t which,
                                        size_t *bytes) {
   REQUIRE_ARG(plan);

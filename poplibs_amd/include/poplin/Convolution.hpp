@@ -10,13 +10,16 @@
 #ifndef poplibs_amd_poplin_Convolution_hpp
 #define poplibs_amd_poplin_Convolution_hpp
 #include "poplar/OptionFlags.hpp"
+#include "poplar/Target.hpp"
 #include "poplar/Type.hpp"
 #include "poplin/ConvParams.hpp"
 
 #include <cstddef>
 #include <cstdint>
 #include <iosfwd>
+#include <limits>
 #include <memory>
+#include <tuple>
 #include <vector>
 
 struct mxconv_plan;
@@ -181,6 +184,29 @@ void addBias(const DeviceTensor &in, const DeviceTensor &biases, Stream &prog);
 void reportPlanInfo(std::ostream &out, const ConvParams &params,
                     const poplar::OptionFlags &options = {},
                     PlanningCache *cache = nullptr);
+
+/// Estimated costs of a plan (include/poplin/Convolution.hpp:590-594 of
+/// PopLibs).  cycles: shader-clock cycles of one launch at 2.1 GHz, by the
+/// cost model the planner weighs tilings with; `unknown` where that model does
+/// not cover the kernel chosen.  memory: bytes of temporary device memory a
+/// launch uses.
+struct PlanCosts {
+  std::size_t cycles;
+  std::size_t memory;
+  constexpr static std::size_t unknown =
+      std::numeric_limits<std::size_t>::max();
+};
+
+/// include/poplin/Convolution.hpp:608-611 of PopLibs.
+PlanCosts reportPlanEstimatedCosts(const ConvParams &params,
+                                   const poplar::OptionFlags &options = {},
+                                   PlanningCache *cache = nullptr);
+
+/// What poplin::preplan takes for one convolution
+/// (include/poplin/Convolution.hpp:386-388 of PopLibs): the target (may be
+/// null), the parameters and a pointer to the options.
+using ConvPlanParams = std::tuple<const poplar::Target *, const ConvParams,
+                                  const poplar::OptionFlags *>;
 
 /// Throws poplar::invalid_option for an unknown key or value.
 void convolutionValidateOptions(const poplar::OptionFlags &options);

@@ -21,6 +21,8 @@
 #include "poplin/Convolution.hpp"
 
 #include <iosfwd>
+#include <set>
+#include <unordered_map>
 #include <vector>
 
 namespace poplin {
@@ -124,6 +126,32 @@ DeviceTensor createMatMulGroupedOutput(const poplar::Type &inputType,
 
 /// Throws poplar::invalid_option for an unknown matMul option key or value.
 void matmulValidateOptions(const poplar::OptionFlags &options);
+
+/// C = A * B as poplin::preplan takes it (include/poplin/MatMul.hpp:613-631 of
+/// PopLibs): aShape [g][m][k] and bShape [g][k][n], or [m][k] and [k][n] for
+/// one group.
+struct MatMulParams {
+  poplar::Type inputType;
+  poplar::Type outputType;
+  std::vector<std::size_t> aShape;
+  std::vector<std::size_t> bShape;
+  friend bool operator<(const MatMulParams &a, const MatMulParams &b);
+};
+
+/// include/poplin/MatMul.hpp:641-642 of PopLibs; the target may be null.
+using MatMulPlanParams = std::tuple<const poplar::Target *, const MatMulParams,
+                                    const poplar::OptionFlags *>;
+/// The convolution options made from each multiplication's options, kept
+/// alive for the pointers in the set matMulGetConvPlanParams returns
+/// (include/poplin/MatMul.hpp:648-649 of PopLibs).
+using MatMulToConvOptions =
+    std::unordered_map<const poplar::OptionFlags *, poplar::OptionFlags>;
+
+/// The convolutions `matmuls` are planned as
+/// (include/poplin/MatMul.hpp:661-663 of PopLibs).
+std::set<ConvPlanParams>
+matMulGetConvPlanParams(const std::set<MatMulPlanParams> &matmuls,
+                        MatMulToConvOptions &matmulToConvOpts);
 
 } // namespace poplin
 #endif

@@ -2,12 +2,17 @@
 // memory and host transfers use the HIP runtime directly; every kernel launch
 // goes through an mxconv_* call.
 #include "poplin/Convolution.hpp"
+#include "poplin/ConvPreplan.hpp"
 #include "LayerInternal.hpp"
 #include "mxconv.h"
 #include "poplar/exceptions.hpp"
 #include "poputil/exceptions.hpp"
 
 #include <algorithm>
+#include <atomic>
+#include <exception>
+#include <set>
+#include <thread>
 #include <hip/hip_runtime_api.h>
 
 #include <map>
@@ -424,6 +429,78 @@ void reportPlanInfo(std::ostream &out, const ConvParams &params,
   check(mxconv_plan_describe(plan->plan, &text[0], text.size(), &needed));
   text.resize(needed - 1);
   out << text;
+}
+
+PlanCosts reportPlanEstimatedCosts(const ConvParams &params,
+                                   const poplar::OptionFlags &options,
+                                   PlanningCache *cache) {
+  auto plan = getPlan(params, options, cache);
+  std::uint64_t cycles = 0, memory = 0;
+  check(mxconv_plan_estimated_costs(plan->plan, &cycles, &memory));
+  return {cycles == MXCONV_COST_UNKNOWN ? PlanCosts::unknown
+                                        : std::size_t(cycles),
+          std::size_t(memory)};
+}
+
+void preplan(const std::set<ConvPlanParams> &convs,
+             const std::set<MatMulPlanParams> &matmuls, PlanningCache &cache) {
+  if (convs.empty() && matmuls.empty())
+    return;
+  MatMulToConvOptions matmulOptions;
+  const std::set<ConvPlanParams> matmulConvs =
+      matMulGetConvPlanParams(matmuls, matmulOptions);
+
+  // Distinct cache keys that the cache does not hold yet.
+  using Key = PlanningCache::Impl::Key;
+  struct Job {
+    Key key;
+    const ConvParams *params;
+    std::shared_ptr<PlanHandle> plan;
+    std::exception_ptr error;
+  };
+  std::vector<Job> jobs;
+  {
+    std::set<Key> seen;
+    std::lock_guard<std::mutex> lock(cache.impl->mutex);
+    for (const auto *set : {&convs, &matmulConvs})
+      for (const auto &conv : *set) {
+        if (!std::get<2>(conv))
+          throw poputil::poplibs_error(
+              "preplan: null pointer to the options");
+        Key key{std::get<1>(conv).canonicalize(), *std::get<2>(conv)};
+        if (cache.impl->plans.count(key) || !seen.insert(key).second)
+          continue;
+        jobs.push_back(Job{std::move(key), &std::get<1>(conv), nullptr,
+                           nullptr});
+      }
+  }
+  // Plans are independent host computations: make them on as many threads
+  // as the host offers (each job writes its own slot), then insert them one
+  // after the other (lib/poplin/ConvPlan.cpp:1839-1875).
+  const std::size_t workers = std::min<std::size_t>(
+      jobs.size(), std::max(1u, std::thread::hardware_concurrency()));
+  std::atomic<std::size_t> next{0};
+  auto work = [&] {
+    for (std::size_t i; (i = next.fetch_add(1)) < jobs.size();) {
+      try {
+        jobs[i].plan = createPlan(*jobs[i].params, jobs[i].key.second);
+      } catch (...) {
+        jobs[i].error = std::current_exception();
+      }
+    }
+  };
+  std::vector<std::thread> threads;
+  for (std::size_t t = 1; t < workers; ++t)
+    threads.emplace_back(work);
+  work();
+  for (auto &t : threads)
+    t.join();
+  for (const Job &job : jobs)
+    if (job.error)
+      std::rethrow_exception(job.error);
+  std::lock_guard<std::mutex> lock(cache.impl->mutex);
+  for (Job &job : jobs)
+    cache.impl->plans.emplace(std::move(job.key), std::move(job.plan));
 }
 
 void convolutionValidateOptions(const poplar::OptionFlags &options) {

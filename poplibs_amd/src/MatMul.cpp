@@ -8,6 +8,7 @@
 #include "poputil/exceptions.hpp"
 
 #include <ostream>
+#include <tuple>
 
 namespace poplin {
 
@@ -336,6 +337,36 @@ DeviceTensor createMatMulGroupedOutput(const poplar::Type &,
   const Shapes s = checkShapes(aShape, bShape, true);
   matmulValidateOptions(options);
   return allocate(outputType, {s.g, s.m, s.n});
+}
+
+bool operator<(const MatMulParams &a, const MatMulParams &b) {
+  return std::tie(a.inputType, a.outputType, a.aShape, a.bShape) <
+         std::tie(b.inputType, b.outputType, b.aShape, b.bShape);
+}
+
+std::set<ConvPlanParams>
+matMulGetConvPlanParams(const std::set<MatMulPlanParams> &matmuls,
+                        MatMulToConvOptions &matmulToConvOpts) {
+  // lib/poplin/MatMul.cpp:344-366: one set of convolution options per
+  // distinct options pointer; the map's nodes stay put, so the pointers into
+  // it remain valid as it grows.
+  std::set<ConvPlanParams> convs;
+  for (const auto &matmul : matmuls) {
+    const MatMulParams &mm = std::get<1>(matmul);
+    const poplar::OptionFlags *options = std::get<2>(matmul);
+    if (!options)
+      throw poputil::poplibs_error(
+          "matMulGetConvPlanParams: null pointer to the options");
+    auto res = matmulToConvOpts.emplace(options, poplar::OptionFlags{});
+    if (res.second)
+      res.first->second = convOptions(*options);
+    const bool grouped = mm.aShape.size() == 3;
+    const Shapes s = checkShapes(mm.aShape, mm.bShape, grouped);
+    convs.emplace(std::get<0>(matmul),
+                  convParams(mm.inputType, mm.outputType, s),
+                  &res.first->second);
+  }
+  return convs;
 }
 
 void matmulValidateOptions(const poplar::OptionFlags &options) {

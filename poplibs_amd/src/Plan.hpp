@@ -110,6 +110,16 @@ struct mxconv_plan {
   std::size_t biasBytes() const { return biasElems * params.outputType.size(); }
 
   std::string describe() const;
+
+  /// Time one launch of this plan is estimated to take on the device, in
+  /// microseconds, by the cost model the tilings were weighed with; negative
+  /// when the model does not cover the kernel (the generic one).  The role of
+  /// estimateConvCost behind reportPlanEstimatedCosts
+  /// (lib/poplin/Convolution.cpp:3923-3936).
+  double estimatedMicroseconds() const;
+  /// The shader clock the estimate is converted to cycles with: what the chip
+  /// holds with the matrix cores of most CUs busy.
+  static constexpr double kEstimateClockMHz = 2100.0;
 };
 
 namespace poplin {

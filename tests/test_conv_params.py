@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import poplibs_amd as pa
-from poplibs_amd import MxconvError, Status
+from poplibs_amd import MxconvError, Status, capi
 from helpers import (NONE, input_index_def, make_params, output_size_def,
                      random_data, random_params)
 
@@ -503,6 +503,42 @@ def test_plan_buffers_and_type_rules():
     with pytest.raises(MxconvError) as e:
         q.fwd(1, 1, 1)
     assert "mxconv_fwd_quarter" in e.value.message
+
+
+def test_plan_estimated_costs():
+    """mxconv_plan_estimated_costs (reportPlanEstimatedCosts,
+    include/poplin/Convolution.hpp:590-611): the chosen tiling's estimate in
+    cycles at 2.1 GHz, the workspace as temporary memory, unknown for the
+    generic kernel."""
+    import re
+    p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                    co=128, pad=1)
+    plan = pa.Plan(p)
+    cycles, memory = plan.estimated_costs()
+    chosen = re.search(r"^\s+\*.*?([\d.]+) us$", plan.describe(), re.M)
+    assert abs(cycles - float(chosen.group(1)) * 2100) <= 2100 * 0.05 + 1
+    assert memory == 0 == plan.buffer_bytes(capi.BUF_WORKSPACE)
+    # streamed kernels: time grows with the bytes moved
+    small = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                        groups=96, stride=2, pad=1)
+    large = make_params(pa.HALF, batch=64, field=(112, 112), kernel=(3, 3),
+                        groups=96, stride=2, pad=1)
+    a, b = pa.Plan(small).estimated_costs()[0], \
+        pa.Plan(large).estimated_costs()[0]
+    assert 17.9 * 0.75 < a / 2100 < 17.9 * 1.25  # 17.9 us measured
+    assert 1.7 * a < b < 2.0 * a  # one launch overhead, twice the bytes
+    # K split: the fp32 partial tiles are temporary memory
+    deep = pa.Plan(make_params(pa.HALF, batch=8, field=(28, 28),
+                               kernel=(3, 3), ci=128, co=128, pad=1))
+    assert "K split into parts" in deep.describe()
+    cycles, memory = deep.estimated_costs()
+    assert memory == deep.buffer_bytes(capi.BUF_WORKSPACE) > 0
+    assert cycles != pa.Plan.COST_UNKNOWN
+    # outside the cost model
+    generic = pa.Plan(make_params(pa.FLOAT, pa.FLOAT, batch=1, field=(5, 5),
+                                  kernel=(3, 3), ci=3, co=5))
+    assert "generic direct" in generic.describe()
+    assert generic.estimated_costs()[0] == pa.Plan.COST_UNKNOWN
 
 
 def test_planner_weighs_tilings_and_reports_them():

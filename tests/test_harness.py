@@ -36,6 +36,40 @@ def test_plan_only_reports_flops_and_plan():
     assert "inputPaddingLower          {1,1}" in r.stdout
 
 
+def test_plan_only_preplans_and_reports_estimated_costs():
+    """The tool plans its passes ahead of use (tools/single_conv_layer.cpp:
+    415-417, 831-850) and, with --report-plan, prints each pass's estimated
+    cost; --preplan 0 gives the same plans."""
+    args = ["--input-channels", "128", "--output-channels", "128", "--field",
+            "{28,28}", "--kernel-size", "3", "--padding", "1", "--batch-size",
+            "32", "--data-type", "half", "--plan-only"]
+    r = run(*args)
+    assert r.returncode == 0, r.stderr
+    import re
+    costs = re.findall(r"estimated cycles: (\d+), temporary memory: (\d+) "
+                       r"bytes", r.stdout)
+    assert len(costs) == 2, r.stdout  # forward and backward
+    for cycles, memory in costs:
+        # 8.5 us measured; 2.1 GHz
+        assert 8.5 * 0.75 < int(cycles) / 2100 < 8.5 * 1.25
+        assert int(memory) == 0
+    assert run(*args, "--preplan", "0").stdout == r.stdout
+
+
+def test_preplan_and_estimated_costs_host_checks():
+    """poplin::preplan fills the cache with the plans planning alone makes,
+    once per distinct key, or with nothing when an entry is invalid;
+    reportPlanEstimatedCosts is within a quarter of the measured times of the
+    benchmark configurations (tests/tools/preplan_test.cpp)."""
+    tool = os.path.join(ROOT, "tests", "tools", "preplan_test")
+    if not os.path.exists(tool):
+        subprocess.check_call(["make", "-C", os.path.dirname(tool)],
+                              stdout=subprocess.DEVNULL)
+    r = subprocess.run([tool], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "all checks passed" in r.stdout
+
+
 def test_plan_constraints_and_options_are_validated():
     base = ["--input-channels", "16", "--output-channels", "16", "--field",
             "{8,8}", "--kernel-size", "3", "--plan-only"]

@@ -19,6 +19,7 @@
 #include "poplar/exceptions.hpp"
 #include "poplin/ConvParams.hpp"
 #include "poplin/ConvUtil.hpp"
+#include "poplin/ConvPreplan.hpp"
 #include "poplin/Convolution.hpp"
 #include "poputil/exceptions.hpp"
 
@@ -35,6 +36,7 @@
 #include <iostream>
 #include <map>
 #include <random>
+#include <set>
 #include <sstream>
 #include <string>
 #include <vector>
@@ -144,6 +146,7 @@ int main(int argc, char **argv) try {
       "plan-only", "inference-only", "tolerance", "absolute-tolerance",
       "batch-size", "conv-groups", "fwd-plan-constraints",
       "fwd-plan-constraints-file", "report-plan", "convolution-options",
+      "preplan",
       "use-create-input", "num-determinism-checks", "ignore-data", "seed",
       "device-type", "profile", "timing-runs"};
   for (const auto &kv : opt) {
@@ -276,12 +279,36 @@ int main(int argc, char **argv) try {
   poplin::convolutionValidateOptions(wuOptions);
   const auto flops = poplin::getFwdFlops(params);
   poplin::PlanningCache cache;
+  // Plan the passes that run ahead of their use
+  // (tools/single_conv_layer.cpp:415-417, 831-850).
+  if (parseBool(get("preplan", "true"))) {
+    std::set<poplin::ConvPlanParams> convs;
+    if (doFwdPass)
+      convs.insert(std::make_tuple(nullptr, params, &options));
+    if (doBwdPass)
+      convs.insert(std::make_tuple(nullptr, bwdParams, &bwdOptions));
+    if (doWuPass)
+      convs.insert(std::make_tuple(
+          nullptr, poplin::getWeightUpdateParams(params), &wuOptions));
+    poplin::preplan(convs, {}, cache);
+  }
   const bool reportPlan = parseBool(get("report-plan", "false")) || has("plan-only");
+  auto reportCosts = [&](const ConvParams &p, const poplar::OptionFlags &o) {
+    const poplin::PlanCosts costs =
+        poplin::reportPlanEstimatedCosts(p, o, &cache);
+    std::cout << "  estimated cycles: ";
+    if (costs.cycles == poplin::PlanCosts::unknown)
+      std::cout << "unknown";
+    else
+      std::cout << costs.cycles;
+    std::cout << ", temporary memory: " << costs.memory << " bytes\n";
+  };
   if (doFwdPass) {
     std::cout << "Forward FLOPs: " << flops << "\n";
     if (reportPlan) {
       std::cout << "Forward plan:\n";
       poplin::reportPlanInfo(std::cout, params, options, &cache);
+      reportCosts(params, options);
     }
   }
   if (doBwdPass) {
@@ -289,6 +316,7 @@ int main(int argc, char **argv) try {
     if (reportPlan) {
       std::cout << "Backward plan:\n";
       poplin::reportPlanInfo(std::cout, bwdParams, bwdOptions, &cache);
+      reportCosts(bwdParams, bwdOptions);
     }
   }
   if (doWuPass) {
