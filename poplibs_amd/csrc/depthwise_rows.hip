@@ -52,6 +52,10 @@ constexpr uint32_t kNoByte = 0x80000000u;           // beyond any buffer here
 /// wider strips (N = 32, 56 x 56, 144 channels: 16.5 us with six waves
 /// reading nine vectors per step, 13.8 with eight, 13.1 with the register
 /// window as well).  At stride 2 both cost time (17.8 -> 18.0 and 18.2 us).
+/// (Strips of channels as well as of columns, so that wide pixels get wider
+/// column strips and fewer halo columns, lose: pieces of 256 to 640 bytes of
+/// every pixel read by different workgroups - N = 32, 28 x 28, 512 channels
+/// 11.5 -> 12.7 us, N = 128, 14 x 14, 576 channels 12.2 -> 16.8 us.)
 template <int S> struct Ring {
   static constexpr int kAhead = 6 / S;
   static constexpr int kEarlyRows = S == 1 ? 1 : 0;

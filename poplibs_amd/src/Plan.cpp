@@ -893,17 +893,20 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                  mxk::depthwise3x3Takes(d, mxk::kHalf);
     // Layers that give every CU a band of at least four output rows go to
     // the persistent kernel with a ring of input rows in LDS: its start-up
-    // (seven rows before the first output) wants rows to spread over.
-    if (d.dense3x3 && pc.rowRing != 0) {
+    // (seven rows before the first output; 3.5 us for the smallest layer
+    // against 2.9 us) wants rows to spread over.  Layers of more channels
+    // than the small-workgroup kernel takes (224) always do: the kernel of
+    // LDS halo tiles needs 5 to 8 us for the smallest of them.
+    if (!s.inputDilated() && !(pc.tileH || pc.tileW) && pc.rowRing != 0) {
       d.cus = gfx950::numCUs;
       const mxk::DepthwiseRowsLaunch l = mxk::depthwiseRowsLaunchShape(d);
       const bool takes = mxk::depthwiseRowsTakes(d, mxk::kHalf);
       if (pc.rowRing == 1 && !takes)
         throw poplar::invalid_option(
             "planConstraints gfx950 rowRing: that kernel takes 3x3 taps, "
-            "stride 1 or 2, channels in vectors of 8, at most 256 to a "
+            "stride 1 or 2, channels in vectors of 8, at most 2048 to a "
             "pixel");
-      if (takes && (pc.rowRing == 1 ||
+      if (takes && (pc.rowRing == 1 || !d.dense3x3 ||
                     (l.workgroups * 2 >= gfx950::numCUs && l.rowsOut >= 4)))
         d.dense3x3 = 2;
     } else if (pc.rowRing == 1) {

@@ -192,6 +192,14 @@ RING = "input rows streamed through an LDS ring"
     # stride 1, rows longer than a strip
     dict(batch=40, field=(30, 150), kernel=(3, 3), groups=64, stride=1,
          pad=1),
+    # more channels than the small-workgroup kernel takes: strips of a few
+    # columns, eight and six compute waves
+    dict(batch=6, field=(20, 37), kernel=(3, 3), groups=256, stride=1, pad=1),
+    dict(batch=5, field=(14, 14), kernel=(3, 3), groups=576, stride=2, pad=1),
+    dict(batch=3, field=(7, 7), kernel=(3, 3), groups=960, stride=1, pad=1),
+    # the most the kernel takes: one output column per strip
+    dict(batch=2, field=(6, 5), kernel=(3, 3), groups=2048, stride=1, pad=1),
+    dict(batch=2, field=(9, 7), kernel=(3, 3), groups=2048, stride=2, pad=1),
 ])
 @pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
 def test_depthwise_row_ring_matches_oracle(oracle, kw, out_type):
@@ -217,9 +225,23 @@ def test_depthwise_row_ring_plan_choice():
             "bands of 14 output rows") in text, text
     off = pa.Plan(big, {"planConstraints": '{"gfx950": {"rowRing": 0}}'})
     assert "dense row loads" in off.describe()
+    assert "read by 6 compute waves" in text, text
+    # stride 1: eight compute waves take wider strips
+    s1 = make_params(pa.HALF, batch=32, field=(56, 56), kernel=(3, 3),
+                     groups=144, stride=1, pad=1)
+    text = pa.Plan(s1).describe()
+    assert ("256 on 256 CUs: per image 2 strips of 28 output columns x 4 "
+            "bands of 14 output rows") in text, text
+    assert "read by 8 compute waves" in text, text
     # few rows per CU: the small workgroups stay
     small = make_params(pa.HALF, **DW3X3_CASES[0])
     assert "dense row loads" in pa.Plan(small).describe()
+    # ... unless the layer has more channels than they take (224)
+    wide = make_params(pa.HALF, batch=1, field=(14, 14), kernel=(3, 3),
+                       groups=576, stride=1, pad=1)
+    assert RING in pa.Plan(wide).describe()
+    assert "LDS halo tiles" in pa.Plan(
+        wide, {"planConstraints": '{"gfx950": {"rowRing": 0}}'}).describe()
     # not a 3x3 kernel: the constraint cannot be met
     with pytest.raises(pa.MxconvError):
         pa.Plan(make_params(pa.HALF, batch=2, field=(20, 20), kernel=(5, 5),

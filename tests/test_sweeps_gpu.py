@@ -187,7 +187,9 @@ def test_depthwise_row_rings_random_layers(oracle):
         lo, hi = _pads(rng, (0, 0), 2)
         kw = dict(batch=rng.randint(1, 9),
                   field=(rng.randint(3, 45), rng.randint(3, 90)),
-                  kernel=(3, 3), ci=1, co=1, groups=8 * rng.randint(1, 28),
+                  kernel=(3, 3), ci=1, co=1,
+                  groups=8 * (rng.randint(1, 28) if case % 4
+                              else rng.randint(29, 256)),
                   padLower=lo, padUpper=hi, stride=(s, s))
         if rng.random() < 0.15:
             kw["itl"] = (rng.randint(0, 1), rng.randint(0, 1))
