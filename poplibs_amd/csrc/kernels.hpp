@@ -258,8 +258,14 @@ hipError_t launchIgemmFused(const IgemmFusedItem *items, size_t count,
 struct PointwiseDesc {
   uint32_t batch, pixels; // pixels per image
   uint32_t groups, inChansPerGroup, outChansPerGroup;
+  // 64-channel tiles of the output a workgroup owns: 0 = the launch's choice
+  uint32_t chanTiles = 0;
 };
 bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType);
+/// Whether a workgroup can own `chanTiles` 64-channel tiles of this layer's
+/// output (they divide the layer's; 4 at most with 64 input channels, 2 with
+/// 128 or 256, 1 with 512).
+bool pointwiseChanTilesOk(const PointwiseDesc &d, uint32_t chanTiles);
 /// Elements of the packed weights ([G][32-channel block][k-slice][lane][8]).
 uint64_t pointwisePackedElems(const PointwiseDesc &d);
 hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
@@ -270,6 +276,7 @@ hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
 /// through a ring of `ring` LDS buffers filled by `loaderWaves` waves.
 struct PointwiseLaunch {
   uint32_t tilePixels, ring, loaderWaves, tilesPerWorkgroup;
+  uint32_t chansPerWorkgroup; // 64, 128 or 256 output channels
   uint64_t workgroups;
 };
 PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus);

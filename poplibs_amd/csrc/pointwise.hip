@@ -6,8 +6,9 @@
 // igemm.hip's big tiles and deep k-pipeline have nothing to pipeline here:
 // with K = 256 a 128-pixel tile is four k-steps of prologue and epilogue.
 // This kernel streams instead:
-//   * a workgroup is 2 or 4 compute waves + 1 loader wave and owns 64 output
-//     channels; it walks over tiles of 32 or 64 pixels, all of K each;
+//   * a workgroup is 2 to 8 compute waves + 2 or 4 loader waves and owns 64,
+//     128 or 256 output channels; it walks over tiles of 32 to 128 pixels,
+//     all of K each, and multiplies a tile by its channels 64 at a time;
 //   * the weights never touch LDS: they are packed per (32-channel block,
 //     16-deep k-slice) in MFMA operand order, each compute wave fetches its
 //     block once - one coalesced 16-byte load per lane and slice - and keeps
@@ -35,6 +36,7 @@ namespace {
 
 constexpr int kPwChans = 64;         // output channels per workgroup
 constexpr int kPwStageRow = 64 + 16; // staging: 64 bytes of a pixel + padding
+constexpr int kPwPairRow = 128 + 16; // ... 128 bytes: two blocks' channels
 
 struct PwArgs {
   PointwiseDesc d;
@@ -48,8 +50,12 @@ struct PwArgs {
 /// KS: k-slices of 16 channels (Ci / 16).  TM: pixels per tile (32, 64, 128);
 /// the workgroup has TM / 16 compute waves and LW loader waves, which take
 /// the loads of a tile in turn.  NB: tile buffers in LDS; NB - 1 tiles are in
-/// flight.
-template <int KS, int TM, int NB, int LW, class OutT>
+/// flight.  NT: 64-channel tiles of the output a workgroup owns (a.nTiles
+/// counts the workgroups' shares, NT * 64 channels each): a layer that widens
+/// the channels reads its input once per share, so fewer, wider shares read
+/// less - 64 -> 256 channels on N = 32, 56 x 56: four shares of 64 re-read
+/// 13 MB four times beside 51 MB of output.
+template <int KS, int TM, int NB, int LW, int NT, class OutT>
 __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
     PwArgs a, const char *__restrict__ in, const char *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
@@ -65,13 +71,21 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
   static_assert(kLoads % LW == 0, "the loader waves share a tile evenly");
   constexpr int kOwnLoads = kLoads / LW; // ... per loader wave
   static_assert((NB - 2) * kOwnLoads <= 63, "wait count fits s_waitcnt");
-  // NB tile buffers | staging
+  // NB tile buffers | staging | bias of the workgroup's channels (fp32)
   extern __shared__ __align__(16) char lds[];
 
   const PointwiseDesc &d = a.d;
-  const uint32_t walker = blockIdx.x % a.walkers;
-  const uint32_t nTile = (blockIdx.x / a.walkers) % a.nTiles;
-  const uint32_t g = blockIdx.x / (a.walkers * a.nTiles);
+  // The workgroups that take the same pixel tiles for different channels
+  // are neighbours in an XCD's run of workgroups: they start together and
+  // meet in its L2, which then fetches a tile once for all of them.  (Dealt
+  // out walker-fastest they land on different XCDs unless the walkers are a
+  // multiple of eight: N = 32, 56 x 56, 128 -> 256 channels with 61 walkers
+  // 25.1 us, with 56 of them 14.8.)
+  const uint32_t logical =
+      a.nTiles > 1 ? xcdSwizzle(blockIdx.x, gridDim.x) : blockIdx.x;
+  const uint32_t nTile = logical % a.nTiles;
+  const uint32_t walker = (logical / a.nTiles) % a.walkers;
+  const uint32_t g = logical / (a.walkers * a.nTiles);
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
   const uint32_t pixelBytes = d.groups * d.inChansPerGroup * 2;
 
@@ -117,24 +131,40 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
   // ---- compute waves.  This wave's weights -> registers: block nb of the
   // two 32-channel blocks, every k-slice.
   const int mb = wave >> 1, nb = wave & 1;
-  half8 wf[KS];
-  {
+  half8 wf[NT][KS];
+#pragma unroll
+  for (int nt = 0; nt != NT; ++nt) {
     const uintx4 *src =
         reinterpret_cast<const uintx4 *>(w) +
-        (size_t(g * a.nBlocks + nTile * 2 + nb) * KS) * 64 + lane;
+        (size_t(g * a.nBlocks + nTile * NT * 2 + nb * NT + nt) * KS) * 64 + lane;
 #pragma unroll
     for (int ks = 0; ks != KS; ++ks)
-      wf[ks] = __builtin_bit_cast(half8, src[ks * 64]);
+      wf[nt][ks] = __builtin_bit_cast(half8, src[ks * 64]);
   }
-  // Bias of this lane's channels 8 q + 4 (lane / 32) + e.
-  float biasV[16];
+  // One channel tile: the bias of this lane's channels 8 q + 4 (lane / 32) +
+  // e stays in registers.  More: the workgroup's bias waits in LDS (registers
+  // hold the weights), visible to all behind the first tile's barrier.
+  float biasV[NT == 1 ? 16 : 1] = {};
+  if constexpr (NT == 1) {
 #pragma unroll
-  for (int v = 0; v != 16; ++v) {
-    const uint32_t n =
-        nTile * kPwChans + nb * 32 + 8 * (v / 4) + 4 * (lane >> 5) + v % 4;
-    biasV[v] = bias && n < d.outChansPerGroup
-                   ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
-                   : 0.0f;
+    for (int v = 0; v != 16; ++v) {
+      const uint32_t n =
+          nTile * kPwChans + nb * 32 + 8 * (v / 4) + 4 * (lane >> 5) + v % 4;
+      biasV[v] = bias && n < d.outChansPerGroup
+                     ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
+                     : 0.0f;
+    }
+  }
+  float *biasLds = reinterpret_cast<float *>(
+      lds + NB * kTileBytes + kComputeWaves * 32 * kPwStageRow);
+  if (NT > 1 && bias) {
+    for (uint32_t i = t; i < NT * kPwChans; i += kComputeWaves * 64) {
+      const uint32_t n = nTile * NT * kPwChans + i;
+      biasLds[i] = n < d.outChansPerGroup
+                       ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
+                       : 0.0f;
+    }
+    MXK_WAIT_LGKMCNT0();
   }
   const uint32_t rowLocal = mb * 32 + (lane & 31);
   const uint32_t swizzle = rowLocal & kSwizzle, half = lane >> 5;
@@ -151,52 +181,152 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
     const char *rowPtr = lds + buffer * kTileBytes + rowLocal * kRow;
     if (++buffer == NB)
       buffer = 0;
-    floatx16 acc;
+    if constexpr (NT % 2 == 0 && sizeof(OutT) == 2) {
+      // Two adjacent 32-channel blocks at a time: one read of the pixels
+      // feeds both, and their 64 channels leave as 128 contiguous bytes per
+      // pixel and store - whole lines, where a block alone writes half of
+      // one.  (64 -> 256 channels on N = 32, 56 x 56: 16.1 us with one
+      // 64-channel tile per workgroup, 14.5 with four and a wave's blocks
+      // adjacent; storing them together or even fully contiguously changes
+      // no more than 5 % of that, and neither do the staging waits: the
+      // layer's 51 MB of output take 9.6 us as a plain fill.)  Sixteen pixels
+      // at a time fit the wave's staging block.
+      static_assert(16 * kPwPairRow <= 32 * kPwStageRow, "staging fits");
 #pragma unroll
-    for (int v = 0; v != 16; ++v)
-      acc[v] = biasV[v];
+      for (int np = 0; np != NT / 2; ++np) {
+        floatx16 acc[2];
 #pragma unroll
-    for (int ks = 0; ks != KS; ++ks) {
-      const half8 x = *reinterpret_cast<const half8 *>(
-          rowPtr + (((ks * 2 + half) ^ swizzle) << 4));
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[ks], x, acc, 0, 0, 0);
-    }
-    // lane = pixel lane % 32, registers = channels 8 (v / 4) + 4 (lane / 32)
-    // + v % 4: transpose through this wave's staging block and store.
+        for (int j = 0; j != 2; ++j) {
+          if (bias) {
+            const float *b =
+                biasLds + (nb * NT + 2 * np + j) * 32 + 4 * half;
 #pragma unroll
-    for (int pass = 0; pass != 32 / kPassChans; ++pass) {
+            for (int q = 0; q != 4; ++q) {
+              const floatx4 four =
+                  *reinterpret_cast<const floatx4 *>(b + 8 * q);
 #pragma unroll
-      for (int q = pass * (kPassChans / 8); q != (pass + 1) * (kPassChans / 8);
-           ++q) {
-        float v[4];
+              for (int e = 0; e != 4; ++e)
+                acc[j][4 * q + e] = four[e];
+            }
+          } else {
 #pragma unroll
-        for (int e = 0; e != 4; ++e)
-          v[e] = acc[q * 4 + e];
-        storeOut4(reinterpret_cast<OutT *>(stage + (lane & 31) * kPwStageRow) +
-                      (8 * q + 4 * half - pass * kPassChans),
-                  v);
-      }
-      // wave-private: only this wave's LDS writes have to be visible
-      MXK_WAIT_LGKMCNT0();
-      const uint32_t vec = lane & 3; // 4 x 16 bytes per pixel and pass
-      const uint32_t n =
-          nTile * kPwChans + nb * 32 + pass * kPassChans + vec * kVecElems;
+            for (int v = 0; v != 16; ++v)
+              acc[j][v] = 0.0f;
+          }
+        }
 #pragma unroll
-      for (int rows = 0; rows != 2; ++rows) {
-        const uint32_t r = rows * 16 + (lane >> 2);
-        const uint32_t m = mTile * TM + mb * 32 + r;
-        const uintx4 data =
-            *reinterpret_cast<const uintx4 *>(stage + r * kPwStageRow + vec * 16);
-        if (m < a.M && n < d.outChansPerGroup) {
-          uintx4 *dst = reinterpret_cast<uintx4 *>(
-              out + size_t(m) * outChans + g * d.outChansPerGroup + n);
-          // streaming store (the output is not read again here): 15.2 ->
-          // 12.4 us on the 56 x 56, 256 -> 64 layer.  The same hint on the
-          // loads loses a microsecond of that.
-          __builtin_nontemporal_store(data, dst);
+        for (int ks = 0; ks != KS; ++ks) {
+          const half8 x = *reinterpret_cast<const half8 *>(
+              rowPtr + (((ks * 2 + half) ^ swizzle) << 4));
+#pragma unroll
+          for (int j = 0; j != 2; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                wf[2 * np + j][ks], x, acc[j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int ph = 0; ph != 2; ++ph) {
+          if (((lane >> 4) & 1) == ph) {
+#pragma unroll
+            for (int j = 0; j != 2; ++j)
+#pragma unroll
+              for (int q = 0; q != 4; ++q) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e != 4; ++e)
+                  v[e] = acc[j][q * 4 + e];
+                storeOut4(
+                    reinterpret_cast<OutT *>(stage + (lane & 15) * kPwPairRow) +
+                        (32 * j + 8 * q + 4 * half),
+                    v);
+              }
+          }
+          MXK_WAIT_LGKMCNT0(); // (wave-private staging)
+#pragma unroll
+          for (int i = 0; i != 2; ++i) {
+            const uint32_t u = lane + 64 * i;
+            const uint32_t r = u >> 3, vec = u & 7;
+            const uint32_t m = mTile * TM + mb * 32 + ph * 16 + r;
+            const uint32_t n =
+                nTile * NT * kPwChans + (nb * NT + 2 * np) * 32 + vec * 8;
+            const uintx4 data = *reinterpret_cast<const uintx4 *>(
+                stage + r * kPwPairRow + vec * 16);
+            if (m < a.M && n < d.outChansPerGroup)
+              __builtin_nontemporal_store(
+                  data, reinterpret_cast<uintx4 *>(
+                            out + size_t(m) * outChans +
+                            g * d.outChansPerGroup + n));
+          }
+          MXK_WAIT_LGKMCNT0(); // read before the next pixels overwrite it
         }
       }
-      MXK_WAIT_LGKMCNT0(); // staging is read before the next pass rewrites it
+    } else
+#pragma unroll
+    for (int nt = 0; nt != NT; ++nt) {
+      floatx16 acc;
+      if constexpr (NT == 1) {
+#pragma unroll
+        for (int v = 0; v != 16; ++v)
+          acc[v] = biasV[v];
+      } else if (bias) {
+        // lane's channels 8 q + 4 (lane / 32) + e of the block
+        const float *b = biasLds + (nb * NT + nt) * 32 + 4 * half;
+#pragma unroll
+        for (int q = 0; q != 4; ++q) {
+          const floatx4 four = *reinterpret_cast<const floatx4 *>(b + 8 * q);
+#pragma unroll
+          for (int e = 0; e != 4; ++e)
+            acc[4 * q + e] = four[e];
+        }
+      } else {
+#pragma unroll
+        for (int v = 0; v != 16; ++v)
+          acc[v] = 0.0f;
+      }
+#pragma unroll
+      for (int ks = 0; ks != KS; ++ks) {
+        const half8 x = *reinterpret_cast<const half8 *>(
+            rowPtr + (((ks * 2 + half) ^ swizzle) << 4));
+        acc =
+            __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[nt][ks], x, acc, 0, 0, 0);
+      }
+      // lane = pixel lane % 32, registers = channels 8 (v / 4) + 4 (lane /
+      // 32) + v % 4: transpose through this wave's staging block and store.
+#pragma unroll
+      for (int pass = 0; pass != 32 / kPassChans; ++pass) {
+#pragma unroll
+        for (int q = pass * (kPassChans / 8);
+             q != (pass + 1) * (kPassChans / 8); ++q) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e != 4; ++e)
+            v[e] = acc[q * 4 + e];
+          storeOut4(
+              reinterpret_cast<OutT *>(stage + (lane & 31) * kPwStageRow) +
+                  (8 * q + 4 * half - pass * kPassChans),
+              v);
+        }
+        // wave-private: only this wave's LDS writes have to be visible
+        MXK_WAIT_LGKMCNT0();
+        const uint32_t vec = lane & 3; // 4 x 16 bytes per pixel and pass
+        const uint32_t n = nTile * NT * kPwChans + (nb * NT + nt) * 32 +
+                           pass * kPassChans + vec * kVecElems;
+#pragma unroll
+        for (int rows = 0; rows != 2; ++rows) {
+          const uint32_t r = rows * 16 + (lane >> 2);
+          const uint32_t m = mTile * TM + mb * 32 + r;
+          const uintx4 data = *reinterpret_cast<const uintx4 *>(
+              stage + r * kPwStageRow + vec * 16);
+          if (m < a.M && n < d.outChansPerGroup) {
+            uintx4 *dst = reinterpret_cast<uintx4 *>(
+                out + size_t(m) * outChans + g * d.outChansPerGroup + n);
+            // streaming store (the output is not read again here): 15.2 ->
+            // 12.4 us on the 56 x 56, 256 -> 64 layer.  The same hint on the
+            // loads loses a microsecond of that.
+            __builtin_nontemporal_store(data, dst);
+          }
+        }
+        MXK_WAIT_LGKMCNT0(); // staging is read before the next pass rewrites it
+      }
     }
   }
 }
@@ -260,19 +390,40 @@ constexpr PwShape shapeFor(uint32_t ci) {
   return ci == 64 ? kShape64 : ci == 128 ? kShape128 : ci == 256 ? kShape256
                                                                  : kShape512;
 }
-constexpr uint32_t ldsBytesOf(PwShape s, uint32_t ci) {
-  return uint32_t(s.nb * s.tm * (ci / 16) * 32 + (s.tm / 16) * 32 * kPwStageRow);
+constexpr uint32_t ldsBytesOf(PwShape s, uint32_t ci, uint32_t nt = 1) {
+  return uint32_t(s.nb * s.tm * (ci / 16) * 32 +
+                  (s.tm / 16) * 32 * kPwStageRow + nt * kPwChans * 4);
 }
 
-template <int KS, int TM, int NB, int LW, class OutT>
-hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
-               void *out, hipStream_t stream) {
-  constexpr int ldsBytes = ldsBytesOf(PwShape{TM, NB, LW}, KS * 16);
-  static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void *>(&pointwiseKernel<KS, TM, NB, LW, OutT>),
-      hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
-  if (attr != hipSuccess)
-    return attr;
+/// 64-channel tiles of the output per workgroup.  With 64 input channels as
+/// many (4, 3, 2, 1) as divide the layer's and still leave the chip two
+/// workgroups per CU to share out.  With 128 input channels two, where every
+/// workgroup still walks over six tiles or more: N = 32, 56 x 56, 128 -> 256
+/// channels reads its 26 MB of input four times with one tile per workgroup
+/// (25.1 us); on N = 32, 28 x 28, 128 -> 512 two tiles leave each workgroup
+/// four pixel tiles instead of seven and lose (9.0 -> 10.6 us).
+uint32_t chanTilesFor(const PointwiseDesc &d, uint32_t cus) {
+  if (d.chanTiles)
+    return d.chanTiles; // asked for by name (checked by pointwiseTakes)
+  const PwShape s = shapeFor(d.inChansPerGroup);
+  const uint64_t mTiles = (uint64_t(d.batch) * d.pixels + s.tm - 1) / s.tm;
+  const uint64_t tiles64 = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
+  if (d.inChansPerGroup == 64) {
+    for (uint32_t nt = 4; nt > 1; --nt)
+      if (tiles64 % nt == 0 && mTiles * (tiles64 / nt) * d.groups >= 2ull * cus)
+        return nt;
+  } else if ((d.inChansPerGroup == 128 || d.inChansPerGroup == 256) &&
+             tiles64 % 2 == 0) {
+    const uint64_t pairs = tiles64 / 2 * d.groups;
+    const uint64_t walkers = walkersFor(
+        mTiles, pairs, ldsBytesOf(s, d.inChansPerGroup, 2), cus);
+    if ((mTiles + walkers - 1) / walkers >= 6)
+      return 2;
+  }
+  return 1;
+}
+
+int deviceCUs() {
   static const int cus = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -282,6 +433,21 @@ hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
       n = 256;
     return n;
   }();
+  return cus;
+}
+
+template <int KS, int TM, int NB, int LW, int NT, class OutT>
+hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
+               void *out, hipStream_t stream) {
+  constexpr int ldsBytes = ldsBytesOf(PwShape{TM, NB, LW}, KS * 16, NT);
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void *>(
+          &pointwiseKernel<KS, TM, NB, LW, NT, OutT>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+  if (attr != hipSuccess)
+    return attr;
+  const int cus = deviceCUs();
+  a.nTiles /= NT; // the workgroups' shares of NT * 64 channels
   a.mTiles = (a.M + TM - 1) / TM;
   const uint64_t pairs = uint64_t(a.nTiles) * a.d.groups;
   if (pairs == 0 || a.mTiles == 0)
@@ -293,7 +459,7 @@ hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
   if (blocks > 0x7fffffffull ||
       uint64_t(a.mTiles) + uint64_t(NB) * walkers > 0x7fffffffull / TM)
     return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((pointwiseKernel<KS, TM, NB, LW, OutT>),
+  hipLaunchKernelGGL((pointwiseKernel<KS, TM, NB, LW, NT, OutT>),
                      dim3(uint32_t(blocks)), dim3(TM * 4 + 64 * LW), ldsBytes,
                      stream, a, static_cast<const char *>(in),
                      static_cast<const char *>(w),
@@ -304,18 +470,34 @@ hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
 template <class OutT>
 hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
                      const void *bias, void *out, hipStream_t stream) {
+  const uint32_t nt = chanTilesFor(a.d, uint32_t(deviceCUs()));
   switch (a.d.inChansPerGroup) {
   case 64:
-    return run<4, kShape64.tm, kShape64.nb, kShape64.lw, OutT>(a, in, w, bias,
-                                                              out, stream);
+    if (nt == 4)
+      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT>(
+          a, in, w, bias, out, stream);
+    if (nt == 3)
+      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT>(
+          a, in, w, bias, out, stream);
+    if (nt == 2)
+      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT>(
+          a, in, w, bias, out, stream);
+    return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT>(
+        a, in, w, bias, out, stream);
   case 128:
-    return run<8, kShape128.tm, kShape128.nb, kShape128.lw, OutT>(
+    if (nt == 2)
+      return run<8, kShape128.tm, kShape128.nb, kShape128.lw, 2, OutT>(
+          a, in, w, bias, out, stream);
+    return run<8, kShape128.tm, kShape128.nb, kShape128.lw, 1, OutT>(
         a, in, w, bias, out, stream);
   case 256:
-    return run<16, kShape256.tm, kShape256.nb, kShape256.lw, OutT>(
+    if (nt == 2)
+      return run<16, kShape256.tm, kShape256.nb, kShape256.lw, 2, OutT>(
+          a, in, w, bias, out, stream);
+    return run<16, kShape256.tm, kShape256.nb, kShape256.lw, 1, OutT>(
         a, in, w, bias, out, stream);
   case 512:
-    return run<32, kShape512.tm, kShape512.nb, kShape512.lw, OutT>(
+    return run<32, kShape512.tm, kShape512.nb, kShape512.lw, 1, OutT>(
         a, in, w, bias, out, stream);
   }
   return hipErrorInvalidValue;
@@ -323,12 +505,21 @@ hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
 
 } // namespace
 
+bool pointwiseChanTilesOk(const PointwiseDesc &d, uint32_t chanTiles) {
+  const uint32_t tiles64 = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
+  const uint32_t most = d.inChansPerGroup == 64    ? 4
+                        : d.inChansPerGroup == 512 ? 1
+                                                   : 2;
+  return chanTiles >= 1 && chanTiles <= most && tiles64 % chanTiles == 0;
+}
+
 bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType) {
   const uint32_t ci = d.inChansPerGroup, co = d.outChansPerGroup;
   const uint64_t m = uint64_t(d.batch) * d.pixels;
   const uint64_t inBytes = m * d.groups * ci * 2;
   return inType == kHalf && (outType == kHalf || outType == kFloat) &&
          (ci == 64 || ci == 128 || ci == 256 || ci == 512) && co != 0 &&
+         (d.chanTiles == 0 || pointwiseChanTilesOk(d, d.chanTiles)) &&
          co % (outType == kHalf ? 8 : 4) == 0 && m != 0 && m < 0x7fffffffull &&
          inBytes < kOutOfRange &&
          pointwisePackedElems(d) * 2 < kOutOfRange;
@@ -362,12 +553,14 @@ PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus) {
   l.tilePixels = uint32_t(s.tm), l.ring = uint32_t(s.nb);
   l.loaderWaves = uint32_t(s.lw);
   const uint64_t mTiles = (uint64_t(d.batch) * d.pixels + s.tm - 1) / s.tm;
+  const uint32_t nt = chanTilesFor(d, cus);
+  l.chansPerWorkgroup = nt * kPwChans;
   const uint64_t pairs =
-      uint64_t((d.outChansPerGroup + kPwChans - 1) / kPwChans) * d.groups;
+      uint64_t((d.outChansPerGroup + kPwChans - 1) / kPwChans) / nt * d.groups;
   if (mTiles == 0 || pairs == 0)
     return l;
   const uint64_t walkers =
-      walkersFor(mTiles, pairs, ldsBytesOf(s, d.inChansPerGroup), cus);
+      walkersFor(mTiles, pairs, ldsBytesOf(s, d.inChansPerGroup, nt), cus);
   l.workgroups = walkers * pairs;
   l.tilesPerWorkgroup = uint32_t((mTiles + walkers - 1) / walkers);
   return l;

@@ -206,6 +206,10 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       if (v > 1)
         throw invalid_option("'" + sub + "': Must be 0 or 1");
       pc.rowRing = int(v);
+    } else if (m.first == "chanTiles") {
+      pc.chanTiles = requireUnsigned(sub, m.second);
+      if (pc.chanTiles < 1 || pc.chanTiles > 4)
+        throw invalid_option("'" + sub + "': Must be 1 to 4");
     } else if (m.first == "tileH") {
       pc.tileH = requireUnsigned(sub, m.second);
     } else if (m.first == "tileW") {

@@ -50,6 +50,9 @@ struct PlanConstraints {
   /// input rows in LDS: -1 planner's choice, 0 never, 1 whenever it can take
   /// the layer.
   int rowRing = -1;
+  /// 64-channel tiles of the output per workgroup of the pointwise streaming
+  /// kernel (1 to 4); 0 = planner's choice.
+  unsigned chanTiles = 0;
   std::string text; // the JSON as given, kept for reporting and cache keys
 };
 

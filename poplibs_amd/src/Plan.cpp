@@ -336,7 +336,10 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       if (options.planConstraints.rowRing != 0 &&
           mxk::depthwiseRowsDeltaTakes(f) &&
           (options.planConstraints.rowRing == 1 ||
-           (l.workgroups * 2 >= gfx950::numCUs && l.rowsOut >= 4)))
+           // (strips of fewer than four columns read mostly halo: N = 32,
+           // 7 x 7, 960 channels 20.5 us against 13.1)
+           (l.workgroups * 2 >= gfx950::numCUs && l.rowsOut >= 4 &&
+            (l.colsOut >= 4 || l.strips == 1))))
         f.dense3x3 = 2;
     }
   }
@@ -747,6 +750,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     pw.batch = g.batch, pw.pixels = s.outH * s.outW;
     pw.groups = g.groups, pw.inChansPerGroup = g.inChansPerGroup;
     pw.outChansPerGroup = g.outChansPerGroup;
+    pw.chanTiles = pc.chanTiles;
     const bool unitWindow =
         !s.hasDepth() && !s.outputPadded() && !s.kernelSelected &&
         !s.inputDilated() &&
@@ -768,6 +772,12 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                                                               : mxk::kFloat);
     if (plan.pointwiseOn)
       plan.weightPackedElems = mxk::pointwisePackedElems(pw);
+    else if (pc.chanTiles)
+      throw poplar::invalid_option(
+          "planConstraints gfx950 chanTiles: the pointwise streaming kernel "
+          "does not take this convolution with that many 64-channel tiles "
+          "per workgroup (they divide the layer's; at most 4 with 64 input "
+          "channels, 2 with 128 or 256, 1 with 512)");
     // Unit stride and whole 128-byte slices of channels: the kernel that
     // keeps the tile's input patch in LDS reads every input element once
     // instead of once per tap.
@@ -1037,7 +1047,7 @@ std::string mxconv_plan::describe() const {
       const mxk::PointwiseLaunch l =
           mxk::pointwiseLaunchShape(pointwise, gfx950::numCUs);
       os << "        block M x N x K            " << l.tilePixels
-         << " x 64 x " << k << "\n";
+         << " x " << l.chansPerWorkgroup << " x " << k << "\n";
       os << "        workgroups                 " << l.workgroups << " on "
          << gfx950::numCUs << " CUs, each taking " << l.tilesPerWorkgroup
          << " tiles in turn through a ring of " << l.ring

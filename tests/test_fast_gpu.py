@@ -113,6 +113,65 @@ def test_pointwise_matches_oracle(oracle, kw, out_type):
     _run(oracle, p, 8, 1e-3, "implicit GEMM", wscale=0.1)
 
 
+# Several 64-channel tiles of the output per workgroup (the planner's choice
+# for large layers that widen the channels), forced onto small ones: pixels
+# ragged against the tile, channels that fill the last tile partly, groups.
+CHAN_TILE_CASES = [
+    (dict(batch=2, field=(28, 29), kernel=(1, 1), ci=64, co=256), 4),
+    (dict(batch=2, field=(28, 29), kernel=(1, 1), ci=64, co=256), 2),
+    (dict(batch=3, field=(7, 11), kernel=(1, 1), ci=64, co=168), 3),
+    (dict(batch=1, field=(19, 9), kernel=(1, 1), ci=64, co=200, groups=2), 4),
+    (dict(batch=3, field=(13, 11), kernel=(1, 1), ci=128, co=256), 2),
+    (dict(batch=2, field=(9, 31), kernel=(1, 1), ci=128, co=104, groups=3), 2),
+    (dict(batch=2, field=(17, 12), kernel=(1, 1), ci=256, co=128), 2),
+    (dict(batch=1, field=(6, 40), kernel=(1, 1), ci=256, co=72, groups=2), 2),
+]
+
+
+@pytest.mark.parametrize("kw,tiles", CHAN_TILE_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+@pytest.mark.parametrize("bias", [False, True])
+def test_pointwise_channel_tiles_match_oracle(oracle, kw, tiles, out_type,
+                                              bias):
+    p = make_params(pa.HALF, out_type, **kw)
+    options = {"planConstraints": '{"gfx950": {"chanTiles": %d}}' % tiles}
+    text = pa.Plan(p, options).describe()
+    assert "pointwise streaming variant" in text, text
+    assert " x %d x %d\n" % (64 * tiles, kw["ci"]) in text, text
+    _run(oracle, p, 14, 1e-3, "implicit GEMM", wscale=0.1, options=options,
+         bias=bias)
+
+
+def test_pointwise_channel_tiles_pm1_exact_and_plan_choice(oracle):
+    kw, tiles = CHAN_TILE_CASES[0]
+    options = {"planConstraints": '{"gfx950": {"chanTiles": %d}}' % tiles}
+    for out_type in (pa.HALF, pa.FLOAT):
+        p = make_params(pa.HALF, out_type, **kw)
+        _run(oracle, p, 15, 0, "implicit GEMM", dist="pm1", options=options)
+    # the planner's own choice: large layers that widen the channels
+    def block(**kw):
+        import re
+        text = pa.Plan(make_params(pa.HALF, **kw)).describe()
+        return re.search(r"block M x N x K +(.*)", text).group(1)
+    big = dict(batch=32, field=(56, 56), kernel=(1, 1))
+    assert block(ci=64, co=256, **big) == "128 x 256 x 64"
+    assert block(ci=64, co=192, **big) == "128 x 192 x 64"
+    assert block(ci=128, co=256, **big) == "128 x 128 x 128"
+    assert block(ci=256, co=128, **big) == "64 x 128 x 256"
+    assert block(ci=256, co=64, **big) == "64 x 64 x 256"
+    # few pixel tiles per workgroup: one channel tile each
+    assert block(ci=128, co=512, batch=32, field=(28, 28),
+                 kernel=(1, 1)) == "128 x 64 x 128"
+    assert block(**kw) == "128 x 64 x 64"
+    # tiles that do not divide the layer's, or too many for the registers
+    for bad_kw, bad in ((dict(ci=64, co=192), 2), (dict(ci=128, co=256), 4),
+                        (dict(ci=512, co=128), 2)):
+        with pytest.raises(pa.MxconvError):
+            pa.Plan(make_params(pa.HALF, **bad_kw, **big),
+                    {"planConstraints":
+                     '{"gfx950": {"chanTiles": %d}}' % bad})
+
+
 def test_pointwise_pm1_exact_and_big_tile_on_request(oracle):
     p = make_params(pa.HALF, pa.FLOAT, **POINTWISE_CASES[1])
     _run(oracle, p, 9, 0, "implicit GEMM", dist="pm1")
