@@ -227,8 +227,9 @@ double roundsOf(std::size_t workgroups, std::size_t perCU) {
 /// igemmKernel: 1.45 us start-up + 1.5 us epilogue, 0.345 us per k-step of a
 /// 128 x 128 tile (0.24 for 128 x 64); further rounds on a CU pay another
 /// 1.5 us (nothing overlaps the next workgroup's start-up); two workgroups
-/// sharing a CU take 2.1 times one's time between them; K split adds the
-/// second kernel's 5 us.
+/// sharing a CU take 2.1 times one's time between them; K split adds 9 us
+/// (fp32 partial tiles out and in again, the second kernel: 20.4 us measured
+/// where the tiles alone are estimated at 11.2, 15.0 against 6.7).
 double estimateStreaming(std::size_t workgroups, std::size_t kSteps,
                          std::size_t perCU, unsigned blockN, unsigned splitK) {
   const double rounds = roundsOf(workgroups, perCU);
@@ -238,7 +239,7 @@ double estimateStreaming(std::size_t workgroups, std::size_t kSteps,
     tile += 1.5;
   if (perCU == 2)
     tile *= double(workgroups) > double(gfx950::numCUs) ? 2.1 : 1.0;
-  return kLaunchUs + rounds * tile + (splitK > 1 ? 5.0 : 0.0);
+  return kLaunchUs + rounds * tile + (splitK > 1 ? 9.0 : 0.0);
 }
 
 /// igemmPatchKernel (mode 1): 1.9 us to the first MFMA + 0.5 us reduction and
@@ -783,7 +784,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     // instead of once per tap.
     if (!plan.pointwiseOn && plan.igemmPhases.empty() &&
         !plan.paddedInputChans &&
-        (g.splitK == 1 || (pc.patch >= 1 && !pc.splitK)) && pc.patch != 0 &&
+        (g.splitK == 1 || !pc.splitK) && pc.patch != 0 &&
         !pc.blockN && !pc.blockK && !pc.stages) {
       const int inId = halfIn ? mxk::kHalf : floatIn ? mxk::kFloat
                                                      : mxk::kQuarter;
@@ -861,7 +862,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         const std::size_t i = addPatch(uint32_t(pc.patch), bm);
         if (i != none)
           best = i;
-      } else if (g.splitK == 1 && s.kH * s.kW > 1 && co > 64) {
+      } else if (s.kH * s.kW > 1 && co > 64) {
+        // (also against a streaming plan that splits K: the patch kernel's
+        // equal tiles fill the chip without the second kernel - N = 32,
+        // 14 x 14, 256 -> 256 channels 20.4 -> 12.4 us, N = 8, 28 x 28,
+        // 128 -> 128 15.0 -> 7.7)
         for (Tiling t : {Tiling{1, 128}, Tiling{1, 64}, Tiling{2, equalM}}) {
           // (a forced tile height picks among the patch tilings only)
           if (pc.blockM && pc.blockM != t.blockM)

@@ -19,7 +19,9 @@ FAKE = 0x1000  # a device "pointer" no checked path touches
 def _split_k_plan():
     p = make_params(pa.HALF, batch=4, field=(14, 14), kernel=(3, 3), ci=256,
                     co=256, pad=1)
-    plan = pa.Plan(p)
+    # (without the constraint the planner prefers the resident-patch kernel,
+    # which needs no workspace)
+    plan = pa.Plan(p, {"planConstraints": '{"gfx950": {"patch": 0}}'})
     assert "K split" in plan.describe()
     assert plan.buffer_bytes(capi.BUF_WORKSPACE) > 0
     return plan

@@ -529,7 +529,8 @@ def test_plan_estimated_costs():
     assert 1.7 * a < b < 2.0 * a  # one launch overhead, twice the bytes
     # K split: the fp32 partial tiles are temporary memory
     deep = pa.Plan(make_params(pa.HALF, batch=8, field=(28, 28),
-                               kernel=(3, 3), ci=128, co=128, pad=1))
+                               kernel=(3, 3), ci=128, co=128, pad=1),
+                   {"planConstraints": '{"gfx950": {"patch": 0}}'})
     assert "K split into parts" in deep.describe()
     cycles, memory = deep.estimated_costs()
     assert memory == deep.buffer_bytes(capi.BUF_WORKSPACE) > 0
