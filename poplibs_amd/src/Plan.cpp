@@ -246,15 +246,16 @@ double estimateStreaming(std::size_t workgroups, std::size_t kSteps,
 /// stores, 0.333 us per k-step of 128 pixels (half of that for 64); one
 /// workgroup per CU, so further rounds pay their start-up in full (4.5 us
 /// instead of 2.4).  igemmPatch16Kernel (mode 2): seven blocks of 16 pixels
-/// whatever the tile's height, 0.34 us per k-step, 1.5 us around them (2.6 us
-/// in further rounds).  Measured: 9.6 us for 256 tiles of 18 k-steps, 20.5 us
-/// for 50 k-steps, 128.6 us for 14 rounds of 18, 60 us for 4 rounds of 36.
+/// whatever the tile's height, 0.29 us per k-step and 1.5 us around them in
+/// a launch of one round (8.6 us measured for 224 tiles of 18 k-steps, 17.1
+/// for 50 k-steps), 0.34 and 2.6 us in launches of several (55 us for 4
+/// rounds of 36, 110 us for 7 rounds of 36, 35 us for 4 rounds of 18).
 double estimatePatch(std::size_t workgroups, std::size_t kSteps, unsigned mode,
                      unsigned blockM) {
   const double rounds = roundsOf(workgroups, 1);
   if (mode == 2)
-    return kLaunchUs +
-           rounds * ((rounds > 1 ? 2.6 : 1.5) + 0.34 * double(kSteps));
+    return kLaunchUs + rounds * ((rounds > 1 ? 2.6 : 1.5) +
+                                 (rounds > 1 ? 0.34 : 0.29) * double(kSteps));
   const double step = blockM == 128 ? 0.333 : 0.167;
   const double fixed = rounds > 1 ? 4.5 : 2.4;
   return kLaunchUs + rounds * (fixed + step * double(kSteps));
