@@ -382,12 +382,26 @@ __global__ __launch_bounds__(1024) void depthwiseDeltaSumKernel(
 #pragma unroll
     for (int u = 0; u != width; ++u)
       sum[u] += sum[u + width];
+  // The 64 sums of an output meet in two steps of eight, each in order (one
+  // thread adding all 64 is a chain of 64 LDS reads at the kernel's end).
   meet[part][column] = sum[0];
+  __syncthreads();
+  float eight = 0.0f;
+  if (part < 8) {
+    eight = meet[part * 8][column];
+#pragma unroll
+    for (int w = 1; w != 8; ++w)
+      eight += meet[part * 8 + w][column];
+  }
+  __syncthreads();
+  if (part < 8)
+    meet[part][column] = eight;
   __syncthreads();
   if (part != 0 || i >= outputs)
     return;
   float total = meet[0][column];
-  for (int w = 1; w != 64; ++w)
+#pragma unroll
+  for (int w = 1; w != 8; ++w)
     total += meet[w][column];
   const uint32_t tap = i / channels, c = i - tap * channels;
   storeOut(out, size_t(c) * taps + tap, total);
