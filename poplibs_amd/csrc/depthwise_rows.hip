@@ -325,20 +325,33 @@ constexpr int kSumRow = 73; // floats a thread leaves for the columns' meeting
 
 /// Rings of the weight-delta kernel: rows of activations as in the forward
 /// kernel, one row of deltas per step; four steps' rows on the way at stride
-/// 1, three at stride 2 (140 / 124 KB of LDS).
+/// 1, three at stride 2 (124 / 140 KB of LDS).  Eight compute waves at stride
+/// 1, as in the forward kernel (a step moves half a stride-2 step's bytes for
+/// the same multiply-adds); the rings' memory is where the columns' sums meet
+/// at the end, 73 floats per compute thread.
 template <int S> struct DeltaRing {
   static constexpr int kAhead = S == 2 ? 3 : 4;
   static constexpr int kSlots = kAhead * S + 3;
   static constexpr int kDeltaSlots = kAhead + 1;
-  static constexpr int kBytes =
+  static constexpr int kComputeWaves = S == 1 ? 8 : 6;
+  static constexpr int kComputeThreads = 64 * kComputeWaves;
+  static constexpr int kThreads = 64 * (kComputeWaves + kLoaderWaves);
+  static constexpr int kRingBytes =
       kSlots * kSlotBytes + kDeltaSlots * kDeltaSlotBytes;
-  static_assert(kBytes >= kComputeThreads * kSumRow * 4, "the sums fit");
+  static constexpr int kSumBytes = kComputeThreads * kSumRow * 4;
+  static constexpr int kBytes = kRingBytes > kSumBytes ? kRingBytes : kSumBytes;
+  static_assert(kComputeThreads * 16 <= kDeltaSlotBytes,
+                "every compute thread has a unit of a row of deltas");
   static_assert(kBytes <= 160 * 1024, "LDS of a CU");
 };
+constexpr uint32_t deltaComputeThreads(uint32_t stride) {
+  return stride == 1 ? DeltaRing<1>::kComputeThreads
+                     : DeltaRing<2>::kComputeThreads;
+}
 
 /// partial[walker][tap][c] = the walker's band's sum.
 template <int S>
-__global__ __launch_bounds__(kRowsThreads) void depthwiseRowsDeltaKernel(
+__global__ __launch_bounds__(DeltaRing<S>::kThreads) void depthwiseRowsDeltaKernel(
     RowsArgs a, const __half *__restrict__ acts,
     const __half *__restrict__ deltas, uint32_t deltaBytes,
     float *__restrict__ partial) {
@@ -364,10 +377,10 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsDeltaKernel(
   const uint32_t pixelBytes = d.channels * 2;
   const uint32_t rowsIn = (steps - 1) * S + 3;
 
-  if (wave >= kComputeWaves) {
+  if (wave >= R::kComputeWaves) {
     // ---- loaders: per step the new rows of activations, then the step's
     // row of deltas (output columns [ow0, ow0 + colsOut) of row oh0 + j).
-    const int loader = wave - kComputeWaves;
+    const int loader = wave - R::kComputeWaves;
     const __amdgpu_buffer_rsrc_t actBuf = bufferOf(acts, a.inBytes);
     const __amdgpu_buffer_rsrc_t deltaBuf = bufferOf(deltas, deltaBytes);
     StripRow<kOwnLoads> actStrip;
@@ -477,7 +490,7 @@ __global__ __launch_bounds__(kRowsThreads) void depthwiseRowsDeltaKernel(
   __syncthreads();
   const uint32_t outputs = 9 * d.channels;
   float *dst = partial + size_t(walker) * outputs;
-  for (uint32_t o = t; o < outputs; o += kComputeThreads) {
+  for (uint32_t o = t; o < outputs; o += R::kComputeThreads) {
     const uint32_t tap = o / d.channels, c = o - tap * d.channels;
     const float *from = sums + (c >> 3) * kSumRow + tap * 8 + (c & 7);
     float sum = 0.0f;
@@ -600,11 +613,11 @@ hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
 bool depthwiseRowsDeltaTakes(const DepthwiseDesc &d) {
   const uint64_t deltaBytes =
       uint64_t(d.batch) * d.outH * d.outW * d.channels * 2;
-  return takes(d, kHalf, kComputeThreads) && deltaBytes < kNoByte;
+  return takes(d, kHalf, deltaComputeThreads(d.strideH)) && deltaBytes < kNoByte;
 }
 
 DepthwiseRowsLaunch depthwiseRowsDeltaLaunchShape(const DepthwiseDesc &d) {
-  DepthwiseRowsLaunch l = launchShapeOf(d, kComputeThreads);
+  DepthwiseRowsLaunch l = launchShapeOf(d, deltaComputeThreads(d.strideH));
   l.ringRows = d.strideH == 2 ? DeltaRing<2>::kSlots : DeltaRing<1>::kSlots;
   return l;
 }
@@ -620,7 +633,7 @@ hipError_t launchDepthwiseRowsDeltas(const DepthwiseDesc &d, const void *acts,
   if (!depthwiseRowsDeltaTakes(d) || !partial)
     return hipErrorInvalidValue;
   RowsArgs a{};
-  shapeFor(d, d.cus, a);
+  shapeFor(d, d.cus, a, deltaComputeThreads(d.strideH));
   a.d = d;
   a.inBytes = uint32_t(uint64_t(d.batch) * d.inH * d.inW * d.channels * 2);
   a.divVecs = makeFastDiv(a.vecs);
@@ -638,7 +651,8 @@ hipError_t launchDepthwiseRowsDeltas(const DepthwiseDesc &d, const void *acts,
     if (attr != hipSuccess)
       return attr;
     hipLaunchKernelGGL(depthwiseRowsDeltaKernel<S>, dim3(blocks),
-                       dim3(kRowsThreads), DeltaRing<S>::kBytes, stream, a,
+                       dim3(DeltaRing<S>::kThreads), DeltaRing<S>::kBytes,
+                       stream, a,
                        static_cast<const __half *>(acts),
                        static_cast<const __half *>(deltas), deltaBytes,
                        static_cast<float *>(partial));
