@@ -362,6 +362,9 @@ struct WuTapDesc {
   uint32_t groups, ci, co;
   // pixels (batch, y, x flattened) a workgroup sums over: a multiple of 64
   uint32_t chunkPixels;
+  // the layer's stride: output pixel (y, x) meets input pixel
+  // (y strideH + kh - padH, x strideW + kw - padW)
+  uint32_t strideH = 1, strideW = 1;
 };
 bool wuTapTakes(const WuTapDesc &d);
 /// Pixels per workgroup that give about one workgroup per compute unit.

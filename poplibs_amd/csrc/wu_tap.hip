@@ -1,7 +1,8 @@
-// Weight deltas of a dense unit-stride layer on the matrix cores, straight
+// Weight deltas of a dense layer (any stride) on the matrix cores, straight
 // from the layer's own tensors:
 //   dW[g][co][ci][kh][kw] = sum over b, y, x of
-//       deltas[b][y][x][g][co] * acts[b][y + kh - padH][x + kw - padW][g][ci]
+//       deltas[b][y][x][g][co] *
+//           acts[b][y strideH + kh - padH][x strideW + kw - padW][g][ci]
 // (PopLibs runs this as a convolution of its own with batch and channels
 // exchanged, lib/poplin/Convolution.cpp:3437-3483 calculateWeightDeltas, whose
 // tensors Poplar rearranges on the exchange; here that would be two transposes
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(kWuThreads) void wuTapKernel(
 #pragma unroll
     for (int h = 0; h != 2; ++h) {
       Walker &w = at[h];
-      const uint32_t iy = w.y + tapY, ix = w.x + tapX;
+      const uint32_t iy = w.y * d.strideH + tapY, ix = w.x * d.strideW + tapX;
       const bool inside = w.p < p1;
       const uint32_t deltaAt = inside ? w.deltaAt : kWuInvalid;
       const uint32_t actAt =
@@ -369,7 +370,7 @@ uint64_t tilesOf(const WuTapDesc &d) {
 bool wuTapTakes(const WuTapDesc &d) {
   const uint64_t M = uint64_t(d.batch) * d.outH * d.outW;
   if (M == 0 || d.ci % 8 != 0 || d.co % 8 != 0 || d.ci == 0 || d.co == 0 ||
-      d.kH == 0 || d.kW == 0)
+      d.kH == 0 || d.kW == 0 || d.strideH == 0 || d.strideW == 0)
     return false;
   const uint64_t actBytes =
       uint64_t(d.batch) * d.inH * d.inW * d.groups * d.ci * 2;

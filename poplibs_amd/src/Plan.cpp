@@ -345,16 +345,17 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         f.dense3x3 = 2;
     }
   }
-  // The weight update pass of a dense layer with unit stride and nothing
-  // dilated: batch = the layer's input channels, input channels = its batch,
-  // kernel = its output field, output field = its kernel.  (Opt out:
+  // The weight update pass of a dense layer with an undilated kernel and
+  // input: batch = the layer's input channels, input channels = its batch,
+  // kernel = its output field, output field = its kernel, kernel dilation =
+  // its stride.  (Opt out:
   // planConstraints gfx950 kernel names one.)
   {
     const Simple2D w = asSimple2D(p);
     if (w.ok && !w.hasDepth() && !w.outputPadded() && !w.kernelSelected &&
         !plan.zeroConv && !plan.depthwiseWeightUpdate && !w.inputDilated() &&
         w.batch == p.batchSize && w.strideH == 1 && w.strideW == 1 &&
-        w.dilH == 1 && w.dilW == 1 && params.inputType == poplar::HALF &&
+        params.inputType == poplar::HALF &&
         options.planConstraints.kernel.empty() &&
         options.planConstraints.method == PlanConstraints::Method::ANY) {
       mxk::WuTapDesc &f = plan.denseForward;
@@ -362,6 +363,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       f.inH = w.inH, f.inW = w.inW;
       f.outH = w.kH, f.outW = w.kW, f.kH = w.outH, f.kW = w.outW;
       f.padH = w.padH, f.padW = w.padW;
+      f.strideH = w.dilH, f.strideW = w.dilW; // (the layer's stride)
       f.loH = w.loH, f.hiH = w.hiH, f.loW = w.loW, f.hiW = w.hiW;
       f.groups = uint32_t(p.numConvGroups);
       f.ci = uint32_t(p.batchSize);

@@ -56,7 +56,7 @@ struct mxconv_plan {
   // the parameters as an ordinary convolution).
   bool depthwiseWeightUpdate = false;
   mxk::DepthwiseDesc depthwiseForward{};
-  // ... or of a dense unit-stride layer: the matrix-core kernel that reads
+  // ... or of a dense layer (any stride): the matrix-core kernel that reads
   // the layer's tensors as they are (mxk::launchWuTap).
   bool denseWeightUpdate = false;
   mxk::WuTapDesc denseForward{};

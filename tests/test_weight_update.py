@@ -226,6 +226,15 @@ DENSE_WU_CASES = [
     dict(batch=70, field=(4, 4), kernel=(3, 3), ci=16, co=16, pad=1),
     # one image
     dict(batch=1, field=(40, 36), kernel=(3, 3), ci=16, co=48, pad=1),
+    # strided layers: the 3 x 3 and 1 x 1 downsampling layers of a ResNet at
+    # a small batch, odd fields, strides that differ by dimension
+    # (1024 output pixels or more, or the pass stays a convolution)
+    dict(batch=8, field=(28, 28), kernel=(3, 3), ci=64, co=128, pad=1,
+         stride=2),
+    dict(batch=20, field=(15, 13), kernel=(1, 1), ci=48, co=80, stride=2),
+    dict(batch=18, field=(17, 20), kernel=(3, 2), ci=24, co=40, groups=2,
+         padLower=(1, 0), padUpper=(0, 1), stride=(3, 2)),
+    dict(batch=120, field=(33,), kernel=(7,), ci=16, co=16, pad=3, stride=4),
 ]
 
 
@@ -254,7 +263,7 @@ def test_dense_weight_deltas_from_the_layers_own_tensors(oracle, kw, out_type):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kw", DENSE_WU_CASES[:3])
+@pytest.mark.parametrize("kw", DENSE_WU_CASES[:3] + DENSE_WU_CASES[-4:])
 def test_dense_weight_deltas_of_signs_are_exact(oracle, kw):
     # +-1 tensors: every product and every partial sum is a small integer
     p = make_params(pa.HALF, pa.FLOAT, **kw)
@@ -302,10 +311,14 @@ def test_dense_weight_update_plan_choice():
     assert DENSE_WU in text
     assert "9 tap x channel tiles x 28 chunks of 896 pixels = 252 workgroups" \
         in text
-    # strided layers, tiny pixel counts and fp32 tensors stay with the pass's
-    # own convolution
+    # strided layers take it too
+    assert DENSE_WU in pa.WeightUpdatePlan(
+        make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                    co=128, pad=1, stride=2)).describe()
+    # dilated kernels, tiny pixel counts and fp32 tensors stay with the
+    # pass's own convolution
     for kw in (dict(batch=32, field=(28, 28), kernel=(3, 3), ci=128, co=128,
-                    pad=1, stride=2),
+                    pad=2, kdil=2),
                dict(batch=1, field=(8, 8), kernel=(3, 3), ci=128, co=128,
                     pad=1)):
         assert DENSE_WU not in pa.WeightUpdatePlan(
