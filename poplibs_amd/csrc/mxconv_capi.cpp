@@ -139,19 +139,34 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
   const int outType = plan->params.outputType.id();
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   switch (plan->kernel) {
-  case mxconv_plan::Kernel::IGEMM:
-    if (plan->outputPadded) {
+  case mxconv_plan::Kernel::IGEMM: {
+    // Phases of a zero-stuffed input that no tap reaches (a 1x1 layer's
+    // backward pass at stride 2: three in four) only write zeros (the bias):
+    // where they are half of the phases or more, one fill of the whole output
+    // does that and the launch leaves them out.
+    size_t deadPhases = 0;
+    for (const auto &phase : plan->igemmPhases)
+      deadPhases += phase.d.noTaps ? 1 : 0;
+    const bool fillAll = deadPhases && 2 * deadPhases >= plan->igemmPhases.size();
+    if (plan->outputPadded || fillAll) {
       // zeros (the bias) around the convolution's own outputs
       const mxk::IgemmDesc &g = plan->igemm;
       const uint32_t fullD = g.outFullD ? g.outFullD : g.outD;
-      const uint32_t insideD = fullD - plan->outputPadLoD - plan->outputPadHiD,
-                     insideH = g.outFullH - plan->outputPadLoH -
-                               plan->outputPadHiH,
-                     insideW = g.outFullW - plan->outputPadLoW -
-                               plan->outputPadHiW;
+      const uint32_t fullH = g.outFullH ? g.outFullH : g.outH,
+                     fullW = g.outFullW ? g.outFullW : g.outW;
+      const uint32_t insideD =
+                         fillAll ? 0
+                                 : fullD - plan->outputPadLoD -
+                                       plan->outputPadHiD,
+                     insideH = fillAll ? 0
+                                       : fullH - plan->outputPadLoH -
+                                             plan->outputPadHiH,
+                     insideW = fillAll ? 0
+                                       : fullW - plan->outputPadLoW -
+                                             plan->outputPadHiW;
       const mxconv_status st = hipStatus(
           mxk::launchFillOutputPadding(
-              outType, out, bias, g.batch, fullD, g.outFullH, g.outFullW,
+              outType, out, bias, g.batch, fullD, fullH, fullW,
               plan->outputPadLoD, plan->outputPadLoH, plan->outputPadLoW,
               insideD, insideH, insideW,
               uint32_t(plan->params.getNumOutputChans()), s),
@@ -187,7 +202,9 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
       mxk::IgemmFusedItem items[mxk::kIgemmMaxFused];
       size_t count = 0;
       const size_t elemBytes = plan->params.inputType.size();
-      for (const auto &phase : plan->igemmPhases)
+      for (const auto &phase : plan->igemmPhases) {
+        if (fillAll && phase.d.noTaps)
+          continue;
         items[count++] = {&phase.d,
                           inType,
                           outType,
@@ -197,12 +214,16 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
                           bias,
                           out,
                           q};
+      }
+      if (count == 0)
+        return MXCONV_OK; // (the fill was all there is)
       return hipStatus(mxk::launchIgemmFused(items, count, s),
                        "implicit-GEMM convolution launch (phases)");
     }
     return hipStatus(mxk::launchIgemm(plan->igemm, inType, outType, in, w,
                                       bias, out, workspace, q, s),
                      "implicit-GEMM convolution launch");
+  }
   case mxconv_plan::Kernel::DEPTHWISE:
     return hipStatus(mxk::launchDepthwise(plan->depthwise, inType, outType, in,
                                           w, bias, out, s),
