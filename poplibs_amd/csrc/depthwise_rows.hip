@@ -56,14 +56,18 @@ constexpr uint32_t kNoByte = 0x80000000u;           // beyond any buffer here
 /// column strips and fewer halo columns, lose: pieces of 256 to 640 bytes of
 /// every pixel read by different workgroups - N = 32, 28 x 28, 512 channels
 /// 11.5 -> 12.7 us, N = 128, 14 x 14, 576 channels 12.2 -> 16.8 us.)
-template <int S> struct Ring {
+/// (K: the kernel is K x K, 3 or 5.  At 5 x 5 the 25 taps fill the registers
+/// the window would want, so both strides read their window from LDS; eight
+/// compute waves at stride 1 as for 3 x 3.)
+template <int S, int K = 3> struct Ring {
   static constexpr int kAhead = 6 / S;
-  static constexpr int kEarlyRows = S == 1 ? 1 : 0;
-  static constexpr int kWindow = 3 + kEarlyRows; // rows landed at a barrier
+  static constexpr int kEarlyRows = S == 1 && K == 3 ? 1 : 0;
+  static constexpr int kWindow = K + kEarlyRows; // rows landed at a barrier
   static constexpr int kSlots = kAhead * S + kWindow;
   static constexpr int kComputeWaves = S == 1 ? 8 : 6;
   static constexpr int kComputeThreads = 64 * kComputeWaves;
   static constexpr int kThreads = 64 * (kComputeWaves + kLoaderWaves);
+  static_assert(kSlots * kSlotBytes <= 160 * 1024, "LDS of a CU");
 };
 constexpr uint32_t fwdComputeThreads(uint32_t stride) {
   return stride == 1 ? Ring<1>::kComputeThreads : Ring<2>::kComputeThreads;
@@ -139,11 +143,12 @@ template <int LOADS> struct StripRow {
   }
 };
 
-template <int S, class OutT>
-__global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
+template <int S, int K, class OutT>
+__global__ __launch_bounds__((Ring<S, K>::kThreads)) void depthwiseRowsKernel(
     RowsArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
-  constexpr int kAhead = Ring<S>::kAhead, kSlots = Ring<S>::kSlots;
+  using R = Ring<S, K>;
+  constexpr int kAhead = R::kAhead, kSlots = R::kSlots;
   extern __shared__ __align__(16) char lds[];
   const DepthwiseDesc &d = a.d;
   const uint32_t t = threadIdx.x;
@@ -164,13 +169,13 @@ __global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
   const int ih0 = int(oh0 * S) - d.padH, iw0 = int(ow0 * S) - d.padW;
   const uint32_t pixelBytes = d.channels * 2;
   // relative input rows [0, rowsIn) are what the band reads
-  const uint32_t rowsIn = (steps - 1) * S + 3;
+  const uint32_t rowsIn = (steps - 1) * S + K;
 
-  if (wave >= Ring<S>::kComputeWaves) {
+  if (wave >= R::kComputeWaves) {
     // ---- loaders.  Load L of a row fills bytes [1024 L, 1024 L + 1024) of
     // its slot: 16-byte unit u = 64 L + lane is channel vector u % vecs of
     // strip column u / vecs.  Loader l takes L = l, l + kLoaderWaves, ...
-    const int loader = wave - Ring<S>::kComputeWaves;
+    const int loader = wave - R::kComputeWaves;
     const __amdgpu_buffer_rsrc_t inBuf = bufferOf(in, a.inBytes);
     StripRow<kOwnLoads> strip;
     strip.setup(iw0, a.colsIn, int(d.loW), int(d.hiW), pixelBytes, a.vecs,
@@ -188,7 +193,7 @@ __global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
     };
     // rows of steps 0 .. kAhead - 1
 #pragma unroll 1
-    for (int r = 0; r != (kAhead - 1) * S + Ring<S>::kWindow; ++r)
+    for (int r = 0; r != (kAhead - 1) * S + R::kWindow; ++r)
       loadRow();
     for (uint32_t j = 0; j < steps; ++j) {
       // step j's window has landed when all but the rows of the kAhead - 1
@@ -210,9 +215,9 @@ __global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
   const uint32_t ow = ow0 + col;
   const bool active = col < a.colsOut && ow < d.outW;
   const uint32_t c = (active ? v : 0) * 8;
-  Vec8 taps[9];
+  Vec8 taps[K * K];
 #pragma unroll
-  for (int tap = 0; tap != 9; ++tap)
+  for (int tap = 0; tap != K * K; ++tap)
     taps[tap].raw =
         *reinterpret_cast<const uintx4 *>(w + tap * d.channels + c);
   float biasV[8];
@@ -226,25 +231,27 @@ __global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
   auto rowOf = [&](uint32_t slot) {
     return lds + slot * kSlotBytes + windowByte;
   };
-  auto readRow = [&](Vec8(&row)[3], const char *from) {
+  auto readRow = [&](Vec8(&row)[K], const char *from) {
 #pragma unroll
-    for (int kw = 0; kw != 3; ++kw)
+    for (int kw = 0; kw != K; ++kw)
       row[kw].raw =
           *reinterpret_cast<const uintx4 *>(from + kw * a.vecs * 16);
   };
-  // out row = bias + the nine taps over three window rows, kh then kw
-  auto multiply = [&](const Vec8(&r0)[3], const Vec8(&r1)[3],
-                      const Vec8(&r2)[3]) {
+  // out row = bias + the taps over the window's rows, kh then kw; row kh of
+  // the window is rows[(first + kh) % ROWS]
+  auto multiply = [&](auto &rows, auto firstRow) {
+    constexpr int FIRST = decltype(firstRow)::value;
+    constexpr int ROWS = int(sizeof(rows) / sizeof(rows[0]));
     float acc[8];
 #pragma unroll
     for (int e = 0; e != 8; ++e)
       acc[e] = biasV[e];
 #pragma unroll
-    for (int kh = 0; kh != 3; ++kh)
+    for (int kh = 0; kh != K; ++kh)
 #pragma unroll
-      for (int kw = 0; kw != 3; ++kw) {
-        const Vec8 &x = kh == 0 ? r0[kw] : kh == 1 ? r1[kw] : r2[kw];
-        const Vec8 &k = taps[kh * 3 + kw];
+      for (int kw = 0; kw != K; ++kw) {
+        const Vec8 &x = rows[(FIRST + kh) % ROWS][kw];
+        const Vec8 &k = taps[kh * K + kw];
 #pragma unroll
         for (int e = 0; e != 4; ++e) {
           const float2 xf = __half22float2(x.h2[e]);
@@ -261,21 +268,57 @@ __global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
     return slot + 1 == uint32_t(kSlots) ? 0u : slot + 1;
   };
 
-  if constexpr (Ring<S>::kEarlyRows == 0) {
-    // A step reads its three rows behind its barrier.  (The reads are done -
+  if constexpr (R::kEarlyRows == 0) {
+    // A step reads its K rows behind its barrier.  (The reads are done -
     // their values were used - before the next barrier lets the loaders
     // overwrite the rows.)
     uint32_t slot = 0; // slot of relative row j * S
     for (uint32_t j = 0; j < steps; ++j) {
       stepBarrier(); // step j's rows are in the ring
-      Vec8 win[3][3];
       uint32_t rowSlot = slot;
+      if constexpr (K == 3) {
+        Vec8 win[K][K];
 #pragma unroll
-      for (int kh = 0; kh != 3; ++kh) {
-        readRow(win[kh], rowOf(rowSlot));
-        rowSlot = next(rowSlot);
+        for (int kh = 0; kh != K; ++kh) {
+          readRow(win[kh], rowOf(rowSlot));
+          rowSlot = next(rowSlot);
+        }
+        multiply(win, std::integral_constant<int, 0>{});
+      } else {
+        // (the 25 taps leave no room for the whole window, nor for a second
+        // row to read ahead: a row at a time, the other waves' work under
+        // the reads)
+        // (the taps stay packed halves: as loop constants the compiler
+        // would keep fp32 copies of them, 200 registers)
+#pragma unroll
+        for (int tap = 0; tap != K * K; ++tap)
+          asm volatile("" : "+v"(taps[tap].raw));
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e != 8; ++e)
+          acc[e] = biasV[e];
+#pragma unroll
+        for (int kh = 0; kh != K; ++kh) {
+          Vec8 row[K];
+          readRow(row, rowOf(rowSlot));
+          rowSlot = next(rowSlot);
+#pragma unroll
+          for (int kw = 0; kw != K; ++kw) {
+            const Vec8 &x = row[kw];
+            const Vec8 &k = taps[kh * K + kw];
+#pragma unroll
+            for (int e = 0; e != 4; ++e) {
+              const float2 xf = __half22float2(x.h2[e]);
+              const float2 kf = __half22float2(k.h2[e]);
+              acc[2 * e] = fmaf(xf.x, kf.x, acc[2 * e]);
+              acc[2 * e + 1] = fmaf(xf.y, kf.y, acc[2 * e + 1]);
+            }
+          }
+        }
+        if (active)
+          PutVec<OutT>::put(dst, acc);
+        dst += outRow;
       }
-      multiply(win[0], win[1], win[2]);
       slot += S;
       slot -= slot >= uint32_t(kSlots) ? kSlots : 0;
     }
@@ -285,7 +328,7 @@ __global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
     // adds into the fourth, so every row is read from LDS once and that read
     // hides behind the multiplications.  A row's slot is loaded into again
     // only after the barrier of the step behind the one that used the row.
-    static_assert(S == 1 && Ring<S>::kEarlyRows == 1, "one row per step");
+    static_assert(S == 1 && K == 3 && R::kEarlyRows == 1, "one row per step");
     Vec8 win[4][3];
     uint32_t readSlot = 0; // slot of the next row to read
     auto step = [&](auto off, bool first) {
@@ -300,7 +343,7 @@ __global__ __launch_bounds__(Ring<S>::kThreads) void depthwiseRowsKernel(
       }
       readRow(win[(OFF + 3) % 4], rowOf(readSlot));
       readSlot = next(readSlot);
-      multiply(win[OFF], win[(OFF + 1) % 4], win[(OFF + 2) % 4]);
+      multiply(win, off);
     };
     // the register rows come round every four steps
     for (uint32_t j = 0; j < steps; j += 4) {
@@ -504,7 +547,7 @@ __global__ __launch_bounds__(DeltaRing<S>::kThreads) void depthwiseRowsDeltaKern
 /// when the kernel does not take the layer.
 bool shapeFor(const DepthwiseDesc &d, uint32_t cus, RowsArgs &a,
               uint32_t computeThreads = kComputeThreads) {
-  if (d.kH != 3 || d.kW != 3 || d.dilH != 1 || d.dilW != 1 ||
+  if ((d.kH != 3 && d.kH != 5) || d.kW != d.kH || d.dilH != 1 || d.dilW != 1 ||
       d.strideH != d.strideW || (d.strideH != 1 && d.strideH != 2) ||
       d.channels % 8 != 0 || d.channels == 0 || d.inDilH != 1 ||
       d.inDilW != 1 || d.batch == 0 || d.outH == 0 || d.outW == 0)
@@ -513,15 +556,15 @@ bool shapeFor(const DepthwiseDesc &d, uint32_t cus, RowsArgs &a,
   a.vecs = d.channels / 8;
   // a strip's input row fits a slot, its output row the compute threads
   const uint32_t unitsPerSlot = kSlotBytes / 16;
-  if (a.vecs * 3 > unitsPerSlot || a.vecs > computeThreads)
+  if (a.vecs * d.kW > unitsPerSlot || a.vecs > computeThreads)
     return false;
   const uint32_t maxColsIn = unitsPerSlot / a.vecs;
-  uint32_t maxColsOut = (maxColsIn - 3) / s + 1;
+  uint32_t maxColsOut = (maxColsIn - d.kW) / s + 1;
   if (maxColsOut > computeThreads / a.vecs)
     maxColsOut = computeThreads / a.vecs;
   a.strips = (d.outW + maxColsOut - 1) / maxColsOut;
   a.colsOut = (d.outW + a.strips - 1) / a.strips;
-  a.colsIn = (a.colsOut - 1) * s + 3;
+  a.colsIn = (a.colsOut - 1) * s + d.kW;
   // about one workgroup per CU
   const uint64_t columns = uint64_t(d.batch) * a.strips;
   uint64_t bands = cus / columns;
@@ -534,18 +577,18 @@ bool shapeFor(const DepthwiseDesc &d, uint32_t cus, RowsArgs &a,
   return true;
 }
 
-template <int S, class OutT>
+template <int S, int K, class OutT>
 hipError_t run(const RowsArgs &a, const void *in, const void *w,
                const void *bias, void *out, hipStream_t stream) {
-  constexpr int ldsBytes = Ring<S>::kSlots * kSlotBytes;
+  constexpr int ldsBytes = Ring<S, K>::kSlots * kSlotBytes;
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void *>(&depthwiseRowsKernel<S, OutT>),
+      reinterpret_cast<const void *>(&depthwiseRowsKernel<S, K, OutT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
   if (attr != hipSuccess)
     return attr;
   const uint32_t blocks = a.d.batch * a.strips * a.bands;
-  hipLaunchKernelGGL((depthwiseRowsKernel<S, OutT>), dim3(blocks),
-                     dim3(Ring<S>::kThreads), ldsBytes, stream, a,
+  hipLaunchKernelGGL((depthwiseRowsKernel<S, K, OutT>), dim3(blocks),
+                     dim3(Ring<S, K>::kThreads), ldsBytes, stream, a,
                      static_cast<const __half *>(in),
                      static_cast<const __half *>(w),
                      static_cast<const OutT *>(bias), static_cast<OutT *>(out));
@@ -573,7 +616,8 @@ DepthwiseRowsLaunch launchShapeOf(const DepthwiseDesc &d,
   l.strips = a.strips, l.colsOut = a.colsOut;
   l.bands = a.bands, l.rowsOut = a.rowsOut;
   l.workgroups = uint64_t(d.batch) * a.strips * a.bands;
-  l.ringRows = d.strideH == 2 ? Ring<2>::kSlots : Ring<1>::kSlots;
+  l.ringRows = d.kH == 5 ? (d.strideH == 2 ? Ring<2, 5>::kSlots : Ring<1, 5>::kSlots)
+                         : (d.strideH == 2 ? Ring<2>::kSlots : Ring<1>::kSlots);
   l.loaderWaves = kLoaderWaves;
   l.computeWaves = computeThreads / 64;
   return l;
@@ -602,18 +646,24 @@ hipError_t launchDepthwiseRows(const DepthwiseDesc &d, int inType, int outType,
   a.divVecs = makeFastDiv(a.vecs);
   a.divStrips = makeFastDiv(a.strips);
   a.divBands = makeFastDiv(a.bands);
-  const bool s1 = d.strideH == 1;
+  const bool s1 = d.strideH == 1, k3 = d.kH == 3;
   if (outType == kHalf)
-    return s1 ? run<1, __half>(a, in, weightsPacked, bias, out, stream)
-              : run<2, __half>(a, in, weightsPacked, bias, out, stream);
-  return s1 ? run<1, float>(a, in, weightsPacked, bias, out, stream)
-            : run<2, float>(a, in, weightsPacked, bias, out, stream);
+    return s1 ? (k3 ? run<1, 3, __half>(a, in, weightsPacked, bias, out, stream)
+                    : run<1, 5, __half>(a, in, weightsPacked, bias, out, stream))
+              : (k3 ? run<2, 3, __half>(a, in, weightsPacked, bias, out, stream)
+                    : run<2, 5, __half>(a, in, weightsPacked, bias, out,
+                                        stream));
+  return s1 ? (k3 ? run<1, 3, float>(a, in, weightsPacked, bias, out, stream)
+                  : run<1, 5, float>(a, in, weightsPacked, bias, out, stream))
+            : (k3 ? run<2, 3, float>(a, in, weightsPacked, bias, out, stream)
+                  : run<2, 5, float>(a, in, weightsPacked, bias, out, stream));
 }
 
 bool depthwiseRowsDeltaTakes(const DepthwiseDesc &d) {
   const uint64_t deltaBytes =
       uint64_t(d.batch) * d.outH * d.outW * d.channels * 2;
-  return takes(d, kHalf, deltaComputeThreads(d.strideH)) && deltaBytes < kNoByte;
+  return d.kH == 3 && takes(d, kHalf, deltaComputeThreads(d.strideH)) &&
+         deltaBytes < kNoByte;
 }
 
 DepthwiseRowsLaunch depthwiseRowsDeltaLaunchShape(const DepthwiseDesc &d) {

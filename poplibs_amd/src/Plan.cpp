@@ -921,11 +921,23 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       const bool takes = mxk::depthwiseRowsTakes(d, mxk::kHalf);
       if (pc.rowRing == 1 && !takes)
         throw poplar::invalid_option(
-            "planConstraints gfx950 rowRing: that kernel takes 3x3 taps, "
-            "stride 1 or 2, channels in vectors of 8, at most 2048 to a "
-            "pixel");
-      if (takes && (pc.rowRing == 1 || !d.dense3x3 ||
-                    (l.workgroups * 2 >= gfx950::numCUs && l.rowsOut >= 4)))
+            "planConstraints gfx950 rowRing: that kernel takes 3x3 or 5x5 "
+            "taps, stride 1 or 2, channels in vectors of 8, at most 2048 "
+            "(5x5: 1224) to a pixel");
+      // 5 x 5 taps (25 multiply-adds per output and channel: the vector ALU
+      // shares the bound): strips of four columns or more, and at stride 2
+      // bands of six rows or more - N = 32, 56 x 56, 144 channels, stride 2
+      // 26.0 -> 13.1 us and 14 x 14, 480 channels 14.7 -> 9.3, but 28 x 28,
+      // 240 channels, stride 2 8.1 -> 9.3 and 7 x 7, 1152 channels (strips of
+      // one column) 10.6 -> 12.6.
+      const bool five = d.kH == 5;
+      const bool fiveWorth = (l.colsOut >= 4 || l.strips == 1) &&
+                             (d.strideH == 1 || l.rowsOut >= 6);
+      if (takes &&
+          (pc.rowRing == 1 ||
+           (five ? fiveWorth
+                 : !d.dense3x3 || (l.workgroups * 2 >= gfx950::numCUs &&
+                                   l.rowsOut >= 4))))
         d.dense3x3 = 2;
     } else if (pc.rowRing == 1) {
       throw poplar::invalid_option(

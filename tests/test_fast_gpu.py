@@ -259,6 +259,14 @@ RING = "input rows streamed through an LDS ring"
     # the most the kernel takes: one output column per strip
     dict(batch=2, field=(6, 5), kernel=(3, 3), groups=2048, stride=1, pad=1),
     dict(batch=2, field=(9, 7), kernel=(3, 3), groups=2048, stride=2, pad=1),
+    # 5 x 5 taps: both strides, strips and bands ragged, more padding on one
+    # side than the other, wide pixels
+    dict(batch=9, field=(28, 28), kernel=(5, 5), groups=240, stride=1, pad=2),
+    dict(batch=7, field=(31, 45), kernel=(5, 5), groups=144, stride=2, pad=2),
+    dict(batch=3, field=(14, 14), kernel=(5, 5), groups=672, stride=1,
+         padLower=(2, 1), padUpper=(3, 2)),
+    dict(batch=2, field=(11, 9), kernel=(5, 5), groups=1152, stride=2, pad=2),
+    dict(batch=40, field=(20, 70), kernel=(5, 5), groups=16, stride=1, pad=2),
 ])
 @pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
 def test_depthwise_row_ring_matches_oracle(oracle, kw, out_type):
@@ -301,10 +309,21 @@ def test_depthwise_row_ring_plan_choice():
     assert RING in pa.Plan(wide).describe()
     assert "LDS halo tiles" in pa.Plan(
         wide, {"planConstraints": '{"gfx950": {"rowRing": 0}}'}).describe()
-    # not a 3x3 kernel: the constraint cannot be met
+    # 5 x 5 taps take it too where strips are four columns wide or more (and
+    # at stride 2 bands six rows long)
+    five = dict(batch=32, kernel=(5, 5), pad=2)
+    assert RING in pa.Plan(make_params(
+        pa.HALF, field=(28, 28), groups=240, **five)).describe()
+    assert RING in pa.Plan(make_params(
+        pa.HALF, field=(56, 56), groups=144, stride=2, **five)).describe()
+    assert "LDS halo tiles" in pa.Plan(make_params(
+        pa.HALF, field=(28, 28), groups=240, stride=2, **five)).describe()
+    assert "LDS halo tiles" in pa.Plan(make_params(
+        pa.HALF, field=(7, 7), groups=1152, **five)).describe()
+    # not a 3x3 or 5x5 kernel: the constraint cannot be met
     with pytest.raises(pa.MxconvError):
-        pa.Plan(make_params(pa.HALF, batch=2, field=(20, 20), kernel=(5, 5),
-                            groups=32, pad=2), ROW_RING)
+        pa.Plan(make_params(pa.HALF, batch=2, field=(20, 20), kernel=(7, 7),
+                            groups=32, pad=3), ROW_RING)
 
 
 def test_depthwise_fp32_out_pm1_exact(oracle):

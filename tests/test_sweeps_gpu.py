@@ -176,8 +176,8 @@ def test_weight_deltas_random_dense_layers(oracle):
 
 
 def test_depthwise_row_rings_random_layers(oracle):
-    """The persistent depthwise 3x3 kernels (forward and weight deltas),
-    forced onto random layers: strips and bands of every raggedness."""
+    """The persistent depthwise kernels (forward 3x3 and 5x5, weight deltas
+    3x3), forced onto random layers: strips and bands of every raggedness."""
     from test_weight_update import run_weight_update
     rng = random.Random(20250614)
     options = {"planConstraints": json.dumps({"gfx950": {"rowRing": 1}})}
@@ -185,9 +185,10 @@ def test_depthwise_row_rings_random_layers(oracle):
     for case in range(160):
         s = rng.choice([1, 2])
         lo, hi = _pads(rng, (0, 0), 2)
+        k = 5 if case % 3 == 2 else 3
         kw = dict(batch=rng.randint(1, 9),
                   field=(rng.randint(3, 45), rng.randint(3, 90)),
-                  kernel=(3, 3), ci=1, co=1,
+                  kernel=(k, k), ci=1, co=1,
                   groups=8 * (rng.randint(1, 28) if case % 4
                               else rng.randint(29, 256)),
                   padLower=lo, padUpper=hi, stride=(s, s))
@@ -198,12 +199,14 @@ def test_depthwise_row_rings_random_layers(oracle):
             plan = pa.Plan(p, options)
         except pa.MxconvError:
             continue  # no valid convolution
+        if "depthwise direct" not in plan.describe():
+            continue  # (too small a layer for the depthwise kernels)
         print("case", case, kw, flush=True)
         assert "LDS ring" in plan.describe(), plan.describe()
         _exact(oracle, p, options, 9000 + case)
         fwd += 1
-        if case % 2:
-            continue
+        if case % 2 or k == 5:
+            continue  # (the weight-delta kernel takes 3 x 3 taps)
         r = np.random.default_rng(9500 + case)
         C = p.numConvGroups
         x = r.choice([-1.0, 1.0], (p.batchSize, C, *p.inputFieldShape))
@@ -214,4 +217,4 @@ def test_depthwise_row_rings_random_layers(oracle):
         np.testing.assert_array_equal(
             got, oracle.weight_deltas(p, x, dz, threads=8))
         wu += 1
-    assert fwd >= 100 and wu >= 50, (fwd, wu)
+    assert fwd >= 100 and wu >= 40, (fwd, wu)
