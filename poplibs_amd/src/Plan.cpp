@@ -594,6 +594,15 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       else if (tiles != 0 && tiles * 2 <= gfx950::numCUs && kSteps >= 16)
         parts = std::min<std::size_t>(gfx950::numCUs / tiles, kSteps / 4);
       parts = std::max<std::size_t>(1, std::min(parts, kSteps));
+      // ... where that is estimated to pay for the partial tiles' round trip
+      // and the second kernel: N = 32, 14 x 14, 1 x 1, 1024 -> 256 channels
+      // (98 tiles of 16 k-steps) 16.4 us in two parts, 8.9 us whole; 7 x 7,
+      // 3 x 3, 512 -> 512 (52 tiles of 72 k-steps) 18.7 in four, 21.1 whole.
+      if (!pc.splitK && parts > 1 &&
+          estimateStreaming(tiles, kSteps, 1, g.blockN, 1) <=
+              estimateStreaming(tiles * parts, (kSteps + parts - 1) / parts,
+                                1, g.blockN, unsigned(parts)))
+        parts = 1;
       const std::size_t chans = p.numConvGroups * co;
       // the reduction reads and writes vectors of four channels; partial
       // tiles of more than 1 GB are not worth it

@@ -408,6 +408,14 @@ def test_planner_choices():
     assert "K split into parts         28" in many.describe()
     assert many.buffer_bytes(4) == 28 * 128 * 9 * 128 * 4
     assert "K split" not in pa.Plan(c2).describe()
+    # ... unless the parts' round trip through memory costs more than it
+    # saves: 98 tiles of 16 k-steps stay whole
+    assert "K split" not in pa.Plan(make_params(
+        pa.HALF, batch=32, field=(14, 14), kernel=(1, 1), ci=1024,
+        co=256)).describe()
+    assert "K split into parts         4" in pa.Plan(make_params(
+        pa.HALF, batch=32, field=(7, 7), kernel=(3, 3), ci=512, co=512,
+        pad=1)).describe()
     # one workgroup per CU or fewer: four LDS stages; more workgroups than
     # CUs: two stages, two workgroups per CU
     # (c2 itself goes to the kernel with the input patch resident in LDS)
@@ -528,8 +536,8 @@ def test_plan_estimated_costs():
     assert 17.9 * 0.75 < a / 2100 < 17.9 * 1.25  # 17.9 us measured
     assert 1.7 * a < b < 2.0 * a  # one launch overhead, twice the bytes
     # K split: the fp32 partial tiles are temporary memory
-    deep = pa.Plan(make_params(pa.HALF, batch=8, field=(28, 28),
-                               kernel=(3, 3), ci=128, co=128, pad=1),
+    deep = pa.Plan(make_params(pa.HALF, batch=4, field=(14, 14),
+                               kernel=(3, 3), ci=256, co=256, pad=1),
                    {"planConstraints": '{"gfx950": {"patch": 0}}'})
     assert "K split into parts" in deep.describe()
     cycles, memory = deep.estimated_costs()

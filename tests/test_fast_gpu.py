@@ -551,7 +551,8 @@ SPLIT_K_CASES = [
     (dict(batch=2, field=(9, 7), kernel=(3, 3), ci=64, co=40, pad=1), 9),
     (dict(batch=2, field=(9, 7), kernel=(3, 3), ci=8, co=136, pad=1,
           groups=2), 2),
-    (dict(batch=16, field=(26, 26), kernel=(12, 12), ci=8, co=24, kdil=2,
+    # (72 k-steps: long enough for the parts to pay for their round trip)
+    (dict(batch=16, field=(26, 26), kernel=(12, 12), ci=32, co=24, kdil=2,
           padLower=(1, 1), padUpper=(0, 0)), None),
 ]
 
