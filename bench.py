@@ -335,13 +335,16 @@ def measured_traffic(key):
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     try:
         with open(path) as f:
-            entry = json.load(f).get(key, {})
+            data = json.load(f)
     except (OSError, ValueError):
         return None, None
+    entry = data.get(key, {})
     if "bytes_per_launch" not in entry:
         return None, None
-    return (entry["bytes_per_launch"],
-            entry.get("kernel_sources_sha256") != kernel_sources_hash())
+    # (one stamp for the file: all its entries come from one pass)
+    stamp = entry.get("kernel_sources_sha256",
+                      data.get("kernel_sources_sha256"))
+    return entry["bytes_per_launch"], stamp != kernel_sources_hash()
 
 
 def cpu_model():
