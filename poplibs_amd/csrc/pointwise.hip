@@ -380,12 +380,16 @@ uint64_t walkersFor(uint64_t mTiles, uint64_t pairs, uint32_t ldsBytes,
 /// 256 -> 64 11.65 against 13.1, 512 -> 128 9.4 against 13.9.  One loader wave
 /// does not issue a tile's loads - ten instructions each - as fast as HBM
 /// delivers them; a deeper ring, or 128-pixel tiles where 64 are listed, is
-/// slower.
+/// slower.  512 channels: 64-pixel tiles (four compute waves, one on every
+/// SIMD) in a ring of two, for layers that are as much the matrix cores' as
+/// the memory's - against 32-pixel tiles in a ring of three, N = 32: 28 x 28,
+/// 512 -> 512 21.8 -> 18.5 us, 512 -> 256 13.1 -> 11.3, 7 x 7, 512 -> 2048 8.3 ->
+/// 7.3, 14 x 14, 512 -> 512 8.4 -> 7.6, but 28 x 28, 512 -> 128 8.8 -> 9.1.
 struct PwShape {
   int tm, nb, lw;
 };
 constexpr PwShape kShape64{128, 3, 2}, kShape128{128, 3, 4},
-    kShape256{64, 3, 2}, kShape512{32, 3, 4};
+    kShape256{64, 3, 2}, kShape512{64, 2, 4};
 constexpr PwShape shapeFor(uint32_t ci) {
   return ci == 64 ? kShape64 : ci == 128 ? kShape128 : ci == 256 ? kShape256
                                                                  : kShape512;
