@@ -236,6 +236,18 @@ void mxconv_plan_destroy(mxconv_plan *plan);
 mxconv_status mxconv_plan_describe(const mxconv_plan *plan, char *buffer,
                                    size_t capacity, size_t *needed);
 
+/* getPlanConstraints (lib/poplin/ConvPlan.cpp:1574-1636): the plan as a
+ * complete `planConstraints` JSON document ({"gfx950": {...}}).  Passed back
+ * as that option with the same parameters it reproduces the plan exactly.
+ * The option `planConstraintsOutputFilename`
+ * (include/poplin/Convolution.hpp:191-199) makes mxconv_plan_create and
+ * mxconv_weight_update_plan_create write the same text to
+ * <name>_FWD.json / _BWD.json / _WU.json by the `pass` option, <name>.json
+ * without one (lib/poplin/ConvPlan.cpp:1638-1666, 1764).  Same buffer
+ * protocol as mxconv_plan_describe. */
+mxconv_status mxconv_plan_constraints(const mxconv_plan *plan, char *buffer,
+                                      size_t capacity, size_t *needed);
+
 /* reportPlanEstimatedCosts (include/poplin/Convolution.hpp:590-611,
  * lib/poplin/Convolution.cpp:3923-3936): the planner's estimate for one
  * launch of the plan.  *cycles: shader-clock cycles at 2.1 GHz from the cost

@@ -162,6 +162,8 @@ def lib():
         "mxconv_plan_destroy": (None, [c_void_p]),
         "mxconv_plan_describe": (c_int, [c_void_p, c_char_p, c_size_t,
                                          POINTER(c_size_t)]),
+        "mxconv_plan_constraints": (c_int, [c_void_p, c_char_p, c_size_t,
+                                         POINTER(c_size_t)]),
         "mxconv_plan_buffer_bytes": (c_int, [c_void_p, c_int32,
                                              POINTER(c_size_t)]),
         "mxconv_plan_estimated_costs": (c_int, [c_void_p, POINTER(c_uint64),
@@ -582,6 +584,15 @@ class Plan:
         buf = ctypes.create_string_buffer(need.value)
         _check(lib().mxconv_plan_describe(self._h, buf, need.value,
                                           byref(need)))
+        return buf.value.decode()
+
+    def constraints(self):
+        """The plan as a complete planConstraints JSON document."""
+        need = c_size_t()
+        _check(lib().mxconv_plan_constraints(self._h, None, 0, byref(need)))
+        buf = ctypes.create_string_buffer(need.value)
+        _check(lib().mxconv_plan_constraints(self._h, buf, need.value,
+                                             byref(need)))
         return buf.value.decode()
 
     COST_UNKNOWN = 2 ** 64 - 1

@@ -17,6 +17,7 @@
 #include <cmath>
 #include <cstring>
 #include <new>
+#include <fstream>
 #include <sstream>
 #include <memory>
 #include <mutex>
@@ -539,6 +540,23 @@ mxconv_status mxconv_validate_options(const char *const *keys,
   });
 }
 
+namespace {
+/// The option planConstraintsOutputFilename: the plan just made, dumped as a
+/// complete planConstraints document to <name>_FWD|_BWD|_WU.json
+/// (lib/poplin/ConvPlan.cpp:1638-1666, 1764).
+void writeConstraintsFile(const mxconv_plan &plan,
+                          const poplin::ConvOptions &options) {
+  const std::string path = poplin::getPlanConstraintsOutputFile(options);
+  if (path.empty())
+    return;
+  std::ofstream os(path);
+  os << plan.constraintsJson() << "\n";
+  if (!os.good())
+    throw poputil::poplibs_error("planConstraintsOutputFilename: cannot write '" +
+                                 path + "'");
+}
+} // namespace
+
 mxconv_status mxconv_plan_create(const mxconv_params *p,
                                  const char *const *option_keys,
                                  const char *const *option_values,
@@ -551,6 +569,7 @@ mxconv_status mxconv_plan_create(const mxconv_params *p,
         collectOptions(option_keys, option_values, num_options));
     *plan = new mxconv_plan(
         poplin::makePlan(poplin::ConvParams::fromC(*p), options));
+    writeConstraintsFile(**plan, options);
     return MXCONV_OK;
   });
 }
@@ -564,6 +583,14 @@ mxconv_status mxconv_plan_describe(const mxconv_plan *plan, char *buffer,
     std::ostringstream os;
     os << plan->params << plan->describe();
     return copyOut(os.str(), buffer, capacity, needed);
+  });
+}
+
+mxconv_status mxconv_plan_constraints(const mxconv_plan *plan, char *buffer,
+                                      size_t capacity, size_t *needed) {
+  REQUIRE_ARG(plan);
+  return guarded([&] {
+    return copyOut(plan->constraintsJson(), buffer, capacity, needed);
   });
 }
 
@@ -1477,6 +1504,7 @@ mxconv_status mxconv_weight_update_plan_create(const mxconv_params *fwd,
     *plan = new mxconv_plan(poplin::makePlan(
         poplin::getWeightUpdateParams(poplin::ConvParams::fromC(*fwd)),
         options));
+    writeConstraintsFile(**plan, options);
     return MXCONV_OK;
   });
 }

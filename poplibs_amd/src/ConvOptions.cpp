@@ -206,6 +206,16 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       if (v > 1)
         throw invalid_option("'" + sub + "': Must be 0 or 1");
       pc.rowRing = int(v);
+    } else if (m.first == "pointwise") {
+      const unsigned v = requireUnsigned(sub, m.second);
+      if (v > 1)
+        throw invalid_option("'" + sub + "': Must be 0 or 1");
+      pc.pointwise = int(v);
+    } else if (m.first == "weightDeltas") {
+      const unsigned v = requireUnsigned(sub, m.second);
+      if (v > 1)
+        throw invalid_option("'" + sub + "': Must be 0 or 1");
+      pc.weightDeltas = int(v);
     } else if (m.first == "chanTiles") {
       pc.chanTiles = requireUnsigned(sub, m.second);
       if (pc.chanTiles < 1 || pc.chanTiles > 4)
@@ -305,6 +315,36 @@ bool isFullyConnected(Pass p) {
 }
 
 } // namespace
+
+bool isWeightUpdatePass(Pass p) {
+  return p == Pass::TRAINING_WU || p == Pass::FC_TRAINING_WU;
+}
+
+std::string getPlanConstraintsOutputFile(const ConvOptions &options) {
+  if (options.planConstraintsOutputFilename.empty())
+    return {};
+  std::string path = options.planConstraintsOutputFilename;
+  switch (options.pass) {
+  case Pass::INFERENCE_FWD:
+  case Pass::TRAINING_FWD:
+  case Pass::FC_INFERENCE_FWD:
+  case Pass::FC_TRAINING_FWD:
+    path += "_FWD";
+    break;
+  case Pass::TRAINING_BWD:
+  case Pass::FC_TRAINING_BWD:
+    path += "_BWD";
+    break;
+  case Pass::TRAINING_WU:
+  case Pass::FC_TRAINING_WU:
+    path += "_WU";
+    break;
+  case Pass::NONE:
+  case Pass::NONE_MATMUL:
+    break;
+  }
+  return path + ".json";
+}
 
 ConvOptions getWeightUpdateOptions(ConvOptions fwdOptions) {
   fwdOptions.pass = isFullyConnected(fwdOptions.pass) ? Pass::FC_TRAINING_WU

@@ -53,6 +53,14 @@ struct PlanConstraints {
   /// 64-channel tiles of the output per workgroup of the pointwise streaming
   /// kernel (1 to 4); 0 = planner's choice.
   unsigned chanTiles = 0;
+  /// The pointwise streaming kernel (1x1, unit stride, unpadded): -1
+  /// planner's choice, 0 never, 1 required (an error where it cannot take the
+  /// convolution).
+  int pointwise = -1;
+  /// A weight update pass's deltas: -1 planner's choice, 0 through the pass's
+  /// own convolution (batch and channels exchanged), 1 by the kernel that
+  /// reads the layer's own tensors (an error where none takes the layer).
+  int weightDeltas = -1;
   std::string text; // the JSON as given, kept for reporting and cache keys
 };
 
@@ -80,6 +88,13 @@ public:
 /// fully-connected family if it started there
 /// (lib/poplin/ConvUtilInternal.cpp:941-970).
 ConvOptions getWeightUpdateOptions(ConvOptions fwdOptions);
+/// Whether these are the options of a weight update pass.
+bool isWeightUpdatePass(Pass p);
+/// The file a plan made under `options` dumps its constraints to:
+/// planConstraintsOutputFilename + _FWD / _BWD / _WU by the pass (nothing for
+/// NONE and NONE_MATMUL) + .json (lib/poplin/ConvPlan.cpp:1642-1666); empty
+/// when the option is not set.
+std::string getPlanConstraintsOutputFile(const ConvOptions &options);
 ConvOptions getGradientOptions(ConvOptions fwdOptions);
 
 } // namespace poplin

@@ -70,6 +70,20 @@ std::size_t bufferBytes(const mxconv_plan *plan, mxconv_buffer which) {
   return bytes;
 }
 
+void requirePackedFor(const mxconv_plan *plan, const DeviceTensor &packed,
+                      const char *what) {
+  const auto *packing = static_cast<const PlanHandle *>(packed.packedFor.get());
+  int32_t same = 0;
+  if (packing)
+    check(mxconv_plans_pack_alike(plan, packing->plan, &same));
+  if (!same)
+    throw poputil::poplibs_error(
+        std::string("The ") + what +
+        " were arranged (createWeights, preArrangeMatMulInputRHS) for another "
+        "plan than the one these parameters and options give: pass them in "
+        "the external layout or create them with the same options");
+}
+
 static std::vector<std::size_t> actsShape(std::size_t batch, std::size_t chans,
                                    const std::vector<std::size_t> &field) {
   std::vector<std::size_t> shape{batch, chans};
@@ -272,22 +286,8 @@ void run(const PlanHandle &plan, const ConvParams &params,
     check(mxconv_acts_to_internal(plan.plan, in.data(), inCl.data(),
                                   streamOf(prog)));
   }
-  if (weights.layout() == DeviceTensor::Layout::PackedWeights) {
-    // A packed buffer is only good for plans that pack the same way (kernel,
-    // tile padding, phases ...): another plan would read it wrongly, possibly
-    // beyond its end.  (PopLibs would rearrange such a tensor,
-    // lib/poplin/Convolution.cpp:2569-2628; packing cannot be undone here.)
-    const auto *packing =
-        static_cast<const PlanHandle *>(weights.packedFor.get());
-    int32_t same = 0;
-    if (packing)
-      check(mxconv_plans_pack_alike(plan.plan, packing->plan, &same));
-    if (!same)
-      throw poputil::poplibs_error(
-          "The weights were arranged (createWeights) for another plan than "
-          "the one these parameters and options give: pass them in the "
-          "external layout or create them with the same options");
-  }
+  if (weights.layout() == DeviceTensor::Layout::PackedWeights)
+    requirePackedFor(plan.plan, weights, "weights");
   if (weights.layout() == DeviceTensor::Layout::External) {
     wPacked = DeviceTensor(weights.elementType(), weights.shape(),
                            DeviceTensor::Layout::PackedWeights,

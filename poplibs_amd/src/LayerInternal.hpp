@@ -28,6 +28,14 @@ std::shared_ptr<PlanHandle> getPlan(const ConvParams &params,
                                     const poplar::OptionFlags &options,
                                     PlanningCache *cache);
 std::size_t bufferBytes(const mxconv_plan *plan, mxconv_buffer which);
+/// Throws unless `packed` (a PackedWeights tensor) was arranged for a plan
+/// that packs as `plan` does - same kernel, tiling, padding, operand order.
+/// A buffer of the right size arranged for another kernel would be read in
+/// the wrong operand order.  (PopLibs would rearrange such a tensor,
+/// lib/poplin/Convolution.cpp:2569-2628; packing cannot be undone here.)
+/// `what` names the operand in the message.
+void requirePackedFor(const mxconv_plan *plan, const DeviceTensor &packed,
+                      const char *what);
 mxconv_stream streamOf(const Stream &s);
 
 } // namespace detail

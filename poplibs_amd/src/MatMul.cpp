@@ -96,10 +96,14 @@ void run(const DeviceTensor &A, const DeviceTensor &B, const DeviceTensor &out,
     packed = DeviceTensor(B.elementType(), B.shape(),
                           DeviceTensor::Layout::PackedWeights, packedBytes);
     check(mxconv_matmul_pack_rhs(plan->plan, B.data(), packed.data(), stream));
-  } else if (B.bytes() != packedBytes) {
-    throw poputil::poplibs_error(
-        "The pre-arranged right-hand side was made for another "
-        "multiplication (other shapes, types or options)");
+  } else {
+    // (a size match alone would let a buffer arranged for another kernel
+    // through: several packed layouts share a size)
+    requirePackedFor(plan->plan, B, "right-hand side");
+    if (B.bytes() != packedBytes)
+      throw poputil::poplibs_error(
+          "The pre-arranged right-hand side was made for another "
+          "multiplication (other shapes, types or options)");
   }
   const std::size_t wsBytes = bufferBytes(plan->plan, MXCONV_BUFFER_WORKSPACE);
   DeviceTensor workspace;

@@ -124,6 +124,8 @@ std::vector<DeviceTensor> convolution(const std::vector<ConvolutionArgs> &args,
       weights[i] = flipped;
       temporaries = true;
     }
+    if (weights[i].layout() == DeviceTensor::Layout::PackedWeights)
+      requirePackedFor(plan, weights[i], "weights");
     if (weights[i].layout() == DeviceTensor::Layout::External) {
       DeviceTensor packed(weights[i].elementType(), weights[i].shape(),
                           DeviceTensor::Layout::PackedWeights,

@@ -301,6 +301,7 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   plan.biasElems = params.getNumOutputChans();
   plan.generic = makeGenericDesc(p);
   plan.zeroConv = isZeroConvolution(p);
+  plan.madeForWeightUpdate = isWeightUpdatePass(options.pass);
 
   using Kernel = mxconv_plan::Kernel;
   using Method = PlanConstraints::Method;
@@ -311,8 +312,9 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   // dilation the layer's stride and its stride the layer's kernel dilation.
   {
     const Simple2D w = asSimple2D(p);
-    if (w.ok && !w.hasDepth() && !w.outputPadded() && !w.kernelSelected &&
-        w.batch == 1 &&
+    if (isWeightUpdatePass(options.pass) &&
+        options.planConstraints.weightDeltas != 0 && w.ok && !w.hasDepth() &&
+        !w.outputPadded() && !w.kernelSelected && w.batch == 1 &&
         !plan.zeroConv &&
         !w.inputDilated() && p.batchSize == 1 &&
         p.outputChannelsPerConvGroup == 1 &&
@@ -352,12 +354,15 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   // planConstraints gfx950 kernel names one.)
   {
     const Simple2D w = asSimple2D(p);
-    if (w.ok && !w.hasDepth() && !w.outputPadded() && !w.kernelSelected &&
+    const int asked = options.planConstraints.weightDeltas;
+    if (isWeightUpdatePass(options.pass) && asked != 0 && w.ok &&
+        !w.hasDepth() && !w.outputPadded() && !w.kernelSelected &&
         !plan.zeroConv && !plan.depthwiseWeightUpdate && !w.inputDilated() &&
         w.batch == p.batchSize && w.strideH == 1 && w.strideW == 1 &&
         params.inputType == poplar::HALF &&
-        options.planConstraints.kernel.empty() &&
-        options.planConstraints.method == PlanConstraints::Method::ANY) {
+        (asked == 1 ||
+         (options.planConstraints.kernel.empty() &&
+          options.planConstraints.method == PlanConstraints::Method::ANY))) {
       mxk::WuTapDesc &f = plan.denseForward;
       f.batch = uint32_t(p.inputChannelsPerConvGroup);
       f.inH = w.inH, f.inW = w.inW;
@@ -372,9 +377,23 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       // (enough pixels to be worth the matrix cores: a kernel-sized field
       // of a tiny batch stays with the general path)
       const std::size_t pixels = std::size_t(f.batch) * f.outH * f.outW;
-      plan.denseWeightUpdate = pixels >= 1024 && f.ci >= 16 && f.co >= 16 &&
-                               mxk::wuTapTakes(f);
+      // ... and channels that fill a sixteenth of the kernel's 128 x 128 tile
+      // per (group, tap): a grouped layer of 16 -> 16 channels would run 1/64
+      // of every MFMA on real data and write an fp32 tile a hundred times the
+      // size of its weights.
+      const std::size_t tileArea = std::size_t((f.ci + 127) / 128 * 128) *
+                                   ((f.co + 127) / 128 * 128);
+      const bool worth = pixels >= 1024 && f.ci >= 16 && f.co >= 16 &&
+                         std::size_t(f.ci) * f.co * 16 >= tileArea;
+      plan.denseWeightUpdate = (asked == 1 || worth) && mxk::wuTapTakes(f);
     }
+    if (asked == 1 && isWeightUpdatePass(options.pass) &&
+        !plan.denseWeightUpdate && !plan.depthwiseWeightUpdate)
+      throw poplar::invalid_option(
+          "planConstraints gfx950 weightDeltas: no weight-delta kernel takes "
+          "this layer's own tensors (half inputs, nothing dilated, truncated, "
+          "padded or flipped on the kernel side, channels in whole 16-byte "
+          "vectors)");
   }
   const auto &pc = options.planConstraints;
   const Simple2D s = asSimple2D(p);
@@ -774,7 +793,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         s.hiH == s.inH && s.hiW == s.inW && s.outH == s.inH &&
         s.outW == s.inW;
     plan.pointwiseOn =
-        unitWindow && ciPadded == ci && pc.kernel != "igemm" &&
+        unitWindow && ciPadded == ci &&
+        (pc.kernel != "igemm" || pc.pointwise == 1) && pc.pointwise != 0 &&
         pc.patch < 1 && !pc.blockM &&
         !pc.blockN && !pc.blockK &&
         mxk::pointwiseTakes(pw,
@@ -785,6 +805,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                                                               : mxk::kFloat);
     if (plan.pointwiseOn)
       plan.weightPackedElems = mxk::pointwisePackedElems(pw);
+    else if (pc.pointwise == 1)
+      throw poplar::invalid_option(
+          "planConstraints gfx950 pointwise: that kernel takes 1x1, unit "
+          "stride, unpadded convolutions of 64, 128, 256 or 512 input "
+          "channels per group, with no other tile constraint");
     else if (pc.chanTiles)
       throw poplar::invalid_option(
           "planConstraints gfx950 chanTiles: the pointwise streaming kernel "
@@ -972,6 +997,47 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
 }
 
 } // namespace poplin
+
+std::string mxconv_plan::constraintsJson() const {
+  std::ostringstream os;
+  os << "{\"gfx950\": {";
+  switch (kernel) {
+  case Kernel::GENERIC:
+    os << "\"kernel\": \"generic\"";
+    break;
+  case Kernel::DEPTHWISE:
+    os << "\"kernel\": \"depthwise\", \"rowRing\": "
+       << (depthwise.dense3x3 == 2 ? 1 : 0);
+    // (an explicit tile names the LDS-tiled kernel)
+    if (!depthwise.dense3x3 && depthwise.inDilH == 1 && depthwise.inDilW == 1)
+      os << ", \"tileH\": " << depthwise.tileH << ", \"tileW\": "
+         << depthwise.tileW;
+    break;
+  case Kernel::IGEMM:
+    os << "\"kernel\": \"igemm\"";
+    if (pointwiseOn) {
+      os << ", \"pointwise\": 1, \"chanTiles\": "
+         << mxk::pointwiseLaunchShape(pointwise, gfx950::numCUs).chansPerWorkgroup / 64;
+    } else if (igemm.patch) {
+      os << ", \"pointwise\": 0, \"patch\": " << igemm.patch
+         << ", \"blockM\": " << igemm.blockM;
+    } else {
+      os << ", \"pointwise\": 0, \"patch\": 0, \"blockM\": "
+         << igemm.blockM << ", \"blockN\": " << igemm.blockN
+         << ", \"blockK\": " << igemm.blockK << ", \"splitK\": "
+         << igemm.splitK << ", \"stages\": " << igemm.stages;
+    }
+    break;
+  }
+  if (madeForWeightUpdate) {
+    os << ", \"weightDeltas\": "
+       << (denseWeightUpdate || depthwiseWeightUpdate ? 1 : 0);
+    if (depthwiseWeightUpdate && kernel != Kernel::DEPTHWISE)
+      os << ", \"rowRing\": " << (depthwiseForward.dense3x3 == 2 ? 1 : 0);
+  }
+  os << "}}";
+  return os.str();
+}
 
 double mxconv_plan::estimatedMicroseconds() const {
   // Kernels that stream their tensors once (1x1 with few channels, depthwise,

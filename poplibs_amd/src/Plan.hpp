@@ -54,6 +54,10 @@ struct mxconv_plan {
   // forms the weight deltas straight from the layer's tensors
   // (mxconv_calculate_weight_deltas; the kernel chosen above still serves
   // the parameters as an ordinary convolution).
+  // (Both weight-delta kernels are planned only under a weight update pass's
+  // options, `pass` TRAINING_WU or FC_TRAINING_WU - what
+  // mxconv_weight_update_plan_create sets.)
+  bool madeForWeightUpdate = false;
   bool depthwiseWeightUpdate = false;
   mxk::DepthwiseDesc depthwiseForward{};
   // ... or of a dense layer (any stride): the matrix-core kernel that reads
@@ -110,6 +114,12 @@ struct mxconv_plan {
   std::size_t biasBytes() const { return biasElems * params.outputType.size(); }
 
   std::string describe() const;
+  /// The plan as a complete `planConstraints` document
+  /// ({"gfx950": {...}}): given back as that option with the same
+  /// parameters it reproduces this plan's kernel, tiling, packing and
+  /// workspace exactly, whatever the planner would choose by itself (the
+  /// role of getPlanConstraints, lib/poplin/ConvPlan.cpp:1574-1636).
+  std::string constraintsJson() const;
 
   /// Time one launch of this plan is estimated to take on the device, in
   /// microseconds, by the cost model the tilings were weighed with; negative

@@ -326,6 +326,21 @@ def test_gemm_reference_cases(name, args):
     assert r.returncode == 0, (name, r.stdout[-2000:], r.stderr[-2000:])
 
 
+@pytest.mark.gpu
+def test_gemm_prearranged_for_another_kernel_is_refused():
+    """A right-hand side arranged for the streaming matrix-core kernel has the
+    byte count of one arranged for the 1x1 kernel (k = 256, n = 64) but
+    another operand order: the multiplication must refuse it, not read it."""
+    base = ("--m 4100 --k 256 --n 64 --input-type=half --output-type=float "
+            "--tolerance 0.01 --pre-arrange-rhs=true").split()
+    ok = gemm(*base)
+    assert ok.returncode == 0, (ok.stdout[-2000:], ok.stderr[-2000:])
+    r = gemm(*base, "--pre-arrange-plan-constraints",
+             '{"gfx950":{"kernel":"igemm"}}')
+    assert r.returncode == 1, (r.stdout[-2000:], r.stderr[-2000:])
+    assert "arranged" in r.stderr + r.stdout
+
+
 # ---------------------------------------------------------------------------
 # multi_conv_layer: the reference's cases for its tool of that name
 # (tests/poplin/CMakeLists.txt:4019-4069), --conv arguments from the same JSON

@@ -54,7 +54,10 @@ int main(int argc, char **argv) try {
       "available-memory-proportion", "enable-fast-reduce", "report-plan",
       "show-execution-steps", "show-var-storage", "ipus", "plan-constraints",
       "num-executions", "remap-output-tensor", "plan-constraints-file",
-      "use-create-output", "pre-arrange-rhs", "seed", "timing-runs"};
+      "use-create-output", "pre-arrange-rhs", "seed", "timing-runs",
+      // (this harness's own: arrange the right-hand side under other plan
+      // constraints than the multiplication runs with, which must be refused)
+      "pre-arrange-plan-constraints"};
   for (const auto &kv : opt) {
     bool ok = false;
     for (const char *k : known)
@@ -208,9 +211,13 @@ int main(int argc, char **argv) try {
   // op(A), op(B) as row-major tensors (PopLibs shuffles views; this copies)
   DeviceTensor lhs = transposeA ? transposeGroupedMatrix(matA, prog) : matA;
   DeviceTensor rhs = transposeB ? transposeGroupedMatrix(matB, prog) : matB;
-  if (preArrange)
+  if (preArrange) {
+    poplar::OptionFlags arrangeOpt = mmOpt;
+    if (has("pre-arrange-plan-constraints"))
+      arrangeOpt.set("planConstraints", get("pre-arrange-plan-constraints"));
     rhs = preArrangeMatMulGroupedInputRHS({g, m, k}, rhs, prog, outputType,
-                                          mmOpt, &cache);
+                                          arrangeOpt, &cache);
+  }
 
   // Only the last execution's result is kept, so that repeated accumulation
   // does not saturate it (tools/general_matrix_multiply.cpp:355-372).
