@@ -399,6 +399,11 @@ def main():
                     help="headline workload (c2, c3, c4, c5)")
     ap.add_argument("--only", action="store_true",
                     help="skip the other workloads and the CPU baseline")
+    ap.add_argument("--cache-hot", action="store_true",
+                    help="with --only: also time the HBM-bound workload on "
+                         "one buffer set (tensors in the Infinity Cache); "
+                         "left out by default there, so that a kernel trace "
+                         "of the command averages launches of one kind")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 64 MiB device copy, so that a "
                          "counter run of this command holds a kernel of known "
@@ -436,7 +441,7 @@ def main():
         # ... and, labelled as such, the figure with one buffer set (tensors
         # in the Infinity Cache from the launch before)
         hot = None
-        if sets != 1:
+        if sets != 1 and (args.cache_hot or not args.only):
             _, hot, _, _ = time_steps(torch, probe, steps, warmup)
         if wl["bound"] == "mfma":
             achieved = runner.flops / kernel / 1e12

@@ -250,11 +250,17 @@ mxconv_status mxconv_plan_constraints(const mxconv_plan *plan, char *buffer,
 
 /* reportPlanEstimatedCosts (include/poplin/Convolution.hpp:590-611,
  * lib/poplin/Convolution.cpp:3923-3936): the planner's estimate for one
- * launch of the plan.  *cycles: shader-clock cycles at 2.1 GHz from the cost
- * model the tilings were weighed with, or MXCONV_COST_UNKNOWN where the model
- * does not cover the kernel (the generic one).  *memory_bytes: the temporary
- * device memory of a launch (the workspace).  Touches no GPU. */
+ * launch of the plan.  *cycles: shader-clock cycles from the cost model the
+ * tilings were weighed with, or MXCONV_COST_UNKNOWN where the model does not
+ * cover the kernel (the generic one).  The model is in microseconds (its
+ * constants are measured launch and k-step times); cycles = microseconds x
+ * MXCONV_ESTIMATE_CLOCK_MHZ, the one clock figure used for the conversion:
+ * 2100 MHz, what the chip holds with the matrix cores of 224 of its 256 CUs
+ * busy (2120 MHz measured; 1930 MHz with all 256, 2390 MHz with one).
+ * *memory_bytes: the temporary device memory of a launch (the workspace).
+ * Touches no GPU. */
 #define MXCONV_COST_UNKNOWN UINT64_MAX
+#define MXCONV_ESTIMATE_CLOCK_MHZ 2100
 mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
                                           uint64_t *cycles,
                                           uint64_t *memory_bytes);

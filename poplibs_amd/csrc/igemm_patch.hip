@@ -64,6 +64,29 @@ constexpr int kLdsLimit = 160 * 1024;
 // An offset no buffer the kernel makes reaches: marks padding rows / columns.
 constexpr uint32_t kInvalid = 0x40000000u;
 
+// Cycle stamps of igemmPatch16Kernel's phases, for the build with
+// -DMXK_PATCH_STAMPS only (libmxconv_stamps.so; the product library carries
+// none of this).  Waves 0 and 4 of every workgroup - the older and the younger
+// wave of SIMD 0 - write s_memtime at the marked points, and the wall clock
+// (s_memrealtime, 100 MHz) at both ends, to the buffer
+// mxk_patch_stamp_sink() names: [workgroup][wave 0 | 4][kStampSlots] of 8
+// bytes.
+#ifdef MXK_PATCH_STAMPS
+constexpr int kStampSlots = 16;
+__device__ uint64_t *patchStampSink = nullptr;
+#define MXK_STAMP_DECL uint64_t stamps_[kStampSlots] = {}
+#define MXK_STAMP(i) stamps_[i] = __builtin_amdgcn_s_memtime()
+#define MXK_STAMP_REAL(i) stamps_[i] = __builtin_amdgcn_s_memrealtime()
+#define MXK_STAMP_ARG , stamps_
+#define MXK_STAMP_PARAM , uint64_t *stamps_
+#else
+#define MXK_STAMP_DECL
+#define MXK_STAMP(i)
+#define MXK_STAMP_REAL(i)
+#define MXK_STAMP_ARG
+#define MXK_STAMP_PARAM
+#endif
+
 struct PatchArgs {
   uint32_t M, mTiles, nTiles, groups;
   uint32_t tileM; // output pixels per tile
@@ -136,7 +159,7 @@ template <int WEIGHT_LOADS, int UNITS, class Between, class Behind>
 __device__ __forceinline__ void
 loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
           int lane, uint32_t g, const TileSpan &span, Between &&between,
-          Behind &&behind) {
+          Behind &&behind MXK_STAMP_PARAM) {
   // Patch row `lane`: where its input row starts, from the first image the
   // tile reads (32-bit offsets), or kInvalid for a row of padding.  A load
   // adds the lane's own offset, itself kInvalid for padding columns: any sum
@@ -187,12 +210,15 @@ loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
   // A wave with no block of slice 0 issues its first block of a later slice
   // right away (behind `between`, so that slice 0 gets ahead); the others do
   // so after the barrier.
+  MXK_STAMP(1); // set-up done: the first load of the patch goes out
   const uint32_t blocks = a.slices * a.rowLoads;
   uint32_t next = wave;
   for (; next < a.rowLoads; next += kPatchWaves)
     loadColumns(0, next);
+  MXK_STAMP(2); // slice 0 requested
   const bool early = uint32_t(wave) >= a.rowLoads;
   between();
+  MXK_STAMP(3); // first weights requested, pixel offsets worked out
   if (early) {
     if (next < blocks) {
       const uint32_t s = a.divRowLoads(next);
@@ -203,7 +229,9 @@ loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
     // slice 0 is in LDS once all but the weight loads have landed
     MXK_WAIT_VMCNT(WEIGHT_LOADS);
   }
+  MXK_STAMP(4); // own part of slice 0 landed
   __builtin_amdgcn_s_barrier();
+  MXK_STAMP(5); // everybody's has
   behind();
   for (; next < blocks; next += kPatchWaves) {
     const uint32_t s = a.divRowLoads(next);
@@ -297,6 +325,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
   constexpr int H = RB / 2; // row blocks a wave finishes
   extern __shared__ __align__(16) char lds[];
   using Mma = PatchMma<EB>;
+  MXK_STAMP_DECL; // (only igemmPatch16Kernel writes them out)
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -349,7 +378,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatchKernel(
 #pragma unroll
     for (int i = 0; i != RB; ++i)
       asm volatile("" ::"v"(pixelByte[i]));
-  }, [] {});
+  }, [] {} MXK_STAMP_ARG);
 
   floatx16 acc[RB][kTN];
 #pragma unroll
@@ -658,6 +687,9 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
   extern __shared__ __align__(16) char lds[];
   using Mma = PatchMma16<EB>;
   constexpr int kUnits = Mma::kUnits, kReads = Mma::kReads;
+  MXK_STAMP_DECL;
+  MXK_STAMP_REAL(14);
+  MXK_STAMP(0);
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -732,7 +764,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
 #pragma unroll
     for (int u = kFirst; u != D; ++u)
       loadB(bf[u]);
-  });
+  } MXK_STAMP_ARG);
 
   floatx4 acc[RB][2];
 #pragma unroll
@@ -849,6 +881,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
   // the waits inside it count reads)
   MXK_WAIT_LGKMCNT0();
   readA(even, tapByte);
+  MXK_STAMP(6); // the other slices and weights requested: the k loop begins
   uint32_t j = 0;
   auto group = [&](auto guard) {
     if (j - tableBase == 64) {
@@ -871,6 +904,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
   for (; j + D < own; j += D)
     group(std::false_type{});
   group(std::true_type{});
+  MXK_STAMP(7); // own k-steps done
 
   // Sum the two waves' halves of K: wave grp 0 finishes row blocks
   // [0, kKeep16), wave grp 1 the others; each hands the other its sums of the
@@ -899,6 +933,7 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
     else
       give(std::integral_constant<int, 1>{});
     __syncthreads();
+    MXK_STAMP(8); // both halves' sums handed over
     // the lane's channels of the tile: nLane + 16 c + e, e < 4
     const uint32_t nLane = wn * 32 + (lane >> 4) * 4;
     char *laneOut = tileOut + (lane & 15) * kOutRow + nLane * sizeof(OutT);
@@ -967,8 +1002,22 @@ __global__ __launch_bounds__(kPatchThreads) void igemmPatch16Kernel(
         keep(std::integral_constant<int, 1>{}, std::false_type{});
     }
     __syncthreads();
+    MXK_STAMP(9); // the tile is in LDS
     storeTile<128>(a, tileOut, out, t, g, nTile, span);
   }
+#ifdef MXK_PATCH_STAMPS
+  MXK_STAMP(10); // stores issued
+  __builtin_amdgcn_s_waitcnt(0);
+  MXK_STAMP(11); // ... and landed
+  MXK_STAMP_REAL(15);
+  stamps_[12] = own;
+  if (patchStampSink && (t == 0 || t == kPatchThreads / 2)) {
+    uint64_t *to = patchStampSink +
+                   (size_t(blockIdx.x) * 2 + (t != 0)) * kStampSlots;
+    for (int i = 0; i != kStampSlots; ++i)
+      to[i] = stamps_[i];
+  }
+#endif
 }
 
 /// One element of the packed weights per thread:
@@ -1321,3 +1370,12 @@ hipError_t launchIgemmPatch(const IgemmDesc &d, int inType, int outType,
 }
 
 } // namespace mxk
+
+#ifdef MXK_PATCH_STAMPS
+/// Stamps build only: the device buffer the stamped kernel writes to
+/// ([workgroups][2][16] of 8 bytes), or null to switch the stamps off.
+extern "C" int mxk_patch_stamp_sink(void *deviceBuffer) {
+  return int(hipMemcpyToSymbol(HIP_SYMBOL(mxk::patchStampSink), &deviceBuffer,
+                               sizeof(deviceBuffer)));
+}
+#endif

@@ -195,6 +195,10 @@ struct PlanCosts {
   std::size_t memory;
   constexpr static std::size_t unknown =
       std::numeric_limits<std::size_t>::max();
+  /// (This build's addition.)  The cost model works in microseconds; `cycles`
+  /// is that time at this shader clock (MXCONV_ESTIMATE_CLOCK_MHZ), so
+  /// cycles / clockMHz gives the microseconds back.
+  constexpr static double clockMHz = 2100.0;
 };
 
 /// include/poplin/Convolution.hpp:608-611 of PopLibs.

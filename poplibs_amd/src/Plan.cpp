@@ -377,14 +377,19 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       // (enough pixels to be worth the matrix cores: a kernel-sized field
       // of a tiny batch stays with the general path)
       const std::size_t pixels = std::size_t(f.batch) * f.outH * f.outW;
-      // ... and channels that fill a sixteenth of the kernel's 128 x 128 tile
-      // per (group, tap): a grouped layer of 16 -> 16 channels would run 1/64
-      // of every MFMA on real data and write an fp32 tile a hundred times the
-      // size of its weights.
+      // ... and, in a grouped layer, channels that fill a quarter of the
+      // kernel's 128 x 128 tile per (group, tap): every group brings its own
+      // tiles, and poorly filled ones lose to the pass's own convolution
+      // (N = 32, 28 x 28, 3 x 3: 32 groups of 16 -> 16 channels 420 against
+      // 117 us, 8 groups of 32 -> 32 78 against 49, 2 groups of 64 -> 64 26
+      // against 26.5; without groups 16 -> 16 on 56 x 56 ties at 39 us and
+      // 32 -> 64 wins with 18 against 25).
       const std::size_t tileArea = std::size_t((f.ci + 127) / 128 * 128) *
                                    ((f.co + 127) / 128 * 128);
-      const bool worth = pixels >= 1024 && f.ci >= 16 && f.co >= 16 &&
-                         std::size_t(f.ci) * f.co * 16 >= tileArea;
+      const bool filled =
+          f.groups == 1 || std::size_t(f.ci) * f.co * 4 >= tileArea;
+      const bool worth =
+          pixels >= 1024 && f.ci >= 16 && f.co >= 16 && filled;
       plan.denseWeightUpdate = (asked == 1 || worth) && mxk::wuTapTakes(f);
     }
     if (asked == 1 && isWeightUpdatePass(options.pass) &&
@@ -1049,6 +1054,26 @@ double mxconv_plan::estimatedMicroseconds() const {
   };
   if (zeroConv)
     return streamed(outputBytes());
+  // A weight update pass that runs on the layer's own tensors: what those
+  // kernels were measured at.  Matrix-core kernel + ordered sum, two
+  // launches, about 350 TFLOP/s of the dense count while the loop waits for
+  // its loads (N = 32, 28 x 28, 128 -> 128, 3 x 3: 24.5 us); depthwise rows +
+  // the sum of the workgroups' tiles (4.5 us) behind one pass over both
+  // tensors (N = 32, 112 x 112, 96 channels, stride 2: 20.4 us).
+  if (denseWeightUpdate) {
+    const auto &f = denseForward;
+    const double flops = 2.0 * f.batch * f.outH * f.outW * f.groups * f.ci *
+                         f.co * f.kH * f.kW;
+    return 2 * poplin::kLaunchUs + flops / 3.5e8;
+  }
+  if (depthwiseWeightUpdate) {
+    const auto &f = depthwiseForward;
+    const std::size_t bytes =
+        (std::size_t(f.batch) * f.inH * f.inW + std::size_t(f.batch) * f.outH *
+                                                     f.outW) *
+        f.channels * 2;
+    return streamed(bytes) + 4.5;
+  }
   double us = 0;
   switch (kernel) {
   case Kernel::GENERIC:

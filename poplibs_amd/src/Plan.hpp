@@ -6,6 +6,7 @@
 #ifndef poplibs_amd_Plan_hpp
 #define poplibs_amd_Plan_hpp
 #include "ConvOptions.hpp"
+#include "mxconv.h"
 #include "kernels.hpp"
 #include "poplin/ConvParams.hpp"
 #include <cstddef>
@@ -127,9 +128,10 @@ struct mxconv_plan {
   /// estimateConvCost behind reportPlanEstimatedCosts
   /// (lib/poplin/Convolution.cpp:3923-3936).
   double estimatedMicroseconds() const;
-  /// The shader clock the estimate is converted to cycles with: what the chip
-  /// holds with the matrix cores of most CUs busy.
-  static constexpr double kEstimateClockMHz = 2100.0;
+  /// The shader clock the estimate is converted to cycles with
+  /// (MXCONV_ESTIMATE_CLOCK_MHZ): what the chip holds with the matrix cores
+  /// of most CUs busy.
+  static constexpr double kEstimateClockMHz = MXCONV_ESTIMATE_CLOCK_MHZ;
 };
 
 namespace poplin {

@@ -417,16 +417,25 @@ def test_quarter_small_integer_data_is_exact(oracle):
 # ---- benchmark configurations at full size ---------------------------------
 
 def _full_size(oracle, p, seed, tol, kernel, act_fn=None, w_std=1.0,
-               images=8):
+               images=8, recipe=False):
+    """recipe: the benchmark's seeded inputs (poplibs_amd.synthetic:
+    mt19937_64(seed) for the activations, seed + 1 for the weights, Box-Muller
+    normals in the order of the external arrays) instead of numpy's
+    generator, so that the test sees the very tensors bench.py times."""
     from gpu_helpers import quantize, run_conv
-    g = np.random.default_rng(seed)
-    acts = g.standard_normal((p.batchSize, p.getNumInputChans(),
-                              *p.inputFieldShape))
+    ashape = (p.batchSize, p.getNumInputChans(), *p.inputFieldShape)
+    wshape = (p.numConvGroups, p.outputChannelsPerConvGroup,
+              p.inputChannelsPerConvGroup, *p.kernelShape)
+    if recipe:
+        from poplibs_amd import synthetic
+        acts = synthetic.normal(seed, ashape)
+        weights = synthetic.normal(seed + 1, wshape, w_std)
+    else:
+        g = np.random.default_rng(seed)
+        acts = g.standard_normal(ashape)
+        weights = g.standard_normal(wshape) * w_std
     if act_fn:
         acts = act_fn(acts)
-    weights = g.standard_normal(
-        (p.numConvGroups, p.outputChannelsPerConvGroup,
-         p.inputChannelsPerConvGroup, *p.kernelShape)) * w_std
     aq, ad = quantize(acts, p.inputType)
     wq, wd = quantize(weights, p.inputType)
     got, plan = run_conv(p, aq, wq, None, None, return_plan=True)
@@ -499,6 +508,59 @@ def test_baseline_config5_full(oracle):
     for i, b in enumerate(picked):
         # against the dequantised inputs only accumulation and the fp16
         # output round: well inside the 3e-2 fp8 budget
+        err = rel_l2(got[b], want[i])
+        assert err <= 3e-2 and err <= 1e-3, (b, err)
+
+
+# The same four configurations on the benchmark's own seeded inputs (the
+# recipe of poplibs_amd/synthetic.py that bench.py draws from, seed 0 for the
+# activations and 1 for the weights): tests and benchmark see identical data.
+
+def test_baseline_config2_recipe_inputs(oracle):
+    p = make_params(pa.HALF, batch=32, field=(28, 28), kernel=(3, 3), ci=128,
+                    co=128, pad=1)
+    _full_size(oracle, p, 0, 1e-3, "implicit GEMM",
+               w_std=(2 / (9 * 128)) ** .5, recipe=True)
+
+
+def test_baseline_config3_recipe_inputs(oracle):
+    p = make_params(pa.HALF, batch=32, field=(56, 56), kernel=(1, 1), ci=256,
+                    co=64)
+    _full_size(oracle, p, 0, 1e-3, "implicit GEMM",
+               act_fn=lambda x: np.maximum(x, 0), w_std=(2 / 256) ** .5,
+               recipe=True)
+
+
+def test_baseline_config4_recipe_inputs(oracle):
+    p = make_params(pa.HALF, batch=32, field=(112, 112), kernel=(3, 3),
+                    groups=96, stride=2, pad=1)
+    _full_size(oracle, p, 0, 1e-3, "depthwise direct", w_std=(2 / 9) ** .5,
+               recipe=True)
+
+
+def test_baseline_config5_recipe_inputs(oracle):
+    """configs[4] as bench.py prepares it: normals from the recipe, per-tensor
+    power-of-two scales e = ceil(log2(max|x| / 448)), values / 2^e rounded to
+    E4M3; eight images against the oracle on the dequantised values."""
+    from gpu_helpers import quantize, run_conv
+    from poplibs_amd import synthetic
+    p = make_params(pa.QUARTER, pa.HALF, batch=64, field=(14, 14),
+                    kernel=(3, 3), ci=256, co=256, pad=1)
+    acts = synthetic.normal(0, (64, 256, 14, 14))
+    weights = synthetic.normal(1, (1, 256, 256, 3, 3), (2 / (9 * 256)) ** .5)
+    sa = int(np.ceil(np.log2(np.abs(acts).max() / 448.0)))
+    sw = int(np.ceil(np.log2(np.abs(weights).max() / 448.0)))
+    aq, ad = quantize(acts, pa.QUARTER, oracle, 1, sa)
+    wq, wd = quantize(weights, pa.QUARTER, oracle, 1, sw)
+    got, plan = run_conv(p, aq, wq, None, None,
+                         in_meta=pa.quarter_metadata(1, sa),
+                         w_meta=pa.quarter_metadata(1, sw), return_plan=True)
+    assert _plan_kernel(plan) == "implicit GEMM"
+    picked = [0, 9, 18, 27, 36, 45, 54, 63]
+    some = pa.ConvParams.from_c(p.to_c())
+    some.batchSize = len(picked)
+    want = oracle.convolution(some, ad[picked], wd, threads=8)
+    for i, b in enumerate(picked):
         err = rel_l2(got[b], want[i])
         assert err <= 3e-2 and err <= 1e-3, (b, err)
 

@@ -326,6 +326,116 @@ def test_gemm_reference_cases(name, args):
     assert r.returncode == 0, (name, r.stdout[-2000:], r.stderr[-2000:])
 
 
+C2_ARGS = ("--input-channels 128 --output-channels 128 --field {28,28} "
+           "--kernel-size 3 --padding 1 --batch-size 32 --data-type half "
+           "--bias 0").split()
+
+
+@pytest.mark.gpu
+def test_test_planner_compares_estimates_with_measurements():
+    """--test-planner (tools/single_conv_layer.cpp:183, 857-888, 1490-1520):
+    every pass's planner estimate against the time between two HIP events;
+    within the stated factor on the benchmark's 3x3 layer, and a failure
+    when the tolerance is made impossible."""
+    r = run(*C2_ARGS, "--test-planner", timeout=300)
+    assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-3000:])
+    import re
+    rows = dict((m[0], (float(m[1]), float(m[2]))) for m in re.findall(
+        r"^  (fwd|bwd|wu): estimated ([0-9.]+) us, measured ([0-9.]+) us",
+        r.stdout, re.M))
+    assert set(rows) == {"fwd", "bwd", "wu"}, r.stdout
+    for est, measured in rows.values():
+        assert measured <= 2.5 * est + 15 and est <= 2.5 * measured + 15
+    bad = run(*C2_ARGS, "--test-planner", "--test-planner-tolerance", "0.001",
+              "--single-phase", "wu", timeout=300)
+    assert bad.returncode == 1 and "beyond the tolerance" in bad.stdout
+
+
+@pytest.mark.gpu
+def test_tensor_files_chain_two_layers(tmp_path):
+    """--fwd-out-file of one run is --fwd-in-file of the next, whose batch
+    size, field and type come from the file
+    (tools/single_conv_layer.cpp:418-429, 593-626, 1376-1382)."""
+    first = str(tmp_path / "layer1.bin")
+    r = run("--input-channels", "16", "--output-channels", "32", "--field",
+            "{12,10}", "--kernel-size", "3", "--padding", "1", "--batch-size",
+            "3", "--data-type", "half", "--single-phase", "fwd",
+            "--fwd-out-file", first)
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-2000:])
+    assert "Saving FWD tensor with shape:[3,32,12,10]" in r.stdout
+    second = str(tmp_path / "layer2.bin")
+    r = run("--input-channels", "32", "--output-channels", "8",
+            "--kernel-size", "{1,3}", "--single-phase", "fwd",
+            "--fwd-in-file", first, "--fwd-out-file", second,
+            "--tolerance", "0.02")
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-2000:])
+    assert "Importing FWD input from file, shape:[3,32,12,10]" in r.stdout
+    assert "Saving FWD tensor with shape:[3,8,12,8]" in r.stdout
+    # the options the file replaces may not be given beside it
+    r = run("--input-channels", "32", "--output-channels", "8", "--field",
+            "{12,10}", "--fwd-in-file", first)
+    assert r.returncode == 1 and "Cannot specify --field" in r.stderr
+    r = run("--input-channels", "31", "--output-channels", "8",
+            "--fwd-in-file", first)
+    assert r.returncode == 1 and "dimension 1" in r.stderr
+    r = run("--input-channels", "32", "--output-channels", "8",
+            "--fwd-in-file", str(tmp_path / "missing.bin"))
+    assert r.returncode == 1 and "could not be opened" in r.stderr
+    # the backward pass's input and output likewise
+    grads = str(tmp_path / "grads.bin")
+    r = run("--input-channels", "8", "--output-channels", "32", "--field",
+            "{12,10}", "--kernel-size", "3", "--padding", "1", "--batch-size",
+            "3", "--single-phase", "bwd", "--bwd-in-file", first,
+            "--bwd-out-file", grads, "--tolerance", "0.05")
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-2000:])
+    assert "Importing BWD input from file, shape:[3,32,12,10]" in r.stdout
+    assert "Saving BWD tensor with shape:[3,8,12,10]" in r.stdout
+
+
+@pytest.mark.gpu
+def test_create_output_and_generic_input_layout():
+    """--use-create-output=true (tools/single_conv_layer.cpp:407) and
+    --use-create-input=false (an input in the plan-independent layout)."""
+    for extra in (["--use-create-output=true"], ["--use-create-input=false"],
+                  ["--use-create-output=true", "--use-create-input=false",
+                   "--single-phase=all"]):
+        r = run("--input-channels", "64", "--output-channels", "64", "--field",
+                "{14,14}", "--kernel-size", "3", "--padding", "1",
+                "--batch-size", "4", *extra)
+        assert r.returncode == 0, (extra, r.stdout[-2000:], r.stderr[-2000:])
+        assert "Validation passed" in r.stdout
+
+
+@pytest.mark.gpu
+def test_backward_fp8_metadata_and_per_pass_constraint_files(tmp_path):
+    """--fp8-format-bwd / --fp8-scale-bwd describe the backward pass's input;
+    --bwd-plan-constraints-file / --wu-plan-constraints-file give a pass its
+    own constraints."""
+    base = ["--input-channels", "32", "--output-channels", "32", "--field",
+            "{10,10}", "--kernel-size", "3", "--padding", "1", "--batch-size",
+            "2", "--input-type", "quarter", "--output-type", "half"]
+    for fmt, scale in (("quart143", "-1"), ("quart152", "3")):
+        r = run(*base, "--single-phase", "bwd", "--fp8-format-bwd", fmt,
+                "--fp8-scale-bwd", scale)
+        assert r.returncode == 0, (fmt, r.stdout[-2000:], r.stderr[-2000:])
+    assert run(*base, "--fp8-format-bwd", "quart8").returncode == 1
+    generic = tmp_path / "generic.json"
+    generic.write_text('{"gfx950": {"kernel": "generic"}}')
+    half = ["--input-channels", "32", "--output-channels", "32", "--field",
+            "{10,10}", "--kernel-size", "3", "--padding", "1", "--batch-size",
+            "2", "--report-plan", "1"]
+    r = run(*half, "--bwd-plan-constraints-file", str(generic),
+            "--wu-plan-constraints-file", str(generic))
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-2000:])
+    fwd, rest = r.stdout.split("Backward plan:")
+    bwd, wu = rest.split("WU plan:")
+    assert "implicit GEMM" in fwd and "generic direct" not in fwd
+    assert "generic direct" in bwd and "generic direct" in wu
+    r = run(*half, "--bwd-plan-constraints-file", str(generic),
+            "--bwd-plan-constraints", '{"gfx950": {"kernel": "igemm"}}')
+    assert r.returncode == 1 and "Both bwd-plan-constraints" in r.stderr
+
+
 @pytest.mark.gpu
 def test_gemm_prearranged_for_another_kernel_is_refused():
     """A right-hand side arranged for the streaming matrix-core kernel has the

@@ -15,6 +15,24 @@
 //   * element-wise checkIsClose (lib/poplibs_test/Util.cpp:198-217, 316-348)
 //   * exit 0 = match, 1 = mismatch or bad usage, 77 = out of device memory
 //     (tools/single_conv_layer.cpp:1531-1537).
+// Options that only steer the IPU build of the graph (--tiles-per-ipu, --ipus,
+// --input-load-width, --workers-per-tile, --remap-output-tensor,
+// --enable-convolution-reuse, --report-var-storage, --profile, --profile-dir,
+// the --test-planner-report-* family) are accepted and have no effect here.
+// --test-planner compares the planner's estimate of every pass that ran with
+// the time measured between two HIP events (reportPlanEstimatedCosts against
+// the clock; tools/single_conv_layer.cpp:183, 857-888, 1490-1520 compare the
+// IPU planner's estimates with a profile): the case fails when they differ
+// by more than the factor --test-planner-tolerance (default 2.5) beyond 15 us
+// of launch overhead.  --fwd-in-file / --fwd-out-file / --bwd-in-file /
+// --bwd-out-file read and write a tensor in this harness's own container
+// (magic "MXT1", element type, rank, dimensions, raw values in the external
+// layout); Poplar's own binary tensor format is part of the closed SDK.
+//
+//   single_conv_layer --batch-file cases.json
+// runs many invocations in one process (one HIP start-up for all):
+// cases.json is [{"name": ..., "args": [...]}, ...]; every case prints
+// "### CASE <name>", its output and "### RESULT <name> <exit code>".
 #include "poplar/OptionFlags.hpp"
 #include "poplar/exceptions.hpp"
 #include "poplin/ConvParams.hpp"
@@ -25,6 +43,10 @@
 
 #include "../../poplibs_amd/src/Json.hpp"
 #include "harness_util.hpp"
+
+#include "mxconv.h"
+#define __HIP_PLATFORM_AMD__ 1
+#include <hip/hip_runtime_api.h>
 
 #include <chrono>
 #include <cmath>
@@ -80,13 +102,12 @@ namespace {
 
 using poplin::ConvParams;
 
+struct UsageError : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
 [[noreturn]] void usage(const std::string &message) {
-  std::cerr << "error: " << message << "\n"
-            << "usage: single_conv_layer --input-channels N --output-channels "
-               "N --field {H,W} --kernel-size {h,w} [options]\n"
-               "  see the header of tests/tools/single_conv_layer.cpp for the "
-               "option list\n";
-  std::exit(1);
+  throw UsageError(message);
 }
 
 /// "{1,2,3}" gives one value per dimension; a bare "2" is broadcast
@@ -128,7 +149,80 @@ template <class T> std::vector<T> expand(const Shape &s, size_t n, T dflt) {
 
 } // namespace
 
-int main(int argc, char **argv) try {
+/// The harness's own tensor container: "MXT1", element type id (0 float,
+/// 1 half, 2 quarter), rank, dimensions (uint64), then the raw values in the
+/// external layout.
+void saveTensor(const std::string &path, poplar::Type type,
+                const std::vector<size_t> &shape,
+                const std::vector<uint8_t> &bytes) {
+  std::ofstream f(path, std::ios::binary);
+  if (!f.good())
+    throw poputil::poplibs_error("file " + path + " could not be opened");
+  const uint32_t id = type == poplar::FLOAT ? 0 : type == poplar::HALF ? 1 : 2;
+  const uint32_t rank = uint32_t(shape.size());
+  f.write("MXT1", 4);
+  f.write(reinterpret_cast<const char *>(&id), 4);
+  f.write(reinterpret_cast<const char *>(&rank), 4);
+  for (size_t d : shape) {
+    const uint64_t v = d;
+    f.write(reinterpret_cast<const char *>(&v), 8);
+  }
+  f.write(reinterpret_cast<const char *>(bytes.data()),
+          std::streamsize(bytes.size()));
+}
+
+struct LoadedTensor {
+  poplar::Type type = poplar::HALF;
+  std::vector<size_t> shape;
+  std::vector<uint8_t> bytes;
+};
+
+LoadedTensor loadTensor(const std::string &what, const std::string &path) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f.good())
+    throw poputil::poplibs_error("<" + what + "> file " + path +
+                                 " could not be opened");
+  char magic[4];
+  uint32_t id = 0, rank = 0;
+  f.read(magic, 4);
+  f.read(reinterpret_cast<char *>(&id), 4);
+  f.read(reinterpret_cast<char *>(&rank), 4);
+  if (!f.good() || std::memcmp(magic, "MXT1", 4) != 0 || id > 2 || rank > 8)
+    throw poputil::poplibs_error("No Tensors in " + what);
+  LoadedTensor t;
+  t.type = id == 0 ? poplar::FLOAT : id == 1 ? poplar::HALF : poplar::QUARTER;
+  size_t elems = 1;
+  for (uint32_t d = 0; d != rank; ++d) {
+    uint64_t v = 0;
+    f.read(reinterpret_cast<char *>(&v), 8);
+    t.shape.push_back(size_t(v));
+    elems *= size_t(v);
+  }
+  t.bytes.resize(elems * t.type.size());
+  f.read(reinterpret_cast<char *>(t.bytes.data()),
+         std::streamsize(t.bytes.size()));
+  if (!f.good() && !t.bytes.empty())
+    throw poputil::poplibs_error("file " + path + " is truncated");
+  return t;
+}
+
+std::string shapeText(const std::vector<size_t> &shape) {
+  std::string s = "[";
+  for (size_t i = 0; i != shape.size(); ++i)
+    s += (i ? "," : "") + std::to_string(shape[i]);
+  return s + "]";
+}
+
+std::string readFile(const std::string &path) {
+  std::ifstream f(path);
+  if (!f)
+    usage("cannot read '" + path + "'");
+  std::stringstream ss;
+  ss << f.rdbuf();
+  return ss.str();
+}
+
+int runCase(int argc, char **argv) try {
   std::map<std::string, std::string> opt = parseCommandLine(argc, argv);
   static const char *known[] = {
       "help", "input-channels", "output-channels", "field", "kernel-size",
@@ -148,7 +242,18 @@ int main(int argc, char **argv) try {
       "fwd-plan-constraints-file", "report-plan", "convolution-options",
       "preplan",
       "use-create-input", "num-determinism-checks", "ignore-data", "seed",
-      "device-type", "profile", "timing-runs"};
+      "device-type", "profile", "timing-runs",
+      "use-create-output", "fp8-scale-bwd", "fp8-format-bwd",
+      "bwd-plan-constraints-file", "wu-plan-constraints-file", "fwd-in-file",
+      "fwd-out-file", "bwd-in-file", "bwd-out-file", "test-planner",
+      "test-planner-tolerance", "compile-only",
+      // steer the IPU graph only: accepted, no effect
+      "tiles-per-ipu", "ipus", "input-load-width", "workers-per-tile",
+      "remap-output-tensor", "enable-convolution-reuse", "report-var-storage",
+      "profile-dir", "test-planner-existing-profile",
+      "test-planner-simulated-execution-file", "test-planner-report-all-tiles",
+      "test-planner-report-all-serial-splits", "test-planner-report-verbose",
+      "test-planner-print-vars"};
   for (const auto &kv : opt) {
     bool ok = false;
     for (const char *k : known)
@@ -162,10 +267,22 @@ int main(int argc, char **argv) try {
   };
   if (has("help"))
     usage("help requested");
-  for (const char *required :
-       {"input-channels", "output-channels", "field", "kernel-size"})
+  for (const char *required : {"input-channels", "output-channels"})
     if (!has(required))
       usage(std::string("the option '--") + required + "' is required");
+  // (tools/single_conv_layer.cpp:450-463)
+  if (has("fwd-in-file") || has("bwd-in-file")) {
+    if (has("fwd-in-file") &&
+        (has("field") || has("input-type") || has("batch-size"))) {
+      std::cerr << "Cannot specify --field, --batch-size or --input-type with "
+                   "an input file\n";
+      return 1;
+    }
+  }
+  if (!has("field") && !has("fwd-in-file")) {
+    std::cerr << "Must use an input file or specify --field\n";
+    return 1;
+  }
   // Passes (tools/single_conv_layer.cpp:715-735).
   const std::string phase = get("single-phase", "all");
   if (phase != "fwd" && phase != "bwd" && phase != "wu" && phase != "all")
@@ -176,18 +293,48 @@ int main(int argc, char **argv) try {
   bool doWuPass = !inferenceOnly && (phase == "wu" || phase == "all");
 
   // ---- parameters (tools/single_conv_layer.cpp:768-790) -------------------
-  const Shape field = parseShape(get("field"));
-  if (field.broadcast)
-    usage("--field needs one size per dimension, e.g. {32,32}");
-  const size_t n = field.values.size();
-  const auto fieldShape = expand<size_t>(field, n, 1);
-  const auto kernelShape = expand<size_t>(parseShape(get("kernel-size")), n, 1);
   poplar::Type inputType = parseType(get("data-type", "half"));
   poplar::Type outputType = inputType;
   if (has("input-type"))
     inputType = parseType(get("input-type"));
   if (has("output-type"))
     outputType = parseType(get("output-type"));
+  size_t batchSize = std::stoul(get("batch-size", "1"));
+  Shape field = has("field") ? parseShape(get("field")) : Shape{};
+  // The forward input from a file: its type, batch size and field replace the
+  // options' (tools/single_conv_layer.cpp:593-626).
+  LoadedTensor fwdIn, bwdIn;
+  if (has("fwd-in-file")) {
+    fwdIn = loadTensor("fwd-in-file", get("fwd-in-file"));
+    std::cout << "Importing FWD input from file, shape:"
+              << shapeText(fwdIn.shape)
+              << " Element type:" << fwdIn.type.toString() << "\n";
+    if (fwdIn.shape.size() < 2)
+      throw poputil::poplibs_error("No Tensors in fwd-in-file");
+    if (!has("output-type") && outputType == inputType)
+      outputType = fwdIn.type == poplar::QUARTER ? poplar::HALF : fwdIn.type;
+    inputType = fwdIn.type;
+    batchSize = fwdIn.shape[0];
+    if (fwdIn.shape[1] != std::stoul(get("input-channels")) *
+                              std::stoul(get("conv-groups", "1"))) {
+      std::cerr << "The product of conv-groups and input-channels must be "
+                   "equal to dimension 1 of the FWD input file tensor, which "
+                   "is "
+                << fwdIn.shape[1] << "\n";
+      return 1;
+    }
+    field = Shape{};
+    for (size_t d = 2; d != fwdIn.shape.size(); ++d)
+      field.values.push_back(long(fwdIn.shape[d]));
+  }
+  // (a bare number is a one-dimensional field:
+  // tools/single_conv_layer.cpp:653-654 takes the rank from the values given)
+  field.broadcast = false;
+  const size_t n = field.values.size();
+  const auto fieldShape = expand<size_t>(field, n, 1);
+  // (--kernel-size defaults to 1, tools/single_conv_layer.cpp:208-212)
+  const auto kernelShape = expand<size_t>(
+      has("kernel-size") ? parseShape(get("kernel-size")) : Shape{}, n, 1);
   auto both = [&](const char *base, const char *suffix) {
     const std::string specific = std::string(base) + suffix;
     return has(specific.c_str()) ? parseShape(opt[specific])
@@ -223,7 +370,7 @@ int main(int argc, char **argv) try {
       expand<unsigned>(both("output-padding", "-lower"), n, 0),
       expand<unsigned>(both("output-padding", "-upper"), n, 0));
   const ConvParams params(
-      inputType, outputType, std::stoul(get("batch-size", "1")), fieldShape,
+      inputType, outputType, batchSize, fieldShape,
       kernelShape, std::stoul(get("input-channels")),
       std::stoul(get("output-channels")), std::stoul(get("conv-groups", "1")),
       inT, kT, outT);
@@ -239,16 +386,30 @@ int main(int argc, char **argv) try {
   // ---- options (tools/single_conv_layer.cpp:803-832) ----------------------
   poplar::OptionFlags options;
   options.set("pass", has("inference-only") ? "INFERENCE_FWD" : "TRAINING_FWD");
-  if (has("fwd-plan-constraints-file")) {
-    std::ifstream f(get("fwd-plan-constraints-file"));
-    if (!f)
-      usage("cannot read '" + get("fwd-plan-constraints-file") + "'");
-    std::stringstream ss;
-    ss << f.rdbuf();
-    options.set("planConstraints", ss.str());
+  // (a constraints string and a constraints file for one pass exclude each
+  // other, tools/single_conv_layer.cpp:437-461)
+  for (const char *pass : {"fwd", "bwd", "wu"}) {
+    const std::string text = std::string(pass) + "-plan-constraints";
+    if (has(text.c_str()) && has((text + "-file").c_str()) &&
+        !get(text.c_str()).empty() && !get((text + "-file").c_str()).empty())
+      throw poputil::poplibs_error("Both " + text + " and " + text +
+                                   "-file were specified");
   }
-  if (has("fwd-plan-constraints"))
-    options.set("planConstraints", get("fwd-plan-constraints"));
+  auto constraintsFor = [&](const char *pass) -> std::pair<bool, std::string> {
+    const std::string text = std::string(pass) + "-plan-constraints";
+    const std::string file = text + "-file";
+    if (has(file.c_str()) && !get(file.c_str()).empty())
+      return {true, readFile(get(file.c_str()))};
+    if (has(text.c_str()))
+      return {true, get(text.c_str())};
+    return {false, ""};
+  };
+  const auto fwdConstraints = constraintsFor("fwd");
+  if (fwdConstraints.first)
+    options.set("planConstraints", fwdConstraints.second);
+  if (has("remap-output-tensor"))
+    options.set("remapOutputTensor",
+                parseBool(get("remap-output-tensor")) ? "true" : "false");
   if (has("convolution-options")) {
     const auto doc = poplibs_amd::json::parse(get("convolution-options"));
     if (!doc.isObject())
@@ -263,18 +424,20 @@ int main(int argc, char **argv) try {
   // (tools/single_conv_layer.cpp:793, 1064-1082).
   const ConvParams bwdParams = poplin::getGradientParams(params);
   poplar::OptionFlags bwdOptions = options;
-  if (has("bwd-plan-constraints"))
-    bwdOptions.set("planConstraints", get("bwd-plan-constraints"));
-  else if (has("fwd-plan-constraints"))
+  const auto bwdConstraints = constraintsFor("bwd");
+  if (bwdConstraints.first)
+    bwdOptions.set("planConstraints", bwdConstraints.second);
+  else if (fwdConstraints.first)
     bwdOptions.set("planConstraints", "");
   poplin::convolutionValidateOptions(bwdOptions);
   // Weight update: the forward options with pass TRAINING_WU
   // (tools/single_conv_layer.cpp:821-824).
   poplar::OptionFlags wuOptions = options;
   wuOptions.set("pass", "TRAINING_WU");
-  if (has("wu-plan-constraints"))
-    wuOptions.set("planConstraints", get("wu-plan-constraints"));
-  else if (has("fwd-plan-constraints"))
+  const auto wuConstraints = constraintsFor("wu");
+  if (wuConstraints.first)
+    wuOptions.set("planConstraints", wuConstraints.second);
+  else if (fwdConstraints.first)
     wuOptions.set("planConstraints", "");
   poplin::convolutionValidateOptions(wuOptions);
   const auto flops = poplin::getFwdFlops(params);
@@ -326,7 +489,7 @@ int main(int argc, char **argv) try {
       poplin::reportWeightUpdatePlanInfo(std::cout, params, wuOptions, &cache);
     }
   }
-  if (has("plan-only"))
+  if (has("plan-only") || has("compile-only"))
     return 0;
 
   // ---- data (tools/single_conv_layer.cpp:941-1005, 1183-1213) -------------
@@ -378,6 +541,11 @@ int main(int argc, char **argv) try {
   wMeta.format = fmt("fp8-format-weights");
   inMeta.scale = std::stoi(get("fp8-scale-fwd", "1"));
   wMeta.scale = std::stoi(get("fp8-scale-weights", "2"));
+  // the backward pass's input, the gradient of the forward output
+  // (tools/single_conv_layer.cpp:155-158: quart143, scale 1 by default)
+  poplin::QuarterMetadata zMeta;
+  zMeta.format = fmt("fp8-format-bwd");
+  zMeta.scale = std::stoi(get("fp8-scale-bwd", "1"));
 
   std::mt19937 rng(unsigned(std::stoul(get("seed", "5489"))));
   auto fill = [&](std::vector<double> &v, poplar::Type type, double lo,
@@ -414,16 +582,98 @@ int main(int argc, char **argv) try {
     for (auto &x : weights)
       x = std::ldexp(x, wMeta.scale);
     for (auto &x : zDeltas)
-      x = std::ldexp(x, inMeta.scale);
+      x = std::ldexp(x, zMeta.scale);
+  }
+  if (has("fwd-in-file")) {
+    // (the file's values as they are; quarter values under --fp8-scale-fwd)
+    if (fwdIn.bytes.size() != inElems * inputType.size())
+      throw poputil::poplibs_error("fwd-in-file does not hold the input");
+    if (inputType == poplar::QUARTER) {
+      for (size_t i = 0; i != inElems; ++i)
+        acts[i] = std::ldexp(
+            oracle_fp8_decode(fwdIn.bytes[i], int(inMeta.format)),
+            inMeta.scale);
+    } else {
+      acts = decode(fwdIn.bytes, inputType);
+    }
+  }
+  if (has("bwd-in-file")) {
+    bwdIn = loadTensor("bwd-in-file", get("bwd-in-file"));
+    std::cout << "Importing BWD input from file, shape:"
+              << shapeText(bwdIn.shape)
+              << " Element type:" << bwdIn.type.toString() << "\n";
+    if (bwdIn.type != inputType ||
+        bwdIn.bytes.size() != outElems * inputType.size())
+      throw poputil::poplibs_error(
+          "bwd-in-file does not hold the gradient of the forward output");
+    if (inputType == poplar::QUARTER) {
+      for (size_t i = 0; i != outElems; ++i)
+        zDeltas[i] = std::ldexp(
+            oracle_fp8_decode(bwdIn.bytes[i], int(zMeta.format)), zMeta.scale);
+    } else {
+      zDeltas = decode(bwdIn.bytes, inputType);
+    }
   }
   const auto actBytes = encode(acts, inputType, inMeta);
   const auto weightBytes = encode(weights, inputType, wMeta);
   const auto biasBytes = encode(biases, outputType, {});
-  const auto zDeltaBytes = encode(zDeltas, inputType, inMeta);
+  const auto zDeltaBytes = encode(zDeltas, inputType, zMeta);
 
   // ---- device run ----------------------------------------------------------
   poplin::Stream prog;
-  auto in = poplin::createInput(params, options, &cache);
+  // --test-planner: per pass, the planner's estimate against the time
+  // between two HIP events around 20 calls (after 3 untimed ones).
+  struct PlannerCheck {
+    std::string pass;
+    double estimateUs, measuredUs;
+  };
+  std::vector<PlannerCheck> plannerChecks;
+  const bool testPlanner = has("test-planner");
+  auto measure = [&](const std::string &pass, const ConvParams &p,
+                     const poplar::OptionFlags &o, auto &&call) {
+    if (!testPlanner)
+      return;
+    const poplin::PlanCosts costs =
+        poplin::reportPlanEstimatedCosts(p, o, &cache);
+    for (int i = 0; i != 3; ++i)
+      call();
+    prog.synchronize();
+    hipEvent_t start, stop;
+    if (hipEventCreate(&start) != hipSuccess ||
+        hipEventCreate(&stop) != hipSuccess)
+      throw poputil::poplibs_error("hipEventCreate failed");
+    const hipStream_t stream = static_cast<hipStream_t>(prog.handle());
+    const int reps = 20;
+    (void)hipEventRecord(start, stream);
+    for (int i = 0; i != reps; ++i)
+      call();
+    (void)hipEventRecord(stop, stream);
+    (void)hipEventSynchronize(stop);
+    float ms = 0;
+    (void)hipEventElapsedTime(&ms, start, stop);
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+    plannerChecks.push_back(
+        {pass,
+         costs.cycles == poplin::PlanCosts::unknown
+             ? -1.0
+             : double(costs.cycles) / poplin::PlanCosts::clockMHz,
+         double(ms) * 1e3 / reps});
+  };
+  // --use-create-input=false: an input in the plan-independent external
+  // layout [B][C][field...], which the convolution rearranges itself
+  // (tools/single_conv_layer.cpp:399-406, 1009-1020).
+  const bool useCreateInput = parseBool(get("use-create-input", "true"));
+  poplin::DeviceTensor in;
+  if (useCreateInput) {
+    in = poplin::createInput(params, options, &cache);
+  } else {
+    std::vector<size_t> shape{params.batchSize, params.getNumInputChans()};
+    shape.insert(shape.end(), fieldShape.begin(), fieldShape.end());
+    in = poplin::DeviceTensor(inputType, shape,
+                              poplin::DeviceTensor::Layout::External,
+                              std::max<size_t>(inElems * inputType.size(), 1));
+  }
   auto w = poplin::createWeights(params, options, &cache);
   in.metadata = inMeta;
   w.metadata = wMeta;
@@ -433,10 +683,21 @@ int main(int argc, char **argv) try {
   const unsigned runs = doFwdPass ? 1 + determinismChecks : 0;
   for (unsigned run = 0; run != runs; ++run) {
     if (!ignoreData) {
-      poplin::writeTensor(in, actBytes.data(), prog, params, options, &cache);
+      if (useCreateInput)
+        poplin::writeTensor(in, actBytes.data(), prog, params, options, &cache);
+      else
+        poplin::writeTensor(in, actBytes.data(), prog);
       poplin::writeTensor(w, weightBytes.data(), prog, params, options, &cache);
     }
-    auto out = poplin::convolution(in, w, params, false, prog, options, &cache);
+    poplin::DeviceTensor out;
+    if (parseBool(get("use-create-output", "false"))) {
+      // (tools/single_conv_layer.cpp:407, 1027-1035)
+      out = poplin::createConvOutput(params, options, &cache);
+      poplin::convolutionWithOutput(in, w, out, params, false, prog, options,
+                                    &cache);
+    } else {
+      out = poplin::convolution(in, w, params, false, prog, options, &cache);
+    }
     if (useBias) {
       auto b = poplin::createBiases(out);
       if (!ignoreData)
@@ -455,6 +716,20 @@ int main(int argc, char **argv) try {
       return 1;
     }
   }
+  if (doFwdPass && testPlanner) {
+    auto out = poplin::createConvOutput(params, options, &cache);
+    measure("fwd", params, options, [&] {
+      poplin::convolutionWithOutput(in, w, out, params, false, prog, options,
+                                    &cache);
+    });
+  }
+  if (has("fwd-out-file") && doFwdPass && !has("ignore-data")) {
+    std::vector<size_t> shape{params.batchSize, params.getNumOutputChans()};
+    shape.insert(shape.end(), outField.begin(), outField.end());
+    std::cout << "Saving FWD tensor with shape:" << shapeText(shape)
+              << " Element type:" << outputType.toString() << "\n";
+    saveTensor(get("fwd-out-file"), outputType, shape, result);
+  }
   // Backward pass: the forward weights, in the external layout, go in with
   // transposeAndFlipWeights = true.
   std::vector<uint8_t> bwdResult(inElems * outputType.size());
@@ -468,7 +743,7 @@ int main(int argc, char **argv) try {
                                     std::max<size_t>(weightBytes.size(), 1));
     fwdWeights.metadata = wMeta;
     auto deltas = poplin::createInput(bwdParams, bwdOptions, &cache);
-    deltas.metadata = inMeta;
+    deltas.metadata = zMeta;
     if (!ignoreData) {
       poplin::writeTensor(fwdWeights, weightBytes.data(), prog, params, options,
                           &cache);
@@ -481,6 +756,35 @@ int main(int argc, char **argv) try {
       poplin::readTensor(prevDeltas, bwdResult.data(), prog, bwdParams,
                          bwdOptions, &cache);
     prog.synchronize();
+    if (testPlanner) {
+      // (the estimate covers the convolution: the weights are turned round
+      // once, outside the timed calls)
+      std::vector<size_t> flippedShape = wShape;
+      std::swap(flippedShape[1], flippedShape[2]);
+      poplin::DeviceTensor flipped(inputType, flippedShape,
+                                   poplin::DeviceTensor::Layout::External,
+                                   std::max<size_t>(weightBytes.size(), 1));
+      flipped.metadata = wMeta;
+      poplin::weightsTransposeChansFlipXY(fwdWeights, flipped, prog);
+      std::vector<uint8_t> flippedBytes(weightBytes.size());
+      poplin::readTensor(flipped, flippedBytes.data(), prog);
+      auto packed = poplin::createWeights(bwdParams, bwdOptions, &cache);
+      packed.metadata = wMeta;
+      poplin::writeTensor(packed, flippedBytes.data(), prog, bwdParams,
+                          bwdOptions, &cache);
+      auto out = poplin::createConvOutput(bwdParams, bwdOptions, &cache);
+      measure("bwd", bwdParams, bwdOptions, [&] {
+        poplin::convolutionWithOutput(deltas, packed, out, bwdParams, false,
+                                      prog, bwdOptions, &cache);
+      });
+    }
+    if (has("bwd-out-file") && !ignoreData) {
+      std::vector<size_t> shape{params.batchSize, params.getNumInputChans()};
+      shape.insert(shape.end(), fieldShape.begin(), fieldShape.end());
+      std::cout << "Saving BWD tensor with shape:" << shapeText(shape)
+                << " Element type:" << outputType.toString() << "\n";
+      saveTensor(get("bwd-out-file"), outputType, shape, bwdResult);
+    }
   }
   // Weight update: weights += -learningRate * deltas on a copy of the
   // weights in the external layout, biases likewise
@@ -503,7 +807,10 @@ int main(int argc, char **argv) try {
       poplin::writeTensor(master, weightBytes.data(), prog);
       poplin::writeTensor(zIn, zDeltaBytes.data(), prog, bwdParams, bwdOptions,
                           &cache);
-      poplin::writeTensor(in, actBytes.data(), prog, params, options, &cache);
+      if (useCreateInput)
+        poplin::writeTensor(in, actBytes.data(), prog, params, options, &cache);
+      else
+        poplin::writeTensor(in, actBytes.data(), prog);
     }
     poplin::convolutionWeightUpdate(zIn, master, in, params,
                                     float(-learningRate), prog, wuOptions,
@@ -522,6 +829,42 @@ int main(int argc, char **argv) try {
     if (!ignoreData)
       poplin::readTensor(master, wuWeights.data(), prog);
     prog.synchronize();
+    if (testPlanner) {
+      // The estimate covers the pass's kernels: they are timed through the C
+      // ABI on tensors already in the device layouts, without the C++
+      // layer's allocations and conversions around them.
+      std::vector<const char *> keys, values;
+      for (const auto &kv : wuOptions) {
+        keys.push_back(kv.first.c_str());
+        values.push_back(kv.second.c_str());
+      }
+      mxconv_params c;
+      params.toC(c);
+      mxconv_plan *wuPlan = nullptr;
+      size_t wsBytes = 0;
+      if (mxconv_weight_update_plan_create(&c, keys.data(), values.data(),
+                                           keys.size(), &wuPlan) != MXCONV_OK ||
+          mxconv_weight_update_workspace_bytes(wuPlan, &wsBytes) != MXCONV_OK)
+        throw poputil::poplibs_error(mxconv_last_error());
+      auto actsCl = poplin::createInput(params, options, &cache);
+      if (!ignoreData)
+        poplin::writeTensor(actsCl, actBytes.data(), prog, params, options,
+                            &cache);
+      poplin::DeviceTensor deltasOut(
+          inputType, wShape, poplin::DeviceTensor::Layout::External,
+          std::max<size_t>(weightBytes.size(), 1));
+      poplin::DeviceTensor ws(poplar::FLOAT, {wsBytes / 4 + 1},
+                              poplin::DeviceTensor::Layout::External,
+                              wsBytes + 4);
+      measure("wu", poplin::getWeightUpdateParams(params), wuOptions, [&] {
+        if (mxconv_calculate_weight_deltas(
+                wuPlan, zIn.data(), actsCl.data(), deltasOut.data(), ws.data(),
+                wsBytes,
+                reinterpret_cast<mxconv_stream>(prog.handle())) != MXCONV_OK)
+          throw poputil::poplibs_error(mxconv_last_error());
+      });
+      mxconv_plan_destroy(wuPlan);
+    }
   }
   if (has("timing-runs") && doFwdPass) {
     const unsigned reps = unsigned(std::stoul(get("timing-runs")));
@@ -541,9 +884,30 @@ int main(int argc, char **argv) try {
     std::cout << "Forward time per call: " << s * 1e6 << " us, "
               << flops / s / 1e12 << " TFLOP/s\n";
   }
+  bool plannerOk = true;
+  if (testPlanner) {
+    const double tol = std::stod(get("test-planner-tolerance", "2.5"));
+    std::cout << "Planner estimates against measurements (factor " << tol
+              << " beyond 15 us of launch overhead allowed):\n";
+    for (const auto &c : plannerChecks) {
+      std::cout << "  " << c.pass << ": estimated ";
+      if (c.estimateUs < 0) {
+        std::cout << "unknown (the cost model does not cover this kernel), "
+                     "measured "
+                  << c.measuredUs << " us\n";
+        continue;
+      }
+      const bool ok = c.measuredUs <= tol * c.estimateUs + 15.0 &&
+                      c.estimateUs <= tol * c.measuredUs + 15.0;
+      std::cout << c.estimateUs << " us, measured " << c.measuredUs
+                << " us per call" << (ok ? "" : "  <-- beyond the tolerance")
+                << "\n";
+      plannerOk = plannerOk && ok;
+    }
+  }
   if (ignoreData) {
     std::cout << "Results not checked (--ignore-data)\n";
-    return 0;
+    return plannerOk ? 0 : 1;
   }
 
   // ---- host model and comparison (tools/single_conv_layer.cpp:1239-1252,
@@ -677,11 +1041,57 @@ int main(int argc, char **argv) try {
   if (!ok)
     return 1;
   std::cout << "Validation passed\n";
+  if (!plannerOk) {
+    std::cerr << "planner estimates beyond the tolerance\n";
+    return 1;
+  }
   return 0;
+} catch (const UsageError &e) {
+  std::cerr << "error: " << e.what() << "\n"
+            << "usage: single_conv_layer --input-channels N --output-channels "
+               "N --field {H,W} [--kernel-size {h,w}] [options]\n"
+               "  see the header of tests/tools/single_conv_layer.cpp for the "
+               "option list\n";
+  return 1;
 } catch (const poplar::graph_memory_allocation_error &e) {
   std::cerr << e.what() << std::endl;
   return 77;
 } catch (const std::exception &e) {
   std::cerr << "error: " << e.what() << std::endl;
   return 1;
+}
+
+int main(int argc, char **argv) {
+  if (argc == 3 && std::string(argv[1]) == "--batch-file") {
+    // many invocations, one process; everything goes to stdout
+    std::cerr.rdbuf(std::cout.rdbuf());
+    poplibs_amd::json::Value doc;
+    try {
+      doc = poplibs_amd::json::parse(readFile(argv[2]));
+    } catch (const std::exception &e) {
+      std::cout << "error: " << e.what() << "\n";
+      return 1;
+    }
+    int failed = 0;
+    for (const auto &test : doc.items) {
+      std::string name;
+      std::vector<std::string> args{"single_conv_layer"};
+      for (const auto &m : test.members) {
+        if (m.first == "name")
+          name = m.second.text;
+        if (m.first == "args")
+          for (const auto &a : m.second.items)
+            args.push_back(a.text);
+      }
+      std::vector<char *> av;
+      for (auto &a : args)
+        av.push_back(const_cast<char *>(a.c_str()));
+      std::cout << "### CASE " << name << std::endl;
+      const int rc = runCase(int(av.size()), av.data());
+      std::cout << "### RESULT " << name << " " << rc << std::endl;
+      failed += rc != 0;
+    }
+    return failed ? 1 : 0;
+  }
+  return runCase(argc, argv);
 }
