@@ -40,6 +40,29 @@ constexpr int kRowsThreads = 64 * (kComputeWaves + kLoaderWaves);
 constexpr int kOwnLoads = kRowLoads / kLoaderWaves; // per loader wave and row
 constexpr uint32_t kNoByte = 0x80000000u;           // beyond any buffer here
 
+// Wall-clock stamps (s_memrealtime, 100 MHz) of depthwiseRowsKernel's
+// milestones, for the build with -DMXK_ROWS_STAMPS only
+// (libmxconv_stamps.so; the product library carries none of this): compute
+// wave 0 and the first loader wave of every workgroup write eight stamps each
+// to the buffer mxk_rows_stamp_sink() names: [workgroup][compute | loader][8].
+#ifdef MXK_ROWS_STAMPS
+__device__ uint64_t *rowsStampSink = nullptr;
+#define MXK_RSTAMP_DECL uint64_t rstamps_[8] = {}
+#define MXK_RSTAMP(i) rstamps_[i] = __builtin_amdgcn_s_memrealtime()
+#define MXK_RSTAMP_IF(c, i)                                                    \
+  if (c)                                                                       \
+  rstamps_[i] = __builtin_amdgcn_s_memrealtime()
+#define MXK_RSTAMP_OUT(who, on)                                                \
+  if (rowsStampSink && (on))                                                   \
+    for (int i_ = 0; i_ != 8; ++i_)                                            \
+  rowsStampSink[(size_t(blockIdx.x) * 2 + (who)) * 8 + i_] = rstamps_[i_]
+#else
+#define MXK_RSTAMP_DECL
+#define MXK_RSTAMP(i)
+#define MXK_RSTAMP_IF(c, i)
+#define MXK_RSTAMP_OUT(who, on)
+#endif
+
 /// The forward kernel's ring by stride.  kAhead: steps (output rows) the
 /// loads run ahead; a step needs rows [j S, j S + 2], so `ahead` steps on the
 /// way take ahead * S + 3 slots.  Six rows on the way: on N = 32, 112 x 112,
@@ -171,6 +194,8 @@ __global__ __launch_bounds__((Ring<S, K>::kThreads)) void depthwiseRowsKernel(
   // relative input rows [0, rowsIn) are what the band reads
   const uint32_t rowsIn = (steps - 1) * S + K;
 
+  MXK_RSTAMP_DECL;
+  MXK_RSTAMP(0); // the wave starts
   if (wave >= R::kComputeWaves) {
     // ---- loaders.  Load L of a row fills bytes [1024 L, 1024 L + 1024) of
     // its slot: 16-byte unit u = 64 L + lane is channel vector u % vecs of
@@ -182,6 +207,7 @@ __global__ __launch_bounds__((Ring<S, K>::kThreads)) void depthwiseRowsKernel(
                 a.divVecs, loader, lane);
     const uint32_t imageByte = b * d.inH * d.inW * pixelBytes;
     const uint32_t rowBytes = d.inW * pixelBytes;
+    MXK_RSTAMP(1); // set-up done: the first load goes out
     uint32_t next = 0; // the relative row loaded next
     auto loadRow = [&] {
       const int ih = ih0 + int(next);
@@ -193,8 +219,11 @@ __global__ __launch_bounds__((Ring<S, K>::kThreads)) void depthwiseRowsKernel(
     };
     // rows of steps 0 .. kAhead - 1
 #pragma unroll 1
-    for (int r = 0; r != (kAhead - 1) * S + R::kWindow; ++r)
+    for (int r = 0; r != (kAhead - 1) * S + R::kWindow; ++r) {
       loadRow();
+      MXK_RSTAMP_IF(r == R::kWindow - 1, 2); // step 0's rows requested
+    }
+    MXK_RSTAMP(3); // the rows of the first kAhead steps requested
     for (uint32_t j = 0; j < steps; ++j) {
       // step j's window has landed when all but the rows of the kAhead - 1
       // steps behind it have
@@ -205,7 +234,10 @@ __global__ __launch_bounds__((Ring<S, K>::kThreads)) void depthwiseRowsKernel(
       for (int r = 0; r != S; ++r)
         loadRow();
     }
+    MXK_RSTAMP(4); // last loads issued
     MXK_WAIT_VMCNT(0);
+    MXK_RSTAMP(5); // ... and landed
+    MXK_RSTAMP_OUT(1, wave == R::kComputeWaves && lane == 0);
     return;
   }
 
@@ -275,6 +307,9 @@ __global__ __launch_bounds__((Ring<S, K>::kThreads)) void depthwiseRowsKernel(
     uint32_t slot = 0; // slot of relative row j * S
     for (uint32_t j = 0; j < steps; ++j) {
       stepBarrier(); // step j's rows are in the ring
+      MXK_RSTAMP_IF(j == 0, 1);         // step 0's rows have landed
+      MXK_RSTAMP_IF(j == 1, 2);         // step 1's
+      MXK_RSTAMP_IF(j + 1 == steps, 3); // the last step's
       uint32_t rowSlot = slot;
       if constexpr (K == 3) {
         Vec8 win[K][K];
@@ -356,6 +391,12 @@ __global__ __launch_bounds__((Ring<S, K>::kThreads)) void depthwiseRowsKernel(
         step(std::integral_constant<int, 3>{}, false);
     }
   }
+#ifdef MXK_ROWS_STAMPS
+  MXK_RSTAMP(4); // last store issued
+  __builtin_amdgcn_s_waitcnt(0);
+  MXK_RSTAMP(5); // ... and landed
+  MXK_RSTAMP_OUT(0, t == 0);
+#endif
 }
 
 
@@ -713,3 +754,12 @@ hipError_t launchDepthwiseRowsDeltas(const DepthwiseDesc &d, const void *acts,
 }
 
 } // namespace mxk
+
+#ifdef MXK_ROWS_STAMPS
+/// Stamps build only: the device buffer the stamped kernel writes to
+/// ([workgroups][2][8] of 8 bytes), or null to switch the stamps off.
+extern "C" int mxk_rows_stamp_sink(void *deviceBuffer) {
+  return int(hipMemcpyToSymbol(HIP_SYMBOL(mxk::rowsStampSink), &deviceBuffer,
+                               sizeof(deviceBuffer)));
+}
+#endif

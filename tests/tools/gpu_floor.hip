@@ -16,6 +16,16 @@
 //       sustains.  The MFMA peak of 2.5 PFLOP/s is 256 CUs x 4096 flop/clk at
 //       2.4 GHz: clock / 2400 MHz x busy CUs / 256 is the share of it any
 //       schedule on that many CUs can reach.
+//
+//   gpu_floor stream
+//       what a kernel that does nothing but stream reaches at the depthwise
+//       benchmark layer's size and mix (77.1 MB read, 19.3 MB written per
+//       launch): every thread loads four 16-byte vectors from four input
+//       planes and stores one, consecutive threads consecutive vectors,
+//       buffers rotated over four sets (385 MB, beyond the 256 MB Infinity
+//       Cache), 200 launches in a replayed HIP graph as bench.py issues its
+//       steps.  Variants: U outputs per thread, plain or non-temporal loads
+//       and stores, the four loads of an output far apart or adjacent.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -58,7 +68,7 @@ double launchFloor(int grid, int block, int ldsBytes, int launches = 200,
     hipLaunchKernelGGL(emptyKernel, dim3(grid), dim3(block), ldsBytes, stream,
                        static_cast<int *>(nullptr));
   CHECK(hipStreamEndCapture(stream, &graph));
-  CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+  CHECK(hipGraphInstantiateWithFlags(&exec, graph, 0));
   CHECK(hipGraphLaunch(exec, stream));
   CHECK(hipStreamSynchronize(stream));
   hipEvent_t start, stop;
@@ -129,6 +139,85 @@ __global__ __launch_bounds__(512) void mfmaLoop(int iters, const uint32_t *seed,
   (void)lane;
 }
 
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+/// U outputs per thread; NT: non-temporal loads and stores; ADJ: the four
+/// loads of an output are neighbours in memory instead of a plane apart.
+template <int U, bool NT, bool ADJ>
+__global__ __launch_bounds__(256) void streamMix(const uintx4 *__restrict__ in,
+                                                 uintx4 *__restrict__ out,
+                                                 size_t outVecs) {
+  uintx4 v[U][4];
+#pragma unroll
+  for (int u = 0; u != U; ++u) {
+    const size_t o = (size_t(blockIdx.x) * U + u) * 256 + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k != 4; ++k) {
+      const uintx4 *p = ADJ ? in + ((size_t(blockIdx.x) * U + u) * 4 + k) * 256 +
+                                  threadIdx.x
+                            : in + size_t(k) * outVecs + o;
+      if (o < outVecs)
+        v[u][k] = NT ? __builtin_nontemporal_load(p) : *p;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u != U; ++u) {
+    const size_t o = (size_t(blockIdx.x) * U + u) * 256 + threadIdx.x;
+    if (o < outVecs) {
+      const uintx4 sum = v[u][0] + v[u][1] + v[u][2] + v[u][3];
+      if (NT)
+        __builtin_nontemporal_store(sum, out + o);
+      else
+        out[o] = sum;
+    }
+  }
+}
+
+template <int U, bool NT, bool ADJ>
+void streamCeiling(const char *name, const std::vector<uintx4 *> &ins,
+                   const std::vector<uintx4 *> &outs, size_t outVecs,
+                   double bytes) {
+  const int sets = int(ins.size());
+  const int blocks = int((outVecs + size_t(256) * U - 1) / (size_t(256) * U));
+  hipStream_t stream;
+  CHECK(hipStreamCreate(&stream));
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+  const int launches = 200;
+  CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeGlobal));
+  for (int i = 0; i != launches; ++i)
+    hipLaunchKernelGGL((streamMix<U, NT, ADJ>), dim3(blocks), dim3(256), 0,
+                       stream, ins[i % sets], outs[i % sets], outVecs);
+  CHECK(hipStreamEndCapture(stream, &graph));
+  CHECK(hipGraphInstantiateWithFlags(&exec, graph, 0));
+  CHECK(hipGraphLaunch(exec, stream));
+  CHECK(hipStreamSynchronize(stream));
+  hipEvent_t start, stop;
+  CHECK(hipEventCreate(&start));
+  CHECK(hipEventCreate(&stop));
+  std::vector<double> us;
+  for (int p = 0; p != 7; ++p) {
+    CHECK(hipEventRecord(start, stream));
+    for (int r = 0; r != 2; ++r)
+      CHECK(hipGraphLaunch(exec, stream));
+    CHECK(hipEventRecord(stop, stream));
+    CHECK(hipStreamSynchronize(stream));
+    float ms = 0;
+    CHECK(hipEventElapsedTime(&ms, start, stop));
+    us.push_back(double(ms) * 1e3 / (2 * launches));
+  }
+  std::sort(us.begin(), us.end());
+  const double t = us[us.size() / 2];
+  std::printf("| %s | %d | %s | %.2f | %.0f | %.1f %% |\n", name, U,
+              NT ? "non-temporal" : "plain", t, bytes / t / 1e3,
+              bytes / t / 1e3 / 80.0);
+  CHECK(hipGraphExecDestroy(exec));
+  CHECK(hipGraphDestroy(graph));
+  CHECK(hipEventDestroy(start));
+  CHECK(hipEventDestroy(stop));
+  CHECK(hipStreamDestroy(stream));
+}
+
 void clockUnderLoad(int workgroups) {
   const int iters = 400; // x 64 MFMAs of 16 cycles: ~0.2 ms per launch
   uint32_t *seed;
@@ -182,8 +271,10 @@ void clockUnderLoad(int workgroups) {
 }
 
 int main(int argc, char **argv) {
-  if (argc < 2 || (std::strcmp(argv[1], "launch") && std::strcmp(argv[1], "clock"))) {
-    std::fprintf(stderr, "usage: gpu_floor launch | gpu_floor clock [workgroups ...]\n");
+  if (argc < 2 || (std::strcmp(argv[1], "launch") && std::strcmp(argv[1], "clock") &&
+                   std::strcmp(argv[1], "stream"))) {
+    std::fprintf(stderr, "usage: gpu_floor launch | gpu_floor clock "
+                         "[workgroups ...] | gpu_floor stream\n");
     return 2;
   }
   hipDeviceProp_t prop;
@@ -201,6 +292,31 @@ int main(int argc, char **argv) {
     for (const auto &s : shapes)
       std::printf("| %d | %d | %d | %.2f |\n", s[0], s[1], s[2],
                   launchFloor(s[0], s[1], s[2]));
+    return 0;
+  }
+  if (!std::strcmp(argv[1], "stream")) {
+    const size_t outBytes = 19267584, inBytes = 4 * outBytes;
+    const size_t outVecs = outBytes / 16;
+    std::vector<uintx4 *> ins(4), outs(4);
+    for (int i = 0; i != 4; ++i) {
+      CHECK(hipMalloc(&ins[i], inBytes));
+      CHECK(hipMemset(ins[i], i + 1, inBytes));
+      CHECK(hipMalloc(&outs[i], outBytes));
+    }
+    const double bytes = double(inBytes + outBytes);
+    std::printf("4 : 1 stream of %.0f bytes per launch (%zu read, %zu "
+                "written), 4 buffer sets in turn, 200 launches in a replayed "
+                "HIP graph, median of 7 passes\n\n",
+                bytes, inBytes, outBytes);
+    std::printf("| the four loads of an output | outputs per thread | loads "
+                "and stores | us per launch | GB/s | of 8 TB/s |\n");
+    std::printf("|---|---|---|---|---|---|\n");
+    streamCeiling<1, false, false>("a plane apart", ins, outs, outVecs, bytes);
+    streamCeiling<1, true, false>("a plane apart", ins, outs, outVecs, bytes);
+    streamCeiling<2, true, false>("a plane apart", ins, outs, outVecs, bytes);
+    streamCeiling<4, true, false>("a plane apart", ins, outs, outVecs, bytes);
+    streamCeiling<1, false, true>("adjacent", ins, outs, outVecs, bytes);
+    streamCeiling<1, true, true>("adjacent", ins, outs, outVecs, bytes);
     return 0;
   }
   std::printf("8 waves per workgroup (two per SIMD) of back-to-back "
