@@ -62,6 +62,16 @@ def _workloads(pa):
                           1, 1, 1),
             dtype="fp8", bound="mfma", relu=False,
             w_std=(2 / (9 * 256)) ** .5),
+        # Not one of the benchmark configurations: a layer that fills the chip
+        # seven times over, where the launch is a small part of the time.
+        "steady_state": dict(
+            name="steady state (not a benchmark configuration): 3x3 conv "
+                 "N=128 28x28 Cin=Cout=256 stride 1 pad 1, fp16, 1792 tiles "
+                 "= 7 rounds on 256 CUs",
+            params=params(pa.HALF, pa.HALF, 128, (28, 28), (3, 3), 256, 256,
+                          1, 1, 1),
+            dtype="fp16", bound="mfma", relu=False,
+            w_std=(2 / (9 * 256)) ** .5),
     }
 
 
@@ -396,7 +406,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2",
-                    help="headline workload (c2, c3, c4, c5)")
+                    help="headline workload (c2, c3, c4, c5; steady_state)")
     ap.add_argument("--only", action="store_true",
                     help="skip the other workloads and the CPU baseline")
     ap.add_argument("--cache-hot", action="store_true",

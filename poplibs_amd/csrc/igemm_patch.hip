@@ -1149,7 +1149,7 @@ bool patchShape(const IgemmDesc &d, int inType, int outType, PatchShape &s) {
   const uint64_t pitch =
       uint64_t(d.outW) * 16 * units +
       ((cols - d.outW) * 16 * units + 255) / 256 * 256;
-  s.maxRows = maxPatchRows(d);
+  s.maxRows = d.patchMaxRows ? d.patchMaxRows : maxPatchRows(d);
   // (a lane per patch row works out where the rows start)
   if (s.maxRows > 64)
     return false;
@@ -1255,6 +1255,8 @@ hipError_t dispatchPatchOut(int outType, const PatchShape &s,
 }
 
 } // namespace
+
+uint32_t igemmPatchMaxRows(const IgemmDesc &d) { return maxPatchRows(d); }
 
 bool igemmPatchTakes(const IgemmDesc &d, int inType, int outType) {
   PatchShape s;

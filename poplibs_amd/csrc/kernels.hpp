@@ -200,6 +200,10 @@ struct IgemmDesc {
   // MFMA blocks, blockM 64 or 128; 2: 16-pixel MFMA blocks, blockM = pixels
   // per tile, any number up to 112.
   uint32_t patch = 0;
+  // Patch rows the tallest tile of that kernel spans (igemmPatchMaxRows),
+  // worked out once when the plan is made - it takes a walk over the tiles -
+  // so that a launch does not repeat it; 0 = not known, work it out.
+  uint32_t patchMaxRows = 0;
 };
 /// How the kernel finds out which kernel taps of an output pixel read inside
 /// the input: a bit mask per pixel (up to 32 taps), ranges of valid kernel
@@ -222,6 +226,9 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
 /// undilated input, two field dimensions, half or quarter inputs whose
 /// channels per group fill whole 128-byte slices, K not split.
 bool igemmPatchTakes(const IgemmDesc &d, int inType, int outType);
+/// Patch rows a tile of d.blockM consecutive output pixels can span: what a
+/// planner stores in d.patchMaxRows.
+uint32_t igemmPatchMaxRows(const IgemmDesc &d);
 /// Elements of its packed weights:
 /// [G][32-channel block][K half][k-step][operand][lane][16 bytes].
 uint64_t igemmPatchPackedElems(const IgemmDesc &d, int inType);

@@ -925,6 +925,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         g.blockM = tilings[best].blockM;
         g.splitK = 1;
         g.blockN = 128;
+        g.patchMaxRows = 0;
+        g.patchMaxRows = mxk::igemmPatchMaxRows(g);
         plan.workspaceBytes = 0;
         plan.coPadded = (co + 127) / 128 * 128;
         plan.weightPackedElems = mxk::igemmPatchPackedElems(g, inId);
@@ -1084,6 +1086,13 @@ double mxconv_plan::estimatedMicroseconds() const {
   case Kernel::IGEMM: {
     if (pointwiseOn) {
       us = streamed(inputBytes() + outputBytes() + weightPackedBytes());
+      // With many input channels a 1x1 layer is as much the matrix cores' as
+      // the memory's: N = 32, 28 x 28, 512 -> 512 runs at 710 TFLOP/s
+      // (18.5 us where its bytes alone would stream in 10).
+      const double flops = 2.0 * pointwise.batch * pointwise.pixels *
+                           pointwise.groups * pointwise.inChansPerGroup *
+                           pointwise.outChansPerGroup;
+      us = std::max(us, poplin::kLaunchUs + flops / 7.0e8);
       break;
     }
     bool weighed = false;
