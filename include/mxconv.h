@@ -265,6 +265,34 @@ mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
                                           uint64_t *cycles,
                                           uint64_t *memory_bytes);
 
+/* reportDetailedPlanEstimatedCosts (include/poplin/Convolution.hpp:613-676,
+ * lib/poplin/Convolution.cpp:3940-3962): the same estimate taken apart.  Of
+ * the reference's phases a launch on this device has three: rearrangement
+ * (the zero-padded copy of an input whose channels do not fill a vector, the
+ * fill of an output field the kernel does not cover), compute (the
+ * convolution kernel) and reduction (the ordered sum of fp32 partial tiles
+ * where K or the pixels are split over workgroups).  Each phase: cycles as in
+ * mxconv_plan_estimated_costs and the temporary bytes it owns.
+ * parallel_split: workgroups that run side by side (at most the CUs times
+ * the workgroups a CU holds); serial_split: rounds of them.  The phases'
+ * cycles add up to total.cycles, which is what mxconv_plan_estimated_costs
+ * returns; every cycles field is MXCONV_COST_UNKNOWN where that is.
+ * Touches no GPU. */
+typedef struct mxconv_phase_cost {
+  uint64_t cycles;
+  uint64_t memory_bytes;
+} mxconv_phase_cost;
+typedef struct mxconv_detailed_costs {
+  uint64_t parallel_split;
+  uint64_t serial_split;
+  mxconv_phase_cost rearrangement;
+  mxconv_phase_cost compute;
+  mxconv_phase_cost reduction;
+  mxconv_phase_cost total;
+} mxconv_detailed_costs;
+mxconv_status mxconv_plan_detailed_costs(const mxconv_plan *plan,
+                                         mxconv_detailed_costs *costs);
+
 /* Whether weights packed for `packed_for` are laid out as `plan` reads them
  * (*same = 1) or not (0).  In the reference the options given to
  * createWeights only decide a tensor layout and convolution() rearranges a

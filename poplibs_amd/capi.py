@@ -73,6 +73,17 @@ class CParams(Structure):
                 ("output_transform", _COutputTransform)]
 
 
+class _CPhaseCost(Structure):
+    _fields_ = [("cycles", c_uint64), ("memory_bytes", c_uint64)]
+
+
+class DetailedCosts(Structure):
+    """mxconv_detailed_costs."""
+    _fields_ = [("parallel_split", c_uint64), ("serial_split", c_uint64),
+                ("rearrangement", _CPhaseCost), ("compute", _CPhaseCost),
+                ("reduction", _CPhaseCost), ("total", _CPhaseCost)]
+
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libmxconv.so")
 _lib = None
@@ -168,6 +179,8 @@ def lib():
                                              POINTER(c_size_t)]),
         "mxconv_plan_estimated_costs": (c_int, [c_void_p, POINTER(c_uint64),
                                                 POINTER(c_uint64)]),
+        "mxconv_plan_detailed_costs": (c_int, [c_void_p,
+                                               POINTER(DetailedCosts)]),
         "mxconv_plans_pack_alike": (c_int, [c_void_p, c_void_p,
                                             POINTER(c_int32)]),
         "mxconv_pack_weights": (c_int, [c_void_p, c_void_p, c_void_p,
@@ -606,6 +619,21 @@ class Plan:
         _check(lib().mxconv_plan_estimated_costs(self._h, byref(cycles),
                                                  byref(memory)))
         return cycles.value, memory.value
+
+    def detailed_costs(self):
+        """The estimate of estimated_costs taken apart: a dict with
+        parallelSplit, serialSplit and (cycles, memory bytes) for
+        rearrangement, compute, reduction and total:
+        reportDetailedPlanEstimatedCosts
+        (include/poplin/Convolution.hpp:613-676)."""
+        c = DetailedCosts()
+        _check(lib().mxconv_plan_detailed_costs(self._h, byref(c)))
+        out = {"parallelSplit": c.parallel_split,
+               "serialSplit": c.serial_split}
+        for phase in ("rearrangement", "compute", "reduction", "total"):
+            p = getattr(c, phase)
+            out[phase] = (p.cycles, p.memory_bytes)
+        return out
 
     def packs_like(self, other):
         """Whether weights packed for `other` are laid out as this plan

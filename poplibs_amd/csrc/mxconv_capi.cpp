@@ -608,6 +608,38 @@ mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
   return MXCONV_OK;
 }
 
+mxconv_status mxconv_plan_detailed_costs(const mxconv_plan *plan,
+                                         mxconv_detailed_costs *costs) {
+  REQUIRE_ARG(plan);
+  REQUIRE_ARG(costs);
+  lastError.clear();
+  const mxconv_plan::DetailedEstimate e = plan->detailedEstimate();
+  *costs = mxconv_detailed_costs{};
+  costs->parallel_split = e.parallelSplit;
+  costs->serial_split = e.serialSplit;
+  costs->rearrangement.memory_bytes = e.rearrangementBytes;
+  costs->reduction.memory_bytes = e.reductionBytes;
+  costs->total.memory_bytes = plan->workspaceBytes;
+  if (!e.known) {
+    costs->rearrangement.cycles = costs->compute.cycles =
+        costs->reduction.cycles = costs->total.cycles = MXCONV_COST_UNKNOWN;
+    return MXCONV_OK;
+  }
+  auto cyclesOf = [](double us) {
+    return uint64_t(us * mxconv_plan::kEstimateClockMHz + 0.5);
+  };
+  // The kernel takes what rounding leaves, so that the phases add up.
+  costs->total.cycles = cyclesOf(e.totalUs());
+  costs->rearrangement.cycles =
+      std::min(cyclesOf(e.rearrangementUs), costs->total.cycles);
+  costs->reduction.cycles =
+      std::min(cyclesOf(e.reductionUs),
+               costs->total.cycles - costs->rearrangement.cycles);
+  costs->compute.cycles = costs->total.cycles - costs->rearrangement.cycles -
+                          costs->reduction.cycles;
+  return MXCONV_OK;
+}
+
 mxconv_status mxconv_plan_buffer_bytes(const mxconv_plan *plan, int32_t which,
                                        size_t *bytes) {
   REQUIRE_ARG(plan);

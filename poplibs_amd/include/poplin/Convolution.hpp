@@ -206,6 +206,87 @@ PlanCosts reportPlanEstimatedCosts(const ConvParams &params,
                                    const poplar::OptionFlags &options = {},
                                    PlanningCache *cache = nullptr);
 
+namespace internal {
+
+/// The estimate of reportPlanEstimatedCosts by phase
+/// (include/poplin/Convolution.hpp:613-665 of PopLibs; same fields, same
+/// text form).  A launch on this device has three of the phases:
+/// `rearrangement` (the zero-padded copy of an input whose channels do not
+/// fill a vector, the fill of an output field the kernel does not cover),
+/// `compute` (the convolution kernel) and `reduction` (the ordered sum of fp32
+/// partial tiles where K or the pixels are split over workgroups); the other
+/// phases are IPU exchange and tile-level steps and stay zero.
+/// parallelSplit: workgroups that run side by side; serialSplit: rounds of
+/// them.  The phases' cycles add up to total.cycles; all cycles are
+/// PlanCosts::unknown where the model does not cover the kernel.
+struct DetailedPlanCosts {
+  std::size_t parallelSplit = 1;
+  std::size_t serialSplit = 1;
+  PlanCosts broadcast = {};
+  PlanCosts rearrangement = {};
+  PlanCosts dynamicSlice = {};
+  PlanCosts transform = {};
+  PlanCosts exchange = {};
+  PlanCosts tileLevelTransform = {};
+  PlanCosts inputsCast = {};
+  PlanCosts compute = {};
+  PlanCosts reduction = {};
+  PlanCosts dynamicUpdate = {};
+  PlanCosts addInPlace = {};
+  PlanCosts outputCast = {};
+  PlanCosts total = {};
+
+  /// Calls fn on each phase in the order above; serialSplitOnly leaves out
+  /// the phases that happen once however the convolution is split in series
+  /// (broadcast, rearrangement, addInPlace, outputCast).
+  template <typename Function>
+  void apply(Function fn, bool includeTotal = true,
+             bool serialSplitOnly = false) {
+    struct Phase {
+      PlanCosts DetailedPlanCosts::*member;
+      bool oncePerConv;
+    };
+    static constexpr Phase order[] = {
+        {&DetailedPlanCosts::broadcast, true},
+        {&DetailedPlanCosts::rearrangement, true},
+        {&DetailedPlanCosts::dynamicSlice, false},
+        {&DetailedPlanCosts::transform, false},
+        {&DetailedPlanCosts::exchange, false},
+        {&DetailedPlanCosts::tileLevelTransform, false},
+        {&DetailedPlanCosts::inputsCast, false},
+        {&DetailedPlanCosts::compute, false},
+        {&DetailedPlanCosts::reduction, false},
+        {&DetailedPlanCosts::dynamicUpdate, false},
+        {&DetailedPlanCosts::addInPlace, true},
+        {&DetailedPlanCosts::outputCast, true}};
+    for (const Phase &p : order)
+      if (!(serialSplitOnly && p.oncePerConv))
+        fn(this->*p.member);
+    if (includeTotal)
+      fn(total);
+  }
+  template <typename Function>
+  void apply(Function fn, bool includeTotal = true,
+             bool serialSplitOnly = false) const {
+    DetailedPlanCosts copy = *this;
+    copy.apply([&fn](PlanCosts &c) { fn(static_cast<const PlanCosts &>(c)); },
+               includeTotal, serialSplitOnly);
+  }
+};
+
+/// "parallelSplit serialSplit" on one line, then "cycles memory" per phase
+/// and for the total (lib/poplin/Convolution.cpp:3940-3951 of PopLibs).
+std::ostream &operator<<(std::ostream &os, DetailedPlanCosts const &c);
+std::istream &operator>>(std::istream &is, DetailedPlanCosts &c);
+
+/// include/poplin/Convolution.hpp:670-676 of PopLibs.
+DetailedPlanCosts
+reportDetailedPlanEstimatedCosts(const ConvParams &params,
+                                 const poplar::OptionFlags &options = {},
+                                 PlanningCache *cache = nullptr);
+
+} // namespace internal
+
 /// What poplin::preplan takes for one convolution
 /// (include/poplin/Convolution.hpp:386-388 of PopLibs): the target (may be
 /// null), the parameters and a pointer to the options.

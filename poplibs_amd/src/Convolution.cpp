@@ -442,6 +442,46 @@ PlanCosts reportPlanEstimatedCosts(const ConvParams &params,
           std::size_t(memory)};
 }
 
+namespace internal {
+
+std::ostream &operator<<(std::ostream &os, DetailedPlanCosts const &c) {
+  os << c.parallelSplit << ' ' << c.serialSplit << '\n';
+  c.apply([&](const PlanCosts &phase) {
+    os << phase.cycles << ' ' << phase.memory << '\n';
+  });
+  return os;
+}
+
+std::istream &operator>>(std::istream &is, DetailedPlanCosts &c) {
+  is >> c.parallelSplit >> c.serialSplit;
+  c.apply([&](PlanCosts &phase) { is >> phase.cycles >> phase.memory; });
+  return is;
+}
+
+DetailedPlanCosts
+reportDetailedPlanEstimatedCosts(const ConvParams &params,
+                                 const poplar::OptionFlags &options,
+                                 PlanningCache *cache) {
+  auto plan = detail::getPlan(params, options, cache);
+  mxconv_detailed_costs raw{};
+  detail::check(mxconv_plan_detailed_costs(plan->plan, &raw));
+  auto phase = [](const mxconv_phase_cost &p) {
+    return PlanCosts{p.cycles == MXCONV_COST_UNKNOWN ? PlanCosts::unknown
+                                                     : std::size_t(p.cycles),
+                     std::size_t(p.memory_bytes)};
+  };
+  DetailedPlanCosts c;
+  c.parallelSplit = std::size_t(raw.parallel_split);
+  c.serialSplit = std::size_t(raw.serial_split);
+  c.rearrangement = phase(raw.rearrangement);
+  c.compute = phase(raw.compute);
+  c.reduction = phase(raw.reduction);
+  c.total = phase(raw.total);
+  return c;
+}
+
+} // namespace internal
+
 void preplan(const std::set<ConvPlanParams> &convs,
              const std::set<MatMulPlanParams> &matmuls, PlanningCache &cache) {
   if (convs.empty() && matmuls.empty())

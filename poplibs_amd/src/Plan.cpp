@@ -1046,7 +1046,7 @@ std::string mxconv_plan::constraintsJson() const {
   return os.str();
 }
 
-double mxconv_plan::estimatedMicroseconds() const {
+mxconv_plan::DetailedEstimate mxconv_plan::detailedEstimate() const {
   // Kernels that stream their tensors once (1x1 with few channels, depthwise,
   // fills) run at about 6.4 TB/s behind the launch: 64 MB in 11.6 us and
   // 96 MB in 17.9 us measured.
@@ -1054,19 +1054,39 @@ double mxconv_plan::estimatedMicroseconds() const {
   auto streamed = [&](std::size_t bytes) {
     return poplin::kLaunchUs + double(bytes) / kStreamBytesPerUs;
   };
-  if (zeroConv)
-    return streamed(outputBytes());
+  auto spread = [](DetailedEstimate &e, std::size_t workgroups,
+                   std::size_t perCU) {
+    const std::size_t slots = std::size_t(gfx950::numCUs) * perCU;
+    e.parallelSplit = std::max<std::size_t>(1, std::min(workgroups, slots));
+    e.serialSplit =
+        std::max<std::size_t>(1, (workgroups + slots - 1) / slots);
+  };
+  DetailedEstimate e;
+  if (zeroConv) {
+    e.computeUs = streamed(outputBytes());
+    return e;
+  }
   // A weight update pass that runs on the layer's own tensors: what those
   // kernels were measured at.  Matrix-core kernel + ordered sum, two
   // launches, about 350 TFLOP/s of the dense count while the loop waits for
-  // its loads (N = 32, 28 x 28, 128 -> 128, 3 x 3: 24.5 us); depthwise rows +
-  // the sum of the workgroups' tiles (4.5 us) behind one pass over both
-  // tensors (N = 32, 112 x 112, 96 channels, stride 2: 20.4 us).
+  // its loads (N = 32, 28 x 28, 128 -> 128, 3 x 3: 24.5 us, of which the sum
+  // of the chunks' 16.8 MB of fp32 tiles 5.2); depthwise rows + the sum of
+  // the workgroups' tiles (4.5 us) behind one pass over both tensors (N = 32,
+  // 112 x 112, 96 channels, stride 2: 20.4 us).
   if (denseWeightUpdate) {
     const auto &f = denseForward;
     const double flops = 2.0 * f.batch * f.outH * f.outW * f.groups * f.ci *
                          f.co * f.kH * f.kW;
-    return 2 * poplin::kLaunchUs + flops / 3.5e8;
+    const double all = 2 * poplin::kLaunchUs + flops / 3.5e8;
+    e.reductionBytes = mxk::wuTapWorkspaceBytes(f);
+    e.reductionUs = std::min(all / 2, streamed(e.reductionBytes));
+    e.computeUs = all - e.reductionUs;
+    const std::size_t m = std::size_t(f.batch) * f.outH * f.outW;
+    spread(e,
+           std::size_t(f.groups) * f.kH * f.kW * ((f.ci + 127) / 128) *
+               ((f.co + 127) / 128) * ((m + f.chunkPixels - 1) / f.chunkPixels),
+           1);
+    return e;
   }
   if (depthwiseWeightUpdate) {
     const auto &f = depthwiseForward;
@@ -1074,31 +1094,49 @@ double mxconv_plan::estimatedMicroseconds() const {
         (std::size_t(f.batch) * f.inH * f.inW + std::size_t(f.batch) * f.outH *
                                                      f.outW) *
         f.channels * 2;
-    return streamed(bytes) + 4.5;
+    e.computeUs = streamed(bytes);
+    e.reductionUs = 4.5;
+    if (f.dense3x3 == 2) {
+      e.reductionBytes = mxk::depthwiseRowsDeltaWorkspaceBytes(f);
+      spread(e, mxk::depthwiseRowsDeltaLaunchShape(f).workgroups, 1);
+    }
+    return e;
   }
-  double us = 0;
   switch (kernel) {
   case Kernel::GENERIC:
-    return -1.0;
+    e.known = false;
+    return e;
   case Kernel::DEPTHWISE:
-    us = streamed(inputBytes() + outputBytes() + weightPackedBytes());
+    e.computeUs = streamed(inputBytes() + outputBytes() + weightPackedBytes());
+    if (depthwise.dense3x3 == 2)
+      spread(e, mxk::depthwiseRowsLaunchShape(depthwise).workgroups, 1);
     break;
   case Kernel::IGEMM: {
     if (pointwiseOn) {
-      us = streamed(inputBytes() + outputBytes() + weightPackedBytes());
+      e.computeUs =
+          streamed(inputBytes() + outputBytes() + weightPackedBytes());
       // With many input channels a 1x1 layer is as much the matrix cores' as
       // the memory's: N = 32, 28 x 28, 512 -> 512 runs at 710 TFLOP/s
       // (18.5 us where its bytes alone would stream in 10).
       const double flops = 2.0 * pointwise.batch * pointwise.pixels *
                            pointwise.groups * pointwise.inChansPerGroup *
                            pointwise.outChansPerGroup;
-      us = std::max(us, poplin::kLaunchUs + flops / 7.0e8);
+      e.computeUs = std::max(e.computeUs, poplin::kLaunchUs + flops / 7.0e8);
+      spread(e, mxk::pointwiseLaunchShape(pointwise, gfx950::numCUs).workgroups,
+             1);
       break;
     }
+    // (the streaming kernel's K split: 9 us for the fp32 partial tiles' way
+    // out and in again and the second kernel, see estimateStreaming)
+    const double kSplitUs = igemm.splitK > 1 && !igemm.patch ? 9.0 : 0.0;
+    e.reductionUs = kSplitUs;
+    e.reductionBytes = kSplitUs > 0 ? mxk::igemmWorkspaceBytes(igemm) : 0;
     bool weighed = false;
     for (const auto &c : candidates)
-      if (c.chosen)
-        us = c.estimateUs, weighed = true;
+      if (c.chosen) {
+        e.computeUs = c.estimateUs - kSplitUs, weighed = true;
+        spread(e, c.workgroups, c.perCU);
+      }
     if (weighed)
       break;
     const auto &g = igemm;
@@ -1108,18 +1146,28 @@ double mxconv_plan::estimatedMicroseconds() const {
     const std::size_t steps =
         (kPadded / g.blockK + g.splitK - 1) / g.splitK;
     const std::size_t perCU = g.blockN == 64 || g.stages == 2 ? 2 : 1;
-    us = poplin::estimateStreaming(tiles, steps, perCU, g.blockN, g.splitK);
+    double us =
+        poplin::estimateStreaming(tiles, steps, perCU, g.blockN, g.splitK);
     // No kernel is faster than its tensors stream.
     us = std::max(us, streamed(inputBytes() + outputBytes() +
                                weightPackedBytes()));
+    e.computeUs = us - kSplitUs;
+    spread(e, tiles, perCU);
     break;
   }
   }
-  if (paddedInputChans) // the zero-filling copy of the input
-    us += streamed(2 * inputBytes());
+  if (paddedInputChans) { // the zero-filling copy of the input
+    e.rearrangementUs += streamed(2 * inputBytes());
+    e.rearrangementBytes += workspaceBytes - paddedInputOffset;
+  }
   if (outputPadded) // the fill of the output before the kernel
-    us += streamed(outputBytes());
-  return us;
+    e.rearrangementUs += streamed(outputBytes());
+  return e;
+}
+
+double mxconv_plan::estimatedMicroseconds() const {
+  const DetailedEstimate e = detailedEstimate();
+  return e.known ? e.totalUs() : -1.0;
 }
 
 std::string mxconv_plan::describe() const {

@@ -128,6 +128,24 @@ struct mxconv_plan {
   /// estimateConvCost behind reportPlanEstimatedCosts
   /// (lib/poplin/Convolution.cpp:3923-3936).
   double estimatedMicroseconds() const;
+  /// The same estimate taken apart, the role of estimateDetailedConvCost
+  /// behind reportDetailedPlanEstimatedCosts
+  /// (lib/poplin/Convolution.cpp:3953-3962): operands brought into the shape
+  /// the kernel takes (the zero-padded copy of an input whose channels are no
+  /// whole vector, the fill of a padded output field), the convolution
+  /// kernel, and the ordered sum of fp32 partial tiles where K or the pixels
+  /// are split over workgroups; workgroups running side by side and rounds
+  /// of them.
+  struct DetailedEstimate {
+    bool known = true; ///< false: the model does not cover the kernel
+    double rearrangementUs = 0, computeUs = 0, reductionUs = 0;
+    std::size_t rearrangementBytes = 0, reductionBytes = 0;
+    std::size_t parallelSplit = 1, serialSplit = 1;
+    double totalUs() const {
+      return rearrangementUs + computeUs + reductionUs;
+    }
+  };
+  DetailedEstimate detailedEstimate() const;
   /// The shader clock the estimate is converted to cycles with
   /// (MXCONV_ESTIMATE_CLOCK_MHZ): what the chip holds with the matrix cores
   /// of most CUs busy.

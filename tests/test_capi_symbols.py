@@ -24,6 +24,23 @@ def test_header_symbols_are_exported():
         assert hasattr(raw, name), name
 
 
+def test_stamped_twin_exports_the_same_abi_and_its_two_switches():
+    """libmxconv_stamps.so (the library with cycle and wall-clock stamps
+    compiled into the two benchmark kernels, for tests/tools/kernel_stamps.py)
+    is the same C ABI plus one switch per stamped kernel; the product library
+    carries neither switch."""
+    twin = os.path.join(os.path.dirname(pa.library_path()),
+                        "libmxconv_stamps.so")
+    assert os.path.exists(twin), "make -C poplibs_amd stamps"
+    raw = ctypes.CDLL(twin)
+    for name in _declared_symbols():
+        assert hasattr(raw, name), name
+    product = ctypes.CDLL(pa.library_path())
+    for switch in ("mxk_patch_stamp_sink", "mxk_rows_stamp_sink"):
+        assert hasattr(raw, switch)
+        assert not hasattr(product, switch)
+
+
 def test_python_binding_declares_every_symbol():
     assert set(_declared_symbols()) == set(pa.lib()._declared)
 

@@ -550,6 +550,61 @@ def test_plan_estimated_costs():
     assert generic.estimated_costs()[0] == pa.Plan.COST_UNKNOWN
 
 
+def test_plan_detailed_costs():
+    """mxconv_plan_detailed_costs (reportDetailedPlanEstimatedCosts,
+    include/poplin/Convolution.hpp:613-676): the estimate by phase.  The
+    phases add up to the total, the total is what
+    mxconv_plan_estimated_costs returns, and each phase appears exactly where
+    the plan has that step."""
+    def parts(plan):
+        d = plan.detailed_costs()
+        assert d["total"] == plan.estimated_costs()
+        assert sum(d[k][0] for k in ("rearrangement", "compute",
+                                     "reduction")) == d["total"][0]
+        assert d["rearrangement"][1] + d["reduction"][1] <= d["total"][1]
+        assert d["parallelSplit"] >= 1 and d["serialSplit"] >= 1
+        return d
+    # one kernel and nothing else; 224 workgroups in one round
+    d = parts(pa.Plan(make_params(pa.HALF, batch=32, field=(28, 28),
+                                  kernel=(3, 3), ci=128, co=128, pad=1)))
+    assert d["rearrangement"] == (0, 0) and d["reduction"] == (0, 0)
+    assert (d["parallelSplit"], d["serialSplit"]) == (224, 1)
+    # many tiles: rounds of them, no more side by side than the chip holds
+    d = parts(pa.Plan(make_params(pa.HALF, batch=128, field=(56, 56),
+                                  kernel=(3, 3), ci=64, co=64, pad=1)))
+    assert d["serialSplit"] > 1 and d["parallelSplit"] in (256, 512)
+    # K split over workgroups: the second kernel and its fp32 tiles
+    deep = pa.Plan(make_params(pa.HALF, batch=4, field=(14, 14),
+                               kernel=(3, 3), ci=256, co=256, pad=1),
+                   {"planConstraints": '{"gfx950": {"patch": 0}}'})
+    assert "K split into parts" in deep.describe()
+    d = parts(deep)
+    assert d["reduction"][0] == 9 * 2100
+    assert d["reduction"][1] == deep.buffer_bytes(capi.BUF_WORKSPACE) > 0
+    # three input channels: copied into whole vectors first
+    stem = pa.Plan(make_params(pa.HALF, batch=8, field=(56, 56),
+                               kernel=(3, 3), ci=3, co=64, pad=1))
+    assert "generic direct" not in stem.describe()
+    d = parts(stem)
+    assert d["rearrangement"][0] > 2.0 * 2100  # at least a launch
+    assert d["rearrangement"][1] == stem.buffer_bytes(capi.BUF_WORKSPACE) > 0
+    assert d["compute"][0] > 0
+    # the weight update pass of a dense layer on its own tensors: the matrix
+    # core kernel, then the ordered sum of the chunks' tiles
+    wu = pa.WeightUpdatePlan(make_params(pa.HALF, batch=32, field=(28, 28),
+                                         kernel=(3, 3), ci=128, co=128,
+                                         pad=1))
+    d = parts(wu)
+    assert d["reduction"][0] > 0 and d["reduction"][1] > 0
+    assert d["compute"][0] > d["reduction"][0]
+    # outside the cost model
+    generic = pa.Plan(make_params(pa.FLOAT, pa.FLOAT, batch=1, field=(5, 5),
+                                  kernel=(3, 3), ci=3, co=5))
+    d = generic.detailed_costs()
+    assert all(d[k][0] == pa.Plan.COST_UNKNOWN
+               for k in ("rearrangement", "compute", "reduction", "total"))
+
+
 def test_planner_weighs_tilings_and_reports_them():
     """The matrix-core plan lists the tilings it weighed with their estimated
     times, picks the cheapest, and says how many CUs the launch occupies;

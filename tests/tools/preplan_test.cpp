@@ -180,6 +180,79 @@ int main() {
       CHECK(costs.cycles == poplin::PlanCosts::unknown);
   }
 
+  // the same estimate by phase (include/poplin/Convolution.hpp:613-676)
+  {
+    using poplin::internal::DetailedPlanCosts;
+    auto sumOfPhases = [](const DetailedPlanCosts &d) {
+      std::size_t sum = 0;
+      d.apply([&](const poplin::PlanCosts &c) { sum += c.cycles; },
+              /*includeTotal=*/false);
+      return sum;
+    };
+    // one kernel, nothing else: all of it is compute, 256 workgroups at once
+    const DetailedPlanCosts plain =
+        poplin::internal::reportDetailedPlanEstimatedCosts(c2, fwd, &cache);
+    CHECK(plain.total.cycles ==
+          poplin::reportPlanEstimatedCosts(c2, fwd, &cache).cycles);
+    CHECK(plain.compute.cycles == plain.total.cycles);
+    CHECK(plain.rearrangement.cycles == 0 && plain.reduction.cycles == 0);
+    CHECK(sumOfPhases(plain) == plain.total.cycles);
+    CHECK(plain.parallelSplit >= 1 && plain.parallelSplit <= 2 * 256);
+    CHECK(plain.serialSplit >= 1);
+    // a K split: the sum of the partial tiles is the reduction and owns the
+    // temporary memory
+    const ConvParams deep = conv(poplar::HALF, 8, 28, 3, 128, 128);
+    const DetailedPlanCosts split =
+        poplin::internal::reportDetailedPlanEstimatedCosts(deep, fwd);
+    const poplin::PlanCosts whole = poplin::reportPlanEstimatedCosts(deep, fwd);
+    CHECK(split.total.cycles == whole.cycles);
+    CHECK(split.total.memory == whole.memory);
+    CHECK(sumOfPhases(split) == split.total.cycles);
+    if (planText(deep, fwd, nullptr).find("K split into parts") !=
+        std::string::npos) {
+      CHECK(split.reduction.cycles > 0);
+      CHECK(split.reduction.memory == whole.memory);
+    }
+    // three input channels are copied into whole vectors first
+    const ConvParams stem = conv(poplar::HALF, 8, 56, 3, 3, 64);
+    const DetailedPlanCosts padded =
+        poplin::internal::reportDetailedPlanEstimatedCosts(stem, fwd);
+    if (planText(stem, fwd, nullptr).find("generic direct") ==
+        std::string::npos) {
+      CHECK(padded.rearrangement.cycles > 0);
+      CHECK(padded.rearrangement.memory > 0);
+      CHECK(padded.rearrangement.memory <= padded.total.memory);
+      CHECK(sumOfPhases(padded) == padded.total.cycles);
+    }
+    // text form: two numbers, then a pair per phase and the total; reads back
+    std::stringstream ss;
+    ss << split;
+    std::size_t lines = 0;
+    for (char ch : ss.str())
+      lines += ch == '\n';
+    CHECK(lines == 14);
+    DetailedPlanCosts back;
+    ss >> back;
+    CHECK(back.parallelSplit == split.parallelSplit);
+    CHECK(back.serialSplit == split.serialSplit);
+    CHECK(back.compute.cycles == split.compute.cycles);
+    CHECK(back.reduction.memory == split.reduction.memory);
+    CHECK(back.total.cycles == split.total.cycles);
+    // serialSplitOnly visits the eight per-slice phases
+    std::size_t visited = 0;
+    split.apply([&](const poplin::PlanCosts &) { ++visited; }, false, true);
+    CHECK(visited == 8);
+    // outside the cost model
+    const ConvParams odd = conv(poplar::FLOAT, 1, 5, 3, 3, 5);
+    if (planText(odd, none, nullptr).find("generic direct") !=
+        std::string::npos) {
+      const DetailedPlanCosts d =
+          poplin::internal::reportDetailedPlanEstimatedCosts(odd, none);
+      CHECK(d.total.cycles == poplin::PlanCosts::unknown);
+      CHECK(d.compute.cycles == poplin::PlanCosts::unknown);
+    }
+  }
+
   if (failures == 0)
     std::cout << "preplan_test: all checks passed\n";
   return failures == 0 ? 0 : 1;
