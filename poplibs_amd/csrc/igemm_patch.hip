@@ -233,9 +233,20 @@ loadPatch(const PatchArgs &a, const char *__restrict__ in, char *lds, int wave,
   __builtin_amdgcn_s_barrier();
   MXK_STAMP(5); // everybody's has
   behind();
-  for (; next < blocks; next += kPatchWaves) {
-    const uint32_t s = a.divRowLoads(next);
-    loadColumns(s, next - s * a.rowLoads);
+  // What is left of the later slices goes to the older wave of each SIMD
+  // (waves 0 .. kWavesN - 1): it wins the MFMA slots, is through its k-steps
+  // long before the younger one and waits for it at the end, while the
+  // kernel's end waits for the younger one - which so enters the k loop
+  // without standing in the queue of the vector memory path (22 cycles per
+  // load of 1 KB: 1 600 cycles for three slices of a 112-pixel tile).
+  // Issued so far: slice 0's blocks and one block per wave without any.
+  if (wave < kWavesN) {
+    const uint32_t issued =
+        a.rowLoads > uint32_t(kPatchWaves) ? a.rowLoads : uint32_t(kPatchWaves);
+    for (next = issued + wave; next < blocks; next += kWavesN) {
+      const uint32_t s = a.divRowLoads(next);
+      loadColumns(s, next - s * a.rowLoads);
+    }
   }
 }
 
