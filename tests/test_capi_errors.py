@@ -77,6 +77,38 @@ def test_plan_describe_short_buffer():
     assert len(buf.value) <= 15  # still terminated
 
 
+def test_plan_queries_refuse_null_arguments():
+    """The calls that only read a plan (costs, detailed costs, constraints)
+    check their pointers like the launching ones."""
+    plan = _split_k_plan()
+    L = pa.lib()
+    costs = capi.DetailedCosts()
+    u64 = ctypes.c_uint64()
+    need = ctypes.c_size_t()
+    assert L.mxconv_plan_detailed_costs(None, ctypes.byref(costs)) \
+        == Status.NULL_ARGUMENT
+    assert L.mxconv_plan_detailed_costs(plan._h, None) == Status.NULL_ARGUMENT
+    assert L.mxconv_plan_estimated_costs(None, ctypes.byref(u64),
+                                         ctypes.byref(u64)) \
+        == Status.NULL_ARGUMENT
+    assert L.mxconv_plan_estimated_costs(plan._h, None, ctypes.byref(u64)) \
+        == Status.NULL_ARGUMENT
+    assert L.mxconv_plan_constraints(None, None, 0, ctypes.byref(need)) \
+        == Status.NULL_ARGUMENT
+    # and a short buffer for the constraints document reports its size
+    assert L.mxconv_plan_constraints(plan._h, None, 0, ctypes.byref(need)) \
+        == Status.OK
+    buf = ctypes.create_string_buffer(8)
+    got = ctypes.c_size_t()
+    assert L.mxconv_plan_constraints(plan._h, buf, 8, ctypes.byref(got)) \
+        == Status.BUFFER_TOO_SMALL
+    assert got.value == need.value > 8
+    whole = ctypes.create_string_buffer(need.value)
+    assert L.mxconv_plan_constraints(plan._h, whole, need.value,
+                                     ctypes.byref(got)) == Status.OK
+    assert json.loads(whole.value)["gfx950"]["patch"] == 0
+
+
 def test_weight_update_workspace_and_type_checks():
     fwd = make_params(pa.HALF, batch=8, field=(14, 14), kernel=(3, 3), ci=64,
                       co=64, pad=1)
