@@ -21,5 +21,11 @@ namespace poplin {
 void preplan(const std::set<ConvPlanParams> &convs,
              const std::set<MatMulPlanParams> &matmuls, PlanningCache &cache);
 
+/// The older name for planning convolutions only
+/// (include/poplin/Convolution.hpp:386-401 of PopLibs, deprecated there in
+/// favour of preplan).
+void preplanConvolutions(const std::set<ConvPlanParams> &convs,
+                         PlanningCache &cache);
+
 } // namespace poplin
 #endif

@@ -105,6 +105,18 @@ std::uint64_t getFwdFlops(const ConvParams &params);
 std::uint64_t getBwdFlops(const ConvParams &params);
 std::uint64_t getWuFlops(const ConvParams &params);
 
+/// Shader cycles of a pass if every matrix core of the chip retired its peak
+/// number of multiply-accumulates in every cycle and nothing else took time
+/// (include/poplin/Convolution.hpp:34-77 of PopLibs: MACs / (MACs per cycle and
+/// tile x tiles); here MACs / (MACs per cycle and SIMD x 4 SIMDs x 256 CUs)).
+/// Per SIMD and cycle gfx950's dense MFMA retires 512 fp16, 1 024 fp8 and 32
+/// fp32 MACs - the 2.5 / 5.0 PFLOP/s and 157.3 TFLOP/s peaks at 2.4 GHz.
+/// An optimistic figure for efficiency estimates; all three passes perform
+/// the forward pass's MACs.  `params` are the forward parameters.
+double getFwdPerfectCycleCount(const ConvParams &params);
+double getBwdPerfectCycleCount(const ConvParams &params);
+double getWuPerfectCycleCount(const ConvParams &params);
+
 /// Weights [convGroups][outChansPerGroup][inChansPerGroup][kernel...], held
 /// packed for the plan of (params, options).
 DeviceTensor createWeights(const ConvParams &params,
@@ -146,6 +158,18 @@ void convolutionWithOutput(const DeviceTensor &in, const DeviceTensor &weights,
 /// the external layout (include/poplin/Convolution.hpp:407-412 of PopLibs).
 void weightsTransposeChansFlipXY(const DeviceTensor &weightsIn,
                                  const DeviceTensor &weightsOut, Stream &prog);
+
+/// The weights of a fully connected layer arranged for its backward pass
+/// (include/poplin/Convolution.hpp:695-711 of PopLibs).  `params` are the
+/// backward pass's, a convolution over one field dimension (anything else
+/// throws poputil::poplibs_error, lib/poplin/Convolution.cpp:3849-3852);
+/// `weights` are the forward pass's [G][params.inChans][params.outChans][k] in
+/// the external layout.  Returns [G][params.outChans][params.inChans][k] -
+/// the channel axes exchanged, nothing flipped - packed for the plan of
+/// (params, options), as createWeights would hand it out.
+DeviceTensor fullyConnectedWeightTranspose(
+    const DeviceTensor &weights, const ConvParams &params, Stream &prog,
+    const poplar::OptionFlags &options = {}, PlanningCache *cache = nullptr);
 
 /// Gradient with respect to the forward weights, [G][Co][Ci][kernel...] in the
 /// external layout and the forward output type, from the gradient with

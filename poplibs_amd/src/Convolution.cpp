@@ -183,6 +183,28 @@ std::uint64_t getFwdFlops(const ConvParams &params) {
   return flops;
 }
 
+namespace {
+double perfectCycleCount(const ConvParams &params) {
+  // Dense MFMA, MACs per cycle and SIMD: 16x16x32 fp16 in 16 cycles,
+  // 16x16x128 fp8 in 32, 32x32x2 fp32 in 64.
+  const double perSimd = params.inputType == poplar::FLOAT     ? 32.0
+                         : params.inputType == poplar::QUARTER ? 1024.0
+                                                               : 512.0;
+  const double perChip = perSimd * 4 * poplar::Target::gfx950().getNumComputeUnits();
+  return double(getFwdFlops(params) / 2) / perChip;
+}
+} // namespace
+
+double getFwdPerfectCycleCount(const ConvParams &params) {
+  return perfectCycleCount(params);
+}
+double getBwdPerfectCycleCount(const ConvParams &params) {
+  return perfectCycleCount(params);
+}
+double getWuPerfectCycleCount(const ConvParams &params) {
+  return perfectCycleCount(params);
+}
+
 DeviceTensor createWeights(const ConvParams &params,
                            const poplar::OptionFlags &options,
                            PlanningCache *cache) {
@@ -391,6 +413,60 @@ void weightsTransposeChansFlipXY(const DeviceTensor &weightsIn,
                                                streamOf(prog)));
 }
 
+DeviceTensor fullyConnectedWeightTranspose(const DeviceTensor &weights,
+                                           const ConvParams &params,
+                                           Stream &prog,
+                                           const poplar::OptionFlags &options,
+                                           PlanningCache *cache) {
+  if (params.getNumFieldDims() != 1)
+    throw poputil::poplibs_error(
+        "fullyConnectedWeightTranspose() expects a 1-d convolution");
+  const std::vector<std::size_t> fwdShape{
+      params.numConvGroups, params.inputChannelsPerConvGroup,
+      params.outputChannelsPerConvGroup, params.kernelShape[0]};
+  if (weights.layout() != DeviceTensor::Layout::External ||
+      weights.shape() != fwdShape || weights.elementType() != params.inputType)
+    throw poputil::poplibs_error(
+        "fullyConnectedWeightTranspose: expected the forward pass's weights, "
+        "[G][params.inChans][params.outChans][k] in the external layout and "
+        "the parameters' input type");
+  auto plan = getPlan(params, options, cache);
+  const std::vector<std::size_t> bwdShape{fwdShape[0], fwdShape[2], fwdShape[1],
+                                          fwdShape[3]};
+  DeviceTensor swapped(weights.elementType(), bwdShape,
+                       DeviceTensor::Layout::External, weights.bytes());
+  swapped.metadata = weights.metadata;
+  const std::size_t k = fwdShape[3];
+  if (k == 1) {
+    check(mxconv_transpose_grouped_matrix(
+        weights.elementType().id(), fwdShape[0], fwdShape[1], fwdShape[2],
+        weights.data(), swapped.data(), streamOf(prog)));
+  } else {
+    // The channel axes exchanged with the taps flipped, then every
+    // (group, channel pair)'s taps flipped back as a kernel of its own.
+    DeviceTensor flipped(weights.elementType(), bwdShape,
+                         DeviceTensor::Layout::External, weights.bytes());
+    weightsTransposeChansFlipXY(weights, flipped, prog);
+    ConvParams each(weights.elementType(), 1, {k}, {k}, 1, 1,
+                    fwdShape[0] * fwdShape[1] * fwdShape[2]);
+    mxconv_params c;
+    each.toC(c);
+    check(mxconv_weights_transpose_chans_flip_xy(&c, flipped.data(),
+                                                 swapped.data(),
+                                                 streamOf(prog)));
+    prog.synchronize(); // `flipped` is released on leaving this block
+  }
+  DeviceTensor packed(weights.elementType(), bwdShape,
+                      DeviceTensor::Layout::PackedWeights,
+                      bufferBytes(plan->plan, MXCONV_BUFFER_WEIGHTS_PACKED));
+  packed.metadata = weights.metadata;
+  packed.packedFor = plan;
+  check(mxconv_pack_weights(plan->plan, swapped.data(), packed.data(),
+                            streamOf(prog)));
+  prog.synchronize(); // `swapped` is released on return
+  return packed;
+}
+
 DeviceTensor convolution(const DeviceTensor &in, const DeviceTensor &weights,
                          const ConvParams &params,
                          bool transposeAndFlipWeights, Stream &prog,
@@ -481,6 +557,11 @@ reportDetailedPlanEstimatedCosts(const ConvParams &params,
 }
 
 } // namespace internal
+
+void preplanConvolutions(const std::set<ConvPlanParams> &convs,
+                         PlanningCache &cache) {
+  preplan(convs, {}, cache);
+}
 
 void preplan(const std::set<ConvPlanParams> &convs,
              const std::set<MatMulPlanParams> &matmuls, PlanningCache &cache) {

@@ -70,6 +70,21 @@ def test_preplan_and_estimated_costs_host_checks():
     assert "all checks passed" in r.stdout
 
 
+@pytest.mark.gpu
+def test_fully_connected_weight_transpose_on_the_device():
+    """poplin::fullyConnectedWeightTranspose (include/poplin/Convolution.hpp:
+    695-711): the forward weights with the channel axes exchanged and nothing
+    flipped, packed for the backward pass's plan - read back through
+    readTensor and compared element by element with the exchange done on the
+    host, for kernels of one and three taps, two groups, half and float; the
+    result is accepted by convolution() of the backward parameters."""
+    tool = os.path.join(ROOT, "tests", "tools", "preplan_test")
+    r = subprocess.run([tool, "--device"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "device checks passed" in r.stdout
+
+
 def test_plan_constraints_and_options_are_validated():
     base = ["--input-channels", "16", "--output-channels", "16", "--field",
             "{8,8}", "--kernel-size", "3", "--plan-only"]

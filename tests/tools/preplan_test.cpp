@@ -8,9 +8,11 @@
 #include "poplar/exceptions.hpp"
 #include "poputil/exceptions.hpp"
 
+#include <cstring>
 #include <iostream>
 #include <sstream>
 #include <string>
+#include <vector>
 
 using poplin::ConvParams;
 
@@ -43,7 +45,106 @@ static std::string planText(const ConvParams &p,
   return os.str();
 }
 
-int main() {
+// fullyConnectedWeightTranspose on the device against the same exchange of
+// axes done on the host: kernels of one tap (a fully connected layer) and of
+// three (nothing may be flipped), several groups, half and float.
+static int transposeOnDevice() {
+  poplin::Stream prog;
+  for (const auto type : {poplar::HALF, poplar::FLOAT})
+    for (const std::size_t k : {std::size_t(1), std::size_t(3)}) {
+      const std::size_t g = 2, ci = 48, co = 80; // of the backward pass
+      ConvParams bwd(type, type, 4, {8}, {k}, ci, co, g);
+      const std::size_t n = g * ci * co * k;
+      const std::size_t es = type == poplar::HALF ? 2 : 4;
+      // forward weights [g][ci][co][k]: element (a, i, o, t) holds a small
+      // integer both types represent exactly
+      std::vector<float> fwdW(n);
+      for (std::size_t i = 0; i != n; ++i)
+        fwdW[i] = float(int(i * 7919 % 31) - 15);
+      std::vector<unsigned char> raw(n * es);
+      for (std::size_t i = 0; i != n; ++i) {
+        if (type == poplar::FLOAT) {
+          std::memcpy(&raw[i * 4], &fwdW[i], 4);
+        } else { // integers below 2048 are exact halves
+          const float v = fwdW[i];
+          unsigned u;
+          std::memcpy(&u, &v, 4);
+          const unsigned sign = (u >> 16) & 0x8000u;
+          const int e = int((u >> 23) & 0xff) - 127 + 15;
+          const unsigned short h =
+              v == 0.0f ? 0
+                        : (unsigned short)(sign | unsigned(e << 10) |
+                                           ((u >> 13) & 0x3ffu));
+          std::memcpy(&raw[i * 2], &h, 2);
+        }
+      }
+      poplin::DeviceTensor w(type, {g, ci, co, k},
+                             poplin::DeviceTensor::Layout::External, n * es);
+      poplin::writeTensor(w, raw.data(), prog);
+      const poplin::DeviceTensor t =
+          poplin::fullyConnectedWeightTranspose(w, bwd, prog);
+      CHECK(t.layout() == poplin::DeviceTensor::Layout::PackedWeights);
+      CHECK((t.shape() == std::vector<std::size_t>{g, co, ci, k}));
+      // The same exchange of axes on the host, given to convolution() in the
+      // external layout, must give the bit-identical output: both runs pack
+      // for the same plan, so any misplaced element shows.
+      std::vector<unsigned char> swappedRaw(n * es);
+      for (std::size_t a = 0; a != g; ++a)
+        for (std::size_t o = 0; o != co; ++o)
+          for (std::size_t i = 0; i != ci; ++i)
+            for (std::size_t tap = 0; tap != k; ++tap)
+              std::memcpy(
+                  &swappedRaw[(((a * co + o) * ci + i) * k + tap) * es],
+                  &raw[(((a * ci + i) * co + o) * k + tap) * es], es);
+      poplin::DeviceTensor expected(type, {g, co, ci, k},
+                                    poplin::DeviceTensor::Layout::External,
+                                    n * es);
+      poplin::writeTensor(expected, swappedRaw.data(), prog);
+      // input: every element a small integer (+-1, +-2 pattern)
+      poplin::DeviceTensor in = poplin::createInput(bwd);
+      const std::size_t inElems = in.numElements();
+      std::vector<unsigned char> inRaw(inElems * es);
+      for (std::size_t i = 0; i != inElems; ++i) {
+        const float v = float(int(i * 31 % 5) - 2);
+        if (type == poplar::FLOAT) {
+          std::memcpy(&inRaw[i * 4], &v, 4);
+        } else {
+          const unsigned short table[5] = {0xc000, 0xbc00, 0x0000, 0x3c00,
+                                           0x4000}; // -2 -1 0 1 2
+          std::memcpy(&inRaw[i * 2], &table[i * 31 % 5], 2);
+        }
+      }
+      poplin::writeTensor(in, inRaw.data(), prog, bwd);
+      const poplin::DeviceTensor viaArranged =
+          poplin::convolution(in, t, bwd, false, prog);
+      const poplin::DeviceTensor viaHost =
+          poplin::convolution(in, expected, bwd, false, prog);
+      const std::size_t outBytes = viaHost.numElements() * es;
+      std::vector<unsigned char> got(outBytes), want(outBytes);
+      poplin::readTensor(viaArranged, got.data(), prog, bwd);
+      poplin::readTensor(viaHost, want.data(), prog, bwd);
+      prog.synchronize();
+      CHECK(std::memcmp(got.data(), want.data(), outBytes) == 0);
+      // ... and is not all zeros
+      bool any = false;
+      for (unsigned char b : want)
+        any |= b != 0;
+      CHECK(any);
+    }
+  if (failures == 0)
+    std::cout << "preplan_test: device checks passed\n";
+  return failures == 0 ? 0 : 1;
+}
+
+int main(int argc, char **argv) {
+  if (argc > 1 && std::string(argv[1]) == "--device") {
+    try {
+      return transposeOnDevice();
+    } catch (const std::exception &e) {
+      std::cerr << "preplan_test --device: " << e.what() << "\n";
+      return 1;
+    }
+  }
   const poplar::OptionFlags fwd{{"pass", "TRAINING_FWD"}};
   const poplar::OptionFlags wu{{"pass", "TRAINING_WU"}};
   const poplar::OptionFlags none;
@@ -251,6 +352,61 @@ int main() {
       CHECK(d.total.cycles == poplin::PlanCosts::unknown);
       CHECK(d.compute.cycles == poplin::PlanCosts::unknown);
     }
+  }
+
+  // perfect cycle counts: MACs over what the matrix cores retire per cycle
+  // (include/poplin/Convolution.hpp:34-77)
+  {
+    const double macs = 32.0 * 28 * 28 * 128 * 128 * 9; // c2, padding MACs in
+    const double perfect = poplin::getFwdPerfectCycleCount(c2);
+    CHECK(perfect == double(poplin::getFwdFlops(c2) / 2) / (512.0 * 4 * 256));
+    CHECK(perfect < macs / (512.0 * 4 * 256) && perfect > 6000);
+    CHECK(poplin::getBwdPerfectCycleCount(c2) == perfect);
+    CHECK(poplin::getWuPerfectCycleCount(c2) == perfect);
+    // fp8 retires twice, fp32 a sixteenth of fp16's MACs per cycle
+    const ConvParams q = conv(poplar::QUARTER, 32, 28, 3, 128, 128);
+    ConvParams f = c2;
+    f.inputType = f.outputType = poplar::FLOAT;
+    CHECK(poplin::getFwdPerfectCycleCount(q) * 2 == perfect);
+    CHECK(poplin::getFwdPerfectCycleCount(f) == perfect * 16);
+    // against the estimate: no plan is faster than perfect
+    CHECK(double(poplin::reportPlanEstimatedCosts(c2, fwd, &cache).cycles) >
+          perfect);
+  }
+
+  // preplanConvolutions, the older name: convolutions only, same cache
+  {
+    poplin::PlanningCache old;
+    poplin::preplanConvolutions(convs, old);
+    CHECK(old.size() == 5);
+    poplin::preplanConvolutions({}, old);
+    CHECK(old.size() == 5);
+  }
+
+  // fullyConnectedWeightTranspose refuses what the reference refuses, before
+  // anything touches a device
+  {
+    bool threw = false;
+    try {
+      poplin::Stream defaultStream(nullptr);
+      poplin::fullyConnectedWeightTranspose(poplin::DeviceTensor(), c2,
+                                            defaultStream);
+    } catch (const poputil::poplibs_error &e) {
+      threw = std::string(e.what()).find("expects a 1-d convolution") !=
+              std::string::npos;
+    }
+    CHECK(threw);
+    threw = false;
+    try {
+      poplin::Stream defaultStream(nullptr);
+      ConvParams fc(poplar::HALF, poplar::HALF, 4, {1}, {1}, 64, 32, 1);
+      poplin::fullyConnectedWeightTranspose(poplin::DeviceTensor(), fc,
+                                            defaultStream);
+    } catch (const poputil::poplibs_error &e) {
+      threw = std::string(e.what()).find("forward pass's weights") !=
+              std::string::npos;
+    }
+    CHECK(threw);
   }
 
   if (failures == 0)
