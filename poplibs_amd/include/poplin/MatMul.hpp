@@ -153,5 +153,20 @@ std::set<ConvPlanParams>
 matMulGetConvPlanParams(const std::set<MatMulPlanParams> &matmuls,
                         MatMulToConvOptions &matmulToConvOpts);
 
+namespace matmul {
+/// The older name of the planning cache (include/poplin/MatMul.hpp:682-688 of
+/// PopLibs, deprecated there in favour of poplin::PlanningCache).
+class PlanningCache : public poplin::PlanningCache {
+public:
+  poplin::PlanningCache &getImpl() { return *this; }
+};
+} // namespace matmul
+
+/// The older name for planning matrix multiplications only
+/// (include/poplin/MatMul.hpp:665-672 of PopLibs, deprecated there in favour
+/// of preplan).
+void preplanMatMuls(const std::set<MatMulPlanParams> &matmuls,
+                    matmul::PlanningCache &cache);
+
 } // namespace poplin
 #endif

@@ -563,6 +563,11 @@ void preplanConvolutions(const std::set<ConvPlanParams> &convs,
   preplan(convs, {}, cache);
 }
 
+void preplanMatMuls(const std::set<MatMulPlanParams> &matmuls,
+                    matmul::PlanningCache &cache) {
+  preplan({}, matmuls, cache.getImpl());
+}
+
 void preplan(const std::set<ConvPlanParams> &convs,
              const std::set<MatMulPlanParams> &matmuls, PlanningCache &cache) {
   if (convs.empty() && matmuls.empty())

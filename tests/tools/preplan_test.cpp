@@ -383,6 +383,14 @@ int main(int argc, char **argv) {
     CHECK(old.size() == 5);
   }
 
+  // ... and preplanMatMuls with the older cache type
+  {
+    poplin::matmul::PlanningCache old;
+    poplin::preplanMatMuls(matmuls, old);
+    CHECK(old.size() == 2);
+    CHECK(&old.getImpl() == &old);
+  }
+
   // fullyConnectedWeightTranspose refuses what the reference refuses, before
   // anything touches a device
   {
