@@ -274,9 +274,11 @@ mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
  * where K or the pixels are split over workgroups).  Each phase: cycles as in
  * mxconv_plan_estimated_costs and the temporary bytes it owns.
  * parallel_split: workgroups that run side by side (at most the CUs times
- * the workgroups a CU holds); serial_split: rounds of them.  The phases'
- * cycles add up to total.cycles, which is what mxconv_plan_estimated_costs
- * returns; every cycles field is MXCONV_COST_UNKNOWN where that is.
+ * the workgroups a CU holds); serial_split: rounds of them (both 1 where the
+ * model prices a kernel by its bytes alone: fills, the tiled depthwise
+ * kernels).  The phases' cycles add up to total.cycles, which is what
+ * mxconv_plan_estimated_costs returns; every cycles field is
+ * MXCONV_COST_UNKNOWN where that is.
  * Touches no GPU. */
 typedef struct mxconv_phase_cost {
   uint64_t cycles;
