@@ -125,6 +125,31 @@ def test_patch_16_pixel_blocks_pm1_exact(oracle, kw):
     _run(oracle, p, 16, 0, dist="pm1", options=FORCED16)
 
 
+# Who loads which part of the patch: slice 0 goes to all eight waves before
+# the first barrier, the later slices to the older wave of each SIMD behind
+# it.  The cases: more column blocks per row than waves (a 56-wide field: ten
+# of them), a single block per row with eight slices, and a row of three
+# blocks with four slices - each with a tile height that makes the rows of
+# the patch ragged against the tiles.
+@pytest.mark.parametrize("kw,tile_pixels", [
+    (dict(batch=2, field=(12, 56), kernel=(3, 3), ci=128, co=128, pad=1), 0),
+    (dict(batch=2, field=(12, 56), kernel=(3, 3), ci=128, co=128, pad=1), 112),
+    (dict(batch=6, field=(4, 4), kernel=(3, 3), ci=256, co=64, pad=1), 48),
+    (dict(batch=3, field=(9, 17), kernel=(3, 3), ci=256, co=136, pad=1), 0),
+    (dict(batch=3, field=(9, 17), kernel=(3, 3), ci=256, co=136, pad=1), 80),
+])
+def test_patch_later_slices_loaded_by_the_older_waves(oracle, kw, tile_pixels):
+    """tile_pixels 0: the 32-pixel-block kernel, else the 16-pixel-block one
+    with tiles of that many pixels."""
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    print("case", p, tile_pixels, flush=True)
+    opts = _forced16(tile_pixels) if tile_pixels else FORCED
+    _, plan = _run(oracle, p, 18, 0, dist="pm1", options=opts,
+                   return_plan=True)
+    assert PATCH in plan.describe()
+    assert (BLOCKS16 in plan.describe()) == bool(tile_pixels)
+
+
 def test_patch_16_pixel_blocks_refuse_one_tap():
     p = make_params(pa.HALF, **CASES[7])
     assert PATCH not in pa.Plan(p, FORCED16).describe()
