@@ -1,6 +1,7 @@
 #!/usr/bin/env python3
-"""Extracts the reference's ctest invocations of `single_conv_layer` into a
-JSON fixture (data only: test names and argument lists).
+"""Extracts the reference's ctest invocations of `single_conv_layer` and
+`general_matrix_multiply` into JSON fixtures (data only: test names and
+argument lists).
 
     python3 tests/golden/extract_ctest_matrix.py [/root/reference]
 
@@ -8,9 +9,9 @@ reads <reference>/tests/poplin/CMakeLists.txt, interprets the few CMake
 commands that file uses around its tests (set, foreach / endforeach over
 literal lists and RANGE, if / elseif / else / endif - every branch is taken,
 a test's platform conditions do not matter here) and writes
-tests/golden/single_conv_layer_ctest_matrix.json: one record per
-add_multitarget_test / add_test whose COMMAND is single_conv_layer, with
-${VAR} references substituted.  Plan-constraint files the invocations name
+tests/golden/<tool>_ctest_matrix.json for each of the two tools: one record
+per add_multitarget_test / add_test whose COMMAND is that tool, with ${VAR}
+references substituted.  Plan-constraint files the invocations name
 (tests/poplin/json/*.json: data the reference holds) are copied next to the
 fixture and the arguments rewritten to "@golden/<file>".  Runs only where the
 reference tree is present; the GPU tests read the fixture, never the tree.
@@ -22,6 +23,7 @@ import shutil
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+TOOLS = ("single_conv_layer", "general_matrix_multiply")
 REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
 SRC = os.path.join(REF, "tests", "poplin", "CMakeLists.txt")
 
@@ -134,7 +136,7 @@ def run(cmds, env, tests):
             a = [substitute(x, env) for x in args]
             if "COMMAND" in a and "NAME" in a:
                 k = a.index("COMMAND")
-                if k + 1 < len(a) and a[k + 1] == "single_conv_layer":
+                if k + 1 < len(a) and a[k + 1] in TOOLS:
                     rest = a[k + 2:]
                     stops = {"VARIANTS", "LABELS", "ALLOW_SKIP", "TEST_IPUMODEL",
                              "PROPERTIES", "WORKING_DIRECTORY", "NAME"}
@@ -144,7 +146,8 @@ def run(cmds, env, tests):
                             break
                         argv.append(x)
                     tests.append({"name": a[a.index("NAME") + 1],
-                                  "line": line, "args": argv})
+                                  "tool": a[k + 1], "line": line,
+                                  "args": argv})
         i += 1
 
 
@@ -172,13 +175,16 @@ def main():
         names[t["name"]] = names.get(t["name"], 0) + 1
         if names[t["name"]] > 1:
             t["name"] += f"#{names[t['name']]}"
-    out = os.path.join(HERE, "single_conv_layer_ctest_matrix.json")
-    with open(out, "w") as f:
-        json.dump({"source": "tests/poplin/CMakeLists.txt",
-                   "tool": "single_conv_layer", "tests": tests}, f, indent=1)
-        f.write("\n")
-    print(f"{len(tests)} invocations -> {out}; constraint files copied: "
-          f"{sorted(copied)}")
+    for tool in TOOLS:
+        mine = [{k: v for k, v in t.items() if k != "tool"}
+                for t in tests if t["tool"] == tool]
+        out = os.path.join(HERE, tool + "_ctest_matrix.json")
+        with open(out, "w") as f:
+            json.dump({"source": "tests/poplin/CMakeLists.txt",
+                       "tool": tool, "tests": mine}, f, indent=1)
+            f.write("\n")
+        print(f"{len(mine)} invocations -> {out}")
+    print(f"constraint files copied: {sorted(copied)}")
 
 
 if __name__ == "__main__":

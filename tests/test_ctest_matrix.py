@@ -1,4 +1,5 @@
-"""The reference's whole ctest matrix for its `single_conv_layer` tool, carried
+"""The reference's whole ctest matrix for its `single_conv_layer` tool (and, at
+the end of this file, for `general_matrix_multiply`), carried
 as a fixture: every add_multitarget_test(... COMMAND single_conv_layer ...) of
 tests/poplin/CMakeLists.txt:986-3500 with its foreach loops expanded
 (tests/golden/single_conv_layer_ctest_matrix.json, written by
@@ -122,3 +123,63 @@ def test_reference_ctest_case(matrix_results, name):
     text = "\n".join(out[name])
     assert results[name] == 0, text[-3000:]
     assert "Validation passed" in text
+
+
+# ---------------------------------------------------------------------------
+# general_matrix_multiply: the 39 invocations of the same CMakeLists.txt
+# (:519-985), through this build's tool of that name.  The tool compares with
+# a host matrix product itself; plan constraints written for the IPU planner
+# (serial splits of the output or input channels) are validated and have no
+# effect here.
+
+GEMM_TOOL = os.path.join(ROOT, "tests", "tools", "general_matrix_multiply")
+with open(os.path.join(GOLDEN,
+                       "general_matrix_multiply_ctest_matrix.json")) as _f:
+    GEMM_MATRIX = json.load(_f)["tests"]
+
+# Options of the reference tool (tools/general_matrix_multiply.cpp:120-225).
+GEMM_REFERENCE_OPTIONS = {
+    "help", "compile-only", "device-type", "profile", "profile-dir",
+    "ignore-data", "m", "k", "n", "g", "data-type", "input-type",
+    "output-type", "partials-type", "fp8-scale-A", "fp8-scale-B",
+    "fp8-format-A", "fp8-format-B", "alpha", "beta", "left-matrix-op",
+    "right-matrix-op", "tolerance", "tiles-per-ipu",
+    "available-memory-proportion", "enable-fast-reduce", "report-plan",
+    "show-execution-steps", "show-var-storage", "ipus", "plan-constraints",
+    "num-executions", "remap-output-tensor", "plan-constraints-file",
+    "use-create-output"}
+
+
+def test_gemm_fixture_is_the_whole_matrix():
+    assert len(GEMM_MATRIX) == 39
+    assert len({t["name"] for t in GEMM_MATRIX}) == 39
+    used = set().union(*(_options_of(t["args"]) for t in GEMM_MATRIX))
+    assert used <= GEMM_REFERENCE_OPTIONS, used - GEMM_REFERENCE_OPTIONS
+    # ... and this build's tool knows every one of the reference's options
+    src = open(os.path.join(ROOT, "tests", "tools",
+                            "general_matrix_multiply.cpp")).read()
+    known = set(re.findall(r'"([A-Za-z0-9-]+)"',
+                           src.split("static const char *known[]", 1)[1]
+                           .split("};", 1)[0]))
+    assert GEMM_REFERENCE_OPTIONS <= known, GEMM_REFERENCE_OPTIONS - known
+    # empty operands, transposed operands, groups, mixed types, quarter
+    text = " ".join(" ".join(t["args"]) for t in GEMM_MATRIX)
+    for needle in ("--k 0", "--m 0", "--left-matrix-op=transpose",
+                   "--right-matrix-op=transpose", "--g 5",
+                   "--input-type=quarter", "--use-create-output=true"):
+        assert needle in text
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", GEMM_MATRIX, ids=lambda t: t["name"])
+def test_reference_gemm_ctest_case(case):
+    if not os.path.exists(GEMM_TOOL):
+        subprocess.check_call(["make", "-C", os.path.dirname(GEMM_TOOL)],
+                              stdout=subprocess.DEVNULL)
+    args = [a.replace("@golden/", GOLDEN + "/") for a in case["args"]]
+    r = subprocess.run([GEMM_TOOL, *args], capture_output=True, text=True,
+                       timeout=120)
+    # (the tool, like the reference's, says nothing when the product matches
+    # the host model and exits with 1 and "Validation failed" when it does not)
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-2000:])
+    assert "Validation failed" not in r.stderr

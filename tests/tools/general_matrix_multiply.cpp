@@ -48,7 +48,8 @@ int main(int argc, char **argv) try {
   static const char *known[] = {
       "help", "compile-only", "device-type", "profile", "profile-dir",
       "ignore-data", "m", "k", "n", "g", "data-type", "input-type",
-      "output-type", "partials-type", "fp8-format-a", "fp8-format-b",
+      "output-type", "partials-type", "fp8-format-A", "fp8-format-B",
+      "fp8-scale-A", "fp8-scale-B", "fp8-format-a", "fp8-format-b",
       "fp8-scale-a", "fp8-scale-b", "alpha", "beta", "left-matrix-op",
       "right-matrix-op", "tolerance", "tiles-per-ipu",
       "available-memory-proportion", "enable-fast-reduce", "report-plan",
@@ -145,17 +146,26 @@ int main(int argc, char **argv) try {
     return 0;
 
   QuarterMetadata mdA, mdB;
-  auto format = [&](const char *key) {
-    const std::string v = get(key, "quart152");
+  // (--fp8-format-A and so on are the reference's spellings,
+  // tools/general_matrix_multiply.cpp:166-177; the lower-case ones are kept
+  // beside them)
+  auto either = [&](const std::string &upper, const char *fallback) {
+    std::string lower = upper;
+    lower.back() = char(lower.back() - 'A' + 'a');
+    return has(upper.c_str()) ? get(upper.c_str(), fallback)
+                              : get(lower.c_str(), fallback);
+  };
+  auto format = [&](const std::string &key) {
+    const std::string v = either(key, "quart152");
     if (v != "quart152" && v != "quart143")
-      usage(std::string("--") + key + " must be quart152 or quart143");
+      usage("--" + key + " must be quart152 or quart143");
     return v == "quart143" ? QuarterMetadata::Format::F143
                            : QuarterMetadata::Format::F152;
   };
-  mdA.format = format("fp8-format-a");
-  mdB.format = format("fp8-format-b");
-  mdA.scale = std::stoi(get("fp8-scale-a", "0"));
-  mdB.scale = std::stoi(get("fp8-scale-b", "0"));
+  mdA.format = format("fp8-format-A");
+  mdB.format = format("fp8-format-B");
+  mdA.scale = std::stoi(either("fp8-scale-A", "0"));
+  mdB.scale = std::stoi(either("fp8-scale-B", "0"));
 
   // The operands as the caller holds them: op(A) is [g][m][k], so a
   // transposed A is stored [g][k][m]; likewise B.
