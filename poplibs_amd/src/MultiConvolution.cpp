@@ -25,6 +25,24 @@ bool parallelPlan(const poplar::OptionFlags &options) {
   return parallel != 0;
 }
 
+/// The convolutions of a parallel plan share one lowering in PopLibs, so
+/// their `insertTransformsCycleCountProgs` options must agree
+/// (lib/poplin/MultiConvolution.cpp:155-173).  The option itself has no
+/// effect on this device; the error is kept.
+template <class Args> void requireSameCycleCountProgs(const Args &args) {
+  auto wanted = [](const poplar::OptionFlags &options) {
+    for (const auto &kv : options)
+      if (kv.first == "insertTransformsCycleCountProgs")
+        return kv.second == "true";
+    return false;
+  };
+  for (const auto &arg : args)
+    if (wanted(arg.options) != wanted(args.front().options))
+      throw poputil::poplibs_error(
+          "Parallel multi-plans require to have same value for "
+          "<insertTransformsCycleCountProgs> option");
+}
+
 std::vector<std::size_t> actsShape(std::size_t batch, std::size_t chans,
                                    const std::vector<std::size_t> &field) {
   std::vector<std::size_t> shape{batch, chans};
@@ -76,6 +94,8 @@ std::vector<DeviceTensor> convolution(const std::vector<ConvolutionArgs> &args,
                                       const poplar::OptionFlags &options,
                                       PlanningCache *cache) {
   const bool parallel = parallelPlan(options);
+  if (parallel)
+    requireSameCycleCountProgs(args);
   const std::size_t n = args.size();
   std::vector<std::shared_ptr<PlanHandle>> plans(n);
   std::vector<DeviceTensor> in(n), weights(n), out(n), workspace(n);

@@ -5,6 +5,7 @@
 // (include/poplin/Convolution.hpp:590-611).  Exit code 0 = all passed.
 #include "poplin/ConvPreplan.hpp"
 #include "poplin/ConvUtil.hpp"
+#include "poplin/MultiConvolution.hpp"
 #include "poplar/exceptions.hpp"
 #include "poputil/exceptions.hpp"
 
@@ -415,6 +416,39 @@ int main(int argc, char **argv) {
               std::string::npos;
     }
     CHECK(threw);
+  }
+
+  // a parallel multi-convolution whose entries disagree on
+  // insertTransformsCycleCountProgs is refused, a serial one is not asked
+  // (tests/poplin/MultiConvolutionTest.cpp:84-130,
+  // lib/poplin/MultiConvolution.cpp:155-173); decided before any tensor is
+  // looked at
+  {
+    ConvParams a(poplar::HALF, poplar::HALF, 4, {8, 8}, {4, 4}, 1, 1, 10);
+    ConvParams b(poplar::FLOAT, poplar::FLOAT, 4, {5, 5}, {1, 1}, 11, 5, 1);
+    const std::vector<poplin::multiconv::ConvolutionArgs> args{
+        {poplin::DeviceTensor(), poplin::DeviceTensor(), a,
+         {{"insertTransformsCycleCountProgs", "true"}}},
+        {poplin::DeviceTensor(), poplin::DeviceTensor(), b,
+         {{"insertTransformsCycleCountProgs", "false"}}}};
+    poplin::Stream defaultStream(nullptr);
+    std::string message;
+    try {
+      poplin::multiconv::convolution(args, false, defaultStream,
+                                     {{"planType", "parallel"}});
+    } catch (const poputil::poplibs_error &e) {
+      message = e.what();
+    }
+    CHECK(message.find("<insertTransformsCycleCountProgs>") !=
+          std::string::npos);
+    message.clear();
+    try { // serial: gets as far as the (absent) tensors' shapes
+      poplin::multiconv::convolution(args, false, defaultStream,
+                                     {{"planType", "serial"}});
+    } catch (const poputil::poplibs_error &e) {
+      message = e.what();
+    }
+    CHECK(message.find("does not have the shape") != std::string::npos);
   }
 
   if (failures == 0)
