@@ -227,11 +227,21 @@ double roundsOf(std::size_t workgroups, std::size_t perCU) {
 /// igemmKernel: 1.45 us start-up + 1.5 us epilogue, 0.345 us per k-step of a
 /// 128 x 128 tile (0.24 for 128 x 64); further rounds on a CU pay another
 /// 1.5 us (nothing overlaps the next workgroup's start-up); two workgroups
-/// sharing a CU take 2.1 times one's time between them; K split adds 9 us
-/// (fp32 partial tiles out and in again, the second kernel: 20.4 us measured
-/// where the tiles alone are estimated at 11.2, 15.0 against 6.7).
+/// sharing a CU take 2.1 times one's time between them; K split adds
+/// splitPenaltyUs of its `partialBytes` of fp32 tiles.
+/// What K split over workgroups adds: the second kernel with its launch, and
+/// the fp32 partial tiles' way out and in again at what a stream of that size
+/// reaches (N = 32, 14 x 14, 1 x 1, 1024 -> 256 in two parts, 12.8 MB of
+/// tiles: 16.4 us where the tiles' k-steps are estimated at 7.7; 7 x 7, 3 x 3,
+/// 512 -> 512 in four, 12.8 MB: 18.7 against 11.2; N = 1, 14 x 14, 3 x 3,
+/// 256 -> 256 in nine, 1.8 MB: 9.2 against 6.3).
+double splitPenaltyUs(std::size_t partialBytes) {
+  return 4.5 + 2.0 * double(partialBytes) / 6.4e6;
+}
+
 double estimateStreaming(std::size_t workgroups, std::size_t kSteps,
-                         std::size_t perCU, unsigned blockN, unsigned splitK) {
+                         std::size_t perCU, unsigned blockN, unsigned splitK,
+                         std::size_t partialBytes) {
   const double rounds = roundsOf(workgroups, perCU);
   const double step = blockN == 128 ? 0.345 : 0.24;
   double tile = 2.95 + step * double(kSteps);
@@ -239,7 +249,8 @@ double estimateStreaming(std::size_t workgroups, std::size_t kSteps,
     tile += 1.5;
   if (perCU == 2)
     tile *= double(workgroups) > double(gfx950::numCUs) ? 2.1 : 1.0;
-  return kLaunchUs + rounds * tile + (splitK > 1 ? 9.0 : 0.0);
+  return kLaunchUs + rounds * tile +
+         (splitK > 1 ? splitPenaltyUs(partialBytes) : 0.0);
 }
 
 /// igemmPatchKernel (mode 1): 1.9 us to the first MFMA + 0.5 us reduction and
@@ -589,6 +600,39 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     g.blockN = pc.blockN ? pc.blockN : (co <= 64 ? 64 : 128);
     const unsigned stepElems = unsigned(128 / params.inputType.size());
     g.blockK = pc.blockK ? pc.blockK : stepElems;
+    // More than 64 output channels on few pixels (the deep 1 x 1 layers at
+    // the end of a ResNet): 128 x 128 tiles leave CUs idle or need K split
+    // over workgroups with a second kernel; twice as many 128 x 64 tiles, two
+    // workgroups to a CU, fill the chip with K whole.  Weighed by the same
+    // estimates (N = 32, 14 x 14, 1024 -> 256: 8.9 -> 7.1 us; 7 x 7, 2048 ->
+    // 512: 12.8 -> 10.2; but 14 x 14, 1024 -> 512, 392 narrow tiles: 10.2
+    // against 12.1, and the estimate keeps the wide tile there).
+    bool narrowWhole = false; // ... chosen: K stays whole
+    if (!pc.blockN && !pc.splitK && !pc.stages && co > 64 &&
+        g.blockM == 128) {
+      const std::size_t m = s.batch * s.outD * s.outH * s.outW;
+      const std::size_t mTiles = (m + 127) / 128;
+      const std::size_t kSteps =
+          (std::size_t(s.kD) * s.kH * s.kW * ciPadded + stepElems - 1) /
+          stepElems;
+      const std::size_t wide = mTiles * ((co + 127) / 128) * p.numConvGroups;
+      const std::size_t narrow = mTiles * ((co + 63) / 64) * p.numConvGroups;
+      std::size_t parts = 1;
+      if (wide != 0 && wide * 2 <= gfx950::numCUs && kSteps >= 16)
+        parts = std::max<std::size_t>(
+            1, std::min<std::size_t>(gfx950::numCUs / wide, kSteps / 4));
+      const std::size_t partial =
+          parts * m * p.numConvGroups * ((co + 127) / 128 * 128) * 4;
+      const double wideUs = std::min(
+          estimateStreaming(wide, kSteps, wide > gfx950::numCUs ? 2 : 1, 128,
+                            1, 0),
+          parts > 1 ? estimateStreaming(wide * parts,
+                                        (kSteps + parts - 1) / parts, 1, 128,
+                                        unsigned(parts), partial)
+                    : 1e30);
+      if (estimateStreaming(narrow, kSteps, 2, 64, 1, 0) < wideUs)
+        g.blockN = 64, narrowWhole = true;
+    }
     const bool anyHeight = pc.patch == 2 && g.blockM >= 1 && g.blockM <= 112;
     if ((g.blockM != 128 && g.blockM != 64 && !anyHeight) ||
         (g.blockN != 64 && g.blockN != 128) ||
@@ -615,7 +659,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       std::size_t parts = 1;
       if (pc.splitK)
         parts = pc.splitK;
-      else if (tiles != 0 && tiles * 2 <= gfx950::numCUs && kSteps >= 16)
+      else if (!narrowWhole && tiles != 0 && tiles * 2 <= gfx950::numCUs &&
+               kSteps >= 16)
         parts = std::min<std::size_t>(gfx950::numCUs / tiles, kSteps / 4);
       parts = std::max<std::size_t>(1, std::min(parts, kSteps));
       // ... where that is estimated to pay for the partial tiles' round trip
@@ -623,9 +668,12 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
       // (98 tiles of 16 k-steps) 16.4 us in two parts, 8.9 us whole; 7 x 7,
       // 3 x 3, 512 -> 512 (52 tiles of 72 k-steps) 18.7 in four, 21.1 whole.
       if (!pc.splitK && parts > 1 &&
-          estimateStreaming(tiles, kSteps, 1, g.blockN, 1) <=
+          estimateStreaming(tiles, kSteps, g.blockN == 64 ? 2 : 1, g.blockN, 1,
+                            0) <=
               estimateStreaming(tiles * parts, (kSteps + parts - 1) / parts,
-                                1, g.blockN, unsigned(parts)))
+                                1, g.blockN, unsigned(parts),
+                                parts * m * p.numConvGroups * plan.coPadded *
+                                    4))
         parts = 1;
       const std::size_t chans = p.numConvGroups * co;
       // the reduction reads and writes vectors of four channels; partial
@@ -894,7 +942,8 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
                                 : ""),
               Tiling{0, 128}, streamTiles, streamPerCU, streamSteps,
               estimateStreaming(streamTiles, streamSteps, streamPerCU,
-                                g.blockN, g.splitK),
+                                g.blockN, g.splitK,
+                                mxk::igemmWorkspaceBytes(g)),
               roundsOf(streamTiles, streamPerCU));
       std::size_t best = iStream;
       if (pc.patch >= 1) {
@@ -1126,9 +1175,12 @@ mxconv_plan::DetailedEstimate mxconv_plan::detailedEstimate() const {
              1);
       break;
     }
-    // (the streaming kernel's K split: 9 us for the fp32 partial tiles' way
-    // out and in again and the second kernel, see estimateStreaming)
-    const double kSplitUs = igemm.splitK > 1 && !igemm.patch ? 9.0 : 0.0;
+    // (the streaming kernel's K split: the fp32 partial tiles' way out and
+    // in again and the second kernel, see splitPenaltyUs)
+    const double kSplitUs =
+        igemm.splitK > 1 && !igemm.patch
+            ? poplin::splitPenaltyUs(mxk::igemmWorkspaceBytes(igemm))
+            : 0.0;
     e.reductionUs = kSplitUs;
     e.reductionBytes = kSplitUs > 0 ? mxk::igemmWorkspaceBytes(igemm) : 0;
     bool weighed = false;
@@ -1146,8 +1198,9 @@ mxconv_plan::DetailedEstimate mxconv_plan::detailedEstimate() const {
     const std::size_t steps =
         (kPadded / g.blockK + g.splitK - 1) / g.splitK;
     const std::size_t perCU = g.blockN == 64 || g.stages == 2 ? 2 : 1;
-    double us =
-        poplin::estimateStreaming(tiles, steps, perCU, g.blockN, g.splitK);
+    double us = poplin::estimateStreaming(tiles, steps, perCU, g.blockN,
+                                          g.splitK,
+                                          mxk::igemmWorkspaceBytes(igemm));
     // No kernel is faster than its tensors stream.
     us = std::max(us, streamed(inputBytes() + outputBytes() +
                                weightPackedBytes()));
