@@ -260,8 +260,10 @@ hipError_t launchIgemmFused(const IgemmFusedItem *items, size_t count,
                             hipStream_t stream);
 
 /// Pointwise convolution (every kernel extent 1, stride 1, no padding or
-/// truncation, half inputs) with 64, 128, 256 or 512 input channels per group:
-/// a streaming kernel of small workgroups instead of igemm's big tiles.
+/// truncation, half inputs) with a multiple of 8 up to 512 input channels per
+/// group: a streaming kernel of small workgroups instead of igemm's big tiles
+/// (compiled for rows of 16, 32, 64, 128, 256 and 512 channels; a layer in
+/// between runs as the next one up).
 struct PointwiseDesc {
   uint32_t batch, pixels; // pixels per image
   uint32_t groups, inChansPerGroup, outChansPerGroup;

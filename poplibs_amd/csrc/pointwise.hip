@@ -29,10 +29,25 @@
 //     leaves as 16-byte stores, 64 bytes per pixel and store;
 //   * one workgroup barrier per tile: the tile has landed / the buffer before
 //     it has been read.
+//
+// Input channels per group: any multiple of 8 up to 512.  The kernel is
+// compiled for rows of 16, 32, 64, 128, 256 and 512 channels; a layer in
+// between runs as the next one up, its rows padded in LDS only - the loads of
+// the 16-byte chunks past the layer's channels lie beyond the buffer and
+// bring zeros without touching memory, and the packed weights carry zeros
+// there.
 #include "igemm_common.hpp"
 
 namespace mxk {
 namespace {
+
+/// The row the kernel is compiled for: the next of 16, 32, ..., 512 channels.
+constexpr uint32_t pwPaddedChans(uint32_t ci) {
+  uint32_t p = 16;
+  while (p < ci)
+    p *= 2;
+  return p;
+}
 
 constexpr int kPwChans = 64;         // output channels per workgroup
 constexpr int kPwStageRow = 64 + 16; // staging: 64 bytes of a pixel + padding
@@ -60,10 +75,14 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
     PwArgs a, const char *__restrict__ in, const char *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
   constexpr int kRow = KS * 32;                 // bytes of one activation row
-  constexpr int kChunkBits =
-      KS == 4 ? 3 : KS == 8 ? 4 : KS == 16 ? 5 : 6; // log2(kRow / 16)
+  constexpr int kChunkBits = KS == 1   ? 1
+                             : KS == 2 ? 2
+                             : KS == 4 ? 3
+                             : KS == 8 ? 4
+                             : KS == 16 ? 5
+                                        : 6; // log2(kRow / 16)
   // chunk c of row r sits at chunk position c ^ (r & kSwizzle)
-  constexpr uint32_t kSwizzle = KS == 4 ? 7u : 15u;
+  constexpr uint32_t kSwizzle = KS == 1 ? 1u : KS == 2 ? 3u : KS == 4 ? 7u : 15u;
   constexpr int kRowsPerLoad = 1024 / kRow;
   constexpr int kLoads = TM / kRowsPerLoad; // wave-wide loads per tile
   constexpr int kTileBytes = TM * kRow;
@@ -88,6 +107,7 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
   const uint32_t g = logical / (a.walkers * a.nTiles);
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
   const uint32_t pixelBytes = d.groups * d.inChansPerGroup * 2;
+  const uint32_t groupBytes = d.inChansPerGroup * 2; // (may be below kRow)
 
   if (wave >= kComputeWaves) {
     const int loader = wave - kComputeWaves;
@@ -105,8 +125,9 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
         const uint32_t chunk = pos ^ (row & kSwizzle);
         const uint32_t m = mTile * TM + row;
         loadToLds(inBuf, (LdsPtr)(buffer + load * 1024),
-                  m < a.M ? m * pixelBytes + g * kRow + chunk * 16
-                          : kOutOfRange,
+                  m < a.M && chunk * 16 < groupBytes
+                      ? m * pixelBytes + g * groupBytes + chunk * 16
+                      : kOutOfRange,
                   0);
       }
     };
@@ -334,15 +355,17 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
 /// Weights [G][Co][Ci] -> [G][32-channel block][k-slice][lane][8 halves]:
 /// lane l of a slice holds channel l % 32 of the block, input channels
 /// 16 slice + 8 (l / 32) ... + 8 - the row operand of v_mfma_f32_32x32x16_f16.
-/// Channels past Co are zero.
+/// Channels past Co are zero, and so are input channels past Ci (the slices
+/// run to the padded row).
 __global__ __launch_bounds__(256) void packPointwiseWeightsKernel(
     const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, uint32_t co,
-    uint32_t ci, uint32_t nBlocks, uint64_t total, bool chansTransposed) {
+    uint32_t ci, uint32_t ciPadded, uint32_t nBlocks, uint64_t total,
+    bool chansTransposed) {
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
     return;
   const uint32_t e = uint32_t(tid & 7), lane = uint32_t(tid >> 3) & 63;
-  const uint32_t slices = ci / 16;
+  const uint32_t slices = ciPadded / 16;
   uint64_t r = tid >> 9;
   const uint32_t ks = uint32_t(r % slices);
   r /= slices;
@@ -352,9 +375,9 @@ __global__ __launch_bounds__(256) void packPointwiseWeightsKernel(
   const uint32_t k = ks * 16 + 8 * (lane >> 5) + e;
   // source [G][Co][Ci], or [G][Ci][Co] (a matrix multiplication's right-hand
   // side)
-  dst[tid] = n >= co           ? uint16_t(0)
-             : chansTransposed ? src[(g * ci + k) * co + n]
-                               : src[(g * co + n) * ci + k];
+  dst[tid] = n >= co || k >= ci ? uint16_t(0)
+             : chansTransposed  ? src[(g * ci + k) * co + n]
+                                : src[(g * co + n) * ci + k];
 }
 
 /// Workgroups that share the pixel tiles of one (group, channel tile) pair:
@@ -390,12 +413,16 @@ struct PwShape {
 };
 constexpr PwShape kShape64{128, 3, 2}, kShape128{128, 3, 4},
     kShape256{64, 3, 2}, kShape512{64, 2, 4};
+/// (`ci`: the layer's channels; rows of 16 and 32 channels take the shape of
+/// 64: such layers are all output)
 constexpr PwShape shapeFor(uint32_t ci) {
-  return ci == 64 ? kShape64 : ci == 128 ? kShape128 : ci == 256 ? kShape256
-                                                                 : kShape512;
+  return pwPaddedChans(ci) <= 64    ? kShape64
+         : pwPaddedChans(ci) == 128 ? kShape128
+         : pwPaddedChans(ci) == 256 ? kShape256
+                                    : kShape512;
 }
 constexpr uint32_t ldsBytesOf(PwShape s, uint32_t ci, uint32_t nt = 1) {
-  return uint32_t(s.nb * s.tm * (ci / 16) * 32 +
+  return uint32_t(s.nb * s.tm * (pwPaddedChans(ci) / 16) * 32 +
                   (s.tm / 16) * 32 * kPwStageRow + nt * kPwChans * 4);
 }
 
@@ -412,12 +439,12 @@ uint32_t chanTilesFor(const PointwiseDesc &d, uint32_t cus) {
   const PwShape s = shapeFor(d.inChansPerGroup);
   const uint64_t mTiles = (uint64_t(d.batch) * d.pixels + s.tm - 1) / s.tm;
   const uint64_t tiles64 = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
-  if (d.inChansPerGroup == 64) {
+  const uint32_t padded = pwPaddedChans(d.inChansPerGroup);
+  if (padded <= 64) {
     for (uint32_t nt = 4; nt > 1; --nt)
       if (tiles64 % nt == 0 && mTiles * (tiles64 / nt) * d.groups >= 2ull * cus)
         return nt;
-  } else if ((d.inChansPerGroup == 128 || d.inChansPerGroup == 256) &&
-             tiles64 % 2 == 0) {
+  } else if ((padded == 128 || padded == 256) && tiles64 % 2 == 0) {
     const uint64_t pairs = tiles64 / 2 * d.groups;
     const uint64_t walkers = walkersFor(
         mTiles, pairs, ldsBytesOf(s, d.inChansPerGroup, 2), cus);
@@ -475,7 +502,31 @@ template <class OutT>
 hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
                      const void *bias, void *out, hipStream_t stream) {
   const uint32_t nt = chanTilesFor(a.d, uint32_t(deviceCUs()));
-  switch (a.d.inChansPerGroup) {
+  switch (pwPaddedChans(a.d.inChansPerGroup)) {
+  case 16:
+    if (nt == 4)
+      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT>(
+          a, in, w, bias, out, stream);
+    if (nt == 3)
+      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT>(
+          a, in, w, bias, out, stream);
+    if (nt == 2)
+      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT>(
+          a, in, w, bias, out, stream);
+    return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT>(
+        a, in, w, bias, out, stream);
+  case 32:
+    if (nt == 4)
+      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT>(
+          a, in, w, bias, out, stream);
+    if (nt == 3)
+      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT>(
+          a, in, w, bias, out, stream);
+    if (nt == 2)
+      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT>(
+          a, in, w, bias, out, stream);
+    return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT>(
+        a, in, w, bias, out, stream);
   case 64:
     if (nt == 4)
       return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT>(
@@ -511,9 +562,8 @@ hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
 
 bool pointwiseChanTilesOk(const PointwiseDesc &d, uint32_t chanTiles) {
   const uint32_t tiles64 = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
-  const uint32_t most = d.inChansPerGroup == 64    ? 4
-                        : d.inChansPerGroup == 512 ? 1
-                                                   : 2;
+  const uint32_t padded = pwPaddedChans(d.inChansPerGroup);
+  const uint32_t most = padded <= 64 ? 4 : padded == 512 ? 1 : 2;
   return chanTiles >= 1 && chanTiles <= most && tiles64 % chanTiles == 0;
 }
 
@@ -522,7 +572,7 @@ bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType) {
   const uint64_t m = uint64_t(d.batch) * d.pixels;
   const uint64_t inBytes = m * d.groups * ci * 2;
   return inType == kHalf && (outType == kHalf || outType == kFloat) &&
-         (ci == 64 || ci == 128 || ci == 256 || ci == 512) && co != 0 &&
+         ci != 0 && ci % 8 == 0 && ci <= 512 && co != 0 &&
          (d.chanTiles == 0 || pointwiseChanTilesOk(d, d.chanTiles)) &&
          co % (outType == kHalf ? 8 : 4) == 0 && m != 0 && m < 0x7fffffffull &&
          inBytes < kOutOfRange &&
@@ -531,7 +581,8 @@ bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType) {
 
 uint64_t pointwisePackedElems(const PointwiseDesc &d) {
   const uint64_t nBlocks = (d.outChansPerGroup + kPwChans - 1) / kPwChans * 2;
-  return uint64_t(d.groups) * nBlocks * (d.inChansPerGroup / 16) * 512;
+  return uint64_t(d.groups) * nBlocks *
+         (pwPaddedChans(d.inChansPerGroup) / 16) * 512;
 }
 
 hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
@@ -547,7 +598,8 @@ hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
   hipLaunchKernelGGL(packPointwiseWeightsKernel, dim3(uint32_t(blocks)),
                      dim3(256), 0, stream, static_cast<const uint16_t *>(src),
                      static_cast<uint16_t *>(dst), d.outChansPerGroup,
-                     d.inChansPerGroup, nBlocks, total, chansTransposed);
+                     d.inChansPerGroup, pwPaddedChans(d.inChansPerGroup),
+                     nBlocks, total, chansTransposed);
   return hipGetLastError();
 }
 

@@ -845,8 +845,16 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
         s.padH == 0 && s.padW == 0 && s.loH == 0 && s.loW == 0 &&
         s.hiH == s.inH && s.hiW == s.inW && s.outH == s.inH &&
         s.outW == s.inW;
+    // (The kernel runs 136 to 248 input channels as rows of 256, up to 44 %
+    // of them padding it multiplies and makes room for: the big tile is
+    // faster on small layers - N = 32, 28 x 28, 144 -> 32: 4.6 against 5.3 us,
+    // 192 -> 32: 4.6 against 5.4, 7 x 7, 160 -> 960: 4.8 against 5.5 - and
+    // slower on large ones: 56 x 56, 144 -> 24: 11.9 against 8.9.)
+    const bool paddedSmall = ci > 128 && ci < 256 &&
+                             std::size_t(pw.batch) * pw.pixels < 65536 &&
+                             pc.pointwise != 1;
     plan.pointwiseOn =
-        unitWindow && ciPadded == ci &&
+        unitWindow && ciPadded == ci && !paddedSmall &&
         (pc.kernel != "igemm" || pc.pointwise == 1) && pc.pointwise != 0 &&
         pc.patch < 1 && !pc.blockM &&
         !pc.blockN && !pc.blockK &&
@@ -861,14 +869,15 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
     else if (pc.pointwise == 1)
       throw poplar::invalid_option(
           "planConstraints gfx950 pointwise: that kernel takes 1x1, unit "
-          "stride, unpadded convolutions of 64, 128, 256 or 512 input "
-          "channels per group, with no other tile constraint");
+          "stride, unpadded convolutions of half inputs with a multiple of 8 "
+          "up to 512 input channels per group, with no other tile "
+          "constraint");
     else if (pc.chanTiles)
       throw poplar::invalid_option(
           "planConstraints gfx950 chanTiles: the pointwise streaming kernel "
           "does not take this convolution with that many 64-channel tiles "
-          "per workgroup (they divide the layer's; at most 4 with 64 input "
-          "channels, 2 with 128 or 256, 1 with 512)");
+          "per workgroup (they divide the layer's; at most 4 with up to 64 "
+          "input channels, 2 with up to 256, 1 beyond)");
     // Unit stride and whole 128-byte slices of channels: the kernel that
     // keeps the tile's input patch in LDS reads every input element once
     // instead of once per tap.

@@ -656,3 +656,20 @@ def test_planner_weighs_tilings_and_reports_them():
     with pytest.raises(MxconvError):
         forced(patch=2, blockM=113)
     assert "LDS stages                 2" in forced(stages=2)
+
+
+def test_pointwise_planner_choice_for_padded_rows():
+    """Rows padded to 256 channels go to the big tile on small layers."""
+    def kernel_of(**kw):
+        return pa.Plan(make_params(pa.HALF, kernel=(1, 1), **kw)).describe()
+    assert "pointwise streaming variant" in kernel_of(
+        batch=32, field=(56, 56), ci=144, co=24)
+    assert "pointwise streaming variant" not in kernel_of(
+        batch=32, field=(28, 28), ci=144, co=32)
+    assert "pointwise streaming variant" in kernel_of(
+        batch=32, field=(112, 112), ci=16, co=96)
+    assert "pointwise streaming variant" in kernel_of(
+        batch=32, field=(14, 14), ci=384, co=64)
+    # not a multiple of eight: the big tile, channels padded in a copy
+    assert "pointwise streaming variant" not in kernel_of(
+        batch=2, field=(14, 14), ci=20, co=64)

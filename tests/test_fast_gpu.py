@@ -172,6 +172,41 @@ def test_pointwise_channel_tiles_pm1_exact_and_plan_choice(oracle):
                      '{"gfx950": {"chanTiles": %d}}' % bad})
 
 
+# Input channels that are no power of two, or fewer than 64: the kernel runs
+# them as rows of the next size up (16, 32, 64, 128, 256, 512), the chunks
+# past the layer's channels loaded from beyond the buffer - zeros - and the
+# packed weights zero there.  MobileNet's thin layers and their neighbours:
+# pixels ragged against the tile, groups, output channels that fill the last
+# tile partly.
+THIN_POINTWISE_CASES = [
+    dict(batch=2, field=(28, 29), kernel=(1, 1), ci=8, co=48),
+    dict(batch=3, field=(17, 9), kernel=(1, 1), ci=16, co=96),
+    dict(batch=2, field=(13, 22), kernel=(1, 1), ci=24, co=144),
+    dict(batch=1, field=(31, 19), kernel=(1, 1), ci=32, co=16),
+    dict(batch=2, field=(9, 14), kernel=(1, 1), ci=40, co=72, groups=2),
+    dict(batch=2, field=(12, 12), kernel=(1, 1), ci=96, co=24),
+    dict(batch=3, field=(7, 11), kernel=(1, 1), ci=144, co=32),
+    dict(batch=1, field=(15, 15), kernel=(1, 1), ci=192, co=64, groups=2),
+    dict(batch=2, field=(7, 7), kernel=(1, 1), ci=320, co=1280),
+    dict(batch=2, field=(8, 5), kernel=(1, 1), ci=384, co=96),
+    dict(batch=1, field=(5, 6), kernel=(1, 1), ci=504, co=40),
+]
+FORCE_POINTWISE = {"planConstraints": '{"gfx950": {"pointwise": 1}}'}
+
+
+@pytest.mark.parametrize("kw", THIN_POINTWISE_CASES)
+@pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
+def test_pointwise_any_multiple_of_eight_channels(oracle, kw, out_type):
+    p = make_params(pa.HALF, out_type, **kw)
+    text = pa.Plan(p, FORCE_POINTWISE).describe()
+    assert "pointwise streaming variant" in text, text
+    # +-1 data: exact, whatever the padding multiplies
+    _run(oracle, p, 21, 0 if out_type == pa.FLOAT else 1e-3, "implicit GEMM",
+         dist="pm1" if out_type == pa.FLOAT else "normal",
+         options=FORCE_POINTWISE, bias=bool(kw["ci"] % 16),
+         **({} if out_type == pa.FLOAT else {"wscale": 0.1}))
+
+
 def test_pointwise_pm1_exact_and_big_tile_on_request(oracle):
     p = make_params(pa.HALF, pa.FLOAT, **POINTWISE_CASES[1])
     _run(oracle, p, 9, 0, "implicit GEMM", dist="pm1")
