@@ -56,6 +56,13 @@ hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
 /// (strides in elements; elements of 2 or 4 bytes): channels-last activations
 /// with the batch axis moved innermost, as the weight update pass wants both
 /// of its operands.
+/// Weights in external order [groups][co][ci][taps] -> the block-diagonal
+/// weights [groups / perGroup][perGroup co][perGroup ci][taps] of the layer
+/// with `perGroup` neighbouring groups taken as one.
+hipError_t launchFuseGroupWeights(const void *src, void *dst, uint64_t groups,
+                                  uint64_t perGroup, uint64_t co, uint64_t ci,
+                                  uint64_t taps, int elemBytes,
+                                  hipStream_t stream);
 hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
                                 uint32_t pixels, uint32_t groups,
                                 uint32_t chans, uint64_t strideG,

@@ -329,6 +329,30 @@ __global__ __launch_bounds__(256) void biasUpdateKernel(
   storeOut(biases, c, Load<T>::at(biases, c, 0) + scale * total);
 }
 
+/// Weights [G][co][ci][taps] of G conv groups -> [G / f][f co][f ci][taps] of
+/// G / f groups that each take f of them as one: block (a, b) of a fused
+/// group's f x f blocks of co x ci channels is group (f g' + a)'s weights
+/// where a == b and zero elsewhere.  One element of the result per thread.
+template <class T>
+__global__ __launch_bounds__(256) void
+fuseGroupWeightsKernel(const T *__restrict__ src, T *__restrict__ dst,
+                       uint64_t f, uint64_t co, uint64_t ci, uint64_t taps,
+                       uint64_t total) {
+  const uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total)
+    return;
+  const uint64_t tap = i % taps;
+  uint64_t rest = i / taps;
+  const uint64_t k = rest % (f * ci);
+  rest /= f * ci;
+  const uint64_t n = rest % (f * co);
+  const uint64_t fused = rest / (f * co);
+  const uint64_t a = n / co, b = k / ci;
+  dst[i] = a == b ? src[(((fused * f + a) * co + n % co) * ci + k % ci) * taps +
+                        tap]
+                  : T(0);
+}
+
 } // namespace
 
 hipError_t launchPermute4(const void *src, void *dst, const uint64_t srcDims[4],
@@ -793,6 +817,37 @@ hipError_t launchBiasUpdate(int deltasType, const void *zDeltas, uint64_t rows,
     hipLaunchKernelGGL(biasUpdateKernel<__half>, grid2, block, 0, stream,
                        static_cast<__half *>(biases), partial, scale, channels,
                        splits);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launchFuseGroupWeights(const void *src, void *dst, uint64_t groups,
+                                  uint64_t perGroup, uint64_t co, uint64_t ci,
+                                  uint64_t taps, int elemBytes,
+                                  hipStream_t stream) {
+  const uint64_t total = groups * perGroup * co * ci * taps;
+  if (total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull || groups % perGroup != 0)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  if (elemBytes == 4)
+    hipLaunchKernelGGL(fuseGroupWeightsKernel<uint32_t>, grid, block, 0, stream,
+                       static_cast<const uint32_t *>(src),
+                       static_cast<uint32_t *>(dst), perGroup, co, ci, taps,
+                       total);
+  else if (elemBytes == 2)
+    hipLaunchKernelGGL(fuseGroupWeightsKernel<uint16_t>, grid, block, 0, stream,
+                       static_cast<const uint16_t *>(src),
+                       static_cast<uint16_t *>(dst), perGroup, co, ci, taps,
+                       total);
+  else if (elemBytes == 1)
+    hipLaunchKernelGGL(fuseGroupWeightsKernel<uint8_t>, grid, block, 0, stream,
+                       static_cast<const uint8_t *>(src),
+                       static_cast<uint8_t *>(dst), perGroup, co, ci, taps,
+                       total);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

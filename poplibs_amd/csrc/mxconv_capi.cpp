@@ -673,7 +673,8 @@ namespace {
 std::string packingSignature(const mxconv_plan &p) {
   std::ostringstream os;
   os << int(p.kernel) << '/' << p.params.inputType.toString() << '/'
-     << p.weightElems << '/' << p.weightPackedElems;
+     << p.weightElems << '/' << p.weightPackedElems << "/cg"
+     << p.convGroupsPerGroup;
   if (p.kernel == mxconv_plan::Kernel::IGEMM) {
     os << "/pw" << p.pointwiseOn << "/patch" << p.igemm.patch << "/co"
        << p.coPadded << "/k" << p.kPadded << "/ci" << p.paddedInputChans
@@ -723,6 +724,25 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
   if (plan->kernel == mxconv_plan::Kernel::IGEMM) {
     if (plan->weightElems != 0)
       REQUIRE_ARG(weights_external);
+    // Conv groups run as one: their block-diagonal weights, in external
+    // order, are laid out behind the packed weights first and packed from
+    // there as the weights of the fused groups.
+    uint32_t groups = uint32_t(p.numConvGroups);
+    uint32_t co = uint32_t(p.outputChannelsPerConvGroup);
+    uint32_t ci = uint32_t(p.inputChannelsPerConvGroup);
+    if (plan->convGroupsPerGroup > 1) {
+      const uint32_t f = plan->convGroupsPerGroup;
+      void *fused = static_cast<char *>(weights_packed) +
+                    plan->weightPackedElems * elemBytes;
+      const mxconv_status st = hipStatus(
+          mxk::launchFuseGroupWeights(weights_external, fused, groups, f, co,
+                                      ci, taps, elemBytes, s),
+          "weight packing");
+      if (st != MXCONV_OK)
+        return st;
+      weights_external = fused;
+      groups /= f, co *= f, ci *= f;
+    }
     if (plan->pointwiseOn)
       return hipStatus(mxk::launchPackPointwiseWeights(
                            plan->pointwise, weights_external, weights_packed, s),
@@ -733,8 +753,7 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
               weights_external,
               static_cast<char *>(weights_packed) +
                   phase.packedOffset * elemBytes,
-              uint32_t(p.numConvGroups), uint32_t(p.outputChannelsPerConvGroup),
-              uint32_t(p.inputChannelsPerConvGroup), uint32_t(taps),
+              groups, co, ci, uint32_t(taps),
               uint32_t(plan->coPadded), uint32_t(phase.kPadded), elemBytes, s,
               false, uint32_t(plan->paddedInputChans), &phase.taps),
           "weight packing");
@@ -752,9 +771,7 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
           "weight packing");
     return hipStatus(
         mxk::launchPackIgemmWeights(
-            weights_external, weights_packed, uint32_t(p.numConvGroups),
-            uint32_t(p.outputChannelsPerConvGroup),
-            uint32_t(p.inputChannelsPerConvGroup), uint32_t(taps),
+            weights_external, weights_packed, groups, co, ci, uint32_t(taps),
             uint32_t(plan->coPadded), uint32_t(plan->kPadded), elemBytes, s,
             false, uint32_t(plan->paddedInputChans),
             plan->kernelSelected ? &plan->igemmTaps : nullptr),

@@ -247,8 +247,9 @@ PlanConstraints parsePlanConstraints(const std::string &text) {
   for (const auto &m : root.members) {
     if (m.first == "method")
       pc.method = checkMethod(m.first, m.second);
-    else if (m.first == "convGroupsPerGroup" || m.first == "inChansPerGroup" ||
-             m.first == "partialChansPerGroup")
+    else if (m.first == "convGroupsPerGroup")
+      pc.convGroupsPerGroup = requireUnsigned(m.first, m.second);
+    else if (m.first == "inChansPerGroup" || m.first == "partialChansPerGroup")
       requireUnsigned(m.first, m.second);
     else if (m.first == "gfx950")
       checkGfx950(m.first, m.second, pc);

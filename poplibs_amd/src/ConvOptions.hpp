@@ -31,6 +31,9 @@ const char *toString(Pass p);
 struct PlanConstraints {
   enum class Method { ANY, AMP, SLIC, HMAC, VMAC, OUTER_PRODUCT };
   Method method = Method::ANY;
+  /// Conv groups the matrix-core kernels run as one (the reference's
+  /// top-level constraint of that name); 0 = planner's choice.
+  unsigned convGroupsPerGroup = 0;
   /// "gfx950" section: force a kernel ("generic", "igemm", "depthwise") and
   /// tile extents; 0 / empty = planner's choice.
   std::string kernel;

@@ -274,13 +274,83 @@ double estimatePatch(std::size_t workgroups, std::size_t kSteps, unsigned mode,
 
 } // namespace
 
+namespace {
+
+/// Conv groups to run as one (see mxconv_plan::convGroupsPerGroup), 1 = each
+/// by itself.  By the planner's own choice: layers whose groups have fewer
+/// input channels than half a 128-byte slice and few output channels - the
+/// smallest number of groups that makes a whole slice, where that keeps the
+/// fused group within 256 output channels (32 groups of 4 -> 4 channels run
+/// as 2 groups of 64 -> 64: 16 times the multiply-adds, on matrix cores that
+/// stood idle behind 16-byte vectors half empty and 64-channel tiles with 4
+/// channels in them).  A `convGroupsPerGroup` plan constraint is taken where
+/// it can be (it divides the groups and the fused channels are whole 16-byte
+/// vectors) and means "by itself" elsewhere: the reference accepts values
+/// that only its own vertices give a meaning to.
+unsigned chooseConvGroupsPerGroup(const ConvParams &p,
+                                  const ConvOptions &options) {
+  const auto &pc = options.planConstraints;
+  switch (options.pass) {
+  case Pass::NONE:
+  case Pass::INFERENCE_FWD:
+  case Pass::TRAINING_FWD:
+  case Pass::TRAINING_BWD:
+    break;
+  default:
+    return 1;
+  }
+  const std::size_t groups = p.numConvGroups;
+  const std::size_t ci = p.inputChannelsPerConvGroup;
+  const std::size_t co = p.outputChannelsPerConvGroup;
+  const std::size_t eb = p.inputType.size();
+  if (groups < 2 || ci == 0 || co == 0 || (ci == 1 && co == 1) ||
+      (!pc.kernel.empty() && pc.kernel != "igemm") || p.batchSize == 0)
+    return 1;
+  auto usable = [&](std::size_t f) {
+    return f >= 1 && groups % f == 0 && (f * ci * eb) % 16 == 0;
+  };
+  if (pc.convGroupsPerGroup != 0)
+    return usable(pc.convGroupsPerGroup) ? pc.convGroupsPerGroup : 1u;
+  if (ci < 2 || ci * eb >= 64)
+    return 1;
+  for (std::size_t f = 2; f <= groups; ++f)
+    if (usable(f) && f * ci * eb >= 128)
+      return f * co <= 256 ? unsigned(f) : 1u;
+  return 1;
+}
+
+mxconv_plan makePlanWith(const ConvParams &params,
+                         const ConvOptions &optionsIn,
+                         unsigned convGroupsPerGroup);
+
+} // namespace
+
 mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
+  const unsigned fuse =
+      chooseConvGroupsPerGroup(params.canonicalize(), optionsIn);
+  if (fuse > 1) {
+    // (only the matrix-core kernels run groups as one)
+    mxconv_plan plan = makePlanWith(params, optionsIn, fuse);
+    if (plan.kernel == mxconv_plan::Kernel::IGEMM)
+      return plan;
+  }
+  return makePlanWith(params, optionsIn, 1);
+}
+
+namespace {
+
+mxconv_plan makePlanWith(const ConvParams &params,
+                         const ConvOptions &optionsIn,
+                         unsigned convGroupsPerGroup) {
   mxconv_plan plan;
   plan.params = params;
   plan.canonical = params.canonicalize(); // validates
   plan.options = optionsIn;
   ConvOptions &options = plan.options;
-  const ConvParams &p = plan.canonical;
+  // What the kernels are planned for: the canonical parameters, with
+  // `convGroupsPerGroup` groups taken as one further down.
+  ConvParams planned = plan.canonical;
+  const ConvParams &p = planned;
 
   if (p.getNumFieldDims() > mxk::kMaxDims)
     throw poputil::poplibs_error("At most " + std::to_string(mxk::kMaxDims) +
@@ -412,6 +482,11 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
           "vectors)");
   }
   const auto &pc = options.planConstraints;
+  if (convGroupsPerGroup > 1) {
+    planned.numConvGroups /= convGroupsPerGroup;
+    planned.inputChannelsPerConvGroup *= convGroupsPerGroup;
+    planned.outputChannelsPerConvGroup *= convGroupsPerGroup;
+  }
   const Simple2D s = asSimple2D(p);
   const bool halfIn = params.inputType == poplar::HALF;
   const bool quarterIn = params.inputType == poplar::QUARTER;
@@ -1058,14 +1133,23 @@ mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   } else {
     plan.weightPackedElems = plan.weightElems; // [G][K][Ci][Co]
   }
+  if (convGroupsPerGroup > 1 && chosen == Kernel::IGEMM) {
+    plan.convGroupsPerGroup = convGroupsPerGroup;
+    plan.weightExpandElems = plan.weightElems * convGroupsPerGroup;
+  }
   return plan;
 }
+
+} // namespace
 
 } // namespace poplin
 
 std::string mxconv_plan::constraintsJson() const {
   std::ostringstream os;
-  os << "{\"gfx950\": {";
+  os << "{";
+  if (kernel == Kernel::IGEMM && canonical.numConvGroups > 1)
+    os << "\"convGroupsPerGroup\": " << convGroupsPerGroup << ", ";
+  os << "\"gfx950\": {";
   switch (kernel) {
   case Kernel::GENERIC:
     os << "\"kernel\": \"generic\"";
@@ -1281,6 +1365,13 @@ std::string mxconv_plan::describe() const {
     os << "        gemm M x N x K             " << m << " x "
        << g.outChansPerGroup << " x " << k << " (x " << g.groups
        << " groups)\n";
+    if (convGroupsPerGroup > 1)
+      os << "        conv groups per group      " << convGroupsPerGroup
+         << " (" << canonical.numConvGroups << " groups of "
+         << canonical.inputChannelsPerConvGroup << " -> "
+         << canonical.outputChannelsPerConvGroup << " channels run as "
+         << g.groups << " of " << g.inChansPerGroup << " -> "
+         << g.outChansPerGroup << ", weights block-diagonal)\n";
     if (pointwiseOn) {
       const std::size_t nTiles = (g.outChansPerGroup + 63) / 64;
       const mxk::PointwiseLaunch l =

@@ -98,6 +98,21 @@ struct mxconv_plan {
   // byte offset paddedInputOffset, before every launch.
   std::size_t paddedInputChans = 0, paddedInputOffset = 0;
 
+  // Conv groups run as one by the matrix-core kernels (1: each by itself).
+  // A layer of many groups of a few channels (4 or 8 per group of 32, say)
+  // fills neither a 16-byte vector of input channels nor a tile of output
+  // channels; `convGroupsPerGroup` neighbouring groups are planned, packed
+  // and run as ONE group of that many times the channels, whose weights are
+  // block-diagonal - the groups' channels are neighbours in the tensors
+  // already, so only the weight packing knows.  The role of the reference
+  // planner's convGroupsPerGroup (lib/poplin/ConvPlan.cpp, the AMP and SLIC
+  // vertices that take several conv groups at once).  The packed-weights
+  // buffer then has room behind the packed weights for the block-diagonal
+  // weights in external order, `weightExpandElems` elements, which the
+  // packing fills first.
+  unsigned convGroupsPerGroup = 1;
+  std::size_t weightExpandElems = 0;
+
   std::size_t inputElems = 0, outputElems = 0, weightElems = 0,
               weightPackedElems = 0, biasElems = 0;
   std::size_t workspaceBytes = 0;
@@ -110,7 +125,7 @@ struct mxconv_plan {
     return weightElems * params.inputType.size();
   }
   std::size_t weightPackedBytes() const {
-    return weightPackedElems * params.inputType.size();
+    return (weightPackedElems + weightExpandElems) * params.inputType.size();
   }
   std::size_t biasBytes() const { return biasElems * params.outputType.size(); }
 

@@ -673,3 +673,50 @@ def test_pointwise_planner_choice_for_padded_rows():
     # not a multiple of eight: the big tile, channels padded in a copy
     assert "pointwise streaming variant" not in kernel_of(
         batch=2, field=(14, 14), ci=20, co=64)
+
+
+def test_planner_runs_small_conv_groups_as_one():
+    """Groups of fewer input channels than half a 128-byte slice: the
+    smallest number of groups that makes a whole slice runs as one."""
+    import json
+
+    def per_group(options=None, dtype=pa.HALF, out=None, **kw):
+        text = pa.Plan(make_params(dtype, out, kernel=(3, 3), pad=1,
+                                   batch=4, field=(14, 14), **kw),
+                       options).describe()
+        for line in text.splitlines():
+            if "conv groups per group" in line:
+                return int(line.split()[4])
+        return 1
+    assert per_group(ci=4, co=4, groups=32) == 16
+    assert per_group(ci=8, co=8, groups=32) == 8
+    assert per_group(ci=16, co=24, groups=12) == 4
+    assert per_group(ci=24, co=24, groups=6) == 3
+    assert per_group(dtype=pa.QUARTER, out=pa.HALF, ci=16, co=16,
+                     groups=16) == 8
+    # left alone: half a slice or more per group, depthwise, fused groups of
+    # more than 256 output channels, too few groups for a whole slice
+    assert per_group(ci=32, co=32, groups=8) == 1
+    assert per_group(ci=1, co=1, groups=64) == 1
+    assert per_group(ci=4, co=64, groups=32) == 1
+    assert per_group(ci=4, co=4, groups=8) == 1
+    # the weight update pass plans for the layer's own tensors
+    assert per_group({"pass": "TRAINING_WU"}, ci=4, co=4, groups=32) == 1
+    assert per_group({"pass": "TRAINING_BWD"}, ci=4, co=4, groups=32) == 16
+    # the reference's constraint, where it can be taken
+    def forced(n):
+        return {"planConstraints": json.dumps({"convGroupsPerGroup": n})}
+    assert per_group(forced(4), ci=4, co=4, groups=32) == 4
+    assert per_group(forced(1), ci=4, co=4, groups=32) == 1
+    assert per_group(forced(5), ci=4, co=4, groups=32) == 1
+    assert per_group(forced(2), ci=32, co=32, groups=8) == 2
+    # room for the block-diagonal weights behind the packed ones
+    p = make_params(pa.HALF, batch=4, field=(14, 14), kernel=(3, 3), ci=4,
+                    co=4, groups=32, pad=1)
+    plan, alone = pa.Plan(p), pa.Plan(p, forced(1))
+    external = 32 * 4 * 4 * 9 * 2
+    assert plan.buffer_bytes(pa.capi.BUF_WEIGHTS_EXTERNAL) == external
+    packed = 2 * 64 * 576 * 2
+    assert plan.buffer_bytes(pa.capi.BUF_WEIGHTS_PACKED) == \
+        packed + 16 * external
+    assert not plan.packs_like(alone)
