@@ -63,6 +63,12 @@ hipError_t launchFuseGroupWeights(const void *src, void *dst, uint64_t groups,
                                   uint64_t perGroup, uint64_t co, uint64_t ci,
                                   uint64_t taps, int elemBytes,
                                   hipStream_t stream);
+/// ... and back, for weight deltas: the diagonal blocks of
+/// [groups / perGroup][perGroup co][perGroup ci][taps] -> [groups][co][ci][taps].
+hipError_t launchUnfuseGroupWeights(const void *src, void *dst,
+                                    uint64_t groups, uint64_t perGroup,
+                                    uint64_t co, uint64_t ci, uint64_t taps,
+                                    int elemBytes, hipStream_t stream);
 hipError_t launchSwapBatchChans(const void *src, void *dst, uint32_t batch,
                                 uint32_t pixels, uint32_t groups,
                                 uint32_t chans, uint64_t strideG,

@@ -329,6 +329,28 @@ __global__ __launch_bounds__(256) void biasUpdateKernel(
   storeOut(biases, c, Load<T>::at(biases, c, 0) + scale * total);
 }
 
+/// The other way round, for weight deltas: the f diagonal blocks of every
+/// fused group of [G / f][f co][f ci][taps] -> [G][co][ci][taps].  One element
+/// of the result per thread.
+template <class T>
+__global__ __launch_bounds__(256) void
+unfuseGroupWeightsKernel(const T *__restrict__ src, T *__restrict__ dst,
+                         uint64_t f, uint64_t co, uint64_t ci, uint64_t taps,
+                         uint64_t total) {
+  const uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= total)
+    return;
+  const uint64_t tap = i % taps;
+  uint64_t rest = i / taps;
+  const uint64_t k = rest % ci;
+  rest /= ci;
+  const uint64_t n = rest % co;
+  const uint64_t g = rest / co;
+  const uint64_t fused = g / f, a = g % f;
+  dst[i] = src[((fused * f * co + a * co + n) * (f * ci) + a * ci + k) * taps +
+               tap];
+}
+
 /// Weights [G][co][ci][taps] of G conv groups -> [G / f][f co][f ci][taps] of
 /// G / f groups that each take f of them as one: block (a, b) of a fused
 /// group's f x f blocks of co x ci channels is group (f g' + a)'s weights
@@ -817,6 +839,32 @@ hipError_t launchBiasUpdate(int deltasType, const void *zDeltas, uint64_t rows,
     hipLaunchKernelGGL(biasUpdateKernel<__half>, grid2, block, 0, stream,
                        static_cast<__half *>(biases), partial, scale, channels,
                        splits);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launchUnfuseGroupWeights(const void *src, void *dst,
+                                    uint64_t groups, uint64_t perGroup,
+                                    uint64_t co, uint64_t ci, uint64_t taps,
+                                    int elemBytes, hipStream_t stream) {
+  const uint64_t total = groups * co * ci * taps;
+  if (total == 0)
+    return hipSuccess;
+  const uint64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffull || groups % perGroup != 0)
+    return hipErrorInvalidConfiguration;
+  const dim3 grid{uint32_t(blocks)}, block{256};
+  if (elemBytes == 4)
+    hipLaunchKernelGGL(unfuseGroupWeightsKernel<uint32_t>, grid, block, 0,
+                       stream, static_cast<const uint32_t *>(src),
+                       static_cast<uint32_t *>(dst), perGroup, co, ci, taps,
+                       total);
+  else if (elemBytes == 2)
+    hipLaunchKernelGGL(unfuseGroupWeightsKernel<uint16_t>, grid, block, 0,
+                       stream, static_cast<const uint16_t *>(src),
+                       static_cast<uint16_t *>(dst), perGroup, co, ci, taps,
+                       total);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

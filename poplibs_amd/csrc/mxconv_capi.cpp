@@ -1355,8 +1355,14 @@ size_t alignUp(size_t v) { return (v + 255) & ~size_t(255); }
 /// Where the weight update pass keeps its intermediates in the workspace.
 struct WuWorkspace {
   size_t input, weightsExternal, weightsPacked, output, deltas, planWorkspace,
-      total;
+      fusedDeltas, total;
 };
+
+/// Bytes of the weight deltas the pass hands back (of the layer's own groups,
+/// where the plan is for the layer with several groups taken as one).
+size_t wuResultBytes(const mxconv_plan *plan) {
+  return plan->outputBytes() / plan->wuGroupsPerGroup;
+}
 
 WuWorkspace wuWorkspace(const mxconv_plan *plan) {
   WuWorkspace w{};
@@ -1366,18 +1372,22 @@ WuWorkspace wuWorkspace(const mxconv_plan *plan) {
     at += alignUp(bytes);
     return offset;
   };
+  // (groups taken as one: the fused layer's deltas, whose diagonal blocks
+  // are the result)
+  if (plan->wuGroupsPerGroup > 1)
+    w.fusedDeltas = take(plan->outputBytes());
   if (plan->depthwiseWeightUpdate) {
     // the depthwise weight-delta kernel reads the layer's tensors as they
     // are: only its partial sums and, for the update, the deltas
     w.planWorkspace =
         take(mxk::depthwiseWeightDeltaWorkspaceBytes(plan->depthwiseForward));
-    w.deltas = take(plan->outputBytes());
+    w.deltas = take(wuResultBytes(plan));
     w.total = at;
     return w;
   }
   if (plan->denseWeightUpdate) {
     w.planWorkspace = take(mxk::wuTapWorkspaceBytes(plan->denseForward));
-    w.deltas = take(plan->outputBytes());
+    w.deltas = take(wuResultBytes(plan));
     w.total = at;
     return w;
   }
@@ -1385,7 +1395,7 @@ WuWorkspace wuWorkspace(const mxconv_plan *plan) {
   w.weightsExternal = take(plan->weightBytes());
   w.weightsPacked = take(plan->weightPackedBytes());
   w.output = take(plan->outputBytes());
-  w.deltas = take(plan->outputBytes());
+  w.deltas = take(wuResultBytes(plan));
   w.planWorkspace = take(plan->workspaceBytes);
   w.total = at;
   return w;
@@ -1398,9 +1408,40 @@ uint64_t product(const std::vector<std::size_t> &shape) {
   return n;
 }
 
+mxconv_status fusedWeightDeltas(const mxconv_plan *plan, const void *zDeltas,
+                                const void *acts, void *deltasOut, char *ws,
+                                mxconv_stream stream);
+
+/// The pass's result into `deltasOut`, [G][Co][Ci][kernel] of the layer.
 mxconv_status weightDeltas(const mxconv_plan *plan, const void *zDeltas,
                            const void *acts, void *deltasOut, char *ws,
                            mxconv_stream stream) {
+  const unsigned f = plan->wuGroupsPerGroup;
+  if (f == 1)
+    return fusedWeightDeltas(plan, zDeltas, acts, deltasOut, ws, stream);
+  // Planned for the layer with f groups taken as one: that layer's deltas
+  // into the workspace, their diagonal blocks out.
+  char *fused = ws + wuWorkspace(plan).fusedDeltas;
+  const mxconv_status st =
+      fusedWeightDeltas(plan, zDeltas, acts, fused, ws, stream);
+  if (st != MXCONV_OK)
+    return st;
+  const auto &p = plan->params;
+  uint64_t taps = 1;
+  for (auto k : p.getOutputFieldShape())
+    taps *= k;
+  return hipStatus(
+      mxk::launchUnfuseGroupWeights(
+          fused, deltasOut, uint64_t(p.numConvGroups) * f, f,
+          p.outputChannelsPerConvGroup / f, p.batchSize / f, taps,
+          int(p.outputType.size()), reinterpret_cast<hipStream_t>(stream)),
+      "weight deltas of the layer's own groups");
+}
+
+/// The weight deltas of the layer the plan was made for.
+mxconv_status fusedWeightDeltas(const mxconv_plan *plan, const void *zDeltas,
+                                const void *acts, void *deltasOut, char *ws,
+                                mxconv_stream stream) {
   // The pass's convolution (lib/poplin/Convolution.cpp:3437-3483): batch =
   // forward input channels, input channels = forward batch, kernel = forward
   // output field, output field = forward kernel.
@@ -1606,7 +1647,8 @@ mxconv_status mxconv_convolution_weight_update(const mxconv_plan *plan,
     return st;
   return hipStatus(mxk::launchScaledAdd(plan->params.outputType.id(),
                                         weights_external, 1.f, deltas, scale,
-                                        plan->outputElems,
+                                        plan->outputElems /
+                                            plan->wuGroupsPerGroup,
                                         reinterpret_cast<hipStream_t>(stream)),
                    "weight update");
 }

@@ -287,24 +287,34 @@ namespace {
 /// it can be (it divides the groups and the fused channels are whole 16-byte
 /// vectors) and means "by itself" elsewhere: the reference accepts values
 /// that only its own vertices give a meaning to.
+///
+/// A weight update pass (its parameters are getWeightUpdateParams of the
+/// layer's: batch = the layer's input channels, input channels = its batch)
+/// is planned for the layer with that many groups taken as one - the same
+/// rule on the layer's channels - and the diagonal blocks of the fused
+/// layer's weight deltas are what the pass hands back
+/// (mxconv_plan::wuGroupsPerGroup).
 unsigned chooseConvGroupsPerGroup(const ConvParams &p,
                                   const ConvOptions &options) {
   const auto &pc = options.planConstraints;
+  const bool wu = isWeightUpdatePass(options.pass);
   switch (options.pass) {
   case Pass::NONE:
   case Pass::INFERENCE_FWD:
   case Pass::TRAINING_FWD:
   case Pass::TRAINING_BWD:
+  case Pass::TRAINING_WU:
     break;
   default:
     return 1;
   }
   const std::size_t groups = p.numConvGroups;
-  const std::size_t ci = p.inputChannelsPerConvGroup;
+  const std::size_t ci = wu ? p.batchSize : p.inputChannelsPerConvGroup;
   const std::size_t co = p.outputChannelsPerConvGroup;
   const std::size_t eb = p.inputType.size();
   if (groups < 2 || ci == 0 || co == 0 || (ci == 1 && co == 1) ||
-      (!pc.kernel.empty() && pc.kernel != "igemm") || p.batchSize == 0)
+      (!pc.kernel.empty() && pc.kernel != "igemm") || p.batchSize == 0 ||
+      p.inputChannelsPerConvGroup == 0)
     return 1;
   auto usable = [&](std::size_t f) {
     return f >= 1 && groups % f == 0 && (f * ci * eb) % 16 == 0;
@@ -328,6 +338,16 @@ mxconv_plan makePlanWith(const ConvParams &params,
 mxconv_plan makePlan(const ConvParams &params, const ConvOptions &optionsIn) {
   const unsigned fuse =
       chooseConvGroupsPerGroup(params.canonicalize(), optionsIn);
+  if (fuse > 1 && isWeightUpdatePass(optionsIn.pass)) {
+    // the weight update pass of the layer with `fuse` groups taken as one
+    ConvParams fused = params;
+    fused.numConvGroups /= fuse;
+    fused.batchSize *= fuse;
+    fused.outputChannelsPerConvGroup *= fuse;
+    mxconv_plan plan = makePlanWith(fused, optionsIn, 1);
+    plan.wuGroupsPerGroup = fuse;
+    return plan;
+  }
   if (fuse > 1) {
     // (only the matrix-core kernels run groups as one)
     mxconv_plan plan = makePlanWith(params, optionsIn, fuse);
@@ -463,12 +483,13 @@ mxconv_plan makePlanWith(const ConvParams &params,
       // tiles, and poorly filled ones lose to the pass's own convolution
       // (N = 32, 28 x 28, 3 x 3: 32 groups of 16 -> 16 channels 420 against
       // 117 us, 8 groups of 32 -> 32 78 against 49, 2 groups of 64 -> 64 26
-      // against 26.5; without groups 16 -> 16 on 56 x 56 ties at 39 us and
-      // 32 -> 64 wins with 18 against 25).
+      // against 26.5, 4 groups of 64 -> 64 41 against 34 and 2 such groups on
+      // 56 x 56 70 against 52; without groups 16 -> 16 on 56 x 56 ties at
+      // 39 us and 32 -> 64 wins with 18 against 25).
       const std::size_t tileArea = std::size_t((f.ci + 127) / 128 * 128) *
                                    ((f.co + 127) / 128 * 128);
       const bool filled =
-          f.groups == 1 || std::size_t(f.ci) * f.co * 4 >= tileArea;
+          f.groups == 1 || std::size_t(f.ci) * f.co * 4 > tileArea;
       const bool worth =
           pixels >= 1024 && f.ci >= 16 && f.co >= 16 && filled;
       plan.denseWeightUpdate = (asked == 1 || worth) && mxk::wuTapTakes(f);
@@ -1147,7 +1168,10 @@ mxconv_plan makePlanWith(const ConvParams &params,
 std::string mxconv_plan::constraintsJson() const {
   std::ostringstream os;
   os << "{";
-  if (kernel == Kernel::IGEMM && canonical.numConvGroups > 1)
+  if (wuGroupsPerGroup > 1 ||
+      (madeForWeightUpdate && canonical.numConvGroups > 1))
+    os << "\"convGroupsPerGroup\": " << wuGroupsPerGroup << ", ";
+  else if (kernel == Kernel::IGEMM && canonical.numConvGroups > 1)
     os << "\"convGroupsPerGroup\": " << convGroupsPerGroup << ", ";
   os << "\"gfx950\": {";
   switch (kernel) {
@@ -1355,6 +1379,12 @@ std::string mxconv_plan::describe() const {
   os << "        zeroConv                   " << (zeroConv ? "true" : "false")
      << "\n";
   os << "        partialsType               float\n";
+  if (wuGroupsPerGroup > 1)
+    os << "        conv groups per group      " << wuGroupsPerGroup
+       << " (the weight update pass of the layer with that many of its "
+       << canonical.numConvGroups * wuGroupsPerGroup
+       << " groups taken as one; the diagonal blocks of the fused layer's "
+          "deltas are handed back)\n";
   if (kernel == Kernel::IGEMM) {
     const auto &g = igemm;
     const std::size_t m = std::size_t(g.batch) * g.outD * g.outH * g.outW;

@@ -112,6 +112,12 @@ struct mxconv_plan {
   // packing fills first.
   unsigned convGroupsPerGroup = 1;
   std::size_t weightExpandElems = 0;
+  // A weight update pass planned for the layer with that many conv groups
+  // taken as one (1: as it is): `params` are that fused layer's weight update
+  // parameters, the pass forms the fused layer's weight deltas
+  // [G / f][f co][f ci][kernel] in its workspace and hands back the f diagonal
+  // blocks of every fused group - the layer's own deltas [G][co][ci][kernel].
+  unsigned wuGroupsPerGroup = 1;
 
   std::size_t inputElems = 0, outputElems = 0, weightElems = 0,
               weightPackedElems = 0, biasElems = 0;

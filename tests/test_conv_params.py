@@ -700,9 +700,17 @@ def test_planner_runs_small_conv_groups_as_one():
     assert per_group(ci=1, co=1, groups=64) == 1
     assert per_group(ci=4, co=64, groups=32) == 1
     assert per_group(ci=4, co=4, groups=8) == 1
-    # the weight update pass plans for the layer's own tensors
-    assert per_group({"pass": "TRAINING_WU"}, ci=4, co=4, groups=32) == 1
     assert per_group({"pass": "TRAINING_BWD"}, ci=4, co=4, groups=32) == 16
+    # the weight update pass of such a layer is planned for the layer with
+    # the same groups taken as one
+    layer = make_params(pa.HALF, batch=4, field=(14, 14), kernel=(3, 3), ci=4,
+                        co=4, groups=32, pad=1)
+    wu = pa.WeightUpdatePlan(layer).describe()
+    assert "conv groups per group      16 (the weight update pass" in wu
+    assert "numConvGroups              2" in wu
+    assert "conv groups per group" not in pa.WeightUpdatePlan(
+        make_params(pa.HALF, batch=4, field=(14, 14), kernel=(3, 3), ci=32,
+                    co=32, groups=8, pad=1)).describe()
     # the reference's constraint, where it can be taken
     def forced(n):
         return {"planConstraints": json.dumps({"convGroupsPerGroup": n})}

@@ -138,3 +138,57 @@ def test_grouped_backward_pass(oracle):
     assert FUSED in plan.describe(), plan.describe()
     want = oracle.convolution_backward(p, dz, w, threads=8)
     np.testing.assert_array_equal(got, want)
+
+
+WU_CASES = [
+    # (layer, groups taken as one)
+    (dict(batch=4, field=(9, 8), kernel=(3, 3), ci=4, co=4, groups=32,
+          pad=1), 16),
+    (dict(batch=3, field=(12, 12), kernel=(3, 3), ci=8, co=16, groups=16,
+          pad=1, stride=2), 8),
+    (dict(batch=2, field=(10, 10), kernel=(1, 1), ci=16, co=8, groups=8), 4),
+    (dict(batch=4, field=(9, 8), kernel=(3, 3), ci=32, co=32, groups=4,
+          pad=1), 1),
+]
+
+
+@pytest.mark.parametrize("kw,expect", WU_CASES)
+@pytest.mark.parametrize("weight_deltas", [None, 0, 1])
+def test_grouped_weight_deltas(oracle, kw, expect, weight_deltas):
+    """The pass is planned for the layer with the groups taken as one and
+    hands back the diagonal blocks: +-1 tensors, exact.  Through the planner's
+    choice of kernel, the pass's own convolution (0) and the kernel that
+    reads the layer's tensors as they are (1)."""
+    from test_weight_update import run_weight_update
+    p = make_params(pa.HALF, pa.FLOAT, **kw)
+    print("case", p, weight_deltas, flush=True)
+    rng = np.random.default_rng(47)
+    G, Ci, Co = (p.numConvGroups, p.inputChannelsPerConvGroup,
+                 p.outputChannelsPerConvGroup)
+    x = rng.choice([-1.0, 1.0], (p.batchSize, G * Ci, *p.inputFieldShape))
+    dz = rng.choice([-1.0, 1.0],
+                    (p.batchSize, G * Co, *p.getOutputFieldShape()))
+    options = None if weight_deltas is None else _opts(
+        None, weightDeltas=weight_deltas)
+    got, plan = run_weight_update(p, x.astype(np.float16),
+                                  dz.astype(np.float16), options)
+    assert ("%s      %d (the weight update" % (FUSED, expect)
+            in plan.describe()) == (expect > 1), plan.describe()
+    np.testing.assert_array_equal(got, oracle.weight_deltas(p, x, dz,
+                                                            threads=8))
+
+
+def test_grouped_weight_update_in_place(oracle):
+    from test_weight_update import run_weight_update
+    p = make_params(pa.HALF, pa.HALF, batch=2, field=(8, 7), kernel=(3, 3),
+                    ci=4, co=8, groups=32, pad=1)
+    rng = np.random.default_rng(48)
+    x = rng.choice([-1.0, 1.0], (2, 32 * 4, 8, 7))
+    dz = rng.choice([-1.0, 1.0], (2, 32 * 8, 8, 7))
+    w = rng.integers(-3, 4, (32, 8, 4, 3, 3)).astype(np.float64)
+    got, plan = run_weight_update(p, x.astype(np.float16),
+                                  dz.astype(np.float16), None,
+                                  w.astype(np.float16), -0.25)
+    assert FUSED in plan.describe()
+    np.testing.assert_array_equal(
+        got, w - 0.25 * oracle.weight_deltas(p, x, dz, threads=8))
