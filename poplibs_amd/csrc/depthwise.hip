@@ -91,7 +91,15 @@ struct DwArgs {
 
 /// KH, KW > 0: kernel extents known at compile time (taps fully unrolled);
 /// 0: taken from the descriptor.
-template <int KH, int KW, class OutT>
+/// PX > 0 (unit stride and dilation, KH and KW known): a thread forms PX
+/// neighbouring output pixels of a row at once - for large kernels, where the
+/// multiply-adds, not the bytes, are what a layer costs (7 x 7: 49 per
+/// output) and a pixel at a time spends an LDS read and a tap load on every
+/// one of them.  Per kernel row the thread reads the row's KW taps (kept in
+/// LDS behind the patch, one copy per workgroup) and the PX + KW - 1 input
+/// vectors under them once and multiplies PX x KW times: 13 multiply-adds per
+/// 16-byte LDS read at 7 x 7 and PX = 7, against one.
+template <int KH, int KW, class OutT, int PX = 0>
 __global__ __launch_bounds__(kThreads) void depthwiseKernel(
     DwArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
@@ -185,6 +193,73 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
   for (int i = 0; i != 8; ++i)
     biasV[i] = bias ? Load<OutT>::at(bias, c + i, 0) : 0.0f;
 
+  if constexpr (PX != 0) {
+    static_assert(KH != 0 && KW != 0, "strips want the kernel's extents");
+    // the taps, [tap][vecBlock] behind the patch
+    uint4 *tapsLds =
+        reinterpret_cast<uint4 *>(lds + a.patchH * a.rowPitch * 16);
+    for (uint32_t i = threadIdx.x; i < KH * KW * a.vecBlock; i += kThreads) {
+      const uint32_t tap = i / a.vecBlock, tv = i - tap * a.vecBlock;
+      tapsLds[i] = *reinterpret_cast<const uint4 *>(
+          w + tap * d.channels + (cv0 + (tv < nvec ? tv : 0)) * 8);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's loads landed
+    __syncthreads();
+    const uint32_t strips = (d.tileW + PX - 1) / PX;
+    const uint32_t items = d.tileH * strips * a.vecBlock;
+    const uint32_t owEnd = min(d.outW, ow0 + d.tileW);
+    for (uint32_t item = threadIdx.x; item < items; item += kThreads) {
+      const uint32_t iv = item % a.vecBlock, rest = item / a.vecBlock;
+      const uint32_t sy = rest / strips, sx = (rest - sy * strips) * PX;
+      const uint32_t oh = oh0 + sy;
+      if (iv >= nvec || oh >= d.outH || ow0 + sx >= owEnd)
+        continue;
+      const uint32_t ic = (cv0 + iv) * 8;
+      float acc[PX][8];
+#pragma unroll
+      for (int px = 0; px != PX; ++px)
+#pragma unroll
+        for (int i = 0; i != 8; ++i)
+          acc[px][i] = bias ? Load<OutT>::at(bias, ic + i, 0) : 0.0f;
+      const char *rowAt = lds + (sy * a.rowPitch + sx * a.vecBlock + iv) * 16;
+      // (a kernel row at a time: unrolled over the rows the compiler asks for
+      // every row's taps and inputs at once, 560 registers)
+#pragma unroll 1
+      for (int kh = 0; kh != KH; ++kh) {
+        Vec8 k[KW], x[PX + KW - 1];
+#pragma unroll
+        for (int kw = 0; kw != KW; ++kw)
+          k[kw].raw = tapsLds[(kh * KW + kw) * a.vecBlock + iv];
+        // (a strip that ends beyond the tile reads on into the row's padding
+        // or the next row - inside the LDS - for pixels that are not stored)
+#pragma unroll
+        for (int j = 0; j != PX + KW - 1; ++j)
+          x[j].raw = *reinterpret_cast<const uint4 *>(rowAt +
+                                                      j * a.vecBlock * 16);
+#pragma unroll
+        for (int px = 0; px != PX; ++px)
+#pragma unroll
+          for (int kw = 0; kw != KW; ++kw)
+#pragma unroll
+            for (int i = 0; i != 4; ++i) {
+              const float2 xf = __half22float2(x[px + kw].h2[i]);
+              const float2 kf = __half22float2(k[kw].h2[i]);
+              acc[px][2 * i] = fmaf(xf.x, kf.x, acc[px][2 * i]);
+              acc[px][2 * i + 1] = fmaf(xf.y, kf.y, acc[px][2 * i + 1]);
+            }
+        rowAt += a.rowPitch * 16;
+      }
+      OutT *to = out +
+                 ((size_t(b) * d.outH + oh) * d.outW + ow0 + sx) * d.channels +
+                 ic;
+#pragma unroll
+      for (int px = 0; px != PX; ++px)
+        if (ow0 + sx + px < owEnd)
+          StoreVec<OutT>::put(to + size_t(px) * d.channels, acc[px]);
+    }
+    return;
+  }
+
   __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's loads landed
   __syncthreads();
 
@@ -241,16 +316,22 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
     }
 }
 
-template <int KH, int KW, class OutT>
+constexpr uint32_t kLdsMost = kDepthwiseTileLdsMost;
+
+template <int KH, int KW, class OutT, int PX = 0>
 hipError_t run(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
                const void *in, const void *w, const void *bias, void *out,
                hipStream_t stream) {
+  // (strips: the taps behind the patch)
+  ldsBytes += PX ? KH * KW * a.vecBlock * 16 : 0;
+  if (ldsBytes > kLdsMost)
+    return hipErrorInvalidConfiguration;
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void *>(&depthwiseKernel<KH, KW, OutT>),
-      hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+      reinterpret_cast<const void *>(&depthwiseKernel<KH, KW, OutT, PX>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMost);
   if (attr != hipSuccess)
     return attr;
-  hipLaunchKernelGGL((depthwiseKernel<KH, KW, OutT>), dim3(blocks),
+  hipLaunchKernelGGL((depthwiseKernel<KH, KW, OutT, PX>), dim3(blocks),
                      dim3(kThreads), ldsBytes, stream, a,
                      static_cast<const __half *>(in),
                      static_cast<const __half *>(w),
@@ -264,12 +345,35 @@ hipError_t runKernelShape(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
                           void *out, hipStream_t stream) {
   if (a.d.kH == 3 && a.d.kW == 3)
     return run<3, 3, OutT>(a, blocks, ldsBytes, in, w, bias, out, stream);
+  const bool unit = a.d.strideH == 1 && a.d.strideW == 1 && a.d.dilH == 1 &&
+                    a.d.dilW == 1;
+  if (a.d.kH == 7 && a.d.kW == 7 && unit && a.d.stripPixels == 7)
+    return run<7, 7, OutT, 7>(a, blocks, ldsBytes, in, w, bias, out, stream);
+  if (a.d.kH == 7 && a.d.kW == 7 && unit && a.d.stripPixels == 4)
+    return run<7, 7, OutT, 4>(a, blocks, ldsBytes, in, w, bias, out, stream);
   if (a.d.kH == 5 && a.d.kW == 5)
     return run<5, 5, OutT>(a, blocks, ldsBytes, in, w, bias, out, stream);
   return run<0, 0, OutT>(a, blocks, ldsBytes, in, w, bias, out, stream);
 }
 
 } // namespace
+
+bool depthwiseStripTakes(const DepthwiseDesc &d) {
+  return d.kH == 7 && d.kW == 7 && d.strideH == 1 && d.strideW == 1 &&
+         d.dilH == 1 && d.dilW == 1 && d.inDilH == 1 && d.inDilW == 1 &&
+         d.channels % 8 == 0;
+}
+
+uint64_t depthwiseTileLdsBytes(const DepthwiseDesc &d) {
+  const uint64_t vecs = d.channels / 8, vecBlock = vecs <= 16 ? vecs : 16;
+  const uint64_t patchH = uint64_t(d.tileH - 1) * d.strideH +
+                          uint64_t(d.kH - 1) * d.dilH + 1;
+  const uint64_t patchW = uint64_t(d.tileW - 1) * d.strideW +
+                          uint64_t(d.kW - 1) * d.dilW + 1;
+  const uint64_t rowPitch = (patchW * vecBlock + 63) / 64 * 64;
+  return patchH * rowPitch * 16 +
+         (d.stripPixels ? uint64_t(d.kH) * d.kW * vecBlock * 16 : 0);
+}
 
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
@@ -330,7 +434,9 @@ hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
   const uint64_t ldsBytes = uint64_t(a.patchH) * a.rowPitch * 16;
   const uint64_t blocks =
       uint64_t(d.batch) * a.tilesH * a.tilesW * a.vecBlocks;
-  if (inBytes >= kOutOfRange || ldsBytes > 64 * 1024 || blocks > 0x7fffffffull)
+  if (inBytes >= kOutOfRange || blocks > 0x7fffffffull ||
+      depthwiseTileLdsBytes(d) > (d.stripPixels ? kLdsMost : 64 * 1024) ||
+      (d.stripPixels != 0 && !depthwiseStripTakes(d)))
     return hipErrorInvalidConfiguration;
   a.inBytes = uint32_t(inBytes);
   if (outType == kHalf)

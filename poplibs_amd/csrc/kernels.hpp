@@ -326,7 +326,17 @@ struct DepthwiseDesc {
   // Zeros stuffed between input elements, as in IgemmDesc; other than 1 the
   // direct kernel of launchDepthwiseDirect runs.
   uint32_t inDilH = 1, inDilW = 1;
+  // The LDS-tiled kernel with a thread forming that many neighbouring output
+  // pixels of a row at once (7 x 7 taps, unit stride and dilation:
+  // depthwiseStripTakes): 4 or 7; 0 = a pixel at a time.
+  uint32_t stripPixels = 0;
 };
+/// True for the layers whose LDS-tiled kernel can work in strips of pixels.
+bool depthwiseStripTakes(const DepthwiseDesc &d);
+/// LDS of a workgroup of the LDS-tiled kernel for d's tile: the input patch
+/// and, with strips, the taps; what it may take at most.
+uint64_t depthwiseTileLdsBytes(const DepthwiseDesc &d);
+constexpr uint32_t kDepthwiseTileLdsMost = 80 * 1024;
 /// True for the shapes launchDepthwise3x3 takes.
 bool depthwise3x3Takes(const DepthwiseDesc &d, int inType);
 hipError_t launchDepthwise3x3(const DepthwiseDesc &d, int inType,

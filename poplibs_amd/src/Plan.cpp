@@ -204,6 +204,60 @@ std::pair<unsigned, unsigned> chooseDepthwiseTile(const Simple2D &s,
   return {0, 0};
 }
 
+/// Tile and strip of the LDS-tiled depthwise kernel where a thread forms a
+/// strip of neighbouring pixels (mxk::depthwiseStripTakes): such layers cost
+/// what their multiply-adds cost, so the tile is the one that keeps most of a
+/// workgroup's 256 threads busy - rows x strips x channel vectors close to a
+/// multiple of 256, few rows beyond the field's last, strips of seven pixels
+/// where the tile's width is a multiple of seven and of four elsewhere
+/// (ConvNeXt's 7 x 7 field: two strips of four, 224 threads, against one of
+/// seven, 112) - within the LDS two workgroups of a CU can have.
+/// Busy share of a workgroup's threads with strips of `px` pixels on a tile.
+double stripFill(const mxk::DepthwiseDesc &d, unsigned th, unsigned tw,
+                 unsigned px) {
+  const unsigned vb = std::min(d.channels / 8, 16u);
+  const unsigned strips = (tw + px - 1) / px;
+  const double lanes = double(th) * strips * vb;
+  return lanes / (std::ceil(lanes / 256.0) * 256.0) * double(tw) /
+         (strips * px);
+}
+
+/// Strips of seven pixels where the tile's width is a multiple of seven and
+/// that keeps at least as many threads busy as strips of four.
+unsigned stripPixelsFor(const mxk::DepthwiseDesc &d, unsigned th,
+                        unsigned tw) {
+  return tw % 7 == 0 && stripFill(d, th, tw, 7) >= stripFill(d, th, tw, 4)
+             ? 7
+             : 4;
+}
+
+void chooseDepthwiseStripTile(mxk::DepthwiseDesc &d) {
+  const unsigned vecs = d.channels / 8, vb = std::min(vecs, 16u);
+  // (channel blocks of 16 vectors: the last block's share of busy lanes)
+  const double chanFill =
+      double(vecs) / double((vecs + vb - 1) / vb * vb);
+  double best = 0;
+  mxk::DepthwiseDesc chosen = d;
+  for (unsigned tw = 1; tw <= std::min(16u, d.outW); ++tw)
+    for (unsigned th = 1; th <= std::min(32u, d.outH); ++th) {
+      mxk::DepthwiseDesc t = d;
+      t.tileH = th, t.tileW = tw, t.stripPixels = stripPixelsFor(d, th, tw);
+      if (mxk::depthwiseTileLdsBytes(t) > mxk::kDepthwiseTileLdsMost)
+        break;
+      const double edgeH =
+          double(d.outH) / double((d.outH + th - 1) / th * th);
+      const double edgeW =
+          double(d.outW) / double((d.outW + tw - 1) / tw * tw);
+      // (the patch's halo is loaded, not multiplied: a quarter's weight)
+      const double halo = double(th) * tw / (double(th + 6) * (tw + 6));
+      const double score = stripFill(d, th, tw, t.stripPixels) * edgeH *
+                           edgeW * chanFill * (0.75 + 0.25 * halo);
+      if (score > best)
+        best = score, chosen = t;
+    }
+  d = chosen;
+}
+
 } // namespace
 
 namespace {
@@ -1101,6 +1155,10 @@ mxconv_plan makePlanWith(const ConvParams &params,
     d.loH = s.loH, d.hiH = s.hiH, d.loW = s.loW, d.hiW = s.hiW;
     d.tileH = dwTile.first, d.tileW = dwTile.second;
     d.inDilH = s.inDilH, d.inDilW = s.inDilW;
+    // 7 x 7 taps at unit stride: a thread forms a strip of neighbouring
+    // pixels, and the tile is chosen to fill the workgroup's 256 threads.
+    if (mxk::depthwiseStripTakes(d) && !(pc.tileH || pc.tileW))
+      chooseDepthwiseStripTile(d);
     // An explicit tile asks for the LDS-tiled kernel.
     d.dense3x3 = !s.inputDilated() && !(pc.tileH || pc.tileW) &&
                  mxk::depthwise3x3Takes(d, mxk::kHalf);
@@ -1142,10 +1200,10 @@ mxconv_plan makePlanWith(const ConvParams &params,
     if (!s.inputDilated() && (pc.tileH || pc.tileW)) {
       d.tileH = pc.tileH ? pc.tileH : d.tileH;
       d.tileW = pc.tileW ? pc.tileW : d.tileW;
-      const std::size_t vb = std::min<std::size_t>(p.numConvGroups / 8, 16);
-      const std::size_t ph = (d.tileH - 1) * d.strideH + (d.kH - 1) * d.dilH + 1;
-      const std::size_t pw = (d.tileW - 1) * d.strideW + (d.kW - 1) * d.dilW + 1;
-      if (ph * ((pw * vb + 63) / 64 * 64) * 16 > 64 * 1024)
+      if (mxk::depthwiseStripTakes(d))
+        d.stripPixels = stripPixelsFor(d, d.tileH, d.tileW);
+      if (mxk::depthwiseTileLdsBytes(d) >
+          (d.stripPixels ? mxk::kDepthwiseTileLdsMost : 64 * 1024))
         throw poplar::invalid_option(
             "planConstraints gfx950 tileH x tileW: the input patch of such a "
             "tile does not fit 64 KB of LDS");
@@ -1482,7 +1540,13 @@ std::string mxconv_plan::describe() const {
     os << "        channels                   " << d.channels << "\n";
     if (!d.dense3x3)
       os << "        output tile H x W          " << d.tileH << " x "
-         << d.tileW << "\n";
+         << d.tileW
+         << (d.stripPixels == 7
+                 ? ", a strip of 7 neighbouring pixels per thread"
+                 : d.stripPixels == 4
+                       ? ", a strip of 4 neighbouring pixels per thread"
+                       : "")
+         << "\n";
     if (d.dense3x3 == 2) {
       const mxk::DepthwiseRowsLaunch l = mxk::depthwiseRowsLaunchShape(d);
       os << "        workgroups                 " << l.workgroups << " on "

@@ -728,3 +728,38 @@ def test_planner_runs_small_conv_groups_as_one():
     assert plan.buffer_bytes(pa.capi.BUF_WEIGHTS_PACKED) == \
         packed + 16 * external
     assert not plan.packs_like(alone)
+
+
+def test_depthwise_7x7_tiles_fill_the_workgroup():
+    """7 x 7 taps at unit stride: a thread forms a strip of neighbouring
+    pixels; the planner's tile keeps most of the 256 threads busy."""
+    def tile(**kw):
+        text = pa.Plan(make_params(pa.HALF, batch=32, kernel=(7, 7), pad=3,
+                                   **kw)).describe()
+        line = [l for l in text.splitlines() if "output tile H x W" in l][0]
+        return " ".join(line.split()[5:])
+    # 12 channel vectors x 7 rows x 3 strips of 4 = 252 threads
+    assert tile(field=(56, 56), groups=96) == \
+        "7 x 12, a strip of 4 neighbouring pixels per thread"
+    # 16 x 7 x 2 strips of 7 = 224
+    assert tile(field=(14, 14), groups=384) == \
+        "7 x 14, a strip of 7 neighbouring pixels per thread"
+    # a 7 x 7 field: two strips of four (224 threads) rather than one of
+    # seven (112)
+    assert tile(field=(7, 7), groups=768) == \
+        "7 x 7, a strip of 4 neighbouring pixels per thread"
+    # strided or dilated 7 x 7, and other kernels: a pixel at a time
+    assert "strip" not in tile(field=(28, 28), groups=64, stride=2)
+    assert "strip" not in pa.Plan(make_params(
+        pa.HALF, batch=4, field=(28, 28), kernel=(9, 9), groups=64,
+        pad=4)).describe()
+    # a forced tile keeps the strips; one that does not fit is refused
+    forced = pa.Plan(make_params(pa.HALF, batch=4, field=(28, 28),
+                                 kernel=(7, 7), groups=64, pad=3),
+                     {"planConstraints":
+                      '{"gfx950": {"tileH": 5, "tileW": 14}}'}).describe()
+    assert "5 x 14, a strip of 4 neighbouring pixels" in forced
+    with pytest.raises(MxconvError):
+        pa.Plan(make_params(pa.HALF, batch=4, field=(64, 64), kernel=(7, 7),
+                            groups=128, pad=3),
+                {"planConstraints": '{"gfx950": {"tileH": 32, "tileW": 16}}'})
