@@ -282,13 +282,16 @@ struct PointwiseDesc {
   uint32_t groups, inChansPerGroup, outChansPerGroup;
   // 64-channel tiles of the output a workgroup owns: 0 = the launch's choice
   uint32_t chanTiles = 0;
+  // bytes of an input element: 2 (fp16) or 1 (fp8)
+  uint32_t elemBytes = 2;
 };
 bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType);
 /// Whether a workgroup can own `chanTiles` 64-channel tiles of this layer's
 /// output (they divide the layer's; 4 at most with 64 input channels, 2 with
 /// 128 or 256, 1 with 512).
 bool pointwiseChanTilesOk(const PointwiseDesc &d, uint32_t chanTiles);
-/// Elements of the packed weights ([G][32-channel block][k-slice][lane][8]).
+/// Elements of the packed weights ([G][32-channel block][32-byte k-slice]
+/// [lane][16 bytes]).
 uint64_t pointwisePackedElems(const PointwiseDesc &d);
 hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
                                       void *dst, hipStream_t stream,
@@ -304,7 +307,8 @@ struct PointwiseLaunch {
 PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus);
 hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
-                           const void *bias, void *out, hipStream_t stream);
+                           const void *bias, void *out, const QuarterInfo &q,
+                           hipStream_t stream);
 
 /// Depthwise (one input and one output channel per group) direct convolution,
 /// 2-D field, stride, zero padding, kernel dilation.

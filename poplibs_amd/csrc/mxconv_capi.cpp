@@ -177,7 +177,7 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
     }
     if (plan->pointwiseOn)
       return hipStatus(mxk::launchPointwise(plan->pointwise, inType, outType,
-                                            in, w, bias, out, s),
+                                            in, w, bias, out, q, s),
                        "pointwise convolution launch");
     if (plan->paddedInputChans) {
       // the kernel reads whole 16-byte vectors of channels: give it a copy

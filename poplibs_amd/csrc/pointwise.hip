@@ -49,6 +49,12 @@ constexpr uint32_t pwPaddedChans(uint32_t ci) {
   return p;
 }
 
+/// A layer's input channels per group in units of two bytes - fp16 channels,
+/// or pairs of fp8 ones: rows, tiles and rings are a matter of bytes.
+constexpr uint32_t pwRowChans(const PointwiseDesc &d) {
+  return d.inChansPerGroup * d.elemBytes / 2;
+}
+
 constexpr int kPwChans = 64;         // output channels per workgroup
 constexpr int kPwStageRow = 64 + 16; // staging: 64 bytes of a pixel + padding
 constexpr int kPwPairRow = 128 + 16; // ... 128 bytes: two blocks' channels
@@ -60,7 +66,45 @@ struct PwArgs {
   uint32_t nBlocks;    // 32-channel blocks per group in the packed weights
   uint32_t walkers;    // workgroups sharing the pixel tiles of one (g, nTile)
   uint32_t inBytes, wBytes;
+  // fp8: 2^(scaleIn + scaleWeights), applied to the sums on their way out,
+  // and its inverse, by which the bias enters them
+  float scale, invScale;
 };
+
+/// One 32-byte k-slice of a 32 x 32 block: `w` and `x` are a lane's 16 bytes
+/// of the weights' and the pixels' rows.  F = 0: fp16, one MFMA of K = 16
+/// (the lane's 8 halves are k = 8 (lane / 32) ...).  F > 0: fp8, activations'
+/// format (F - 1) & 1 and weights' (F - 1) >> 1 (0 = E4M3, 1 = E5M2): two MFMAs
+/// of K = 16 on the low and the high 8 bytes - which 16 channels of the slice
+/// a lane multiplies does not matter as long as the weights are packed alike.
+template <int F>
+__device__ __forceinline__ floatx16 pwMma(const uintx4 &w, const uintx4 &x,
+                                          floatx16 acc) {
+  if constexpr (F == 0) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+        __builtin_bit_cast(half8, w), __builtin_bit_cast(half8, x), acc, 0, 0,
+        0);
+  } else {
+    const long w0 = long(uint64_t(w.x) | (uint64_t(w.y) << 32));
+    const long w1 = long(uint64_t(w.z) | (uint64_t(w.w) << 32));
+    const long x0 = long(uint64_t(x.x) | (uint64_t(x.y) << 32));
+    const long x1 = long(uint64_t(x.z) | (uint64_t(x.w) << 32));
+    constexpr int FA = (F - 1) & 1, FB = (F - 1) >> 1;
+    if constexpr (FB == 0 && FA == 0) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(w0, x0, acc, 0, 0, 0);
+      return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(w1, x1, acc, 0, 0, 0);
+    } else if constexpr (FB == 0 && FA == 1) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_bf8(w0, x0, acc, 0, 0, 0);
+      return __builtin_amdgcn_mfma_f32_32x32x16_fp8_bf8(w1, x1, acc, 0, 0, 0);
+    } else if constexpr (FB == 1 && FA == 0) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_fp8(w0, x0, acc, 0, 0, 0);
+      return __builtin_amdgcn_mfma_f32_32x32x16_bf8_fp8(w1, x1, acc, 0, 0, 0);
+    } else {
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(w0, x0, acc, 0, 0, 0);
+      return __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(w1, x1, acc, 0, 0, 0);
+    }
+  }
+}
 
 /// KS: k-slices of 16 channels (Ci / 16).  TM: pixels per tile (32, 64, 128);
 /// the workgroup has TM / 16 compute waves and LW loader waves, which take
@@ -70,7 +114,9 @@ struct PwArgs {
 /// the channels reads its input once per share, so fewer, wider shares read
 /// less - 64 -> 256 channels on N = 32, 56 x 56: four shares of 64 re-read
 /// 13 MB four times beside 51 MB of output.
-template <int KS, int TM, int NB, int LW, int NT, class OutT>
+/// F: the operands' type, see pwMma (a k-slice is 32 bytes of a row: 16 fp16
+/// channels or 32 fp8 ones).
+template <int KS, int TM, int NB, int LW, int NT, class OutT, int F = 0>
 __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
     PwArgs a, const char *__restrict__ in, const char *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
@@ -106,8 +152,9 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
   const uint32_t walker = (logical / a.nTiles) % a.walkers;
   const uint32_t g = logical / (a.walkers * a.nTiles);
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
-  const uint32_t pixelBytes = d.groups * d.inChansPerGroup * 2;
-  const uint32_t groupBytes = d.inChansPerGroup * 2; // (may be below kRow)
+  const uint32_t groupBytes =
+      d.inChansPerGroup * d.elemBytes; // (may be below kRow)
+  const uint32_t pixelBytes = d.groups * groupBytes;
 
   if (wave >= kComputeWaves) {
     const int loader = wave - kComputeWaves;
@@ -152,7 +199,7 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
   // ---- compute waves.  This wave's weights -> registers: block nb of the
   // two 32-channel blocks, every k-slice.
   const int mb = wave >> 1, nb = wave & 1;
-  half8 wf[NT][KS];
+  uintx4 wf[NT][KS];
 #pragma unroll
   for (int nt = 0; nt != NT; ++nt) {
     const uintx4 *src =
@@ -160,8 +207,11 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
         (size_t(g * a.nBlocks + nTile * NT * 2 + nb * NT + nt) * KS) * 64 + lane;
 #pragma unroll
     for (int ks = 0; ks != KS; ++ks)
-      wf[nt][ks] = __builtin_bit_cast(half8, src[ks * 64]);
+      wf[nt][ks] = src[ks * 64];
   }
+  // (fp8: the sums are scaled on their way out, so the bias enters them
+  // divided by the scale - a power of two)
+  const float biasScale = F == 0 ? 1.0f : a.invScale;
   // One channel tile: the bias of this lane's channels 8 q + 4 (lane / 32) +
   // e stays in registers.  More: the workgroup's bias waits in LDS (registers
   // hold the weights), visible to all behind the first tile's barrier.
@@ -172,7 +222,8 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
       const uint32_t n =
           nTile * kPwChans + nb * 32 + 8 * (v / 4) + 4 * (lane >> 5) + v % 4;
       biasV[v] = bias && n < d.outChansPerGroup
-                     ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
+                     ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0) *
+                           biasScale
                      : 0.0f;
     }
   }
@@ -182,7 +233,8 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
     for (uint32_t i = t; i < NT * kPwChans; i += kComputeWaves * 64) {
       const uint32_t n = nTile * NT * kPwChans + i;
       biasLds[i] = n < d.outChansPerGroup
-                       ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0)
+                       ? Load<OutT>::at(bias, g * d.outChansPerGroup + n, 0) *
+                             biasScale
                        : 0.0f;
     }
     MXK_WAIT_LGKMCNT0();
@@ -237,12 +289,11 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
         }
 #pragma unroll
         for (int ks = 0; ks != KS; ++ks) {
-          const half8 x = *reinterpret_cast<const half8 *>(
+          const uintx4 x = *reinterpret_cast<const uintx4 *>(
               rowPtr + (((ks * 2 + half) ^ swizzle) << 4));
 #pragma unroll
           for (int j = 0; j != 2; ++j)
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                wf[2 * np + j][ks], x, acc[j], 0, 0, 0);
+            acc[j] = pwMma<F>(wf[2 * np + j][ks], x, acc[j]);
         }
 #pragma unroll
         for (int ph = 0; ph != 2; ++ph) {
@@ -254,7 +305,8 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
                 float v[4];
 #pragma unroll
                 for (int e = 0; e != 4; ++e)
-                  v[e] = acc[j][q * 4 + e];
+                  v[e] = F == 0 ? acc[j][q * 4 + e]
+                                : acc[j][q * 4 + e] * a.scale;
                 storeOut4(
                     reinterpret_cast<OutT *>(stage + (lane & 15) * kPwPairRow) +
                         (32 * j + 8 * q + 4 * half),
@@ -305,10 +357,9 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
       }
 #pragma unroll
       for (int ks = 0; ks != KS; ++ks) {
-        const half8 x = *reinterpret_cast<const half8 *>(
+        const uintx4 x = *reinterpret_cast<const uintx4 *>(
             rowPtr + (((ks * 2 + half) ^ swizzle) << 4));
-        acc =
-            __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[nt][ks], x, acc, 0, 0, 0);
+        acc = pwMma<F>(wf[nt][ks], x, acc);
       }
       // lane = pixel lane % 32, registers = channels 8 (v / 4) + 4 (lane /
       // 32) + v % 4: transpose through this wave's staging block and store.
@@ -320,7 +371,7 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
           float v[4];
 #pragma unroll
           for (int e = 0; e != 4; ++e)
-            v[e] = acc[q * 4 + e];
+            v[e] = F == 0 ? acc[q * 4 + e] : acc[q * 4 + e] * a.scale;
           storeOut4(
               reinterpret_cast<OutT *>(stage + (lane & 31) * kPwStageRow) +
                   (8 * q + 4 * half - pass * kPassChans),
@@ -352,30 +403,30 @@ __global__ __launch_bounds__(TM * 4 + 64 * LW) void pointwiseKernel(
   }
 }
 
-/// Weights [G][Co][Ci] -> [G][32-channel block][k-slice][lane][8 halves]:
-/// lane l of a slice holds channel l % 32 of the block, input channels
-/// 16 slice + 8 (l / 32) ... + 8 - the row operand of v_mfma_f32_32x32x16_f16.
-/// Channels past Co are zero, and so are input channels past Ci (the slices
-/// run to the padded row).
+/// Weights [G][Co][Ci] -> [G][32-channel block][k-slice][lane][16 bytes]:
+/// lane l of a slice holds channel l % 32 of the block, and of its input
+/// channels the E = 8 (fp16) or 16 (fp8) from 2 E slice + E (l / 32) on - the
+/// row operand of pwMma.  Channels past Co are zero, and so are input channels
+/// past Ci (the slices run to the padded row, `slices` of 32 bytes).
+template <class T>
 __global__ __launch_bounds__(256) void packPointwiseWeightsKernel(
-    const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, uint32_t co,
-    uint32_t ci, uint32_t ciPadded, uint32_t nBlocks, uint64_t total,
-    bool chansTransposed) {
+    const T *__restrict__ src, T *__restrict__ dst, uint32_t co, uint32_t ci,
+    uint32_t slices, uint32_t nBlocks, uint64_t total, bool chansTransposed) {
+  constexpr uint32_t E = 16 / sizeof(T);
   const uint64_t tid = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= total)
     return;
-  const uint32_t e = uint32_t(tid & 7), lane = uint32_t(tid >> 3) & 63;
-  const uint32_t slices = ciPadded / 16;
-  uint64_t r = tid >> 9;
+  const uint32_t e = uint32_t(tid % E), lane = uint32_t(tid / E) & 63;
+  uint64_t r = tid / (64 * E);
   const uint32_t ks = uint32_t(r % slices);
   r /= slices;
   const uint32_t block = uint32_t(r % nBlocks);
   const uint64_t g = r / nBlocks;
   const uint32_t n = block * 32 + (lane & 31);
-  const uint32_t k = ks * 16 + 8 * (lane >> 5) + e;
+  const uint32_t k = ks * 2 * E + E * (lane >> 5) + e;
   // source [G][Co][Ci], or [G][Ci][Co] (a matrix multiplication's right-hand
   // side)
-  dst[tid] = n >= co || k >= ci ? uint16_t(0)
+  dst[tid] = n >= co || k >= ci ? T(0)
              : chansTransposed  ? src[(g * ci + k) * co + n]
                                 : src[(g * co + n) * ci + k];
 }
@@ -436,10 +487,10 @@ constexpr uint32_t ldsBytesOf(PwShape s, uint32_t ci, uint32_t nt = 1) {
 uint32_t chanTilesFor(const PointwiseDesc &d, uint32_t cus) {
   if (d.chanTiles)
     return d.chanTiles; // asked for by name (checked by pointwiseTakes)
-  const PwShape s = shapeFor(d.inChansPerGroup);
+  const PwShape s = shapeFor(pwRowChans(d));
   const uint64_t mTiles = (uint64_t(d.batch) * d.pixels + s.tm - 1) / s.tm;
   const uint64_t tiles64 = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
-  const uint32_t padded = pwPaddedChans(d.inChansPerGroup);
+  const uint32_t padded = pwPaddedChans(pwRowChans(d));
   if (padded <= 64) {
     for (uint32_t nt = 4; nt > 1; --nt)
       if (tiles64 % nt == 0 && mTiles * (tiles64 / nt) * d.groups >= 2ull * cus)
@@ -447,7 +498,7 @@ uint32_t chanTilesFor(const PointwiseDesc &d, uint32_t cus) {
   } else if ((padded == 128 || padded == 256) && tiles64 % 2 == 0) {
     const uint64_t pairs = tiles64 / 2 * d.groups;
     const uint64_t walkers = walkersFor(
-        mTiles, pairs, ldsBytesOf(s, d.inChansPerGroup, 2), cus);
+        mTiles, pairs, ldsBytesOf(s, pwRowChans(d), 2), cus);
     if ((mTiles + walkers - 1) / walkers >= 6)
       return 2;
   }
@@ -467,13 +518,13 @@ int deviceCUs() {
   return cus;
 }
 
-template <int KS, int TM, int NB, int LW, int NT, class OutT>
+template <int KS, int TM, int NB, int LW, int NT, class OutT, int F>
 hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
                void *out, hipStream_t stream) {
   constexpr int ldsBytes = ldsBytesOf(PwShape{TM, NB, LW}, KS * 16, NT);
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void *>(
-          &pointwiseKernel<KS, TM, NB, LW, NT, OutT>),
+          &pointwiseKernel<KS, TM, NB, LW, NT, OutT, F>),
       hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
   if (attr != hipSuccess)
     return attr;
@@ -490,7 +541,7 @@ hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
   if (blocks > 0x7fffffffull ||
       uint64_t(a.mTiles) + uint64_t(NB) * walkers > 0x7fffffffull / TM)
     return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((pointwiseKernel<KS, TM, NB, LW, NT, OutT>),
+  hipLaunchKernelGGL((pointwiseKernel<KS, TM, NB, LW, NT, OutT, F>),
                      dim3(uint32_t(blocks)), dim3(TM * 4 + 64 * LW), ldsBytes,
                      stream, a, static_cast<const char *>(in),
                      static_cast<const char *>(w),
@@ -498,61 +549,61 @@ hipError_t run(PwArgs a, const void *in, const void *w, const void *bias,
   return hipGetLastError();
 }
 
-template <class OutT>
+template <class OutT, int F>
 hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
                      const void *bias, void *out, hipStream_t stream) {
   const uint32_t nt = chanTilesFor(a.d, uint32_t(deviceCUs()));
-  switch (pwPaddedChans(a.d.inChansPerGroup)) {
+  switch (pwPaddedChans(pwRowChans(a.d))) {
   case 16:
     if (nt == 4)
-      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT>(
+      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT, F>(
           a, in, w, bias, out, stream);
     if (nt == 3)
-      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT>(
+      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT, F>(
           a, in, w, bias, out, stream);
     if (nt == 2)
-      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT>(
+      return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT, F>(
           a, in, w, bias, out, stream);
-    return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT>(
+    return run<1, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT, F>(
         a, in, w, bias, out, stream);
   case 32:
     if (nt == 4)
-      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT>(
+      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT, F>(
           a, in, w, bias, out, stream);
     if (nt == 3)
-      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT>(
+      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT, F>(
           a, in, w, bias, out, stream);
     if (nt == 2)
-      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT>(
+      return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT, F>(
           a, in, w, bias, out, stream);
-    return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT>(
+    return run<2, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT, F>(
         a, in, w, bias, out, stream);
   case 64:
     if (nt == 4)
-      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT>(
+      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 4, OutT, F>(
           a, in, w, bias, out, stream);
     if (nt == 3)
-      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT>(
+      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 3, OutT, F>(
           a, in, w, bias, out, stream);
     if (nt == 2)
-      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT>(
+      return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 2, OutT, F>(
           a, in, w, bias, out, stream);
-    return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT>(
+    return run<4, kShape64.tm, kShape64.nb, kShape64.lw, 1, OutT, F>(
         a, in, w, bias, out, stream);
   case 128:
     if (nt == 2)
-      return run<8, kShape128.tm, kShape128.nb, kShape128.lw, 2, OutT>(
+      return run<8, kShape128.tm, kShape128.nb, kShape128.lw, 2, OutT, F>(
           a, in, w, bias, out, stream);
-    return run<8, kShape128.tm, kShape128.nb, kShape128.lw, 1, OutT>(
+    return run<8, kShape128.tm, kShape128.nb, kShape128.lw, 1, OutT, F>(
         a, in, w, bias, out, stream);
   case 256:
     if (nt == 2)
-      return run<16, kShape256.tm, kShape256.nb, kShape256.lw, 2, OutT>(
+      return run<16, kShape256.tm, kShape256.nb, kShape256.lw, 2, OutT, F>(
           a, in, w, bias, out, stream);
-    return run<16, kShape256.tm, kShape256.nb, kShape256.lw, 1, OutT>(
+    return run<16, kShape256.tm, kShape256.nb, kShape256.lw, 1, OutT, F>(
         a, in, w, bias, out, stream);
   case 512:
-    return run<32, kShape512.tm, kShape512.nb, kShape512.lw, 1, OutT>(
+    return run<32, kShape512.tm, kShape512.nb, kShape512.lw, 1, OutT, F>(
         a, in, w, bias, out, stream);
   }
   return hipErrorInvalidValue;
@@ -562,7 +613,7 @@ hipError_t runSlices(const PwArgs &a, const void *in, const void *w,
 
 bool pointwiseChanTilesOk(const PointwiseDesc &d, uint32_t chanTiles) {
   const uint32_t tiles64 = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
-  const uint32_t padded = pwPaddedChans(d.inChansPerGroup);
+  const uint32_t padded = pwPaddedChans(pwRowChans(d));
   const uint32_t most = padded <= 64 ? 4 : padded == 512 ? 1 : 2;
   return chanTiles >= 1 && chanTiles <= most && tiles64 % chanTiles == 0;
 }
@@ -570,19 +621,26 @@ bool pointwiseChanTilesOk(const PointwiseDesc &d, uint32_t chanTiles) {
 bool pointwiseTakes(const PointwiseDesc &d, int inType, int outType) {
   const uint32_t ci = d.inChansPerGroup, co = d.outChansPerGroup;
   const uint64_t m = uint64_t(d.batch) * d.pixels;
-  const uint64_t inBytes = m * d.groups * ci * 2;
-  return inType == kHalf && (outType == kHalf || outType == kFloat) &&
-         ci != 0 && ci % 8 == 0 && ci <= 512 && co != 0 &&
+  const uint64_t inBytes = m * d.groups * ci * d.elemBytes;
+  // fp16 (fp16 or fp32 out) or fp8 (fp16 out); rows of whole 16-byte
+  // vectors, 1024 bytes at most
+  const bool types =
+      (inType == kHalf && d.elemBytes == 2 &&
+       (outType == kHalf || outType == kFloat)) ||
+      (inType == kQuarter && d.elemBytes == 1 && outType == kHalf);
+  return types && ci != 0 && (ci * d.elemBytes) % 16 == 0 &&
+         ci * d.elemBytes <= 1024 && co != 0 &&
          (d.chanTiles == 0 || pointwiseChanTilesOk(d, d.chanTiles)) &&
          co % (outType == kHalf ? 8 : 4) == 0 && m != 0 && m < 0x7fffffffull &&
          inBytes < kOutOfRange &&
-         pointwisePackedElems(d) * 2 < kOutOfRange;
+         pointwisePackedElems(d) * d.elemBytes < kOutOfRange;
 }
 
 uint64_t pointwisePackedElems(const PointwiseDesc &d) {
   const uint64_t nBlocks = (d.outChansPerGroup + kPwChans - 1) / kPwChans * 2;
-  return uint64_t(d.groups) * nBlocks *
-         (pwPaddedChans(d.inChansPerGroup) / 16) * 512;
+  // (1 KB per block and 32-byte k-slice)
+  return uint64_t(d.groups) * nBlocks * (pwPaddedChans(pwRowChans(d)) / 16) *
+         (1024 / d.elemBytes);
 }
 
 hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
@@ -595,16 +653,26 @@ hipError_t launchPackPointwiseWeights(const PointwiseDesc &d, const void *src,
   if (blocks > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
   const uint32_t nBlocks = (d.outChansPerGroup + kPwChans - 1) / kPwChans * 2;
-  hipLaunchKernelGGL(packPointwiseWeightsKernel, dim3(uint32_t(blocks)),
-                     dim3(256), 0, stream, static_cast<const uint16_t *>(src),
-                     static_cast<uint16_t *>(dst), d.outChansPerGroup,
-                     d.inChansPerGroup, pwPaddedChans(d.inChansPerGroup),
-                     nBlocks, total, chansTransposed);
+  const uint32_t slices = pwPaddedChans(pwRowChans(d)) / 16;
+  if (d.elemBytes == 2)
+    hipLaunchKernelGGL(packPointwiseWeightsKernel<uint16_t>,
+                       dim3(uint32_t(blocks)), dim3(256), 0, stream,
+                       static_cast<const uint16_t *>(src),
+                       static_cast<uint16_t *>(dst), d.outChansPerGroup,
+                       d.inChansPerGroup, slices, nBlocks, total,
+                       chansTransposed);
+  else
+    hipLaunchKernelGGL(packPointwiseWeightsKernel<uint8_t>,
+                       dim3(uint32_t(blocks)), dim3(256), 0, stream,
+                       static_cast<const uint8_t *>(src),
+                       static_cast<uint8_t *>(dst), d.outChansPerGroup,
+                       d.inChansPerGroup, slices, nBlocks, total,
+                       chansTransposed);
   return hipGetLastError();
 }
 
 PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus) {
-  const PwShape s = shapeFor(d.inChansPerGroup);
+  const PwShape s = shapeFor(pwRowChans(d));
   PointwiseLaunch l{};
   l.tilePixels = uint32_t(s.tm), l.ring = uint32_t(s.nb);
   l.loaderWaves = uint32_t(s.lw);
@@ -616,7 +684,7 @@ PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus) {
   if (mTiles == 0 || pairs == 0)
     return l;
   const uint64_t walkers =
-      walkersFor(mTiles, pairs, ldsBytesOf(s, d.inChansPerGroup, nt), cus);
+      walkersFor(mTiles, pairs, ldsBytesOf(s, pwRowChans(d), nt), cus);
   l.workgroups = walkers * pairs;
   l.tilesPerWorkgroup = uint32_t((mTiles + walkers - 1) / walkers);
   return l;
@@ -624,7 +692,8 @@ PointwiseLaunch pointwiseLaunchShape(const PointwiseDesc &d, uint32_t cus) {
 
 hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
-                           const void *bias, void *out, hipStream_t stream) {
+                           const void *bias, void *out, const QuarterInfo &q,
+                           hipStream_t stream) {
   if (!pointwiseTakes(d, inType, outType))
     return hipErrorInvalidValue;
   PwArgs a;
@@ -633,11 +702,24 @@ hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
   a.mTiles = 0; // set for the tile height of the kernel that runs
   a.nTiles = (d.outChansPerGroup + kPwChans - 1) / kPwChans;
   a.nBlocks = a.nTiles * 2;
-  a.inBytes = uint32_t(uint64_t(a.M) * d.groups * d.inChansPerGroup * 2);
-  a.wBytes = uint32_t(pointwisePackedElems(d) * 2);
+  a.inBytes =
+      uint32_t(uint64_t(a.M) * d.groups * d.inChansPerGroup * d.elemBytes);
+  a.wBytes = uint32_t(pointwisePackedElems(d) * d.elemBytes);
+  a.scale = inType == kQuarter ? q.scale : 1.0f;
+  a.invScale = 1.0f / a.scale;
+  if (inType == kQuarter) {
+    const bool actsE5M2 = q.inFormat != kE4M3, wE5M2 = q.weightFormat != kE4M3;
+    if (!actsE5M2 && !wE5M2)
+      return runSlices<__half, 1>(a, in, weightsPacked, bias, out, stream);
+    if (actsE5M2 && !wE5M2)
+      return runSlices<__half, 2>(a, in, weightsPacked, bias, out, stream);
+    if (!actsE5M2 && wE5M2)
+      return runSlices<__half, 3>(a, in, weightsPacked, bias, out, stream);
+    return runSlices<__half, 4>(a, in, weightsPacked, bias, out, stream);
+  }
   if (outType == kHalf)
-    return runSlices<__half>(a, in, weightsPacked, bias, out, stream);
-  return runSlices<float>(a, in, weightsPacked, bias, out, stream);
+    return runSlices<__half, 0>(a, in, weightsPacked, bias, out, stream);
+  return runSlices<float, 0>(a, in, weightsPacked, bias, out, stream);
 }
 
 } // namespace mxk

@@ -986,6 +986,7 @@ mxconv_plan makePlanWith(const ConvParams &params,
     pw.groups = g.groups, pw.inChansPerGroup = g.inChansPerGroup;
     pw.outChansPerGroup = g.outChansPerGroup;
     pw.chanTiles = pc.chanTiles;
+    pw.elemBytes = uint32_t(params.inputType.size());
     const bool unitWindow =
         !s.hasDepth() && !s.outputPadded() && !s.kernelSelected &&
         !s.inputDilated() &&
@@ -1000,11 +1001,21 @@ mxconv_plan makePlanWith(const ConvParams &params,
     // faster on small layers - N = 32, 28 x 28, 144 -> 32: 4.6 against 5.3 us,
     // 192 -> 32: 4.6 against 5.4, 7 x 7, 160 -> 960: 4.8 against 5.5 - and
     // slower on large ones: 56 x 56, 144 -> 24: 11.9 against 8.9.)
-    const bool paddedSmall = ci > 128 && ci < 256 &&
+    // (fp8 rows count by their bytes: two channels for one of fp16)
+    const std::size_t rowChans = ci * params.inputType.size() / 2;
+    const bool paddedSmall = rowChans > 128 && rowChans < 256 &&
                              std::size_t(pw.batch) * pw.pixels < 65536 &&
                              pc.pointwise != 1;
+    // (fp8 rows of 512 bytes or more: the kernel's MFMAs take 16 channels at
+    // a time whatever the type, so deep fp8 layers are the matrix cores' -
+    // N = 32, 28 x 28, 512 -> 128: 7.4 us against the big tile's 6.5,
+    // N = 64, 14 x 14, 1024 -> 256: 8.5 against 7.8; with 256 channels and
+    // fewer it wins, 14 x 14, 256 -> 1024: 10.0 against 12.2, 56 x 56,
+    // 256 -> 64: 8.4 against 11.0, 112 x 112, 32 -> 64: 14.6 against 24.1)
+    const bool deepQuarter =
+        quarterIn && ci >= 512 && pc.pointwise != 1;
     plan.pointwiseOn =
-        unitWindow && ciPadded == ci && !paddedSmall &&
+        unitWindow && ciPadded == ci && !paddedSmall && !deepQuarter &&
         (pc.kernel != "igemm" || pc.pointwise == 1) && pc.pointwise != 0 &&
         pc.patch < 1 && !pc.blockM &&
         !pc.blockN && !pc.blockK &&
@@ -1020,8 +1031,8 @@ mxconv_plan makePlanWith(const ConvParams &params,
       throw poplar::invalid_option(
           "planConstraints gfx950 pointwise: that kernel takes 1x1, unit "
           "stride, unpadded convolutions of half inputs with a multiple of 8 "
-          "up to 512 input channels per group, with no other tile "
-          "constraint");
+          "up to 512 input channels per group (quarter inputs: a multiple of "
+          "16 up to 1024), with no other tile constraint");
     else if (pc.chanTiles)
       throw poplar::invalid_option(
           "planConstraints gfx950 chanTiles: the pointwise streaming kernel "

@@ -673,6 +673,18 @@ def test_pointwise_planner_choice_for_padded_rows():
     # not a multiple of eight: the big tile, channels padded in a copy
     assert "pointwise streaming variant" not in kernel_of(
         batch=2, field=(14, 14), ci=20, co=64)
+    # fp8 inputs: rows of fewer than 512 bytes
+    def quarter(**kw):
+        return pa.Plan(make_params(pa.QUARTER, pa.HALF, kernel=(1, 1),
+                                   **kw)).describe()
+    assert "pointwise streaming variant" in quarter(
+        batch=32, field=(56, 56), ci=256, co=64)
+    assert "pointwise streaming variant" in quarter(
+        batch=32, field=(112, 112), ci=32, co=64)
+    assert "pointwise streaming variant" not in quarter(
+        batch=32, field=(28, 28), ci=512, co=128)
+    assert "pointwise streaming variant" not in quarter(
+        batch=32, field=(28, 28), ci=24, co=128)
 
 
 def test_planner_runs_small_conv_groups_as_one():

@@ -207,6 +207,65 @@ def test_pointwise_any_multiple_of_eight_channels(oracle, kw, out_type):
          **({} if out_type == pa.FLOAT else {"wscale": 0.1}))
 
 
+# fp8 inputs through the same kernel: rows of 16 to 1024 channels (the bytes
+# of 8 to 512 fp16 ones), the four pairs of formats, several channel tiles
+# per workgroup, groups, bias (which enters the sums divided by the scale).
+FP8_POINTWISE_CASES = [
+    dict(batch=2, field=(28, 29), kernel=(1, 1), ci=16, co=48),
+    dict(batch=3, field=(17, 9), kernel=(1, 1), ci=48, co=96),
+    dict(batch=2, field=(13, 22), kernel=(1, 1), ci=128, co=256),
+    dict(batch=2, field=(9, 14), kernel=(1, 1), ci=80, co=72, groups=2),
+    dict(batch=3, field=(7, 11), kernel=(1, 1), ci=256, co=64),
+    dict(batch=1, field=(15, 15), kernel=(1, 1), ci=512, co=128, groups=2),
+    dict(batch=2, field=(7, 7), kernel=(1, 1), ci=1024, co=256),
+    dict(batch=2, field=(8, 5), kernel=(1, 1), ci=592, co=40),
+]
+
+
+@pytest.mark.parametrize("kw", FP8_POINTWISE_CASES)
+@pytest.mark.parametrize("fmt_a,fmt_w", [(1, 1), (1, 0), (0, 1), (0, 0)])
+def test_pointwise_fp8_matches_oracle(oracle, kw, fmt_a, fmt_w):
+    from gpu_helpers import quantize, run_conv
+    p = make_params(pa.QUARTER, pa.HALF, **kw)
+    print("case", p, fmt_a, fmt_w, flush=True)
+    acts, weights, biases = random_data(p, 23, "normal")
+    fan_in = p.inputChannelsPerConvGroup
+    weights = weights * np.sqrt(2.0 / fan_in)
+
+    def scale_for(x, fmt):
+        maxv = 448.0 if fmt == oracle.E4M3 else 57344.0
+        return int(np.ceil(np.log2(np.abs(x).max() / maxv)))
+
+    sa, sw = scale_for(acts, fmt_a), scale_for(weights, fmt_w)
+    aq, ad = quantize(acts, pa.QUARTER, oracle, fmt_a, sa)
+    wq, wd = quantize(weights, pa.QUARTER, oracle, fmt_w, sw)
+    bq, bd = quantize(biases, pa.HALF)
+    got, plan = run_conv(p, aq, wq, bq, FORCE_POINTWISE,
+                         in_meta=pa.quarter_metadata(fmt_a, sa),
+                         w_meta=pa.quarter_metadata(fmt_w, sw),
+                         return_plan=True)
+    assert "pointwise streaming variant" in plan.describe(), plan.describe()
+    want = oracle.convolution(p, ad, wd, bd, threads=8)
+    err = rel_l2(got, want)
+    assert err <= 1e-3, err
+
+
+def test_pointwise_fp8_equals_the_big_tile(oracle):
+    """The same sums in fp32 from the same fp8 operands: the streaming kernel
+    and the big tile agree to the last bit of the half output but for the
+    order of the additions (a few results in a thousand differ by one ulp)."""
+    from test_fast_gpu import _fp8_case as case
+    p = make_params(pa.QUARTER, pa.HALF, batch=2, field=(14, 14),
+                    kernel=(1, 1), ci=256, co=128)
+    small, _, plan = case(oracle, p, 24, 1, 0)
+    assert "pointwise streaming variant" in plan.describe()
+    big, want, plan = case(oracle, p, 24, 1, 0, options={
+        "planConstraints": '{"gfx950": {"pointwise": 0}}'})
+    assert "pointwise streaming variant" not in plan.describe()
+    assert rel_l2(small, want) <= 1e-3 and rel_l2(big, want) <= 1e-3
+    assert np.mean(small != big) < 0.01
+
+
 def test_pointwise_pm1_exact_and_big_tile_on_request(oracle):
     p = make_params(pa.HALF, pa.FLOAT, **POINTWISE_CASES[1])
     _run(oracle, p, 9, 0, "implicit GEMM", dist="pm1")
