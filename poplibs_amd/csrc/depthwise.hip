@@ -73,9 +73,100 @@ template <> struct StoreVec<float> {
   }
 };
 
+/// A 16-byte vector of E channels of the input type as fp32 (fp8: `format`
+/// as in decodeFp8).
+template <class InT> struct InVec;
+template <> struct InVec<__half> {
+  static constexpr int E = 8;
+  static __device__ __forceinline__ void unpack(const uint4 &raw, int,
+                                                float (&f)[8]) {
+    Vec8 v;
+    v.raw = raw;
+#pragma unroll
+    for (int i = 0; i != 4; ++i) {
+      const float2 two = __half22float2(v.h2[i]);
+      f[2 * i] = two.x, f[2 * i + 1] = two.y;
+    }
+  }
+};
+template <> struct InVec<float> {
+  static constexpr int E = 4;
+  static __device__ __forceinline__ void unpack(const uint4 &raw, int,
+                                                float (&f)[4]) {
+    f[0] = __uint_as_float(raw.x), f[1] = __uint_as_float(raw.y);
+    f[2] = __uint_as_float(raw.z), f[3] = __uint_as_float(raw.w);
+  }
+};
+template <> struct InVec<uint8_t> {
+  static constexpr int E = 16;
+  static __device__ __forceinline__ void unpack(const uint4 &raw, int format,
+                                                float (&f)[16]) {
+    // (the hardware's conversions of OCP E4M3 / E5M2 pairs: the decoding in
+    // software costs the kernel a factor of ten)
+    const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    if (format == 1) {
+#pragma unroll
+      for (int i = 0; i != 4; ++i) {
+        const floatx2 lo =
+            __builtin_amdgcn_cvt_pk_f32_fp8(int(words[i]), false);
+        const floatx2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(int(words[i]), true);
+        f[4 * i] = lo.x, f[4 * i + 1] = lo.y;
+        f[4 * i + 2] = hi.x, f[4 * i + 3] = hi.y;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i != 4; ++i) {
+        const floatx2 lo =
+            __builtin_amdgcn_cvt_pk_f32_bf8(int(words[i]), false);
+        const floatx2 hi = __builtin_amdgcn_cvt_pk_f32_bf8(int(words[i]), true);
+        f[4 * i] = lo.x, f[4 * i + 1] = lo.y;
+        f[4 * i + 2] = hi.x, f[4 * i + 3] = hi.y;
+      }
+    }
+#else
+    for (int i = 0; i != 16; ++i)
+      f[i] = 0.0f * float(words[i / 4]) * float(format);
+#endif
+  }
+};
+
+/// E consecutive channels of the output.
+template <class OutT, int E>
+__device__ __forceinline__ void putVec(OutT *p, const float (&v)[E]) {
+  if constexpr (E == 8) {
+    StoreVec<OutT>::put(p, v);
+  } else if constexpr (sizeof(OutT) == 4) {
+#pragma unroll
+    for (int i = 0; i != E; i += 4)
+      *reinterpret_cast<float4 *>(p + i) =
+          float4{v[i], v[i + 1], v[i + 2], v[i + 3]};
+  } else if constexpr (E == 4) {
+    const __half2 lo = roundPairToHalf(v[0], v[1]),
+                  hi = roundPairToHalf(v[2], v[3]);
+    *reinterpret_cast<uint2 *>(p) = uint2{__builtin_bit_cast(uint32_t, lo),
+                                          __builtin_bit_cast(uint32_t, hi)};
+  } else {
+    static_assert(E == 16, "vectors of 4, 8 or 16 channels");
+#pragma unroll
+    for (int h = 0; h != 2; ++h) {
+      Vec8 o;
+#pragma unroll
+      for (int i = 0; i != 4; ++i)
+        o.h2[i] = roundPairToHalf(v[8 * h + 2 * i], v[8 * h + 2 * i + 1]);
+      *reinterpret_cast<uint4 *>(p + 8 * h) = o.raw;
+    }
+  }
+}
+
 struct DwArgs {
   DepthwiseDesc d;
-  uint32_t vecs;      // channels / 8
+  // fp8 inputs: the tensors' formats (as decodeFp8 takes them) and
+  // 2^(scaleIn + scaleWeights), applied to the sums before the bias
+  int formatIn, formatWeights;
+  float scale;
+  uint32_t vecs;      // channels in 16-byte vectors (of 4, 8 or 16)
   uint32_t vecBlock;  // channel vectors per workgroup: vecs if <= 16, else 16
   uint32_t vecShift;  // log2(vecBlock) when the channels are split in blocks
   uint32_t vecBlocks; // ceil(vecs / vecBlock)
@@ -99,10 +190,13 @@ struct DwArgs {
 /// LDS behind the patch, one copy per workgroup) and the PX + KW - 1 input
 /// vectors under them once and multiplies PX x KW times: 13 multiply-adds per
 /// 16-byte LDS read at 7 x 7 and PX = 7, against one.
-template <int KH, int KW, class OutT, int PX = 0>
+/// InT: __half, float or uint8_t (fp8) inputs; the strips are for half.
+template <int KH, int KW, class OutT, int PX = 0, class InT = __half>
 __global__ __launch_bounds__(kThreads) void depthwiseKernel(
-    DwArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
+    DwArgs a, const InT *__restrict__ in, const InT *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  constexpr int E = InVec<InT>::E; // channels of a 16-byte vector
+  static_assert(PX == 0 || E == 8, "strips: half inputs");
   extern __shared__ __align__(16) char lds[]; // patchH * rowPitch * 16 bytes
   const DepthwiseDesc &d = a.d;
   const uint32_t kH = KH ? KH : d.kH, kW = KW ? KW : d.kW;
@@ -127,8 +221,8 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
   // channels in one block the row is contiguous in memory as well, otherwise
   // vecBlock is 16 and (pw, v) are a shift and a mask of j.
   const __amdgpu_buffer_rsrc_t inBuf = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<__half *>(in), short(0), int(a.inBytes), 0x00020000);
-  const uint32_t pixelBytes = d.channels * 2;
+      const_cast<InT *>(in), short(0), int(a.inBytes), 0x00020000);
+  const uint32_t pixelBytes = d.channels * sizeof(InT);
   const uint32_t imageOff = b * d.inH * d.inW * pixelBytes;
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t chunksPerRow = a.rowPitch >> 6;
@@ -178,8 +272,8 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
   const uint32_t v = threadIdx.x % a.vecBlock;
   uint32_t p = threadIdx.x / a.vecBlock;
   const bool active = p < a.pixelsPerRound && v < nvec;
-  const uint32_t c = (cv0 + (v < nvec ? v : 0)) * 8;
-  const __half *wC = w + c;
+  const uint32_t c = (cv0 + (v < nvec ? v : 0)) * E;
+  const InT *wC = w + c;
   constexpr bool kTapsInRegs = KH * KW != 0 && KH * KW <= 9;
   Vec8 taps[kTapsInRegs ? KH * KW : 1];
   if constexpr (kTapsInRegs) {
@@ -188,9 +282,9 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
       taps[tap].raw =
           *reinterpret_cast<const uint4 *>(wC + tap * d.channels);
   }
-  float biasV[8];
+  float biasV[E];
 #pragma unroll
-  for (int i = 0; i != 8; ++i)
+  for (int i = 0; i != E; ++i)
     biasV[i] = bias ? Load<OutT>::at(bias, c + i, 0) : 0.0f;
 
   if constexpr (PX != 0) {
@@ -274,10 +368,10 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
     for (; p < pixels; p += a.pixelsPerRound) {
       const uint32_t oh = oh0 + ty, ow = ow0 + tx;
       if (oh < d.outH && ow < d.outW) {
-        float acc[8];
+        float acc[E];
 #pragma unroll
-        for (int i = 0; i != 8; ++i)
-          acc[i] = biasV[i];
+        for (int i = 0; i != E; ++i)
+          acc[i] = E == 8 ? biasV[i] : 0.0f;
         const char *patch =
             lds + (ty * d.strideH * a.rowPitch +
                    tx * d.strideW * a.vecBlock + v) *
@@ -295,15 +389,30 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
             else
               k.raw = *reinterpret_cast<const uint4 *>(
                   wC + (kh * kW + kw) * d.channels);
+            if constexpr (E == 8) {
 #pragma unroll
-            for (int i = 0; i != 4; ++i) {
-              const float2 xf = __half22float2(x.h2[i]);
-              const float2 kf = __half22float2(k.h2[i]);
-              acc[2 * i] = fmaf(xf.x, kf.x, acc[2 * i]);
-              acc[2 * i + 1] = fmaf(xf.y, kf.y, acc[2 * i + 1]);
+              for (int i = 0; i != 4; ++i) {
+                const float2 xf = __half22float2(x.h2[i]);
+                const float2 kf = __half22float2(k.h2[i]);
+                acc[2 * i] = fmaf(xf.x, kf.x, acc[2 * i]);
+                acc[2 * i + 1] = fmaf(xf.y, kf.y, acc[2 * i + 1]);
+              }
+            } else {
+              float xf[E], kf[E];
+              InVec<InT>::unpack(x.raw, a.formatIn, xf);
+              InVec<InT>::unpack(k.raw, a.formatWeights, kf);
+#pragma unroll
+              for (int i = 0; i != E; ++i)
+                acc[i] = fmaf(xf[i], kf[i], acc[i]);
             }
           }
-        StoreVec<OutT>::put(
+        if constexpr (E != 8) {
+          // (fp8: the scale on the sum, then the bias)
+#pragma unroll
+          for (int i = 0; i != E; ++i)
+            acc[i] = (E == 16 ? acc[i] * a.scale : acc[i]) + biasV[i];
+        }
+        putVec<OutT, E>(
             out + ((size_t(b) * d.outH + oh) * d.outW + ow) * d.channels + c,
             acc);
       }
@@ -318,7 +427,7 @@ __global__ __launch_bounds__(kThreads) void depthwiseKernel(
 
 constexpr uint32_t kLdsMost = kDepthwiseTileLdsMost;
 
-template <int KH, int KW, class OutT, int PX = 0>
+template <int KH, int KW, class OutT, int PX = 0, class InT = __half>
 hipError_t run(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
                const void *in, const void *w, const void *bias, void *out,
                hipStream_t stream) {
@@ -327,16 +436,29 @@ hipError_t run(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
   if (ldsBytes > kLdsMost)
     return hipErrorInvalidConfiguration;
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void *>(&depthwiseKernel<KH, KW, OutT, PX>),
+      reinterpret_cast<const void *>(
+          &depthwiseKernel<KH, KW, OutT, PX, InT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMost);
   if (attr != hipSuccess)
     return attr;
-  hipLaunchKernelGGL((depthwiseKernel<KH, KW, OutT, PX>), dim3(blocks),
+  hipLaunchKernelGGL((depthwiseKernel<KH, KW, OutT, PX, InT>), dim3(blocks),
                      dim3(kThreads), ldsBytes, stream, a,
-                     static_cast<const __half *>(in),
-                     static_cast<const __half *>(w),
+                     static_cast<const InT *>(in),
+                     static_cast<const InT *>(w),
                      static_cast<const OutT *>(bias), static_cast<OutT *>(out));
   return hipGetLastError();
+}
+
+/// float or fp8 inputs: the kernel a pixel at a time, 3 x 3 taps unrolled.
+template <class OutT, class InT>
+hipError_t runOtherType(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
+                        const void *in, const void *w, const void *bias,
+                        void *out, hipStream_t stream) {
+  if (a.d.kH == 3 && a.d.kW == 3)
+    return run<3, 3, OutT, 0, InT>(a, blocks, ldsBytes, in, w, bias, out,
+                                   stream);
+  return run<0, 0, OutT, 0, InT>(a, blocks, ldsBytes, in, w, bias, out,
+                                 stream);
 }
 
 template <class OutT>
@@ -361,11 +483,12 @@ hipError_t runKernelShape(const DwArgs &a, uint32_t blocks, uint32_t ldsBytes,
 bool depthwiseStripTakes(const DepthwiseDesc &d) {
   return d.kH == 7 && d.kW == 7 && d.strideH == 1 && d.strideW == 1 &&
          d.dilH == 1 && d.dilW == 1 && d.inDilH == 1 && d.inDilW == 1 &&
-         d.channels % 8 == 0;
+         d.channels % 8 == 0 && d.elemBytes == 2;
 }
 
 uint64_t depthwiseTileLdsBytes(const DepthwiseDesc &d) {
-  const uint64_t vecs = d.channels / 8, vecBlock = vecs <= 16 ? vecs : 16;
+  const uint64_t vecs = uint64_t(d.channels) * d.elemBytes / 16,
+                 vecBlock = vecs <= 16 ? vecs : 16;
   const uint64_t patchH = uint64_t(d.tileH - 1) * d.strideH +
                           uint64_t(d.kH - 1) * d.dilH + 1;
   const uint64_t patchW = uint64_t(d.tileW - 1) * d.strideW +
@@ -377,13 +500,14 @@ uint64_t depthwiseTileLdsBytes(const DepthwiseDesc &d) {
 
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
-                           const void *bias, void *out, hipStream_t stream) {
+                           const void *bias, void *out, const QuarterInfo &q,
+                           hipStream_t stream) {
   // The kernels address a launch's tensors with 32-bit offsets.  Images are
   // independent: a batch whose input or output exceeds that goes out as
   // several launches of as many images as fit.
   {
     const uint64_t outBytes = outType == kHalf ? 2 : 4;
-    const uint64_t inImage = uint64_t(d.inH) * d.inW * d.channels * 2;
+    const uint64_t inImage = uint64_t(d.inH) * d.inW * d.channels * d.elemBytes;
     const uint64_t outImage = uint64_t(d.outH) * d.outW * d.channels * outBytes;
     const uint64_t limit = kOutOfRange / 2;
     const uint64_t image = inImage > outImage ? inImage : outImage;
@@ -395,7 +519,7 @@ hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
         const hipError_t e = launchDepthwise(
             part, inType, outType,
             static_cast<const char *>(in) + first * inImage, weightsPacked,
-            bias, static_cast<char *>(out) + first * outImage, stream);
+            bias, static_cast<char *>(out) + first * outImage, q, stream);
         if (e != hipSuccess)
           return e;
       }
@@ -411,13 +535,19 @@ hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
   if (d.dense3x3)
     return launchDepthwise3x3(d, inType, outType, in, weightsPacked, bias,
                                  out, stream);
-  if (inType != kHalf || d.channels % 8 != 0 || d.tileH == 0 || d.tileW == 0)
+  const uint32_t elemBytes = inType == kHalf ? 2 : inType == kFloat ? 4 : 1;
+  const uint32_t perVec = 16 / elemBytes;
+  if (d.elemBytes != elemBytes || d.channels % perVec != 0 || d.tileH == 0 ||
+      d.tileW == 0 || (inType == kQuarter && outType != kHalf))
     return hipErrorInvalidValue;
   if (uint64_t(d.batch) * d.outH * d.outW * d.channels == 0)
     return hipSuccess;
   DwArgs a;
   a.d = d;
-  a.vecs = d.channels / 8;
+  a.formatIn = q.inFormat == kE4M3 ? 1 : 0;
+  a.formatWeights = q.weightFormat == kE4M3 ? 1 : 0;
+  a.scale = inType == kQuarter ? q.scale : 1.0f;
+  a.vecs = d.channels / perVec;
   a.vecBlock = a.vecs <= 16 ? a.vecs : 16;
   a.vecShift = 4;
   a.vecBlocks = (a.vecs + a.vecBlock - 1) / a.vecBlock;
@@ -430,7 +560,8 @@ hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
   a.pixelsPerRound = kThreads / a.vecBlock;
   a.stepY = a.pixelsPerRound / d.tileW;
   a.stepX = a.pixelsPerRound % d.tileW;
-  const uint64_t inBytes = uint64_t(d.batch) * d.inH * d.inW * d.channels * 2;
+  const uint64_t inBytes =
+      uint64_t(d.batch) * d.inH * d.inW * d.channels * elemBytes;
   const uint64_t ldsBytes = uint64_t(a.patchH) * a.rowPitch * 16;
   const uint64_t blocks =
       uint64_t(d.batch) * a.tilesH * a.tilesW * a.vecBlocks;
@@ -439,6 +570,16 @@ hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
       (d.stripPixels != 0 && !depthwiseStripTakes(d)))
     return hipErrorInvalidConfiguration;
   a.inBytes = uint32_t(inBytes);
+  if (inType == kFloat && outType == kFloat)
+    return runOtherType<float, float>(a, uint32_t(blocks), uint32_t(ldsBytes),
+                                      in, weightsPacked, bias, out, stream);
+  if (inType == kFloat && outType == kHalf)
+    return runOtherType<__half, float>(a, uint32_t(blocks), uint32_t(ldsBytes),
+                                       in, weightsPacked, bias, out, stream);
+  if (inType == kQuarter)
+    return runOtherType<__half, uint8_t>(a, uint32_t(blocks),
+                                         uint32_t(ldsBytes), in, weightsPacked,
+                                         bias, out, stream);
   if (outType == kHalf)
     return runKernelShape<__half>(a, uint32_t(blocks), uint32_t(ldsBytes), in,
                                   weightsPacked, bias, out, stream);

@@ -334,6 +334,9 @@ struct DepthwiseDesc {
   // pixels of a row at once (7 x 7 taps, unit stride and dilation:
   // depthwiseStripTakes): 4 or 7; 0 = a pixel at a time.
   uint32_t stripPixels = 0;
+  // Bytes of an input element: 2 (fp16: every depthwise kernel), 4 (fp32) or
+  // 1 (fp8) - those two by the LDS-tiled kernel only.
+  uint32_t elemBytes = 2;
 };
 /// True for the layers whose LDS-tiled kernel can work in strips of pixels.
 bool depthwiseStripTakes(const DepthwiseDesc &d);
@@ -372,7 +375,8 @@ hipError_t launchDepthwiseRowsDeltas(const DepthwiseDesc &d, const void *acts,
                                      uint32_t *walkers, hipStream_t stream);
 hipError_t launchDepthwise(const DepthwiseDesc &d, int inType, int outType,
                            const void *in, const void *weightsPacked,
-                           const void *bias, void *out, hipStream_t stream);
+                           const void *bias, void *out, const QuarterInfo &q,
+                           hipStream_t stream);
 /// The same convolution by one thread per output vector, reading the input
 /// from global memory; takes a dilated input (d.inDilH, d.inDilW), ignores
 /// the tile fields.

@@ -227,7 +227,7 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
   }
   case mxconv_plan::Kernel::DEPTHWISE:
     return hipStatus(mxk::launchDepthwise(plan->depthwise, inType, outType, in,
-                                          w, bias, out, s),
+                                          w, bias, out, q, s),
                      "depthwise convolution launch");
   case mxconv_plan::Kernel::GENERIC:
     break;

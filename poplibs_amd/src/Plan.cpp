@@ -645,19 +645,21 @@ mxconv_plan makePlanWith(const ConvParams &params,
       dwWhyNot = "kernel truncation, padding or flip";
     else if (s.outputPadded())
       dwWhyNot = "output padding";
-    else if (!halfIn)
-      dwWhyNot = "depthwise kernel takes half inputs";
+    else if (!halfIn && s.inputDilated())
+      dwWhyNot = "depthwise kernel takes a dilated input as half only";
     else if (ci != 1 || co != 1)
       dwWhyNot = "not one channel per group";
-    else if (p.numConvGroups % 8 != 0)
-      dwWhyNot = "channel count not a multiple of 8";
-    else if (std::size_t(s.inH) * s.inW * p.numConvGroups * 2 >=
+    else if (p.numConvGroups % vecElems != 0)
+      dwWhyNot = "channel count not a multiple of a 16-byte vector";
+    else if (std::size_t(s.inH) * s.inW * p.numConvGroups *
+                     params.inputType.size() >=
                  (1ull << 30) ||
              std::size_t(s.outH) * s.outW * p.numConvGroups * 4 >=
                  (1ull << 30))
       dwWhyNot = "image too large for 32-bit buffer addressing";
     else if (!s.inputDilated() &&
-             (dwTile = chooseDepthwiseTile(s, p.numConvGroups / 8)).first == 0)
+             (dwTile = chooseDepthwiseTile(s, p.numConvGroups / vecElems))
+                     .first == 0)
       dwWhyNot = "input patch of a single output pixel exceeds the LDS budget";
 
   }
@@ -1166,13 +1168,17 @@ mxconv_plan makePlanWith(const ConvParams &params,
     d.loH = s.loH, d.hiH = s.hiH, d.loW = s.loW, d.hiW = s.hiW;
     d.tileH = dwTile.first, d.tileW = dwTile.second;
     d.inDilH = s.inDilH, d.inDilW = s.inDilW;
+    d.elemBytes = uint32_t(params.inputType.size());
+    const int dwType = halfIn ? mxk::kHalf
+                       : floatIn ? mxk::kFloat
+                                 : mxk::kQuarter;
     // 7 x 7 taps at unit stride: a thread forms a strip of neighbouring
     // pixels, and the tile is chosen to fill the workgroup's 256 threads.
     if (mxk::depthwiseStripTakes(d) && !(pc.tileH || pc.tileW))
       chooseDepthwiseStripTile(d);
     // An explicit tile asks for the LDS-tiled kernel.
     d.dense3x3 = !s.inputDilated() && !(pc.tileH || pc.tileW) &&
-                 mxk::depthwise3x3Takes(d, mxk::kHalf);
+                 mxk::depthwise3x3Takes(d, dwType);
     // Layers that give every CU a band of at least four output rows go to
     // the persistent kernel with a ring of input rows in LDS: its start-up
     // (seven rows before the first output; 3.5 us for the smallest layer
@@ -1182,7 +1188,7 @@ mxconv_plan makePlanWith(const ConvParams &params,
     if (!s.inputDilated() && !(pc.tileH || pc.tileW) && pc.rowRing != 0) {
       d.cus = gfx950::numCUs;
       const mxk::DepthwiseRowsLaunch l = mxk::depthwiseRowsLaunchShape(d);
-      const bool takes = mxk::depthwiseRowsTakes(d, mxk::kHalf);
+      const bool takes = mxk::depthwiseRowsTakes(d, dwType);
       if (pc.rowRing == 1 && !takes)
         throw poplar::invalid_option(
             "planConstraints gfx950 rowRing: that kernel takes 3x3 or 5x5 "
