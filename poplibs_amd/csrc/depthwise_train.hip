@@ -55,6 +55,24 @@ __device__ __forceinline__ void store8(float *p, const float (&v)[8]) {
   *reinterpret_cast<float4 *>(p + 4) = float4{v[4], v[5], v[6], v[7]};
 }
 
+// The same for fp32 inputs: a 16-byte vector holds four channels.
+__device__ __forceinline__ void fma4(float (&acc)[4], const uint4 &x,
+                                     const uint4 &k) {
+  acc[0] = fmaf(__uint_as_float(x.x), __uint_as_float(k.x), acc[0]);
+  acc[1] = fmaf(__uint_as_float(x.y), __uint_as_float(k.y), acc[1]);
+  acc[2] = fmaf(__uint_as_float(x.z), __uint_as_float(k.z), acc[2]);
+  acc[3] = fmaf(__uint_as_float(x.w), __uint_as_float(k.w), acc[3]);
+}
+__device__ __forceinline__ void store4(float *p, const float (&v)[4]) {
+  *reinterpret_cast<float4 *>(p) = float4{v[0], v[1], v[2], v[3]};
+}
+__device__ __forceinline__ void store4(__half *p, const float (&v)[4]) {
+  const __half2 lo = roundPairToHalf(v[0], v[1]),
+                hi = roundPairToHalf(v[2], v[3]);
+  *reinterpret_cast<uint2 *>(p) = uint2{__builtin_bit_cast(uint32_t, lo),
+                                        __builtin_bit_cast(uint32_t, hi)};
+}
+
 struct DirectArgs {
   DepthwiseDesc d;
   FastDiv divVecs, divOutW, divOutH, divInDilH, divInDilW;
@@ -62,10 +80,12 @@ struct DirectArgs {
   uint64_t items; // batch * outH * outW * vecs
 };
 
-template <class OutT>
+/// InT: __half (vectors of 8 channels) or float (of 4).
+template <class OutT, class InT = __half>
 __global__ __launch_bounds__(256) void depthwiseDirectKernel(
-    DirectArgs a, const __half *__restrict__ in, const __half *__restrict__ w,
+    DirectArgs a, const InT *__restrict__ in, const InT *__restrict__ w,
     const OutT *__restrict__ bias, OutT *__restrict__ out) {
+  constexpr int E = 16 / int(sizeof(InT));
   const DepthwiseDesc &d = a.d;
   const uint64_t item = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (item >= a.items)
@@ -77,14 +97,14 @@ __global__ __launch_bounds__(256) void depthwiseDirectKernel(
   const uint32_t ow = pixel - row * d.outW;
   const uint32_t b = a.divOutH(row);
   const uint32_t oh = row - b * d.outH;
-  const uint32_t c = v * 8;
-  float acc[8];
+  const uint32_t c = v * E;
+  float acc[E];
 #pragma unroll
-  for (int i = 0; i != 8; ++i)
+  for (int i = 0; i != E; ++i)
     acc[i] = bias ? Load<OutT>::at(bias, c + i, 0) : 0.0f;
   const int ihBase = int(oh * d.strideH) - d.padH;
   const int iwBase = int(ow * d.strideW) - d.padW;
-  const __half *image = in + size_t(b) * d.inH * d.inW * d.channels + c;
+  const InT *image = in + size_t(b) * d.inH * d.inW * d.channels + c;
   // Validity is separable: the kernel columns that read an input element
   // are worked out once (a bit each - up to 32 columns at a time), then for
   // every valid kernel row only those columns are visited.
@@ -106,8 +126,8 @@ __global__ __launch_bounds__(256) void depthwiseDirectKernel(
       if (ihD < 0 || ih * d.inDilH != uint32_t(ihD) || ih < d.loH ||
           ih >= d.hiH)
         continue;
-      const __half *row = image + size_t(ih) * d.inW * d.channels;
-      const __half *taps = w + size_t(kh * d.kW + kw0) * d.channels + c;
+      const InT *row = image + size_t(ih) * d.inW * d.channels;
+      const InT *taps = w + size_t(kh * d.kW + kw0) * d.channels + c;
       for (uint32_t rest = columns; rest != 0; rest &= rest - 1) {
         const uint32_t j = uint32_t(__ffs(int(rest))) - 1;
         const uint32_t iw =
@@ -115,11 +135,17 @@ __global__ __launch_bounds__(256) void depthwiseDirectKernel(
         Vec8 x, k;
         x.raw = *reinterpret_cast<const uint4 *>(row + size_t(iw) * d.channels);
         k.raw = *reinterpret_cast<const uint4 *>(taps + size_t(j) * d.channels);
-        fma8(acc, x, k);
+        if constexpr (E == 8)
+          fma8(acc, x, k);
+        else
+          fma4(acc, x.raw, k.raw);
       }
     }
   }
-  store8(out + size_t(pixel) * d.channels + c, acc);
+  if constexpr (E == 8)
+    store8(out + size_t(pixel) * d.channels + c, acc);
+  else
+    store4(out + size_t(pixel) * d.channels + c, acc);
 }
 
 struct BlockArgs {
@@ -441,18 +467,22 @@ hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
                                  int outType, const void *in,
                                  const void *weightsPacked, const void *bias,
                                  void *out, hipStream_t stream) {
-  if (inType != kHalf || d.channels % 8 != 0 || d.inDilH == 0 || d.inDilW == 0)
+  const uint32_t perVec = inType == kFloat ? 4 : 8;
+  if ((inType != kHalf && inType != kFloat) ||
+      d.elemBytes != (inType == kFloat ? 4u : 2u) ||
+      d.channels % perVec != 0 || d.inDilH == 0 || d.inDilW == 0)
     return hipErrorInvalidValue;
   DirectArgs a;
   a.d = d;
-  a.vecs = d.channels / 8;
+  a.vecs = d.channels / perVec;
   a.items = uint64_t(d.batch) * d.outH * d.outW * a.vecs;
   if (a.items == 0)
     return hipSuccess;
   // item numbers are divided with 31-bit arithmetic
   if (a.items >= (1ull << 31))
     return hipErrorInvalidConfiguration;
-  if ((outType == kHalf || outType == kFloat) && depthwiseDirectInBlocks(d)) {
+  if (inType == kHalf && (outType == kHalf || outType == kFloat) &&
+      depthwiseDirectInBlocks(d)) {
     if (d.kH == 3)
       return launchDilatedBlock<2, 3, 4>(d, outType, in, weightsPacked, bias,
                                          out, stream);
@@ -466,7 +496,19 @@ hipError_t launchDepthwiseDirect(const DepthwiseDesc &d, int inType,
   a.divInDilH = makeFastDiv(d.inDilH);
   a.divInDilW = makeFastDiv(d.inDilW);
   const dim3 grid{uint32_t((a.items + 255) / 256)}, block{256};
-  if (outType == kHalf)
+  if (inType == kFloat && outType == kFloat)
+    hipLaunchKernelGGL((depthwiseDirectKernel<float, float>), grid, block, 0,
+                       stream, a, static_cast<const float *>(in),
+                       static_cast<const float *>(weightsPacked),
+                       static_cast<const float *>(bias),
+                       static_cast<float *>(out));
+  else if (inType == kFloat && outType == kHalf)
+    hipLaunchKernelGGL((depthwiseDirectKernel<__half, float>), grid, block, 0,
+                       stream, a, static_cast<const float *>(in),
+                       static_cast<const float *>(weightsPacked),
+                       static_cast<const __half *>(bias),
+                       static_cast<__half *>(out));
+  else if (outType == kHalf)
     hipLaunchKernelGGL(depthwiseDirectKernel<__half>, grid, block, 0, stream, a,
                        static_cast<const __half *>(in),
                        static_cast<const __half *>(weightsPacked),

@@ -645,8 +645,8 @@ mxconv_plan makePlanWith(const ConvParams &params,
       dwWhyNot = "kernel truncation, padding or flip";
     else if (s.outputPadded())
       dwWhyNot = "output padding";
-    else if (!halfIn && s.inputDilated())
-      dwWhyNot = "depthwise kernel takes a dilated input as half only";
+    else if (quarterIn && s.inputDilated())
+      dwWhyNot = "depthwise kernel takes a dilated input as half or float";
     else if (ci != 1 || co != 1)
       dwWhyNot = "not one channel per group";
     else if (p.numConvGroups % vecElems != 0)

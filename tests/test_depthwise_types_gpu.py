@@ -95,3 +95,30 @@ def test_depthwise_quarter_fixtures_plan_the_depthwise_kernel():
         p = pa.ConvParams.from_json(open(os.path.join(golden, name)).read())
         text = pa.Plan(p).describe()
         print(name, [l for l in text.splitlines() if "kernel  " in l])
+
+
+@pytest.mark.parametrize("kw", [
+    # the backward pass of strided depthwise layers: the deltas dilated by the
+    # stride (3 x 3 and 5 x 5 at stride 2, a stride of 3, uneven strides)
+    dict(batch=2, field=(14, 15), kernel=(3, 3), groups=32, idil=2, pad=1),
+    dict(batch=2, field=(9, 8), kernel=(5, 5), groups=16, idil=2, pad=3),
+    dict(batch=1, field=(7, 9), kernel=(3, 3), groups=20, idil=(3, 1), pad=2),
+])
+@pytest.mark.parametrize("out_type", [pa.FLOAT, pa.HALF])
+def test_depthwise_fp32_dilated_input(oracle, kw, out_type):
+    from gpu_helpers import quantize, run_conv
+    p = make_params(pa.FLOAT, out_type, **kw)
+    print("case", p, flush=True)
+    exact = out_type == pa.FLOAT
+    acts, weights, biases = random_data(p, 64, "pm1" if exact else "normal")
+    got, plan = run_conv(p, quantize(acts, pa.FLOAT)[0],
+                         quantize(weights, pa.FLOAT)[0],
+                         quantize(biases, out_type)[0], None,
+                         return_plan=True)
+    assert KERNEL in plan.describe(), plan.describe()
+    want = oracle.convolution(p, acts, weights,
+                              quantize(biases, out_type)[1], threads=8)
+    if exact:
+        np.testing.assert_array_equal(got, want)
+    else:
+        assert rel_l2(got, want) <= 1e-3
