@@ -293,9 +293,12 @@ struct DeltaArgs {
 /// takes itemsPerBlock (tap, channel vector) items and one slice of the
 /// pixels; when there are few items, `slots` groups of threads walk a part of
 /// the slice each and their sums meet in LDS.
+/// InT: __half (vectors of 8 channels) or float (of 4).
+template <class InT>
 __global__ __launch_bounds__(256) void depthwiseWeightDeltaKernel(
-    DeltaArgs a, const __half *__restrict__ acts,
-    const __half *__restrict__ deltas, float *__restrict__ partial) {
+    DeltaArgs a, const InT *__restrict__ acts, const InT *__restrict__ deltas,
+    float *__restrict__ partial) {
+  constexpr int E = 16 / int(sizeof(InT));
   __shared__ float meet[256][9]; // 8 sums per thread, padded
   const DepthwiseDesc &d = a.d;
   const uint32_t slot = threadIdx.x / a.itemsPerBlock;
@@ -304,7 +307,7 @@ __global__ __launch_bounds__(256) void depthwiseWeightDeltaKernel(
   const bool active = slot < a.slots && item < a.items;
   // item = tap * vecs + v: neighbouring threads read neighbouring channels
   const uint32_t tap = a.divVecs(active ? item : 0);
-  const uint32_t c = ((active ? item : 0) - tap * a.vecs) * 8;
+  const uint32_t c = ((active ? item : 0) - tap * a.vecs) * E;
   const uint32_t kh = tap / d.kW, kw = tap - kh * d.kW;
   const uint32_t slice = blockIdx.y;
   const uint32_t sliceEnd =
@@ -318,7 +321,7 @@ __global__ __launch_bounds__(256) void depthwiseWeightDeltaKernel(
   uint32_t b = a.divOutH(row);
   uint32_t oh = row - b * d.outH;
   const int khd = int(kh * d.dilH) - d.padH, kwd = int(kw * d.dilW) - d.padW;
-  float acc[8] = {};
+  float acc[E] = {};
   // Four pixels a round: their loads are issued together, so that a wave has
   // eight of them in flight (the walk is bound by load latency, not by
   // arithmetic).
@@ -350,26 +353,31 @@ __global__ __launch_bounds__(256) void depthwiseWeightDeltaKernel(
       }
     }
 #pragma unroll
-    for (int u = 0; u != kUnroll; ++u)
-      fma8(acc, x[u], z[u]);
+    for (int u = 0; u != kUnroll; ++u) {
+      if constexpr (E == 8)
+        fma8(acc, x[u], z[u]);
+      else
+        fma4(acc, x[u].raw, z[u].raw);
+    }
   }
   if (a.slots > 1) {
 #pragma unroll
-    for (int i = 0; i != 8; ++i)
+    for (int i = 0; i != E; ++i)
       meet[threadIdx.x][i] = acc[i];
     __syncthreads();
     if (slot == 0)
       for (uint32_t s2 = 1; s2 != a.slots; ++s2)
 #pragma unroll
-        for (int i = 0; i != 8; ++i)
+        for (int i = 0; i != E; ++i)
           acc[i] += meet[s2 * a.itemsPerBlock + itemLocal][i];
   }
   if (!active || slot != 0)
     return;
   float *dst = partial + (size_t(slice) * a.taps + tap) * d.channels + c;
-  *reinterpret_cast<float4 *>(dst) = float4{acc[0], acc[1], acc[2], acc[3]};
-  *reinterpret_cast<float4 *>(dst + 4) =
-      float4{acc[4], acc[5], acc[6], acc[7]};
+#pragma unroll
+  for (int i = 0; i != E; i += 4)
+    *reinterpret_cast<float4 *>(dst + i) =
+        float4{acc[i], acc[i + 1], acc[i + 2], acc[i + 3]};
 }
 
 /// out[c][tap] = sum over slices of partial[slice][tap][c], in a fixed order:
@@ -436,7 +444,8 @@ __global__ __launch_bounds__(1024) void depthwiseDeltaSumKernel(
 /// Threads of a workgroup: itemsPerBlock items by `slots` parts of a slice.
 void deltaBlockShape(const DepthwiseDesc &d, uint32_t &itemsPerBlock,
                      uint32_t &slots) {
-  const uint64_t items = uint64_t(d.kH) * d.kW * (d.channels / 8);
+  const uint64_t items =
+      uint64_t(d.kH) * d.kW * (uint64_t(d.channels) * d.elemBytes / 16);
   itemsPerBlock = uint32_t(std::min<uint64_t>(std::max<uint64_t>(items, 1), 256));
   slots = 256 / itemsPerBlock;
 }
@@ -446,7 +455,8 @@ uint32_t deltaSlices(const DepthwiseDesc &d) {
   uint32_t itemsPerBlock, slots;
   deltaBlockShape(d, itemsPerBlock, slots);
   const uint64_t pixels = uint64_t(d.batch) * d.outH * d.outW;
-  const uint64_t items = uint64_t(d.kH) * d.kW * (d.channels / 8);
+  const uint64_t items =
+      uint64_t(d.kH) * d.kW * (uint64_t(d.channels) * d.elemBytes / 16);
   const uint64_t itemBlocks = (items + itemsPerBlock - 1) / itemsPerBlock;
   uint64_t slices = (1024 + itemBlocks - 1) / std::max<uint64_t>(itemBlocks, 1);
   slices = std::min<uint64_t>(slices, (pixels + 16 * slots - 1) / (16 * slots));
@@ -535,11 +545,14 @@ hipError_t launchDepthwiseWeightDeltas(const DepthwiseDesc &d, int outType,
                                        const void *acts, const void *deltas,
                                        void *workspace, void *weightDeltas,
                                        hipStream_t stream) {
-  if (d.channels % 8 != 0 || d.inDilH != 1 || d.inDilW != 1)
+  // half tensors, or fp32 ones (the slices' walk only)
+  const uint32_t perVec = 16 / d.elemBytes;
+  if ((d.elemBytes != 2 && d.elemBytes != 4) || d.channels % perVec != 0 ||
+      d.inDilH != 1 || d.inDilW != 1 || (d.elemBytes == 4 && d.dense3x3 == 2))
     return hipErrorInvalidValue;
   DeltaArgs a;
   a.d = d;
-  a.vecs = d.channels / 8;
+  a.vecs = d.channels / perVec;
   a.taps = d.kH * d.kW;
   const uint64_t items = uint64_t(a.taps) * a.vecs;
   const uint64_t pixels = uint64_t(d.batch) * d.outH * d.outW;
@@ -567,9 +580,14 @@ hipError_t launchDepthwiseWeightDeltas(const DepthwiseDesc &d, int outType,
     const dim3 grid{uint32_t((items + a.itemsPerBlock - 1) / a.itemsPerBlock),
                     a.slices},
         block{256};
-    hipLaunchKernelGGL(depthwiseWeightDeltaKernel, grid, block, 0, stream, a,
-                       static_cast<const __half *>(acts),
-                       static_cast<const __half *>(deltas), partial);
+    if (d.elemBytes == 4)
+      hipLaunchKernelGGL(depthwiseWeightDeltaKernel<float>, grid, block, 0,
+                         stream, a, static_cast<const float *>(acts),
+                         static_cast<const float *>(deltas), partial);
+    else
+      hipLaunchKernelGGL(depthwiseWeightDeltaKernel<__half>, grid, block, 0,
+                         stream, a, static_cast<const __half *>(acts),
+                         static_cast<const __half *>(deltas), partial);
   }
   const uint32_t outputs = a.taps * d.channels;
   const dim3 grid2{(outputs + 15) / 16};

@@ -473,12 +473,15 @@ mxconv_plan makePlanWith(const ConvParams &params,
         !plan.zeroConv &&
         !w.inputDilated() && p.batchSize == 1 &&
         p.outputChannelsPerConvGroup == 1 &&
-        params.inputType == poplar::HALF && p.numConvGroups % 8 == 0 &&
+        (params.inputType == poplar::HALF ||
+         params.inputType == poplar::FLOAT) &&
+        p.numConvGroups % (16 / params.inputType.size()) == 0 &&
         p.numConvGroups * p.inputChannelsPerConvGroup *
-                std::size_t(w.inH) * w.inW * 2 <
+                std::size_t(w.inH) * w.inW * params.inputType.size() <
             (1ull << 31)) {
       plan.depthwiseWeightUpdate = true;
       mxk::DepthwiseDesc &f = plan.depthwiseForward;
+      f.elemBytes = uint32_t(params.inputType.size());
       f.batch = uint32_t(p.inputChannelsPerConvGroup);
       f.channels = uint32_t(p.numConvGroups);
       f.inH = w.inH, f.inW = w.inW;
@@ -493,6 +496,7 @@ mxconv_plan makePlanWith(const ConvParams &params,
       const mxk::DepthwiseRowsLaunch l =
           mxk::depthwiseRowsDeltaLaunchShape(f);
       if (options.planConstraints.rowRing != 0 &&
+          params.inputType == poplar::HALF &&
           mxk::depthwiseRowsDeltaTakes(f) &&
           (options.planConstraints.rowRing == 1 ||
            // (strips of fewer than four columns read mostly halo: N = 32,

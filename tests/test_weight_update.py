@@ -412,6 +412,23 @@ def test_depthwise_weight_deltas_on_gpu(oracle, kw, out_type):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kw", DEPTHWISE_WU_CASES[:5] + [
+    dict(batch=3, field=(9, 9), kernel=(3, 3), groups=12, pad=1)])
+def test_depthwise_weight_deltas_fp32(oracle, kw):
+    """fp32 tensors: vectors of four channels, +-1 data exact."""
+    p = make_params(pa.FLOAT, pa.FLOAT, **kw)
+    rng = np.random.default_rng(25)
+    C = p.numConvGroups
+    x = rng.choice([-1.0, 1.0], (p.batchSize, C, *p.inputFieldShape))
+    dz = rng.choice([-1.0, 1.0], (p.batchSize, C, *p.getOutputFieldShape()))
+    got, plan = run_weight_update(p, x.astype(np.float32),
+                                  dz.astype(np.float32))
+    assert "depthwise weight-delta kernel" in plan.describe(), plan.describe()
+    np.testing.assert_array_equal(got, oracle.weight_deltas(p, x, dz,
+                                                            threads=8))
+
+
+@pytest.mark.gpu
 def test_depthwise_weight_deltas_of_signs_are_exact(oracle):
     p = make_params(pa.HALF, pa.FLOAT, batch=2, field=(9, 9), kernel=(3, 3),
                     groups=16, stride=2, pad=1)
