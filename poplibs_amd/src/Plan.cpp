@@ -375,11 +375,18 @@ unsigned chooseConvGroupsPerGroup(const ConvParams &p,
   };
   if (pc.convGroupsPerGroup != 0)
     return usable(pc.convGroupsPerGroup) ? pc.convGroupsPerGroup : 1u;
-  if (ci < 2 || ci * eb >= 64)
+  // (one input channel per group with several output channels - a depthwise
+  // layer with a channel multiplier - included: 64 groups of 1 -> 2 channels
+  // run as one of 64 -> 128)
+  if (ci * eb >= 64)
     return 1;
   for (std::size_t f = 2; f <= groups; ++f)
     if (usable(f) && f * ci * eb >= 128)
       return f * co <= 256 ? unsigned(f) : 1u;
+  // (too few groups for a whole slice: all of them, where that makes two
+  // vectors of channels or more)
+  if (usable(groups) && groups * ci * eb >= 32 && groups * co <= 256)
+    return unsigned(groups);
   return 1;
 }
 

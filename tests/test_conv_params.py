@@ -710,8 +710,13 @@ def test_planner_runs_small_conv_groups_as_one():
     # more than 256 output channels, too few groups for a whole slice
     assert per_group(ci=32, co=32, groups=8) == 1
     assert per_group(ci=1, co=1, groups=64) == 1
+    # ... but a depthwise layer with a channel multiplier is not
+    assert per_group(ci=1, co=2, groups=64) == 64
+    assert per_group(ci=1, co=6, groups=64) == 1
     assert per_group(ci=4, co=64, groups=32) == 1
-    assert per_group(ci=4, co=4, groups=8) == 1
+    # too few groups for a whole slice: all of them as one
+    assert per_group(ci=4, co=4, groups=8) == 8
+    assert per_group(ci=2, co=2, groups=4) == 1
     assert per_group({"pass": "TRAINING_BWD"}, ci=4, co=4, groups=32) == 16
     # the weight update pass of such a layer is planned for the layer with
     # the same groups taken as one

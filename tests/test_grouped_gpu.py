@@ -64,6 +64,9 @@ CASES = [
     # a 1-D field, kernel dilation
     (dict(batch=2, field=(40,), kernel=(3,), ci=8, co=4, groups=16, pad=2,
           kdil=2), 8),
+    # a depthwise layer with a channel multiplier: 64 groups of 1 -> 2
+    (dict(batch=2, field=(10, 9), kernel=(3, 3), ci=1, co=2, groups=64,
+          pad=1), 64),
     # left alone: groups of 32 channels, depthwise, many outputs per group
     (dict(batch=2, field=(9, 9), kernel=(3, 3), ci=32, co=32, groups=4,
           pad=1), 1),
@@ -149,6 +152,8 @@ WU_CASES = [
     (dict(batch=2, field=(10, 10), kernel=(1, 1), ci=16, co=8, groups=8), 4),
     (dict(batch=4, field=(9, 8), kernel=(3, 3), ci=32, co=32, groups=4,
           pad=1), 1),
+    (dict(batch=3, field=(8, 8), kernel=(3, 3), ci=1, co=2, groups=64,
+          pad=1), 64),
 ]
 
 
