@@ -369,13 +369,15 @@ __device__ __forceinline__ void igemmTile(
                      : UNI && MODE == kMaskTaps ? ~e.y
                                                 : e.y;
         originW[r] = int(e.y & 0xffffu) - 32768;
-        khLo[r] = e.y & 0xffu, khSpan[r] = (e.y >> 8) & 0xffu;
-        kwLo[r] = (e.y >> 16) & 0xffu, kwSpan[r] = e.y >> 24;
         if constexpr (MODE == kRangeTaps) {
+          // columns: 16 bits a piece; rows and planes: 8 bits a piece
+          kwLo[r] = e.y & 0xffffu, kwSpan[r] = e.y >> 16;
           const uint32_t planes = depthTable[(r * 4 + pw) * 8 + rowInBlock];
-          kdLo[r] = planes & 0xffu, kdSpan[r] = planes >> 8;
+          khLo[r] = planes & 0xffu, khSpan[r] = (planes >> 8) & 0xffu;
+          kdLo[r] = (planes >> 16) & 0xffu, kdSpan[r] = planes >> 24;
         } else {
-          kdLo[r] = 0, kdSpan[r] = 1;
+          khLo[r] = kwLo[r] = kdLo[r] = 0;
+          khSpan[r] = kwSpan[r] = kdSpan[r] = 1;
         }
       }
       // The consumers start as soon as step 0 is there; the input loads of
@@ -453,24 +455,27 @@ __device__ __forceinline__ void igemmTile(
                      : 0u};
       } else if (mode == kRangeTaps) {
         // Kernel rows kh with lo <= base + kh * dilation < hi form an
-        // interval; so do the columns.  {first, length} of each, 8 bits a
-        // piece; an invalid row gets empty ones.
-        auto range = [](int base, int lo, int hi, int dil, int size) {
+        // interval; so do the columns and the planes.  {first, length} of
+        // each: the columns' in 16 bits a piece (the kernel of a 1-D layer's
+        // weight update pass is as long as the layer's output), the others'
+        // in 8; an invalid row gets an empty interval of columns.
+        auto range = [](int base, int lo, int hi, int dil, int size,
+                        int bits) {
           auto ceilDiv = [](int n, int dv) {
             return n >= 0 ? (n + dv - 1) / dv : -((-n) / dv);
           };
           int first = ceilDiv(lo - base, dil), last = ceilDiv(hi - base, dil);
           first = first < 0 ? 0 : first > size ? size : first;
           last = last < first ? first : last > size ? size : last;
-          return uint32_t(first) | (uint32_t(last - first) << 8);
+          return uint32_t(first) | (uint32_t(last - first) << bits);
         };
-        const uint32_t ranges =
-            range(ihBase, int(d.loH), int(d.hiH), int(d.dilH), int(d.kH)) |
-            (range(iwBase, int(d.loW), int(d.hiW), int(d.dilW), int(d.kW))
-             << 16);
-        rowTable[t] = uint2{originOffset, rowValid ? ranges : 0u};
+        const uint32_t columns =
+            range(iwBase, int(d.loW), int(d.hiW), int(d.dilW), int(d.kW), 16);
+        rowTable[t] = uint2{originOffset, rowValid ? columns : 0u};
         depthTable[t] =
-            range(idBase, int(d.loD), int(d.hiD), int(d.dilD), int(d.kD));
+            range(ihBase, int(d.loH), int(d.hiH), int(d.dilH), int(d.kH), 8) |
+            (range(idBase, int(d.loD), int(d.hiD), int(d.dilD), int(d.kD), 8)
+             << 16);
       } else {
         uint32_t mask = 0;
         if (d.dilD == 1 && d.dilH == 1 && d.dilW == 1) {
@@ -762,50 +767,75 @@ hipError_t dispatch(const KernelKey &k, const Launch &launch) {
 
 /// out[i] = sum over parts of partial[part][i] (+ bias of i's channel).  The
 /// parts are added in a fixed order: four interleaved running sums (so that
-/// four loads are in flight per lane), combined at the end.
-template <class OutT>
+/// four loads are in flight per lane), combined at the end.  A thread takes V
+/// neighbouring channels of one pixel: 4 where the channel count is a multiple
+/// of 4 (one 16-byte load per part), else 1.
+template <class OutT, int V>
 __global__ __launch_bounds__(64) void splitKReduceKernel(
     const float *__restrict__ partial, uint32_t parts, uint64_t elems,
     uint32_t channels, const OutT *__restrict__ bias, OutT *__restrict__ out,
     bool transposed) {
-  const uint64_t i = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+  const uint64_t i = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) * V;
   if (i >= elems)
     return;
-  // elems and channels are multiples of 4 (checked by the launcher)
-  float4 sum[4] = {};
+  float sum[4][V] = {};
+  const auto add = [&](int u, uint32_t part) {
+    const float *src = partial + uint64_t(part) * elems + i;
+    if constexpr (V == 4) {
+      const float4 v = *reinterpret_cast<const float4 *>(src);
+      sum[u][0] += v.x, sum[u][1] += v.y, sum[u][2] += v.z, sum[u][3] += v.w;
+    } else {
+      sum[u][0] += *src;
+    }
+  };
   uint32_t p = 0;
   for (; p + 4 <= parts; p += 4) {
 #pragma unroll
-    for (int u = 0; u != 4; ++u) {
-      const float4 v = *reinterpret_cast<const float4 *>(
-          partial + uint64_t(p + u) * elems + i);
-      sum[u].x += v.x, sum[u].y += v.y, sum[u].z += v.z, sum[u].w += v.w;
-    }
+    for (int u = 0; u != 4; ++u)
+      add(u, p + u);
   }
-  for (; p != parts; ++p) {
-    const float4 v =
-        *reinterpret_cast<const float4 *>(partial + uint64_t(p) * elems + i);
-    sum[0].x += v.x, sum[0].y += v.y, sum[0].z += v.z, sum[0].w += v.w;
-  }
-  float v[4] = {(sum[0].x + sum[1].x) + (sum[2].x + sum[3].x),
-                (sum[0].y + sum[1].y) + (sum[2].y + sum[3].y),
-                (sum[0].z + sum[1].z) + (sum[2].z + sum[3].z),
-                (sum[0].w + sum[1].w) + (sum[2].w + sum[3].w)};
+  for (; p != parts; ++p)
+    add(0, p);
+  float v[V];
+#pragma unroll
+  for (int e = 0; e != V; ++e)
+    v[e] = (sum[0][e] + sum[1][e]) + (sum[2][e] + sum[3][e]);
   const uint32_t c = uint32_t(i % channels);
   if (bias) {
 #pragma unroll
-    for (int e = 0; e != 4; ++e)
+    for (int e = 0; e != V; ++e)
       v[e] += Load<OutT>::at(bias, c + e, 0);
   }
   if (transposed) {
     // [channel][pixel]
     const uint64_t pixels = elems / channels, pixel = i / channels;
 #pragma unroll
-    for (int e = 0; e != 4; ++e)
+    for (int e = 0; e != V; ++e)
       storeOut(out, (c + e) * pixels + pixel, v[e]);
     return;
   }
-  storeOut4(out + i, v);
+  if constexpr (V == 4)
+    storeOut4(out + i, v);
+  else
+    storeOut(out, i, v[0]);
+}
+
+template <class OutT>
+void launchSplitKReduce(const float *partial, uint32_t parts, uint64_t elems,
+                        uint32_t channels, const void *bias, void *out,
+                        bool transposed, hipStream_t stream) {
+  const int v = channels % 4 == 0 ? 4 : 1;
+  const uint32_t blocks = uint32_t((elems / v + 63) / 64);
+  if (v == 4)
+    hipLaunchKernelGGL((splitKReduceKernel<OutT, 4>), dim3(blocks), dim3(64),
+                       0, stream, partial, parts, elems, channels,
+                       static_cast<const OutT *>(bias),
+                       static_cast<OutT *>(out), transposed);
+  else
+    hipLaunchKernelGGL((splitKReduceKernel<OutT, 1>), dim3(blocks), dim3(64),
+                       0, stream, partial, parts, elems, channels,
+                       static_cast<const OutT *>(bias),
+                       static_cast<OutT *>(out), transposed);
 }
 
 } // namespace
@@ -873,8 +903,9 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
        d.inH >= (1u << 24) || d.inDilH >= (1u << 24) ||
        d.inDilW >= (1u << 24)))
     return hipErrorInvalidValue;
-  // the ranges of valid kernel rows and columns are kept in 8 bits each
-  if (mode == kRangeTaps && (d.kH > 255 || d.kW > 255))
+  // the ranges of valid kernel rows are kept in 8 bits a piece, of columns
+  // in 16
+  if (mode == kRangeTaps && (d.kH > 255 || d.kW > 32767))
     return hipErrorInvalidValue;
   // a depth dimension goes with the tap mask and the ranges
   if (mode == kDilatedTaps && (d.inD != 1 || d.outD != 1 || d.kD != 1))
@@ -893,8 +924,7 @@ hipError_t prepare(const IgemmDesc &d, int inType, bool haveWorkspace,
        (d.outH != 0 && (d.outH - 1) * d.outStepH + d.outOffH >= d.outFullH) ||
        (d.outW != 0 && (d.outW - 1) * d.outStepW + d.outOffW >= d.outFullW)))
     return hipErrorInvalidValue;
-  if (d.splitK > 1 &&
-      (!haveWorkspace || (d.groups * d.outChansPerGroup) % 4 != 0))
+  if (d.splitK > 1 && !haveWorkspace)
     return hipErrorInvalidValue;
   a.d = d;
   a.d.outFullD = fullD;
@@ -972,20 +1002,15 @@ hipError_t launchIgemm(const IgemmDesc &d, int inType, int outType,
   const uint64_t elems = uint64_t(a.M) * channels;
   if (elems == 0)
     return hipSuccess;
-  const uint64_t blocks = (elems / 4 + 63) / 64;
-  if (blocks > 0x7fffffffull)
+  if ((elems + 63) / 64 > 0x7fffffffull)
     return hipErrorInvalidConfiguration;
   const float *partial = static_cast<const float *>(workspace);
   if (outType == kHalf)
-    hipLaunchKernelGGL(splitKReduceKernel<__half>, dim3(uint32_t(blocks)),
-                       dim3(64), 0, stream, partial, d.splitK, elems,
-                       channels, static_cast<const __half *>(bias),
-                       static_cast<__half *>(out), d.outTransposed != 0);
+    launchSplitKReduce<__half>(partial, d.splitK, elems, channels, bias, out,
+                               d.outTransposed != 0, stream);
   else if (outType == kFloat)
-    hipLaunchKernelGGL(splitKReduceKernel<float>, dim3(uint32_t(blocks)),
-                       dim3(64), 0, stream, partial, d.splitK, elems,
-                       channels, static_cast<const float *>(bias),
-                       static_cast<float *>(out), d.outTransposed != 0);
+    launchSplitKReduce<float>(partial, d.splitK, elems, channels, bias, out,
+                              d.outTransposed != 0, stream);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

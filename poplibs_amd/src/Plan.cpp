@@ -642,8 +642,8 @@ mxconv_plan makePlanWith(const ConvParams &params,
               s.inDilH >= (1u << 24) || s.inDilW >= (1u << 24)))
       igemmWhyNot = "input rows too long for the arithmetic tap addressing";
     else if (!s.inputDilated() && std::size_t(s.kD) * s.kH * s.kW > 32 &&
-             (s.kD > 255 || s.kH > 255 || s.kW > 255))
-      igemmWhyNot = "kernel extent above 255";
+             (s.kD > 255 || s.kH > 255 || s.kW > 32767))
+      igemmWhyNot = "kernel extent above 255 (32 767 in the last dimension)";
     else if (!inputAddressable() ||
              s.batch * s.outD * s.outH * s.outW >= (1ull << 31) ||
              p.numConvGroups * ((co + 127) / 128 * 128) * s.kD * s.kH * s.kW *
@@ -839,9 +839,8 @@ mxconv_plan makePlanWith(const ConvParams &params,
                                     4))
         parts = 1;
       const std::size_t chans = p.numConvGroups * co;
-      // the reduction reads and writes vectors of four channels; partial
-      // tiles of more than 1 GB are not worth it
-      if (chans % 4 != 0 || parts * m * chans * 4 > (1ull << 30))
+      // partial tiles of more than 1 GB are not worth it
+      if (parts * m * chans * 4 > (1ull << 30))
         parts = 1;
       // (the sum of the parts is written pixel after pixel: not into a
       // padded output field)

@@ -681,6 +681,15 @@ GENERAL_CASES = [
     # a weight-update-like pass: the "kernel" is a whole 12x12 field, dilated
     dict(batch=16, field=(26, 26), kernel=(12, 12), ci=8, co=24, kdil=2,
          padLower=(1, 1), padUpper=(0, 0)),
+    # one dimension, a kernel of more than 255 taps (a 1-D layer's weight
+    # update pass): windows that hang over both ends of the field, and a
+    # dilated kernel that steps over it
+    dict(batch=3, field=(500,), kernel=(300,), ci=8, co=24, pad=40),
+    dict(batch=2, field=(1200,), kernel=(397,), ci=16, co=8, kdil=3,
+         padLower=(5,), padUpper=(17,), stride=2),
+    # (and with rows: 3 x 280)
+    dict(batch=2, field=(6, 300), kernel=(3, 280), ci=8, co=16,
+         padLower=(1, 3), padUpper=(1, 0)),
 ]
 
 
@@ -710,6 +719,11 @@ SPLIT_K_CASES = [
     # (72 k-steps: long enough for the parts to pay for their round trip)
     (dict(batch=16, field=(26, 26), kernel=(12, 12), ci=32, co=24, kdil=2,
           padLower=(1, 1), padUpper=(0, 0)), None),
+    # channel counts that are no multiple of four: the parts are added one
+    # channel per thread
+    (dict(batch=2, field=(9, 7), kernel=(3, 3), ci=64, co=3, pad=1), 4),
+    (dict(batch=1, field=(8, 8), kernel=(5, 5), ci=96, co=7, pad=2, groups=3),
+     None),
 ]
 
 

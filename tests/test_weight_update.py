@@ -353,6 +353,51 @@ def test_weight_deltas_of_a_small_batch_run_on_the_matrix_cores(oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("co", [3, 5])
+@pytest.mark.parametrize("dt", [pa.HALF, pa.FLOAT])
+def test_weight_deltas_of_a_layer_with_few_output_channels(oracle, co, dt):
+    # (an RGB head.)  The pass has `co` output channels, a long K (the layer's
+    # field x its batch) and a handful of output tiles: K is cut into parts,
+    # and the parts are added one channel per thread where the channel count
+    # is no multiple of four.
+    from gpu_helpers import quantize
+    p = make_params(dt, pa.FLOAT, batch=8, field=(28, 28), kernel=(3, 3),
+                    ci=32, co=co, pad=1)
+    rng = np.random.default_rng(28)
+    xq, xd = quantize(rng.standard_normal((8, 32, 28, 28)), dt)
+    dq, dd = quantize(rng.standard_normal((8, co, 28, 28)) * 0.1, dt)
+    got, plan = run_weight_update(p, xq, dq)
+    assert "implicit GEMM" in plan.describe(), plan.describe()
+    assert "K split into parts" in plan.describe(), plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert rel_l2(got, want) <= 1e-5, (rel_l2(got, want), plan.describe())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [pa.HALF, pa.FLOAT])
+@pytest.mark.parametrize("kw", [
+    dict(batch=8, field=(1500,), kernel=(3,), ci=16, co=24, pad=1),
+    dict(batch=5, field=(900,), kernel=(5,), ci=8, co=8, pad=2, stride=2,
+         groups=2),
+])
+def test_weight_deltas_of_a_long_1d_layer(oracle, kw, dt):
+    # the pass's own convolution has a kernel as long as the layer's output:
+    # hundreds of taps in one dimension, on the matrix cores all the same
+    from gpu_helpers import quantize
+    p = make_params(dt, pa.FLOAT, **kw)
+    rng = np.random.default_rng(29)
+    xq, xd = quantize(rng.standard_normal(
+        (p.batchSize, p.getNumInputChans(), *p.inputFieldShape)), dt)
+    dq, dd = quantize(rng.standard_normal(
+        (p.batchSize, p.getNumOutputChans(), *p.getOutputFieldShape())) * 0.1,
+        dt)
+    got, plan = run_weight_update(p, xq, dq)
+    assert "generic direct" not in plan.describe(), plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert rel_l2(got, want) <= 1e-5, (rel_l2(got, want), plan.describe())
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("batch", [8, 16])
 @pytest.mark.parametrize("out_type", [pa.HALF, pa.FLOAT])
 def test_weight_deltas_of_a_truncated_kernel(oracle, batch, out_type):
