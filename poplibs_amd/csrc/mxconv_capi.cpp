@@ -594,6 +594,19 @@ mxconv_status mxconv_plan_constraints(const mxconv_plan *plan, char *buffer,
   });
 }
 
+namespace {
+size_t ownTensorsWorkspaceBytes(const mxconv_plan *plan);
+
+/// Workspace the planned launch sequence needs.  (A weight update pass on
+/// the layer's own tensors keeps its partial sums and deltas there, not the
+/// intermediates of the pass's convolution.)
+size_t estimatedWorkspaceBytes(const mxconv_plan *plan) {
+  return plan->denseWeightUpdate || plan->depthwiseWeightUpdate
+             ? ownTensorsWorkspaceBytes(plan)
+             : plan->workspaceBytes;
+}
+} // namespace
+
 mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
                                           uint64_t *cycles,
                                           uint64_t *memory_bytes) {
@@ -604,7 +617,7 @@ mxconv_status mxconv_plan_estimated_costs(const mxconv_plan *plan,
   const double us = plan->estimatedMicroseconds();
   *cycles = us < 0 ? MXCONV_COST_UNKNOWN
                    : uint64_t(us * mxconv_plan::kEstimateClockMHz + 0.5);
-  *memory_bytes = plan->workspaceBytes;
+  *memory_bytes = estimatedWorkspaceBytes(plan);
   return MXCONV_OK;
 }
 
@@ -619,7 +632,7 @@ mxconv_status mxconv_plan_detailed_costs(const mxconv_plan *plan,
   costs->serial_split = e.serialSplit;
   costs->rearrangement.memory_bytes = e.rearrangementBytes;
   costs->reduction.memory_bytes = e.reductionBytes;
-  costs->total.memory_bytes = plan->workspaceBytes;
+  costs->total.memory_bytes = estimatedWorkspaceBytes(plan);
   if (!e.known) {
     costs->rearrangement.cycles = costs->compute.cycles =
         costs->reduction.cycles = costs->total.cycles = MXCONV_COST_UNKNOWN;
@@ -1399,6 +1412,10 @@ WuWorkspace wuWorkspace(const mxconv_plan *plan) {
   w.planWorkspace = take(plan->workspaceBytes);
   w.total = at;
   return w;
+}
+
+size_t ownTensorsWorkspaceBytes(const mxconv_plan *plan) {
+  return wuWorkspace(plan).total;
 }
 
 uint64_t product(const std::vector<std::size_t> &shape) {

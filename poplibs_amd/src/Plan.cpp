@@ -770,7 +770,8 @@ mxconv_plan makePlanWith(const ConvParams &params,
     // estimates (N = 32, 14 x 14, 1024 -> 256: 8.9 -> 7.1 us; 7 x 7, 2048 ->
     // 512: 12.8 -> 10.2; but 14 x 14, 1024 -> 512, 392 narrow tiles: 10.2
     // against 12.1, and the estimate keeps the wide tile there).
-    bool narrowWhole = false; // ... chosen: K stays whole
+    bool narrowWhole = false;    // ... chosen: K stays whole
+    std::size_t narrowSplit = 0; // ... or narrow tiles with K in this many parts
     if (!pc.blockN && !pc.splitK && !pc.stages && co > 64 &&
         g.blockM == 128) {
       const std::size_t m = s.batch * s.outD * s.outH * s.outW;
@@ -793,8 +794,25 @@ mxconv_plan makePlanWith(const ConvParams &params,
                                         (kSteps + parts - 1) / parts, 1, 128,
                                         unsigned(parts), partial)
                     : 1e30);
-      if (estimateStreaming(narrow, kSteps, 2, 64, 1, 0) < wideUs)
+      const double wideWholeUs = estimateStreaming(
+          wide, kSteps, wide > gfx950::numCUs ? 2 : 1, 128, 1, 0);
+      if (estimateStreaming(narrow, kSteps, 2, 64, 1, 0) < wideUs) {
         g.blockN = 64, narrowWhole = true;
+      } else if (wideUs < wideWholeUs && narrow * 2 <= gfx950::numCUs) {
+        // K split wins: then over narrow tiles, in half as many parts of at
+        // least 8 k-steps - the same number of workgroups, each with half the
+        // weights to fetch per k-step and half the fp32 tile to write, and
+        // half the partial tiles in all.  Measured for skinny products and
+        // deep layers alike (wide -> narrow, us): 32 x 4096 x 4096 13.3 ->
+        // 11.4, 256 x 4096 x 1024 17.5 -> 12.2, 512 x 4096 x 1024 18.1 ->
+        // 14.2, N = 8 7 x 7 3 x 3 512 -> 512 15.2 -> 11.0, N = 1 9.9 -> 8.4;
+        // level where the rule already chose few parts (N = 32 7 x 7 3 x 3
+        // 512 -> 512 19.0 -> 18.6, 14 x 14 stride 2 18.2 -> 18.4).
+        const std::size_t narrowParts = std::min<std::size_t>(
+            gfx950::numCUs / narrow, kSteps / 8);
+        if (narrowParts > 1)
+          g.blockN = 64, narrowSplit = narrowParts;
+      }
     }
     const bool anyHeight = pc.patch == 2 && g.blockM >= 1 && g.blockM <= 112;
     if ((g.blockM != 128 && g.blockM != 64 && !anyHeight) ||
@@ -822,6 +840,8 @@ mxconv_plan makePlanWith(const ConvParams &params,
       std::size_t parts = 1;
       if (pc.splitK)
         parts = pc.splitK;
+      else if (narrowSplit)
+        parts = narrowSplit;
       else if (!narrowWhole && tiles != 0 && tiles * 2 <= gfx950::numCUs &&
                kSteps >= 16)
         parts = std::min<std::size_t>(gfx950::numCUs / tiles, kSteps / 4);
@@ -830,7 +850,7 @@ mxconv_plan makePlanWith(const ConvParams &params,
       // and the second kernel: N = 32, 14 x 14, 1 x 1, 1024 -> 256 channels
       // (98 tiles of 16 k-steps) 16.4 us in two parts, 8.9 us whole; 7 x 7,
       // 3 x 3, 512 -> 512 (52 tiles of 72 k-steps) 18.7 in four, 21.1 whole.
-      if (!pc.splitK && parts > 1 &&
+      if (!pc.splitK && !narrowSplit && parts > 1 &&
           estimateStreaming(tiles, kSteps, g.blockN == 64 ? 2 : 1, g.blockN, 1,
                             0) <=
               estimateStreaming(tiles * parts, (kSteps + parts - 1) / parts,

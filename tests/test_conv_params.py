@@ -404,16 +404,18 @@ def test_planner_choices():
                                kernel=(28, 28), ci=32, co=128, pad=1))
     assert "implicit GEMM" in many.describe()
     assert "ranges of valid kernel rows" in many.describe()
-    # few output tiles, long K: K is cut into parts
-    assert "K split into parts         28" in many.describe()
-    assert many.buffer_bytes(4) == 28 * 128 * 9 * 128 * 4
+    # few output tiles, long K: K is cut into parts, over narrow tiles
+    assert "K split into parts         14" in many.describe()
+    assert "block M x N x K            128 x 64 x 64" in many.describe()
+    assert many.buffer_bytes(4) == 14 * 128 * 9 * 128 * 4
     assert "K split" not in pa.Plan(c2).describe()
     # ... unless the parts' round trip through memory costs more than it
     # saves: 98 tiles of 16 k-steps stay whole
     assert "K split" not in pa.Plan(make_params(
         pa.HALF, batch=32, field=(14, 14), kernel=(1, 1), ci=1024,
         co=256)).describe()
-    assert "K split into parts         4" in pa.Plan(make_params(
+    # (two parts over 104 narrow tiles rather than four over 52 wide ones)
+    assert "K split into parts         2" in pa.Plan(make_params(
         pa.HALF, batch=32, field=(7, 7), kernel=(3, 3), ci=512, co=512,
         pad=1)).describe()
     # one workgroup per CU or fewer: four LDS stages; more workgroups than
