@@ -310,6 +310,35 @@ hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
                            const void *bias, void *out, const QuarterInfo &q,
                            hipStream_t stream);
 
+/// Convolution of an input with 1 to 4 channels (one group, half inputs, a
+/// 2-D field, stride, zero padding, input truncation; nothing dilated) on the
+/// matrix cores without padding the channels: a kernel row's kW * Ci
+/// neighbouring elements (32 at most) are one k-step.  16, 32, 48 or 64 output
+/// channels, up to 7 kernel rows.
+struct ThinInputDesc {
+  uint32_t batch, inChans, outChans;
+  uint32_t inH, inW, outH, outW, kH, kW;
+  int32_t padH, padW; // as in IgemmDesc; padW >= 0
+  uint32_t strideH, strideW;
+  uint32_t loH, hiH, loW, hiW; // rows and columns outside read as zeros
+};
+bool thinInputTakes(const ThinInputDesc &d, int inType, int outType);
+/// Elements of the packed weights ([16-channel block][kernel row][lane][8]).
+uint64_t thinInputPackedElems(const ThinInputDesc &d);
+hipError_t launchPackThinInputWeights(const ThinInputDesc &d, const void *src,
+                                      void *dst, hipStream_t stream);
+/// How launchThinInput runs a layer on a chip of `cus` compute units:
+/// persistent workgroups, each taking tiles of `tileRows` output rows of one
+/// image in turn, the input rows under a tile in `ldsBytes` of LDS.
+struct ThinInputLaunch {
+  uint32_t tileRows, ldsBytes;
+  uint64_t tiles, workgroups;
+};
+ThinInputLaunch thinInputLaunchShape(const ThinInputDesc &d, uint32_t cus);
+hipError_t launchThinInput(const ThinInputDesc &d, int inType, int outType,
+                           const void *in, const void *weightsPacked,
+                           const void *bias, void *out, hipStream_t stream);
+
 /// Depthwise (one input and one output channel per group) direct convolution,
 /// 2-D field, stride, zero padding, kernel dilation.
 struct DepthwiseDesc {

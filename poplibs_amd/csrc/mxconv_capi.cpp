@@ -175,6 +175,10 @@ mxconv_status forward(const mxconv_plan *plan, const void *in, const void *w,
       if (st != MXCONV_OK)
         return st;
     }
+    if (plan->thinInputOn)
+      return hipStatus(mxk::launchThinInput(plan->thinInput, inType, outType,
+                                            in, w, bias, out, s),
+                       "thin-input convolution launch");
     if (plan->pointwiseOn)
       return hipStatus(mxk::launchPointwise(plan->pointwise, inType, outType,
                                             in, w, bias, out, q, s),
@@ -689,7 +693,8 @@ std::string packingSignature(const mxconv_plan &p) {
      << p.weightElems << '/' << p.weightPackedElems << "/cg"
      << p.convGroupsPerGroup;
   if (p.kernel == mxconv_plan::Kernel::IGEMM) {
-    os << "/pw" << p.pointwiseOn << "/patch" << p.igemm.patch << "/co"
+    os << "/pw" << p.pointwiseOn << "/thin" << p.thinInputOn << "/patch"
+       << p.igemm.patch << "/co"
        << p.coPadded << "/k" << p.kPadded << "/ci" << p.paddedInputChans
        << "/sel" << p.kernelSelected;
     auto taps = [&](const mxk::IgemmTapSelection &t) {
@@ -756,6 +761,10 @@ mxconv_status mxconv_pack_weights(const mxconv_plan *plan,
       weights_external = fused;
       groups /= f, co *= f, ci *= f;
     }
+    if (plan->thinInputOn)
+      return hipStatus(mxk::launchPackThinInputWeights(
+                           plan->thinInput, weights_external, weights_packed, s),
+                       "weight packing");
     if (plan->pointwiseOn)
       return hipStatus(mxk::launchPackPointwiseWeights(
                            plan->pointwise, weights_external, weights_packed, s),
@@ -1008,7 +1017,8 @@ mxconv_status mxconv_multi_fwd(size_t n, const mxconv_plan *const *plans,
     // (a plan with more to a launch than its one kernel - a padded copy of
     // the input, several phases, an output border to fill - runs on its own)
     if (p->outputElems == 0 || p->kernel != mxconv_plan::Kernel::IGEMM ||
-        p->pointwiseOn || p->paddedInputChans || !p->igemmPhases.empty() ||
+        p->pointwiseOn || p->thinInputOn || p->paddedInputChans ||
+        !p->igemmPhases.empty() ||
         p->outputPadded || p->igemm.patch)
       return false;
     unsplit[slot] = p->igemm;
@@ -1490,7 +1500,8 @@ mxconv_status fusedWeightDeltas(const mxconv_plan *plan, const void *zDeltas,
       acts,        ws + w.input, uint32_t(B), uint32_t(X), uint32_t(G),
       uint32_t(Ci), B,           X * G * B,   G * B};
   const bool direct = plan->kernel == mxconv_plan::Kernel::IGEMM &&
-                      !plan->pointwiseOn && !plan->paddedInputChans &&
+                      !plan->pointwiseOn && !plan->thinInputOn &&
+                      !plan->paddedInputChans &&
                       plan->igemmPhases.empty() && !plan->kernelSelected &&
                       !plan->igemm.patch &&
                       // (a padded output field - the forward kernel was

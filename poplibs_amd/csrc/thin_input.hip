@@ -1,0 +1,482 @@
+// Convolution of an input with very few channels (an image's three, a
+// waveform's one) on the matrix cores, without padding the channels.
+//
+// In a channels-last image the kW pixels under one kernel row are kW * Ci
+// neighbouring elements - 21 for a 7 x 7 kernel over RGB - so a kernel row is
+// one k-step of 32: K = kH * 32 where padding the channels to a whole 16-byte
+// vector gives kH * kW * 8 (224 against 392 for that layer) and costs a copy
+// of the input besides.  The price is alignment: a window starts at any even
+// byte, so the operand is read from LDS as five aligned dwords and shifted
+// into place.
+//
+//   workgroup  = 4 waves; one image's TH output rows at a time (persistent);
+//                the input rows under them lie in LDS, zeros around them
+//   wave       = blocks of 16 neighbouring output pixels, round robin
+//   MFMA       = v_mfma_f32_16x16x32_f16, weights as the row operand:
+//                D[co][pixel] += W[co][k] * X[k][pixel], one per kernel row and
+//                block of 16 output channels; all weights stay in registers
+//   output     = output channels are dealt to the MFMA rows so that a lane
+//                ends up with 4 * CB neighbouring channels of one pixel
+#include "igemm_common.hpp"
+#include "kernels.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+
+namespace mxk {
+namespace {
+
+constexpr int kThinThreads = 256;
+
+struct ThinArgs {
+  ThinInputDesc d;
+  uint32_t tileRows;   // TH: output rows per tile
+  uint32_t ldsRows;    // (TH - 1) * strideH + KH
+  uint32_t pitch;      // bytes of an LDS row
+  uint32_t dataOff;    // byte of input column 0 in an LDS row (16-aligned)
+  uint32_t rowBytes;   // inW * ci * 2
+  uint32_t tilesPerImage, tiles;
+  uint32_t colBlocks;  // blocks of 16 output pixels per row
+  FastDiv divTilesPerImage, divColBlocks;
+  FastDiv divRowUnits; // by the 16-byte vectors (or dwords) of an input row
+  FastDiv divBorder;   // by the dwords of zeros left and right of a row
+  uint32_t biasByte;   // where the fp32 bias lies in LDS
+  uint32_t cutElems;   // elements of a row in truncated columns
+  FastDiv divCut;
+};
+
+/// Output channel held by MFMA row m of channel block cb: lane quarter
+/// Q = m / 4 gets channels Q * 4 * CB + 4 * cb + m % 4, so that its 4 * CB
+/// results are neighbours.
+__host__ __device__ inline uint32_t thinChannelOf(uint32_t cb, uint32_t m,
+                                                  uint32_t blocks) {
+  return (m / 4) * 4 * blocks + 4 * cb + m % 4;
+}
+
+/// Packed weights [cb][kh][lane][8]: lane l holds MFMA row l % 16 and
+/// k = 8 * (l / 16) .. + 7 of kernel row kh, k = kw * Ci + c, zeros beyond
+/// kW * Ci and for kernel rows beyond kH.
+__global__ void packThinWeightsKernel(const __half *__restrict__ src,
+                                      __half *__restrict__ dst,
+                                      ThinInputDesc d, uint32_t rowsPacked,
+                                      uint32_t total) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total)
+    return;
+  const uint32_t e = i % 8, lane = (i / 8) % 64;
+  const uint32_t kh = (i / 512) % rowsPacked, cb = i / 512 / rowsPacked;
+  const uint32_t k = 8 * (lane / 16) + e;
+  const uint32_t co = thinChannelOf(cb, lane % 16, d.outChans / 16);
+  const uint32_t kw = k / d.inChans, c = k % d.inChans;
+  __half v = __float2half(0.0f);
+  if (kh < d.kH && kw < d.kW)
+    v = src[((size_t(co) * d.inChans + c) * d.kH + kh) * d.kW + kw];
+  dst[i] = v;
+}
+
+/// Input rows ih0 .. ih0 + ldsRows - 1 of an image into LDS in units of V
+/// (16 or 4 bytes), zeros for rows outside [loH, hiH).
+template <class V>
+__device__ __forceinline__ void copyRows(const ThinArgs &a, char *lds,
+                                         const char *img, int32_t ih0, int t) {
+  constexpr int kBatch = 8;
+  const uint32_t units = a.rowBytes / uint32_t(sizeof(V));
+  const uint32_t total = a.ldsRows * units;
+  for (uint32_t first = 0; first < total; first += kBatch * kThinThreads) {
+    V v[kBatch];
+    uint32_t at[kBatch];
+#pragma unroll
+    for (int u = 0; u != kBatch; ++u) {
+      const uint32_t i = first + u * kThinThreads + t;
+      const uint32_t row = a.divRowUnits(i), c = i - row * units;
+      const int32_t ih = ih0 + int32_t(row);
+      at[u] = i < total ? row * a.pitch + a.dataOff + c * uint32_t(sizeof(V))
+                        : ~0u;
+      v[u] = V{};
+      if (i < total && ih >= int32_t(a.d.loH) && ih < int32_t(a.d.hiH))
+        v[u] = reinterpret_cast<const V *>(img + size_t(ih) * a.rowBytes)[c];
+    }
+#pragma unroll
+    for (int u = 0; u != kBatch; ++u)
+      if (at[u] != ~0u)
+        *reinterpret_cast<V *>(lds + at[u]) = v[u];
+  }
+}
+
+template <int CB, int KH, class OutT>
+__global__ __launch_bounds__(kThinThreads)
+    __attribute__((amdgpu_waves_per_eu(2))) void thinInputKernel(
+    ThinArgs a, const __half *__restrict__ in,
+    const __half *__restrict__ weightsPacked, const OutT *__restrict__ bias,
+    OutT *__restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const ThinInputDesc &d = a.d;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+
+  // The weights, through LDS into every wave's registers.
+  {
+    const uintx4 *src = reinterpret_cast<const uintx4 *>(weightsPacked);
+    uintx4 *dst = reinterpret_cast<uintx4 *>(lds);
+    constexpr int kVecs = CB * KH * 64;
+    uintx4 v[(kVecs + kThinThreads - 1) / kThinThreads];
+#pragma unroll
+    for (int u = 0; u * kThinThreads < kVecs; ++u)
+      if (u * kThinThreads + t < kVecs)
+        v[u] = src[u * kThinThreads + t];
+#pragma unroll
+    for (int u = 0; u * kThinThreads < kVecs; ++u)
+      if (u * kThinThreads + t < kVecs)
+        dst[u * kThinThreads + t] = v[u];
+  }
+  __syncthreads();
+  half8 w[CB][KH];
+#pragma unroll
+  for (int cb = 0; cb != CB; ++cb)
+#pragma unroll
+    for (int kh = 0; kh != KH; ++kh)
+      w[cb][kh] =
+          reinterpret_cast<const half8 *>(lds)[(cb * KH + kh) * 64 + lane];
+  __syncthreads();
+
+  // Zeros left and right of the rows' data: written once, never overwritten.
+  {
+    const uint32_t left = a.dataOff / 4;
+    const uint32_t right = (a.pitch - a.dataOff - a.rowBytes) / 4;
+    const uint32_t per = left + right;
+    for (uint32_t i = t; i < a.ldsRows * per; i += kThinThreads) {
+      const uint32_t row = a.divBorder(i), c = i - row * per;
+      const uint32_t byte =
+          c < left ? c * 4 : a.dataOff + a.rowBytes + (c - left) * 4;
+      *reinterpret_cast<uint32_t *>(lds + row * a.pitch + byte) = 0;
+    }
+  }
+
+  // This lane's part of an operand: pixel lane % 16 of a block, elements
+  // 8 * (lane / 16) .. + 7 of a kernel row.  Its byte within an LDS row, for
+  // block 0 (a block further on is 16 * strideW pixels further on):
+  const uint32_t pixelBytes = d.inChans * 2;
+  const int32_t colByte0 =
+      int32_t(a.dataOff) +
+      (int32_t((lane & 15) * d.strideW) - d.padW) * int32_t(pixelBytes) +
+      (lane >> 4) * 16;
+  // (a multiple of 32 bytes: every block's operand starts at the same byte
+  // of a dword)
+  const uint32_t blockStep = 16 * d.strideW * pixelBytes;
+  const uint32_t colWord0 = uint32_t(colByte0) & ~3u;
+  const uint32_t shift = uint32_t(colByte0) & 3u;
+  // The operand's dword i is bytes shift .. shift + 3 of the aligned dwords
+  // i and i + 1, with the elements beyond the kernel row's kW * Ci wiped:
+  // one byte permute does both (selector byte b + shift picks that byte of
+  // the pair, 0x0c a zero).
+  uint32_t pick[4];
+#pragma unroll
+  for (int i = 0; i != 4; ++i) {
+    const uint32_t k = (lane >> 4) * 8 + 2 * i, kEnd = d.kW * d.inChans;
+    const uint32_t lo = k < kEnd ? (shift | ((shift + 1) << 8)) : 0x0c0cu;
+    const uint32_t hi =
+        k + 1 < kEnd ? ((shift + 2) | ((shift + 3) << 8)) : 0x0c0cu;
+    pick[i] = lo | (hi << 16);
+  }
+  // the bias, as fp32, behind the rows in LDS: a lane's 4 * CB channels are
+  // read back when a block is stored
+  const uint32_t chan0 = (lane >> 4) * 4 * CB;
+  float *biasLds = reinterpret_cast<float *>(lds + a.biasByte);
+  if (t < CB * 16)
+    biasLds[t] = bias ? Load<OutT>::at(bias, t, 0) : 0.0f;
+
+  const bool vec16 = (a.rowBytes & 15) == 0;
+  for (uint32_t tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+    const uint32_t image = a.divTilesPerImage(tile);
+    const uint32_t oh0 = (tile - image * a.tilesPerImage) * a.tileRows;
+    const int32_t ih0 = int32_t(oh0 * d.strideH) - d.padH;
+    const __half *img = in + size_t(image) * d.inH * d.inW * d.inChans;
+    // Input rows ih0 .. ih0 + ldsRows - 1 into LDS, zeros for rows outside.
+    // (loads in batches of eight per thread, all on their way before the
+    // first is written to LDS)
+    if (vec16)
+      copyRows<uintx4>(a, lds, reinterpret_cast<const char *>(img), ih0, t);
+    else
+      copyRows<uint32_t>(a, lds, reinterpret_cast<const char *>(img), ih0, t);
+    if (a.cutElems) {
+      // truncated columns read as zeros: wiped once the rows are in
+      __syncthreads();
+      const uint32_t left = d.loW * d.inChans;
+      for (uint32_t i = t; i < a.ldsRows * a.cutElems; i += kThinThreads) {
+        const uint32_t row = a.divCut(i), c = i - row * a.cutElems;
+        const uint32_t elem = c < left ? c : d.hiW * d.inChans + (c - left);
+        *reinterpret_cast<__half *>(lds + row * a.pitch + a.dataOff +
+                                    elem * 2) = __float2half(0.0f);
+      }
+    }
+    __syncthreads();
+
+    const uint32_t rowsHere =
+        a.tileRows < d.outH - oh0 ? a.tileRows : d.outH - oh0;
+    const uint32_t blocks = rowsHere * a.colBlocks;
+    constexpr uint32_t kWaves = kThinThreads / 64;
+    for (uint32_t b = wave; b < blocks; b += kWaves) {
+      const uint32_t r = a.divColBlocks(b), cbk = b - r * a.colBlocks;
+      const char *base =
+          lds + r * d.strideH * a.pitch + colWord0 + cbk * blockStep;
+      // all of the block's reads, then its arithmetic
+      uint32_t x[KH][5];
+#pragma unroll
+      for (int kh = 0; kh != KH; ++kh)
+#pragma unroll
+        for (int i = 0; i != 5; ++i)
+          x[kh][i] =
+              reinterpret_cast<const uint32_t *>(base + kh * a.pitch)[i];
+      // the sums start from the bias
+      floatx4 acc[CB];
+#pragma unroll
+      for (int cb = 0; cb != CB; ++cb)
+        acc[cb] =
+            *reinterpret_cast<const floatx4 *>(biasLds + chan0 + 4 * cb);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kh = 0; kh != KH; ++kh) {
+        uintx4 u;
+        u.x = __builtin_amdgcn_perm(x[kh][1], x[kh][0], pick[0]);
+        u.y = __builtin_amdgcn_perm(x[kh][2], x[kh][1], pick[1]);
+        u.z = __builtin_amdgcn_perm(x[kh][3], x[kh][2], pick[2]);
+        u.w = __builtin_amdgcn_perm(x[kh][4], x[kh][3], pick[3]);
+        half8 xs;
+        __builtin_memcpy(&xs, &u, 16);
+#pragma unroll
+        for (int cb = 0; cb != CB; ++cb)
+          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[cb][kh], xs,
+                                                           acc[cb], 0, 0, 0);
+      }
+      const uint32_t ow = cbk * 16 + (lane & 15);
+      if (ow < d.outW) {
+        OutT *dst = out +
+                    ((size_t(image) * d.outH + oh0 + r) * d.outW + ow) *
+                        d.outChans +
+                    chan0;
+        if constexpr (sizeof(OutT) == 2 && CB % 2 == 0) {
+          // two channel blocks' results, eight neighbouring channels, as one
+          // 16-byte store
+#pragma unroll
+          for (int cb = 0; cb != CB; cb += 2) {
+            const __half2 h[4] = {
+                roundPairToHalf(acc[cb][0], acc[cb][1]),
+                roundPairToHalf(acc[cb][2], acc[cb][3]),
+                roundPairToHalf(acc[cb + 1][0], acc[cb + 1][1]),
+                roundPairToHalf(acc[cb + 1][2], acc[cb + 1][3])};
+            uintx4 u;
+            __builtin_memcpy(&u, h, 16);
+            *reinterpret_cast<uintx4 *>(dst + 4 * cb) = u;
+          }
+        } else {
+#pragma unroll
+          for (int cb = 0; cb != CB; ++cb) {
+            const float v[4] = {acc[cb][0], acc[cb][1], acc[cb][2],
+                                acc[cb][3]};
+            storeOut4(dst + 4 * cb, v);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+struct ThinShape {
+  uint32_t rowsPacked; // kernel rows the kernel is compiled for: 1, 3, 5 or 7
+  uint32_t tileRows, ldsRows, pitch, dataOff, rowBytes, colBlocks;
+  uint32_t ldsBytes;
+  bool ok;
+};
+
+uint32_t alignUp(uint32_t v, uint32_t to) { return (v + to - 1) / to * to; }
+
+ThinShape thinShape(const ThinInputDesc &d, uint32_t cus) {
+  ThinShape s{};
+  s.rowsPacked = d.kH <= 1 ? 1 : d.kH <= 3 ? 3 : d.kH <= 5 ? 5 : 7;
+  const uint32_t pixelBytes = d.inChans * 2;
+  s.rowBytes = d.inW * pixelBytes;
+  s.colBlocks = (d.outW + 15) / 16;
+  const uint32_t padLeft = d.padW > 0 ? uint32_t(d.padW) : 0;
+  s.dataOff = alignUp(padLeft * pixelBytes, 16);
+  // the last lane of the last block reads 20 bytes from (at most) here
+  const int64_t lastRead =
+      int64_t(s.dataOff) +
+      (int64_t(s.colBlocks * 16 - 1) * d.strideW - d.padW) * pixelBytes + 48 +
+      24;
+  const int64_t extent =
+      std::max<int64_t>(lastRead, int64_t(s.dataOff) + s.rowBytes);
+  if (extent > (1 << 16))
+    return s;
+  s.pitch = alignUp(uint32_t(extent), 16);
+  const uint32_t weightBytes = (d.outChans / 16) * s.rowsPacked * 1024;
+  // the largest tile of 16, 8, ... output rows that fits 64 KB and leaves
+  // three tiles to two CUs; failing that the smallest
+  uint32_t chosen = 0;
+  for (uint32_t th = 16; th != 0; th /= 2) {
+    const uint32_t rows = (th - 1) * d.strideH + s.rowsPacked;
+    if (uint64_t(rows) * s.pitch > 64 * 1024)
+      continue;
+    chosen = th;
+    if (uint64_t(d.batch) * ((d.outH + th - 1) / th) * 2 >= 3ull * cus)
+      break;
+  }
+  if (!chosen)
+    return s;
+  if (const char *e = getenv("MXK_THIN_TH")) chosen = atoi(e); // EXPERIMENT
+  s.tileRows = std::min(chosen, std::max(1u, d.outH));
+  s.ldsRows = (s.tileRows - 1) * d.strideH + s.rowsPacked;
+  // (+ 256 bytes behind them for the bias)
+  s.ldsBytes = std::max(s.ldsRows * s.pitch, weightBytes) + 256;
+  s.ok = true;
+  return s;
+}
+
+template <int CB, int KH, class OutT>
+hipError_t launchOne(const ThinArgs &a, uint32_t grid, uint32_t ldsBytes,
+                     const void *in, const void *w, const void *bias,
+                     void *out, hipStream_t stream) {
+  hipLaunchKernelGGL((thinInputKernel<CB, KH, OutT>), dim3(grid),
+                     dim3(kThinThreads), ldsBytes, stream, a,
+                     static_cast<const __half *>(in),
+                     static_cast<const __half *>(w),
+                     static_cast<const OutT *>(bias),
+                     static_cast<OutT *>(out));
+  return hipGetLastError();
+}
+
+template <int CB, class OutT>
+hipError_t launchRows(uint32_t rows, const ThinArgs &a, uint32_t grid,
+                      uint32_t ldsBytes, const void *in, const void *w,
+                      const void *bias, void *out, hipStream_t stream) {
+  switch (rows) {
+  case 1:
+    return launchOne<CB, 1, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
+  case 3:
+    return launchOne<CB, 3, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
+  case 5:
+    return launchOne<CB, 5, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
+  case 7:
+    return launchOne<CB, 7, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+template <class OutT>
+hipError_t launchBlocks(uint32_t cb, uint32_t rows, const ThinArgs &a,
+                        uint32_t grid, uint32_t ldsBytes, const void *in,
+                        const void *w, const void *bias, void *out,
+                        hipStream_t stream) {
+  switch (cb) {
+  case 1:
+    return launchRows<1, OutT>(rows, a, grid, ldsBytes, in, w, bias, out,
+                               stream);
+  case 2:
+    return launchRows<2, OutT>(rows, a, grid, ldsBytes, in, w, bias, out,
+                               stream);
+  case 3:
+    return launchRows<3, OutT>(rows, a, grid, ldsBytes, in, w, bias, out,
+                               stream);
+  case 4:
+    return launchRows<4, OutT>(rows, a, grid, ldsBytes, in, w, bias, out,
+                               stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+} // namespace
+
+bool thinInputTakes(const ThinInputDesc &d, int inType, int outType) {
+  if (inType != kHalf || (outType != kHalf && outType != kFloat))
+    return false;
+  if (d.batch == 0 || d.outH == 0 || d.outW == 0 || d.inH == 0 || d.inW == 0)
+    return false;
+  if (d.loH > d.hiH || d.hiH > d.inH || d.loW > d.hiW || d.hiW > d.inW)
+    return false;
+  if (d.inChans == 0 || d.inChans > 4 || d.kW * d.inChans > 32 ||
+      d.kH == 0 || d.kH > 7 || d.kH * d.kW < 2)
+    return false;
+  if (d.outChans % 16 != 0 || d.outChans > 64)
+    return false;
+  // rows are copied in dwords
+  if ((d.inW * d.inChans) % 2 != 0)
+    return false;
+  if (d.strideH == 0 || d.strideW == 0 || d.strideW > 64 ||
+      d.padW > 4096 || d.padW < -4096 || d.padH > (1 << 20) ||
+      d.padH < -(1 << 20))
+    return false;
+  // every window inside the (padded) rows kept in LDS: nothing is read
+  // left of the row's start
+  if (d.padW < 0)
+    return false;
+  if (uint64_t(d.batch) * d.outH * d.outW * d.outChans >= (1ull << 32) ||
+      uint64_t(d.batch) * d.inH * d.inW * d.inChans >= (1ull << 32))
+    return false;
+  return thinShape(d, 256).ok;
+}
+
+uint64_t thinInputPackedElems(const ThinInputDesc &d) {
+  const uint32_t rows = d.kH <= 1 ? 1 : d.kH <= 3 ? 3 : d.kH <= 5 ? 5 : 7;
+  return uint64_t(d.outChans / 16) * rows * 512;
+}
+
+ThinInputLaunch thinInputLaunchShape(const ThinInputDesc &d, uint32_t cus) {
+  const ThinShape s = thinShape(d, cus);
+  ThinInputLaunch l{};
+  l.tileRows = s.tileRows;
+  l.ldsBytes = s.ldsBytes;
+  const uint64_t tiles =
+      uint64_t(d.batch) * ((d.outH + s.tileRows - 1) / std::max(1u, s.tileRows));
+  // (two workgroups to a CU: what the registers of the largest variant -
+  // 64 output channels, 7 kernel rows - allow)
+  l.workgroups = std::min<uint64_t>(tiles, uint64_t(cus) * 2);
+  l.tiles = tiles;
+  return l;
+}
+
+hipError_t launchPackThinInputWeights(const ThinInputDesc &d, const void *src,
+                                      void *dst, hipStream_t stream) {
+  const uint32_t total = uint32_t(thinInputPackedElems(d));
+  const uint32_t rows = total / 512 / (d.outChans / 16);
+  hipLaunchKernelGGL(packThinWeightsKernel, dim3((total + 255) / 256),
+                     dim3(256), 0, stream, static_cast<const __half *>(src),
+                     static_cast<__half *>(dst), d, rows, total);
+  return hipGetLastError();
+}
+
+hipError_t launchThinInput(const ThinInputDesc &d, int inType, int outType,
+                           const void *in, const void *weightsPacked,
+                           const void *bias, void *out, hipStream_t stream) {
+  if (!thinInputTakes(d, inType, outType))
+    return hipErrorInvalidValue;
+  const ThinShape s = thinShape(d, 256);
+  const ThinInputLaunch l = thinInputLaunchShape(d, 256);
+  ThinArgs a{};
+  a.d = d;
+  a.tileRows = s.tileRows, a.ldsRows = s.ldsRows, a.pitch = s.pitch;
+  a.dataOff = s.dataOff, a.rowBytes = s.rowBytes;
+  a.tilesPerImage = (d.outH + s.tileRows - 1) / s.tileRows;
+  a.tiles = uint32_t(l.tiles);
+  a.colBlocks = s.colBlocks;
+  a.divTilesPerImage = makeFastDiv(a.tilesPerImage);
+  a.divColBlocks = makeFastDiv(a.colBlocks);
+  a.divRowUnits =
+      makeFastDiv((s.rowBytes & 15) == 0 ? s.rowBytes / 16 : s.rowBytes / 4);
+  a.divBorder = makeFastDiv((s.pitch - s.rowBytes) / 4);
+  a.biasByte = s.ldsBytes - 256;
+  a.cutElems = (d.loW + (d.inW - d.hiW)) * d.inChans;
+  a.divCut = makeFastDiv(a.cutElems);
+  if (l.tiles >= (1ull << 31))
+    return hipErrorInvalidConfiguration;
+  const uint32_t grid = uint32_t(l.workgroups);
+  if (outType == kHalf)
+    return launchBlocks<__half>(d.outChans / 16, s.rowsPacked, a, grid,
+                                s.ldsBytes, in, weightsPacked, bias, out,
+                                stream);
+  return launchBlocks<float>(d.outChans / 16, s.rowsPacked, a, grid,
+                             s.ldsBytes, in, weightsPacked, bias, out, stream);
+}
+
+} // namespace mxk

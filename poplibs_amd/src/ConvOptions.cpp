@@ -211,6 +211,11 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       if (v > 1)
         throw invalid_option("'" + sub + "': Must be 0 or 1");
       pc.pointwise = int(v);
+    } else if (m.first == "thinInput") {
+      const unsigned v = requireUnsigned(sub, m.second);
+      if (v > 1)
+        throw invalid_option("'" + sub + "': Must be 0 or 1");
+      pc.thinInput = int(v);
     } else if (m.first == "weightDeltas") {
       const unsigned v = requireUnsigned(sub, m.second);
       if (v > 1)

@@ -60,6 +60,10 @@ struct PlanConstraints {
   /// planner's choice, 0 never, 1 required (an error where it cannot take the
   /// convolution).
   int pointwise = -1;
+  /// The matrix-core kernel for inputs of 1 to 4 channels (a kernel row's
+  /// pixels as one k-step, no padded copy of the input): -1 planner's choice
+  /// (never with "kernel" or a tile named), 0 never, 1 required.
+  int thinInput = -1;
   /// A weight update pass's deltas: -1 planner's choice, 0 through the pass's
   /// own convolution (batch and channels exchanged), 1 by the kernel that
   /// reads the layer's own tensors (an error where none takes the layer).

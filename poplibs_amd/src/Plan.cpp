@@ -718,10 +718,57 @@ mxconv_plan makePlanWith(const ConvParams &params,
   } else {
     reason = "generic direct kernel (" + igemmWhyNot + ")";
   }
+  // An input of 1 to 4 channels (an image, a waveform): the matrix-core
+  // kernel that takes the kW * Ci neighbouring elements under a kernel row as
+  // one k-step instead of padding the channels to a whole vector - no copy
+  // of the input, K = kH * 32 instead of kH * kW * 8 (N = 32, 224 x 224,
+  // 7 x 7 stride 2, 3 -> 64: 64 -> 17 us).
+  {
+    mxk::ThinInputDesc &t = plan.thinInput;
+    t.batch = uint32_t(s.batch), t.inChans = uint32_t(ci);
+    t.outChans = uint32_t(co);
+    t.inH = s.inH, t.inW = s.inW, t.outH = s.outH, t.outW = s.outW;
+    t.kH = s.kH, t.kW = s.kW, t.padH = s.padH, t.padW = s.padW;
+    t.strideH = s.strideH, t.strideW = s.strideW;
+    t.loH = s.loH, t.hiH = s.hiH, t.loW = s.loW, t.hiW = s.hiW;
+    const bool shapeOk =
+        !plan.zeroConv && s.ok && !s.hasDepth() && !s.inputDilated() &&
+        !s.kernelSelected && !s.outputPadded() && s.dilH == 1 &&
+        s.dilW == 1 && p.numConvGroups == 1 && s.batch < (1ull << 31) &&
+        mxk::thinInputTakes(t,
+                            halfIn    ? mxk::kHalf
+                            : floatIn ? mxk::kFloat
+                                      : mxk::kQuarter,
+                            params.outputType == poplar::HALF ? mxk::kHalf
+                                                              : mxk::kFloat);
+    const bool unconstrained =
+        pc.kernel.empty() && !pc.blockM && !pc.blockN && !pc.blockK &&
+        !pc.splitK && !pc.stages && pc.patch < 1 && pc.pointwise != 1 &&
+        (pc.method == Method::ANY || pc.method == Method::AMP);
+    if (pc.thinInput == 1 && !shapeOk)
+      throw poplar::invalid_option(
+          "planConstraints gfx950 thinInput: that kernel takes 2-D "
+          "convolutions of half inputs with 1 to 4 channels in one group "
+          "(kW * Ci <= 32, at most 7 kernel rows; 16, 32, 48 or 64 output "
+          "channels; nothing dilated or flipped, no kernel truncation or "
+          "padding, no output padding, no negative padding of the columns)");
+    if (shapeOk && pc.thinInput != 0 &&
+        (pc.thinInput == 1 || (unconstrained && chosen == Kernel::IGEMM))) {
+      plan.thinInputOn = true;
+      if (chosen != Kernel::IGEMM)
+        chosen = Kernel::IGEMM, reason = "forced by planConstraints";
+      else
+        reason = "few input channels: a kernel row's pixels as one k-step on "
+                 "the matrix cores";
+    }
+  }
   plan.kernel = chosen;
   plan.reason = reason;
 
-  if (chosen == Kernel::IGEMM) {
+  if (plan.thinInputOn) {
+    plan.weightPackedElems = mxk::thinInputPackedElems(plan.thinInput);
+    plan.workspaceBytes = 0;
+  } else if (chosen == Kernel::IGEMM) {
     mxk::IgemmDesc &g = plan.igemm;
     g.batch = uint32_t(s.batch);
     g.groups = uint32_t(p.numConvGroups);
@@ -1293,7 +1340,9 @@ std::string mxconv_plan::constraintsJson() const {
     break;
   case Kernel::IGEMM:
     os << "\"kernel\": \"igemm\"";
-    if (pointwiseOn) {
+    if (thinInputOn) {
+      os << ", \"thinInput\": 1";
+    } else if (pointwiseOn) {
       os << ", \"pointwise\": 1, \"chanTiles\": "
          << mxk::pointwiseLaunchShape(pointwise, gfx950::numCUs).chansPerWorkgroup / 64;
     } else if (igemm.patch) {
@@ -1383,6 +1432,25 @@ mxconv_plan::DetailedEstimate mxconv_plan::detailedEstimate() const {
       spread(e, mxk::depthwiseRowsLaunchShape(depthwise).workgroups, 1);
     break;
   case Kernel::IGEMM: {
+    if (thinInputOn) {
+      // its tensors' bytes at streaming rate (to be calibrated: the padded
+      // MFMA work of kH k-steps of 32 per 16 pixels and 16 channels at half
+      // the matrix cores' rate, whichever is longer)
+      const mxk::ThinInputLaunch l =
+          mxk::thinInputLaunchShape(thinInput, gfx950::numCUs);
+      const double flops = 2.0 * thinInput.batch * thinInput.outH *
+                           ((thinInput.outW + 15) / 16 * 16) *
+                           thinInput.outChans * 32.0 *
+                           (thinInput.kH <= 1   ? 1
+                            : thinInput.kH <= 3 ? 3
+                            : thinInput.kH <= 5 ? 5
+                                                : 7);
+      e.computeUs = std::max(
+          streamed(inputBytes() + outputBytes() + weightPackedBytes()),
+          poplin::kLaunchUs + flops / 1.0e9);
+      spread(e, l.workgroups, 1);
+      break;
+    }
     if (pointwiseOn) {
       e.computeUs =
           streamed(inputBytes() + outputBytes() + weightPackedBytes());
@@ -1462,6 +1530,7 @@ std::string mxconv_plan::describe() const {
                                                : "fp16")
        << " operands, fp32 accumulate)"
        << (pointwiseOn ? ", pointwise streaming variant" : "")
+       << (thinInputOn ? ", kernel rows as k-steps" : "")
        << (igemm.patch ? ", input patch resident in LDS" : "");
     break;
   case Kernel::DEPTHWISE:
@@ -1490,7 +1559,27 @@ std::string mxconv_plan::describe() const {
        << canonical.numConvGroups * wuGroupsPerGroup
        << " groups taken as one; the diagonal blocks of the fused layer's "
           "deltas are handed back)\n";
-  if (kernel == Kernel::IGEMM) {
+  if (kernel == Kernel::IGEMM && thinInputOn) {
+    const auto &t = thinInput;
+    const mxk::ThinInputLaunch l =
+        mxk::thinInputLaunchShape(t, gfx950::numCUs);
+    const unsigned rows = t.kH <= 1 ? 1 : t.kH <= 3 ? 3 : t.kH <= 5 ? 5 : 7;
+    os << "        gemm M x N x K             "
+       << std::size_t(t.batch) * t.outH * t.outW << " x " << t.outChans
+       << " x " << rows * 32 << " (a kernel row's " << t.kW << " x "
+       << t.inChans << " = " << t.kW * t.inChans
+       << " neighbouring elements as one k-step of 32; " << t.kH
+       << " kernel rows run as " << rows << ")\n";
+    os << "        block M x N x K            16 x " << t.outChans
+       << " x 32 per wave; tiles of " << l.tileRows
+       << " output rows of one image, their input rows in " << l.ldsBytes
+       << " bytes of LDS\n";
+    os << "        workgroups                 " << l.workgroups
+       << " persistent (4 waves) taking " << l.tiles << " tiles in turn on "
+       << gfx950::numCUs << " CUs\n";
+    os << "        packed weights             [" << t.outChans / 16
+       << " blocks of 16][" << rows << " kernel rows][64 lanes][8]\n";
+  } else if (kernel == Kernel::IGEMM) {
     const auto &g = igemm;
     const std::size_t m = std::size_t(g.batch) * g.outD * g.outH * g.outW;
     const std::size_t k =

@@ -49,6 +49,10 @@ struct mxconv_plan {
   // weights then have its layout.
   bool pointwiseOn = false;
   mxk::PointwiseDesc pointwise{};
+  // ... or, for an input of 1 to 4 channels, the kernel that takes a kernel
+  // row's pixels as one k-step
+  bool thinInputOn = false;
+  mxk::ThinInputDesc thinInput{};
   mxk::DepthwiseDesc depthwise{}; // valid when kernel == DEPTHWISE
   // These parameters are the weight update pass of a depthwise layer: the
   // descriptor of that layer's FORWARD convolution, for the kernel that

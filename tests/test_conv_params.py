@@ -465,11 +465,35 @@ def test_planner_choices():
     # channel counts that are no whole 16-byte vector are padded for the
     # matrix cores (a zero-filled copy in the workspace) ...
     few = pa.Plan(make_params(pa.HALF, batch=2, field=(32, 32), kernel=(3, 3),
-                              ci=3, co=64))
+                              ci=5, co=64))
     assert "implicit GEMM" in few.describe()
-    assert "input channels padded      3 -> 8" in few.describe()
+    assert "input channels padded      5 -> 8" in few.describe()
     assert few.buffer_bytes(4) == 2 * 32 * 32 * 8 * 2
-    assert few.buffer_bytes(0) == 2 * 32 * 32 * 3 * 2   # the caller's input
+    assert few.buffer_bytes(0) == 2 * 32 * 32 * 5 * 2   # the caller's input
+    # ... unless there are at most 4 of them in one group: then a kernel
+    # row's pixels, neighbours in a channels-last image, make one k-step, and
+    # the input is read as it is
+    thin = pa.Plan(make_params(pa.HALF, batch=2, field=(32, 32),
+                               kernel=(3, 3), ci=3, co=64))
+    assert "kernel rows as k-steps" in thin.describe()
+    assert "a kernel row's 3 x 3 = 9 neighbouring elements" in thin.describe()
+    assert thin.buffer_bytes(4) == 0
+    assert thin.buffer_bytes(1) == 4 * 3 * 64 * 8 * 2
+    off = {"planConstraints": '{"gfx950": {"thinInput": 0}}'}
+    assert "input channels padded      3 -> 8" in pa.Plan(
+        make_params(pa.HALF, batch=2, field=(32, 32), kernel=(3, 3), ci=3,
+                    co=64), off).describe()
+    # (48 output channels: three blocks of 16; 80: not this kernel's)
+    assert "kernel rows as k-steps" in pa.Plan(make_params(
+        pa.HALF, batch=2, field=(32, 32), kernel=(5, 5), ci=4,
+        co=48)).describe()
+    assert "kernel rows as k-steps" not in pa.Plan(make_params(
+        pa.HALF, batch=2, field=(32, 32), kernel=(5, 5), ci=4,
+        co=80)).describe()
+    with pytest.raises(MxconvError, match="thinInput"):
+        pa.Plan(make_params(pa.HALF, batch=2, field=(32, 32), kernel=(5, 5),
+                            ci=4, co=80),
+                {"planConstraints": '{"gfx950": {"thinInput": 1}}'})
     # ... except when there is too little work to pay for the copy
     assert _kernel_of(make_params(pa.HALF, field=(8, 8), kernel=(3, 3), ci=4,
                                   co=8)) == "generic direct"
@@ -585,9 +609,9 @@ def test_plan_detailed_costs():
     # the second kernel (4.5 us) and the partial tiles out and in at 6.4 TB/s
     assert d["reduction"][0] == round(
         (4.5 + 2 * d["reduction"][1] / 6.4e6) * 2100)
-    # three input channels: copied into whole vectors first
+    # six input channels: copied into whole vectors first
     stem = pa.Plan(make_params(pa.HALF, batch=8, field=(56, 56),
-                               kernel=(3, 3), ci=3, co=64, pad=1))
+                               kernel=(3, 3), ci=6, co=64, pad=1))
     assert "generic direct" not in stem.describe()
     d = parts(stem)
     assert d["rearrangement"][0] > 2.0 * 2100  # at least a launch

@@ -315,8 +315,8 @@ int main(int argc, char **argv) {
       CHECK(split.reduction.cycles > 0);
       CHECK(split.reduction.memory == whole.memory);
     }
-    // three input channels are copied into whole vectors first
-    const ConvParams stem = conv(poplar::HALF, 8, 56, 3, 3, 64);
+    // six input channels are copied into whole vectors first
+    const ConvParams stem = conv(poplar::HALF, 8, 56, 3, 6, 64);
     const DetailedPlanCosts padded =
         poplin::internal::reportDetailedPlanEstimatedCosts(stem, fwd);
     if (planText(stem, fwd, nullptr).find("generic direct") ==
