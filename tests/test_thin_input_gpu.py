@@ -111,3 +111,62 @@ def test_thin_input_is_the_planners_choice_for_a_first_layer():
     named = {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'}
     assert "input channels padded      3 -> 8" in pa.Plan(stem,
                                                           named).describe()
+
+
+def _random_thin_case(r):
+    """A random layer within what the kernel takes (or close to it: what the
+    canonical form then moves outside - padded outputs, say - is skipped)."""
+    ci = r.choice([1, 2, 3, 3, 4])
+    kw = r.randint(1, 32 // ci)
+    kh = r.randint(1, 7)
+    if kh * kw < 2:
+        kh = 2
+    one_d = r.random() < 0.15
+    if one_d:
+        kh = None
+    width = r.randint(kw, kw + 40)
+    if (width * ci) % 2:
+        width += 1
+    field = (width,) if one_d else (r.randint(kh, kh + 24), width)
+    kernel = (kw,) if one_d else (kh, kw)
+    n = len(field)
+    kw_args = dict(
+        batch=r.randint(1, 5), field=field, kernel=kernel, ci=ci,
+        co=r.choice([16, 32, 48, 64]),
+        stride=[r.choice([1, 1, 2, 2, 3, 4]) for _ in range(n)],
+        # (no window wholly in the border: that is output padding)
+        padLower=[r.randint(0, min(4, k - 1)) for k in kernel],
+        padUpper=[r.randint(0, min(4, k - 1)) for k in kernel])
+    if r.random() < 0.2:
+        kw_args["itl"] = [r.randint(0, 1) for _ in range(n)]
+        kw_args["itu"] = [r.randint(0, 1) for _ in range(n)]
+    return kw_args
+
+
+def test_thin_input_random_params(oracle):
+    import random
+    from gpu_helpers import quantize, run_conv
+    from poplibs_amd.capi import MxconvError
+    r = random.Random(44)
+    ran = 0
+    for case in range(260):
+        kw = _random_thin_case(r)
+        out_type = r.choice([pa.HALF, pa.FLOAT])
+        try:
+            p = make_params(pa.HALF, out_type, **kw)
+            p.validate()
+            plan = pa.Plan(p, FORCED)
+        except MxconvError:
+            continue  # (not a layer, or not this kernel's after canonicalize)
+        print("case", case, kw, flush=True)
+        acts, weights, biases = random_data(p, 100 + case, "normal")
+        aq, ad = quantize(acts, pa.HALF)
+        wq, wd = quantize(weights * 0.2, pa.HALF)
+        bq, bd = quantize(biases, out_type)
+        got = run_conv(p, aq, wq, bq, plan=plan)
+        assert THIN in plan.describe()
+        want = oracle.convolution(p, ad, wd, bd, threads=8)
+        tol = 1e-3 if out_type == pa.HALF else 1e-5
+        assert rel_l2(got, want) <= tol, (case, kw, rel_l2(got, want))
+        ran += 1
+    assert ran >= 150, ran
