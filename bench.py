@@ -72,6 +72,13 @@ def _workloads(pa):
                           1, 1, 1),
             dtype="fp16", bound="mfma", relu=False,
             w_std=(2 / (9 * 256)) ** .5),
+        # ... and a first layer: three input channels, read as they are.
+        "first_layer": dict(
+            name="first layer (not a benchmark configuration): 7x7 conv "
+                 "stride 2 pad 3 N=32 224x224 Cin=3 Cout=64, fp16",
+            params=params(pa.HALF, pa.HALF, 32, (224, 224), (7, 7), 3, 64, 1,
+                          2, 3),
+            dtype="fp16", bound="hbm", relu=False, w_std=(2 / 147) ** .5),
     }
 
 

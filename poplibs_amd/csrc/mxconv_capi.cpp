@@ -605,7 +605,8 @@ size_t ownTensorsWorkspaceBytes(const mxconv_plan *plan);
 /// the layer's own tensors keeps its partial sums and deltas there, not the
 /// intermediates of the pass's convolution.)
 size_t estimatedWorkspaceBytes(const mxconv_plan *plan) {
-  return plan->denseWeightUpdate || plan->depthwiseWeightUpdate
+  return plan->denseWeightUpdate || plan->depthwiseWeightUpdate ||
+                 plan->weightUpdateProduct
              ? ownTensorsWorkspaceBytes(plan)
              : plan->workspaceBytes;
 }
@@ -1414,6 +1415,16 @@ WuWorkspace wuWorkspace(const mxconv_plan *plan) {
     w.total = at;
     return w;
   }
+  if (const mxconv_plan *product = plan->weightUpdateProduct.get()) {
+    // transposed deltas [Co][batch], the activations packed as the
+    // product's right-hand side, the product's own workspace
+    w.input = take(product->inputBytes());
+    w.weightsPacked = take(product->weightPackedBytes());
+    w.planWorkspace = take(product->workspaceBytes);
+    w.deltas = take(wuResultBytes(plan));
+    w.total = at;
+    return w;
+  }
   w.input = take(plan->inputBytes());
   w.weightsExternal = take(plan->weightBytes());
   w.weightsPacked = take(plan->weightPackedBytes());
@@ -1495,6 +1506,23 @@ mxconv_status fusedWeightDeltas(const mxconv_plan *plan, const void *zDeltas,
                                       deltasOut, s),
                      "matrix-core weight deltas");
   mxconv_status st;
+  if (const mxconv_plan *product = plan->weightUpdateProduct.get()) {
+    // No spatial extent: deltas[co][ci] = sum over the batch of
+    // dZ[b][co] * x[b][ci] - transpose(dZ) [Co][B] times x [B][Ci], and the
+    // result is in weight order as it is.
+    st = hipStatus(mxk::launchSwapBatchChans(zDeltas, ws + w.input,
+                                             uint32_t(B), 1, 1, uint32_t(Co),
+                                             B, B, B, inBytes, s),
+                   "delta rearrangement");
+    if (st != MXCONV_OK)
+      return st;
+    st = mxconv_matmul_pack_rhs(product, acts, ws + w.weightsPacked, stream);
+    if (st != MXCONV_OK)
+      return st;
+    return forward(product, ws + w.input, ws + w.weightsPacked, nullptr,
+                   deltasOut, ws + w.planWorkspace, product->workspaceBytes,
+                   mxk::QuarterInfo{}, stream);
+  }
   // activations [B][X][G][Ci] -> the pass's input [Ci][X][G][B]
   const mxk::SwapBatchChans actsSwap{
       acts,        ws + w.input, uint32_t(B), uint32_t(X), uint32_t(G),
@@ -1622,6 +1650,41 @@ mxconv_status mxconv_weight_update_plan_create(const mxconv_params *fwd,
     *plan = new mxconv_plan(poplin::makePlan(
         poplin::getWeightUpdateParams(poplin::ConvParams::fromC(*fwd)),
         options));
+    // A layer without spatial extent (every field and kernel dimension 1,
+    // one group): its deltas as one matrix product [Co] x [batch] x [Ci] on
+    // the transposed deltas - where nothing in the constraints names a
+    // kernel or tile for the pass's own convolution.
+    mxconv_plan &made = **plan;
+    const auto &pc = options.planConstraints;
+    const auto &wp = made.params; // batch = Ci, input channels = the batch
+    const bool shapeOk =
+        isMatMulPlan(&made) && wp.numConvGroups == 1 && !made.zeroConv &&
+        made.outputElems != 0 && made.inputElems != 0 &&
+        made.wuGroupsPerGroup == 1 && !made.depthwiseWeightUpdate &&
+        wp.inputType != poplar::QUARTER;
+    const bool unconstrained =
+        pc.weightDeltas == -1 && pc.kernel.empty() &&
+        pc.method == poplin::PlanConstraints::Method::ANY && !pc.blockM &&
+        !pc.blockN && !pc.blockK && !pc.splitK && !pc.stages &&
+        pc.patch < 0 && pc.pointwise < 0;
+    if (pc.weightDeltas == 2 && !shapeOk)
+      throw poplar::invalid_option(
+          "planConstraints gfx950 weightDeltas 2: the deltas are one matrix "
+          "product only for a layer without spatial extent (every field and "
+          "kernel dimension 1, nothing padded or strided) and one group, of "
+          "half or float tensors");
+    if (shapeOk && (pc.weightDeltas == 2 || unconstrained)) {
+      poplin::ConvOptions productOptions = options;
+      productOptions.pass = poplin::Pass::NONE_MATMUL;
+      productOptions.planConstraints = poplin::PlanConstraints{};
+      made.weightUpdateProduct = std::make_shared<const mxconv_plan>(
+          poplin::makePlan(
+              matMulParams(wp.inputType.id(), wp.outputType.id(), 1,
+                           wp.outputChannelsPerConvGroup,
+                           wp.inputChannelsPerConvGroup, wp.batchSize),
+              productOptions));
+      made.denseWeightUpdate = false;
+    }
     writeConstraintsFile(**plan, options);
     return MXCONV_OK;
   });

@@ -218,8 +218,8 @@ void checkGfx950(const std::string &path, const Value &v, PlanConstraints &pc) {
       pc.thinInput = int(v);
     } else if (m.first == "weightDeltas") {
       const unsigned v = requireUnsigned(sub, m.second);
-      if (v > 1)
-        throw invalid_option("'" + sub + "': Must be 0 or 1");
+      if (v > 2)
+        throw invalid_option("'" + sub + "': Must be 0, 1 or 2");
       pc.weightDeltas = int(v);
     } else if (m.first == "chanTiles") {
       pc.chanTiles = requireUnsigned(sub, m.second);

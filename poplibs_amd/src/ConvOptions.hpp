@@ -66,7 +66,9 @@ struct PlanConstraints {
   int thinInput = -1;
   /// A weight update pass's deltas: -1 planner's choice, 0 through the pass's
   /// own convolution (batch and channels exchanged), 1 by the kernel that
-  /// reads the layer's own tensors (an error where none takes the layer).
+  /// reads the layer's own tensors (an error where none takes the layer), 2
+  /// as one matrix product on the transposed deltas (a layer without spatial
+  /// extent; an error for any other).
   int weightDeltas = -1;
   std::string text; // the JSON as given, kept for reporting and cache keys
 };

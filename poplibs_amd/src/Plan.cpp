@@ -1358,7 +1358,9 @@ std::string mxconv_plan::constraintsJson() const {
   }
   if (madeForWeightUpdate) {
     os << ", \"weightDeltas\": "
-       << (denseWeightUpdate || depthwiseWeightUpdate ? 1 : 0);
+       << (weightUpdateProduct                           ? 2
+           : denseWeightUpdate || depthwiseWeightUpdate ? 1
+                                                        : 0);
     if (depthwiseWeightUpdate && kernel != Kernel::DEPTHWISE)
       os << ", \"rowRing\": " << (depthwiseForward.dense3x3 == 2 ? 1 : 0);
   }
@@ -1393,6 +1395,19 @@ mxconv_plan::DetailedEstimate mxconv_plan::detailedEstimate() const {
   // of the chunks' 16.8 MB of fp32 tiles 5.2); depthwise rows + the sum of
   // the workgroups' tiles (4.5 us) behind one pass over both tensors (N = 32,
   // 112 x 112, 96 channels, stride 2: 20.4 us).
+  if (weightUpdateProduct) {
+    // the product as planned, behind the deltas' transpose and the packing
+    // of the activations (each read once and written once)
+    DetailedEstimate e = weightUpdateProduct->detailedEstimate();
+    if (e.known) {
+      e.rearrangementBytes += weightUpdateProduct->inputBytes() +
+                              weightUpdateProduct->weightPackedBytes();
+      e.rearrangementUs +=
+          streamed(2 * weightUpdateProduct->inputBytes()) +
+          streamed(2 * weightUpdateProduct->weightPackedBytes());
+    }
+    return e;
+  }
   if (denseWeightUpdate) {
     const auto &f = denseForward;
     const double flops = 2.0 * f.batch * f.outH * f.outW * f.groups * f.ci *
@@ -1720,6 +1735,20 @@ std::string mxconv_plan::describe() const {
        << tiles << " tap x channel tiles x " << chunks << " chunks of "
        << f.chunkPixels << " pixels = " << tiles * chunks
        << " workgroups, fp32 partial tiles summed in order\n";
+  }
+  if (weightUpdateProduct) {
+    const auto &q = weightUpdateProduct->params;
+    std::string tiling;
+    for (const auto &c : weightUpdateProduct->candidates)
+      if (c.chosen)
+        tiling = c.name;
+    os << "        as a weight update pass    one matrix product, "
+          "transpose(deltas) x activations: "
+       << q.batchSize << " x " << q.inputChannelsPerConvGroup << " x "
+       << q.outputChannelsPerConvGroup
+       << " (output channels x batch x input channels), its result in "
+          "weight order as it is"
+       << (tiling.empty() ? "" : "; " + tiling) << "\n";
   }
   os << "        workspaceBytes             " << workspaceBytes << "\n";
   return os.str();

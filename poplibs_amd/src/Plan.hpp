@@ -10,6 +10,7 @@
 #include "kernels.hpp"
 #include "poplin/ConvParams.hpp"
 #include <cstddef>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -63,6 +64,11 @@ struct mxconv_plan {
   // options, `pass` TRAINING_WU or FC_TRAINING_WU - what
   // mxconv_weight_update_plan_create sets.)
   bool madeForWeightUpdate = false;
+  // ... of a layer without spatial extent (a fully connected layer): the
+  // deltas are one matrix product, transpose(dZ) x X, whose result is in
+  // weight order as it is - the plan of that product ([Co] x [batch] x [Ci],
+  // made by mxconv_weight_update_plan_create).
+  std::shared_ptr<const mxconv_plan> weightUpdateProduct;
   bool depthwiseWeightUpdate = false;
   mxk::DepthwiseDesc depthwiseForward{};
   // ... or of a dense layer (any stride): the matrix-core kernel that reads

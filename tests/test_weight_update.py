@@ -575,6 +575,83 @@ def test_weight_update_applies_scaled_deltas(oracle):
     assert e.value.status == pa.Status.INVALID_PARAMS
 
 
+PRODUCT_WU = "one matrix product, transpose(deltas) x activations"
+FC_CASES = [
+    # (batch, input channels, output channels, field)
+    (70, 96, 64, ()),
+    (5, 20, 24, ()),          # channel counts that are no whole vector
+    (256, 512, 136, (1,)),
+    (33, 8, 1000, (1, 1)),
+    (1, 64, 32, ()),          # one sample
+    (300, 3, 7, ()),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,ot", [(pa.HALF, pa.HALF), (pa.HALF, pa.FLOAT),
+                                   (pa.FLOAT, pa.FLOAT)])
+@pytest.mark.parametrize("batch,ci,co,field", FC_CASES)
+def test_weight_deltas_of_a_layer_without_spatial_extent(oracle, batch, ci,
+                                                         co, field, dt, ot):
+    # deltas[co][ci] = sum over the batch of dZ[b][co] x[b][ci]: one matrix
+    # product whose result is in weight order as it is
+    from gpu_helpers import quantize
+    p = make_params(dt, ot, batch=batch, field=field, kernel=(1,) * len(field),
+                    ci=ci, co=co)
+    rng = np.random.default_rng(31)
+    xq, xd = quantize(rng.standard_normal((batch, ci, *field)), dt)
+    dq, dd = quantize(rng.standard_normal((batch, co, *field)) * 0.1, dt)
+    got, plan = run_weight_update(p, xq, dq)
+    assert PRODUCT_WU in plan.describe(), plan.describe()
+    want = oracle.weight_deltas(p, xd, dd, threads=8)
+    assert got.shape == want.shape
+    tol = 1e-3 if ot == pa.HALF else 1e-5
+    assert rel_l2(got, want) <= tol, (rel_l2(got, want), plan.describe())
+    # the pass's own convolution, by name, gives the same deltas
+    own, plan0 = run_weight_update(
+        p, xq, dq, {"planConstraints": '{"gfx950": {"weightDeltas": 0}}'})
+    assert PRODUCT_WU not in plan0.describe()
+    assert rel_l2(own, want) <= tol
+
+
+@pytest.mark.gpu
+def test_weight_update_of_a_fully_connected_layer(oracle):
+    from gpu_helpers import quantize
+    p = make_params(pa.HALF, pa.HALF, batch=48, field=(), kernel=(), ci=40,
+                    co=72)
+    rng = np.random.default_rng(32)
+    xq, xd = quantize(rng.standard_normal((48, 40)), pa.HALF)
+    dq, dd = quantize(rng.standard_normal((48, 72)) * 0.1, pa.HALF)
+    wq, wd = quantize(rng.standard_normal((1, 72, 40)), pa.HALF)
+    got, plan = run_weight_update(p, xq, dq, weights_q=wq, scale=-0.25)
+    assert PRODUCT_WU in plan.describe()
+    want, _ = oracle.weight_update(p, 0.25, xd, dd, wd, np.zeros(72))
+    assert rel_l2(got, want) <= 2e-3, rel_l2(got, want)
+
+
+def test_weight_deltas_as_a_product_plan_choice():
+    fc = make_params(pa.HALF, batch=256, field=(), kernel=(), ci=1024, co=512)
+    assert PRODUCT_WU in pa.WeightUpdatePlan(fc).describe()
+    by_name = {"planConstraints": '{"gfx950": {"weightDeltas": 2}}'}
+    assert PRODUCT_WU in pa.WeightUpdatePlan(fc, by_name).describe()
+    # its workspace: transposed deltas, packed activations, the deltas of an
+    # update
+    assert pa.WeightUpdatePlan(fc).workspace_bytes() >= \
+        2 * (256 * 512 + 256 * 1024 + 512 * 1024)
+    # a layer with a field is not one product over the batch ...
+    conv = make_params(pa.HALF, batch=8, field=(6, 6), kernel=(1, 1), ci=64,
+                       co=64)
+    assert PRODUCT_WU not in pa.WeightUpdatePlan(conv).describe()
+    with pytest.raises(pa.MxconvError, match="weightDeltas 2"):
+        pa.WeightUpdatePlan(conv, by_name)
+    # ... nor are groups, and a named kernel keeps the pass's own convolution
+    grouped = make_params(pa.HALF, batch=64, field=(), kernel=(), ci=32,
+                          co=32, groups=4)
+    assert PRODUCT_WU not in pa.WeightUpdatePlan(grouped).describe()
+    named = {"planConstraints": '{"gfx950": {"kernel": "igemm"}}'}
+    assert PRODUCT_WU not in pa.WeightUpdatePlan(fc, named).describe()
+
+
 @pytest.mark.gpu
 def test_weight_update_random_params_on_gpu(oracle):
     from gpu_helpers import quantize
