@@ -830,10 +830,13 @@ def test_igemm_pads_odd_channel_counts(oracle, in_type, kw):
         wq, wd = quantize(weights * 0.1, in_type)
         bq, bd = quantize(biases, out_type)
         # (each group by itself: taken as one, the two groups of six fp32
-        # channels are whole vectors and need no padding)
-        got, plan = run_conv(p, aq, wq, bq,
-                             {"planConstraints": '{"convGroupsPerGroup": 1}'},
-                             return_plan=True)
+        # channels are whole vectors and need no padding; and not the kernel
+        # that reads up to four half channels as they are)
+        got, plan = run_conv(
+            p, aq, wq, bq,
+            {"planConstraints":
+             '{"convGroupsPerGroup": 1, "gfx950": {"thinInput": 0}}'},
+            return_plan=True)
         want = oracle.convolution(p, ad, wd, bd, threads=8)
     assert "input channels padded" in plan.describe(), plan.describe()
     assert rel_l2(got, want) <= (2e-6 if in_type == pa.FLOAT else 1e-3)

@@ -83,14 +83,14 @@ def test_static_scratch_matches_fwd_twice_second_smaller():
 
 
 def test_static_scratch_padded_channels_float_out():
-    # 3 input channels: a zero-filled copy [pixels][8] goes to the scratch
+    # 5 input channels: a zero-filled copy [pixels][8] goes to the scratch
     p = make_params(pa.HALF, pa.FLOAT, batch=2, field=(32, 32), kernel=(7, 7),
-                    ci=3, co=64, pad=3, stride=2)
+                    ci=5, co=64, pad=3, stride=2)
     assert "input channels padded" in pa.Plan(p).describe()
     _both(p, 34, setup=True)  # (first call on the device if run by itself)
     _both(p, 34)
     _both(make_params(pa.HALF, pa.FLOAT, batch=1, field=(32, 28),
-                      kernel=(7, 7), ci=3, co=64, pad=3, stride=2), 35)
+                      kernel=(7, 7), ci=5, co=64, pad=3, stride=2), 35)
 
 
 def test_static_scratch_refuses_what_does_not_fit():
