@@ -44,6 +44,7 @@ struct ThinArgs {
   FastDiv divRowUnits; // by the 16-byte vectors (or dwords) of an input row
   FastDiv divBorder;   // by the dwords of zeros left and right of a row
   uint32_t biasByte;   // where the fp32 bias lies in LDS
+  uint32_t weightByte; // ... and the packed weights, on their way to registers
   uint32_t cutElems;   // elements of a row in truncated columns
   FastDiv divCut;
 };
@@ -116,30 +117,16 @@ __global__ __launch_bounds__(kThinThreads)
   const ThinInputDesc &d = a.d;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
-  // The weights, through LDS into every wave's registers.
-  {
-    const uintx4 *src = reinterpret_cast<const uintx4 *>(weightsPacked);
-    uintx4 *dst = reinterpret_cast<uintx4 *>(lds);
-    constexpr int kVecs = CB * KH * 64;
-    uintx4 v[(kVecs + kThinThreads - 1) / kThinThreads];
+  // The weights go through LDS into every wave's registers; their loads are
+  // issued first and written to LDS behind the first tile's rows, so that
+  // one trip to memory covers both.
+  constexpr int kWeightVecs = CB * KH * 64;
+  uintx4 weightVec[(kWeightVecs + kThinThreads - 1) / kThinThreads];
 #pragma unroll
-    for (int u = 0; u * kThinThreads < kVecs; ++u)
-      if (u * kThinThreads + t < kVecs)
-        v[u] = src[u * kThinThreads + t];
-#pragma unroll
-    for (int u = 0; u * kThinThreads < kVecs; ++u)
-      if (u * kThinThreads + t < kVecs)
-        dst[u * kThinThreads + t] = v[u];
-  }
-  __syncthreads();
-  half8 w[CB][KH];
-#pragma unroll
-  for (int cb = 0; cb != CB; ++cb)
-#pragma unroll
-    for (int kh = 0; kh != KH; ++kh)
-      w[cb][kh] =
-          reinterpret_cast<const half8 *>(lds)[(cb * KH + kh) * 64 + lane];
-  __syncthreads();
+  for (int u = 0; u * kThinThreads < kWeightVecs; ++u)
+    if (u * kThinThreads + t < kWeightVecs)
+      weightVec[u] = reinterpret_cast<const uintx4 *>(
+          weightsPacked)[u * kThinThreads + t];
 
   // Zeros left and right of the rows' data: written once, never overwritten.
   {
@@ -188,18 +175,19 @@ __global__ __launch_bounds__(kThinThreads)
     biasLds[t] = bias ? Load<OutT>::at(bias, t, 0) : 0.0f;
 
   const bool vec16 = (a.rowBytes & 15) == 0;
-  for (uint32_t tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+  // Input rows of a tile into LDS, zeros for rows outside the image (loads in
+  // batches of eight per thread, all on their way before the first is
+  // written to LDS).
+  auto stage = [&](uint32_t tile) {
     const uint32_t image = a.divTilesPerImage(tile);
     const uint32_t oh0 = (tile - image * a.tilesPerImage) * a.tileRows;
     const int32_t ih0 = int32_t(oh0 * d.strideH) - d.padH;
-    const __half *img = in + size_t(image) * d.inH * d.inW * d.inChans;
-    // Input rows ih0 .. ih0 + ldsRows - 1 into LDS, zeros for rows outside.
-    // (loads in batches of eight per thread, all on their way before the
-    // first is written to LDS)
+    const char *img = reinterpret_cast<const char *>(
+        in + size_t(image) * d.inH * d.inW * d.inChans);
     if (vec16)
-      copyRows<uintx4>(a, lds, reinterpret_cast<const char *>(img), ih0, t);
+      copyRows<uintx4>(a, lds, img, ih0, t);
     else
-      copyRows<uint32_t>(a, lds, reinterpret_cast<const char *>(img), ih0, t);
+      copyRows<uint32_t>(a, lds, img, ih0, t);
     if (a.cutElems) {
       // truncated columns read as zeros: wiped once the rows are in
       __syncthreads();
@@ -211,7 +199,32 @@ __global__ __launch_bounds__(kThinThreads)
                                     elem * 2) = __float2half(0.0f);
       }
     }
-    __syncthreads();
+  };
+  if (blockIdx.x < a.tiles)
+    stage(blockIdx.x);
+  {
+    uintx4 *dst = reinterpret_cast<uintx4 *>(lds + a.weightByte);
+#pragma unroll
+    for (int u = 0; u * kThinThreads < kWeightVecs; ++u)
+      if (u * kThinThreads + t < kWeightVecs)
+        dst[u * kThinThreads + t] = weightVec[u];
+  }
+  __syncthreads();
+  half8 w[CB][KH];
+#pragma unroll
+  for (int cb = 0; cb != CB; ++cb)
+#pragma unroll
+    for (int kh = 0; kh != KH; ++kh)
+      w[cb][kh] = reinterpret_cast<const half8 *>(
+          lds + a.weightByte)[(cb * KH + kh) * 64 + lane];
+
+  for (uint32_t tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
+    const uint32_t image = a.divTilesPerImage(tile);
+    const uint32_t oh0 = (tile - image * a.tilesPerImage) * a.tileRows;
+    if (tile != blockIdx.x) {
+      stage(tile);
+      __syncthreads();
+    }
 
     const uint32_t rowsHere =
         a.tileRows < d.outH - oh0 ? a.tileRows : d.outH - oh0;
@@ -328,8 +341,8 @@ ThinShape thinShape(const ThinInputDesc &d, uint32_t cus) {
   if (const char *e = getenv("MXK_THIN_TH")) chosen = atoi(e); // EXPERIMENT
   s.tileRows = std::min(chosen, std::max(1u, d.outH));
   s.ldsRows = (s.tileRows - 1) * d.strideH + s.rowsPacked;
-  // (+ 256 bytes behind them for the bias)
-  s.ldsBytes = std::max(s.ldsRows * s.pitch, weightBytes) + 256;
+  // (+ 256 bytes behind them for the bias, then the weights)
+  s.ldsBytes = s.ldsRows * s.pitch + 256 + weightBytes;
   s.ok = true;
   return s;
 }
@@ -465,7 +478,8 @@ hipError_t launchThinInput(const ThinInputDesc &d, int inType, int outType,
   a.divRowUnits =
       makeFastDiv((s.rowBytes & 15) == 0 ? s.rowBytes / 16 : s.rowBytes / 4);
   a.divBorder = makeFastDiv((s.pitch - s.rowBytes) / 4);
-  a.biasByte = s.ldsBytes - 256;
+  a.biasByte = s.ldsRows * s.pitch;
+  a.weightByte = a.biasByte + 256;
   a.cutElems = (d.loW + (d.inW - d.hiW)) * d.inChans;
   a.divCut = makeFastDiv(a.cutElems);
   if (l.tiles >= (1ull << 31))
