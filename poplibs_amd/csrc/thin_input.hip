@@ -49,12 +49,23 @@ struct ThinArgs {
   FastDiv divCut;
 };
 
-/// Output channel held by MFMA row m of channel block cb: lane quarter
-/// Q = m / 4 gets channels Q * 4 * CB + 4 * cb + m % 4, so that its 4 * CB
-/// results are neighbours.
+/// First of the four neighbouring output channels that lane quarter Q holds
+/// of channel block cb (MFMA rows 4 Q .. 4 Q + 3), of `blocks` blocks.  The
+/// blocks go in pairs of 32 channels: within a pair quarter Q holds channels
+/// 8 Q .. 8 Q + 7 (four from either block), so that a pixel's 64 bytes (fp16)
+/// are written by one store instruction's four quarters, whole; an odd last
+/// block stands alone with channels 4 Q .. 4 Q + 3.
+__host__ __device__ inline uint32_t thinChannelBase(uint32_t cb, uint32_t Q,
+                                                    uint32_t blocks) {
+  const uint32_t pair = cb / 2;
+  return (cb ^ 1u) < blocks ? pair * 32 + Q * 8 + (cb & 1u) * 4
+                            : pair * 32 + Q * 4;
+}
+
+/// Output channel held by MFMA row m of channel block cb.
 __host__ __device__ inline uint32_t thinChannelOf(uint32_t cb, uint32_t m,
                                                   uint32_t blocks) {
-  return (m / 4) * 4 * blocks + 4 * cb + m % 4;
+  return thinChannelBase(cb, m / 4, blocks) + m % 4;
 }
 
 /// Packed weights [cb][kh][lane][8]: lane l holds MFMA row l % 16 and
@@ -169,7 +180,7 @@ __global__ __launch_bounds__(kThinThreads)
   }
   // the bias, as fp32, behind the rows in LDS: a lane's 4 * CB channels are
   // read back when a block is stored
-  const uint32_t chan0 = (lane >> 4) * 4 * CB;
+  const uint32_t quarter = lane >> 4;
   float *biasLds = reinterpret_cast<float *>(lds + a.biasByte);
   if (t < CB * 16)
     biasLds[t] = bias ? Load<OutT>::at(bias, t, 0) : 0.0f;
@@ -247,7 +258,8 @@ __global__ __launch_bounds__(kThinThreads)
 #pragma unroll
       for (int cb = 0; cb != CB; ++cb)
         acc[cb] =
-            *reinterpret_cast<const floatx4 *>(biasLds + chan0 + 4 * cb);
+            *reinterpret_cast<const floatx4 *>(
+                biasLds + thinChannelBase(cb, quarter, CB));
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int kh = 0; kh != KH; ++kh) {
@@ -265,15 +277,13 @@ __global__ __launch_bounds__(kThinThreads)
       }
       const uint32_t ow = cbk * 16 + (lane & 15);
       if (ow < d.outW) {
-        OutT *dst = out +
-                    ((size_t(image) * d.outH + oh0 + r) * d.outW + ow) *
-                        d.outChans +
-                    chan0;
-        if constexpr (sizeof(OutT) == 2 && CB % 2 == 0) {
-          // two channel blocks' results, eight neighbouring channels, as one
-          // 16-byte store
+        OutT *dst = out + ((size_t(image) * d.outH + oh0 + r) * d.outW + ow) *
+                              d.outChans;
+        // a pair of channel blocks: eight neighbouring channels per lane
 #pragma unroll
-          for (int cb = 0; cb != CB; cb += 2) {
+        for (int cb = 0; cb + 1 < CB; cb += 2) {
+          OutT *at = dst + thinChannelBase(cb, quarter, CB);
+          if constexpr (sizeof(OutT) == 2) {
             const __half2 h[4] = {
                 roundPairToHalf(acc[cb][0], acc[cb][1]),
                 roundPairToHalf(acc[cb][2], acc[cb][3]),
@@ -281,15 +291,20 @@ __global__ __launch_bounds__(kThinThreads)
                 roundPairToHalf(acc[cb + 1][2], acc[cb + 1][3])};
             uintx4 u;
             __builtin_memcpy(&u, h, 16);
-            *reinterpret_cast<uintx4 *>(dst + 4 * cb) = u;
+            *reinterpret_cast<uintx4 *>(at) = u;
+          } else {
+            const float v0[4] = {acc[cb][0], acc[cb][1], acc[cb][2],
+                                 acc[cb][3]};
+            const float v1[4] = {acc[cb + 1][0], acc[cb + 1][1],
+                                 acc[cb + 1][2], acc[cb + 1][3]};
+            storeOut4(at, v0);
+            storeOut4(at + 4, v1);
           }
-        } else {
-#pragma unroll
-          for (int cb = 0; cb != CB; ++cb) {
-            const float v[4] = {acc[cb][0], acc[cb][1], acc[cb][2],
-                                acc[cb][3]};
-            storeOut4(dst + 4 * cb, v);
-          }
+        }
+        if constexpr (CB % 2 == 1) {
+          const float v[4] = {acc[CB - 1][0], acc[CB - 1][1], acc[CB - 1][2],
+                              acc[CB - 1][3]};
+          storeOut4(dst + thinChannelBase(CB - 1, quarter, CB), v);
         }
       }
     }
