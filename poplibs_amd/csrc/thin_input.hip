@@ -126,7 +126,11 @@ __global__ __launch_bounds__(kThinThreads)
     OutT *__restrict__ out) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const ThinInputDesc &d = a.d;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  // (the same for every lane of a wave, and said so: what depends on it and
+  // the launch's constants alone - a block's row and column, the start of
+  // its outputs - is then worked out on the scalar unit)
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
 
   // The weights go through LDS into every wave's registers; their loads are
   // issued first and written to LDS behind the first tile's rows, so that
