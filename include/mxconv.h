@@ -469,7 +469,11 @@ mxconv_status mxconv_matmul_out_to_external(const mxconv_plan *plan,
  * (lib/poplin/ConvUtilInternal.cpp:941-954).  For
  * mxconv_convolution_weight_update give forward parameters whose output type
  * equals the input type, as the reference does (:3535), so that the deltas
- * come out in the weights' type. */
+ * come out in the weights' type.  For a layer without spatial extent (every
+ * field and kernel dimension 1, one group) the plan also holds the plan of
+ * one matrix product, transpose(deltas) x activations, which
+ * mxconv_calculate_weight_deltas then runs instead of the pass's convolution;
+ * mxconv_weight_update_workspace_bytes is the size either way. */
 mxconv_status mxconv_weight_update_plan_create(const mxconv_params *fwd,
                                                const char *const *option_keys,
                                                const char *const *option_values,
