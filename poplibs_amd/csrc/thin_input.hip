@@ -24,7 +24,6 @@
 
 #include <algorithm>
 #include <cstdint>
-#include <cstdlib>
 
 namespace mxk {
 namespace {
@@ -357,7 +356,6 @@ ThinShape thinShape(const ThinInputDesc &d, uint32_t cus) {
   }
   if (!chosen)
     return s;
-  if (const char *e = getenv("MXK_THIN_TH")) chosen = atoi(e); // EXPERIMENT
   s.tileRows = std::min(chosen, std::max(1u, d.outH));
   s.ldsRows = (s.tileRows - 1) * d.strideH + s.rowsPacked;
   // (+ 256 bytes behind them for the bias, then the weights)
