@@ -313,8 +313,8 @@ hipError_t launchPointwise(const PointwiseDesc &d, int inType, int outType,
 /// Convolution of an input with 1 to 4 channels (one group, half inputs, a
 /// 2-D field, stride, zero padding, input truncation; nothing dilated) on the
 /// matrix cores without padding the channels: a kernel row's kW * Ci
-/// neighbouring elements (32 at most) are one k-step.  16, 32, 48 or 64 output
-/// channels, up to 7 kernel rows.
+/// neighbouring elements (32 at most), in chunks of 8, fill k-steps of 32.
+/// 16, 32, 48 or 64 output channels, up to 28 chunks (7 k-steps).
 struct ThinInputDesc {
   uint32_t batch, inChans, outChans;
   uint32_t inH, inW, outH, outW, kH, kW;
@@ -323,8 +323,11 @@ struct ThinInputDesc {
   uint32_t loH, hiH, loW, hiW; // rows and columns outside read as zeros
 };
 bool thinInputTakes(const ThinInputDesc &d, int inType, int outType);
-/// Elements of the packed weights ([16-channel block][kernel row][lane][8]).
+/// Elements of the packed weights ([16-channel block][k-step][lane][8]).
 uint64_t thinInputPackedElems(const ThinInputDesc &d);
+/// k-steps of 32: a kernel row is ceil(kW * Ci / 8) chunks of 8 elements,
+/// four chunks make a k-step.
+uint32_t thinInputKSteps(const ThinInputDesc &d);
 hipError_t launchPackThinInputWeights(const ThinInputDesc &d, const void *src,
                                       void *dst, hipStream_t stream);
 /// How launchThinInput runs a layer on a chip of `cus` compute units:

@@ -2,10 +2,12 @@
 // waveform's one) on the matrix cores, without padding the channels.
 //
 // In a channels-last image the kW pixels under one kernel row are kW * Ci
-// neighbouring elements - 21 for a 7 x 7 kernel over RGB - so a kernel row is
-// one k-step of 32: K = kH * 32 where padding the channels to a whole 16-byte
-// vector gives kH * kW * 8 (224 against 392 for that layer) and costs a copy
-// of the input besides.  The price is alignment: a window starts at any even
+// neighbouring elements - 21 for a 7 x 7 kernel over RGB: a kernel row is
+// ceil(kW * Ci / 8) chunks of 8 elements, and four chunks (of one kernel row
+// or of neighbouring ones) make a k-step of 32.  K = 6 * 32 for that layer
+// where padding the channels to a whole 16-byte vector gives 7 * 7 * 8 = 392
+// and costs a copy of the input besides; a 3 x 3 kernel over RGB is two
+// k-steps.  The price is alignment: a window starts at any even
 // byte, so the operand is read from LDS as five aligned dwords and shifted
 // into place.
 //
@@ -13,7 +15,7 @@
 //                the input rows under them lie in LDS, zeros around them
 //   wave       = blocks of 16 neighbouring output pixels, round robin
 //   MFMA       = v_mfma_f32_16x16x32_f16, weights as the row operand:
-//                D[co][pixel] += W[co][k] * X[k][pixel], one per kernel row and
+//                D[co][pixel] += W[co][k] * X[k][pixel], one per k-step and
 //                block of 16 output channels; all weights stay in registers
 //   output     = output channels are dealt to the MFMA rows so that a lane
 //                ends up with 4 * CB neighbouring channels of one pixel
@@ -33,7 +35,7 @@ constexpr int kThinThreads = 256;
 struct ThinArgs {
   ThinInputDesc d;
   uint32_t tileRows;   // TH: output rows per tile
-  uint32_t ldsRows;    // (TH - 1) * strideH + KH
+  uint32_t ldsRows;    // (TH - 1) * strideH + kH
   uint32_t pitch;      // bytes of an LDS row
   uint32_t dataOff;    // byte of input column 0 in an LDS row (16-aligned)
   uint32_t rowBytes;   // inW * ci * 2
@@ -67,19 +69,32 @@ __host__ __device__ inline uint32_t thinChannelOf(uint32_t cb, uint32_t m,
   return thinChannelBase(cb, m / 4, blocks) + m % 4;
 }
 
-/// Packed weights [cb][kh][lane][8]: lane l holds MFMA row l % 16 and
-/// k = 8 * (l / 16) .. + 7 of kernel row kh, k = kw * Ci + c, zeros beyond
-/// kW * Ci and for kernel rows beyond kH.
+/// Chunks of 8 elements per kernel row, in all, and the k-steps they make.
+__host__ __device__ inline uint32_t thinChunksPerRow(const ThinInputDesc &d) {
+  return (d.kW * d.inChans + 7) / 8;
+}
+__host__ __device__ inline uint32_t thinChunks(const ThinInputDesc &d) {
+  return d.kH * thinChunksPerRow(d);
+}
+__host__ __device__ inline uint32_t thinKSteps(const ThinInputDesc &d) {
+  return (thinChunks(d) + 3) / 4;
+}
+
+/// Packed weights [cb][k-step][lane][8]: lane l holds MFMA row l % 16 and
+/// chunk 4 * step + l / 16 - elements 8 * part .. + 7 of kernel row `row`,
+/// chunk = row * chunksPerRow + part, element = kw * Ci + c - with zeros
+/// beyond kW * Ci and beyond the last chunk.
 __global__ void packThinWeightsKernel(const __half *__restrict__ src,
                                       __half *__restrict__ dst,
-                                      ThinInputDesc d, uint32_t rowsPacked,
-                                      uint32_t total) {
+                                      ThinInputDesc d, uint32_t total) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total)
     return;
+  const uint32_t steps = thinKSteps(d), perRow = thinChunksPerRow(d);
   const uint32_t e = i % 8, lane = (i / 8) % 64;
-  const uint32_t kh = (i / 512) % rowsPacked, cb = i / 512 / rowsPacked;
-  const uint32_t k = 8 * (lane / 16) + e;
+  const uint32_t step = (i / 512) % steps, cb = i / 512 / steps;
+  const uint32_t chunk = 4 * step + lane / 16;
+  const uint32_t kh = chunk / perRow, k = (chunk % perRow) * 8 + e;
   const uint32_t co = thinChannelOf(cb, lane % 16, d.outChans / 16);
   const uint32_t kw = k / d.inChans, c = k % d.inChans;
   __half v = __float2half(0.0f);
@@ -117,7 +132,7 @@ __device__ __forceinline__ void copyRows(const ThinArgs &a, char *lds,
   }
 }
 
-template <int CB, int KH, class OutT>
+template <int CB, int KS, class OutT>
 __global__ __launch_bounds__(kThinThreads)
     __attribute__((amdgpu_waves_per_eu(2))) void thinInputKernel(
     ThinArgs a, const __half *__restrict__ in,
@@ -134,7 +149,7 @@ __global__ __launch_bounds__(kThinThreads)
   // The weights go through LDS into every wave's registers; their loads are
   // issued first and written to LDS behind the first tile's rows, so that
   // one trip to memory covers both.
-  constexpr int kWeightVecs = CB * KH * 64;
+  constexpr int kWeightVecs = CB * KS * 64;
   uintx4 weightVec[(kWeightVecs + kThinThreads - 1) / kThinThreads];
 #pragma unroll
   for (int u = 0; u * kThinThreads < kWeightVecs; ++u)
@@ -155,31 +170,46 @@ __global__ __launch_bounds__(kThinThreads)
     }
   }
 
-  // This lane's part of an operand: pixel lane % 16 of a block, elements
-  // 8 * (lane / 16) .. + 7 of a kernel row.  Its byte within an LDS row, for
-  // block 0 (a block further on is 16 * strideW pixels further on):
+  // This lane's part of a k-step's operand: pixel lane % 16 of a block,
+  // chunk 4 * step + lane / 16 - eight elements of one kernel row.  The
+  // pixel's first byte within an LDS row, for block 0 (a block further on is
+  // 16 * strideW pixels further on):
   const uint32_t pixelBytes = d.inChans * 2;
   const int32_t colByte0 =
       int32_t(a.dataOff) +
-      (int32_t((lane & 15) * d.strideW) - d.padW) * int32_t(pixelBytes) +
-      (lane >> 4) * 16;
-  // (a multiple of 32 bytes: every block's operand starts at the same byte
-  // of a dword)
+      (int32_t((lane & 15) * d.strideW) - d.padW) * int32_t(pixelBytes);
+  // (a multiple of 32 bytes, like a chunk's 16 and the rows' pitch: every
+  // operand of a lane starts at the same byte of a dword)
   const uint32_t blockStep = 16 * d.strideW * pixelBytes;
-  const uint32_t colWord0 = uint32_t(colByte0) & ~3u;
   const uint32_t shift = uint32_t(colByte0) & 3u;
-  // The operand's dword i is bytes shift .. shift + 3 of the aligned dwords
-  // i and i + 1, with the elements beyond the kernel row's kW * Ci wiped:
-  // one byte permute does both (selector byte b + shift picks that byte of
-  // the pair, 0x0c a zero).
-  uint32_t pick[4];
+  // Per k-step: where the lane's chunk lies from the block's first row (the
+  // aligned dword at or below it), and the byte permute that turns the
+  // aligned dwords i and i + 1 into the operand's dword i - selector byte
+  // b + shift picks that byte of the pair, 0x0c a zero: for the elements
+  // beyond the kernel row's kW * Ci (the next pixels') and for chunks beyond
+  // the last.
+  uint32_t chunkAt[KS], pick[KS][4];
+  {
+    const uint32_t perRow = thinChunksPerRow(d), chunks = thinChunks(d);
+    const uint32_t kEnd = d.kW * d.inChans;
 #pragma unroll
-  for (int i = 0; i != 4; ++i) {
-    const uint32_t k = (lane >> 4) * 8 + 2 * i, kEnd = d.kW * d.inChans;
-    const uint32_t lo = k < kEnd ? (shift | ((shift + 1) << 8)) : 0x0c0cu;
-    const uint32_t hi =
-        k + 1 < kEnd ? ((shift + 2) | ((shift + 3) << 8)) : 0x0c0cu;
-    pick[i] = lo | (hi << 16);
+    for (int q = 0; q != KS; ++q) {
+      const uint32_t chunk = 4 * q + (lane >> 4);
+      const bool there = chunk < chunks;
+      const uint32_t row = there ? chunk / perRow : 0;
+      const uint32_t part = there ? chunk - row * perRow : 0;
+      chunkAt[q] = (uint32_t(colByte0) & ~3u) + row * a.pitch + part * 16;
+#pragma unroll
+      for (int i = 0; i != 4; ++i) {
+        const uint32_t k = part * 8 + 2 * i;
+        const uint32_t lo =
+            there && k < kEnd ? (shift | ((shift + 1) << 8)) : 0x0c0cu;
+        const uint32_t hi = there && k + 1 < kEnd
+                                ? ((shift + 2) | ((shift + 3) << 8))
+                                : 0x0c0cu;
+        pick[q][i] = lo | (hi << 16);
+      }
+    }
   }
   // the bias, as fp32, behind the rows in LDS: a lane's 4 * CB channels are
   // read back when a block is stored
@@ -224,13 +254,13 @@ __global__ __launch_bounds__(kThinThreads)
         dst[u * kThinThreads + t] = weightVec[u];
   }
   __syncthreads();
-  half8 w[CB][KH];
+  half8 w[CB][KS];
 #pragma unroll
   for (int cb = 0; cb != CB; ++cb)
 #pragma unroll
-    for (int kh = 0; kh != KH; ++kh)
-      w[cb][kh] = reinterpret_cast<const half8 *>(
-          lds + a.weightByte)[(cb * KH + kh) * 64 + lane];
+    for (int q = 0; q != KS; ++q)
+      w[cb][q] = reinterpret_cast<const half8 *>(
+          lds + a.weightByte)[(cb * KS + q) * 64 + lane];
 
   for (uint32_t tile = blockIdx.x; tile < a.tiles; tile += gridDim.x) {
     const uint32_t image = a.divTilesPerImage(tile);
@@ -246,36 +276,33 @@ __global__ __launch_bounds__(kThinThreads)
     constexpr uint32_t kWaves = kThinThreads / 64;
     for (uint32_t b = wave; b < blocks; b += kWaves) {
       const uint32_t r = a.divColBlocks(b), cbk = b - r * a.colBlocks;
-      const char *base =
-          lds + r * d.strideH * a.pitch + colWord0 + cbk * blockStep;
+      const char *base = lds + r * d.strideH * a.pitch + cbk * blockStep;
       // all of the block's reads, then its arithmetic
-      uint32_t x[KH][5];
+      uint32_t x[KS][5];
 #pragma unroll
-      for (int kh = 0; kh != KH; ++kh)
+      for (int q = 0; q != KS; ++q)
 #pragma unroll
         for (int i = 0; i != 5; ++i)
-          x[kh][i] =
-              reinterpret_cast<const uint32_t *>(base + kh * a.pitch)[i];
+          x[q][i] = reinterpret_cast<const uint32_t *>(base + chunkAt[q])[i];
       // the sums start from the bias
       floatx4 acc[CB];
 #pragma unroll
       for (int cb = 0; cb != CB; ++cb)
-        acc[cb] =
-            *reinterpret_cast<const floatx4 *>(
-                biasLds + thinChannelBase(cb, quarter, CB));
+        acc[cb] = *reinterpret_cast<const floatx4 *>(
+            biasLds + thinChannelBase(cb, quarter, CB));
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int kh = 0; kh != KH; ++kh) {
+      for (int q = 0; q != KS; ++q) {
         uintx4 u;
-        u.x = __builtin_amdgcn_perm(x[kh][1], x[kh][0], pick[0]);
-        u.y = __builtin_amdgcn_perm(x[kh][2], x[kh][1], pick[1]);
-        u.z = __builtin_amdgcn_perm(x[kh][3], x[kh][2], pick[2]);
-        u.w = __builtin_amdgcn_perm(x[kh][4], x[kh][3], pick[3]);
+        u.x = __builtin_amdgcn_perm(x[q][1], x[q][0], pick[q][0]);
+        u.y = __builtin_amdgcn_perm(x[q][2], x[q][1], pick[q][1]);
+        u.z = __builtin_amdgcn_perm(x[q][3], x[q][2], pick[q][2]);
+        u.w = __builtin_amdgcn_perm(x[q][4], x[q][3], pick[q][3]);
         half8 xs;
         __builtin_memcpy(&xs, &u, 16);
 #pragma unroll
         for (int cb = 0; cb != CB; ++cb)
-          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[cb][kh], xs,
+          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[cb][q], xs,
                                                            acc[cb], 0, 0, 0);
       }
       const uint32_t ow = cbk * 16 + (lane & 15);
@@ -316,7 +343,7 @@ __global__ __launch_bounds__(kThinThreads)
 }
 
 struct ThinShape {
-  uint32_t rowsPacked; // kernel rows the kernel is compiled for: 1, 3, 5 or 7
+  uint32_t kSteps; // k-steps of four chunks: 1 to 7
   uint32_t tileRows, ldsRows, pitch, dataOff, rowBytes, colBlocks;
   uint32_t ldsBytes;
   bool ok;
@@ -326,7 +353,7 @@ uint32_t alignUp(uint32_t v, uint32_t to) { return (v + to - 1) / to * to; }
 
 ThinShape thinShape(const ThinInputDesc &d, uint32_t cus) {
   ThinShape s{};
-  s.rowsPacked = d.kH <= 1 ? 1 : d.kH <= 3 ? 3 : d.kH <= 5 ? 5 : 7;
+  s.kSteps = thinKSteps(d);
   const uint32_t pixelBytes = d.inChans * 2;
   s.rowBytes = d.inW * pixelBytes;
   s.colBlocks = (d.outW + 15) / 16;
@@ -342,12 +369,12 @@ ThinShape thinShape(const ThinInputDesc &d, uint32_t cus) {
   if (extent > (1 << 16))
     return s;
   s.pitch = alignUp(uint32_t(extent), 16);
-  const uint32_t weightBytes = (d.outChans / 16) * s.rowsPacked * 1024;
+  const uint32_t weightBytes = (d.outChans / 16) * s.kSteps * 1024;
   // the largest tile of 16, 8, ... output rows that fits 64 KB and leaves
   // three tiles to two CUs; failing that the smallest
   uint32_t chosen = 0;
   for (uint32_t th = 16; th != 0; th /= 2) {
-    const uint32_t rows = (th - 1) * d.strideH + s.rowsPacked;
+    const uint32_t rows = (th - 1) * d.strideH + d.kH;
     if (uint64_t(rows) * s.pitch > 64 * 1024)
       continue;
     chosen = th;
@@ -357,18 +384,18 @@ ThinShape thinShape(const ThinInputDesc &d, uint32_t cus) {
   if (!chosen)
     return s;
   s.tileRows = std::min(chosen, std::max(1u, d.outH));
-  s.ldsRows = (s.tileRows - 1) * d.strideH + s.rowsPacked;
+  s.ldsRows = (s.tileRows - 1) * d.strideH + d.kH;
   // (+ 256 bytes behind them for the bias, then the weights)
   s.ldsBytes = s.ldsRows * s.pitch + 256 + weightBytes;
   s.ok = true;
   return s;
 }
 
-template <int CB, int KH, class OutT>
+template <int CB, int KS, class OutT>
 hipError_t launchOne(const ThinArgs &a, uint32_t grid, uint32_t ldsBytes,
                      const void *in, const void *w, const void *bias,
                      void *out, hipStream_t stream) {
-  hipLaunchKernelGGL((thinInputKernel<CB, KH, OutT>), dim3(grid),
+  hipLaunchKernelGGL((thinInputKernel<CB, KS, OutT>), dim3(grid),
                      dim3(kThinThreads), ldsBytes, stream, a,
                      static_cast<const __half *>(in),
                      static_cast<const __half *>(w),
@@ -382,14 +409,17 @@ hipError_t launchRows(uint32_t rows, const ThinArgs &a, uint32_t grid,
                       uint32_t ldsBytes, const void *in, const void *w,
                       const void *bias, void *out, hipStream_t stream) {
   switch (rows) {
-  case 1:
-    return launchOne<CB, 1, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
-  case 3:
-    return launchOne<CB, 3, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
-  case 5:
-    return launchOne<CB, 5, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
-  case 7:
-    return launchOne<CB, 7, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
+#define MXK_THIN_CASE(n)                                                       \
+  case n:                                                                      \
+    return launchOne<CB, n, OutT>(a, grid, ldsBytes, in, w, bias, out, stream);
+    MXK_THIN_CASE(1)
+    MXK_THIN_CASE(2)
+    MXK_THIN_CASE(3)
+    MXK_THIN_CASE(4)
+    MXK_THIN_CASE(5)
+    MXK_THIN_CASE(6)
+    MXK_THIN_CASE(7)
+#undef MXK_THIN_CASE
   }
   return hipErrorInvalidValue;
 }
@@ -426,7 +456,10 @@ bool thinInputTakes(const ThinInputDesc &d, int inType, int outType) {
   if (d.loH > d.hiH || d.hiH > d.inH || d.loW > d.hiW || d.hiW > d.inW)
     return false;
   if (d.inChans == 0 || d.inChans > 4 || d.kW * d.inChans > 32 ||
-      d.kH == 0 || d.kH > 7 || d.kH * d.kW < 2)
+      d.kH == 0 || d.kH > 28 || d.kH * d.kW < 2)
+    return false;
+  // 7 k-steps of four 8-element chunks at most (the weights' registers)
+  if (thinChunks(d) > 28)
     return false;
   if (d.outChans % 16 != 0 || d.outChans > 64)
     return false;
@@ -448,9 +481,10 @@ bool thinInputTakes(const ThinInputDesc &d, int inType, int outType) {
 }
 
 uint64_t thinInputPackedElems(const ThinInputDesc &d) {
-  const uint32_t rows = d.kH <= 1 ? 1 : d.kH <= 3 ? 3 : d.kH <= 5 ? 5 : 7;
-  return uint64_t(d.outChans / 16) * rows * 512;
+  return uint64_t(d.outChans / 16) * thinKSteps(d) * 512;
 }
+
+uint32_t thinInputKSteps(const ThinInputDesc &d) { return thinKSteps(d); }
 
 ThinInputLaunch thinInputLaunchShape(const ThinInputDesc &d, uint32_t cus) {
   const ThinShape s = thinShape(d, cus);
@@ -469,10 +503,9 @@ ThinInputLaunch thinInputLaunchShape(const ThinInputDesc &d, uint32_t cus) {
 hipError_t launchPackThinInputWeights(const ThinInputDesc &d, const void *src,
                                       void *dst, hipStream_t stream) {
   const uint32_t total = uint32_t(thinInputPackedElems(d));
-  const uint32_t rows = total / 512 / (d.outChans / 16);
   hipLaunchKernelGGL(packThinWeightsKernel, dim3((total + 255) / 256),
                      dim3(256), 0, stream, static_cast<const __half *>(src),
-                     static_cast<__half *>(dst), d, rows, total);
+                     static_cast<__half *>(dst), d, total);
   return hipGetLastError();
 }
 
@@ -503,10 +536,10 @@ hipError_t launchThinInput(const ThinInputDesc &d, int inType, int outType,
     return hipErrorInvalidConfiguration;
   const uint32_t grid = uint32_t(l.workgroups);
   if (outType == kHalf)
-    return launchBlocks<__half>(d.outChans / 16, s.rowsPacked, a, grid,
+    return launchBlocks<__half>(d.outChans / 16, s.kSteps, a, grid,
                                 s.ldsBytes, in, weightsPacked, bias, out,
                                 stream);
-  return launchBlocks<float>(d.outChans / 16, s.rowsPacked, a, grid,
+  return launchBlocks<float>(d.outChans / 16, s.kSteps, a, grid,
                              s.ldsBytes, in, weightsPacked, bias, out, stream);
 }
 

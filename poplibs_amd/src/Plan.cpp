@@ -719,10 +719,10 @@ mxconv_plan makePlanWith(const ConvParams &params,
     reason = "generic direct kernel (" + igemmWhyNot + ")";
   }
   // An input of 1 to 4 channels (an image, a waveform): the matrix-core
-  // kernel that takes the kW * Ci neighbouring elements under a kernel row as
-  // one k-step instead of padding the channels to a whole vector - no copy
-  // of the input, K = kH * 32 instead of kH * kW * 8 (N = 32, 224 x 224,
-  // 7 x 7 stride 2, 3 -> 64: 64 -> 17 us).
+  // kernel that takes the kW * Ci neighbouring elements under a kernel row in
+  // chunks of 8, four to a k-step, instead of padding the channels to a whole
+  // vector - no copy of the input, K = 192 instead of 392 for N = 32,
+  // 224 x 224, 7 x 7 stride 2, 3 -> 64 (58 -> 19 us).
   {
     mxk::ThinInputDesc &t = plan.thinInput;
     t.batch = uint32_t(s.batch), t.inChans = uint32_t(ci);
@@ -749,7 +749,8 @@ mxconv_plan makePlanWith(const ConvParams &params,
       throw poplar::invalid_option(
           "planConstraints gfx950 thinInput: that kernel takes 2-D "
           "convolutions of half inputs with 1 to 4 channels in one group "
-          "(kW * Ci <= 32, at most 7 kernel rows; 16, 32, 48 or 64 output "
+          "(kW * Ci <= 32, at most 28 chunks of 8 elements over the kernel "
+          "rows; 16, 32, 48 or 64 output "
           "channels; nothing dilated or flipped, no kernel truncation or "
           "padding, no output padding, no negative padding of the columns)");
     if (shapeOk && pc.thinInput != 0 &&
@@ -1448,18 +1449,15 @@ mxconv_plan::DetailedEstimate mxconv_plan::detailedEstimate() const {
     break;
   case Kernel::IGEMM: {
     if (thinInputOn) {
-      // its tensors' bytes at streaming rate (to be calibrated: the padded
-      // MFMA work of kH k-steps of 32 per 16 pixels and 16 channels at half
-      // the matrix cores' rate, whichever is longer)
+      // its tensors' bytes at streaming rate, or the MFMA work of its
+      // k-steps of 32 per 16 pixels and 16 channels at 1 PFLOP/s (the vector
+      // ALU's share of the SIMD's time included), whichever is longer
       const mxk::ThinInputLaunch l =
           mxk::thinInputLaunchShape(thinInput, gfx950::numCUs);
       const double flops = 2.0 * thinInput.batch * thinInput.outH *
                            ((thinInput.outW + 15) / 16 * 16) *
                            thinInput.outChans * 32.0 *
-                           (thinInput.kH <= 1   ? 1
-                            : thinInput.kH <= 3 ? 3
-                            : thinInput.kH <= 5 ? 5
-                                                : 7);
+                           mxk::thinInputKSteps(thinInput);
       e.computeUs = std::max(
           streamed(inputBytes() + outputBytes() + weightPackedBytes()),
           poplin::kLaunchUs + flops / 1.0e9);
@@ -1578,13 +1576,15 @@ std::string mxconv_plan::describe() const {
     const auto &t = thinInput;
     const mxk::ThinInputLaunch l =
         mxk::thinInputLaunchShape(t, gfx950::numCUs);
-    const unsigned rows = t.kH <= 1 ? 1 : t.kH <= 3 ? 3 : t.kH <= 5 ? 5 : 7;
+    const unsigned steps = mxk::thinInputKSteps(t);
+    const unsigned perRow = (t.kW * t.inChans + 7) / 8;
     os << "        gemm M x N x K             "
        << std::size_t(t.batch) * t.outH * t.outW << " x " << t.outChans
-       << " x " << rows * 32 << " (a kernel row's " << t.kW << " x "
+       << " x " << steps * 32 << " (a kernel row's " << t.kW << " x "
        << t.inChans << " = " << t.kW * t.inChans
-       << " neighbouring elements as one k-step of 32; " << t.kH
-       << " kernel rows run as " << rows << ")\n";
+       << " neighbouring elements as " << perRow
+       << " chunk(s) of 8; the " << t.kH * perRow << " chunks of " << t.kH
+       << " kernel rows in " << steps << " k-step(s) of four)\n";
     os << "        block M x N x K            16 x " << t.outChans
        << " x 32 per wave; tiles of " << l.tileRows
        << " output rows of one image, their input rows in " << l.ldsBytes
@@ -1593,7 +1593,7 @@ std::string mxconv_plan::describe() const {
        << " persistent (4 waves) taking " << l.tiles << " tiles in turn on "
        << gfx950::numCUs << " CUs\n";
     os << "        packed weights             [" << t.outChans / 16
-       << " blocks of 16][" << rows << " kernel rows][64 lanes][8]\n";
+       << " blocks of 16][" << steps << " k-steps][64 lanes][8]\n";
   } else if (kernel == Kernel::IGEMM) {
     const auto &g = igemm;
     const std::size_t m = std::size_t(g.batch) * g.outD * g.outH * g.outW;

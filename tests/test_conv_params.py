@@ -477,8 +477,10 @@ def test_planner_choices():
                                kernel=(3, 3), ci=3, co=64))
     assert "kernel rows as k-steps" in thin.describe()
     assert "a kernel row's 3 x 3 = 9 neighbouring elements" in thin.describe()
+    # (two chunks of 8 per kernel row, six in all: two k-steps of four)
+    assert "x 64 x 64 (" in thin.describe()
     assert thin.buffer_bytes(4) == 0
-    assert thin.buffer_bytes(1) == 4 * 3 * 64 * 8 * 2
+    assert thin.buffer_bytes(1) == 4 * 2 * 64 * 8 * 2
     off = {"planConstraints": '{"gfx950": {"thinInput": 0}}'}
     assert "input channels padded      3 -> 8" in pa.Plan(
         make_params(pa.HALF, batch=2, field=(32, 32), kernel=(3, 3), ci=3,

@@ -1,6 +1,6 @@
 """Inputs of 1 to 4 channels (images, waveforms) on the matrix cores without
-padding the channels: a kernel row's kW * Ci neighbouring elements are one
-k-step (role of the reference's planner choosing a small inChansPerGroup for
+padding the channels: a kernel row's kW * Ci neighbouring elements fill
+k-steps in chunks of 8 (role of the reference's planner choosing a small inChansPerGroup for
 the first layer, lib/poplin/ConvPlan.cpp:1065-1238, and of the input
 rearrangement it costs there).  Parity against the oracle through the C ABI."""
 import numpy as np
@@ -38,6 +38,13 @@ CASES = [
     dict(batch=1, field=(12, 12), kernel=(4, 4), ci=4, co=32, pad=1,
          stride=2),
     dict(batch=1, field=(14, 16), kernel=(6, 3), ci=3, co=64, pad=1),
+    # more than seven kernel rows of few elements: chunks of several rows
+    # share a k-step
+    dict(batch=2, field=(20, 18), kernel=(9, 4), ci=1, co=16, pad=2),
+    dict(batch=1, field=(30, 30), kernel=(11, 11), ci=1, co=32, pad=5,
+         stride=2),
+    dict(batch=2, field=(16, 16), kernel=(14, 2), ci=4, co=16,
+         padLower=(6, 0), padUpper=(7, 1)),
     # more tiles than workgroups: the persistent loop goes round
     dict(batch=40, field=(64, 32), kernel=(3, 3), ci=3, co=16, pad=1),
     # no padding at all; an output narrower than a block of 16 pixels
@@ -118,7 +125,7 @@ def _random_thin_case(r):
     canonical form then moves outside - padded outputs, say - is skipped)."""
     ci = r.choice([1, 2, 3, 3, 4])
     kw = r.randint(1, 32 // ci)
-    kh = r.randint(1, 7)
+    kh = r.randint(1, min(10, 28 // ((kw * ci + 7) // 8)))
     if kh * kw < 2:
         kh = 2
     one_d = r.random() < 0.15
