@@ -46,6 +46,7 @@ struct ThinArgs {
   FastDiv divBorder;   // by the dwords of zeros left and right of a row
   uint32_t biasByte;   // where the fp32 bias lies in LDS
   uint32_t weightByte; // ... and the packed weights, on their way to registers
+  FastDiv divChunksPerRow; // by the chunks of 8 elements of a kernel row
   uint32_t cutElems;   // elements of a row in truncated columns
   FastDiv divCut;
 };
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(kThinThreads)
     for (int q = 0; q != KS; ++q) {
       const uint32_t chunk = 4 * q + (lane >> 4);
       const bool there = chunk < chunks;
-      const uint32_t row = there ? chunk / perRow : 0;
+      const uint32_t row = there ? a.divChunksPerRow(chunk) : 0;
       const uint32_t part = there ? chunk - row * perRow : 0;
       chunkAt[q] = (uint32_t(colByte0) & ~3u) + row * a.pitch + part * 16;
 #pragma unroll
@@ -530,6 +531,7 @@ hipError_t launchThinInput(const ThinInputDesc &d, int inType, int outType,
   a.divBorder = makeFastDiv((s.pitch - s.rowBytes) / 4);
   a.biasByte = s.ldsRows * s.pitch;
   a.weightByte = a.biasByte + 256;
+  a.divChunksPerRow = makeFastDiv(thinChunksPerRow(d));
   a.cutElems = (d.loW + (d.inW - d.hiW)) * d.inChans;
   a.divCut = makeFastDiv(a.cutElems);
   if (l.tiles >= (1ull << 31))
