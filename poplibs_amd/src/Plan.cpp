@@ -1449,18 +1449,21 @@ mxconv_plan::DetailedEstimate mxconv_plan::detailedEstimate() const {
     break;
   case Kernel::IGEMM: {
     if (thinInputOn) {
-      // its tensors' bytes at streaming rate, or the MFMA work of its
-      // k-steps of 32 per 16 pixels and 16 channels at 1 PFLOP/s (the vector
-      // ALU's share of the SIMD's time included), whichever is longer
+      // Launch, weights and the first tile's rows (3.5 us), then the block
+      // loop - matrix pipe and vector ALU take turns on a SIMD: 1.3 PFLOP/s
+      // of the k-steps' padded work - and the tensors' bytes beside it, which
+      // overlap it only in part.  Against measurements (N = 32, 224 x 224):
+      // 7 x 7 stride 2 3 -> 64 17.9 for 19-21 us, 3 x 3 3 -> 64 37.5 for 35,
+      // 3 x 3 3 -> 32 21.1 for 21.1, stride 2 8.7 for 9.5.
       const mxk::ThinInputLaunch l =
           mxk::thinInputLaunchShape(thinInput, gfx950::numCUs);
       const double flops = 2.0 * thinInput.batch * thinInput.outH *
                            ((thinInput.outW + 15) / 16 * 16) *
                            thinInput.outChans * 32.0 *
                            mxk::thinInputKSteps(thinInput);
-      e.computeUs = std::max(
-          streamed(inputBytes() + outputBytes() + weightPackedBytes()),
-          poplin::kLaunchUs + flops / 1.0e9);
+      e.computeUs =
+          3.5 + flops / 1.3e9 +
+          double(inputBytes() + outputBytes() + weightPackedBytes()) / 9.0e6;
       spread(e, l.workgroups, 1);
       break;
     }
